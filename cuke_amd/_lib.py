@@ -1,0 +1,92 @@
+"""ctypes binding of libkge_mi355.so (the C ABI declared in include/kge_mi355.h).
+
+There is no CPU or PyTorch fallback: if the HIP library has not been built the
+first call raises.
+"""
+from __future__ import annotations
+
+import ctypes as C
+import os
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(HERE, "libkge_mi355.so")
+
+MODELS = {"TransE": 0, "TransH": 1, "TransR": 2, "DistMult": 3, "ComplEx": 4, "RotatE": 5,
+          "TransF": 6, "RESCAL": 7}
+
+
+class KgeError(RuntimeError):
+    pass
+
+
+class Tables(C.Structure):
+    _fields_ = [("model", C.c_int32), ("norm_p", C.c_int32), ("gamma", C.c_float),
+                ("reserved", C.c_int32), ("dim", C.c_int64), ("rel_dim", C.c_int64),
+                ("n_ent", C.c_int64), ("n_rel", C.c_int64),
+                ("ent", C.c_void_p), ("rel", C.c_void_p), ("aux", C.c_void_p)]
+
+
+class Inspection(C.Structure):
+    _fields_ = [("n", C.c_int64), ("n_rows", C.c_int64), ("num_unique", C.c_void_p),
+                ("unique_ids", C.c_void_p), ("seg_offsets", C.c_void_p), ("perm", C.c_void_p),
+                ("inverse", C.c_void_p), ("sorted_seg", C.c_void_p)]
+
+
+class Batch(C.Structure):
+    _fields_ = [("batch", C.c_int64), ("h", C.c_void_p), ("r", C.c_void_p), ("t", C.c_void_p),
+                ("neg", C.c_void_p), ("chunk", C.c_int64), ("n_neg", C.c_int64),
+                ("ent_insp", C.POINTER(Inspection)), ("rel_insp", C.POINTER(Inspection))]
+
+
+class Saved(C.Structure):
+    _fields_ = [("pos", C.c_void_p), ("neg", C.c_void_p), ("side_pos", C.c_void_p),
+                ("side_neg", C.c_void_p), ("residual", C.c_void_p)]
+
+
+class Grads(C.Structure):
+    _fields_ = [("ent_rows", C.c_void_p), ("rel_rows", C.c_void_p), ("aux_rows", C.c_void_p)]
+
+
+EXPORTS = {
+    # name: (restype, argtypes)
+    "kge_strerror": (C.c_char_p, [C.c_int]),
+    "kge_abi_version": (C.c_int, []),
+    "kge_residual_fwd": (C.c_int, [C.POINTER(Tables), C.POINTER(Batch), C.c_void_p, C.c_void_p]),
+    "kge_score_fwd": (C.c_int, [C.POINTER(Tables), C.POINTER(Batch), C.c_void_p, C.c_void_p,
+                                C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p]),
+    "kge_inspect_workspace": (C.c_size_t, [C.c_int64, C.c_int64]),
+    "kge_inspect": (C.c_int, [C.POINTER(C.c_void_p), C.POINTER(C.c_int64), C.c_int, C.c_int64,
+                              C.POINTER(Inspection), C.c_void_p, C.c_size_t, C.c_void_p]),
+    "kge_margin_loss_workspace": (C.c_size_t, [C.c_int64, C.c_int64]),
+    "kge_margin_loss": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int64, C.c_int64, C.c_float,
+                                  C.c_float, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p,
+                                  C.c_size_t, C.c_void_p]),
+    "kge_score_bwd_workspace": (C.c_size_t, [C.POINTER(Tables), C.POINTER(Batch)]),
+    "kge_score_bwd": (C.c_int, [C.POINTER(Tables), C.POINTER(Batch), C.POINTER(Saved), C.c_void_p,
+                                C.c_void_p, C.POINTER(Grads), C.c_void_p, C.c_size_t, C.c_void_p]),
+    "kge_build_index": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int64,
+                                  C.c_int64, C.c_void_p]),
+    "kge_check_indices": (C.c_int, [C.c_void_p, C.c_int64, C.c_int64, C.c_void_p, C.c_void_p]),
+}
+
+_lib = None
+
+
+def lib() -> C.CDLL:
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise KgeError(
+                f"{LIB_PATH} is missing: build it with `python -m cuke_amd.build` "
+                "(hipcc, gfx950). There is no fallback path.")
+        handle = C.CDLL(LIB_PATH)
+        for name, (res, args) in EXPORTS.items():
+            fn = getattr(handle, name)
+            fn.restype, fn.argtypes = res, args
+        _lib = handle
+    return _lib
+
+
+def check(rc: int, what: str) -> None:
+    if rc != 0:
+        raise KgeError(f"{what}: {lib().kge_strerror(rc).decode()} ({rc})")

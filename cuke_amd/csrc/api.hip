@@ -1,0 +1,109 @@
+// extern "C" entry points: argument validation and kernel dispatch.
+#include "common.hpp"
+
+namespace kge {
+int launch_score_pos(const kge_tables *, const kge_batch *, float *, float *, float *, hipStream_t);
+int launch_score_neg(const kge_tables *, const kge_batch *, const float *, float *, float *,
+                     hipStream_t);
+int launch_transr_fwd(const kge_tables *, const kge_batch *, float *, float *, hipStream_t);
+
+__global__ void check_indices_kernel(const int64_t *idx, int64_t n, int64_t n_rows, int32_t *flag)
+{
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) {
+        const int64_t v = idx[i];
+        if (v < 0 || v >= n_rows) *flag = 1;  // benign race: every writer stores 1
+    }
+}
+
+static int validate_tables(const kge_tables *tab)
+{
+    if (!tab || !tab->ent) return KGE_EINVAL;
+    if (tab->model < KGE_TRANSE || tab->model > KGE_RESCAL) return KGE_EINVAL;
+    if (tab->dim <= 0 || tab->dim > (1 << 20) || tab->n_ent <= 0) return KGE_ESHAPE;
+    const bool complex_rows = tab->model == KGE_COMPLEX || tab->model == KGE_ROTATE;
+    if (complex_rows && (tab->dim & 1)) return KGE_ESHAPE;
+    if (tab->rel_dim != rel_width(tab->model, tab->dim)) return KGE_ESHAPE;
+    if (tab->rel_dim > 0 && (!tab->rel || tab->n_rel <= 0)) return KGE_EINVAL;
+    if (aux_width(tab->model, tab->dim) > 0 && !tab->aux) return KGE_EINVAL;
+    const bool normed = tab->model == KGE_TRANSE || tab->model == KGE_TRANSH || tab->model == KGE_TRANSR;
+    if (normed && tab->norm_p != 1 && tab->norm_p != 2) return KGE_EINVAL;
+    return KGE_OK;
+}
+
+static int validate_batch(const kge_batch *bat)
+{
+    if (!bat || bat->batch < 0) return KGE_EINVAL;
+    if (bat->batch > 0 && (!bat->h || !bat->r || !bat->t)) return KGE_EINVAL;
+    if (bat->batch >= (int64_t(1) << 31)) return KGE_ESHAPE;
+    if (bat->neg) {
+        if (bat->chunk <= 0 || bat->n_neg <= 0) return KGE_ESHAPE;
+        if (bat->batch % bat->chunk != 0) return KGE_ESHAPE;
+    }
+    return KGE_OK;
+}
+}  // namespace kge
+
+using namespace kge;
+
+extern "C" {
+
+const char *kge_strerror(int status)
+{
+    switch (status) {
+    case KGE_OK: return "ok";
+    case KGE_EINVAL: return "invalid argument (null pointer, unknown model or norm order)";
+    case KGE_ESHAPE: return "inconsistent sizes (batch % chunk, odd complex dim, bad rel_dim)";
+    case KGE_ELAUNCH: return "kernel launch failed";
+    case KGE_EWORKSPACE: return "workspace missing or too small";
+    case KGE_EUNSUPPORTED: return "combination not supported";
+    default: return "unknown status";
+    }
+}
+
+int kge_abi_version(void) { return 1; }
+
+int kge_residual_fwd(const kge_tables *tab, const kge_batch *bat, float *out, void *stream)
+{
+    int rc = validate_tables(tab);
+    if (rc) return rc;
+    if ((rc = validate_batch(bat))) return rc;
+    if (!out && bat->batch > 0) return KGE_EINVAL;
+    if (tab->model != KGE_TRANSE && tab->model != KGE_TRANSH && tab->model != KGE_TRANSR)
+        return KGE_EUNSUPPORTED;  // the other models have scalar outputs only
+    if (tab->model == KGE_TRANSR && bat->rel_insp)
+        return launch_transr_fwd(tab, bat, nullptr, out, as_stream(stream));
+    return launch_score_pos(tab, bat, nullptr, out, nullptr, as_stream(stream));
+}
+
+int kge_score_fwd(const kge_tables *tab, const kge_batch *bat, float *pos, float *neg,
+                  float *side_pos, float *side_neg, float *residual, void *stream)
+{
+    int rc = validate_tables(tab);
+    if (rc) return rc;
+    if ((rc = validate_batch(bat))) return rc;
+    hipStream_t st = as_stream(stream);
+    const bool want_neg = neg && bat->neg;
+    if (want_neg && tab->model == KGE_TRANSH && !side_pos) return KGE_EINVAL;
+    if (pos || side_pos || residual) {
+        if (tab->model == KGE_TRANSR && bat->rel_insp)
+            rc = launch_transr_fwd(tab, bat, pos, residual, st);
+        else
+            rc = launch_score_pos(tab, bat, pos, residual, side_pos, st);
+        if (rc) return rc;
+    }
+    if (want_neg) return launch_score_neg(tab, bat, side_pos, neg, side_neg, st);
+    return KGE_OK;
+}
+
+int kge_check_indices(const int64_t *idx, int64_t n, int64_t n_rows, int32_t *flag, void *stream)
+{
+    if (!flag || (n > 0 && !idx) || n < 0) return KGE_EINVAL;
+    if (n == 0) return KGE_OK;
+    hipLaunchKernelGGL(check_indices_kernel, dim3((unsigned)ceil_div(n, 256)), dim3(256), 0,
+                       as_stream(stream), idx, n, n_rows, flag);
+    KGE_CHECK_LAUNCH();
+    return KGE_OK;
+}
+
+}  // extern "C"

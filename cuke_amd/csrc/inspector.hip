@@ -1,0 +1,386 @@
+// GPU index inspector: stable LSD radix sort of (id, position) pairs followed by
+// run detection, giving unique rows, segment offsets, the sort permutation and the
+// inverse map.  It stands where the reference runs its per-16 bitonic inspector
+// (apps/kge/inspection/inspector.cu:68-136, called from apps/kge/kge.py:249-271) but
+// produces the whole-batch structure the gather and segmented-reduction kernels use.
+//
+// Keys are the low 32 bits of the ids (tables have < 2^32 rows); only as many digit
+// passes are run as the table's row count needs.  Every pass is: per-block digit
+// histogram -> column scan -> stable scatter.  Stability inside a block comes from
+// wave-level peer matching (ballots), not from atomics, so the result is
+// deterministic and equals a stable argsort.
+#include "common.hpp"
+
+namespace kge {
+
+constexpr int kSortThreads = 256;
+constexpr int kSortWaves = kSortThreads / kWave;
+constexpr int kKeysPerThread = 8;
+constexpr int kKeysPerBlock = kSortThreads * kKeysPerThread;  // 2048
+constexpr int kMaxDigitBits = 11;
+constexpr int kMaxBins = 1 << kMaxDigitBits;
+constexpr int kFusedScanBlocks = 32;  // up to this many blocks the scatter kernel scans the
+                                      // histogram columns itself (one launch less per pass)
+
+struct Parts {
+    const int64_t *p[4];
+    int64_t end[4];  // exclusive end offset of each part in the concatenation
+    int n_parts;
+};
+
+__device__ __forceinline__ uint32_t load_key(const Parts &parts, int64_t i)
+{
+    int q = 0;
+    while (q + 1 < parts.n_parts && i >= parts.end[q]) ++q;
+    const int64_t begin = q ? parts.end[q - 1] : 0;
+    return (uint32_t)parts.p[q][i - begin];
+}
+
+// ---- pass step 1: per-block digit histogram --------------------------------------------
+__global__ __launch_bounds__(kSortThreads) void radix_hist_kernel(Parts parts, const uint32_t *keys_in,
+                                                                  int64_t n, int shift, int bins,
+                                                                  uint32_t *hist)
+{
+    __shared__ uint32_t sh[kMaxBins];
+    for (int i = threadIdx.x; i < bins; i += kSortThreads) sh[i] = 0;
+    __syncthreads();
+    const int64_t base = (int64_t)blockIdx.x * kKeysPerBlock;
+    const uint32_t mask = (uint32_t)bins - 1;
+#pragma unroll
+    for (int j = 0; j < kKeysPerThread; ++j) {
+        const int64_t i = base + j * kSortThreads + threadIdx.x;
+        if (i < n) {
+            const uint32_t k = keys_in ? keys_in[i] : load_key(parts, i);
+            atomicAdd(&sh[(k >> shift) & mask], 1u);
+        }
+    }
+    __syncthreads();
+    for (int i = threadIdx.x; i < bins; i += kSortThreads) hist[(int64_t)blockIdx.x * bins + i] = sh[i];
+}
+
+// ---- pass step 2 (many blocks only): exclusive scan down each histogram column ---------
+__global__ void radix_colscan_kernel(uint32_t *hist, uint32_t *totals, int bins, int nblocks)
+{
+    const int bin = blockIdx.x * blockDim.x + threadIdx.x;
+    if (bin >= bins) return;
+    uint32_t run = 0;
+    for (int b = 0; b < nblocks; ++b) {
+        const uint32_t v = hist[(int64_t)b * bins + bin];
+        hist[(int64_t)b * bins + bin] = run;
+        run += v;
+    }
+    totals[bin] = run;
+}
+
+// exclusive scan of s[0..bins) in place (bins <= 2048, 256 threads)
+__device__ void block_exclusive_scan(uint32_t *s, int bins, uint32_t *wave_tot)
+{
+    const int per = (bins + kSortThreads - 1) / kSortThreads;  // <= 8
+    const int lo = threadIdx.x * per;
+    uint32_t loc[kMaxBins / kSortThreads];
+    uint32_t sum = 0;
+    for (int i = 0; i < per; ++i) {
+        const uint32_t v = lo + i < bins ? s[lo + i] : 0;
+        loc[i] = sum;
+        sum += v;
+    }
+    // inclusive scan of `sum` across the wave, then across the waves
+    const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x >> 6;
+    uint32_t inc = sum;
+#pragma unroll
+    for (int o = 1; o < kWave; o <<= 1) {
+        const uint32_t up = __shfl_up(inc, o, kWave);
+        if (lane >= o) inc += up;
+    }
+    if (lane == kWave - 1) wave_tot[wave] = inc;
+    __syncthreads();
+    uint32_t woff = 0;
+    for (int w = 0; w < wave; ++w) woff += wave_tot[w];
+    const uint32_t excl = woff + inc - sum;
+    for (int i = 0; i < per; ++i)
+        if (lo + i < bins) s[lo + i] = excl + loc[i];
+    __syncthreads();
+}
+
+// ---- pass step 3: stable scatter ---------------------------------------------------------
+__global__ __launch_bounds__(kSortThreads) void radix_scatter_kernel(
+    Parts parts, const uint32_t *keys_in, const int32_t *vals_in, int64_t n, int shift, int digit_bits,
+    const uint32_t *hist, const uint32_t *totals, int nblocks, int fused_scan, uint32_t *keys_out,
+    int32_t *vals_out)
+{
+    __shared__ uint32_t s_base[kMaxBins];               // global start of (bin, this block)
+    __shared__ uint32_t s_cnt[kSortWaves][kMaxBins];    // per-wave running digit counts
+    __shared__ uint32_t s_wtot[kSortWaves];
+    const int bins = 1 << digit_bits;
+    const uint32_t mask = (uint32_t)bins - 1;
+    const int tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid >> 6;
+    const int me = blockIdx.x;
+
+    // bin totals -> s_base (scanned below); this block's offset inside each bin -> s_cnt[0] (temp)
+    for (int bin = tid; bin < bins; bin += kSortThreads) {
+        uint32_t tot, part;
+        if (fused_scan) {
+            tot = 0, part = 0;
+            for (int b = 0; b < nblocks; ++b) {
+                const uint32_t v = hist[(int64_t)b * bins + bin];
+                tot += v;
+                part += b < me ? v : 0;
+            }
+        } else {
+            tot = totals[bin];
+            part = hist[(int64_t)me * bins + bin];
+        }
+        s_base[bin] = tot;
+        s_cnt[0][bin] = part;
+    }
+    __syncthreads();
+    block_exclusive_scan(s_base, bins, s_wtot);
+    for (int bin = tid; bin < bins; bin += kSortThreads) {
+        s_base[bin] += s_cnt[0][bin];
+    }
+    __syncthreads();
+    for (int bin = tid; bin < bins; bin += kSortThreads)
+#pragma unroll
+        for (int w = 0; w < kSortWaves; ++w) s_cnt[w][bin] = 0;
+    __syncthreads();
+
+    // each wave ranks its 512 consecutive keys in 8 rounds of 64, in order
+    const int64_t wbase = (int64_t)me * kKeysPerBlock + (int64_t)wave * (kKeysPerThread * kWave);
+    uint32_t key[kKeysPerThread], lrank[kKeysPerThread];
+    int32_t val[kKeysPerThread];
+    const uint64_t lt_mask = lane ? (~0ull >> (kWave - lane)) : 0ull;
+#pragma unroll
+    for (int j = 0; j < kKeysPerThread; ++j) {
+        const int64_t i = wbase + j * kWave + lane;
+        const bool ok = i < n;
+        key[j] = ok ? (keys_in ? keys_in[i] : load_key(parts, i)) : 0u;
+        val[j] = ok ? (vals_in ? vals_in[i] : (int32_t)i) : 0;
+        const uint32_t dg = (key[j] >> shift) & mask;
+        uint64_t peers = __ballot(ok);
+        for (int bit = 0; bit < digit_bits; ++bit) {
+            const bool one = (dg >> bit) & 1u;
+            const uint64_t m = __ballot(one);
+            peers &= one ? m : ~m;
+        }
+        // lanes with !ok fall out: their `peers` may be anything but they never write
+        const int leader = __ffsll((unsigned long long)peers) - 1;
+        const uint32_t cnt = __popcll(peers);
+        uint32_t old = 0;
+        if (ok && lane == leader) {
+            old = s_cnt[wave][dg];
+            s_cnt[wave][dg] = old + cnt;
+        }
+        old = __shfl(old, leader < 0 ? 0 : leader, kWave);
+        lrank[j] = old + __popcll(peers & lt_mask);
+        __builtin_amdgcn_wave_barrier();  // keep the rounds' LDS counter updates in order
+    }
+    __syncthreads();
+    // turn per-wave counts into per-wave start positions
+    for (int bin = tid; bin < bins; bin += kSortThreads) {
+        uint32_t run = s_base[bin];
+#pragma unroll
+        for (int w = 0; w < kSortWaves; ++w) {
+            const uint32_t c = s_cnt[w][bin];
+            s_cnt[w][bin] = run;
+            run += c;
+        }
+    }
+    __syncthreads();
+#pragma unroll
+    for (int j = 0; j < kKeysPerThread; ++j) {
+        const int64_t i = wbase + j * kWave + lane;
+        if (i < n) {
+            const uint32_t dg = (key[j] >> shift) & mask;
+            const uint32_t pos = s_cnt[wave][dg] + lrank[j];
+            keys_out[pos] = key[j];
+            vals_out[pos] = val[j];
+        }
+    }
+}
+
+// ---- dedup -------------------------------------------------------------------------------
+__global__ __launch_bounds__(kSortThreads) void count_heads_kernel(const uint32_t *keys, int64_t n,
+                                                                   uint32_t *block_heads)
+{
+    __shared__ uint32_t s_w[kSortWaves];
+    const int64_t base = (int64_t)blockIdx.x * kKeysPerBlock;
+    int c = 0;
+#pragma unroll
+    for (int j = 0; j < kKeysPerThread; ++j) {
+        const int64_t i = base + j * kSortThreads + threadIdx.x;
+        if (i < n) c += (i == 0 || keys[i] != keys[i - 1]) ? 1 : 0;
+    }
+    c = wave_sum_i(c);
+    if ((threadIdx.x & (kWave - 1)) == 0) s_w[threadIdx.x >> 6] = (uint32_t)c;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        uint32_t t = 0;
+        for (int w = 0; w < kSortWaves; ++w) t += s_w[w];
+        block_heads[blockIdx.x] = t;
+    }
+}
+
+__global__ __launch_bounds__(kSortThreads) void finalize_kernel(const uint32_t *keys, const int32_t *perm,
+                                                                int64_t n, const uint32_t *block_heads,
+                                                                int nblocks, kge_inspection out)
+{
+    __shared__ uint32_t s_red[kSortWaves], s_all[kSortWaves], s_scan[kSortWaves];
+    const int tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid >> 6;
+    const int me = blockIdx.x;
+    // heads in the blocks before this one, and in all blocks
+    uint32_t before = 0, all = 0;
+    for (int b = tid; b < nblocks; b += kSortThreads) {
+        const uint32_t v = block_heads[b];
+        all += v;
+        before += b < me ? v : 0;
+    }
+    before = (uint32_t)wave_sum_i((int)before);
+    all = (uint32_t)wave_sum_i((int)all);
+    if (lane == 0) s_red[wave] = before, s_all[wave] = all;
+    __syncthreads();
+    before = 0, all = 0;
+    for (int w = 0; w < kSortWaves; ++w) before += s_red[w], all += s_all[w];
+    if (me == 0 && tid == 0) {
+        out.num_unique[0] = (int32_t)all;
+        out.seg_offsets[all] = (int32_t)n;
+    }
+    // thread owns 8 consecutive positions so that a plain running sum gives the ranks
+    const int64_t lo = (int64_t)me * kKeysPerBlock + (int64_t)tid * kKeysPerThread;
+    uint32_t k[kKeysPerThread];
+    bool head[kKeysPerThread];
+    uint32_t mine = 0;
+    uint32_t prev = (lo > 0 && lo < n) ? keys[lo - 1] : 0;
+#pragma unroll
+    for (int j = 0; j < kKeysPerThread; ++j) {
+        const int64_t i = lo + j;
+        k[j] = i < n ? keys[i] : 0;
+        head[j] = i < n && (i == 0 || k[j] != prev);
+        prev = k[j];
+        mine += head[j] ? 1 : 0;
+    }
+    uint32_t inc = mine;
+#pragma unroll
+    for (int o = 1; o < kWave; o <<= 1) {
+        const uint32_t up = __shfl_up(inc, o, kWave);
+        if (lane >= o) inc += up;
+    }
+    if (lane == kWave - 1) s_scan[wave] = inc;
+    __syncthreads();
+    uint32_t run = before + inc - mine;
+    for (int w = 0; w < wave; ++w) run += s_scan[w];
+#pragma unroll
+    for (int j = 0; j < kKeysPerThread; ++j) {
+        const int64_t i = lo + j;
+        if (i >= n) break;
+        if (head[j]) {
+            out.unique_ids[run] = (int64_t)k[j];
+            out.seg_offsets[run] = (int32_t)i;
+            ++run;
+        }
+        const int32_t seg = (int32_t)run - 1;
+        out.sorted_seg[i] = seg;
+        out.inverse[perm[i]] = seg;
+    }
+}
+
+// ---- host side ---------------------------------------------------------------------------
+struct SortPlan {
+    int bits, npass, digit_bits;
+    int64_t nblocks;
+    size_t off_keys0, off_keys1, off_vals, off_hist, off_totals, off_heads, total;
+};
+
+static size_t align_up(size_t x) { return (x + 255) & ~size_t(255); }
+
+static SortPlan make_plan(int64_t n, int64_t n_rows)
+{
+    SortPlan p{};
+    int bits = 1;
+    while (bits < 32 && (int64_t(1) << bits) < n_rows) ++bits;
+    p.bits = bits;
+    p.npass = (bits + kMaxDigitBits - 1) / kMaxDigitBits;
+    p.digit_bits = (bits + p.npass - 1) / p.npass;
+    p.nblocks = n > 0 ? ceil_div(n, kKeysPerBlock) : 1;
+    size_t o = 0;
+    const size_t n4 = align_up(sizeof(uint32_t) * (size_t)(n > 0 ? n : 1));
+    p.off_keys0 = o, o += n4;
+    p.off_keys1 = o, o += n4;
+    p.off_vals = o, o += n4;
+    p.off_hist = o, o += align_up(sizeof(uint32_t) * (size_t)p.nblocks * kMaxBins);
+    p.off_totals = o, o += align_up(sizeof(uint32_t) * kMaxBins);
+    p.off_heads = o, o += align_up(sizeof(uint32_t) * (size_t)p.nblocks);
+    p.total = o;
+    return p;
+}
+
+}  // namespace kge
+
+using namespace kge;
+
+extern "C" {
+
+size_t kge_inspect_workspace(int64_t n, int64_t n_rows)
+{
+    if (n < 0 || n_rows <= 0) return 0;
+    return make_plan(n, n_rows).total;
+}
+
+int kge_inspect(const int64_t *const *parts_in, const int64_t *part_len, int n_parts, int64_t n_rows,
+                const kge_inspection *out, void *workspace, size_t workspace_bytes, void *stream)
+{
+    if (!out || !parts_in || !part_len || n_parts < 1 || n_parts > 4) return KGE_EINVAL;
+    if (n_rows <= 0 || n_rows > (int64_t(1) << 32)) return KGE_ESHAPE;
+    Parts parts{};
+    parts.n_parts = n_parts;
+    int64_t n = 0;
+    for (int q = 0; q < n_parts; ++q) {
+        if (part_len[q] < 0 || (part_len[q] > 0 && !parts_in[q])) return KGE_EINVAL;
+        n += part_len[q];
+        parts.p[q] = parts_in[q];
+        parts.end[q] = n;
+    }
+    if (n != out->n || n >= (int64_t(1) << 31)) return KGE_ESHAPE;
+    if (!out->num_unique || !out->seg_offsets) return KGE_EINVAL;
+    if (n > 0 && (!out->unique_ids || !out->perm || !out->inverse || !out->sorted_seg)) return KGE_EINVAL;
+    const SortPlan p = make_plan(n, n_rows);
+    if (!workspace || workspace_bytes < p.total) return KGE_EWORKSPACE;
+    hipStream_t st = as_stream(stream);
+    char *ws = static_cast<char *>(workspace);
+    uint32_t *keys_final = reinterpret_cast<uint32_t *>(ws + p.off_keys0);
+    uint32_t *keys_tmp = reinterpret_cast<uint32_t *>(ws + p.off_keys1);
+    int32_t *vals_tmp = reinterpret_cast<int32_t *>(ws + p.off_vals);
+    uint32_t *hist = reinterpret_cast<uint32_t *>(ws + p.off_hist);
+    uint32_t *totals = reinterpret_cast<uint32_t *>(ws + p.off_totals);
+    uint32_t *heads = reinterpret_cast<uint32_t *>(ws + p.off_heads);
+    const int nblocks = (int)p.nblocks;
+    const int bins = 1 << p.digit_bits;
+
+    if (n > 0) {
+        const uint32_t *kin = nullptr;
+        const int32_t *vin = nullptr;
+        for (int pass = 0; pass < p.npass; ++pass) {
+            const bool to_final = ((p.npass - 1 - pass) & 1) == 0;
+            uint32_t *kout = to_final ? keys_final : keys_tmp;
+            int32_t *vout = to_final ? out->perm : vals_tmp;
+            const int shift = pass * p.digit_bits;
+            const int fused = nblocks <= kFusedScanBlocks;
+            hipLaunchKernelGGL(radix_hist_kernel, dim3(nblocks), dim3(kSortThreads), 0, st, parts, kin, n,
+                               shift, bins, hist);
+            if (!fused)
+                hipLaunchKernelGGL(radix_colscan_kernel, dim3((bins + 255) / 256), dim3(256), 0, st, hist,
+                                   totals, bins, nblocks);
+            hipLaunchKernelGGL(radix_scatter_kernel, dim3(nblocks), dim3(kSortThreads), 0, st, parts, kin,
+                               vin, n, shift, p.digit_bits, hist, totals, nblocks, fused, kout, vout);
+            kin = kout;
+            vin = vout;
+        }
+        hipLaunchKernelGGL(count_heads_kernel, dim3(nblocks), dim3(kSortThreads), 0, st, keys_final, n,
+                           heads);
+    }
+    hipLaunchKernelGGL(finalize_kernel, dim3(nblocks), dim3(kSortThreads), 0, st, keys_final, out->perm, n,
+                       heads, n > 0 ? nblocks : 0, *out);
+    KGE_CHECK_LAUNCH();
+    return KGE_OK;
+}
+
+}  // extern "C"

@@ -1,0 +1,217 @@
+// Positive-triple kernels: one wavefront per (h, r, t) triple, rows gathered with
+// 128-bit loads straight into registers, norms / dot products reduced with a
+// wave64 butterfly.  Replaces the generated FNAME_kernel of
+// pycuke1/codegen/gpu.py:182-236 (16 triples x 32 lanes per block) for the
+// model definitions of apps/kge/kge.py:273-390.
+#include "common.hpp"
+
+namespace kge {
+
+struct PosArgs {
+    const float *ent, *rel, *aux;
+    const int64_t *h, *r, *t;
+    int64_t B;
+    int d, rel_dim;
+    float gamma;
+    float *pos;       // [B] scores or nullptr
+    float *resid;     // [B, d] residual rows or nullptr (TransE / TransH / TransR)
+    float *side_pos;  // [B] TransH: w.h (used by the shared-negative kernels)
+};
+
+constexpr int kPosWaves = 4;
+
+template <int P>
+__device__ __forceinline__ float norm_term(float u)
+{
+    return P == 1 ? fabsf(u) : u * u;
+}
+
+template <int MODEL, int P, int V>
+__global__ __launch_bounds__(kPosWaves *kWave) void score_pos_kernel(PosArgs a)
+{
+    extern __shared__ float lds[];  // TransR / RESCAL only: kPosWaves * d floats
+    const int lane = threadIdx.x & (kWave - 1);
+    const int wave = threadIdx.x >> 6;
+    const int64_t b = (int64_t)blockIdx.x * kPosWaves + wave;
+    const bool valid = b < a.B;
+    const int64_t bb = valid ? b : 0;
+    const int d = a.d;
+    const int64_t rid = a.r[bb];
+    const float *eh = a.ent + a.h[bb] * (int64_t)d;
+    const float *et = a.ent + a.t[bb] * (int64_t)d;
+    const float *rr = a.rel ? a.rel + rid * (int64_t)a.rel_dim : nullptr;
+    float *out = a.resid ? a.resid + bb * (int64_t)d : nullptr;
+    float acc = 0.0f;
+
+    if constexpr (MODEL == KGE_TRANSE) {
+        for (int j = lane * V; j < d; j += kWave * V) {
+            const Vec<V> vh = Vec<V>::load(eh + j), vt = Vec<V>::load(et + j),
+                         vr = Vec<V>::load(rr + j);
+            Vec<V> u;
+#pragma unroll
+            for (int e = 0; e < V; ++e) {
+                u.v[e] = (vh.v[e] - vt.v[e]) + vr.v[e];  // same order as the generated loop
+                acc += norm_term<P>(u.v[e]);
+            }
+            if (out && valid) u.store(out + j);
+        }
+    } else if constexpr (MODEL == KGE_TRANSH) {
+        const float *w = a.aux + rid * (int64_t)d;
+        float sd = 0.0f, wh = 0.0f;
+        for (int j = lane * V; j < d; j += kWave * V) {
+            const Vec<V> vh = Vec<V>::load(eh + j), vt = Vec<V>::load(et + j),
+                         vw = Vec<V>::load(w + j);
+#pragma unroll
+            for (int e = 0; e < V; ++e) {
+                sd += vw.v[e] * (vh.v[e] - vt.v[e]);
+                wh += vw.v[e] * vh.v[e];
+            }
+        }
+        sd = wave_sum(sd);
+        wh = wave_sum(wh);
+        if (a.side_pos && valid && lane == 0) a.side_pos[b] = wh;
+        for (int j = lane * V; j < d; j += kWave * V) {
+            const Vec<V> vh = Vec<V>::load(eh + j), vt = Vec<V>::load(et + j),
+                         vr = Vec<V>::load(rr + j), vw = Vec<V>::load(w + j);
+            Vec<V> u;
+#pragma unroll
+            for (int e = 0; e < V; ++e) {
+                u.v[e] = ((vh.v[e] - vt.v[e]) + vr.v[e]) - sd * vw.v[e];
+                acc += norm_term<P>(u.v[e]);
+            }
+            if (out && valid) u.store(out + j);
+        }
+    } else if constexpr (MODEL == KGE_TRANSR || MODEL == KGE_RESCAL) {
+        // Ungrouped per-triple vector x matrix product (the shape of the reference's
+        // kernel: every triple streams its own 4*d*d-byte projection).  The grouped MFMA
+        // path in transr.hip is the fast one; this is the fallback without relation groups.
+        const float *m = a.aux + rid * (int64_t)d * d;
+        float *x = lds + wave * d;
+        for (int i = lane; i < d; i += kWave) x[i] = MODEL == KGE_TRANSR ? eh[i] - et[i] : eh[i];
+        __syncthreads();
+        for (int j = lane * V; j < d; j += kWave * V) {
+            Vec<V> s;
+#pragma unroll
+            for (int e = 0; e < V; ++e) s.v[e] = 0.0f;
+            for (int i = 0; i < d; ++i) {
+                const float xi = x[i];
+                const Vec<V> vm = Vec<V>::load(m + (int64_t)i * d + j);
+#pragma unroll
+                for (int e = 0; e < V; ++e) s.v[e] += xi * vm.v[e];
+            }
+            if constexpr (MODEL == KGE_TRANSR) {
+                const Vec<V> vr = Vec<V>::load(rr + j);
+#pragma unroll
+                for (int e = 0; e < V; ++e) {
+                    s.v[e] += vr.v[e];
+                    acc += norm_term<P>(s.v[e]);
+                }
+                if (out && valid) s.store(out + j);
+            } else {
+                const Vec<V> vt = Vec<V>::load(et + j);
+#pragma unroll
+                for (int e = 0; e < V; ++e) acc += s.v[e] * vt.v[e];
+            }
+        }
+    } else if constexpr (MODEL == KGE_DISTMULT) {
+        for (int j = lane * V; j < d; j += kWave * V) {
+            const Vec<V> vh = Vec<V>::load(eh + j), vt = Vec<V>::load(et + j),
+                         vr = Vec<V>::load(rr + j);
+#pragma unroll
+            for (int e = 0; e < V; ++e) acc += (vh.v[e] * vr.v[e]) * vt.v[e];
+        }
+    } else if constexpr (MODEL == KGE_TRANSF) {
+        for (int j = lane * V; j < d; j += kWave * V) {
+            const Vec<V> vh = Vec<V>::load(eh + j), vt = Vec<V>::load(et + j),
+                         vr = Vec<V>::load(rr + j);
+#pragma unroll
+            for (int e = 0; e < V; ++e)
+                acc += (vh.v[e] + vr.v[e]) * vt.v[e] + (vt.v[e] - vr.v[e]) * vh.v[e];
+        }
+    } else if constexpr (MODEL == KGE_COMPLEX) {
+        const int half = d / 2;
+        for (int j = lane * V; j < half; j += kWave * V) {
+            const Vec<V> hr = Vec<V>::load(eh + j), hi = Vec<V>::load(eh + half + j);
+            const Vec<V> tr = Vec<V>::load(et + j), ti = Vec<V>::load(et + half + j);
+            const Vec<V> qr = Vec<V>::load(rr + j), qi = Vec<V>::load(rr + half + j);
+#pragma unroll
+            for (int e = 0; e < V; ++e) {
+                const float ar = hr.v[e] * qr.v[e] - hi.v[e] * qi.v[e];
+                const float ai = hr.v[e] * qi.v[e] + hi.v[e] * qr.v[e];
+                acc += ar * tr.v[e] + ai * ti.v[e];
+            }
+        }
+    } else if constexpr (MODEL == KGE_ROTATE) {
+        const int half = d / 2;
+        for (int j = lane * V; j < half; j += kWave * V) {
+            const Vec<V> hr = Vec<V>::load(eh + j), hi = Vec<V>::load(eh + half + j);
+            const Vec<V> tr = Vec<V>::load(et + j), ti = Vec<V>::load(et + half + j);
+            const Vec<V> th = Vec<V>::load(rr + j);
+#pragma unroll
+            for (int e = 0; e < V; ++e) {
+                float sn, c;
+                sincosf(th.v[e], &sn, &c);
+                const float ur = (hr.v[e] * c - hi.v[e] * sn) - tr.v[e];
+                const float ui = (hr.v[e] * sn + hi.v[e] * c) - ti.v[e];
+                acc += sqrtf(ur * ur + ui * ui);
+            }
+        }
+    }
+
+    acc = wave_sum(acc);
+    if (a.pos && valid && lane == 0) {
+        float s = acc;
+        if constexpr (MODEL == KGE_TRANSE || MODEL == KGE_TRANSH || MODEL == KGE_TRANSR)
+            s = P == 2 ? sqrtf(acc) : acc;
+        if constexpr (MODEL == KGE_ROTATE) s = a.gamma - acc;
+        a.pos[b] = s;
+    }
+}
+
+template <int MODEL, int P>
+static int launch_pos_v(const PosArgs &a, bool vec4, hipStream_t st)
+{
+    const dim3 grid((unsigned)ceil_div(a.B, kPosWaves)), block(kPosWaves * kWave);
+    const size_t lds =
+        (MODEL == KGE_TRANSR || MODEL == KGE_RESCAL) ? sizeof(float) * kPosWaves * (size_t)a.d : 0;
+    if (vec4)
+        hipLaunchKernelGGL((score_pos_kernel<MODEL, P, 4>), grid, block, lds, st, a);
+    else
+        hipLaunchKernelGGL((score_pos_kernel<MODEL, P, 1>), grid, block, lds, st, a);
+    KGE_CHECK_LAUNCH();
+    return KGE_OK;
+}
+
+// Dispatch on model / norm / vector width.  vec4 needs every row start and the
+// re|im split to sit on a 16-byte boundary.
+int launch_score_pos(const kge_tables *tab, const kge_batch *bat, float *pos, float *resid,
+                     float *side_pos, hipStream_t st)
+{
+    if (bat->batch == 0) return KGE_OK;
+    PosArgs a{tab->ent, tab->rel,      tab->aux,          bat->h,     bat->r, bat->t, bat->batch,
+              (int)tab->dim, (int)tab->rel_dim, tab->gamma, pos, resid, side_pos};
+    const bool complex_rows = tab->model == KGE_COMPLEX || tab->model == KGE_ROTATE;
+    const bool vec4 = tab->dim % (complex_rows ? 8 : 4) == 0 && aligned16(tab->ent) &&
+                      (!tab->rel || aligned16(tab->rel)) && (!tab->aux || aligned16(tab->aux)) &&
+                      (!resid || aligned16(resid));
+    const int p = tab->norm_p;
+    switch (tab->model) {
+    case KGE_TRANSE:
+        return p == 1 ? launch_pos_v<KGE_TRANSE, 1>(a, vec4, st) : launch_pos_v<KGE_TRANSE, 2>(a, vec4, st);
+    case KGE_TRANSH:
+        return p == 1 ? launch_pos_v<KGE_TRANSH, 1>(a, vec4, st) : launch_pos_v<KGE_TRANSH, 2>(a, vec4, st);
+    case KGE_TRANSR:
+        if ((size_t)tab->dim * kPosWaves * sizeof(float) > 64 * 1024) return KGE_EUNSUPPORTED;
+        return p == 1 ? launch_pos_v<KGE_TRANSR, 1>(a, vec4, st) : launch_pos_v<KGE_TRANSR, 2>(a, vec4, st);
+    case KGE_RESCAL:
+        if ((size_t)tab->dim * kPosWaves * sizeof(float) > 64 * 1024) return KGE_EUNSUPPORTED;
+        return launch_pos_v<KGE_RESCAL, 2>(a, vec4, st);
+    case KGE_DISTMULT: return launch_pos_v<KGE_DISTMULT, 2>(a, vec4, st);
+    case KGE_COMPLEX: return launch_pos_v<KGE_COMPLEX, 2>(a, vec4, st);
+    case KGE_ROTATE: return launch_pos_v<KGE_ROTATE, 2>(a, vec4, st);
+    case KGE_TRANSF: return launch_pos_v<KGE_TRANSF, 2>(a, vec4, st);
+    default: return KGE_EINVAL;
+    }
+}
+
+}  // namespace kge

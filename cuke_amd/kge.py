@@ -1,0 +1,343 @@
+"""Host side of the KGE score path: the reference's operator surface over the HIP library.
+
+The reference exposes each score function as a generated module whose single
+``run`` takes positional sizes, embedding tensors and index tensors
+(apps/kge/test_cuke.py:54,104,153,198,244) and returns a tensor; its inspector
+is ``inspector(r, rel_num)`` (apps/kge/kge.py:249-271).  ``transE`` ... ``RESCAL``
+and ``inspector`` below keep those names, argument orders and outputs.  On top of
+that :class:`KGEModel` offers what a training step needs and the reference does
+not have: scalar scores, shared negatives, and sparse row gradients.
+
+torch is used for device memory and streams only; every computation is a kernel
+of libkge_mi355.so reached through the C ABI.
+"""
+from __future__ import annotations
+
+import ctypes as C
+from dataclasses import dataclass
+
+import torch
+
+from . import _lib
+from ._lib import KgeError, MODELS
+
+__all__ = ["KGEModel", "Inspection", "Forward", "SparseGrads", "inspect", "inspector", "transE",
+           "transH", "transR", "transF", "RESCAL", "margin_loss", "KgeError"]
+
+
+def _stream() -> C.c_void_p:
+    return C.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def _ptr(t: torch.Tensor | None) -> C.c_void_p | None:
+    return None if t is None else C.c_void_p(t.data_ptr())
+
+
+def _table(x, name: str, ndim: int) -> torch.Tensor:
+    if not isinstance(x, torch.Tensor):
+        raise TypeError(f"{name} must be a torch.Tensor")
+    if not x.is_cuda:
+        raise KgeError(f"{name} must live on the GPU (got {x.device}); there is no CPU path")
+    if x.dtype != torch.float32:
+        raise TypeError(f"{name} must be float32 (got {x.dtype})")
+    if x.dim() != ndim:
+        raise ValueError(f"{name} must have {ndim} dimensions (got {x.dim()})")
+    return x.contiguous()
+
+
+def _index(x, name: str, device) -> torch.Tensor:
+    if not isinstance(x, torch.Tensor):
+        raise TypeError(f"{name} must be a torch.Tensor")
+    if x.dtype not in (torch.int64, torch.int32):
+        raise TypeError(f"{name} must be int64 or int32 (got {x.dtype})")
+    if x.dim() != 1:
+        raise ValueError(f"{name} must be one-dimensional")
+    return x.to(device=device, dtype=torch.int64).contiguous()
+
+
+@dataclass
+class Inspection:
+    """Sorted / deduplicated view of an index multiset (see kge_inspection in the C header)."""
+    n: int
+    n_rows: int
+    num_unique_dev: torch.Tensor  # int32[1]
+    unique_ids: torch.Tensor      # int64[n], first U valid
+    seg_offsets: torch.Tensor     # int32[n+1], first U+1 valid
+    perm: torch.Tensor            # int32[n]
+    inverse: torch.Tensor         # int32[n]
+    sorted_seg: torch.Tensor      # int32[n]
+    _c: _lib.Inspection = None
+    _u: int | None = None
+
+    @property
+    def num_unique(self) -> int:
+        """U (copies one int from the device the first time it is asked for)."""
+        if self._u is None:
+            self._u = int(self.num_unique_dev.item())
+        return self._u
+
+    def ids(self) -> torch.Tensor:
+        return self.unique_ids[: self.num_unique]
+
+    def offsets(self) -> torch.Tensor:
+        return self.seg_offsets[: self.num_unique + 1]
+
+
+def inspect(parts, n_rows: int) -> Inspection:
+    """Radix-sort and dedup the concatenation of up to four int64 index tensors."""
+    if isinstance(parts, torch.Tensor):
+        parts = [parts]
+    if not 1 <= len(parts) <= 4:
+        raise ValueError("inspect takes one to four index tensors")
+    dev = parts[0].device
+    parts = [_index(p, f"parts[{i}]", dev) for i, p in enumerate(parts)]
+    if not parts[0].is_cuda:
+        raise KgeError("inspect needs GPU tensors; there is no CPU path")
+    n = sum(int(p.numel()) for p in parts)
+    L = _lib.lib()
+    i32 = dict(dtype=torch.int32, device=dev)
+    ins = Inspection(n, int(n_rows), torch.zeros(1, **i32),
+                     torch.empty(max(n, 1), dtype=torch.int64, device=dev),
+                     torch.empty(n + 1, **i32), torch.empty(max(n, 1), **i32),
+                     torch.empty(max(n, 1), **i32), torch.empty(max(n, 1), **i32))
+    ins._c = _lib.Inspection(n, int(n_rows), ins.num_unique_dev.data_ptr(),
+                             ins.unique_ids.data_ptr(), ins.seg_offsets.data_ptr(),
+                             ins.perm.data_ptr(), ins.inverse.data_ptr(), ins.sorted_seg.data_ptr())
+    ws_bytes = int(L.kge_inspect_workspace(n, int(n_rows)))
+    ws = torch.empty(max(ws_bytes, 1), dtype=torch.uint8, device=dev)
+    ptrs = (C.c_void_p * len(parts))(*[p.data_ptr() for p in parts])
+    lens = (C.c_int64 * len(parts))(*[int(p.numel()) for p in parts])
+    _lib.check(L.kge_inspect(ptrs, lens, len(parts), int(n_rows), C.byref(ins._c),
+                             _ptr(ws), ws_bytes, _stream()), "kge_inspect")
+    ins._keep = (parts, ws)
+    return ins
+
+
+@dataclass
+class Forward:
+    """Scores plus what backward needs from the forward pass."""
+    pos: torch.Tensor | None
+    neg: torch.Tensor | None
+    side_pos: torch.Tensor | None = None
+    side_neg: torch.Tensor | None = None
+    residual: torch.Tensor | None = None
+    batch: tuple = ()
+    ent_insp: Inspection | None = None
+    rel_insp: Inspection | None = None
+
+
+@dataclass
+class SparseGrads:
+    """One gradient row per distinct table row that occurs in the batch; ids ascending."""
+    ent_ids: torch.Tensor
+    ent_rows: torch.Tensor
+    rel_ids: torch.Tensor
+    rel_rows: torch.Tensor | None
+    aux_rows: torch.Tensor | None
+
+
+class KGEModel:
+    """A KGE model = its name plus its embedding tables; methods score and differentiate batches.
+
+    model  one of TransE, TransH, TransR, DistMult, ComplEx, RotatE, TransF, RESCAL
+    Eemb   [n_ent, dim] float32 (ComplEx / RotatE rows are [re | im])
+    Remb   [n_rel, dim] float32 (RotatE: [n_rel, dim/2] phases; RESCAL: None)
+    aux    TransH: hyperplane normals [n_rel, dim] (the reference's Pemb);
+           TransR / RESCAL: projections [n_rel, dim, dim] (the reference's Proj)
+    """
+
+    def __init__(self, model: str, Eemb, Remb=None, aux=None, norm_p: int = 2, gamma: float = 0.0):
+        if model not in MODELS:
+            raise ValueError(f"unknown model {model!r}; expected one of {sorted(MODELS)}")
+        self.model = model
+        self.E = _table(Eemb, "Eemb", 2)
+        self.dev = self.E.device
+        self.dim = int(self.E.shape[1])
+        self.R = None if Remb is None else _table(Remb, "Remb", 2)
+        self.A = None
+        if model == "TransH":
+            self.A = _table(aux, "aux (hyperplane normals)", 2)
+        elif model in ("TransR", "RESCAL"):
+            self.A = _table(aux, "aux (projection matrices)", 3)
+        self.rel_dim = {"RotatE": self.dim // 2, "RESCAL": 0}.get(model, self.dim)
+        if self.rel_dim and self.R is None:
+            raise ValueError(f"{model} needs a relation table")
+        if self.R is not None and self.rel_dim and int(self.R.shape[1]) != self.rel_dim:
+            raise ValueError(f"Remb has row width {self.R.shape[1]}, {model} needs {self.rel_dim}")
+        self.n_rel = int(self.R.shape[0]) if self.R is not None and self.rel_dim else \
+            (int(self.A.shape[0]) if self.A is not None else 0)
+        if self.A is not None:
+            want = (self.n_rel, self.dim) if model == "TransH" else (self.n_rel, self.dim, self.dim)
+            if tuple(self.A.shape) != want:
+                raise ValueError(f"aux has shape {tuple(self.A.shape)}, {model} needs {want}")
+        self.norm_p, self.gamma = int(norm_p), float(gamma)
+        self._tab = _lib.Tables(MODELS[model], self.norm_p, self.gamma, 0, self.dim, self.rel_dim,
+                                int(self.E.shape[0]), self.n_rel, self.E.data_ptr(),
+                                self.R.data_ptr() if (self.R is not None and self.rel_dim) else None,
+                                self.A.data_ptr() if self.A is not None else None)
+
+    # -- helpers ---------------------------------------------------------------------------
+    def _batch(self, h, r, t, neg=None, chunk=None, ent_insp=None, rel_insp=None):
+        h, r, t = (_index(x, n, self.dev) for x, n in ((h, "h"), (r, "r"), (t, "t")))
+        B = int(h.numel())
+        if int(r.numel()) != B or int(t.numel()) != B:
+            raise ValueError("h, r, t must have the same length")
+        C_, N = 0, 0
+        if neg is not None:
+            neg = _index(neg.reshape(-1), "neg", self.dev)
+            C_ = int(chunk) if chunk else B
+            if C_ <= 0 or B % C_ != 0:
+                raise ValueError(f"batch {B} is not a whole number of chunks of {C_}")
+            n_chunks = B // C_
+            if n_chunks == 0 or int(neg.numel()) % n_chunks != 0:
+                raise ValueError("neg must hold the same number of tails for every chunk")
+            N = int(neg.numel()) // n_chunks
+        bat = _lib.Batch(B, h.data_ptr(), r.data_ptr(), t.data_ptr(),
+                         neg.data_ptr() if neg is not None else None, C_, N,
+                         C.pointer(ent_insp._c) if ent_insp is not None else None,
+                         C.pointer(rel_insp._c) if rel_insp is not None else None)
+        return bat, (h, r, t, neg, C_, N)
+
+    # -- reference-shaped output -------------------------------------------------------------
+    def residual(self, h, r, t, rel_insp: Inspection | None = None) -> torch.Tensor:
+        """[B, dim] residual vector: the reference's output for TransE / TransH / TransR."""
+        bat, keep = self._batch(h, r, t, rel_insp=rel_insp)
+        out = torch.empty((bat.batch, self.dim), dtype=torch.float32, device=self.dev)
+        _lib.check(_lib.lib().kge_residual_fwd(C.byref(self._tab), C.byref(bat), _ptr(out), _stream()),
+                   "kge_residual_fwd")
+        return out
+
+    # -- scalar scores ---------------------------------------------------------------------
+    def score(self, h, r, t, neg=None, chunk=None, ent_insp=None, rel_insp=None) -> Forward:
+        """pos[B] and, with shared negatives, neg[B, N] scores."""
+        bat, keep = self._batch(h, r, t, neg, chunk, ent_insp, rel_insp)
+        B, N = bat.batch, bat.n_neg
+        f32 = dict(dtype=torch.float32, device=self.dev)
+        fw = Forward(torch.empty(B, **f32), torch.empty((B, N), **f32) if neg is not None else None,
+                     batch=keep, ent_insp=ent_insp, rel_insp=rel_insp)
+        if self.model == "TransH":
+            fw.side_pos = torch.empty(B, **f32)
+            if neg is not None:
+                fw.side_neg = torch.empty((B, N), **f32)
+        if self.model == "TransR":
+            fw.residual = torch.empty((B, self.dim), **f32)
+        _lib.check(_lib.lib().kge_score_fwd(C.byref(self._tab), C.byref(bat), _ptr(fw.pos),
+                                            _ptr(fw.neg), _ptr(fw.side_pos), _ptr(fw.side_neg),
+                                            _ptr(fw.residual), _stream()), "kge_score_fwd")
+        return fw
+
+    def inspect_batch(self, h, r, t, neg=None):
+        """Inspections of concat(h, t, neg) over the entity table and of r over the relations."""
+        parts = [h, t] + ([neg.reshape(-1)] if neg is not None else [])
+        return inspect(parts, int(self.E.shape[0])), inspect([r], max(self.n_rel, 1))
+
+    # -- gradients ---------------------------------------------------------------------------
+    def backward(self, fw: Forward, dpos=None, dneg=None) -> SparseGrads:
+        """Sparse row gradients of sum(dpos * pos) + sum(dneg * neg)."""
+        h, r, t, neg, C_, N = fw.batch
+        if fw.ent_insp is None or fw.rel_insp is None:
+            fw.ent_insp, fw.rel_insp = self.inspect_batch(h, r, t, neg)
+        bat, _ = self._batch(h, r, t, neg, C_ or None, fw.ent_insp, fw.rel_insp)
+        B = bat.batch
+        f32 = dict(dtype=torch.float32, device=self.dev)
+        if dpos is not None:
+            dpos = dpos.to(**f32).contiguous()
+        if dneg is not None:
+            dneg = dneg.to(**f32).contiguous()
+        saved = _lib.Saved(*[(x.data_ptr() if x is not None else None) for x in
+                             (fw.pos, fw.neg, fw.side_pos, fw.side_neg, fw.residual)])
+        ent_rows = torch.empty((fw.ent_insp.n, self.dim), **f32)
+        rel_rows = torch.empty((B, self.rel_dim), **f32) if self.rel_dim else None
+        aux_rows = None
+        if self.model == "TransH":
+            aux_rows = torch.empty((B, self.dim), **f32)
+        elif self.model in ("TransR", "RESCAL"):
+            aux_rows = torch.empty((min(B, self.n_rel), self.dim * self.dim), **f32)
+        grads = _lib.Grads(_ptr(ent_rows), _ptr(rel_rows), _ptr(aux_rows))
+        L = _lib.lib()
+        ws_bytes = int(L.kge_score_bwd_workspace(C.byref(self._tab), C.byref(bat)))
+        ws = torch.empty(max(ws_bytes, 1), dtype=torch.uint8, device=self.dev)
+        _lib.check(L.kge_score_bwd(C.byref(self._tab), C.byref(bat), C.byref(saved), _ptr(dpos),
+                                   _ptr(dneg), C.byref(grads), _ptr(ws), ws_bytes, _stream()),
+                   "kge_score_bwd")
+        ue, ur = fw.ent_insp.num_unique, fw.rel_insp.num_unique
+        return SparseGrads(fw.ent_insp.ids(), ent_rows[:ue], fw.rel_insp.ids(),
+                           rel_rows[:ur] if rel_rows is not None else None,
+                           aux_rows[:ur] if aux_rows is not None else None)
+
+
+def margin_loss(pos: torch.Tensor, neg: torch.Tensor, margin: float, sign: float = 1.0):
+    """mean_{b,k} max(0, margin - sign * (pos[b] - neg[b, k])) and its gradients (loss, dpos, dneg)."""
+    B, N = neg.shape
+    L = _lib.lib()
+    loss = torch.empty(1, dtype=torch.float32, device=pos.device)
+    dpos, dneg = torch.empty_like(pos), torch.empty_like(neg)
+    ws_bytes = int(L.kge_margin_loss_workspace(B, N))
+    ws = torch.empty(max(ws_bytes, 1), dtype=torch.uint8, device=pos.device)
+    _lib.check(L.kge_margin_loss(_ptr(pos), _ptr(neg), B, N, float(margin), float(sign), _ptr(loss),
+                                 _ptr(dpos), _ptr(dneg), _ptr(ws), ws_bytes, _stream()),
+               "kge_margin_loss")
+    return loss, dpos, dneg
+
+
+# ---- the reference's positional call shapes --------------------------------------------------
+# run(batch_size, dim, nnodes, Eemb, h, t, nedges, Remb, r [, r_uniq, r_buf, r_cnt] [, extra])
+# The three inspector tensors are accepted and ignored: they only steer the reference kernel's
+# shared-memory relation cache and do not change the result.
+
+def _sizes_ok(batch_size, dim, Eemb, h):
+    if int(batch_size) != int(h.numel()):
+        raise ValueError(f"batch_size {batch_size} != len(h) {h.numel()}")
+    if int(dim) != int(Eemb.shape[1]):
+        raise ValueError(f"dim {dim} != Eemb row width {Eemb.shape[1]}")
+
+
+def transE(batch_size, dim, nnodes, Eemb, h, t, nedges, Remb, r, *reuse):
+    """apps/kge/test_cuke.py:54 -> [batch, dim] = (Eemb[h] - Eemb[t]) + Remb[r]."""
+    _sizes_ok(batch_size, dim, Eemb, h)
+    return KGEModel("TransE", Eemb, Remb).residual(h, r, t)
+
+
+def transH(batch_size, dim, nnodes, Eemb, h, t, nedges, Remb, r, *rest):
+    """apps/kge/test_cuke.py:104: (..., rel_ids, uniq, buf, cnt, projection_emb)."""
+    _sizes_ok(batch_size, dim, Eemb, h)
+    Pemb = rest[-1]
+    return KGEModel("TransH", Eemb, Remb, Pemb).residual(h, r, t)
+
+
+def transR(batch_size, dim, nnodes, Eemb, h, t, nedges, Proj, r, *rest):
+    """apps/kge/test_cuke.py:153: (batch, dim, 0, E, h, t, 0, Proj, r, uniq, buf, cnt, Remb)."""
+    _sizes_ok(batch_size, dim, Eemb, h)
+    Remb = rest[-1]
+    m = KGEModel("TransR", Eemb, Remb, Proj)
+    return m.residual(h, r, t, rel_insp=inspect([r], m.n_rel))
+
+
+def transF(batch_size, dim, nnodes, Eemb, h, nedges, Remb, r, *rest):
+    """apps/kge/test_cuke.py:198: (batch, dim, nnodes, E, h, nedges, R, r, uniq, buf, cnt, t) -> [batch]."""
+    _sizes_ok(batch_size, dim, Eemb, h)
+    t = rest[-1]
+    return KGEModel("TransF", Eemb, Remb).score(h, r, t).pos
+
+
+def RESCAL(batch_size, dim, nnodes, Eemb, h, nedges, Proj, r, *rest):
+    """apps/kge/test_cuke.py:244: (batch, dim, nnodes, E, h, nedges, Proj, r, uniq, buf, cnt, t) -> [batch]."""
+    _sizes_ok(batch_size, dim, Eemb, h)
+    t = rest[-1]
+    return KGEModel("RESCAL", Eemb, None, Proj).score(h, r, t).pos
+
+
+def inspector(r: torch.Tensor, rel_num: int, C_: int = 16):
+    """apps/kge/kge.py:249-271: (uniq[batch/16,16], buf[batch/16,16], cnt[batch/16]) int64 for sorted r."""
+    if C_ != 16:
+        raise ValueError("the reference's chunk size is fixed at 16 (inspector.cu:10)")
+    r = _index(r, "r", r.device)
+    if not r.is_cuda:
+        raise KgeError("inspector needs a GPU tensor; there is no CPU path")
+    nb = int(r.numel()) // 16
+    uniq = torch.zeros((nb, 16), dtype=torch.int64, device=r.device)
+    buf = torch.zeros((nb, 16), dtype=torch.int64, device=r.device)
+    cnt = torch.zeros((nb,), dtype=torch.int64, device=r.device)
+    _lib.check(_lib.lib().kge_build_index(_ptr(r), _ptr(uniq), _ptr(buf), _ptr(cnt), int(r.numel()),
+                                          int(rel_num), _stream()), "kge_build_index")
+    return uniq, buf, cnt

@@ -1,0 +1,199 @@
+/*
+ * kge_mi355 -- C ABI of the MI355X (gfx950) KGE score-function library.
+ *
+ * This is the boundary a host program binds instead of the reference's
+ * JIT-loaded pybind11 modules:
+ *   - pycuke1/run/gpu.py:4-20 + pycuke1/codegen/gpu_template.cu:8-17
+ *       module.run(batch, dim, nnodes, Eemb, h, t, nedges, Remb, r, ...) -> Tensor
+ *       (argument order per model: apps/kge/test_cuke.py:54,104,153,198,244)
+ *   - apps/kge/inspection/inspector.cu:139-147
+ *       gpu_sort(relation, r_Uniq, r_Buffer, uniq_cnt, batch, rel_num)
+ *
+ * Conventions
+ *   - every pointer is DEVICE memory unless its comment says "host";
+ *   - the library never allocates device memory: outputs and workspaces are
+ *     caller-allocated, workspace sizes come from the *_workspace() calls;
+ *   - `stream` is a hipStream_t passed as void*; calls only enqueue work and
+ *     never synchronise;
+ *   - return value: KGE_OK or a negative kge_status_t; kge_strerror() names it;
+ *   - tables are fp32 row-major with 16-byte aligned base pointers; index
+ *     arrays are int64 (the reference's GPU surface, pycuke1/codegen/gpu.py:200-201);
+ *   - entity rows of ComplEx / RotatE are stored [re(dim/2) | im(dim/2)];
+ *     RotatE relation rows are dim/2 phase angles.
+ */
+#ifndef KGE_MI355_H
+#define KGE_MI355_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef enum kge_model_t {
+    KGE_TRANSE = 0,   /* apps/kge/kge.py:273-293 */
+    KGE_TRANSH = 1,   /* apps/kge/kge.py:296-318 */
+    KGE_TRANSR = 2,   /* apps/kge/kge.py:321-343 */
+    KGE_DISTMULT = 3, /* not in the reference: s = sum h*r*t */
+    KGE_COMPLEX = 4,  /* not in the reference: s = Re<h, r, conj t> */
+    KGE_ROTATE = 5,   /* not in the reference: s = gamma - sum |h e^{i theta} - t| */
+    KGE_TRANSF = 6,   /* apps/kge/kge.py:346-366 */
+    KGE_RESCAL = 7    /* apps/kge/kge.py:369-390 */
+} kge_model_t;
+
+typedef enum kge_status_t {
+    KGE_OK = 0,
+    KGE_EINVAL = -1,       /* null pointer, bad enum, bad norm order */
+    KGE_ESHAPE = -2,       /* sizes inconsistent (batch % chunk, dim parity, alignment) */
+    KGE_ELAUNCH = -3,      /* hipGetLastError() reported a failed launch */
+    KGE_EWORKSPACE = -4,   /* workspace missing or too small */
+    KGE_EUNSUPPORTED = -5  /* combination not implemented */
+} kge_status_t;
+
+/* Embedding tables of one model. */
+typedef struct kge_tables {
+    int32_t model;     /* kge_model_t */
+    int32_t norm_p;    /* 1 or 2: norm of the TransE / TransH / TransR residual */
+    float gamma;       /* RotatE offset */
+    int32_t reserved;
+    int64_t dim;       /* floats per entity row */
+    int64_t rel_dim;   /* floats per relation row: dim, or dim/2 for RotatE, 0 for RESCAL */
+    int64_t n_ent;
+    int64_t n_rel;
+    const float *ent;  /* [n_ent, dim]                               (Eemb) */
+    const float *rel;  /* [n_rel, rel_dim]                           (Remb) */
+    const float *aux;  /* TransH normals [n_rel, dim] (Pemb); TransR / RESCAL
+                          projections [n_rel, dim, dim] (Proj); else NULL */
+} kge_tables;
+
+/*
+ * Result of inspecting one index multiset (kge_inspect).  For idx[n]:
+ *   unique_ids[0..U)   distinct ids, strictly ascending
+ *   seg_offsets[0..U]  sorted positions where each id's run starts; [U] = n
+ *   perm[n]            stable sort permutation: idx[perm[p]] ascending in p and
+ *                      perm ascending inside a run
+ *   inverse[n]         unique_ids[inverse[i]] == idx[i]
+ *   sorted_seg[n]      inverse[perm[p]]: the run each sorted position belongs to
+ *   num_unique[1]      U
+ * Positions are int32 (n < 2^31); ids stay int64.
+ */
+typedef struct kge_inspection {
+    int64_t n;
+    int64_t n_rows;
+    int32_t *num_unique;
+    int64_t *unique_ids;   /* capacity n */
+    int32_t *seg_offsets;  /* capacity n + 1 */
+    int32_t *perm;         /* capacity n */
+    int32_t *inverse;      /* capacity n */
+    int32_t *sorted_seg;   /* capacity n */
+} kge_inspection;
+
+/* One batch of triples.  neg == NULL: positives only. */
+typedef struct kge_batch {
+    int64_t batch;       /* B positives */
+    const int64_t *h;    /* [B] head entity ids */
+    const int64_t *r;    /* [B] relation ids */
+    const int64_t *t;    /* [B] tail entity ids */
+    const int64_t *neg;  /* [B / chunk * n_neg] shared negative tail ids, chunk-major */
+    int64_t chunk;       /* positives per chunk; B % chunk == 0 */
+    int64_t n_neg;       /* negatives per chunk: positive b is scored against
+                            neg[(b / chunk) * n_neg + k], k < n_neg
+                            (layout of apps/examples/examples.py:1404-1444) */
+    /* inspection of concat(h, t, neg) (entity table) and of r (relation tables);
+       needed by kge_score_bwd; rel_insp also by TransR forward */
+    const kge_inspection *ent_insp;
+    const kge_inspection *rel_insp;
+} kge_batch;
+
+/* Forward outputs that backward consumes. */
+typedef struct kge_saved {
+    const float *pos;       /* [B] positive scores */
+    const float *neg;       /* [B, n_neg] negative scores (NULL without negatives) */
+    const float *side_pos;  /* [B]: TransH w.h per positive; TransR: unused */
+    const float *side_neg;  /* [B, n_neg]: TransH w_b . t'_k per pair */
+    const float *residual;  /* [B, dim]: TransR residual rows */
+} kge_saved;
+
+/* Sparse row gradients: row u of each array belongs to the u-th unique id of the
+ * matching inspection (ent_insp for ent_rows, rel_insp for rel_rows / aux_rows). */
+typedef struct kge_grads {
+    float *ent_rows;  /* [ent_insp->n, dim]        first U_ent rows written */
+    float *rel_rows;  /* [B, rel_dim]              first U_rel rows written */
+    float *aux_rows;  /* TransH: [B, dim]; TransR / RESCAL: [min(B, n_rel), dim*dim] */
+} kge_grads;
+
+const char *kge_strerror(int status);
+int kge_abi_version(void);
+
+/*
+ * Residual vectors, the reference's output for TransE / TransH / TransR:
+ *   out[b][:] = (E[h]-E[t]) + R[r]                       (kge.py:290)
+ *             ... - (P[r].(E[h]-E[t])) P[r]              (kge.py:315)
+ *             = (E[h]-E[t]) Proj[r] + R[r]               (kge.py:340)
+ * Replaces module.run(...) of pycuke1/codegen/gpu_template.cu:8-13.
+ * out: [B, dim].  TransE is bit-exact with the generated CPU loop.
+ */
+int kge_residual_fwd(const kge_tables *tab, const kge_batch *bat, float *out, void *stream);
+
+/*
+ * Scalar scores.  pos[B]; neg[B, n_neg] when bat->neg is set (either may be
+ * NULL to skip).  side_pos / side_neg are optional save-for-backward outputs
+ * (see kge_saved; required later by kge_score_bwd for TransH).
+ * Scalar-score models of the reference: TransF / RESCAL (kge.py:363,387).
+ * TransR needs bat->rel_insp (relation groups) and `residual` [B, dim] scratch.
+ */
+int kge_score_fwd(const kge_tables *tab, const kge_batch *bat, float *pos, float *neg,
+                  float *side_pos, float *side_neg, float *residual, void *stream);
+
+/*
+ * Index inspector: radix sort + dedup of up to four concatenated int64 index
+ * arrays over a table of n_rows rows.  Stands where the reference calls
+ * inspector() / gpu_sort (apps/kge/kge.py:249-271, inspector.cu:139-143); its
+ * output is the full sorted/unique/segment structure rather than the
+ * reference's per-16 cache slots (for those see kge_build_index).
+ * parts / part_len are HOST arrays of n_parts device pointers / lengths.
+ */
+size_t kge_inspect_workspace(int64_t n, int64_t n_rows);
+int kge_inspect(const int64_t *const *parts, const int64_t *part_len, int n_parts,
+                int64_t n_rows, const kge_inspection *out, void *workspace,
+                size_t workspace_bytes, void *stream);
+
+/*
+ * Margin-ranking loss over score pairs and its gradient:
+ *   L = mean_{b,k} max(0, margin - sign * (pos[b] - neg[b][k]))
+ * loss[1], dpos[B], dneg[B, N].  workspace: kge_margin_loss_workspace(B, N) bytes.
+ */
+size_t kge_margin_loss_workspace(int64_t batch, int64_t n_neg);
+int kge_margin_loss(const float *pos, const float *neg, int64_t batch, int64_t n_neg,
+                    float margin, float sign, float *loss, float *dpos, float *dneg,
+                    void *workspace, size_t workspace_bytes, void *stream);
+
+/*
+ * Backward of kge_score_fwd: upstream dpos[B] (may be NULL = 0), dneg[B, n_neg]
+ * -> one gradient row per unique table row, written once, no atomics.
+ * The reference only prints per-triple dense gradient kernels
+ * (apps/kge/kge.py:393-515); this entry point is what a training step needs
+ * in their place.
+ */
+size_t kge_score_bwd_workspace(const kge_tables *tab, const kge_batch *bat);
+int kge_score_bwd(const kge_tables *tab, const kge_batch *bat, const kge_saved *saved,
+                  const float *dpos, const float *dneg, const kge_grads *grads,
+                  void *workspace, size_t workspace_bytes, void *stream);
+
+/*
+ * Chunk-of-16 relation cache index, same outputs as the reference's
+ * gpu_sort(relation, r_Uniq, r_Buffer, uniq_cnt, batch, rel_num)
+ * (apps/kge/inspection/inspector.cu:68-143): r[batch] sorted ascending,
+ * uniq[batch/16][16], buf[batch/16][16], cnt[batch/16] caller-zeroed int64.
+ */
+int kge_build_index(const int64_t *r, int64_t *uniq, int64_t *buf, int64_t *cnt, int64_t batch,
+                    int64_t rel_num, void *stream);
+
+/* Sets flag[0] (int32, caller-zeroed) to 1 if any idx[i] is outside [0, n_rows). */
+int kge_check_indices(const int64_t *idx, int64_t n, int64_t n_rows, int32_t *flag, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* KGE_MI355_H */

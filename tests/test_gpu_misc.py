@@ -1,0 +1,62 @@
+"""Margin loss and the reference-compatible chunk inspector on the GPU against the oracle."""
+import numpy as np
+import pytest
+import torch
+
+from helpers import assert_close
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+@pytest.mark.parametrize("B,N", [(64, 9), (1024, 256), (5, 1)])
+@pytest.mark.parametrize("sign", [1.0, -1.0])
+def test_margin_loss(oracle, B, N, sign):
+    from cuke_amd.kge import margin_loss
+    rng = np.random.default_rng(B + N)
+    pos = rng.standard_normal(B).astype(np.float32)
+    neg = rng.standard_normal((B, N)).astype(np.float32)
+    loss, dpos, dneg = margin_loss(torch.from_numpy(pos).to(DEV), torch.from_numpy(neg).to(DEV), 0.7, sign)
+    rl, rdp, rdn = oracle.margin_loss(pos, neg, 0.7, sign)
+    assert_close(loss.cpu().numpy(), np.array([rl], np.float32), what="loss")
+    assert_close(dpos.cpu().numpy(), rdp, what="dpos")
+    assert np.array_equal(dneg.cpu().numpy(), rdn)
+
+
+def test_build_index_matches_reference_restatement(oracle):
+    from cuke_amd.kge import inspector
+    rng = np.random.default_rng(5)
+    for rel_num, n in ((7, 16 * 64), (1345, 8192), (3, 16 * 10), (40, 16 * 33 + 5)):
+        r = np.sort(rng.integers(0, rel_num, n)).astype(np.int64)
+        uniq, buf, cnt = inspector(torch.from_numpy(r).to(DEV), rel_num)
+        ru, rb, rc, undefined = oracle.build_index(r, rel_num)
+        keep = np.ones(ru.shape[0], bool)
+        if undefined:  # chunks with 16 distinct ids have no defined result in the reference
+            keep = np.array([len(set(c)) < 16 for c in r[: ru.shape[0] * 16].reshape(-1, 16)])
+        assert np.array_equal(uniq.cpu().numpy()[keep], ru[keep])
+        assert np.array_equal(buf.cpu().numpy()[keep], rb[keep])
+        assert np.array_equal(cnt.cpu().numpy()[keep], rc[keep])
+
+
+def test_build_index_exhaustive_three_values(oracle):
+    from cuke_amd.kge import inspector
+    rows = [[0] * a + [1] * b + [2] * (16 - a - b) for a in range(17) for b in range(17 - a)]
+    r = np.array(rows, np.int64).reshape(-1)
+    uniq, buf, cnt = inspector(torch.from_numpy(r).to(DEV), 5)
+    ru, rb, rc, _ = oracle.build_index(r, 5)
+    assert np.array_equal(uniq.cpu().numpy(), ru)
+    assert np.array_equal(buf.cpu().numpy(), rb)
+    assert np.array_equal(cnt.cpu().numpy(), rc)
+
+
+def test_check_indices():
+    import ctypes as C
+    from cuke_amd import _lib
+    idx = torch.tensor([0, 5, 9], dtype=torch.int64, device=DEV)
+    flag = torch.zeros(1, dtype=torch.int32, device=DEV)
+    L = _lib.lib()
+    st = C.c_void_p(torch.cuda.current_stream().cuda_stream)
+    assert L.kge_check_indices(C.c_void_p(idx.data_ptr()), 3, 10, C.c_void_p(flag.data_ptr()), st) == 0
+    assert int(flag.item()) == 0
+    assert L.kge_check_indices(C.c_void_p(idx.data_ptr()), 3, 9, C.c_void_p(flag.data_ptr()), st) == 0
+    assert int(flag.item()) == 1
