@@ -1,10 +1,773 @@
-// Backward of the score path (placeholder entry points until the kernels land).
-#include "common.hpp"
-extern "C" {
-size_t kge_score_bwd_workspace(const kge_tables *, const kge_batch *) { return 0; }
-int kge_score_bwd(const kge_tables *, const kge_batch *, const kge_saved *, const float *, const float *,
-                  const kge_grads *, void *, size_t, void *)
+// Backward of the score path: per-occurrence gradient rows, then an atomic-free
+// segmented reduction to one row per distinct table row.
+//
+// The reference only prints per-triple dense gradient kernels (apps/kge/kge.py:393-515)
+// and never scatters or reduces them; the gradients here are derived from the forward
+// definitions (apps/kge/kge.py:273-390 and the DistMult / ComplEx / RotatE forms).
+//
+//   1. bwd_tile_kernel, owner = positives: G[b,:] = sum_k dneg[b,k] * d score(b,k) / d a_b
+//   2. bwd_tile_kernel, owner = negatives: gradient row of every negative occurrence
+//   3. bwd_pos_kernel: one wave per positive; chains G through a_b = f(h, r) and adds
+//      the positive triple's own term; writes the h / t / r (/ w) occurrence rows
+//   4. seg_reduce: occurrence rows are summed per distinct id in sorted order
+//      (inspection perm / seg_offsets); every output row is written exactly once.
+#include <stdlib.h>
+
+#include "tile_common.hpp"
+
+namespace kge {
+
+// ---------------------------------------------------------------------------------------
+// 1 + 2: tile kernel.  "Owners" keep their slice of the row in registers and accumulate
+// over all "loopers" of the chunk, which stream through LDS together with the
+// per-(owner, looper) coefficients.
+// ---------------------------------------------------------------------------------------
+struct TileArgs {
+    const float *ent, *rel, *aux;
+    const int64_t *h, *r, *neg;
+    const float *dneg;      // [B, N] upstream gradient
+    const float *sneg;      // [B, N] forward scores (L2 normalisation)
+    const float *side_pos;  // TransH: w.h per positive
+    const float *side_neg;  // TransH: [2, B, N]
+    float *out0, *out1;
+    int64_t plane;  // B * N
+    int C, N, d, rel_dim, vec, vecn;
+};
+
+constexpr int kTI = 64;       // columns of the row per workgroup
+constexpr int kKL = 32;       // looper rows staged per step
+constexpr int kLP = kTI + 4;  // LDS pitch of a staged row
+
+template <int MODEL, int P, bool OWNER_POS, int RO>
+__global__ __launch_bounds__(256) void bwd_tile_kernel(TileArgs a)
 {
-    return KGE_EUNSUPPORTED;
+    constexpr int TO = 16 * RO;
+    constexpr bool kRot = MODEL == KGE_ROTATE, kTH = MODEL == KGE_TRANSH;
+    constexpr bool kDot = MODEL == KGE_DISTMULT || MODEL == KGE_COMPLEX;
+    constexpr bool kL2 = (MODEL == KGE_TRANSE || kTH) && P == 2;
+    constexpr int NPL = (kRot || (kTH && !OWNER_POS)) ? 2 : 1;  // looper planes in LDS
+    constexpr int NPO = (kRot || (kTH && OWNER_POS)) ? 2 : 1;   // owner planes in registers
+    constexpr int NC = kTH ? 3 : 1;                             // coefficient planes: g~, c, e
+    constexpr int NOUT = (kRot || (kTH && OWNER_POS)) ? 2 : 1;
+    constexpr int PG = TO + 4;
+    constexpr int SL = kKL / 16;                        // looper float4 per thread per plane
+    constexpr int CPT = (TO * kKL / 4 + 255) / 256;     // coefficient float4 per thread per plane
+
+    __shared__ __align__(16) float sL[NPL][kKL][kLP];
+    __shared__ __align__(16) float sG[NC][kKL][PG];
+
+    const int tid = threadIdx.x, tx = tid & 15, ty = tid >> 4;
+    const int c = blockIdx.z;
+    const int d = a.d, half = d >> 1;
+    const int klen = pair_len<MODEL>(d);
+    const int col = blockIdx.x * kTI + tx * 4;
+    const int ot0 = blockIdx.y * TO;
+    const int n_own = OWNER_POS ? a.C : a.N, n_loop = OWNER_POS ? a.N : a.C;
+    const bool vec = a.vec != 0;
+
+    // ---- owners: registers -----------------------------------------------------------
+    float4 own[NPO][RO];
+    float alo[RO];
+#pragma unroll
+    for (int o = 0; o < RO; ++o) {
+        const int ol = ot0 + ty * RO + o;
+        const int lim = ol < n_own ? klen : 0;
+        const int oc = ol < n_own ? ol : n_own - 1;
+        alo[o] = 0.0f;
+        if constexpr (OWNER_POS) {
+            const int64_t b = (int64_t)c * a.C + oc;
+            const int64_t rid = a.r[b];
+            if constexpr (kTH) alo[o] = a.side_pos[b];
+            float4 q0 = zero4(), q1 = zero4();
+            if constexpr (!kDot)
+                load_query<MODEL>(a.ent + a.h[b] * (int64_t)d, a.rel + rid * (int64_t)a.rel_dim,
+                                  kTH ? a.aux + rid * (int64_t)d : nullptr, alo[o], col, lim, half, vec, q0,
+                                  q1);
+            own[0][o] = q0;
+            if constexpr (NPO == 2) own[1][o] = q1;
+        } else {
+            const float *pt = a.ent + a.neg[(int64_t)c * a.N + oc] * (int64_t)d;
+            own[0][o] = kDot ? zero4() : ld4(pt, col, lim, vec);
+            if constexpr (NPO == 2) own[1][o] = ld4(pt + half, col, lim, vec);
+        }
+    }
+
+    float4 acc[NOUT][RO];
+#pragma unroll
+    for (int q = 0; q < NOUT; ++q)
+#pragma unroll
+        for (int o = 0; o < RO; ++o) acc[q][o] = zero4();
+
+    // ---- staging registers -------------------------------------------------------------
+    float4 rl[NPL][SL];
+    float4 rc[NC][CPT];
+
+    auto load_step = [&](int l0) {
+        // looper rows: thread stages rows ty + 16*s, columns col..col+3
+#pragma unroll
+        for (int s = 0; s < SL; ++s) {
+            const int ll = l0 + ty + 16 * s;
+            const int lim = ll < n_loop ? klen : 0;
+            const int lc = ll < n_loop ? ll : n_loop - 1;
+            if constexpr (OWNER_POS) {
+                const float *pt = a.ent + a.neg[(int64_t)c * a.N + lc] * (int64_t)d;
+                rl[0][s] = ld4(pt, col, lim, vec);
+                if constexpr (NPL == 2) rl[1][s] = ld4(pt + half, col, lim, vec);
+            } else {
+                const int64_t b = (int64_t)c * a.C + lc;
+                const int64_t rid = a.r[b];
+                float4 q0, q1;
+                load_query<MODEL>(a.ent + a.h[b] * (int64_t)d, a.rel + rid * (int64_t)a.rel_dim,
+                                  kTH ? a.aux + rid * (int64_t)d : nullptr, kTH ? a.side_pos[b] : 0.0f, col,
+                                  lim, half, vec, q0, q1);
+                rl[0][s] = q0;
+                if constexpr (NPL == 2) rl[1][s] = q1;
+            }
+        }
+        // coefficients of the (TO owners x kKL loopers) block, read along k (contiguous)
+#pragma unroll
+        for (int s = 0; s < CPT; ++s) {
+            const int f = tid + 256 * s;  // float4 index inside the block
+            int bl, kl;                   // positive / negative of the first element
+            bool inside;
+            if constexpr (OWNER_POS) {    // rows = owners (positives), 8 float4 of loopers each
+                const int orow = f >> 3;
+                bl = ot0 + orow, kl = l0 + (f & 7) * 4;
+                inside = orow < TO && bl < a.C;
+            } else {                      // rows = loopers (positives), TO/4 float4 of owners each
+                const int lrow = f / (TO / 4);
+                bl = l0 + lrow, kl = ot0 + (f % (TO / 4)) * 4;
+                inside = lrow < kKL && bl < a.C;
+            }
+            const int lim = inside ? a.N : 0;
+            const int64_t off = ((int64_t)c * a.C + (inside ? bl : 0)) * a.N;
+            float4 g = ld4(a.dneg + off, kl, lim, a.vecn);
+            if constexpr (kL2) {
+                const float4 sc = ld4(a.sneg + off, kl, lim, a.vecn);
+                g.x = sc.x > 0.0f ? g.x / sc.x : 0.0f;
+                g.y = sc.y > 0.0f ? g.y / sc.y : 0.0f;
+                g.z = sc.z > 0.0f ? g.z / sc.z : 0.0f;
+                g.w = sc.w > 0.0f ? g.w / sc.w : 0.0f;
+            }
+            rc[0][s] = g;
+            if constexpr (kTH) {
+                const float4 graw = ld4(a.dneg + off, kl, lim, a.vecn);
+                rc[1][s] = ld4(a.side_neg + off, kl, lim, a.vecn);
+                rc[2][s] = mul4(graw, ld4(a.side_neg + a.plane + off, kl, lim, a.vecn));
+            }
+        }
+    };
+
+    auto store_step = [&]() {
+#pragma unroll
+        for (int s = 0; s < SL; ++s)
+#pragma unroll
+            for (int pl = 0; pl < NPL; ++pl)
+                *reinterpret_cast<float4 *>(&sL[pl][ty + 16 * s][tx * 4]) = rl[pl][s];
+#pragma unroll
+        for (int s = 0; s < CPT; ++s) {
+            const int f = tid + 256 * s;
+#pragma unroll
+            for (int pl = 0; pl < NC; ++pl) {
+                const float4 v = rc[pl][s];
+                if constexpr (OWNER_POS) {
+                    const int orow = f >> 3, l = (f & 7) * 4;
+                    if (orow < TO) {
+                        sG[pl][l + 0][orow] = v.x;
+                        sG[pl][l + 1][orow] = v.y;
+                        sG[pl][l + 2][orow] = v.z;
+                        sG[pl][l + 3][orow] = v.w;
+                    }
+                } else {
+                    const int lrow = f / (TO / 4), o4 = (f % (TO / 4)) * 4;
+                    if (lrow < kKL) *reinterpret_cast<float4 *>(&sG[pl][lrow][o4]) = v;
+                }
+            }
+        }
+    };
+
+    const int nstep = (n_loop + kKL - 1) / kKL;
+    load_step(0);
+#pragma unroll 1
+    for (int st = 0; st < nstep; ++st) {
+        store_step();
+        __syncthreads();
+        if (st + 1 < nstep) load_step((st + 1) * kKL);
+        // two-level sum: the kKL loopers of a step go into a fresh accumulator that is folded
+        // into the running one per step, so rounding grows with sqrt(steps) of the large partial
+        // sums instead of sqrt(loopers)
+        float4 sacc[NOUT][RO];
+#pragma unroll
+        for (int q = 0; q < NOUT; ++q)
+#pragma unroll
+            for (int o = 0; o < RO; ++o) sacc[q][o] = zero4();
+#pragma unroll 4
+        for (int l = 0; l < kKL; ++l) {
+            float4 lv[NPL];
+#pragma unroll
+            for (int pl = 0; pl < NPL; ++pl) lv[pl] = *reinterpret_cast<const float4 *>(&sL[pl][l][tx * 4]);
+#pragma unroll
+            for (int o = 0; o < RO; ++o) {
+                const float g = sG[0][l][ty * RO + o];
+                const float *lvp = reinterpret_cast<const float *>(&lv[0]);
+                const float *lv1p = reinterpret_cast<const float *>(&lv[NPL - 1]);
+                const float *o0p = reinterpret_cast<const float *>(&own[0][o]);
+                const float *o1p = reinterpret_cast<const float *>(&own[NPO - 1][o]);
+                float *a0p = reinterpret_cast<float *>(&sacc[0][o]);
+                float *a1p = reinterpret_cast<float *>(&sacc[NOUT - 1][o]);
+                if constexpr (kDot) {
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) a0p[e] = fmaf(g, lvp[e], a0p[e]);
+                } else if constexpr (MODEL == KGE_TRANSE) {
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        const float u = OWNER_POS ? o0p[e] - lvp[e] : lvp[e] - o0p[e];  // a - t'
+                        const float ph = P == 1 ? fast_sgn(u) : u;
+                        a0p[e] = OWNER_POS ? fmaf(g, ph, a0p[e]) : fmaf(-g, ph, a0p[e]);
+                    }
+                } else if constexpr (kRot) {
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        const float ur = OWNER_POS ? o0p[e] - lvp[e] : lvp[e] - o0p[e];
+                        const float ui = OWNER_POS ? o1p[e] - lv1p[e] : lv1p[e] - o1p[e];
+                        const float m2 = fmaf(ur, ur, ui * ui);
+                        const float rs = m2 > 0.0f ? __builtin_amdgcn_rsqf(m2) : 0.0f;
+                        const float k = OWNER_POS ? -g * rs : g * rs;  // d/da = -g u/|u| ; d/dt' = +g u/|u|
+                        a0p[e] = fmaf(k, ur, a0p[e]);
+                        a1p[e] = fmaf(k, ui, a1p[e]);
+                    }
+                } else if constexpr (kTH) {
+                    const float cc = sG[1][l][ty * RO + o], ee = sG[2][l][ty * RO + o];
+                    if constexpr (OWNER_POS) {
+                        const float sdk = alo[o] - cc;  // w.(h - t'_k)
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) {
+                            const float u = fmaf(cc, o1p[e], o0p[e] - lvp[e]);
+                            const float q = g * (P == 1 ? fast_sgn(u) : u);
+                            a0p[e] += q;
+                            a1p[e] = fmaf(ee, lvp[e], fmaf(-sdk, q, a1p[e]));
+                        }
+                    } else {
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) {
+                            const float u = fmaf(cc, lv1p[e], lvp[e] - o0p[e]);
+                            const float q = g * (P == 1 ? fast_sgn(u) : u);
+                            a0p[e] = fmaf(ee, lv1p[e], a0p[e] - q);
+                        }
+                    }
+                }
+            }
+        }
+#pragma unroll
+        for (int q = 0; q < NOUT; ++q)
+#pragma unroll
+            for (int o = 0; o < RO; ++o) acc[q][o] = add4(acc[q][o], sacc[q][o]);
+        __syncthreads();
+    }
+
+#pragma unroll
+    for (int o = 0; o < RO; ++o) {
+        const int ol = ot0 + ty * RO + o;
+        if (ol >= n_own) continue;
+        const int64_t row = OWNER_POS ? (int64_t)c * a.C + ol : (int64_t)c * a.N + ol;
+        float *dst = a.out0 + row * (int64_t)d;
+        st4(dst, col, klen, vec, acc[0][o]);
+        if constexpr (kRot) st4(dst + half, col, klen, vec, acc[1][o]);
+        if constexpr (kTH && OWNER_POS) st4(a.out1 + row * (int64_t)d, col, klen, vec, acc[1][o]);
+    }
 }
+
+template <int MODEL, int P, bool OWNER_POS>
+static int launch_tile_o(const TileArgs &a, int64_t n_chunks, hipStream_t st)
+{
+    const int n_own = OWNER_POS ? a.C : a.N;
+    const int klen = MODEL == KGE_ROTATE ? a.d / 2 : a.d;
+    const unsigned gx = (unsigned)ceil_div(klen, kTI);
+    const int64_t big = (int64_t)gx * ceil_div(n_own, 64) * n_chunks;
+    if (big >= 1024) {
+        hipLaunchKernelGGL((bwd_tile_kernel<MODEL, P, OWNER_POS, 4>),
+                           dim3(gx, (unsigned)ceil_div(n_own, 64), (unsigned)n_chunks), dim3(256), 0, st, a);
+    } else {
+        hipLaunchKernelGGL((bwd_tile_kernel<MODEL, P, OWNER_POS, 2>),
+                           dim3(gx, (unsigned)ceil_div(n_own, 32), (unsigned)n_chunks), dim3(256), 0, st, a);
+    }
+    KGE_CHECK_LAUNCH();
+    return KGE_OK;
 }
+
+template <int MODEL, int P>
+static int launch_tiles(TileArgs a, float *g0, float *g1, float *occ_neg, int64_t n_chunks, hipStream_t st)
+{
+    a.out0 = g0, a.out1 = g1;
+    int rc = launch_tile_o<MODEL, P, true>(a, n_chunks, st);
+    if (rc) return rc;
+    a.out0 = occ_neg, a.out1 = nullptr;
+    return launch_tile_o<MODEL, P, false>(a, n_chunks, st);
+}
+
+// ---------------------------------------------------------------------------------------
+// 3: one wave per positive triple
+// ---------------------------------------------------------------------------------------
+struct PosBwdArgs {
+    const float *ent, *rel, *aux;
+    const int64_t *h, *r, *t;
+    const float *dpos, *spos, *side_pos;
+    const float *g0, *g1;  // [B, d] accumulations over the negatives (may be null)
+    float *occ_h, *occ_t;  // [B, d] each
+    float *occ_r;          // [B, rel_dim]
+    float *occ_w;          // [B, d] TransH
+    int64_t B;
+    int d, rel_dim;
+};
+
+template <int V>
+__device__ __forceinline__ Vec<V> ldz(const float *p, int j)
+{
+    if (p) return Vec<V>::load(p + j);
+    Vec<V> z;
+#pragma unroll
+    for (int e = 0; e < V; ++e) z.v[e] = 0.0f;
+    return z;
+}
+
+template <int MODEL, int P, int V>
+__global__ __launch_bounds__(256) void bwd_pos_kernel(PosBwdArgs a)
+{
+    const int lane = threadIdx.x & (kWave - 1);
+    const int64_t b = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (b >= a.B) return;  // whole waves leave together; no block-level sync below
+    const int d = a.d, half = d >> 1;
+    const int64_t rid = a.r[b];
+    const float *eh = a.ent + a.h[b] * (int64_t)d, *et = a.ent + a.t[b] * (int64_t)d;
+    const float *rr = a.rel ? a.rel + rid * (int64_t)a.rel_dim : nullptr;
+    const float *g0 = a.g0 ? a.g0 + b * (int64_t)d : nullptr;
+    const float *g1 = a.g1 ? a.g1 + b * (int64_t)d : nullptr;
+    float *oh = a.occ_h + b * (int64_t)d, *ot = a.occ_t + b * (int64_t)d;
+    float *orr = a.occ_r ? a.occ_r + b * (int64_t)a.rel_dim : nullptr;
+    const float g = a.dpos ? a.dpos[b] : 0.0f;
+    float gs = g;  // g / ||u|| for the L2 models
+    if constexpr ((MODEL == KGE_TRANSE || MODEL == KGE_TRANSH) && P == 2) {
+        const float s = a.spos[b];
+        gs = s > 0.0f ? g / s : 0.0f;
+    }
+
+    if constexpr (MODEL == KGE_TRANSE) {
+        for (int j = lane * V; j < d; j += kWave * V) {
+            const Vec<V> vh = Vec<V>::load(eh + j), vt = Vec<V>::load(et + j), vr = Vec<V>::load(rr + j);
+            const Vec<V> G = ldz<V>(g0, j);
+            Vec<V> dh, dt;
+#pragma unroll
+            for (int e = 0; e < V; ++e) {
+                const float u = (vh.v[e] - vt.v[e]) + vr.v[e];
+                const float q = gs * (P == 1 ? sgn(u) : u);
+                dh.v[e] = q + G.v[e];
+                dt.v[e] = -q;
+            }
+            dh.store(oh + j), dh.store(orr + j), dt.store(ot + j);
+        }
+    } else if constexpr (MODEL == KGE_DISTMULT) {
+        for (int j = lane * V; j < d; j += kWave * V) {
+            const Vec<V> vh = Vec<V>::load(eh + j), vt = Vec<V>::load(et + j), vr = Vec<V>::load(rr + j);
+            const Vec<V> G = ldz<V>(g0, j);
+            Vec<V> dh, dr, dt;
+#pragma unroll
+            for (int e = 0; e < V; ++e) {
+                const float Q = fmaf(g, vt.v[e], G.v[e]);
+                dh.v[e] = vr.v[e] * Q;
+                dr.v[e] = vh.v[e] * Q;
+                dt.v[e] = g * (vh.v[e] * vr.v[e]);
+            }
+            dh.store(oh + j), dr.store(orr + j), dt.store(ot + j);
+        }
+    } else if constexpr (MODEL == KGE_TRANSF) {
+        for (int j = lane * V; j < d; j += kWave * V) {
+            const Vec<V> vh = Vec<V>::load(eh + j), vt = Vec<V>::load(et + j), vr = Vec<V>::load(rr + j);
+            Vec<V> dh, dr, dt;
+#pragma unroll
+            for (int e = 0; e < V; ++e) {
+                dh.v[e] = g * (2.0f * vt.v[e] - vr.v[e]);
+                dt.v[e] = g * (2.0f * vh.v[e] + vr.v[e]);
+                dr.v[e] = g * (vt.v[e] - vh.v[e]);
+            }
+            dh.store(oh + j), dr.store(orr + j), dt.store(ot + j);
+        }
+    } else if constexpr (MODEL == KGE_COMPLEX) {
+        for (int j = lane * V; j < half; j += kWave * V) {
+            const Vec<V> hr = Vec<V>::load(eh + j), hi = Vec<V>::load(eh + half + j);
+            const Vec<V> tr = Vec<V>::load(et + j), ti = Vec<V>::load(et + half + j);
+            const Vec<V> qr = Vec<V>::load(rr + j), qi = Vec<V>::load(rr + half + j);
+            const Vec<V> Gr = ldz<V>(g0, j), Gi = ldz<V>(g0, half + j);
+            Vec<V> dhr, dhi, drr, dri, dtr, dti;
+#pragma unroll
+            for (int e = 0; e < V; ++e) {
+                const float Qr = fmaf(g, tr.v[e], Gr.v[e]), Qi = fmaf(g, ti.v[e], Gi.v[e]);
+                dhr.v[e] = Qr * qr.v[e] + Qi * qi.v[e];
+                dhi.v[e] = Qi * qr.v[e] - Qr * qi.v[e];
+                drr.v[e] = Qr * hr.v[e] + Qi * hi.v[e];
+                dri.v[e] = Qi * hr.v[e] - Qr * hi.v[e];
+                dtr.v[e] = g * (hr.v[e] * qr.v[e] - hi.v[e] * qi.v[e]);
+                dti.v[e] = g * (hr.v[e] * qi.v[e] + hi.v[e] * qr.v[e]);
+            }
+            dhr.store(oh + j), dhi.store(oh + half + j);
+            drr.store(orr + j), dri.store(orr + half + j);
+            dtr.store(ot + j), dti.store(ot + half + j);
+        }
+    } else if constexpr (MODEL == KGE_ROTATE) {
+        for (int j = lane * V; j < half; j += kWave * V) {
+            const Vec<V> hr = Vec<V>::load(eh + j), hi = Vec<V>::load(eh + half + j);
+            const Vec<V> tr = Vec<V>::load(et + j), ti = Vec<V>::load(et + half + j);
+            const Vec<V> th = Vec<V>::load(rr + j);
+            const Vec<V> Gr = ldz<V>(g0, j), Gi = ldz<V>(g0, half + j);
+            Vec<V> dhr, dhi, dth, dtr, dti;
+#pragma unroll
+            for (int e = 0; e < V; ++e) {
+                float sn, cs;
+                sincosf(th.v[e], &sn, &cs);
+                const float ar = hr.v[e] * cs - hi.v[e] * sn, ai = hr.v[e] * sn + hi.v[e] * cs;
+                const float ur = ar - tr.v[e], ui = ai - ti.v[e];
+                const float m = sqrtf(ur * ur + ui * ui);
+                const float k = m > 0.0f ? -g / m : 0.0f;  // s = gamma - sum m
+                const float qpr = k * ur, qpi = k * ui;
+                const float Qr = qpr + Gr.v[e], Qi = qpi + Gi.v[e];
+                dhr.v[e] = Qr * cs + Qi * sn;
+                dhi.v[e] = Qi * cs - Qr * sn;
+                dth.v[e] = Qi * ar - Qr * ai;
+                dtr.v[e] = -qpr;
+                dti.v[e] = -qpi;
+            }
+            dhr.store(oh + j), dhi.store(oh + half + j);
+            dth.store(orr + j);
+            dtr.store(ot + j), dti.store(ot + half + j);
+        }
+    } else if constexpr (MODEL == KGE_TRANSH) {
+        const float *w = a.aux + rid * (int64_t)d;
+        float *ow = a.occ_w + b * (int64_t)d;
+        float sd = 0.0f;
+        for (int j = lane * V; j < d; j += kWave * V) {
+            const Vec<V> vh = Vec<V>::load(eh + j), vt = Vec<V>::load(et + j), vw = Vec<V>::load(w + j);
+#pragma unroll
+            for (int e = 0; e < V; ++e) sd += vw.v[e] * (vh.v[e] - vt.v[e]);
+        }
+        sd = wave_sum(sd);
+        float qw = 0.0f, gw = 0.0f;  // q_pos . w and G_q . w
+        for (int j = lane * V; j < d; j += kWave * V) {
+            const Vec<V> vh = Vec<V>::load(eh + j), vt = Vec<V>::load(et + j), vr = Vec<V>::load(rr + j),
+                         vw = Vec<V>::load(w + j);
+            const Vec<V> G = ldz<V>(g0, j);
+#pragma unroll
+            for (int e = 0; e < V; ++e) {
+                const float u = ((vh.v[e] - vt.v[e]) + vr.v[e]) - sd * vw.v[e];
+                const float q = gs * (P == 1 ? sgn(u) : u);
+                qw += q * vw.v[e];
+                gw += G.v[e] * vw.v[e];
+            }
+        }
+        qw = wave_sum(qw);
+        gw = wave_sum(gw);
+        for (int j = lane * V; j < d; j += kWave * V) {
+            const Vec<V> vh = Vec<V>::load(eh + j), vt = Vec<V>::load(et + j), vr = Vec<V>::load(rr + j),
+                         vw = Vec<V>::load(w + j);
+            const Vec<V> G = ldz<V>(g0, j), Gw = ldz<V>(g1, j);
+            Vec<V> dh, dt, dr, dw;
+#pragma unroll
+            for (int e = 0; e < V; ++e) {
+                const float d0 = vh.v[e] - vt.v[e];
+                const float u = (d0 + vr.v[e]) - sd * vw.v[e];
+                const float q = gs * (P == 1 ? sgn(u) : u);
+                const float Q = q + G.v[e];
+                dr.v[e] = Q;
+                dh.v[e] = Q - (qw + gw) * vw.v[e];
+                dt.v[e] = -(q - qw * vw.v[e]);
+                dw.v[e] = Gw.v[e] - (qw * d0 + sd * q) - gw * vh.v[e];
+            }
+            dh.store(oh + j), dt.store(ot + j), dr.store(orr + j), dw.store(ow + j);
+        }
+    }
+}
+
+template <int MODEL, int P>
+static int launch_pos_bwd(const PosBwdArgs &a, bool vec4, hipStream_t st)
+{
+    const dim3 grid((unsigned)ceil_div(a.B, 4)), block(256);
+    if (vec4) hipLaunchKernelGGL((bwd_pos_kernel<MODEL, P, 4>), grid, block, 0, st, a);
+    else hipLaunchKernelGGL((bwd_pos_kernel<MODEL, P, 1>), grid, block, 0, st, a);
+    KGE_CHECK_LAUNCH();
+    return KGE_OK;
+}
+
+// ---------------------------------------------------------------------------------------
+// 4: segmented reduction of occurrence rows in sorted order
+// ---------------------------------------------------------------------------------------
+constexpr int kSegL = 32;  // sorted positions per wave
+
+struct SegArgs {
+    const float *occ;  // [n, d]
+    const int32_t *perm, *sorted_seg, *seg_offsets;
+    int64_t n;
+    int d;
+    float *out;      // [U, d]
+    float *partial;  // [ceil(n / kSegL), 2, d]
+};
+
+// Level 1: wave j sums positions [j*L, (j+1)*L) run by run.  A run that lies wholly inside
+// the block is final and written to its output row; a run that started in an earlier block
+// goes to partial slot 0, one that continues into the next block to partial slot 1.
+template <int V>
+__global__ __launch_bounds__(256) void seg_reduce_l1(SegArgs a)
+{
+    const int lane = threadIdx.x & (kWave - 1);
+    const int64_t j = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    const int64_t p0 = j * kSegL;
+    if (p0 >= a.n) return;
+    const int cnt = (int)((a.n - p0) < kSegL ? (a.n - p0) : kSegL);
+    const int my_src = lane < cnt ? a.perm[p0 + lane] : 0;
+    const int my_seg = lane < cnt ? a.sorted_seg[p0 + lane] : -1;
+    const int d = a.d;
+
+    for (int c0 = 0; c0 < d; c0 += kWave * V) {
+        const int colv = c0 + lane * V;
+        const bool active = colv < d;
+        Vec<V> acc;
+#pragma unroll
+        for (int e = 0; e < V; ++e) acc.v[e] = 0.0f;
+        int cur = __shfl(my_seg, 0, kWave);
+
+        auto flush = [&](int seg) {
+            const int s0 = a.seg_offsets[seg], s1 = a.seg_offsets[seg + 1];
+            float *dst;
+            if (s0 >= p0 && s1 <= p0 + kSegL) dst = a.out + (int64_t)seg * d;
+            else dst = a.partial + (j * 2 + (s0 < p0 ? 0 : 1)) * (int64_t)d;
+            if (active) acc.store(dst + colv);
+        };
+
+        for (int q0 = 0; q0 < cnt; q0 += 8) {
+            Vec<V> v[8];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) {
+                const int q = q0 + u;
+                const int src = __shfl(my_src, q < cnt ? q : cnt - 1, kWave);
+                if (active && q < cnt) v[u] = Vec<V>::load(a.occ + (int64_t)src * d + colv);
+                else
+#pragma unroll
+                    for (int e = 0; e < V; ++e) v[u].v[e] = 0.0f;
+            }
+#pragma unroll
+            for (int u = 0; u < 8; ++u) {
+                const int q = q0 + u;
+                if (q < cnt) {
+                    const int sg = __shfl(my_seg, q, kWave);
+                    if (sg != cur) {
+                        flush(cur);
+#pragma unroll
+                        for (int e = 0; e < V; ++e) acc.v[e] = 0.0f;
+                        cur = sg;
+                    }
+#pragma unroll
+                    for (int e = 0; e < V; ++e) acc.v[e] += v[u].v[e];
+                }
+            }
+        }
+        flush(cur);
+    }
+}
+
+// Level 2: block j owns the run that starts inside it and continues past its end; it adds
+// that run's slot-1 partial and the slot-0 partials of the following blocks.
+template <int V>
+__global__ __launch_bounds__(256) void seg_reduce_l2(SegArgs a)
+{
+    const int lane = threadIdx.x & (kWave - 1);
+    const int64_t j = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    const int64_t p0 = j * kSegL;
+    if (p0 >= a.n) return;
+    const int64_t p1 = p0 + kSegL < a.n ? p0 + kSegL : a.n;
+    const int seg = a.sorted_seg[p1 - 1];
+    const int s0 = a.seg_offsets[seg], s1 = a.seg_offsets[seg + 1];
+    if (s1 <= p0 + kSegL || s0 < p0) return;
+    const int64_t je = (s1 - 1) / kSegL;
+    const int d = a.d;
+    for (int c0 = 0; c0 < d; c0 += kWave * V) {
+        const int colv = c0 + lane * V;
+        if (colv >= d) continue;
+        Vec<V> acc = Vec<V>::load(a.partial + (j * 2 + 1) * (int64_t)d + colv);
+        for (int64_t jj = j + 1; jj <= je; ++jj) {
+            const Vec<V> v = Vec<V>::load(a.partial + (jj * 2) * (int64_t)d + colv);
+#pragma unroll
+            for (int e = 0; e < V; ++e) acc.v[e] += v.v[e];
+        }
+        acc.store(a.out + (int64_t)seg * d + colv);
+    }
+}
+
+static int launch_seg_reduce(const float *occ, const kge_inspection *ins, int d, float *out, float *partial,
+                             hipStream_t st)
+{
+    if (ins->n == 0 || d == 0) return KGE_OK;
+    SegArgs a{occ, ins->perm, ins->sorted_seg, ins->seg_offsets, ins->n, d, out, partial};
+    const int64_t nblk = ceil_div(ins->n, kSegL);
+    const dim3 grid((unsigned)ceil_div(nblk, 4)), block(256);
+    const bool v4 = d % 4 == 0 && aligned16(occ) && aligned16(out) && aligned16(partial);
+    if (v4) {
+        hipLaunchKernelGGL(seg_reduce_l1<4>, grid, block, 0, st, a);
+        hipLaunchKernelGGL(seg_reduce_l2<4>, grid, block, 0, st, a);
+    } else {
+        hipLaunchKernelGGL(seg_reduce_l1<1>, grid, block, 0, st, a);
+        hipLaunchKernelGGL(seg_reduce_l2<1>, grid, block, 0, st, a);
+    }
+    KGE_CHECK_LAUNCH();
+    return KGE_OK;
+}
+
+__global__ void fill_zero_kernel(float *p, int64_t n)
+{
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (int64_t)gridDim.x * blockDim.x)
+        p[i] = 0.0f;
+}
+
+// ---------------------------------------------------------------------------------------
+struct BwdPlan {
+    int64_t n_occ, nn;
+    size_t off_occ_e, off_occ_r, off_occ_w, off_g0, off_g1, off_part_e, off_part_r, off_part_w, total;
+};
+
+static size_t up256(size_t x) { return (x + 255) & ~size_t(255); }
+
+static BwdPlan make_bwd_plan(const kge_tables *tab, const kge_batch *bat)
+{
+    BwdPlan p{};
+    const int64_t B = bat->batch, d = tab->dim, rd = tab->rel_dim;
+    p.nn = bat->neg ? (B / bat->chunk) * bat->n_neg : 0;
+    p.n_occ = 2 * B + p.nn;
+    size_t o = 0;
+    auto take = [&](int64_t floats) {
+        const size_t at = o;
+        o += up256(sizeof(float) * (size_t)(floats > 0 ? floats : 1));
+        return at;
+    };
+    p.off_occ_e = take(p.n_occ * d);
+    p.off_occ_r = take(B * rd);
+    p.off_occ_w = take(tab->model == KGE_TRANSH ? B * d : 0);
+    p.off_g0 = take(bat->neg ? B * d : 0);
+    p.off_g1 = take(bat->neg && tab->model == KGE_TRANSH ? B * d : 0);
+    p.off_part_e = take(ceil_div(p.n_occ, kSegL) * 2 * d);
+    p.off_part_r = take(ceil_div(B, kSegL) * 2 * rd);
+    p.off_part_w = take(tab->model == KGE_TRANSH ? ceil_div(B, kSegL) * 2 * d : 0);
+    p.total = o;
+    return p;
+}
+
+int launch_transr_bwd(const kge_tables *, const kge_batch *, const kge_saved *, const float *,
+                      const kge_grads *, void *, size_t, hipStream_t);
+size_t transr_bwd_workspace(const kge_tables *, const kge_batch *);
+
+}  // namespace kge
+
+using namespace kge;
+
+extern "C" {
+
+size_t kge_score_bwd_workspace(const kge_tables *tab, const kge_batch *bat)
+{
+    if (!tab || !bat || bat->batch < 0 || tab->dim <= 0) return 0;
+    if (bat->neg && bat->chunk <= 0) return 0;
+    if (tab->model == KGE_TRANSR || tab->model == KGE_RESCAL) return transr_bwd_workspace(tab, bat);
+    return make_bwd_plan(tab, bat).total;
+}
+
+int kge_score_bwd(const kge_tables *tab, const kge_batch *bat, const kge_saved *saved, const float *dpos,
+                  const float *dneg, const kge_grads *grads, void *workspace, size_t workspace_bytes,
+                  void *stream)
+{
+    if (!tab || !bat || !saved || !grads || !tab->ent) return KGE_EINVAL;
+    if (bat->batch < 0 || tab->dim <= 0) return KGE_ESHAPE;
+    if (bat->batch == 0) return KGE_OK;
+    if (!bat->h || !bat->r || !bat->t || !bat->ent_insp || !bat->rel_insp || !grads->ent_rows) return KGE_EINVAL;
+    if (bat->neg && (bat->chunk <= 0 || bat->n_neg <= 0 || bat->batch % bat->chunk)) return KGE_ESHAPE;
+    hipStream_t st = as_stream(stream);
+    if (tab->model == KGE_TRANSR || tab->model == KGE_RESCAL)
+        return launch_transr_bwd(tab, bat, saved, dpos, grads, workspace, workspace_bytes, st);
+
+    const BwdPlan p = make_bwd_plan(tab, bat);
+    if (!workspace || workspace_bytes < p.total) return KGE_EWORKSPACE;
+    if (bat->ent_insp->n != p.n_occ || bat->rel_insp->n != bat->batch) return KGE_ESHAPE;
+    const int model = tab->model, P = tab->norm_p;
+    const bool normed = model == KGE_TRANSE || model == KGE_TRANSH;
+    if (normed && P != 1 && P != 2) return KGE_EINVAL;
+    if (tab->rel_dim > 0 && !grads->rel_rows) return KGE_EINVAL;
+    if (normed && P == 2 && dpos && !saved->pos) return KGE_EINVAL;
+    const bool have_neg = bat->neg && dneg;
+    if (have_neg) {
+        if (model == KGE_TRANSF) return KGE_EUNSUPPORTED;
+        if (normed && P == 2 && !saved->neg) return KGE_EINVAL;
+        if (model == KGE_TRANSH && (!saved->side_pos || !saved->side_neg)) return KGE_EINVAL;
+    }
+    if (model == KGE_TRANSH && !grads->aux_rows) return KGE_EINVAL;
+
+    const int64_t B = bat->batch, d = tab->dim;
+    char *ws = static_cast<char *>(workspace);
+    float *occ_e = reinterpret_cast<float *>(ws + p.off_occ_e);
+    float *occ_r = reinterpret_cast<float *>(ws + p.off_occ_r);
+    float *occ_w = reinterpret_cast<float *>(ws + p.off_occ_w);
+    float *g0 = have_neg ? reinterpret_cast<float *>(ws + p.off_g0) : nullptr;
+    float *g1 = have_neg && model == KGE_TRANSH ? reinterpret_cast<float *>(ws + p.off_g1) : nullptr;
+    const bool vec = rows_vectorizable(tab);
+    int rc = KGE_OK;
+
+    if (have_neg) {
+        const int64_t n_chunks = B / bat->chunk;
+        if (n_chunks > 65535) return KGE_ESHAPE;
+        const bool vecn = bat->n_neg % 4 == 0 && aligned16(dneg) && (!saved->neg || aligned16(saved->neg)) &&
+                          (!saved->side_neg || aligned16(saved->side_neg));
+        TileArgs a{tab->ent, tab->rel, tab->aux, bat->h, bat->r, bat->neg, dneg, saved->neg, saved->side_pos,
+                   saved->side_neg, nullptr, nullptr, B * bat->n_neg, (int)bat->chunk, (int)bat->n_neg, (int)d,
+                   (int)tab->rel_dim, vec ? 1 : 0, vecn ? 1 : 0};
+        float *occ_neg = occ_e + 2 * B * d;
+        switch (model) {
+        case KGE_TRANSE:
+            rc = P == 1 ? launch_tiles<KGE_TRANSE, 1>(a, g0, g1, occ_neg, n_chunks, st)
+                        : launch_tiles<KGE_TRANSE, 2>(a, g0, g1, occ_neg, n_chunks, st);
+            break;
+        case KGE_TRANSH:
+            rc = P == 1 ? launch_tiles<KGE_TRANSH, 1>(a, g0, g1, occ_neg, n_chunks, st)
+                        : launch_tiles<KGE_TRANSH, 2>(a, g0, g1, occ_neg, n_chunks, st);
+            break;
+        case KGE_DISTMULT: rc = launch_tiles<KGE_DISTMULT, 2>(a, g0, g1, occ_neg, n_chunks, st); break;
+        case KGE_COMPLEX: rc = launch_tiles<KGE_COMPLEX, 2>(a, g0, g1, occ_neg, n_chunks, st); break;
+        case KGE_ROTATE: rc = launch_tiles<KGE_ROTATE, 2>(a, g0, g1, occ_neg, n_chunks, st); break;
+        default: return KGE_EUNSUPPORTED;
+        }
+        if (rc) return rc;
+    } else if (p.nn > 0) {
+        hipLaunchKernelGGL(fill_zero_kernel, dim3(1024), dim3(256), 0, st, occ_e + 2 * B * d, p.nn * d);
+    }
+
+    PosBwdArgs pa{tab->ent, tab->rel, tab->aux, bat->h, bat->r, bat->t, dpos, saved->pos, saved->side_pos,
+                  g0, g1, occ_e, occ_e + B * d, occ_r, occ_w, B, (int)d, (int)tab->rel_dim};
+    switch (model) {
+    case KGE_TRANSE:
+        rc = P == 1 ? launch_pos_bwd<KGE_TRANSE, 1>(pa, vec, st) : launch_pos_bwd<KGE_TRANSE, 2>(pa, vec, st);
+        break;
+    case KGE_TRANSH:
+        rc = P == 1 ? launch_pos_bwd<KGE_TRANSH, 1>(pa, vec, st) : launch_pos_bwd<KGE_TRANSH, 2>(pa, vec, st);
+        break;
+    case KGE_DISTMULT: rc = launch_pos_bwd<KGE_DISTMULT, 2>(pa, vec, st); break;
+    case KGE_COMPLEX: rc = launch_pos_bwd<KGE_COMPLEX, 2>(pa, vec, st); break;
+    case KGE_ROTATE: rc = launch_pos_bwd<KGE_ROTATE, 2>(pa, vec, st); break;
+    case KGE_TRANSF: rc = launch_pos_bwd<KGE_TRANSF, 2>(pa, vec, st); break;
+    default: return KGE_EUNSUPPORTED;
+    }
+    if (rc) return rc;
+
+    rc = launch_seg_reduce(occ_e, bat->ent_insp, (int)d, grads->ent_rows,
+                           reinterpret_cast<float *>(ws + p.off_part_e), st);
+    if (rc) return rc;
+    rc = launch_seg_reduce(occ_r, bat->rel_insp, (int)tab->rel_dim, grads->rel_rows,
+                           reinterpret_cast<float *>(ws + p.off_part_r), st);
+    if (rc) return rc;
+    if (model == KGE_TRANSH)
+        rc = launch_seg_reduce(occ_w, bat->rel_insp, (int)d, grads->aux_rows,
+                               reinterpret_cast<float *>(ws + p.off_part_w), st);
+    return rc;
+}
+
+}  // extern "C"

@@ -10,7 +10,7 @@
 // fp32 VALU; no matrix cores.
 #include <stdlib.h>
 
-#include "common.hpp"
+#include "tile_common.hpp"
 
 namespace kge {
 
@@ -19,7 +19,10 @@ struct NegArgs {
     const int64_t *h, *r, *neg;
     const float *side_pos;  // TransH: w_b . h_b
     float *out;             // [B, N]
-    float *side_neg;        // TransH: w_b . t'_k  [B, N] (optional)
+    float *side_neg;        // TransH save-for-backward [2, B, N] (optional):
+                            //   plane 0: c = w_b . t'_k ; plane 1: sum_i phi(u_i) w_i with
+                            //   phi = sign (L1) or u / ||u|| (L2)
+    int64_t plane;          // B * N
     int C, N, d, rel_dim;
     float gamma;
     int vec;
@@ -29,31 +32,10 @@ constexpr int kKD = 32;        // floats of each row staged per step
 constexpr int kLDW = kKD + 4;  // LDS row pitch: +4 floats keeps 128-bit reads of
                                // 8 consecutive rows on distinct banks
 
-__device__ __forceinline__ float4 ld4(const float *p, int j, int lim, bool vec)
-{
-    if (vec) return j < lim ? *reinterpret_cast<const float4 *>(p + j) : make_float4(0, 0, 0, 0);
-    float4 q;
-    q.x = j + 0 < lim ? p[j + 0] : 0.0f;
-    q.y = j + 1 < lim ? p[j + 1] : 0.0f;
-    q.z = j + 2 < lim ? p[j + 2] : 0.0f;
-    q.w = j + 3 < lim ? p[j + 3] : 0.0f;
-    return q;
-}
-
-__device__ __forceinline__ float4 zero4() { return make_float4(0.f, 0.f, 0.f, 0.f); }
-
-__device__ __forceinline__ float4 mul4(float4 p, float4 q)
-{
-    return make_float4(p.x * q.x, p.y * q.y, p.z * q.z, p.w * q.w);
-}
-__device__ __forceinline__ float4 add4(float4 p, float4 q)
-{
-    return make_float4(p.x + q.x, p.y + q.y, p.z + q.z, p.w + q.w);
-}
-
 // One element of the pair update, per model.
-template <int MODEL, int P>
-__device__ __forceinline__ void pair_elem(float &acc, float a0, float a1, float t0, float t1, float c)
+template <int MODEL, int P, bool SAVE>
+__device__ __forceinline__ void pair_elem(float &acc, float &acc2, float a0, float a1, float t0, float t1,
+                                          float c)
 {
     if constexpr (MODEL == KGE_DISTMULT || MODEL == KGE_COMPLEX) {
         acc = fmaf(a0, t0, acc);
@@ -66,13 +48,14 @@ __device__ __forceinline__ void pair_elem(float &acc, float a0, float a1, float 
         const float u = fmaf(c, a1, a0 - t0);
         if constexpr (P == 1) acc += fabsf(u);
         else acc = fmaf(u, u, acc);
+        if constexpr (SAVE) acc2 = fmaf(P == 1 ? fast_sgn(u) : u, a1, acc2);
     } else if constexpr (MODEL == KGE_ROTATE) {
         const float ur = a0 - t0, ui = a1 - t1;
         acc += __builtin_amdgcn_sqrtf(fmaf(ur, ur, ui * ui));
     }
 }
 
-template <int MODEL, int P, int RB, int RK>
+template <int MODEL, int P, int RB, int RK, bool SAVE>
 __global__ __launch_bounds__(256) void score_neg_kernel(NegArgs a)
 {
     constexpr int TB = 16 * RB, TN = 16 * RK;
@@ -120,66 +103,14 @@ __global__ __launch_bounds__(256) void score_neg_kernel(NegArgs a)
 
     auto load_slice = [&](int j0, int pass) {
         const int j = j0 + scol;
+        (void)pass;
 #pragma unroll
         for (int s = 0; s < SB; ++s) {
             const int lim = okb[s] ? klen : 0;
-            if constexpr (MODEL == KGE_DISTMULT) {
-                const float4 vh = ld4(ph[s], j, lim, vec), vr = ld4(pr[s], j, lim, vec);
-                ra[0][s] = mul4(vh, vr);
-            } else if constexpr (MODEL == KGE_TRANSE) {
-                const float4 vh = ld4(ph[s], j, lim, vec), vr = ld4(pr[s], j, lim, vec);
-                ra[0][s] = add4(vh, vr);
-            } else if constexpr (MODEL == KGE_COMPLEX) {
-                // flat index j over [re | im]: a_re = hr*rr - hi*ri, a_im = hr*ri + hi*rr
-                float q[4];
-                if (vec) {  // half % 4 == 0: the four elements sit on one side of the split
-                    const bool re = j < half;
-                    const int i = re ? j : j - half;
-                    const int l2 = lim ? half : 0;
-                    const float4 hr = ld4(ph[s], i, l2, true), hi = ld4(ph[s] + half, i, l2, true);
-                    const float4 rr = ld4(pr[s], i, l2, true), ri = ld4(pr[s] + half, i, l2, true);
-                    q[0] = re ? hr.x * rr.x - hi.x * ri.x : hr.x * ri.x + hi.x * rr.x;
-                    q[1] = re ? hr.y * rr.y - hi.y * ri.y : hr.y * ri.y + hi.y * rr.y;
-                    q[2] = re ? hr.z * rr.z - hi.z * ri.z : hr.z * ri.z + hi.z * rr.z;
-                    q[3] = re ? hr.w * rr.w - hi.w * ri.w : hr.w * ri.w + hi.w * rr.w;
-                } else
-#pragma unroll
-                for (int e = 0; e < 4; ++e) {
-                    const int jj = j + e;
-                    if (jj < lim) {
-                        const int i = jj < half ? jj : jj - half;
-                        const float hr = ph[s][i], hi = ph[s][i + half];
-                        const float rr = pr[s][i], ri = pr[s][i + half];
-                        q[e] = jj < half ? hr * rr - hi * ri : hr * ri + hi * rr;
-                    } else {
-                        q[e] = 0.0f;
-                    }
-                }
-                ra[0][s] = make_float4(q[0], q[1], q[2], q[3]);
-            } else if constexpr (MODEL == KGE_ROTATE) {
-                const float4 hr = ld4(ph[s], j, lim, vec), hi = ld4(ph[s] + half, j, lim, vec);
-                const float4 th = ld4(pr[s], j, lim, vec);
-                float4 sn, cs;
-                sincosf(th.x, &sn.x, &cs.x);
-                sincosf(th.y, &sn.y, &cs.y);
-                sincosf(th.z, &sn.z, &cs.z);
-                sincosf(th.w, &sn.w, &cs.w);
-                ra[0][s] = make_float4(hr.x * cs.x - hi.x * sn.x, hr.y * cs.y - hi.y * sn.y,
-                                       hr.z * cs.z - hi.z * sn.z, hr.w * cs.w - hi.w * sn.w);
-                ra[1][s] = make_float4(hr.x * sn.x + hi.x * cs.x, hr.y * sn.y + hi.y * cs.y,
-                                       hr.z * sn.z + hi.z * cs.z, hr.w * sn.w + hi.w * cs.w);
-            } else if constexpr (MODEL == KGE_TRANSH) {
-                const float4 vw = ld4(pw[s], j, lim, vec);
-                ra[1][s] = vw;
-                if (pass == 1) {
-                    const float4 vh = ld4(ph[s], j, lim, vec), vr = ld4(pr[s], j, lim, vec);
-                    const float al = pa[s];
-                    ra[0][s] = make_float4((vh.x + vr.x) - al * vw.x, (vh.y + vr.y) - al * vw.y,
-                                           (vh.z + vr.z) - al * vw.z, (vh.w + vr.w) - al * vw.w);
-                } else {
-                    ra[0][s] = zero4();
-                }
-            }
+            float4 q0, q1;
+            load_query<MODEL>(ph[s], pr[s], pw[s], pa[s], j, lim, half, vec, q0, q1);
+            ra[0][s] = q0;
+            if constexpr (NPA == 2) ra[1][s] = q1;
         }
 #pragma unroll
         for (int s = 0; s < SN; ++s) {
@@ -189,11 +120,11 @@ __global__ __launch_bounds__(256) void score_neg_kernel(NegArgs a)
         }
     };
 
-    float acc[RB][RK], cdot[RB][RK];
+    float acc[RB][RK], cdot[RB][RK], acc2[RB][RK];
 #pragma unroll
     for (int i = 0; i < RB; ++i)
 #pragma unroll
-        for (int k = 0; k < RK; ++k) acc[i][k] = 0.0f, cdot[i][k] = 0.0f;
+        for (int k = 0; k < RK; ++k) acc[i][k] = 0.0f, cdot[i][k] = 0.0f, acc2[i][k] = 0.0f;
 
     const int nslice = (klen + kKD - 1) / kKD;
 #pragma unroll 1
@@ -240,10 +171,10 @@ __global__ __launch_bounds__(256) void score_neg_kernel(NegArgs a)
                             cc = fmaf(a1.w, t0.w, cc);
                         } else {
                             const float cc = cdot[i][k];
-                            pair_elem<MODEL, P>(acc[i][k], a0.x, a1.x, t0.x, t1.x, cc);
-                            pair_elem<MODEL, P>(acc[i][k], a0.y, a1.y, t0.y, t1.y, cc);
-                            pair_elem<MODEL, P>(acc[i][k], a0.z, a1.z, t0.z, t1.z, cc);
-                            pair_elem<MODEL, P>(acc[i][k], a0.w, a1.w, t0.w, t1.w, cc);
+                            pair_elem<MODEL, P, SAVE>(acc[i][k], acc2[i][k], a0.x, a1.x, t0.x, t1.x, cc);
+                            pair_elem<MODEL, P, SAVE>(acc[i][k], acc2[i][k], a0.y, a1.y, t0.y, t1.y, cc);
+                            pair_elem<MODEL, P, SAVE>(acc[i][k], acc2[i][k], a0.z, a1.z, t0.z, t1.z, cc);
+                            pair_elem<MODEL, P, SAVE>(acc[i][k], acc2[i][k], a0.w, a1.w, t0.w, t1.w, cc);
                         }
                     }
             }
@@ -264,8 +195,10 @@ __global__ __launch_bounds__(256) void score_neg_kernel(NegArgs a)
             if constexpr (MODEL == KGE_TRANSE || MODEL == KGE_TRANSH) s = P == 2 ? sqrtf(s) : s;
             if constexpr (MODEL == KGE_ROTATE) s = a.gamma - s;
             a.out[rowoff + kl] = s;
-            if constexpr (MODEL == KGE_TRANSH)
-                if (a.side_neg) a.side_neg[rowoff + kl] = cdot[i][k];
+            if constexpr (MODEL == KGE_TRANSH && SAVE) {
+                a.side_neg[rowoff + kl] = cdot[i][k];
+                a.side_neg[a.plane + rowoff + kl] = P == 1 ? acc2[i][k] : (s > 0.0f ? acc2[i][k] / s : 0.0f);
+            }
         }
     }
 }
@@ -288,10 +221,16 @@ static int launch_neg_mp(const NegArgs &a, int64_t n_chunks, hipStream_t st)
     if (tile != 2 && tile != 4) tile = big_tiles >= 1024 ? 4 : 2;
     if (tile == 4) {
         const dim3 grid((unsigned)ceil_div(a.N, 64), (unsigned)ceil_div(a.C, 64), (unsigned)n_chunks);
-        hipLaunchKernelGGL((score_neg_kernel<MODEL, P, 4, 4>), grid, dim3(256), 0, st, a);
+        if (MODEL == KGE_TRANSH && a.side_neg)
+            hipLaunchKernelGGL((score_neg_kernel<MODEL, P, 4, 4, true>), grid, dim3(256), 0, st, a);
+        else
+            hipLaunchKernelGGL((score_neg_kernel<MODEL, P, 4, 4, false>), grid, dim3(256), 0, st, a);
     } else {
         const dim3 grid((unsigned)ceil_div(a.N, 32), (unsigned)ceil_div(a.C, 32), (unsigned)n_chunks);
-        hipLaunchKernelGGL((score_neg_kernel<MODEL, P, 2, 2>), grid, dim3(256), 0, st, a);
+        if (MODEL == KGE_TRANSH && a.side_neg)
+            hipLaunchKernelGGL((score_neg_kernel<MODEL, P, 2, 2, true>), grid, dim3(256), 0, st, a);
+        else
+            hipLaunchKernelGGL((score_neg_kernel<MODEL, P, 2, 2, false>), grid, dim3(256), 0, st, a);
     }
     KGE_CHECK_LAUNCH();
     return KGE_OK;
@@ -303,11 +242,9 @@ int launch_score_neg(const kge_tables *tab, const kge_batch *bat, const float *s
     if (bat->batch == 0) return KGE_OK;
     const int64_t n_chunks = bat->batch / bat->chunk;
     if (n_chunks > 65535 || bat->chunk >= (1 << 30) || bat->n_neg >= (1 << 30)) return KGE_ESHAPE;
-    const bool complex_rows = tab->model == KGE_COMPLEX || tab->model == KGE_ROTATE;
-    const bool vec = tab->dim % (complex_rows ? 8 : 4) == 0 && aligned16(tab->ent) &&
-                     aligned16(tab->rel) && (!tab->aux || aligned16(tab->aux));
+    const bool vec = rows_vectorizable(tab);
     NegArgs a{tab->ent, tab->rel, tab->aux, bat->h, bat->r, bat->neg, side_pos, out, side_neg,
-              (int)bat->chunk, (int)bat->n_neg, (int)tab->dim, (int)tab->rel_dim, tab->gamma, vec ? 1 : 0};
+              bat->batch * bat->n_neg, (int)bat->chunk, (int)bat->n_neg, (int)tab->dim, (int)tab->rel_dim, tab->gamma, vec ? 1 : 0};
     const int p = tab->norm_p;
     switch (tab->model) {
     case KGE_TRANSE:

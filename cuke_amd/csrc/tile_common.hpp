@@ -1,0 +1,127 @@
+// Pieces shared by the shared-negative tile kernels (forward and backward): guarded
+// 128-bit row loads and the per-model "query" row a_b = f(h_b, r_b) that is formed on
+// the fly while a tile is staged, so h and r are gathered inside the consuming kernel.
+#pragma once
+
+#include "common.hpp"
+
+namespace kge {
+
+__device__ __forceinline__ float4 ld4(const float *p, int j, int lim, bool vec)
+{
+    if (vec) return j < lim ? *reinterpret_cast<const float4 *>(p + j) : make_float4(0, 0, 0, 0);
+    float4 q;
+    q.x = j + 0 < lim ? p[j + 0] : 0.0f;
+    q.y = j + 1 < lim ? p[j + 1] : 0.0f;
+    q.z = j + 2 < lim ? p[j + 2] : 0.0f;
+    q.w = j + 3 < lim ? p[j + 3] : 0.0f;
+    return q;
+}
+
+__device__ __forceinline__ void st4(float *p, int j, int lim, bool vec, float4 v)
+{
+    if (vec) {
+        if (j < lim) *reinterpret_cast<float4 *>(p + j) = v;
+        return;
+    }
+    if (j + 0 < lim) p[j + 0] = v.x;
+    if (j + 1 < lim) p[j + 1] = v.y;
+    if (j + 2 < lim) p[j + 2] = v.z;
+    if (j + 3 < lim) p[j + 3] = v.w;
+}
+
+__device__ __forceinline__ float4 zero4() { return make_float4(0.f, 0.f, 0.f, 0.f); }
+__device__ __forceinline__ float4 mul4(float4 p, float4 q)
+{
+    return make_float4(p.x * q.x, p.y * q.y, p.z * q.z, p.w * q.w);
+}
+__device__ __forceinline__ float4 add4(float4 p, float4 q)
+{
+    return make_float4(p.x + q.x, p.y + q.y, p.z + q.z, p.w + q.w);
+}
+
+// sign(u) in two VALU ops: u * 2^100 clamped to [-1, 1] (exact 0 stays 0; |u| < 2^-100
+// would give a fraction, far below any fp32 residual that is not exactly zero)
+__device__ __forceinline__ float fast_sgn(float u)
+{
+    return __builtin_amdgcn_fmed3f(u * 0x1p100f, -1.0f, 1.0f);
+}
+
+// reduction length of the pair kernels: complex pairs for RotatE, floats otherwise
+template <int MODEL>
+__device__ __forceinline__ int pair_len(int d)
+{
+    return MODEL == KGE_ROTATE ? d >> 1 : d;
+}
+
+// Four consecutive elements (index j .. j+3 of the reduction axis) of the query row.
+//   DistMult  q0 = h*r                   ComplEx  q0 = (h o r) laid out [re | im]
+//   TransE    q0 = h+r                   RotatE   q0 = Re(h e^{i theta}), q1 = Im(...)
+//   TransH    q0 = h + r - al*w (al = w.h), q1 = w
+// lim == 0 yields zeros (row outside the tile).
+template <int MODEL>
+__device__ __forceinline__ void load_query(const float *ph, const float *pr, const float *pw, float al,
+                                           int j, int lim, int half, bool vec, float4 &q0, float4 &q1)
+{
+    q1 = zero4();
+    if constexpr (MODEL == KGE_DISTMULT) {
+        q0 = mul4(ld4(ph, j, lim, vec), ld4(pr, j, lim, vec));
+    } else if constexpr (MODEL == KGE_TRANSE) {
+        q0 = add4(ld4(ph, j, lim, vec), ld4(pr, j, lim, vec));
+    } else if constexpr (MODEL == KGE_COMPLEX) {
+        float q[4];
+        if (vec) {  // half % 4 == 0: the four elements sit on one side of the re|im split
+            const bool re = j < half;
+            const int i = re ? j : j - half;
+            const int l2 = lim ? half : 0;
+            const float4 hr = ld4(ph, i, l2, true), hi = ld4(ph + half, i, l2, true);
+            const float4 rr = ld4(pr, i, l2, true), ri = ld4(pr + half, i, l2, true);
+            q[0] = re ? hr.x * rr.x - hi.x * ri.x : hr.x * ri.x + hi.x * rr.x;
+            q[1] = re ? hr.y * rr.y - hi.y * ri.y : hr.y * ri.y + hi.y * rr.y;
+            q[2] = re ? hr.z * rr.z - hi.z * ri.z : hr.z * ri.z + hi.z * rr.z;
+            q[3] = re ? hr.w * rr.w - hi.w * ri.w : hr.w * ri.w + hi.w * rr.w;
+        } else {
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                const int jj = j + e;
+                if (jj < lim) {
+                    const int i = jj < half ? jj : jj - half;
+                    const float hr = ph[i], hi = ph[i + half], rr = pr[i], ri = pr[i + half];
+                    q[e] = jj < half ? hr * rr - hi * ri : hr * ri + hi * rr;
+                } else {
+                    q[e] = 0.0f;
+                }
+            }
+        }
+        q0 = make_float4(q[0], q[1], q[2], q[3]);
+    } else if constexpr (MODEL == KGE_ROTATE) {
+        const float4 hr = ld4(ph, j, lim, vec), hi = ld4(ph + half, j, lim, vec);
+        const float4 th = ld4(pr, j, lim, vec);
+        float4 sn, cs;
+        sincosf(th.x, &sn.x, &cs.x);
+        sincosf(th.y, &sn.y, &cs.y);
+        sincosf(th.z, &sn.z, &cs.z);
+        sincosf(th.w, &sn.w, &cs.w);
+        q0 = make_float4(hr.x * cs.x - hi.x * sn.x, hr.y * cs.y - hi.y * sn.y,
+                         hr.z * cs.z - hi.z * sn.z, hr.w * cs.w - hi.w * sn.w);
+        q1 = make_float4(hr.x * sn.x + hi.x * cs.x, hr.y * sn.y + hi.y * cs.y,
+                         hr.z * sn.z + hi.z * cs.z, hr.w * sn.w + hi.w * cs.w);
+    } else if constexpr (MODEL == KGE_TRANSH) {
+        const float4 vw = ld4(pw, j, lim, vec);
+        const float4 vh = ld4(ph, j, lim, vec), vr = ld4(pr, j, lim, vec);
+        q1 = vw;
+        q0 = make_float4((vh.x + vr.x) - al * vw.x, (vh.y + vr.y) - al * vw.y,
+                         (vh.z + vr.z) - al * vw.z, (vh.w + vr.w) - al * vw.w);
+    } else {
+        q0 = zero4();
+    }
+}
+
+inline bool rows_vectorizable(const kge_tables *tab)
+{
+    const bool complex_rows = tab->model == KGE_COMPLEX || tab->model == KGE_ROTATE;
+    return tab->dim % (complex_rows ? 8 : 4) == 0 && aligned16(tab->ent) &&
+           (!tab->rel || aligned16(tab->rel)) && (!tab->aux || aligned16(tab->aux));
+}
+
+}  // namespace kge

@@ -218,7 +218,7 @@ class KGEModel:
         if self.model == "TransH":
             fw.side_pos = torch.empty(B, **f32)
             if neg is not None:
-                fw.side_neg = torch.empty((B, N), **f32)
+                fw.side_neg = torch.empty((2, B, N), **f32)
         if self.model == "TransR":
             fw.residual = torch.empty((B, self.dim), **f32)
         _lib.check(_lib.lib().kge_score_fwd(C.byref(self._tab), C.byref(bat), _ptr(fw.pos),

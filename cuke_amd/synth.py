@@ -49,6 +49,7 @@ class Workload:
     rel_zipf: float = 0.0
     backward: bool = True
     loss: str = "sum"        # "sum": dL/dscore = 1 everywhere; "margin": margin-ranking loss
+    lattice: bool = False    # tables on a coarse binary grid: every residual is exact in fp32
     seed: int = 0
     arrays: dict = field(default_factory=dict)
 
@@ -115,6 +116,18 @@ def make_tables(w: Workload) -> None:
         a["A"] = wn
     elif w.model in ("TransR", "RESCAL"):
         a["A"] = rng.standard_normal((w.n_rel, w.dim, w.dim), dtype=np.float32) * np.float32(w.sigma)
+    if w.lattice:
+        # Multiples of 1/64 in [-1, 1] for E and R, of 1/4 for the TransH normals: sums and
+        # products of a few hundred such values fit in 24 bits, so translation-model residuals
+        # come out identical whatever the summation order or FMA use.  L1 gradients (a sum of
+        # signs of residual elements) can then be compared without sign flips at |u| ~ 1 ulp.
+        def grid(x, step):
+            return (np.clip(np.rint(x / np.float32(w.sigma) / 3 / step) * step, -1, 1)).astype(np.float32)
+        a["E"] = grid(a["E"], 1 / 64)
+        if w.model != "RotatE":
+            a["R"] = grid(a["R"], 1 / 64)
+        if w.model == "TransH":
+            a["A"] = (np.clip(np.rint(a["A"] * 4 * 3), -4, 4) / 4).astype(np.float32)
 
 
 def make_workload(name: str, seed: int = 0, tables: bool = True, **override) -> Workload:

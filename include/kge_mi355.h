@@ -111,7 +111,8 @@ typedef struct kge_saved {
     const float *pos;       /* [B] positive scores */
     const float *neg;       /* [B, n_neg] negative scores (NULL without negatives) */
     const float *side_pos;  /* [B]: TransH w.h per positive; TransR: unused */
-    const float *side_neg;  /* [B, n_neg]: TransH w_b . t'_k per pair */
+    const float *side_neg;  /* [2, B, n_neg]: TransH, plane 0 = w_b . t'_k per pair,
+                               plane 1 = sum_i phi(u_i) w_i (phi = sign for L1, u/||u|| for L2) */
     const float *residual;  /* [B, dim]: TransR residual rows */
 } kge_saved;
 

@@ -161,7 +161,9 @@ def backward(model, E, R, A, h, r, t, neg=None, chunk=0, dpos=None, dneg=None, p
         ctypes.c_int(MODELS[model]), ctypes.c_int(p), ctypes.c_int64(B), ctypes.c_int64(d),
         _fp(E), _fp(R), _fp(A), _fp(h), _fp(r), _fp(t), _fp(neg),
         ctypes.c_int64(C), ctypes.c_int64(N), _fp(dpos), _fp(dneg),
-        _fp(slot_h), _fp(slot_t), _fp(slot_n), _fp(slot_r), _fp(gE), _fp(gR), _fp(gA))
+        _fp(slot_h), _fp(slot_t), _fp(slot_n), _fp(slot_r),
+        ctypes.c_int64(gE.shape[0]), ctypes.c_int64(ins_r.unique_ids.shape[0]),
+        _fp(gE), _fp(gR), _fp(gA))
     assert rc == 0
     return SparseGrads(ins_e.unique_ids, gE, ins_r.unique_ids, gR, gA)
 

@@ -266,8 +266,11 @@ static void bwd_one(int model, int p, int64_t d, const float *eh, const float *r
         /* u = d0 + r - (w.d0) w ;  dL/dd0 = q - (q.w) w ;  dL/dw = -((q.w) d0 + (w.d0) q) */
         float sd = residual_transh(d, eh, rr, et, aux, u);
         lp_grad(p, d, u, g, q);
-        float qw = 0.0f;
-        for (int64_t j = 0; j < d; ++j) qw += q[j] * aux[j];
+        /* q.w enters every element of the row: a rounding error in it is coherent across the
+         * row and across the triples sharing w, so this scalar is reduced in double */
+        double qwd = 0.0;
+        for (int64_t j = 0; j < d; ++j) qwd += (double)q[j] * (double)aux[j];
+        const float qw = (float)qwd;
         for (int64_t i = 0; i < d; ++i) {
             float gi = q[i] - qw * aux[i];
             dh[i] += gi;
@@ -282,9 +285,9 @@ static void bwd_one(int model, int p, int64_t d, const float *eh, const float *r
         residual_transr(d, eh, rr, et, aux, u);
         lp_grad(p, d, u, g, q);
         for (int64_t i = 0; i < d; ++i) {
-            float acc = 0.0f;
-            for (int64_t j = 0; j < d; ++j) acc += aux[i * d + j] * q[j];
-            x[i] = acc;
+            double acc = 0.0;
+            for (int64_t j = 0; j < d; ++j) acc += (double)aux[i * d + j] * (double)q[j];
+            x[i] = (float)acc;
         }
         for (int64_t i = 0; i < d; ++i) {
             float d0 = eh[i] - et[i];
@@ -360,37 +363,64 @@ static void bwd_one(int model, int p, int64_t d, const float *eh, const float *r
  * Sparse row gradients.  Every occurrence of a row is mapped by the caller to
  * an output row ("slot", e.g. numpy.unique's inverse): slot_h[B], slot_t[B],
  * slot_neg[n_chunks*N] index gE[U_e, d]; slot_r[B] indexes gR[U_r, rel_width]
- * and gA[U_r, aux_width].  Outputs must be zero on entry.  Accumulation order:
- * b ascending; for each b the positive first, then k ascending.
+ * and gA[U_r, aux_width].
+ *
+ * Each triple's contribution is computed in fp32 as bwd_one states it (its inner
+ * contractions in double, rounded once);
+ * the sum ACROSS triples (up to ~10^6 terms for a hot row) is accumulated in
+ * double and rounded to fp32 once, so that the oracle stays a trustworthy
+ * reference for long sums (a serial fp32 sum of n terms drifts by ~sqrt(n)
+ * ulps of its partial sums, more than the parity bar for n > 10^4).
+ * Order: b ascending; for each b the positive first, then k ascending.
  */
+static void add_row(double *acc, const float *src, int64_t n)
+{
+    for (int64_t i = 0; i < n; ++i) acc[i] += (double)src[i];
+}
+
 int orc_backward(int model, int p, int64_t B, int64_t d, const float *E, const float *R,
                  const float *A, const int64_t *h, const int64_t *r, const int64_t *t,
                  const int64_t *neg, int64_t C, int64_t N, const float *dpos, const float *dneg,
                  const int64_t *slot_h, const int64_t *slot_t, const int64_t *slot_neg,
-                 const int64_t *slot_r, float *gE, float *gR, float *gA)
+                 const int64_t *slot_r, int64_t n_slots_e, int64_t n_slots_r, float *gE, float *gR,
+                 float *gA)
 {
     const int64_t rw = rel_width(model, d), aw = aux_width(model, d);
     float *tmp = (float *)malloc(sizeof(float) * (size_t)(3 * d + 1));
-    float *dummy = (float *)calloc((size_t)(d + 1), sizeof(float));
-    if (!tmp || !dummy) return -2;
+    float *one = (float *)malloc(sizeof(float) * (size_t)(3 * d + aw + 1)); /* dh | dr | dt | daux */
+    double *aE = (double *)calloc((size_t)(n_slots_e * d + 1), sizeof(double));
+    double *aR = (double *)calloc((size_t)(n_slots_r * rw + 1), sizeof(double));
+    double *aA = (double *)calloc((size_t)(n_slots_r * aw + 1), sizeof(double));
+    if (!tmp || !one || !aE || !aR || !aA) return -2;
+    float *dh = one, *dr = one + d, *dt = one + 2 * d, *da = one + 3 * d;
     for (int64_t b = 0; b < B; ++b) {
         const float *eh = E + h[b] * d, *rr = R ? R + r[b] * rw : NULL;
         const float *ax = A ? A + r[b] * aw : NULL;
-        float *dh = gE + slot_h[b] * d;
-        float *dr = gR ? gR + slot_r[b] * rw : dummy;
-        float *da = gA ? gA + slot_r[b] * aw : NULL;
-        if (dpos)
-            bwd_one(model, p, d, eh, rr, E + t[b] * d, ax, dpos[b], dh, dr, gE + slot_t[b] * d, da,
-                    tmp);
-        if (neg && dneg) {
-            const int64_t c = b / C;
-            for (int64_t k = 0; k < N; ++k)
-                bwd_one(model, p, d, eh, rr, E + neg[c * N + k] * d, ax, dneg[b * N + k], dh, dr,
-                        gE + slot_neg[c * N + k] * d, da, tmp);
+        const int64_t n_t = 1 + ((neg && dneg) ? N : 0);
+        const int64_t c = C > 0 ? b / C : 0;
+        for (int64_t q = 0; q < n_t; ++q) {
+            float g;
+            const float *et;
+            int64_t slot_tail;
+            if (q == 0) {
+                if (!dpos) continue;
+                g = dpos[b], et = E + t[b] * d, slot_tail = slot_t[b];
+            } else {
+                const int64_t k = q - 1;
+                g = dneg[b * N + k], et = E + neg[c * N + k] * d, slot_tail = slot_neg[c * N + k];
+            }
+            memset(one, 0, sizeof(float) * (size_t)(3 * d + aw));
+            bwd_one(model, p, d, eh, rr, et, ax, g, dh, dr, dt, da, tmp);
+            add_row(aE + slot_h[b] * d, dh, d);
+            add_row(aE + slot_tail * d, dt, d);
+            if (rw) add_row(aR + slot_r[b] * rw, dr, rw);
+            if (aw) add_row(aA + slot_r[b] * aw, da, aw);
         }
     }
-    free(tmp);
-    free(dummy);
+    for (int64_t i = 0; i < n_slots_e * d; ++i) gE[i] = (float)aE[i];
+    if (gR) for (int64_t i = 0; i < n_slots_r * rw; ++i) gR[i] = (float)aR[i];
+    if (gA) for (int64_t i = 0; i < n_slots_r * aw; ++i) gA[i] = (float)aA[i];
+    free(tmp); free(one); free(aE); free(aR); free(aA);
     return 0;
 }
 

@@ -6,19 +6,34 @@ import torch
 # absolute floor for entries that cancel to (nearly) zero: the oracle sums serially with
 # separate multiply and add, the GPU sums as a tree with fused multiply-add, and both are
 # fp32, so entries much smaller than the array's scale cannot agree to a pure relative bound.
+# For gradient rows (rows=True) the floor is taken per row: each row is its own sum over the
+# row's occurrences, and a hot row's scale is orders of magnitude above a cold row's.
 RTOL = 1e-5
 
 
-def assert_close(got, ref, rtol=RTOL, what=""):
+# RotatE gradients contain unit vectors u/|u| of complex differences u = h e^{i theta} - t.
+# Where |u| is ~10^-3 of the operands, the fp32 rounding of the rotated head (the oracle's
+# libm sin/cos and the GPU's differ in the last bit) is magnified by 1/|u| in BOTH
+# implementations, so a few elements per million legitimately differ by more than the bar.
+# `outliers=(fraction, factor)` admits at most that fraction of elements, each within
+# factor x the bound; it is only used by the RotatE gradient tests.
+def assert_close(got, ref, rtol=RTOL, what="", rows=False, outliers=None):
     got = np.asarray(got, np.float64)
     ref = np.asarray(ref, np.float64)
     assert got.shape == ref.shape, (what, got.shape, ref.shape)
     if ref.size == 0:
         return
-    rms = float(np.sqrt(np.mean(ref * ref)))
+    if rows:
+        rms = np.sqrt(np.mean(ref * ref, axis=-1, keepdims=True))
+    else:
+        rms = float(np.sqrt(np.mean(ref * ref)))
     err = np.abs(got - ref)
     bound = rtol * np.abs(ref) + rtol * rms
     bad = err > bound
+    if outliers is not None and bad.any():
+        frac, factor = outliers
+        if bad.mean() <= frac and not (err > factor * bound).any():
+            return
     if bad.any():
         i = np.unravel_index(np.argmax(err - bound), err.shape)
         raise AssertionError(f"{what}: {int(bad.sum())}/{ref.size} outside tolerance; worst at {i}: "
