@@ -1,0 +1,243 @@
+#!/usr/bin/env python3
+"""Benchmark of the KGE score path on one MI355X.
+
+A step is one pass over one batch of synthetic input with every table and index
+array already resident in HBM: index inspection (radix sort + dedup of the entity
+and relation ids) -> scores of the positives and of the shared negatives ->
+(margin loss) -> sparse row gradients.  Prints ONE JSON line.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload cfg2_distmult]
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0       # MI355X HBM3E, published
+FP32_PEAK_TFLOPS = 157.3    # MI355X fp32 vector / fp32 MFMA, published
+
+
+def device_tables(w, dev):
+    """Tables drawn on the GPU (seeded); benchmark-size tables are too large to push through numpy."""
+    import torch
+    g = torch.Generator(device=dev)
+    g.manual_seed(1000 + w.seed)
+    E = torch.randn((w.n_ent, w.dim), generator=g, device=dev, dtype=torch.float32) * w.sigma
+    if w.model == "RotatE":
+        R = (torch.rand((w.n_rel, w.rel_dim), generator=g, device=dev, dtype=torch.float32) * 2 - 1) * np.pi
+    else:
+        R = torch.randn((w.n_rel, w.rel_dim), generator=g, device=dev, dtype=torch.float32) * w.sigma
+    A = None
+    if w.model == "TransH":
+        A = torch.randn((w.n_rel, w.dim), generator=g, device=dev, dtype=torch.float32)
+        A = A / A.norm(dim=1, keepdim=True)
+    elif w.model in ("TransR", "RESCAL"):
+        A = torch.randn((w.n_rel, w.dim, w.dim), generator=g, device=dev, dtype=torch.float32) * w.sigma
+    return E, R, A
+
+
+def algorithmic_bytes(w, u_ent, u_rel):
+    """Bytes the step has to move by the problem statement alone: every gathered row once per
+    gather (h, r, t [, w] per positive; negatives once per chunk), 8 B per index, 4 B per score;
+    backward: 4 B per upstream score gradient, the same row reads again, one row write per
+    distinct row and 8 B per distinct id.  TransR: every distinct projection once per pass and
+    one dense d x d gradient per distinct relation."""
+    B, d, rd, N = w.batch, w.dim, w.rel_dim, w.n_neg
+    nn = w.n_chunks * N
+    aux_row = d if w.model == "TransH" else 0
+    rows = 4 * (B * (2 * d + rd + aux_row) + nn * d)
+    if w.model in ("TransR", "RESCAL"):
+        rows += 4 * u_rel * d * d
+    idx = 8 * (3 * B + nn)
+    scores = 4 * B * (1 + N)
+    fwd = rows + idx + scores
+    bwd = scores + rows + idx + 4 * (u_ent * d + u_rel * (rd + aux_row)) + 8 * (u_ent + u_rel)
+    if w.model in ("TransR", "RESCAL"):
+        bwd += 4 * u_rel * d * d
+    return fwd, bwd
+
+
+def neg_kernel_bytes(w):
+    """Algorithmic bytes of ONE launch of the shared-negative forward kernel: the h and r (and w)
+    rows of every positive, every negative row once per chunk, the indices, the scores out."""
+    B, d, rd, N = w.batch, w.dim, w.rel_dim, w.n_neg
+    nn = w.n_chunks * N
+    aux_row = d if w.model == "TransH" else 0
+    out_planes = 3 if w.model == "TransH" else 1
+    return 4 * (B * (d + rd + aux_row) + nn * d) + 8 * (2 * B + nn) + 4 * out_planes * B * N
+
+
+def neg_kernel_flops(w):
+    per_elem = {"DistMult": 2, "ComplEx": 2, "TransE": 2, "TransH": 9, "RotatE": 8}[w.model]
+    klen = w.dim // 2 if w.model == "RotatE" else w.dim
+    return per_elem * w.batch * w.n_neg * klen
+
+
+def time_events(fn, iters, torch):
+    """Average milliseconds per call of fn over `iters` back-to-back calls, by HIP events on the
+    stream the kernels are launched on (torch's current stream)."""
+    a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    torch.cuda.synchronize()
+    a.record()
+    for _ in range(iters):
+        fn()
+    b.record()
+    torch.cuda.synchronize()
+    return a.elapsed_time(b) / iters
+
+
+def cpu_baseline(w, budget_s=20.0):
+    """The oracle's serial loops (the restatement of cuke's generated CPU code) timed on this
+    host on one chunk-sized sample of the same workload: forward + backward, one thread."""
+    import oracle
+    from cuke_amd import synth
+    oracle.build()
+    n_ent = min(w.n_ent, 200_000)
+    batch = w.chunk if w.chunk else min(w.batch, 1024)
+    over = dict(n_ent=n_ent, batch=batch)
+    if w.model == "TransH" and w.n_neg > 256:  # keep the sample within the time budget
+        over.update(n_neg=256)
+    s = synth.make_workload(w.name, seed=w.seed, **over)
+    a = s.arrays
+    neg = a.get("neg")
+    t0 = time.perf_counter()
+    pos, negs = oracle.score(s.model, a["E"], a["R"], a["A"], a["h"], a["r"], a["t"], neg, s.chunk,
+                             p=s.norm_p, gamma=s.gamma, fast=True)
+    t_fwd = time.perf_counter() - t0
+    dpos = np.ones_like(pos)
+    dneg = np.ones_like(negs) if negs is not None else None
+    t0 = time.perf_counter()
+    if s.backward:
+        oracle.backward(s.model, a["E"], a["R"], a["A"], a["h"], a["r"], a["t"], neg, s.chunk, dpos, dneg,
+                        p=s.norm_p)
+    t_bwd = time.perf_counter() - t0
+    scores = s.scores_per_step
+    return {"value": scores / (t_fwd + t_bwd), "unit": "triples scored/s", "cores": 1, "kind": "port",
+            "sample": f"{s.model} B={s.batch} N={s.n_neg} dim={s.dim} n_ent={s.n_ent}: "
+                      f"fwd {t_fwd:.2f}s (gcc -O3, {oracle.threads()} OpenMP threads over the batch loop) "
+                      f"+ bwd {t_bwd:.2f}s (gcc -O2 serial)",
+            "fwd_s": t_fwd, "bwd_s": t_bwd}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--workload", default="cfg2_distmult")
+    ap.add_argument("--no-graph", action="store_true", help="launch kernels one by one instead of a HIP graph")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--seed", type=int, default=0)
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build runs on one GPU; --gpus must be 1 (nothing here shards across GPUs)",
+              file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+    from cuke_amd import synth
+    from cuke_amd.kge import KGEModel, TrainStep
+
+    dev = torch.device("cuda:0")
+    w = synth.make_workload(args.workload, seed=args.seed, tables=False)
+    E, R, A = device_tables(w, dev)
+    model = KGEModel(w.model, E, R, A, norm_p=w.norm_p, gamma=w.gamma)
+    ix = {k: torch.from_numpy(v).to(dev) for k, v in w.arrays.items() if v is not None}
+    sign = 1.0 if w.model in ("DistMult", "ComplEx", "RotatE", "TransF", "RESCAL") else -1.0
+    step = TrainStep(model, ix["h"], ix["r"], ix["t"], ix.get("neg"), w.chunk or None, loss=w.loss,
+                     margin=w.margin, sign=sign)
+    do_bwd = w.backward
+
+    use_graph = not args.no_graph
+    if use_graph:
+        step.capture(do_bwd)
+        one = step.replay
+    else:
+        one = lambda: step.run(do_bwd)
+
+    for _ in range(args.warmup):
+        one()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    ms = time_events(one, args.steps, torch)
+    wall = time.perf_counter() - t0
+
+    u_ent, u_rel = step.ent_insp.num_unique, step.rel_insp.num_unique
+    fwd_b, bwd_b = algorithmic_bytes(w, u_ent, u_rel)
+    total_b = fwd_b + (bwd_b if do_bwd else 0)
+    scores = w.scores_per_step
+
+    # per-stage times, un-graphed, each stage launched back to back
+    st = torch.cuda.current_stream().cuda_stream
+    import ctypes
+    stc = ctypes.c_void_p(st)
+    stages = {"inspect_ms": time_events(lambda: step.inspect(stc), 50, torch),
+              "forward_ms": time_events(lambda: step.forward(stc), 50, torch)}
+    if do_bwd:
+        stages["loss_ms"] = time_events(lambda: step.loss_grad(stc), 50, torch)
+        stages["backward_ms"] = time_events(lambda: step.backward(stc), 50, torch)
+
+    # dominant kernel in isolation: the shared-negative forward tile kernel (or, for
+    # positive-only workloads, the per-triple kernel), K launches between two events
+    from cuke_amd import _lib
+    L = _lib.lib()
+    if w.chunk:
+        def only_neg():
+            L.kge_score_fwd(ctypes.byref(model._tab), ctypes.byref(step.bat), None,
+                            ctypes.c_void_p(step.neg.data_ptr()),
+                            ctypes.c_void_p(step.side_pos.data_ptr()) if step.side_pos is not None else None,
+                            ctypes.c_void_p(step.side_neg.data_ptr()) if step.side_neg is not None else None,
+                            None, None, 0, stc)
+        kname = "score_neg_kernel"
+        if w.model == "TransH":  # needs w.h from the positive kernel; time the pair and subtract
+            t_pair = time_events(lambda: step.forward(stc), 100, torch)
+            t_pos = time_events(lambda: L.kge_score_fwd(ctypes.byref(model._tab), ctypes.byref(step.bat),
+                                                        ctypes.c_void_p(step.pos.data_ptr()), None,
+                                                        ctypes.c_void_p(step.side_pos.data_ptr()), None, None,
+                                                        None, 0, stc), 100, torch)
+            k_ms = t_pair - t_pos
+        else:
+            k_ms = time_events(only_neg, 100, torch)
+        k_bytes, k_flops = neg_kernel_bytes(w), neg_kernel_flops(w)
+    else:
+        kname = "score_pos_kernel" if w.model not in ("TransR",) else "transr_fwd_kernel"
+        k_ms = time_events(lambda: step.forward(stc), 100, torch)
+        k_bytes, k_flops = fwd_b, 0
+    achieved = k_bytes / (k_ms * 1e-3) / 1e9
+
+    out = {
+        "metric": "triples scored/sec fwd+bwd per KGE model; % of HBM (or MFMA) roofline",
+        "value": scores / (ms * 1e-3),
+        "unit": "triples scored/s",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": ms,
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32",
+        "data": "synthetic (seeded N(0,sigma) tables, Zipf/uniform indices, shared negatives per chunk)",
+        "config": {"workload": w.name, "model": w.model, "n_ent": w.n_ent, "n_rel": w.n_rel, "dim": w.dim,
+                   "batch": w.batch, "chunk": w.chunk, "n_neg": w.n_neg, "norm_p": w.norm_p,
+                   "backward": do_bwd, "loss": w.loss, "hip_graph": use_graph,
+                   "scores_per_step": scores, "positives_per_s": w.batch / (ms * 1e-3),
+                   "unique_entity_rows": u_ent, "unique_relation_rows": u_rel},
+        "step": {"algorithmic_bytes": total_b, "hbm_gbs": total_b / (ms * 1e-3) / 1e9,
+                 "hbm_frac": total_b / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, "wall_s": wall, **stages},
+        "roofline": {"kernel": kname, "bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": achieved / HBM_PEAK_GBS, "traffic": None, "kernel_ms": k_ms,
+                     "algorithmic_bytes_per_launch": k_bytes,
+                     "fp32_valu": {"flops_per_launch": k_flops,
+                                   "achieved_tflops": k_flops / (k_ms * 1e-3) / 1e12,
+                                   "frac_of_157.3": k_flops / (k_ms * 1e-3) / 1e12 / FP32_PEAK_TFLOPS}},
+    }
+    if not args.no_cpu:
+        out["cpu_baseline"] = cpu_baseline(w)
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

@@ -5,7 +5,8 @@ namespace kge {
 int launch_score_pos(const kge_tables *, const kge_batch *, float *, float *, float *, hipStream_t);
 int launch_score_neg(const kge_tables *, const kge_batch *, const float *, float *, float *,
                      hipStream_t);
-int launch_transr_fwd(const kge_tables *, const kge_batch *, float *, float *, hipStream_t);
+int launch_transr_fwd(const kge_tables *, const kge_batch *, float *, float *, void *, size_t, hipStream_t);
+size_t transr_fwd_workspace(const kge_tables *, const kge_batch *);
 
 __global__ void check_indices_kernel(const int64_t *idx, int64_t n, int64_t n_rows, int32_t *flag)
 {
@@ -63,7 +64,15 @@ const char *kge_strerror(int status)
 
 int kge_abi_version(void) { return 1; }
 
-int kge_residual_fwd(const kge_tables *tab, const kge_batch *bat, float *out, void *stream)
+size_t kge_score_fwd_workspace(const kge_tables *tab, const kge_batch *bat)
+{
+    if (!tab || !bat || bat->batch < 0) return 0;
+    if ((tab->model == KGE_TRANSR || tab->model == KGE_RESCAL) && bat->rel_insp) return transr_fwd_workspace(tab, bat);
+    return 0;
+}
+
+int kge_residual_fwd(const kge_tables *tab, const kge_batch *bat, float *out, void *workspace,
+                     size_t workspace_bytes, void *stream)
 {
     int rc = validate_tables(tab);
     if (rc) return rc;
@@ -72,12 +81,13 @@ int kge_residual_fwd(const kge_tables *tab, const kge_batch *bat, float *out, vo
     if (tab->model != KGE_TRANSE && tab->model != KGE_TRANSH && tab->model != KGE_TRANSR)
         return KGE_EUNSUPPORTED;  // the other models have scalar outputs only
     if (tab->model == KGE_TRANSR && bat->rel_insp)
-        return launch_transr_fwd(tab, bat, nullptr, out, as_stream(stream));
+        return launch_transr_fwd(tab, bat, nullptr, out, workspace, workspace_bytes, as_stream(stream));
     return launch_score_pos(tab, bat, nullptr, out, nullptr, as_stream(stream));
 }
 
 int kge_score_fwd(const kge_tables *tab, const kge_batch *bat, float *pos, float *neg,
-                  float *side_pos, float *side_neg, float *residual, void *stream)
+                  float *side_pos, float *side_neg, float *residual, void *workspace, size_t workspace_bytes,
+                  void *stream)
 {
     int rc = validate_tables(tab);
     if (rc) return rc;
@@ -86,8 +96,8 @@ int kge_score_fwd(const kge_tables *tab, const kge_batch *bat, float *pos, float
     const bool want_neg = neg && bat->neg;
     if (want_neg && tab->model == KGE_TRANSH && !side_pos) return KGE_EINVAL;
     if (pos || side_pos || residual) {
-        if (tab->model == KGE_TRANSR && bat->rel_insp)
-            rc = launch_transr_fwd(tab, bat, pos, residual, st);
+        if ((tab->model == KGE_TRANSR || tab->model == KGE_RESCAL) && bat->rel_insp)
+            rc = launch_transr_fwd(tab, bat, pos, residual, workspace, workspace_bytes, st);
         else
             rc = launch_score_pos(tab, bat, pos, residual, side_pos, st);
         if (rc) return rc;

@@ -520,7 +520,7 @@ __global__ __launch_bounds__(256) void seg_reduce_l1(SegArgs a)
     const int64_t p0 = j * kSegL;
     if (p0 >= a.n) return;
     const int cnt = (int)((a.n - p0) < kSegL ? (a.n - p0) : kSegL);
-    const int my_src = lane < cnt ? a.perm[p0 + lane] : 0;
+    const int my_src = lane < cnt ? (a.perm ? a.perm[p0 + lane] : (int)(p0 + lane)) : 0;
     const int my_seg = lane < cnt ? a.sorted_seg[p0 + lane] : -1;
     const int d = a.d;
 
@@ -599,11 +599,12 @@ __global__ __launch_bounds__(256) void seg_reduce_l2(SegArgs a)
     }
 }
 
-static int launch_seg_reduce(const float *occ, const kge_inspection *ins, int d, float *out, float *partial,
-                             hipStream_t st)
+// identity_perm: the occurrence rows are already stored in sorted order
+int launch_seg_reduce(const float *occ, const kge_inspection *ins, int d, float *out, float *partial,
+                      bool identity_perm, hipStream_t st)
 {
     if (ins->n == 0 || d == 0) return KGE_OK;
-    SegArgs a{occ, ins->perm, ins->sorted_seg, ins->seg_offsets, ins->n, d, out, partial};
+    SegArgs a{occ, identity_perm ? nullptr : ins->perm, ins->sorted_seg, ins->seg_offsets, ins->n, d, out, partial};
     const int64_t nblk = ceil_div(ins->n, kSegL);
     const dim3 grid((unsigned)ceil_div(nblk, 4)), block(256);
     const bool v4 = d % 4 == 0 && aligned16(occ) && aligned16(out) && aligned16(partial);
@@ -759,14 +760,14 @@ int kge_score_bwd(const kge_tables *tab, const kge_batch *bat, const kge_saved *
     if (rc) return rc;
 
     rc = launch_seg_reduce(occ_e, bat->ent_insp, (int)d, grads->ent_rows,
-                           reinterpret_cast<float *>(ws + p.off_part_e), st);
+                           reinterpret_cast<float *>(ws + p.off_part_e), false, st);
     if (rc) return rc;
     rc = launch_seg_reduce(occ_r, bat->rel_insp, (int)tab->rel_dim, grads->rel_rows,
-                           reinterpret_cast<float *>(ws + p.off_part_r), st);
+                           reinterpret_cast<float *>(ws + p.off_part_r), false, st);
     if (rc) return rc;
     if (model == KGE_TRANSH)
         rc = launch_seg_reduce(occ_w, bat->rel_insp, (int)d, grads->aux_rows,
-                               reinterpret_cast<float *>(ws + p.off_part_w), st);
+                               reinterpret_cast<float *>(ws + p.off_part_w), false, st);
     return rc;
 }
 

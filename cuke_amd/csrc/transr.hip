@@ -1,19 +1,514 @@
-// TransR grouped per-relation projection (placeholder: ungrouped per-triple path).
+// TransR / RESCAL: per-relation projections as grouped dense contractions on fp32 MFMA.
+//
+// The reference's kernel gives every triple its own vector x matrix product
+// (apps/kge/kge.py:321-343, bvm(vh - vt, Proj[r]) + vr; RESCAL kge.py:369-390) and re-reads
+// the 4*d*d-byte projection per triple.  Here the triples are grouped by relation (relation
+// inspection: sorted order + segment offsets) and every group is multiplied against its
+// projection once, 32 triples at a time, with v_mfma_f32_16x16x4_f32.
+//
+// MFMA operand layout (wave64, 16x16x4 fp32): lane l supplies A[i = l % 16][k = l / 16] and
+// B[k = l / 16][j = l % 16]; it receives D[i = 4 * (l / 16) + r][j = l % 16], r = 0..3.
+// Two re-labelings keep every memory access 128 bits wide:
+//   * k: inside a "superstep" of 16 consecutive k the MFMA step s (0..3) pairs lane group
+//     kk = l / 16 with k = 16 q + 4 kk + s, so a lane's A values for the four steps are one
+//     float4 of the staged row;
+//   * j: a lane's float4 of four consecutive matrix columns feeds four MFMAs (one per element),
+//     so MFMA e owns columns n0 + 4 (l % 16) + e.
 #include "common.hpp"
 
 namespace kge {
-int launch_score_pos(const kge_tables *, const kge_batch *, float *, float *, float *, hipStream_t);
-int launch_transr_fwd(const kge_tables *tab, const kge_batch *bat, float *pos, float *resid, hipStream_t st)
-{
-    return launch_score_pos(tab, bat, pos, resid, nullptr, st);
-}
-}  // namespace kge
 
-namespace kge {
-size_t transr_bwd_workspace(const kge_tables *, const kge_batch *) { return 0; }
-int launch_transr_bwd(const kge_tables *, const kge_batch *, const kge_saved *, const float *,
-                      const kge_grads *, void *, size_t, hipStream_t)
+typedef float floatx4 __attribute__((ext_vector_type(4)));
+
+constexpr int kTM = 32;          // triples per tile
+constexpr int kMaxDimMfma = 1024;
+
+int launch_score_pos(const kge_tables *, const kge_batch *, float *, float *, float *, hipStream_t);
+
+// ---- tile plan: one entry per (relation group, block of 32 sorted positions) ---------------
+struct TilePlan {
+    int32_t *num_tiles;  // [1]
+    int32_t *tile_seg;   // [max_tiles] group (unique-relation index)
+    int32_t *tile_p0;    // [max_tiles] first sorted position
+};
+
+__global__ __launch_bounds__(1024) void transr_plan_kernel(const int32_t *num_unique, const int32_t *seg_offsets,
+                                                          TilePlan plan)
 {
-    return KGE_EUNSUPPORTED;
+    __shared__ int s_scan[1024];
+    __shared__ int s_carry;
+    const int U = num_unique[0];
+    if (threadIdx.x == 0) s_carry = 0;
+    __syncthreads();
+    for (int base = 0; base < U; base += 1024) {
+        const int g = base + threadIdx.x;
+        int s0 = 0, cnt = 0;
+        if (g < U) {
+            s0 = seg_offsets[g];
+            cnt = (seg_offsets[g + 1] - s0 + kTM - 1) / kTM;
+        }
+        s_scan[threadIdx.x] = cnt;
+        __syncthreads();
+        for (int o = 1; o < 1024; o <<= 1) {  // Hillis-Steele inclusive scan
+            const int v = (int)threadIdx.x >= o ? s_scan[threadIdx.x - o] : 0;
+            __syncthreads();
+            s_scan[threadIdx.x] += v;
+            __syncthreads();
+        }
+        const int start = s_carry + s_scan[threadIdx.x] - cnt;
+        for (int q = 0; q < cnt; ++q) {
+            plan.tile_seg[start + q] = g;
+            plan.tile_p0[start + q] = s0 + q * kTM;
+        }
+        __syncthreads();
+        if (threadIdx.x == 1023) s_carry += s_scan[1023];
+        __syncthreads();
+    }
+    if (threadIdx.x == 0) plan.num_tiles[0] = s_carry;
 }
+
+// ---- grouped GEMM tile: Y[32 x d] = X[32 x d] * M (or * M^T) -----------------------------
+struct GemmArgs {
+    const float *ent, *rel, *proj;
+    const int64_t *h, *r, *t;
+    const int32_t *perm, *seg_offsets;
+    const int64_t *unique_ids;
+    TilePlan plan;
+    const float *xs;  // TRANSPOSED pass: left operand rows in sorted order [B, d]
+    float *pos;       // forward: [B] scores (nullable)
+    float *resid;     // forward: [B, d] rows y (nullable)
+    float *occ_h, *occ_t;  // backward-dX: [B, d] each (occ_t nullable)
+    int d, norm_p;
+};
+
+// MODE 0: forward TransR   x = E[h]-E[t], y = x M + R[r], score = ||y||_p
+// MODE 1: forward RESCAL   x = E[h],      y = x M,        score = y . E[t]
+// MODE 2: backward dX      x = xs rows,   y = x M^T -> occ_h = y, occ_t = -y (when occ_t is set)
+template <int MODE>
+__global__ __launch_bounds__(256) void transr_gemm_kernel(GemmArgs a)
+{
+    extern __shared__ __align__(16) float lds[];
+    const int tile = blockIdx.x;
+    if (tile >= a.plan.num_tiles[0]) return;
+    const int d = a.d;
+    const int kpad = (d + 15) & ~15;
+    const int pitch = kpad + 4;
+    float *sX = lds;                 // [kTM][pitch]
+    float *sRed = lds + kTM * pitch; // [4][kTM]
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int g = a.plan.tile_seg[tile], p0 = a.plan.tile_p0[tile];
+    const int seg_end = a.seg_offsets[g + 1];
+    const int rows = seg_end - p0 < kTM ? seg_end - p0 : kTM;
+    const int64_t rid = a.unique_ids[g];
+    const float *M = a.proj + rid * (int64_t)d * d;
+
+    // stage the left operand: 8 lanes per row, float4 along k
+    for (int f = tid; f < kTM * (kpad / 4); f += 256) {
+        const int row = f / (kpad / 4), k4 = (f % (kpad / 4)) * 4;
+        float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
+        if (row < rows && k4 < d) {
+            if constexpr (MODE == 2) {
+                v = *reinterpret_cast<const float4 *>(a.xs + (int64_t)(p0 + row) * d + k4);
+            } else {
+                const int b = a.perm[p0 + row];
+                v = *reinterpret_cast<const float4 *>(a.ent + a.h[b] * (int64_t)d + k4);
+                if constexpr (MODE == 0) {
+                    const float4 u = *reinterpret_cast<const float4 *>(a.ent + a.t[b] * (int64_t)d + k4);
+                    v = make_float4(v.x - u.x, v.y - u.y, v.z - u.z, v.w - u.w);
+                }
+            }
+        }
+        *reinterpret_cast<float4 *>(&sX[row * pitch + k4]) = v;
+    }
+    __syncthreads();
+
+    const int li = lane & 15, kk = lane >> 4;
+    const bool two_blocks = rows > 16;
+    float rowsum[8];  // norm / dot partials for rows 4*kk + r (+16)
+#pragma unroll
+    for (int r = 0; r < 8; ++r) rowsum[r] = 0.0f;
+
+    for (int c0 = 0; c0 < d; c0 += 256) {  // 256 output columns per sweep, split over the waves
+        const int span = d - c0 < 256 ? d - c0 : 256;
+        const int cw = ((span / 4 + 3) / 4) * 4;  // columns per wave, a multiple of 4
+        const int n0 = c0 + wave * cw;
+        const int wcols = n0 >= c0 + span ? 0 : (c0 + span - n0 < cw ? c0 + span - n0 : cw);
+        floatx4 acc_lo[4], acc_hi[4];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) acc_lo[e] = floatx4{0.f, 0.f, 0.f, 0.f}, acc_hi[e] = floatx4{0.f, 0.f, 0.f, 0.f};
+
+        if (wcols > 0) {
+            const int nq = kpad / 16;
+            if constexpr (MODE != 2) {
+                // B[k][j] = M[k][n0 + 4 li + e]: one float4 per (k) row per lane
+                const bool colok = 4 * li < wcols;
+                float4 bn[4];
+                auto loadb = [&](int q, float4 *dst) {
+#pragma unroll
+                    for (int s = 0; s < 4; ++s) {
+                        const int k = 16 * q + 4 * kk + s;
+                        dst[s] = (colok && k < d) ? *reinterpret_cast<const float4 *>(M + (int64_t)k * d + n0 + 4 * li)
+                                                  : make_float4(0.f, 0.f, 0.f, 0.f);
+                    }
+                };
+                loadb(0, bn);
+                for (int q = 0; q < nq; ++q) {
+                    float4 bc[4];
+#pragma unroll
+                    for (int s = 0; s < 4; ++s) bc[s] = bn[s];
+                    if (q + 1 < nq) loadb(q + 1, bn);
+                    const float4 alo = *reinterpret_cast<const float4 *>(&sX[li * pitch + 16 * q + 4 * kk]);
+                    const float4 ahi = *reinterpret_cast<const float4 *>(&sX[(16 + li) * pitch + 16 * q + 4 * kk]);
+                    const float al[4] = {alo.x, alo.y, alo.z, alo.w}, ah[4] = {ahi.x, ahi.y, ahi.z, ahi.w};
+#pragma unroll
+                    for (int s = 0; s < 4; ++s) {
+                        const float bv[4] = {bc[s].x, bc[s].y, bc[s].z, bc[s].w};
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) {
+                            acc_lo[e] = __builtin_amdgcn_mfma_f32_16x16x4f32(al[s], bv[e], acc_lo[e], 0, 0, 0);
+                            if (two_blocks)
+                                acc_hi[e] = __builtin_amdgcn_mfma_f32_16x16x4f32(ah[s], bv[e], acc_hi[e], 0, 0, 0);
+                        }
+                    }
+                }
+            } else {
+                // B[k][j] = M[j][k] (transposed): MFMA e owns output columns n0 + 16 e + li, and a
+                // lane's float4 along k of row (n0 + 16 e + li) serves the four steps
+                float4 bn[4];
+                auto loadb = [&](int q, float4 *dst) {
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        const int col = 16 * e + li, k = 16 * q + 4 * kk;
+                        dst[e] = (col < wcols && k < d)
+                                     ? *reinterpret_cast<const float4 *>(M + (int64_t)(n0 + col) * d + k)
+                                     : make_float4(0.f, 0.f, 0.f, 0.f);
+                    }
+                };
+                loadb(0, bn);
+                for (int q = 0; q < nq; ++q) {
+                    float4 bc[4];
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) bc[e] = bn[e];
+                    if (q + 1 < nq) loadb(q + 1, bn);
+                    const float4 alo = *reinterpret_cast<const float4 *>(&sX[li * pitch + 16 * q + 4 * kk]);
+                    const float4 ahi = *reinterpret_cast<const float4 *>(&sX[(16 + li) * pitch + 16 * q + 4 * kk]);
+                    const float al[4] = {alo.x, alo.y, alo.z, alo.w}, ah[4] = {ahi.x, ahi.y, ahi.z, ahi.w};
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        const float bv[4] = {bc[e].x, bc[e].y, bc[e].z, bc[e].w};
+#pragma unroll
+                        for (int s = 0; s < 4; ++s) {
+                            acc_lo[e] = __builtin_amdgcn_mfma_f32_16x16x4f32(al[s], bv[s], acc_lo[e], 0, 0, 0);
+                            if (two_blocks)
+                                acc_hi[e] = __builtin_amdgcn_mfma_f32_16x16x4f32(ah[s], bv[s], acc_hi[e], 0, 0, 0);
+                        }
+                    }
+                }
+            }
+        }
+
+        // epilogue for this sweep: lane holds rows 4 kk + r (and +16), columns per the mode
+#pragma unroll
+        for (int blk = 0; blk < 2; ++blk) {
+            if (blk == 1 && !two_blocks) break;
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const int row = 16 * blk + 4 * kk + r;
+                if (row >= rows) continue;
+                const int b = a.perm[p0 + row];
+                float y[4];
+#pragma unroll
+                for (int e = 0; e < 4; ++e) y[e] = blk ? acc_hi[e][r] : acc_lo[e][r];
+                if constexpr (MODE != 2) {
+                    const int col = n0 + 4 * li;  // y[e] is column col + e
+                    if (4 * li < wcols) {
+                        if constexpr (MODE == 0) {
+                            const float4 rv = *reinterpret_cast<const float4 *>(a.rel + rid * (int64_t)d + col);
+                            y[0] += rv.x, y[1] += rv.y, y[2] += rv.z, y[3] += rv.w;
+                            float s = 0.0f;
+#pragma unroll
+                            for (int e = 0; e < 4; ++e) s += a.norm_p == 1 ? fabsf(y[e]) : y[e] * y[e];
+                            rowsum[4 * blk + r] += s;
+                        } else {
+                            const float4 tv = *reinterpret_cast<const float4 *>(a.ent + a.t[b] * (int64_t)d + col);
+                            rowsum[4 * blk + r] += y[0] * tv.x + y[1] * tv.y + y[2] * tv.z + y[3] * tv.w;
+                        }
+                        if (a.resid)
+                            *reinterpret_cast<float4 *>(a.resid + (int64_t)b * d + col) =
+                                make_float4(y[0], y[1], y[2], y[3]);
+                    }
+                } else {
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        const int cl = 16 * e + li;
+                        if (cl < wcols) {
+                            a.occ_h[(int64_t)b * d + n0 + cl] = y[e];
+                            if (a.occ_t) a.occ_t[(int64_t)b * d + n0 + cl] = -y[e];
+                        }
+                    }
+                }
+            }
+        }
+    }
+
+    if constexpr (MODE != 2) {
+        if (a.pos) {
+            // row sums: over the 16 lanes that share kk, then over the four waves
+#pragma unroll
+            for (int r = 0; r < 8; ++r) {
+                float v = rowsum[r];
+                v += __shfl_xor(v, 1, kWave);
+                v += __shfl_xor(v, 2, kWave);
+                v += __shfl_xor(v, 4, kWave);
+                v += __shfl_xor(v, 8, kWave);
+                if (li == 0) sRed[wave * kTM + 16 * (r >> 2) + 4 * kk + (r & 3)] = v;
+            }
+            __syncthreads();
+            if (tid < rows) {
+                const float s = sRed[tid] + sRed[kTM + tid] + sRed[2 * kTM + tid] + sRed[3 * kTM + tid];
+                const int b = a.perm[p0 + tid];
+                a.pos[b] = (MODE == 0 && a.norm_p == 2) ? sqrtf(s) : s;
+            }
+        }
+    }
+}
+
+static size_t gemm_lds_bytes(int d)
+{
+    const int kpad = (d + 15) & ~15;
+    return sizeof(float) * ((size_t)kTM * (kpad + 4) + 4 * kTM);
+}
+
+static int64_t max_tiles(const kge_tables *tab, const kge_batch *bat)
+{
+    const int64_t groups = bat->batch < tab->n_rel ? bat->batch : tab->n_rel;
+    return groups + bat->batch / kTM + 1;
+}
+
+static bool mfma_path_ok(const kge_tables *tab, const kge_batch *bat)
+{
+    return bat->rel_insp && tab->dim % 4 == 0 && tab->dim <= kMaxDimMfma && aligned16(tab->ent) &&
+           aligned16(tab->aux) && (!tab->rel || aligned16(tab->rel)) && bat->rel_insp->n == bat->batch;
+}
+
+// ---- backward kernels ----------------------------------------------------------------------
+struct PrepArgs {
+    const float *ent;
+    const int64_t *h, *t;
+    const int32_t *perm;
+    const float *dpos, *spos, *resid;
+    float *xs, *qs;  // [B, d] in sorted order
+    float *occ_t;    // RESCAL: g * v
+    int64_t B;
+    int d, norm_p, rescal;
+};
+
+// One wave per sorted position p (triple b = perm[p]):
+//   TransR: xs[p] = E[h]-E[t], qs[p] = g * d||e||/de     RESCAL: xs[p] = E[h], qs[p] = g * E[t], occ_t[b] = g * v
+__global__ __launch_bounds__(256) void transr_prep_kernel(PrepArgs a)
+{
+    const int lane = threadIdx.x & 63;
+    const int64_t p = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (p >= a.B) return;
+    const int b = a.perm[p];
+    const int d = a.d;
+    const float g = a.dpos ? a.dpos[b] : 0.0f;
+    const float *eh = a.ent + a.h[b] * (int64_t)d, *et = a.ent + a.t[b] * (int64_t)d;
+    const float *e = a.resid + (int64_t)b * d;
+    float gs = g;
+    if (!a.rescal && a.norm_p == 2) {
+        const float s = a.spos[b];
+        gs = s > 0.0f ? g / s : 0.0f;
+    }
+    for (int j = lane * 4; j < d; j += 256) {
+        const float4 vh = *reinterpret_cast<const float4 *>(eh + j), vt = *reinterpret_cast<const float4 *>(et + j);
+        const float4 ve = *reinterpret_cast<const float4 *>(e + j);
+        float4 x, q;
+        if (a.rescal) {
+            x = vh;
+            q = make_float4(g * vt.x, g * vt.y, g * vt.z, g * vt.w);
+            *reinterpret_cast<float4 *>(a.occ_t + (int64_t)b * d + j) = make_float4(g * ve.x, g * ve.y, g * ve.z, g * ve.w);
+        } else {
+            x = make_float4(vh.x - vt.x, vh.y - vt.y, vh.z - vt.z, vh.w - vt.w);
+            if (a.norm_p == 1) q = make_float4(gs * sgn(ve.x), gs * sgn(ve.y), gs * sgn(ve.z), gs * sgn(ve.w));
+            else q = make_float4(gs * ve.x, gs * ve.y, gs * ve.z, gs * ve.w);
+        }
+        *reinterpret_cast<float4 *>(a.xs + p * d + j) = x;
+        *reinterpret_cast<float4 *>(a.qs + p * d + j) = q;
+    }
+}
+
+struct DmArgs {
+    const float *xs, *qs;  // sorted order [B, d]
+    const int32_t *num_unique, *seg_offsets;
+    float *dm;  // [U, d, d]
+    int d;
+};
+
+// dM[g][i][j] = sum_{p in group g} xs[p][i] * qs[p][j]; one workgroup per (group, 32 rows i),
+// the four waves split the columns j, K runs over the group's triples.
+__global__ __launch_bounds__(256) void transr_dm_kernel(DmArgs a)
+{
+    const int d = a.d;
+    const int nib = (d + 31) / 32;
+    const int g = blockIdx.x / nib;
+    if (g >= a.num_unique[0]) return;
+    const int i0 = (blockIdx.x % nib) * 32;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int li = lane & 15, kk = lane >> 4;
+    const int s0 = a.seg_offsets[g], s1 = a.seg_offsets[g + 1];
+    const bool two_blocks = i0 + 16 < d;
+    const bool ilo = i0 + li < d, ihi = i0 + 16 + li < d;
+
+    for (int c0 = 0; c0 < d; c0 += 256) {
+        const int span = d - c0 < 256 ? d - c0 : 256;
+        const int cw = ((span / 4 + 3) / 4) * 4;
+        const int n0 = c0 + wave * cw;
+        const int wcols = n0 >= c0 + span ? 0 : (c0 + span - n0 < cw ? c0 + span - n0 : cw);
+        if (wcols <= 0) continue;
+        const bool colok = 4 * li < wcols;
+        floatx4 acc_lo[4], acc_hi[4];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) acc_lo[e] = floatx4{0.f, 0.f, 0.f, 0.f}, acc_hi[e] = floatx4{0.f, 0.f, 0.f, 0.f};
+        for (int pq = s0; pq < s1; pq += 16) {
+            float al[4], ah[4];
+            float4 bv[4];
+#pragma unroll
+            for (int s = 0; s < 4; ++s) {
+                const int p = pq + 4 * kk + s;
+                const bool ok = p < s1;
+                const float *xr = a.xs + (int64_t)p * d + i0;
+                al[s] = (ok && ilo) ? xr[li] : 0.0f;
+                ah[s] = (ok && ihi) ? xr[16 + li] : 0.0f;
+                bv[s] = (ok && colok) ? *reinterpret_cast<const float4 *>(a.qs + (int64_t)p * d + n0 + 4 * li)
+                                      : make_float4(0.f, 0.f, 0.f, 0.f);
+            }
+#pragma unroll
+            for (int s = 0; s < 4; ++s) {
+                const float b4[4] = {bv[s].x, bv[s].y, bv[s].z, bv[s].w};
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    acc_lo[e] = __builtin_amdgcn_mfma_f32_16x16x4f32(al[s], b4[e], acc_lo[e], 0, 0, 0);
+                    if (two_blocks) acc_hi[e] = __builtin_amdgcn_mfma_f32_16x16x4f32(ah[s], b4[e], acc_hi[e], 0, 0, 0);
+                }
+            }
+        }
+        if (colok) {
+#pragma unroll
+            for (int blk = 0; blk < 2; ++blk)
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    const int row = i0 + 16 * blk + 4 * kk + r;
+                    if (row >= d) continue;
+                    float4 v;
+                    if (blk == 0) v = make_float4(acc_lo[0][r], acc_lo[1][r], acc_lo[2][r], acc_lo[3][r]);
+                    else v = make_float4(acc_hi[0][r], acc_hi[1][r], acc_hi[2][r], acc_hi[3][r]);
+                    *reinterpret_cast<float4 *>(a.dm + ((int64_t)g * d + row) * d + n0 + 4 * li) = v;
+                }
+        }
+    }
+}
+
+// ---- host side -----------------------------------------------------------------------------
+static size_t up256(size_t x) { return (x + 255) & ~size_t(255); }
+
+struct RPlan {
+    size_t off_plan, off_xs, off_qs, off_occ, off_part_e, off_part_r, total;
+    int64_t tiles;
+};
+
+static RPlan make_rplan(const kge_tables *tab, const kge_batch *bat)
+{
+    RPlan p{};
+    const int64_t B = bat->batch, d = tab->dim;
+    p.tiles = max_tiles(tab, bat);
+    size_t o = 0;
+    p.off_plan = o, o += up256(sizeof(int32_t) * (size_t)(2 * p.tiles + 64));
+    p.off_xs = o, o += up256(sizeof(float) * (size_t)(B * d));
+    p.off_qs = o, o += up256(sizeof(float) * (size_t)(B * d));
+    p.off_occ = o, o += up256(sizeof(float) * (size_t)(2 * B * d));
+    p.off_part_e = o, o += up256(sizeof(float) * (size_t)(ceil_div(2 * B, 32) * 2 * d));
+    p.off_part_r = o, o += up256(sizeof(float) * (size_t)(ceil_div(B, 32) * 2 * d));
+    p.total = o;
+    return p;
+}
+
+static TilePlan plan_at(void *base, int64_t tiles)
+{
+    int32_t *q = static_cast<int32_t *>(base);
+    return TilePlan{q, q + 64, q + 64 + tiles};
+}
+
+size_t transr_fwd_workspace(const kge_tables *tab, const kge_batch *bat)
+{
+    return up256(sizeof(int32_t) * (size_t)(2 * max_tiles(tab, bat) + 64));
+}
+
+int launch_transr_fwd(const kge_tables *tab, const kge_batch *bat, float *pos, float *resid, void *workspace,
+                      size_t workspace_bytes, hipStream_t st)
+{
+    if (bat->batch == 0) return KGE_OK;
+    const bool rescal = tab->model == KGE_RESCAL;
+    if (!mfma_path_ok(tab, bat) || !workspace || workspace_bytes < transr_fwd_workspace(tab, bat) ||
+        gemm_lds_bytes((int)tab->dim) > 64 * 1024)
+        return launch_score_pos(tab, bat, pos, resid, nullptr, st);
+    const kge_inspection *ri = bat->rel_insp;
+    const int64_t tiles = max_tiles(tab, bat);
+    TilePlan plan = plan_at(workspace, tiles);
+    hipLaunchKernelGGL(transr_plan_kernel, dim3(1), dim3(1024), 0, st, ri->num_unique, ri->seg_offsets, plan);
+    GemmArgs a{tab->ent, tab->rel, tab->aux, bat->h, bat->r, bat->t, ri->perm, ri->seg_offsets, ri->unique_ids,
+               plan, nullptr, pos, resid, nullptr, nullptr, (int)tab->dim, tab->norm_p};
+    const size_t lds = gemm_lds_bytes((int)tab->dim);
+    if (rescal)
+        hipLaunchKernelGGL(transr_gemm_kernel<1>, dim3((unsigned)tiles), dim3(256), lds, st, a);
+    else
+        hipLaunchKernelGGL(transr_gemm_kernel<0>, dim3((unsigned)tiles), dim3(256), lds, st, a);
+    KGE_CHECK_LAUNCH();
+    return KGE_OK;
+}
+
+size_t transr_bwd_workspace(const kge_tables *tab, const kge_batch *bat) { return make_rplan(tab, bat).total; }
+
+int launch_seg_reduce(const float *occ, const kge_inspection *ins, int d, float *out, float *partial,
+                      bool identity_perm, hipStream_t st);
+
+int launch_transr_bwd(const kge_tables *tab, const kge_batch *bat, const kge_saved *saved, const float *dpos,
+                      const kge_grads *grads, void *workspace, size_t workspace_bytes, hipStream_t st)
+{
+    const bool rescal = tab->model == KGE_RESCAL;
+    if (bat->neg) return KGE_EUNSUPPORTED;  // positives only for the projection models
+    if (!mfma_path_ok(tab, bat) || gemm_lds_bytes((int)tab->dim) > 64 * 1024) return KGE_EUNSUPPORTED;
+    if (!saved->residual || !grads->aux_rows || !grads->ent_rows) return KGE_EINVAL;
+    if (!rescal && (!grads->rel_rows || (tab->norm_p == 2 && !saved->pos))) return KGE_EINVAL;
+    const RPlan p = make_rplan(tab, bat);
+    if (!workspace || workspace_bytes < p.total) return KGE_EWORKSPACE;
+    if (bat->ent_insp->n != 2 * bat->batch) return KGE_ESHAPE;
+    const int64_t B = bat->batch;
+    const int d = (int)tab->dim;
+    char *ws = static_cast<char *>(workspace);
+    float *xs = reinterpret_cast<float *>(ws + p.off_xs), *qs = reinterpret_cast<float *>(ws + p.off_qs);
+    float *occ = reinterpret_cast<float *>(ws + p.off_occ);
+    const kge_inspection *ri = bat->rel_insp;
+    TilePlan plan = plan_at(ws + p.off_plan, p.tiles);
+
+    PrepArgs pa{tab->ent, bat->h, bat->t, ri->perm, dpos, saved->pos, saved->residual, xs, qs, occ + B * d, B, d,
+                tab->norm_p, rescal ? 1 : 0};
+    hipLaunchKernelGGL(transr_prep_kernel, dim3((unsigned)ceil_div(B, 4)), dim3(256), 0, st, pa);
+    hipLaunchKernelGGL(transr_plan_kernel, dim3(1), dim3(1024), 0, st, ri->num_unique, ri->seg_offsets, plan);
+    // dX = Q M^T -> occurrence rows of h (and -dX for t)
+    GemmArgs ga{tab->ent, tab->rel, tab->aux, bat->h, bat->r, bat->t, ri->perm, ri->seg_offsets, ri->unique_ids,
+                plan, qs, nullptr, nullptr, occ, rescal ? nullptr : occ + B * d, d, tab->norm_p};
+    hipLaunchKernelGGL(transr_gemm_kernel<2>, dim3((unsigned)p.tiles), dim3(256), gemm_lds_bytes(d), st, ga);
+    // dM = X^T Q per relation group
+    const int64_t groups = B < tab->n_rel ? B : tab->n_rel;
+    DmArgs da{xs, qs, ri->num_unique, ri->seg_offsets, grads->aux_rows, d};
+    hipLaunchKernelGGL(transr_dm_kernel, dim3((unsigned)(ceil_div(d, 32) * groups)), dim3(256), 0, st, da);
+    KGE_CHECK_LAUNCH();
+    int rc = launch_seg_reduce(occ, bat->ent_insp, d, grads->ent_rows, reinterpret_cast<float *>(ws + p.off_part_e),
+                               false, st);
+    if (rc || rescal) return rc;
+    // dR[g] = sum of the group's q rows (already in sorted order)
+    return launch_seg_reduce(qs, ri, d, grads->rel_rows, reinterpret_cast<float *>(ws + p.off_part_r), true, st);
+}
+
 }  // namespace kge

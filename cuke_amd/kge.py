@@ -21,7 +21,7 @@ import torch
 from . import _lib
 from ._lib import KgeError, MODELS
 
-__all__ = ["KGEModel", "Inspection", "Forward", "SparseGrads", "inspect", "inspector", "transE",
+__all__ = ["KGEModel", "TrainStep", "Inspection", "Forward", "SparseGrads", "inspect", "inspector", "transE",
            "transH", "transR", "transF", "RESCAL", "margin_loss", "KgeError"]
 
 
@@ -203,9 +203,14 @@ class KGEModel:
         """[B, dim] residual vector: the reference's output for TransE / TransH / TransR."""
         bat, keep = self._batch(h, r, t, rel_insp=rel_insp)
         out = torch.empty((bat.batch, self.dim), dtype=torch.float32, device=self.dev)
-        _lib.check(_lib.lib().kge_residual_fwd(C.byref(self._tab), C.byref(bat), _ptr(out), _stream()),
-                   "kge_residual_fwd")
+        ws, nb = self._fwd_workspace(bat)
+        _lib.check(_lib.lib().kge_residual_fwd(C.byref(self._tab), C.byref(bat), _ptr(out), _ptr(ws), nb,
+                                               _stream()), "kge_residual_fwd")
         return out
+
+    def _fwd_workspace(self, bat):
+        nb = int(_lib.lib().kge_score_fwd_workspace(C.byref(self._tab), C.byref(bat)))
+        return torch.empty(max(nb, 1), dtype=torch.uint8, device=self.dev), nb
 
     # -- scalar scores ---------------------------------------------------------------------
     def score(self, h, r, t, neg=None, chunk=None, ent_insp=None, rel_insp=None) -> Forward:
@@ -219,11 +224,12 @@ class KGEModel:
             fw.side_pos = torch.empty(B, **f32)
             if neg is not None:
                 fw.side_neg = torch.empty((2, B, N), **f32)
-        if self.model == "TransR":
+        if self.model in ("TransR", "RESCAL"):
             fw.residual = torch.empty((B, self.dim), **f32)
+        ws, nb = self._fwd_workspace(bat)
         _lib.check(_lib.lib().kge_score_fwd(C.byref(self._tab), C.byref(bat), _ptr(fw.pos),
                                             _ptr(fw.neg), _ptr(fw.side_pos), _ptr(fw.side_neg),
-                                            _ptr(fw.residual), _stream()), "kge_score_fwd")
+                                            _ptr(fw.residual), _ptr(ws), nb, _stream()), "kge_score_fwd")
         return fw
 
     def inspect_batch(self, h, r, t, neg=None):
@@ -324,7 +330,8 @@ def RESCAL(batch_size, dim, nnodes, Eemb, h, nedges, Proj, r, *rest):
     """apps/kge/test_cuke.py:244: (batch, dim, nnodes, E, h, nedges, Proj, r, uniq, buf, cnt, t) -> [batch]."""
     _sizes_ok(batch_size, dim, Eemb, h)
     t = rest[-1]
-    return KGEModel("RESCAL", Eemb, None, Proj).score(h, r, t).pos
+    m = KGEModel("RESCAL", Eemb, None, Proj)
+    return m.score(h, r, t, rel_insp=inspect([r], m.n_rel)).pos
 
 
 def inspector(r: torch.Tensor, rel_num: int, C_: int = 16):
@@ -341,3 +348,132 @@ def inspector(r: torch.Tensor, rel_num: int, C_: int = 16):
     _lib.check(_lib.lib().kge_build_index(_ptr(r), _ptr(uniq), _ptr(buf), _ptr(cnt), int(r.numel()),
                                           int(rel_num), _stream()), "kge_build_index")
     return uniq, buf, cnt
+
+
+class TrainStep:
+    """One forward + backward pass over a fixed-shape batch with every buffer allocated up front.
+
+    ``run()`` enqueues: inspector over concat(h, t, neg) and over r -> scores -> (margin loss)
+    -> sparse row gradients.  Nothing is allocated and nothing synchronises inside ``run()``,
+    so the sequence can be captured into a HIP graph (``capture()``) and replayed.
+    loss = "sum":    upstream gradients are the caller-supplied ``dpos`` / ``dneg`` (default: ones)
+    loss = "margin": margin-ranking loss with ``margin`` and ``sign``
+    """
+
+    def __init__(self, model: KGEModel, h, r, t, neg=None, chunk=None, loss="sum", margin=1.0,
+                 sign=1.0, dpos=None, dneg=None):
+        self.m = model
+        dev = model.dev
+        L = self.L = _lib.lib()
+        f32 = dict(dtype=torch.float32, device=dev)
+        i32 = dict(dtype=torch.int32, device=dev)
+        _, (h, r, t, neg, C_, N) = model._batch(h, r, t, neg, chunk)
+        self.idx = (h, r, t, neg)
+        B = self.B = int(h.numel())
+        self.N, self.C = N, C_
+        self.loss_kind, self.margin, self.sign = loss, float(margin), float(sign)
+
+        def make_insp(n, n_rows):
+            ins = Inspection(n, n_rows, torch.zeros(1, **i32), torch.empty(max(n, 1), dtype=torch.int64, device=dev),
+                             torch.empty(n + 1, **i32), torch.empty(max(n, 1), **i32),
+                             torch.empty(max(n, 1), **i32), torch.empty(max(n, 1), **i32))
+            ins._c = _lib.Inspection(n, n_rows, ins.num_unique_dev.data_ptr(), ins.unique_ids.data_ptr(),
+                                     ins.seg_offsets.data_ptr(), ins.perm.data_ptr(), ins.inverse.data_ptr(),
+                                     ins.sorted_seg.data_ptr())
+            ws = torch.empty(max(int(L.kge_inspect_workspace(n, n_rows)), 1), dtype=torch.uint8, device=dev)
+            return ins, ws
+
+        parts = [h, t] + ([neg] if neg is not None else [])
+        n_occ = sum(int(p.numel()) for p in parts)
+        self.ent_insp, self._ws_e = make_insp(n_occ, int(model.E.shape[0]))
+        self.rel_insp, self._ws_r = make_insp(B, max(model.n_rel, 1))
+        self._parts_e = ((C.c_void_p * len(parts))(*[p.data_ptr() for p in parts]),
+                         (C.c_int64 * len(parts))(*[int(p.numel()) for p in parts]), len(parts))
+        self._parts_r = ((C.c_void_p * 1)(r.data_ptr()), (C.c_int64 * 1)(B), 1)
+
+        self.bat = _lib.Batch(B, h.data_ptr(), r.data_ptr(), t.data_ptr(),
+                              neg.data_ptr() if neg is not None else None, C_, N,
+                              C.pointer(self.ent_insp._c), C.pointer(self.rel_insp._c))
+        self.pos = torch.empty(B, **f32)
+        self.neg = torch.empty((B, N), **f32) if neg is not None else None
+        self.side_pos = torch.empty(B, **f32) if model.model == "TransH" else None
+        self.side_neg = torch.empty((2, B, N), **f32) if (model.model == "TransH" and neg is not None) else None
+        self.residual = torch.empty((B, model.dim), **f32) if model.model in ("TransR", "RESCAL") else None
+        self._ws_f_bytes = int(L.kge_score_fwd_workspace(C.byref(model._tab), C.byref(self.bat)))
+        self._ws_f = torch.empty(max(self._ws_f_bytes, 1), dtype=torch.uint8, device=dev)
+        self.loss = torch.zeros(1, **f32)
+        if loss == "margin":
+            self.dpos, self.dneg = torch.empty(B, **f32), torch.empty((B, N), **f32)
+            self._ws_l = torch.empty(max(int(L.kge_margin_loss_workspace(B, N)), 1), dtype=torch.uint8, device=dev)
+        else:
+            self.dpos = torch.ones(B, **f32) if dpos is None else dpos.to(**f32).contiguous()
+            self.dneg = None
+            if neg is not None:
+                self.dneg = torch.ones((B, N), **f32) if dneg is None else dneg.to(**f32).contiguous()
+        self.saved = _lib.Saved(*[(x.data_ptr() if x is not None else None) for x in
+                                  (self.pos, self.neg, self.side_pos, self.side_neg, self.residual)])
+        self.ent_rows = torch.empty((n_occ, model.dim), **f32)
+        self.rel_rows = torch.empty((B, model.rel_dim), **f32) if model.rel_dim else None
+        self.aux_rows = None
+        if model.model == "TransH":
+            self.aux_rows = torch.empty((B, model.dim), **f32)
+        elif model.model in ("TransR", "RESCAL"):
+            self.aux_rows = torch.empty((min(B, model.n_rel), model.dim * model.dim), **f32)
+        self.grads = _lib.Grads(_ptr(self.ent_rows), _ptr(self.rel_rows), _ptr(self.aux_rows))
+        self._ws_b_bytes = int(L.kge_score_bwd_workspace(C.byref(model._tab), C.byref(self.bat)))
+        self._ws_b = torch.empty(max(self._ws_b_bytes, 1), dtype=torch.uint8, device=dev)
+        self.graph = None
+
+    # the individual stages, each one C call
+    def inspect(self, st):
+        L, ie, ir = self.L, self.ent_insp, self.rel_insp
+        p, l, n = self._parts_e
+        _lib.check(L.kge_inspect(p, l, n, ie.n_rows, C.byref(ie._c), _ptr(self._ws_e), self._ws_e.numel(), st),
+                   "kge_inspect(entities)")
+        p, l, n = self._parts_r
+        _lib.check(L.kge_inspect(p, l, n, ir.n_rows, C.byref(ir._c), _ptr(self._ws_r), self._ws_r.numel(), st),
+                   "kge_inspect(relations)")
+
+    def forward(self, st):
+        _lib.check(self.L.kge_score_fwd(C.byref(self.m._tab), C.byref(self.bat), _ptr(self.pos), _ptr(self.neg),
+                                        _ptr(self.side_pos), _ptr(self.side_neg), _ptr(self.residual),
+                                        _ptr(self._ws_f), self._ws_f_bytes, st), "kge_score_fwd")
+
+    def loss_grad(self, st):
+        if self.loss_kind == "margin":
+            _lib.check(self.L.kge_margin_loss(_ptr(self.pos), _ptr(self.neg), self.B, self.N, self.margin,
+                                              self.sign, _ptr(self.loss), _ptr(self.dpos), _ptr(self.dneg),
+                                              _ptr(self._ws_l), self._ws_l.numel(), st), "kge_margin_loss")
+
+    def backward(self, st):
+        _lib.check(self.L.kge_score_bwd(C.byref(self.m._tab), C.byref(self.bat), C.byref(self.saved),
+                                        _ptr(self.dpos), _ptr(self.dneg), C.byref(self.grads), _ptr(self._ws_b),
+                                        self._ws_b_bytes, st), "kge_score_bwd")
+
+    def run(self, backward=True):
+        st = _stream()
+        self.inspect(st)
+        self.forward(st)
+        if backward:
+            self.loss_grad(st)
+            self.backward(st)
+
+    def capture(self, backward=True):
+        """Record run() into a HIP graph; replay() then launches the whole step at once."""
+        self.run(backward)  # warm-up outside capture (module loading, lazy init)
+        torch.cuda.synchronize()
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g):
+            self.run(backward)
+        self.graph = g
+        return g
+
+    def replay(self):
+        self.graph.replay()
+
+    def sparse_grads(self) -> SparseGrads:
+        ue, ur = self.ent_insp.num_unique, self.rel_insp.num_unique
+        self.ent_insp._u = self.rel_insp._u = None  # counts belong to the batch just run
+        return SparseGrads(self.ent_insp.unique_ids[:ue], self.ent_rows[:ue], self.rel_insp.unique_ids[:ur],
+                           self.rel_rows[:ur] if self.rel_rows is not None else None,
+                           self.aux_rows[:ur] if self.aux_rows is not None else None)

@@ -113,7 +113,7 @@ typedef struct kge_saved {
     const float *side_pos;  /* [B]: TransH w.h per positive; TransR: unused */
     const float *side_neg;  /* [2, B, n_neg]: TransH, plane 0 = w_b . t'_k per pair,
                                plane 1 = sum_i phi(u_i) w_i (phi = sign for L1, u/||u|| for L2) */
-    const float *residual;  /* [B, dim]: TransR residual rows */
+    const float *residual;  /* [B, dim]: TransR residual rows / RESCAL E[h] Proj[r] rows */
 } kge_saved;
 
 /* Sparse row gradients: row u of each array belongs to the u-th unique id of the
@@ -135,17 +135,23 @@ int kge_abi_version(void);
  * Replaces module.run(...) of pycuke1/codegen/gpu_template.cu:8-13.
  * out: [B, dim].  TransE is bit-exact with the generated CPU loop.
  */
-int kge_residual_fwd(const kge_tables *tab, const kge_batch *bat, float *out, void *stream);
+int kge_residual_fwd(const kge_tables *tab, const kge_batch *bat, float *out, void *workspace,
+                     size_t workspace_bytes, void *stream);
 
 /*
  * Scalar scores.  pos[B]; neg[B, n_neg] when bat->neg is set (either may be
  * NULL to skip).  side_pos / side_neg are optional save-for-backward outputs
  * (see kge_saved; required later by kge_score_bwd for TransH).
  * Scalar-score models of the reference: TransF / RESCAL (kge.py:363,387).
- * TransR needs bat->rel_insp (relation groups) and `residual` [B, dim] scratch.
+ * TransR / RESCAL: with bat->rel_insp (relation groups) the projection runs as grouped
+ * per-relation MFMA contractions and needs kge_score_fwd_workspace() bytes of workspace;
+ * without it every triple streams its own projection.  `residual` [B, dim] receives the
+ * projected rows (TransR: the residual, RESCAL: E[h] Proj[r]) that kge_score_bwd consumes.
  */
+size_t kge_score_fwd_workspace(const kge_tables *tab, const kge_batch *bat);
 int kge_score_fwd(const kge_tables *tab, const kge_batch *bat, float *pos, float *neg,
-                  float *side_pos, float *side_neg, float *residual, void *stream);
+                  float *side_pos, float *side_neg, float *residual, void *workspace,
+                  size_t workspace_bytes, void *stream);
 
 /*
  * Index inspector: radix sort + dedup of up to four concatenated int64 index

@@ -1,0 +1,97 @@
+"""TransR / RESCAL: grouped per-relation MFMA path (forward and backward) against the oracle."""
+import numpy as np
+import pytest
+import torch
+
+from cuke_amd import synth
+from helpers import assert_close, gpu_model
+
+pytestmark = pytest.mark.gpu
+
+
+def grouped_forward(m, ix):
+    from cuke_amd.kge import inspect
+    rel = inspect([ix["r"]], m.n_rel)
+    return m.score(ix["h"], ix["r"], ix["t"], rel_insp=rel), rel
+
+
+@pytest.mark.parametrize("model", ["TransR", "RESCAL"])
+@pytest.mark.parametrize("shape", [
+    dict(dim=16, batch=5, n_rel=3),          # one tile, fewer rows than an MFMA block
+    dict(dim=200, batch=300, n_rel=7),       # groups larger than a tile, ragged column split
+    dict(dim=256, batch=1000, n_rel=400),    # mostly singletons
+    dict(dim=64, batch=257, n_rel=1),        # one group, many tiles
+    dict(dim=36, batch=130, n_rel=9),        # K tail (36 = 2 * 16 + 4)
+])
+@pytest.mark.parametrize("p", [1, 2])
+def test_grouped_forward(oracle, model, shape, p):
+    if model == "RESCAL" and p == 1:
+        pytest.skip("no norm in RESCAL")
+    w = synth.custom_workload(model, n_ent=500, norm_p=p, sigma=0.2, rel_zipf=1.2, seed=shape["dim"], **shape)
+    a = w.arrays
+    m, ix = gpu_model(w)
+    fw, rel = grouped_forward(m, ix)
+    pos, _ = oracle.score(model, a["E"], a["R"], a["A"], a["h"], a["r"], a["t"], p=p)
+    assert_close(fw.pos.cpu().numpy(), pos, what=f"{model} {shape} grouped score")
+    if model == "TransR":
+        want = oracle.residual("TransR", a["E"], a["R"], a["A"], a["h"], a["r"], a["t"])
+        assert_close(fw.residual.cpu().numpy(), want, what="grouped residual")
+        assert_close(m.residual(ix["h"], ix["r"], ix["t"], rel_insp=rel).cpu().numpy(), want,
+                     what="grouped residual entry point")
+    # the ungrouped per-triple path must agree as well
+    assert_close(m.score(ix["h"], ix["r"], ix["t"]).pos.cpu().numpy(), pos, what="ungrouped score")
+
+
+@pytest.mark.parametrize("model", ["TransR", "RESCAL"])
+@pytest.mark.parametrize("shape", [
+    dict(dim=16, batch=5, n_rel=3),
+    dict(dim=200, batch=300, n_rel=7),
+    dict(dim=36, batch=130, n_rel=9),
+    dict(dim=64, batch=257, n_rel=1),
+])
+@pytest.mark.parametrize("p", [1, 2])
+def test_grouped_backward(oracle, model, shape, p):
+    if model == "RESCAL" and p == 1:
+        pytest.skip("no norm in RESCAL")
+    w = synth.custom_workload(model, n_ent=120, norm_p=p, sigma=0.2, rel_zipf=1.2, ent_zipf=1.1,
+                              seed=shape["dim"] + p, lattice=(p == 1 and model == "TransR"), **shape)
+    a = w.arrays
+    if w.lattice:  # keep the projected residual exact too: projections on a coarse grid
+        a["A"] = (np.rint(a["A"] / 0.2 * 2) / 8).astype(np.float32)
+    m, ix = gpu_model(w)
+    fw, rel = grouped_forward(m, ix)
+    dpos = np.random.default_rng(1).standard_normal(w.batch).astype(np.float32)
+    g = m.backward(fw, torch.from_numpy(dpos).to(fw.pos.device))
+    ref = oracle.backward(model, a["E"], a["R"], a["A"], a["h"], a["r"], a["t"], dpos=dpos, p=p)
+    assert np.array_equal(g.ent_ids.cpu().numpy(), ref.ent_ids)
+    assert np.array_equal(g.rel_ids.cpu().numpy(), ref.rel_ids)
+    assert_close(g.ent_rows.cpu().numpy(), ref.ent_rows, what="entity rows", rows=True)
+    if model == "TransR":
+        assert_close(g.rel_rows.cpu().numpy(), ref.rel_rows, what="relation rows", rows=True)
+    assert_close(g.aux_rows.cpu().numpy(), ref.aux_rows, what="projection gradients", rows=True)
+
+
+def test_cfg3_scaled(oracle):
+    w = synth.make_workload("cfg3_transr", batch=2048)
+    a = w.arrays
+    m, ix = gpu_model(w)
+    fw, rel = grouped_forward(m, ix)
+    pos, _ = oracle.score("TransR", a["E"], a["R"], a["A"], a["h"], a["r"], a["t"], p=2)
+    assert_close(fw.pos.cpu().numpy(), pos, what="cfg3 scores")
+    dpos = np.random.default_rng(2).standard_normal(w.batch).astype(np.float32)
+    g = m.backward(fw, torch.from_numpy(dpos).to(fw.pos.device))
+    ref = oracle.backward("TransR", a["E"], a["R"], a["A"], a["h"], a["r"], a["t"], dpos=dpos, p=2)
+    assert np.array_equal(g.rel_ids.cpu().numpy(), ref.rel_ids)
+    assert_close(g.ent_rows.cpu().numpy(), ref.ent_rows, what="cfg3 entity rows", rows=True)
+    assert_close(g.rel_rows.cpu().numpy(), ref.rel_rows, what="cfg3 relation rows", rows=True)
+    assert_close(g.aux_rows.cpu().numpy(), ref.aux_rows, what="cfg3 projection gradients", rows=True)
+
+
+def test_proj_identity_reduces_to_transe(oracle):
+    w = synth.custom_workload("TransR", n_ent=300, n_rel=5, dim=64, batch=200, sigma=0.2, seed=3)
+    a = w.arrays
+    a["A"] = np.broadcast_to(np.eye(64, dtype=np.float32), (5, 64, 64)).copy()
+    m, ix = gpu_model(w)
+    fw, _ = grouped_forward(m, ix)
+    te, _ = oracle.score("TransE", a["E"], a["R"], None, a["h"], a["r"], a["t"], p=2)
+    assert_close(fw.pos.cpu().numpy(), te, what="Proj = I")
