@@ -32,10 +32,17 @@ class Inspection(C.Structure):
                 ("inverse", C.c_void_p), ("sorted_seg", C.c_void_p)]
 
 
+class InspectJob(C.Structure):
+    _fields_ = [("parts", C.c_void_p * 4), ("part_len", C.c_int64 * 4), ("n_parts", C.c_int32),
+                ("reserved", C.c_int32), ("n_rows", C.c_int64), ("out", Inspection),
+                ("workspace", C.c_void_p), ("workspace_bytes", C.c_size_t)]
+
+
 class Batch(C.Structure):
     _fields_ = [("batch", C.c_int64), ("h", C.c_void_p), ("r", C.c_void_p), ("t", C.c_void_p),
                 ("neg", C.c_void_p), ("chunk", C.c_int64), ("n_neg", C.c_int64),
-                ("ent_insp", C.POINTER(Inspection)), ("rel_insp", C.POINTER(Inspection))]
+                ("ent_insp", C.POINTER(Inspection)), ("rel_insp", C.POINTER(Inspection)),
+                ("insp_ready", C.c_void_p)]
 
 
 class Saved(C.Structure):
@@ -59,6 +66,7 @@ EXPORTS = {
     "kge_inspect_workspace": (C.c_size_t, [C.c_int64, C.c_int64]),
     "kge_inspect": (C.c_int, [C.POINTER(C.c_void_p), C.POINTER(C.c_int64), C.c_int, C.c_int64,
                               C.POINTER(Inspection), C.c_void_p, C.c_size_t, C.c_void_p]),
+    "kge_inspect_batch": (C.c_int, [C.POINTER(InspectJob), C.c_int, C.c_void_p]),
     "kge_margin_loss_workspace": (C.c_size_t, [C.c_int64, C.c_int64]),
     "kge_margin_loss": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int64, C.c_int64, C.c_float,
                                   C.c_float, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p,

@@ -283,6 +283,180 @@ __global__ __launch_bounds__(kSortThreads) void finalize_kernel(const uint32_t *
     }
 }
 
+// ---- small inputs: the whole inspection in one workgroup ------------------------------------
+// Up to 32768 ids: one 1024-thread workgroup runs every radix pass and the dedup with
+// workgroup barriers only (keys ping-pong through L2, digit counters in LDS), so an
+// inspection is one launch instead of 2 per pass + 2; several index sets are inspected by
+// the same launch, one workgroup each.
+constexpr int kSmallThreads = 1024;
+constexpr int kSmallWaves = kSmallThreads / kWave;  // 16
+constexpr int kSmallMaxBits = 10;
+constexpr int kSmallMaxBins = 1 << kSmallMaxBits;
+constexpr int64_t kSmallMaxN = 32768;
+
+struct SmallJob {
+    Parts parts;
+    int64_t n;
+    int bits;
+    kge_inspection out;
+    uint32_t *keys_final, *keys_tmp;
+    int32_t *vals_tmp;
+};
+struct SmallJobs {
+    SmallJob j[4];
+};
+
+template <int KPT>
+__global__ __launch_bounds__(kSmallThreads) void inspect_small_kernel(SmallJobs jobs)
+{
+    __shared__ unsigned short s_cnt[kSmallWaves][kSmallMaxBins];  // 32 KB
+    __shared__ uint32_t s_tot[kSmallMaxBins];
+    __shared__ uint32_t s_w[kSmallWaves];
+    const SmallJob &J = jobs.j[blockIdx.x];
+    const int tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid >> 6;
+    const int n = (int)J.n;
+    const int npass = (J.bits + kSmallMaxBits - 1) / kSmallMaxBits;
+    const int db = (J.bits + npass - 1) / npass;
+    const int bins = 1 << db;
+    const uint32_t mask = (uint32_t)bins - 1;
+    // wave w owns the contiguous keys [w*m, (w+1)*m), m a multiple of 64
+    const int m = ((n + kSmallWaves * kWave - 1) / (kSmallWaves * kWave)) * kWave;
+    const int nr = m / kWave;  // rounds per wave, <= KPT
+    const int wbase = wave * m;
+    const uint64_t lt_mask = lane ? (~0ull >> (kWave - lane)) : 0ull;
+
+    const uint32_t *kin = nullptr;
+    const int32_t *vin = nullptr;
+    for (int pass = 0; pass < npass; ++pass) {
+        const bool to_final = ((npass - 1 - pass) & 1) == 0;
+        uint32_t *kout = to_final ? J.keys_final : J.keys_tmp;
+        int32_t *vout = to_final ? J.out.perm : J.vals_tmp;
+        const int shift = pass * db;
+        for (int i = tid; i < kSmallWaves * kSmallMaxBins / 2; i += kSmallThreads)
+            reinterpret_cast<uint32_t *>(&s_cnt[0][0])[i] = 0;
+        uint32_t key[KPT];
+        int32_t val[KPT];
+        uint32_t lrank[KPT];
+#pragma unroll
+        for (int j = 0; j < KPT; ++j) {
+            const int i = wbase + j * kWave + lane;
+            const bool ok = j < nr && i < n;
+            key[j] = ok ? (kin ? kin[i] : load_key(J.parts, i)) : 0u;
+            val[j] = ok ? (vin ? vin[i] : i) : 0;
+        }
+        __syncthreads();
+#pragma unroll
+        for (int j = 0; j < KPT; ++j) {
+            if (j < nr) {  // uniform across the workgroup
+                const int i = wbase + j * kWave + lane;
+                const bool ok = i < n;
+                const uint32_t dg = (key[j] >> shift) & mask;
+                uint64_t peers = __ballot(ok);
+                for (int bit = 0; bit < db; ++bit) {
+                    const bool one = (dg >> bit) & 1u;
+                    const uint64_t mm = __ballot(one);
+                    peers &= one ? mm : ~mm;
+                }
+                const int leader = __ffsll((unsigned long long)peers) - 1;
+                uint32_t old = 0;
+                if (ok && lane == leader) {
+                    old = s_cnt[wave][dg];
+                    s_cnt[wave][dg] = (unsigned short)(old + __popcll(peers));
+                }
+                old = __shfl(old, leader < 0 ? 0 : leader, kWave);
+                lrank[j] = old + __popcll(peers & lt_mask);
+                __builtin_amdgcn_wave_barrier();
+            }
+        }
+        __syncthreads();
+        // per bin: exclusive prefix over the waves, total into s_tot
+        uint32_t tot = 0;
+        if (tid < bins) {
+#pragma unroll
+            for (int w = 0; w < kSmallWaves; ++w) {
+                const uint32_t c = s_cnt[w][tid];
+                s_cnt[w][tid] = (unsigned short)tot;
+                tot += c;
+            }
+        }
+        // exclusive scan of the bin totals over the 1024 threads
+        uint32_t inc = tot;
+#pragma unroll
+        for (int o = 1; o < kWave; o <<= 1) {
+            const uint32_t up = __shfl_up(inc, o, kWave);
+            if (lane >= o) inc += up;
+        }
+        if (lane == kWave - 1) s_w[wave] = inc;
+        __syncthreads();
+        uint32_t woff = 0;
+        for (int w = 0; w < wave; ++w) woff += s_w[w];
+        if (tid < bins) s_tot[tid] = woff + inc - tot;
+        __syncthreads();
+#pragma unroll
+        for (int j = 0; j < KPT; ++j) {
+            const int i = wbase + j * kWave + lane;
+            if (j < nr && i < n) {
+                const uint32_t dg = (key[j] >> shift) & mask;
+                const uint32_t pos = s_tot[dg] + s_cnt[wave][dg] + lrank[j];
+                kout[pos] = key[j];
+                vout[pos] = val[j];
+            }
+        }
+        __threadfence_block();
+        __syncthreads();
+        kin = kout;
+        vin = vout;
+    }
+
+    // dedup: thread t owns the sorted positions [t*q, (t+1)*q)
+    const int q = (n + kSmallThreads - 1) / kSmallThreads;  // <= KPT
+    const int lo = tid * q;
+    uint32_t k[KPT];
+    bool head[KPT];
+    uint32_t mine = 0;
+    uint32_t prev = (lo > 0 && lo < n) ? J.keys_final[lo - 1] : 0;
+#pragma unroll
+    for (int j = 0; j < KPT; ++j) {
+        const int i = lo + j;
+        const bool ok = j < q && i < n;
+        k[j] = ok ? J.keys_final[i] : 0;
+        head[j] = ok && (i == 0 || k[j] != prev);
+        prev = k[j];
+        mine += head[j] ? 1 : 0;
+    }
+    uint32_t inc = mine;
+#pragma unroll
+    for (int o = 1; o < kWave; o <<= 1) {
+        const uint32_t up = __shfl_up(inc, o, kWave);
+        if (lane >= o) inc += up;
+    }
+    if (lane == kWave - 1) s_w[wave] = inc;
+    __syncthreads();
+    uint32_t run = inc - mine, all = 0;
+    for (int w = 0; w < kSmallWaves; ++w) {
+        run += w < wave ? s_w[w] : 0;
+        all += s_w[w];
+    }
+    if (tid == 0) {
+        J.out.num_unique[0] = (int32_t)all;
+        J.out.seg_offsets[all] = n;
+    }
+#pragma unroll
+    for (int j = 0; j < KPT; ++j) {
+        const int i = lo + j;
+        if (j < q && i < n) {
+            if (head[j]) {
+                J.out.unique_ids[run] = (int64_t)k[j];
+                J.out.seg_offsets[run] = i;
+                ++run;
+            }
+            const int32_t seg = (int32_t)run - 1;
+            J.out.sorted_seg[i] = seg;
+            J.out.inverse[J.out.perm[i]] = seg;
+        }
+    }
+}
+
 // ---- host side ---------------------------------------------------------------------------
 struct SortPlan {
     int bits, npass, digit_bits;
@@ -292,11 +466,17 @@ struct SortPlan {
 
 static size_t align_up(size_t x) { return (x + 255) & ~size_t(255); }
 
+static int key_bits(int64_t n_rows)
+{
+    int bits = 1;
+    while (bits < 32 && (int64_t(1) << bits) < n_rows) ++bits;
+    return bits;
+}
+
 static SortPlan make_plan(int64_t n, int64_t n_rows)
 {
     SortPlan p{};
-    int bits = 1;
-    while (bits < 32 && (int64_t(1) << bits) < n_rows) ++bits;
+    const int bits = key_bits(n_rows);
     p.bits = bits;
     p.npass = (bits + kMaxDigitBits - 1) / kMaxDigitBits;
     p.digit_bits = (bits + p.npass - 1) / p.npass;
@@ -325,26 +505,32 @@ size_t kge_inspect_workspace(int64_t n, int64_t n_rows)
     return make_plan(n, n_rows).total;
 }
 
-int kge_inspect(const int64_t *const *parts_in, const int64_t *part_len, int n_parts, int64_t n_rows,
-                const kge_inspection *out, void *workspace, size_t workspace_bytes, void *stream)
+static int validate_job(const kge_inspect_job *job, Parts *parts, int64_t *n_out)
 {
-    if (!out || !parts_in || !part_len || n_parts < 1 || n_parts > 4) return KGE_EINVAL;
-    if (n_rows <= 0 || n_rows > (int64_t(1) << 32)) return KGE_ESHAPE;
-    Parts parts{};
-    parts.n_parts = n_parts;
+    if (job->n_parts < 1 || job->n_parts > 4) return KGE_EINVAL;
+    if (job->n_rows <= 0 || job->n_rows > (int64_t(1) << 32)) return KGE_ESHAPE;
+    parts->n_parts = job->n_parts;
     int64_t n = 0;
-    for (int q = 0; q < n_parts; ++q) {
-        if (part_len[q] < 0 || (part_len[q] > 0 && !parts_in[q])) return KGE_EINVAL;
-        n += part_len[q];
-        parts.p[q] = parts_in[q];
-        parts.end[q] = n;
+    for (int q = 0; q < job->n_parts; ++q) {
+        if (job->part_len[q] < 0 || (job->part_len[q] > 0 && !job->parts[q])) return KGE_EINVAL;
+        n += job->part_len[q];
+        parts->p[q] = job->parts[q];
+        parts->end[q] = n;
     }
+    const kge_inspection *out = &job->out;
     if (n != out->n || n >= (int64_t(1) << 31)) return KGE_ESHAPE;
     if (!out->num_unique || !out->seg_offsets) return KGE_EINVAL;
     if (n > 0 && (!out->unique_ids || !out->perm || !out->inverse || !out->sorted_seg)) return KGE_EINVAL;
+    if (!job->workspace || job->workspace_bytes < make_plan(n, job->n_rows).total) return KGE_EWORKSPACE;
+    *n_out = n;
+    return KGE_OK;
+}
+
+// multi-block path: 2-3 launches per digit pass + 2
+static int inspect_large(const Parts &parts, int64_t n, int64_t n_rows, const kge_inspection *out, void *workspace,
+                         hipStream_t st)
+{
     const SortPlan p = make_plan(n, n_rows);
-    if (!workspace || workspace_bytes < p.total) return KGE_EWORKSPACE;
-    hipStream_t st = as_stream(stream);
     char *ws = static_cast<char *>(workspace);
     uint32_t *keys_final = reinterpret_cast<uint32_t *>(ws + p.off_keys0);
     uint32_t *keys_tmp = reinterpret_cast<uint32_t *>(ws + p.off_keys1);
@@ -354,7 +540,6 @@ int kge_inspect(const int64_t *const *parts_in, const int64_t *part_len, int n_p
     uint32_t *heads = reinterpret_cast<uint32_t *>(ws + p.off_heads);
     const int nblocks = (int)p.nblocks;
     const int bins = 1 << p.digit_bits;
-
     if (n > 0) {
         const uint32_t *kin = nullptr;
         const int32_t *vin = nullptr;
@@ -381,6 +566,64 @@ int kge_inspect(const int64_t *const *parts_in, const int64_t *part_len, int n_p
                        heads, n > 0 ? nblocks : 0, *out);
     KGE_CHECK_LAUNCH();
     return KGE_OK;
+}
+
+int kge_inspect_batch(const kge_inspect_job *jobs, int n_jobs, void *stream)
+{
+    if (!jobs || n_jobs < 1 || n_jobs > 4) return KGE_EINVAL;
+    hipStream_t st = as_stream(stream);
+    Parts parts[4];
+    int64_t n[4];
+    for (int q = 0; q < n_jobs; ++q) {
+        const int rc = validate_job(&jobs[q], &parts[q], &n[q]);
+        if (rc) return rc;
+    }
+    SmallJobs small{};
+    int n_small = 0;
+    int64_t small_max = 0;
+    for (int q = 0; q < n_jobs; ++q) {
+        if (n[q] > kSmallMaxN) {
+            const int rc = inspect_large(parts[q], n[q], jobs[q].n_rows, &jobs[q].out, jobs[q].workspace, st);
+            if (rc) return rc;
+            continue;
+        }
+        const SortPlan p = make_plan(n[q], jobs[q].n_rows);
+        char *ws = static_cast<char *>(jobs[q].workspace);
+        SmallJob &J = small.j[n_small++];
+        J.parts = parts[q];
+        J.n = n[q];
+        J.bits = p.bits;
+        J.out = jobs[q].out;
+        J.keys_final = reinterpret_cast<uint32_t *>(ws + p.off_keys0);
+        J.keys_tmp = reinterpret_cast<uint32_t *>(ws + p.off_keys1);
+        J.vals_tmp = reinterpret_cast<int32_t *>(ws + p.off_vals);
+        small_max = n[q] > small_max ? n[q] : small_max;
+    }
+    if (n_small > 0) {
+        const dim3 grid(n_small), block(kSmallThreads);
+        if (small_max <= 8 * kSmallThreads)
+            hipLaunchKernelGGL(inspect_small_kernel<8>, grid, block, 0, st, small);
+        else if (small_max <= 16 * kSmallThreads)
+            hipLaunchKernelGGL(inspect_small_kernel<16>, grid, block, 0, st, small);
+        else
+            hipLaunchKernelGGL(inspect_small_kernel<32>, grid, block, 0, st, small);
+        KGE_CHECK_LAUNCH();
+    }
+    return KGE_OK;
+}
+
+int kge_inspect(const int64_t *const *parts_in, const int64_t *part_len, int n_parts, int64_t n_rows,
+                const kge_inspection *out, void *workspace, size_t workspace_bytes, void *stream)
+{
+    if (!out || !parts_in || !part_len || n_parts < 1 || n_parts > 4) return KGE_EINVAL;
+    kge_inspect_job job{};
+    for (int q = 0; q < n_parts; ++q) job.parts[q] = parts_in[q], job.part_len[q] = part_len[q];
+    job.n_parts = n_parts;
+    job.n_rows = n_rows;
+    job.out = *out;
+    job.workspace = workspace;
+    job.workspace_bytes = workspace_bytes;
+    return kge_inspect_batch(&job, 1, stream);
 }
 
 }  // extern "C"

@@ -759,6 +759,8 @@ int kge_score_bwd(const kge_tables *tab, const kge_batch *bat, const kge_saved *
     }
     if (rc) return rc;
 
+    if (bat->insp_ready && hipStreamWaitEvent(st, reinterpret_cast<hipEvent_t>(bat->insp_ready), 0) != hipSuccess)
+        return KGE_ELAUNCH;
     rc = launch_seg_reduce(occ_e, bat->ent_insp, (int)d, grads->ent_rows,
                            reinterpret_cast<float *>(ws + p.off_part_e), false, st);
     if (rc) return rc;

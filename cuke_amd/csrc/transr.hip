@@ -504,6 +504,8 @@ int launch_transr_bwd(const kge_tables *tab, const kge_batch *bat, const kge_sav
     DmArgs da{xs, qs, ri->num_unique, ri->seg_offsets, grads->aux_rows, d};
     hipLaunchKernelGGL(transr_dm_kernel, dim3((unsigned)(ceil_div(d, 32) * groups)), dim3(256), 0, st, da);
     KGE_CHECK_LAUNCH();
+    if (bat->insp_ready && hipStreamWaitEvent(st, reinterpret_cast<hipEvent_t>(bat->insp_ready), 0) != hipSuccess)
+        return KGE_ELAUNCH;
     int rc = launch_seg_reduce(occ, bat->ent_insp, d, grads->ent_rows, reinterpret_cast<float *>(ws + p.off_part_e),
                                false, st);
     if (rc || rescal) return rc;

@@ -195,7 +195,7 @@ class KGEModel:
         bat = _lib.Batch(B, h.data_ptr(), r.data_ptr(), t.data_ptr(),
                          neg.data_ptr() if neg is not None else None, C_, N,
                          C.pointer(ent_insp._c) if ent_insp is not None else None,
-                         C.pointer(rel_insp._c) if rel_insp is not None else None)
+                         C.pointer(rel_insp._c) if rel_insp is not None else None, None)
         return bat, (h, r, t, neg, C_, N)
 
     # -- reference-shaped output -------------------------------------------------------------
@@ -387,13 +387,21 @@ class TrainStep:
         n_occ = sum(int(p.numel()) for p in parts)
         self.ent_insp, self._ws_e = make_insp(n_occ, int(model.E.shape[0]))
         self.rel_insp, self._ws_r = make_insp(B, max(model.n_rel, 1))
-        self._parts_e = ((C.c_void_p * len(parts))(*[p.data_ptr() for p in parts]),
-                         (C.c_int64 * len(parts))(*[int(p.numel()) for p in parts]), len(parts))
-        self._parts_r = ((C.c_void_p * 1)(r.data_ptr()), (C.c_int64 * 1)(B), 1)
+        jobs = (_lib.InspectJob * 2)()
+        for job, ps, ins, ws in ((jobs[0], parts, self.ent_insp, self._ws_e), (jobs[1], [r], self.rel_insp, self._ws_r)):
+            for q, p_ in enumerate(ps):
+                job.parts[q], job.part_len[q] = p_.data_ptr(), int(p_.numel())
+            job.n_parts, job.n_rows, job.out = len(ps), ins.n_rows, ins._c
+            job.workspace, job.workspace_bytes = ws.data_ptr(), ws.numel()
+        self._jobs = jobs
+        # forward-only scoring needs no inspection unless the relation groups drive TransR / RESCAL
+        self.needs_rel_groups = model.model in ("TransR", "RESCAL")
 
         self.bat = _lib.Batch(B, h.data_ptr(), r.data_ptr(), t.data_ptr(),
                               neg.data_ptr() if neg is not None else None, C_, N,
-                              C.pointer(self.ent_insp._c), C.pointer(self.rel_insp._c))
+                              C.pointer(self.ent_insp._c), C.pointer(self.rel_insp._c), None)
+        self.side = torch.cuda.Stream(device=dev)  # default priority
+        self.insp_event = torch.cuda.Event()
         self.pos = torch.empty(B, **f32)
         self.neg = torch.empty((B, N), **f32) if neg is not None else None
         self.side_pos = torch.empty(B, **f32) if model.model == "TransH" else None
@@ -425,14 +433,12 @@ class TrainStep:
         self.graph = None
 
     # the individual stages, each one C call
-    def inspect(self, st):
-        L, ie, ir = self.L, self.ent_insp, self.rel_insp
-        p, l, n = self._parts_e
-        _lib.check(L.kge_inspect(p, l, n, ie.n_rows, C.byref(ie._c), _ptr(self._ws_e), self._ws_e.numel(), st),
-                   "kge_inspect(entities)")
-        p, l, n = self._parts_r
-        _lib.check(L.kge_inspect(p, l, n, ir.n_rows, C.byref(ir._c), _ptr(self._ws_r), self._ws_r.numel(), st),
-                   "kge_inspect(relations)")
+    def inspect(self, st, backward=True):
+        """Both inspections in one call; forward-only steps inspect r alone, and only if needed."""
+        if backward:
+            _lib.check(self.L.kge_inspect_batch(self._jobs, 2, st), "kge_inspect_batch")
+        elif self.needs_rel_groups:
+            _lib.check(self.L.kge_inspect_batch(C.byref(self._jobs[1]), 1, st), "kge_inspect_batch")
 
     def forward(self, st):
         _lib.check(self.L.kge_score_fwd(C.byref(self.m._tab), C.byref(self.bat), _ptr(self.pos), _ptr(self.neg),
@@ -450,13 +456,34 @@ class TrainStep:
                                         _ptr(self.dpos), _ptr(self.dneg), C.byref(self.grads), _ptr(self._ws_b),
                                         self._ws_b_bytes, st), "kge_score_bwd")
 
-    def run(self, backward=True):
-        st = _stream()
-        self.inspect(st)
+    def run(self, backward=True, overlap=True):
+        """Enqueue one step.  With overlap (default) the inspector runs on a side stream while
+        the main stream computes scores and per-occurrence gradients; backward waits for it
+        right before its segmented reduction.  TransR / RESCAL need the relation groups in the
+        forward pass, so their relation inspection stays on the main stream."""
+        main = torch.cuda.current_stream()
+        st = C.c_void_p(main.cuda_stream)
+        if not (backward and overlap):
+            self.bat.insp_ready = None
+            self.inspect(st, backward)
+            self.forward(st)
+            if backward:
+                self.loss_grad(st)
+                self.backward(st)
+            return
+        side = self.side
+        sst = C.c_void_p(side.cuda_stream)
+        side.wait_stream(main)
+        if self.needs_rel_groups:
+            _lib.check(self.L.kge_inspect_batch(C.byref(self._jobs[1]), 1, st), "kge_inspect_batch(relations)")
+            _lib.check(self.L.kge_inspect_batch(C.byref(self._jobs[0]), 1, sst), "kge_inspect_batch(entities)")
+        else:
+            _lib.check(self.L.kge_inspect_batch(self._jobs, 2, sst), "kge_inspect_batch")
+        self.insp_event.record(side)
+        self.bat.insp_ready = self.insp_event.cuda_event
         self.forward(st)
-        if backward:
-            self.loss_grad(st)
-            self.backward(st)
+        self.loss_grad(st)
+        self.backward(st)
 
     def capture(self, backward=True):
         """Record run() into a HIP graph; replay() then launches the whole step at once."""

@@ -104,6 +104,12 @@ typedef struct kge_batch {
        needed by kge_score_bwd; rel_insp also by TransR forward */
     const kge_inspection *ent_insp;
     const kge_inspection *rel_insp;
+    /* Optional hipEvent_t (as void*).  When set, the inspections may still be in flight on
+       another stream: kge_score_bwd makes its stream wait on this event immediately before
+       the first kernel that reads ent_insp (the segmented reduction), so the inspector runs
+       concurrently with the forward pass and the gradient tile kernels.  rel_insp is NOT
+       covered when the model is TransR / RESCAL (their forward already consumed it). */
+    void *insp_ready;
 } kge_batch;
 
 /* Forward outputs that backward consumes. */
@@ -165,6 +171,24 @@ size_t kge_inspect_workspace(int64_t n, int64_t n_rows);
 int kge_inspect(const int64_t *const *parts, const int64_t *part_len, int n_parts,
                 int64_t n_rows, const kge_inspection *out, void *workspace,
                 size_t workspace_bytes, void *stream);
+
+/*
+ * Several inspections in one call (at most 4 jobs).  Index sets of up to 32768 ids are each
+ * handled by a single workgroup and all of them share ONE kernel launch; larger sets run the
+ * multi-block sort.  Same outputs as kge_inspect.  A training step inspects concat(h, t, neg)
+ * and r together this way.
+ */
+typedef struct kge_inspect_job {
+    const int64_t *parts[4];  /* device pointers of the concatenated index arrays */
+    int64_t part_len[4];
+    int32_t n_parts;
+    int32_t reserved;
+    int64_t n_rows;
+    kge_inspection out;
+    void *workspace;          /* kge_inspect_workspace(n, n_rows) bytes */
+    size_t workspace_bytes;
+} kge_inspect_job;
+int kge_inspect_batch(const kge_inspect_job *jobs, int n_jobs, void *stream);
 
 /*
  * Margin-ranking loss over score pairs and its gradient:

@@ -127,3 +127,40 @@ def test_transh_l1_generic_floats_differ_only_by_sign_flips(oracle):
     bad = np.abs(got - want) > 1e-5 * np.abs(want) + 1e-5 * rms
     assert bad.mean() < 5e-3
     assert np.abs(got - want).max() < 16.0  # a handful of flips, each worth at most 2|g|
+
+
+@pytest.mark.parametrize("name,over", [
+    ("cfg2_distmult", dict(n_ent=50_000, batch=512)),
+    ("cfg4_rotate", dict(batch=256)),
+    ("cfg3_transr", dict(batch=1024)),
+])
+def test_train_step_eager_overlapped_and_graph_replays(oracle, name, over):
+    """The preallocated step: plain order, inspector overlapped on a side stream, and HIP-graph
+    replays (several, with eager work and synchronisation in between) all give the oracle's gradients."""
+    from cuke_amd.kge import TrainStep
+    w = synth.make_workload(name, **over)
+    a = w.arrays
+    m, ix = gpu_model(w)
+    sign = -1.0 if w.model == "TransR" else 1.0
+    step = TrainStep(m, ix["h"], ix["r"], ix["t"], ix.get("neg"), w.chunk or None, loss=w.loss,
+                     margin=w.margin, sign=sign)
+
+    def reference():
+        dpos, dneg = step.dpos.cpu().numpy(), (step.dneg.cpu().numpy() if step.dneg is not None else None)
+        return oracle.backward(w.model, a["E"], a["R"], a["A"], a["h"], a["r"], a["t"], a.get("neg"), w.chunk,
+                               dpos, dneg, p=w.norm_p)
+
+    def check(tag):
+        torch.cuda.synchronize()
+        ref = reference()
+        compare(step.sparse_grads(), ref, f"{name} {tag}", outliers=(1e-5, 4.0) if w.model == "RotatE" else None)
+        step.ent_rows.zero_()  # eager work between runs; also proves the next run rewrites everything
+
+    step.run(overlap=False)
+    check("in order")
+    step.run(overlap=True)
+    check("overlapped")
+    step.capture()
+    for i in range(3):
+        step.replay()
+        check(f"graph replay {i}")
