@@ -94,37 +94,55 @@ def time_events(fn, iters, torch):
     return a.elapsed_time(b) / iters
 
 
-def cpu_baseline(w, budget_s=20.0):
-    """The oracle's serial loops (the restatement of cuke's generated CPU code) timed on this
-    host on one chunk-sized sample of the same workload: forward + backward, one thread."""
+def cpu_baseline(w, target_s=12.0, cap_s=40.0):
+    """The oracle's loops (the restatement of cuke's generated CPU code; gcc -O3, ONE thread)
+    timed on this host over a bounded sample of the same workload: whole chunks of the batch
+    (same dim, chunk size, negatives and index distributions; entity table cut to 200k rows to
+    bound host memory), forward + backward, repeated until about `target_s` seconds of CPU
+    work have been spent.  Beside it: the forward pass alone with OpenMP over all host cores."""
     import oracle
     from cuke_amd import synth
     oracle.build()
     n_ent = min(w.n_ent, 200_000)
-    batch = w.chunk if w.chunk else min(w.batch, 1024)
-    over = dict(n_ent=n_ent, batch=batch)
-    if w.model == "TransH" and w.n_neg > 256:  # keep the sample within the time budget
-        over.update(n_neg=256)
-    s = synth.make_workload(w.name, seed=w.seed, **over)
+    unit = w.chunk if w.chunk else min(w.batch, 1024)
+    s = synth.make_workload(w.name, seed=w.seed, n_ent=n_ent)
     a = s.arrays
-    neg = a.get("neg")
-    t0 = time.perf_counter()
-    pos, negs = oracle.score(s.model, a["E"], a["R"], a["A"], a["h"], a["r"], a["t"], neg, s.chunk,
-                             p=s.norm_p, gamma=s.gamma, fast=True)
-    t_fwd = time.perf_counter() - t0
-    dpos = np.ones_like(pos)
-    dneg = np.ones_like(negs) if negs is not None else None
-    t0 = time.perf_counter()
-    if s.backward:
-        oracle.backward(s.model, a["E"], a["R"], a["A"], a["h"], a["r"], a["t"], neg, s.chunk, dpos, dneg,
-                        p=s.norm_p)
-    t_bwd = time.perf_counter() - t0
-    scores = s.scores_per_step
-    return {"value": scores / (t_fwd + t_bwd), "unit": "triples scored/s", "cores": 1, "kind": "port",
-            "sample": f"{s.model} B={s.batch} N={s.n_neg} dim={s.dim} n_ent={s.n_ent}: "
-                      f"fwd {t_fwd:.2f}s (gcc -O3, {oracle.threads()} OpenMP threads over the batch loop) "
-                      f"+ bwd {t_bwd:.2f}s (gcc -O2 serial)",
-            "fwd_s": t_fwd, "bwd_s": t_bwd}
+
+    def run(b0, b1, fast):
+        sl = slice(b0, b1)
+        neg = a["neg"][(b0 // s.chunk) * s.n_neg:(b1 // s.chunk) * s.n_neg] if s.chunk else None
+        t0 = time.perf_counter()
+        pos, negs = oracle.score(s.model, a["E"], a["R"], a["A"], a["h"][sl], a["r"][sl], a["t"][sl], neg,
+                                 s.chunk, p=s.norm_p, gamma=s.gamma, fast=fast)
+        tf = time.perf_counter() - t0
+        tb = 0.0
+        if s.backward and fast == "o3":
+            dneg = np.ones_like(negs) if negs is not None else None
+            t0 = time.perf_counter()
+            oracle.backward(s.model, a["E"], a["R"], a["A"], a["h"][sl], a["r"][sl], a["t"][sl], neg, s.chunk,
+                            np.ones_like(pos), dneg, p=s.norm_p, fast="o3")
+            tb = time.perf_counter() - t0
+        return tf, tb
+
+    t_fwd = t_bwd = 0.0
+    scored = 0
+    done = 0
+    while True:
+        b0 = (done * unit) % s.batch
+        tf, tb = run(b0, b0 + unit, "o3")
+        t_fwd, t_bwd, done = t_fwd + tf, t_bwd + tb, done + 1
+        scored += unit * (1 + s.n_neg)
+        spent = t_fwd + t_bwd
+        if spent >= target_s or spent + spent / done > cap_s:
+            break
+    run(0, unit, "omp")  # first call starts the OpenMP thread pool
+    tf_omp, _ = run(0, unit, "omp")
+    return {"value": scored / (t_fwd + t_bwd), "unit": "triples scored/s", "cores": 1, "kind": "port",
+            "sample": f"{s.model} dim={s.dim} n_ent={s.n_ent}: {done} x (B={unit}, N={s.n_neg}) = {scored} scores, "
+                      f"fwd {t_fwd:.2f}s + bwd {t_bwd:.2f}s, gcc -O3 -march=x86-64-v3, 1 thread",
+            "fwd_s": t_fwd, "bwd_s": t_bwd,
+            "forward_only_openmp": {"value": unit * (1 + s.n_neg) / tf_omp, "unit": "triples scored/s",
+                                    "cores": oracle.threads("omp")}}
 
 
 def main():
@@ -136,6 +154,9 @@ def main():
     ap.add_argument("--no-graph", action="store_true", help="launch kernels one by one instead of a HIP graph")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--seed", type=int, default=0)
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="also run one 256 MiB device-to-device copy kernel (a known-traffic reference "
+                         "for scaling rocprofv3 FETCH_SIZE / WRITE_SIZE counters)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on one GPU; --gpus must be 1 (nothing here shards across GPUs)",
@@ -147,6 +168,12 @@ def main():
     from cuke_amd.kge import KGEModel, TrainStep
 
     dev = torch.device("cuda:0")
+    if args.calibrate_copy:
+        src = torch.empty(64 * 1024 * 1024, dtype=torch.float32, device=dev).normal_()
+        dst = torch.empty_like(src)
+        dst.copy_(src)  # one elementwise copy kernel: reads 256 MiB, writes 256 MiB
+        torch.cuda.synchronize()
+        del src, dst
     w = synth.make_workload(args.workload, seed=args.seed, tables=False)
     E, R, A = device_tables(w, dev)
     model = KGEModel(w.model, E, R, A, norm_p=w.norm_p, gamma=w.gamma)

@@ -30,8 +30,8 @@ def sources() -> list[str]:
 
 def _compile(src: str, force: bool) -> str:
     obj = os.path.join(OBJ, src[:-4] + ".o")
-    deps = [os.path.join(CSRC, src), os.path.join(CSRC, "common.hpp"),
-            os.path.join(HERE, "..", "include", "kge_mi355.h")]
+    deps = [os.path.join(CSRC, src), os.path.join(HERE, "..", "include", "kge_mi355.h")] + \
+        [os.path.join(CSRC, f) for f in os.listdir(CSRC) if f.endswith(".hpp")]
     if not force and os.path.exists(obj) and all(os.path.getmtime(obj) > os.path.getmtime(d) for d in deps):
         return obj
     cmd = [HIPCC, *FLAGS, "-c", os.path.join(CSRC, src), "-o", obj]

@@ -13,6 +13,7 @@
 //      (inspection perm / seg_offsets); every output row is written exactly once.
 #include <stdlib.h>
 
+#include "seg_reduce.hpp"
 #include "tile_common.hpp"
 
 namespace kge {
@@ -31,7 +32,7 @@ struct TileArgs {
     const float *side_neg;  // TransH: [2, B, N]
     float *out0, *out1;
     int64_t plane;  // B * N
-    int C, N, d, rel_dim, vec, vecn;
+    int C, N, d, rel_dim, vec, vecn, n_chunks;
 };
 
 constexpr int kTI = 64;       // columns of the row per workgroup
@@ -57,12 +58,13 @@ __global__ __launch_bounds__(256) void bwd_tile_kernel(TileArgs a)
     __shared__ __align__(16) float sG[NC][kKL][PG];
 
     const int tid = threadIdx.x, tx = tid & 15, ty = tid >> 4;
-    const int c = blockIdx.z;
     const int d = a.d, half = d >> 1;
     const int klen = pair_len<MODEL>(d);
-    const int col = blockIdx.x * kTI + tx * 4;
-    const int ot0 = blockIdx.y * TO;
     const int n_own = OWNER_POS ? a.C : a.N, n_loop = OWNER_POS ? a.N : a.C;
+    int c, tile_y, tile_x;
+    if (!xcd_tile((klen + kTI - 1) / kTI, (n_own + TO - 1) / TO, a.n_chunks, c, tile_y, tile_x)) return;
+    const int col = tile_x * kTI + tx * 4;
+    const int ot0 = tile_y * TO;
     const bool vec = a.vec != 0;
 
     // ---- owners: registers -----------------------------------------------------------
@@ -286,10 +288,10 @@ static int launch_tile_o(const TileArgs &a, int64_t n_chunks, hipStream_t st)
     const int64_t big = (int64_t)gx * ceil_div(n_own, 64) * n_chunks;
     if (big >= 1024) {
         hipLaunchKernelGGL((bwd_tile_kernel<MODEL, P, OWNER_POS, 4>),
-                           dim3(gx, (unsigned)ceil_div(n_own, 64), (unsigned)n_chunks), dim3(256), 0, st, a);
+                           dim3(xcd_grid(gx, ceil_div(n_own, 64), n_chunks)), dim3(256), 0, st, a);
     } else {
         hipLaunchKernelGGL((bwd_tile_kernel<MODEL, P, OWNER_POS, 2>),
-                           dim3(gx, (unsigned)ceil_div(n_own, 32), (unsigned)n_chunks), dim3(256), 0, st, a);
+                           dim3(xcd_grid(gx, ceil_div(n_own, 32), n_chunks)), dim3(256), 0, st, a);
     }
     KGE_CHECK_LAUNCH();
     return KGE_OK;
@@ -495,130 +497,6 @@ static int launch_pos_bwd(const PosBwdArgs &a, bool vec4, hipStream_t st)
     return KGE_OK;
 }
 
-// ---------------------------------------------------------------------------------------
-// 4: segmented reduction of occurrence rows in sorted order
-// ---------------------------------------------------------------------------------------
-constexpr int kSegL = 32;  // sorted positions per wave
-
-struct SegArgs {
-    const float *occ;  // [n, d]
-    const int32_t *perm, *sorted_seg, *seg_offsets;
-    int64_t n;
-    int d;
-    float *out;      // [U, d]
-    float *partial;  // [ceil(n / kSegL), 2, d]
-};
-
-// Level 1: wave j sums positions [j*L, (j+1)*L) run by run.  A run that lies wholly inside
-// the block is final and written to its output row; a run that started in an earlier block
-// goes to partial slot 0, one that continues into the next block to partial slot 1.
-template <int V>
-__global__ __launch_bounds__(256) void seg_reduce_l1(SegArgs a)
-{
-    const int lane = threadIdx.x & (kWave - 1);
-    const int64_t j = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
-    const int64_t p0 = j * kSegL;
-    if (p0 >= a.n) return;
-    const int cnt = (int)((a.n - p0) < kSegL ? (a.n - p0) : kSegL);
-    const int my_src = lane < cnt ? (a.perm ? a.perm[p0 + lane] : (int)(p0 + lane)) : 0;
-    const int my_seg = lane < cnt ? a.sorted_seg[p0 + lane] : -1;
-    const int d = a.d;
-
-    for (int c0 = 0; c0 < d; c0 += kWave * V) {
-        const int colv = c0 + lane * V;
-        const bool active = colv < d;
-        Vec<V> acc;
-#pragma unroll
-        for (int e = 0; e < V; ++e) acc.v[e] = 0.0f;
-        int cur = __shfl(my_seg, 0, kWave);
-
-        auto flush = [&](int seg) {
-            const int s0 = a.seg_offsets[seg], s1 = a.seg_offsets[seg + 1];
-            float *dst;
-            if (s0 >= p0 && s1 <= p0 + kSegL) dst = a.out + (int64_t)seg * d;
-            else dst = a.partial + (j * 2 + (s0 < p0 ? 0 : 1)) * (int64_t)d;
-            if (active) acc.store(dst + colv);
-        };
-
-        for (int q0 = 0; q0 < cnt; q0 += 8) {
-            Vec<V> v[8];
-#pragma unroll
-            for (int u = 0; u < 8; ++u) {
-                const int q = q0 + u;
-                const int src = __shfl(my_src, q < cnt ? q : cnt - 1, kWave);
-                if (active && q < cnt) v[u] = Vec<V>::load(a.occ + (int64_t)src * d + colv);
-                else
-#pragma unroll
-                    for (int e = 0; e < V; ++e) v[u].v[e] = 0.0f;
-            }
-#pragma unroll
-            for (int u = 0; u < 8; ++u) {
-                const int q = q0 + u;
-                if (q < cnt) {
-                    const int sg = __shfl(my_seg, q, kWave);
-                    if (sg != cur) {
-                        flush(cur);
-#pragma unroll
-                        for (int e = 0; e < V; ++e) acc.v[e] = 0.0f;
-                        cur = sg;
-                    }
-#pragma unroll
-                    for (int e = 0; e < V; ++e) acc.v[e] += v[u].v[e];
-                }
-            }
-        }
-        flush(cur);
-    }
-}
-
-// Level 2: block j owns the run that starts inside it and continues past its end; it adds
-// that run's slot-1 partial and the slot-0 partials of the following blocks.
-template <int V>
-__global__ __launch_bounds__(256) void seg_reduce_l2(SegArgs a)
-{
-    const int lane = threadIdx.x & (kWave - 1);
-    const int64_t j = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
-    const int64_t p0 = j * kSegL;
-    if (p0 >= a.n) return;
-    const int64_t p1 = p0 + kSegL < a.n ? p0 + kSegL : a.n;
-    const int seg = a.sorted_seg[p1 - 1];
-    const int s0 = a.seg_offsets[seg], s1 = a.seg_offsets[seg + 1];
-    if (s1 <= p0 + kSegL || s0 < p0) return;
-    const int64_t je = (s1 - 1) / kSegL;
-    const int d = a.d;
-    for (int c0 = 0; c0 < d; c0 += kWave * V) {
-        const int colv = c0 + lane * V;
-        if (colv >= d) continue;
-        Vec<V> acc = Vec<V>::load(a.partial + (j * 2 + 1) * (int64_t)d + colv);
-        for (int64_t jj = j + 1; jj <= je; ++jj) {
-            const Vec<V> v = Vec<V>::load(a.partial + (jj * 2) * (int64_t)d + colv);
-#pragma unroll
-            for (int e = 0; e < V; ++e) acc.v[e] += v.v[e];
-        }
-        acc.store(a.out + (int64_t)seg * d + colv);
-    }
-}
-
-// identity_perm: the occurrence rows are already stored in sorted order
-int launch_seg_reduce(const float *occ, const kge_inspection *ins, int d, float *out, float *partial,
-                      bool identity_perm, hipStream_t st)
-{
-    if (ins->n == 0 || d == 0) return KGE_OK;
-    SegArgs a{occ, identity_perm ? nullptr : ins->perm, ins->sorted_seg, ins->seg_offsets, ins->n, d, out, partial};
-    const int64_t nblk = ceil_div(ins->n, kSegL);
-    const dim3 grid((unsigned)ceil_div(nblk, 4)), block(256);
-    const bool v4 = d % 4 == 0 && aligned16(occ) && aligned16(out) && aligned16(partial);
-    if (v4) {
-        hipLaunchKernelGGL(seg_reduce_l1<4>, grid, block, 0, st, a);
-        hipLaunchKernelGGL(seg_reduce_l2<4>, grid, block, 0, st, a);
-    } else {
-        hipLaunchKernelGGL(seg_reduce_l1<1>, grid, block, 0, st, a);
-        hipLaunchKernelGGL(seg_reduce_l2<1>, grid, block, 0, st, a);
-    }
-    KGE_CHECK_LAUNCH();
-    return KGE_OK;
-}
-
 __global__ void fill_zero_kernel(float *p, int64_t n)
 {
     for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (int64_t)gridDim.x * blockDim.x)
@@ -650,9 +528,9 @@ static BwdPlan make_bwd_plan(const kge_tables *tab, const kge_batch *bat)
     p.off_occ_w = take(tab->model == KGE_TRANSH ? B * d : 0);
     p.off_g0 = take(bat->neg ? B * d : 0);
     p.off_g1 = take(bat->neg && tab->model == KGE_TRANSH ? B * d : 0);
-    p.off_part_e = take(ceil_div(p.n_occ, kSegL) * 2 * d);
-    p.off_part_r = take(ceil_div(B, kSegL) * 2 * rd);
-    p.off_part_w = take(tab->model == KGE_TRANSH ? ceil_div(B, kSegL) * 2 * d : 0);
+    p.off_part_e = take(seg_partial_floats(p.n_occ, d));
+    p.off_part_r = take(seg_partial_floats(B, rd));
+    p.off_part_w = take(tab->model == KGE_TRANSH ? seg_partial_floats(B, d) : 0);
     p.total = o;
     return p;
 }
@@ -716,12 +594,12 @@ int kge_score_bwd(const kge_tables *tab, const kge_batch *bat, const kge_saved *
 
     if (have_neg) {
         const int64_t n_chunks = B / bat->chunk;
-        if (n_chunks > 65535) return KGE_ESHAPE;
+        if (n_chunks >= (1 << 24)) return KGE_ESHAPE;
         const bool vecn = bat->n_neg % 4 == 0 && aligned16(dneg) && (!saved->neg || aligned16(saved->neg)) &&
                           (!saved->side_neg || aligned16(saved->side_neg));
         TileArgs a{tab->ent, tab->rel, tab->aux, bat->h, bat->r, bat->neg, dneg, saved->neg, saved->side_pos,
                    saved->side_neg, nullptr, nullptr, B * bat->n_neg, (int)bat->chunk, (int)bat->n_neg, (int)d,
-                   (int)tab->rel_dim, vec ? 1 : 0, vecn ? 1 : 0};
+                   (int)tab->rel_dim, vec ? 1 : 0, vecn ? 1 : 0, (int)n_chunks};
         float *occ_neg = occ_e + 2 * B * d;
         switch (model) {
         case KGE_TRANSE:
@@ -761,16 +639,11 @@ int kge_score_bwd(const kge_tables *tab, const kge_batch *bat, const kge_saved *
 
     if (bat->insp_ready && hipStreamWaitEvent(st, reinterpret_cast<hipEvent_t>(bat->insp_ready), 0) != hipSuccess)
         return KGE_ELAUNCH;
-    rc = launch_seg_reduce(occ_e, bat->ent_insp, (int)d, grads->ent_rows,
-                           reinterpret_cast<float *>(ws + p.off_part_e), false, st);
-    if (rc) return rc;
-    rc = launch_seg_reduce(occ_r, bat->rel_insp, (int)tab->rel_dim, grads->rel_rows,
-                           reinterpret_cast<float *>(ws + p.off_part_r), false, st);
-    if (rc) return rc;
-    if (model == KGE_TRANSH)
-        rc = launch_seg_reduce(occ_w, bat->rel_insp, (int)d, grads->aux_rows,
-                               reinterpret_cast<float *>(ws + p.off_part_w), false, st);
-    return rc;
+    const SegJob jobs[3] = {
+        {occ_e, bat->ent_insp, (int)d, grads->ent_rows, reinterpret_cast<float *>(ws + p.off_part_e), false},
+        {occ_r, bat->rel_insp, (int)tab->rel_dim, grads->rel_rows, reinterpret_cast<float *>(ws + p.off_part_r), false},
+        {occ_w, bat->rel_insp, (int)d, grads->aux_rows, reinterpret_cast<float *>(ws + p.off_part_w), false}};
+    return launch_seg_reduce_jobs(jobs, model == KGE_TRANSH ? 3 : 2, st);
 }
 
 }  // extern "C"

@@ -25,7 +25,7 @@ struct NegArgs {
     int64_t plane;          // B * N
     int C, N, d, rel_dim;
     float gamma;
-    int vec;
+    int vec, n_chunks;
 };
 
 constexpr int kKD = 32;        // floats of each row staged per step
@@ -70,7 +70,9 @@ __global__ __launch_bounds__(256) void score_neg_kernel(NegArgs a)
 
     const int tid = threadIdx.x, tx = tid & 15, ty = tid >> 4;
     const int srow = tid >> 3, scol = (tid & 7) * 4;
-    const int c = blockIdx.z, bt0 = blockIdx.y * TB, kt0 = blockIdx.x * TN;
+    int c, tile_y, tile_x;
+    if (!xcd_tile((a.N + TN - 1) / TN, (a.C + TB - 1) / TB, a.n_chunks, c, tile_y, tile_x)) return;
+    const int bt0 = tile_y * TB, kt0 = tile_x * TN;
     const int d = a.d, half = d >> 1;
     const int klen = MODEL == KGE_ROTATE ? half : d;
     const bool vec = a.vec != 0;
@@ -220,13 +222,13 @@ static int launch_neg_mp(const NegArgs &a, int64_t n_chunks, hipStream_t st)
     int tile = neg_tile_override();
     if (tile != 2 && tile != 4) tile = big_tiles >= 1024 ? 4 : 2;
     if (tile == 4) {
-        const dim3 grid((unsigned)ceil_div(a.N, 64), (unsigned)ceil_div(a.C, 64), (unsigned)n_chunks);
+        const dim3 grid(xcd_grid(ceil_div(a.N, 64), ceil_div(a.C, 64), n_chunks));
         if (MODEL == KGE_TRANSH && a.side_neg)
             hipLaunchKernelGGL((score_neg_kernel<MODEL, P, 4, 4, true>), grid, dim3(256), 0, st, a);
         else
             hipLaunchKernelGGL((score_neg_kernel<MODEL, P, 4, 4, false>), grid, dim3(256), 0, st, a);
     } else {
-        const dim3 grid((unsigned)ceil_div(a.N, 32), (unsigned)ceil_div(a.C, 32), (unsigned)n_chunks);
+        const dim3 grid(xcd_grid(ceil_div(a.N, 32), ceil_div(a.C, 32), n_chunks));
         if (MODEL == KGE_TRANSH && a.side_neg)
             hipLaunchKernelGGL((score_neg_kernel<MODEL, P, 2, 2, true>), grid, dim3(256), 0, st, a);
         else
@@ -241,10 +243,10 @@ int launch_score_neg(const kge_tables *tab, const kge_batch *bat, const float *s
 {
     if (bat->batch == 0) return KGE_OK;
     const int64_t n_chunks = bat->batch / bat->chunk;
-    if (n_chunks > 65535 || bat->chunk >= (1 << 30) || bat->n_neg >= (1 << 30)) return KGE_ESHAPE;
+    if (n_chunks >= (1 << 24) || bat->chunk >= (1 << 30) || bat->n_neg >= (1 << 30)) return KGE_ESHAPE;
     const bool vec = rows_vectorizable(tab);
     NegArgs a{tab->ent, tab->rel, tab->aux, bat->h, bat->r, bat->neg, side_pos, out, side_neg,
-              bat->batch * bat->n_neg, (int)bat->chunk, (int)bat->n_neg, (int)tab->dim, (int)tab->rel_dim, tab->gamma, vec ? 1 : 0};
+              bat->batch * bat->n_neg, (int)bat->chunk, (int)bat->n_neg, (int)tab->dim, (int)tab->rel_dim, tab->gamma, vec ? 1 : 0, (int)n_chunks};
     const int p = tab->norm_p;
     switch (tab->model) {
     case KGE_TRANSE:

@@ -1,0 +1,168 @@
+// Atomic-free segmented reduction: the backward pass produces one gradient row per OCCURRENCE
+// of a table row; the inspection's stable sort puts the occurrences of one id next to each
+// other, and each output row is the sum of its run, written exactly once.
+//
+// Level 1: a wave owns kSegL consecutive sorted positions (and one 256-float column chunk of
+// the rows).  All its row loads are issued at once; then the positions are walked in order.
+// A run that lies wholly inside the block is final.  A run that began in an earlier block is
+// stored to partial slot 0 of the block, one that continues past the block to slot 1.
+// Level 2: the block in which a long run STARTS adds that run's slot-1 partial and the slot-0
+// partials of the following blocks (four waves share the blocks, combined through LDS).
+// The summation order is fixed by the sorted order, so results are deterministic.
+#include "seg_reduce.hpp"
+
+namespace kge {
+
+struct SegArgs {
+    const float *occ;
+    const int32_t *perm, *sorted_seg, *seg_offsets;
+    int64_t n;
+    int d;
+    float *out, *partial;
+};
+struct SegArgs3 {
+    SegArgs j[3];
+};
+
+template <int V>
+__global__ __launch_bounds__(256) void seg_reduce_l1(SegArgs3 jobs)
+{
+    const SegArgs &a = jobs.j[blockIdx.y];
+    const int lane = threadIdx.x & (kWave - 1);
+    const int d = a.d;
+    const int nch = (d + kWave * V - 1) / (kWave * V);
+    const int64_t w = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    const int64_t j = w / nch;
+    const int colv = (int)(w % nch) * kWave * V + lane * V;
+    const int64_t p0 = j * kSegL;
+    if (p0 >= a.n) return;
+    const int cnt = (int)((a.n - p0) < kSegL ? (a.n - p0) : kSegL);
+    const bool active = colv < d;
+
+    int seg[kSegL];
+    Vec<V> v[kSegL];
+#pragma unroll
+    for (int q = 0; q < kSegL; ++q) {
+        const bool ok = q < cnt;
+        const int64_t p = p0 + (ok ? q : 0);
+        const int src = a.perm ? a.perm[p] : (int)p;
+        seg[q] = ok ? a.sorted_seg[p] : -1;
+        if (ok && active) v[q] = Vec<V>::load(a.occ + (int64_t)src * d + colv);
+        else
+#pragma unroll
+            for (int e = 0; e < V; ++e) v[q].v[e] = 0.0f;
+    }
+    Vec<V> acc;
+#pragma unroll
+    for (int e = 0; e < V; ++e) acc.v[e] = 0.0f;
+    int cur = seg[0];
+    auto flush = [&](int sg) {
+        const int s0 = a.seg_offsets[sg], s1 = a.seg_offsets[sg + 1];
+        float *dst;
+        if (s0 >= p0 && s1 <= p0 + kSegL) dst = a.out + (int64_t)sg * d;
+        else dst = a.partial + (j * 2 + (s0 < p0 ? 0 : 1)) * (int64_t)d;
+        if (active) acc.store(dst + colv);
+    };
+#pragma unroll
+    for (int q = 0; q < kSegL; ++q) {
+        if (q < cnt) {
+            if (seg[q] != cur) {
+                flush(cur);
+#pragma unroll
+                for (int e = 0; e < V; ++e) acc.v[e] = 0.0f;
+                cur = seg[q];
+            }
+#pragma unroll
+            for (int e = 0; e < V; ++e) acc.v[e] += v[q].v[e];
+        }
+    }
+    flush(cur);
+}
+
+template <int V>
+__global__ __launch_bounds__(256) void seg_reduce_l2(SegArgs3 jobs)
+{
+    __shared__ float s_part[4][kWave * 4];
+    const SegArgs &a = jobs.j[blockIdx.y];
+    const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x >> 6;
+    const int64_t j = blockIdx.x;
+    const int64_t p0 = j * kSegL;
+    if (p0 >= a.n) return;  // uniform for the workgroup
+    const int64_t p1 = p0 + kSegL < a.n ? p0 + kSegL : a.n;
+    const int sg = a.sorted_seg[p1 - 1];
+    const int s0 = a.seg_offsets[sg], s1 = a.seg_offsets[sg + 1];
+    if (s1 <= p0 + kSegL || s0 < p0) return;  // no run starts here and continues
+    const int64_t je = (s1 - 1) / kSegL;
+    const int d = a.d;
+    for (int c0 = 0; c0 < d; c0 += kWave * V) {
+        const int colv = c0 + lane * V;
+        const bool active = colv < d;
+        Vec<V> acc;
+#pragma unroll
+        for (int e = 0; e < V; ++e) acc.v[e] = 0.0f;
+        for (int64_t jj = j + 1 + wave; jj <= je; jj += 16) {  // four loads in flight per wave
+            Vec<V> t[4];
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+                const int64_t jb = jj + 4 * u;
+                if (active && jb <= je) t[u] = Vec<V>::load(a.partial + (jb * 2) * (int64_t)d + colv);
+                else
+#pragma unroll
+                    for (int e = 0; e < V; ++e) t[u].v[e] = 0.0f;
+            }
+#pragma unroll
+            for (int u = 0; u < 4; ++u)
+#pragma unroll
+                for (int e = 0; e < V; ++e) acc.v[e] += t[u].v[e];
+        }
+#pragma unroll
+        for (int e = 0; e < V; ++e) s_part[wave][lane * V + e] = acc.v[e];
+        __syncthreads();
+        if (wave == 0 && active) {
+            Vec<V> r = Vec<V>::load(a.partial + (j * 2 + 1) * (int64_t)d + colv);
+#pragma unroll
+            for (int e = 0; e < V; ++e)
+                r.v[e] += (s_part[0][lane * V + e] + s_part[1][lane * V + e]) +
+                          (s_part[2][lane * V + e] + s_part[3][lane * V + e]);
+            r.store(a.out + (int64_t)sg * d + colv);
+        }
+        __syncthreads();
+    }
+}
+
+int launch_seg_reduce_jobs(const SegJob *jobs, int n_jobs, hipStream_t st)
+{
+    SegArgs3 args{};
+    int m = 0;
+    int64_t max_waves = 0, max_blocks = 0;
+    bool v4 = true;
+    for (int q = 0; q < n_jobs && m < 3; ++q) {
+        const SegJob &jb = jobs[q];
+        if (!jb.ins || jb.ins->n == 0 || jb.d == 0) continue;
+        args.j[m] = SegArgs{jb.occ, jb.identity_perm ? nullptr : jb.ins->perm, jb.ins->sorted_seg,
+                            jb.ins->seg_offsets, jb.ins->n, jb.d, jb.out, jb.partial};
+        v4 = v4 && jb.d % 4 == 0 && aligned16(jb.occ) && aligned16(jb.out) && aligned16(jb.partial);
+        ++m;
+    }
+    if (m == 0) return KGE_OK;
+    for (int q = 0; q < m; ++q) {
+        const int V = v4 ? 4 : 1;
+        const int64_t nblk = ceil_div(args.j[q].n, kSegL);
+        const int64_t nch = ceil_div(args.j[q].d, kWave * V);
+        max_waves = nblk * nch > max_waves ? nblk * nch : max_waves;
+        max_blocks = nblk > max_blocks ? nblk : max_blocks;
+    }
+    for (int q = m; q < 3; ++q) args.j[q] = args.j[0], args.j[q].n = 0;  // unused slots do nothing
+    const dim3 g1((unsigned)ceil_div(max_waves, 4), (unsigned)m), g2((unsigned)max_blocks, (unsigned)m), block(256);
+    if (v4) {
+        hipLaunchKernelGGL(seg_reduce_l1<4>, g1, block, 0, st, args);
+        hipLaunchKernelGGL(seg_reduce_l2<4>, g2, block, 0, st, args);
+    } else {
+        hipLaunchKernelGGL(seg_reduce_l1<1>, g1, block, 0, st, args);
+        hipLaunchKernelGGL(seg_reduce_l2<1>, g2, block, 0, st, args);
+    }
+    KGE_CHECK_LAUNCH();
+    return KGE_OK;
+}
+
+}  // namespace kge

@@ -1,0 +1,24 @@
+// Segmented reduction of per-occurrence gradient rows into one row per distinct id.
+#pragma once
+
+#include "common.hpp"
+
+namespace kge {
+
+constexpr int kSegL = 8;  // sorted positions per level-1 wave
+
+struct SegJob {
+    const float *occ;            // [n, d] occurrence rows
+    const kge_inspection *ins;   // sorted order / runs of the ids the rows belong to
+    int d;
+    float *out;                  // [U, d]
+    float *partial;              // seg_partial_floats(n, d) floats of scratch
+    bool identity_perm;          // occ is already stored in sorted order
+};
+
+inline int64_t seg_partial_floats(int64_t n, int64_t d) { return ceil_div(n > 0 ? n : 1, kSegL) * 2 * d; }
+
+// Up to three jobs share the same two launches.
+int launch_seg_reduce_jobs(const SegJob *jobs, int n_jobs, hipStream_t st);
+
+}  // namespace kge

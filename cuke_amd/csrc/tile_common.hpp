@@ -117,6 +117,27 @@ __device__ __forceinline__ void load_query(const float *ph, const float *pr, con
     }
 }
 
+// XCD-aware tile placement.  The 256 CUs sit in 8 XCDs with one L2 each, and consecutive
+// workgroup ids of a 1-D grid go to consecutive XCDs.  All tiles of one chunk share that
+// chunk's positive and negative rows, so they are steered to one XCD (chunk c -> XCD c % 8):
+// every gathered row is then fetched from HBM by a single L2 instead of by up to eight.
+// Grid: 8 * ceil(n_chunks / 8) * tiles_per_chunk workgroups; returns false for padding ids.
+constexpr int kXcds = 8;
+__device__ __forceinline__ bool xcd_tile(int tiles_x, int tiles_y, int n_chunks, int &c, int &ty, int &tx)
+{
+    const int lid = blockIdx.x, per = tiles_x * tiles_y;
+    const int xcd = lid % kXcds, k = lid / kXcds;
+    c = (k / per) * kXcds + xcd;
+    const int t = k % per;
+    ty = t / tiles_x;
+    tx = t % tiles_x;
+    return c < n_chunks;
+}
+inline unsigned xcd_grid(int64_t tiles_x, int64_t tiles_y, int64_t n_chunks)
+{
+    return (unsigned)(kXcds * ceil_div(n_chunks, kXcds) * tiles_x * tiles_y);
+}
+
 inline bool rows_vectorizable(const kge_tables *tab)
 {
     const bool complex_rows = tab->model == KGE_COMPLEX || tab->model == KGE_ROTATE;

@@ -15,56 +15,92 @@
 //   * j: a lane's float4 of four consecutive matrix columns feeds four MFMAs (one per element),
 //     so MFMA e owns columns n0 + 4 (l % 16) + e.
 #include "common.hpp"
+#include "seg_reduce.hpp"
 
 namespace kge {
 
 typedef float floatx4 __attribute__((ext_vector_type(4)));
 
 constexpr int kTM = 32;          // triples per tile
+constexpr int kRing = 2;         // supersteps of B operands kept in flight per wave
 constexpr int kMaxDimMfma = 1024;
 
 int launch_score_pos(const kge_tables *, const kge_batch *, float *, float *, float *, hipStream_t);
 
-// ---- tile plan: one entry per (relation group, block of 32 sorted positions) ---------------
+// ---- tile plan: one entry per (relation group, block of `tile` sorted positions) -----------
 struct TilePlan {
     int32_t *num_tiles;  // [1]
     int32_t *tile_seg;   // [max_tiles] group (unique-relation index)
     int32_t *tile_p0;    // [max_tiles] first sorted position
+    // groups longer than one tile ("split" groups, used by the dM kernel): every tile of such
+    // a group writes a partial result to slot tile_part[tile]; -1 for unsplit groups
+    int32_t *tile_part;   // [max_tiles] or null
+    int32_t *num_split;   // [1]
+    int32_t *split_seg;   // [max_split] group of the split
+    int32_t *split_first; // [max_split] first partial slot
+    int32_t *split_cnt;   // [max_split] number of partial slots
 };
 
+__device__ int block_inclusive_scan_1024(int v, int *s_scan)
+{
+    s_scan[threadIdx.x] = v;
+    __syncthreads();
+    for (int o = 1; o < 1024; o <<= 1) {  // Hillis-Steele
+        const int u = (int)threadIdx.x >= o ? s_scan[threadIdx.x - o] : 0;
+        __syncthreads();
+        s_scan[threadIdx.x] += u;
+        __syncthreads();
+    }
+    const int r = s_scan[threadIdx.x];
+    __syncthreads();
+    return r;
+}
+
 __global__ __launch_bounds__(1024) void transr_plan_kernel(const int32_t *num_unique, const int32_t *seg_offsets,
-                                                          TilePlan plan)
+                                                          TilePlan plan, int tile)
 {
     __shared__ int s_scan[1024];
-    __shared__ int s_carry;
+    __shared__ int s_carry[3];
     const int U = num_unique[0];
-    if (threadIdx.x == 0) s_carry = 0;
+    if (threadIdx.x < 3) s_carry[threadIdx.x] = 0;
     __syncthreads();
     for (int base = 0; base < U; base += 1024) {
         const int g = base + threadIdx.x;
         int s0 = 0, cnt = 0;
         if (g < U) {
             s0 = seg_offsets[g];
-            cnt = (seg_offsets[g + 1] - s0 + kTM - 1) / kTM;
+            cnt = (seg_offsets[g + 1] - s0 + tile - 1) / tile;
         }
-        s_scan[threadIdx.x] = cnt;
-        __syncthreads();
-        for (int o = 1; o < 1024; o <<= 1) {  // Hillis-Steele inclusive scan
-            const int v = (int)threadIdx.x >= o ? s_scan[threadIdx.x - o] : 0;
+        const int inc_t = block_inclusive_scan_1024(cnt, s_scan);
+        const int start = s_carry[0] + inc_t - cnt;
+        int pstart = -1;
+        if (plan.tile_part) {
+            const int pc = cnt > 1 ? cnt : 0, sg = cnt > 1 ? 1 : 0;
+            const int inc_p = block_inclusive_scan_1024(pc, s_scan);
+            const int inc_s = block_inclusive_scan_1024(sg, s_scan);
+            if (sg) {
+                pstart = s_carry[1] + inc_p - pc;
+                const int si = s_carry[2] + inc_s - 1;
+                plan.split_seg[si] = g;
+                plan.split_first[si] = pstart;
+                plan.split_cnt[si] = cnt;
+            }
             __syncthreads();
-            s_scan[threadIdx.x] += v;
-            __syncthreads();
+            if (threadIdx.x == 1023) s_carry[1] += inc_p, s_carry[2] += inc_s;
         }
-        const int start = s_carry + s_scan[threadIdx.x] - cnt;
         for (int q = 0; q < cnt; ++q) {
             plan.tile_seg[start + q] = g;
-            plan.tile_p0[start + q] = s0 + q * kTM;
+            plan.tile_p0[start + q] = s0 + q * tile;
+            if (plan.tile_part) plan.tile_part[start + q] = pstart >= 0 ? pstart + q : -1;
         }
         __syncthreads();
-        if (threadIdx.x == 1023) s_carry += s_scan[1023];
+        if (threadIdx.x == 1023) s_carry[0] += inc_t;
         __syncthreads();
     }
-    if (threadIdx.x == 0) plan.num_tiles[0] = s_carry;
+    if (threadIdx.x == 0) {
+        plan.num_tiles[0] = s_carry[0];
+        if (plan.num_split) plan.num_split[0] = s_carry[2];
+    }
 }
 
 // ---- grouped GEMM tile: Y[32 x d] = X[32 x d] * M (or * M^T) -----------------------------
@@ -85,7 +121,7 @@ struct GemmArgs {
 // MODE 1: forward RESCAL   x = E[h],      y = x M,        score = y . E[t]
 // MODE 2: backward dX      x = xs rows,   y = x M^T -> occ_h = y, occ_t = -y (when occ_t is set)
 template <int MODE>
-__global__ __launch_bounds__(256) void transr_gemm_kernel(GemmArgs a)
+__global__ __launch_bounds__(256, 3) void transr_gemm_kernel(GemmArgs a)
 {
     extern __shared__ __align__(16) float lds[];
     const int tile = blockIdx.x;
@@ -142,7 +178,6 @@ __global__ __launch_bounds__(256) void transr_gemm_kernel(GemmArgs a)
             if constexpr (MODE != 2) {
                 // B[k][j] = M[k][n0 + 4 li + e]: one float4 per (k) row per lane
                 const bool colok = 4 * li < wcols;
-                float4 bn[4];
                 auto loadb = [&](int q, float4 *dst) {
 #pragma unroll
                     for (int s = 0; s < 4; ++s) {
@@ -151,30 +186,37 @@ __global__ __launch_bounds__(256) void transr_gemm_kernel(GemmArgs a)
                                                   : make_float4(0.f, 0.f, 0.f, 0.f);
                     }
                 };
-                loadb(0, bn);
-                for (int q = 0; q < nq; ++q) {
-                    float4 bc[4];
+                float4 ring[kRing][4];  // supersteps of B in flight
 #pragma unroll
-                    for (int s = 0; s < 4; ++s) bc[s] = bn[s];
-                    if (q + 1 < nq) loadb(q + 1, bn);
-                    const float4 alo = *reinterpret_cast<const float4 *>(&sX[li * pitch + 16 * q + 4 * kk]);
-                    const float4 ahi = *reinterpret_cast<const float4 *>(&sX[(16 + li) * pitch + 16 * q + 4 * kk]);
-                    const float al[4] = {alo.x, alo.y, alo.z, alo.w}, ah[4] = {ahi.x, ahi.y, ahi.z, ahi.w};
+                for (int u = 0; u < kRing; ++u)
+                    if (u < nq) loadb(u, ring[u]);
+                for (int q = 0; q < nq; q += kRing) {
 #pragma unroll
-                    for (int s = 0; s < 4; ++s) {
-                        const float bv[4] = {bc[s].x, bc[s].y, bc[s].z, bc[s].w};
+                    for (int u = 0; u < kRing; ++u) {
+                        if (q + u >= nq) break;
+                        float4 bc[4];
 #pragma unroll
-                        for (int e = 0; e < 4; ++e) {
-                            acc_lo[e] = __builtin_amdgcn_mfma_f32_16x16x4f32(al[s], bv[e], acc_lo[e], 0, 0, 0);
-                            if (two_blocks)
-                                acc_hi[e] = __builtin_amdgcn_mfma_f32_16x16x4f32(ah[s], bv[e], acc_hi[e], 0, 0, 0);
+                        for (int s = 0; s < 4; ++s) bc[s] = ring[u][s];
+                        if (q + u + kRing < nq) loadb(q + u + kRing, ring[u]);
+                        const int qq = q + u;
+                        const float4 alo = *reinterpret_cast<const float4 *>(&sX[li * pitch + 16 * qq + 4 * kk]);
+                        const float4 ahi = *reinterpret_cast<const float4 *>(&sX[(16 + li) * pitch + 16 * qq + 4 * kk]);
+                        const float al[4] = {alo.x, alo.y, alo.z, alo.w}, ah[4] = {ahi.x, ahi.y, ahi.z, ahi.w};
+#pragma unroll
+                        for (int s = 0; s < 4; ++s) {
+                            const float bv[4] = {bc[s].x, bc[s].y, bc[s].z, bc[s].w};
+#pragma unroll
+                            for (int e = 0; e < 4; ++e) {
+                                acc_lo[e] = __builtin_amdgcn_mfma_f32_16x16x4f32(al[s], bv[e], acc_lo[e], 0, 0, 0);
+                                if (two_blocks)
+                                    acc_hi[e] = __builtin_amdgcn_mfma_f32_16x16x4f32(ah[s], bv[e], acc_hi[e], 0, 0, 0);
+                            }
                         }
                     }
                 }
             } else {
                 // B[k][j] = M[j][k] (transposed): MFMA e owns output columns n0 + 16 e + li, and a
                 // lane's float4 along k of row (n0 + 16 e + li) serves the four steps
-                float4 bn[4];
                 auto loadb = [&](int q, float4 *dst) {
 #pragma unroll
                     for (int e = 0; e < 4; ++e) {
@@ -184,23 +226,31 @@ __global__ __launch_bounds__(256) void transr_gemm_kernel(GemmArgs a)
                                      : make_float4(0.f, 0.f, 0.f, 0.f);
                     }
                 };
-                loadb(0, bn);
-                for (int q = 0; q < nq; ++q) {
-                    float4 bc[4];
+                float4 ring[kRing][4];
 #pragma unroll
-                    for (int e = 0; e < 4; ++e) bc[e] = bn[e];
-                    if (q + 1 < nq) loadb(q + 1, bn);
-                    const float4 alo = *reinterpret_cast<const float4 *>(&sX[li * pitch + 16 * q + 4 * kk]);
-                    const float4 ahi = *reinterpret_cast<const float4 *>(&sX[(16 + li) * pitch + 16 * q + 4 * kk]);
-                    const float al[4] = {alo.x, alo.y, alo.z, alo.w}, ah[4] = {ahi.x, ahi.y, ahi.z, ahi.w};
+                for (int u = 0; u < kRing; ++u)
+                    if (u < nq) loadb(u, ring[u]);
+                for (int q = 0; q < nq; q += kRing) {
 #pragma unroll
-                    for (int e = 0; e < 4; ++e) {
-                        const float bv[4] = {bc[e].x, bc[e].y, bc[e].z, bc[e].w};
+                    for (int u = 0; u < kRing; ++u) {
+                        if (q + u >= nq) break;
+                        float4 bc[4];
 #pragma unroll
-                        for (int s = 0; s < 4; ++s) {
-                            acc_lo[e] = __builtin_amdgcn_mfma_f32_16x16x4f32(al[s], bv[s], acc_lo[e], 0, 0, 0);
-                            if (two_blocks)
-                                acc_hi[e] = __builtin_amdgcn_mfma_f32_16x16x4f32(ah[s], bv[s], acc_hi[e], 0, 0, 0);
+                        for (int e = 0; e < 4; ++e) bc[e] = ring[u][e];
+                        if (q + u + kRing < nq) loadb(q + u + kRing, ring[u]);
+                        const int qq = q + u;
+                        const float4 alo = *reinterpret_cast<const float4 *>(&sX[li * pitch + 16 * qq + 4 * kk]);
+                        const float4 ahi = *reinterpret_cast<const float4 *>(&sX[(16 + li) * pitch + 16 * qq + 4 * kk]);
+                        const float al[4] = {alo.x, alo.y, alo.z, alo.w}, ah[4] = {ahi.x, ahi.y, ahi.z, ahi.w};
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) {
+                            const float bv[4] = {bc[e].x, bc[e].y, bc[e].z, bc[e].w};
+#pragma unroll
+                            for (int s = 0; s < 4; ++s) {
+                                acc_lo[e] = __builtin_amdgcn_mfma_f32_16x16x4f32(al[s], bv[s], acc_lo[e], 0, 0, 0);
+                                if (two_blocks)
+                                    acc_hi[e] = __builtin_amdgcn_mfma_f32_16x16x4f32(ah[s], bv[s], acc_hi[e], 0, 0, 0);
+                            }
                         }
                     }
                 }
@@ -338,27 +388,39 @@ __global__ __launch_bounds__(256) void transr_prep_kernel(PrepArgs a)
     }
 }
 
+constexpr int kDmChunk = 256;  // triples of one relation group per dM work item
+
 struct DmArgs {
     const float *xs, *qs;  // sorted order [B, d]
-    const int32_t *num_unique, *seg_offsets;
-    float *dm;  // [U, d, d]
+    const int32_t *seg_offsets;
+    TilePlan plan;   // tiles of kDmChunk positions, with split bookkeeping
+    float *dm;       // [U, d, d]
+    float *part;     // [max_slots, d, d] partial results of split groups
     int d;
 };
 
-// dM[g][i][j] = sum_{p in group g} xs[p][i] * qs[p][j]; one workgroup per (group, 32 rows i),
-// the four waves split the columns j, K runs over the group's triples.
-__global__ __launch_bounds__(256) void transr_dm_kernel(DmArgs a)
+// dM[g][i][j] = sum_{p in group g} xs[p][i] * qs[p][j].  A work item is (chunk of <= 256 triples
+// of one group, 32 rows i); the four waves split the columns j; K runs over the chunk's triples,
+// operands prefetched four supersteps ahead.  Groups longer than one chunk write per-chunk
+// partial matrices that transr_dm_finish_kernel adds up (keeps the longest K loop at 16 supersteps).
+__global__ __launch_bounds__(256, 3) void transr_dm_kernel(DmArgs a)
 {
     const int d = a.d;
     const int nib = (d + 31) / 32;
-    const int g = blockIdx.x / nib;
-    if (g >= a.num_unique[0]) return;
+    const int tile = blockIdx.x / nib;
+    if (tile >= a.plan.num_tiles[0]) return;
     const int i0 = (blockIdx.x % nib) * 32;
+    const int g = a.plan.tile_seg[tile];
+    const int s0 = a.plan.tile_p0[tile];
+    const int seg_end = a.seg_offsets[g + 1];
+    const int s1 = s0 + kDmChunk < seg_end ? s0 + kDmChunk : seg_end;
+    const int slot = a.plan.tile_part[tile];
+    float *dst = slot >= 0 ? a.part + (int64_t)slot * d * d : a.dm + (int64_t)g * d * d;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int li = lane & 15, kk = lane >> 4;
-    const int s0 = a.seg_offsets[g], s1 = a.seg_offsets[g + 1];
     const bool two_blocks = i0 + 16 < d;
     const bool ilo = i0 + li < d, ihi = i0 + 16 + li < d;
+    const int nq = (s1 - s0 + 15) / 16;
 
     for (int c0 = 0; c0 < d; c0 += 256) {
         const int span = d - c0 < 256 ? d - c0 : 256;
@@ -370,26 +432,42 @@ __global__ __launch_bounds__(256) void transr_dm_kernel(DmArgs a)
         floatx4 acc_lo[4], acc_hi[4];
 #pragma unroll
         for (int e = 0; e < 4; ++e) acc_lo[e] = floatx4{0.f, 0.f, 0.f, 0.f}, acc_hi[e] = floatx4{0.f, 0.f, 0.f, 0.f};
-        for (int pq = s0; pq < s1; pq += 16) {
+
+        struct Stage {
             float al[4], ah[4];
             float4 bv[4];
+        };
+        auto load_stage = [&](int q, Stage &st) {
 #pragma unroll
             for (int s = 0; s < 4; ++s) {
-                const int p = pq + 4 * kk + s;
+                const int p = s0 + 16 * q + 4 * kk + s;
                 const bool ok = p < s1;
                 const float *xr = a.xs + (int64_t)p * d + i0;
-                al[s] = (ok && ilo) ? xr[li] : 0.0f;
-                ah[s] = (ok && ihi) ? xr[16 + li] : 0.0f;
-                bv[s] = (ok && colok) ? *reinterpret_cast<const float4 *>(a.qs + (int64_t)p * d + n0 + 4 * li)
-                                      : make_float4(0.f, 0.f, 0.f, 0.f);
+                st.al[s] = (ok && ilo) ? xr[li] : 0.0f;
+                st.ah[s] = (ok && ihi) ? xr[16 + li] : 0.0f;
+                st.bv[s] = (ok && colok) ? *reinterpret_cast<const float4 *>(a.qs + (int64_t)p * d + n0 + 4 * li)
+                                         : make_float4(0.f, 0.f, 0.f, 0.f);
             }
+        };
+        Stage ring[kRing];
 #pragma unroll
-            for (int s = 0; s < 4; ++s) {
-                const float b4[4] = {bv[s].x, bv[s].y, bv[s].z, bv[s].w};
+        for (int u = 0; u < kRing; ++u)
+            if (u < nq) load_stage(u, ring[u]);
+        for (int q = 0; q < nq; q += kRing) {
 #pragma unroll
-                for (int e = 0; e < 4; ++e) {
-                    acc_lo[e] = __builtin_amdgcn_mfma_f32_16x16x4f32(al[s], b4[e], acc_lo[e], 0, 0, 0);
-                    if (two_blocks) acc_hi[e] = __builtin_amdgcn_mfma_f32_16x16x4f32(ah[s], b4[e], acc_hi[e], 0, 0, 0);
+            for (int u = 0; u < kRing; ++u) {
+                if (q + u >= nq) break;
+                const Stage cur = ring[u];
+                if (q + u + kRing < nq) load_stage(q + u + kRing, ring[u]);
+#pragma unroll
+                for (int s = 0; s < 4; ++s) {
+                    const float b4[4] = {cur.bv[s].x, cur.bv[s].y, cur.bv[s].z, cur.bv[s].w};
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        acc_lo[e] = __builtin_amdgcn_mfma_f32_16x16x4f32(cur.al[s], b4[e], acc_lo[e], 0, 0, 0);
+                        if (two_blocks)
+                            acc_hi[e] = __builtin_amdgcn_mfma_f32_16x16x4f32(cur.ah[s], b4[e], acc_hi[e], 0, 0, 0);
+                    }
                 }
             }
         }
@@ -403,45 +481,79 @@ __global__ __launch_bounds__(256) void transr_dm_kernel(DmArgs a)
                     float4 v;
                     if (blk == 0) v = make_float4(acc_lo[0][r], acc_lo[1][r], acc_lo[2][r], acc_lo[3][r]);
                     else v = make_float4(acc_hi[0][r], acc_hi[1][r], acc_hi[2][r], acc_hi[3][r]);
-                    *reinterpret_cast<float4 *>(a.dm + ((int64_t)g * d + row) * d + n0 + 4 * li) = v;
+                    *reinterpret_cast<float4 *>(dst + (int64_t)row * d + n0 + 4 * li) = v;
                 }
         }
     }
+}
+
+// dM of a split group = sum of its partial matrices (slot order = ascending chunk order)
+__global__ __launch_bounds__(256) void transr_dm_finish_kernel(DmArgs a)
+{
+    const int sidx = blockIdx.y;
+    if (sidx >= a.plan.num_split[0]) return;
+    const int64_t dd4 = (int64_t)a.d * a.d / 4;
+    const int64_t f = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (f >= dd4) return;
+    const int g = a.plan.split_seg[sidx], first = a.plan.split_first[sidx], cnt = a.plan.split_cnt[sidx];
+    const float4 *src = reinterpret_cast<const float4 *>(a.part) + (int64_t)first * dd4 + f;
+    float4 acc = src[0];
+    for (int c = 1; c < cnt; ++c) {
+        const float4 v = src[(int64_t)c * dd4];
+        acc.x += v.x, acc.y += v.y, acc.z += v.z, acc.w += v.w;
+    }
+    reinterpret_cast<float4 *>(a.dm)[(int64_t)g * dd4 + f] = acc;
 }
 
 // ---- host side -----------------------------------------------------------------------------
 static size_t up256(size_t x) { return (x + 255) & ~size_t(255); }
 
 struct RPlan {
-    size_t off_plan, off_xs, off_qs, off_occ, off_part_e, off_part_r, total;
-    int64_t tiles;
+    size_t off_plan, off_dplan, off_xs, off_qs, off_occ, off_part_e, off_part_r, off_dpart, total;
+    int64_t tiles, dtiles, dsplit, dslots;
 };
+
+static size_t plan_ints(int64_t tiles, int64_t split) { return (size_t)(64 + 3 * tiles + 3 * split + 8); }
 
 static RPlan make_rplan(const kge_tables *tab, const kge_batch *bat)
 {
     RPlan p{};
     const int64_t B = bat->batch, d = tab->dim;
+    const int64_t groups = B < tab->n_rel ? B : tab->n_rel;
     p.tiles = max_tiles(tab, bat);
+    p.dtiles = groups + B / kDmChunk + 1;
+    p.dsplit = B / kDmChunk + 1;            // a split group has more than kDmChunk triples
+    p.dslots = 2 * (B / kDmChunk) + 2;      // sum over split groups of ceil(n_g / chunk)
     size_t o = 0;
-    p.off_plan = o, o += up256(sizeof(int32_t) * (size_t)(2 * p.tiles + 64));
+    p.off_plan = o, o += up256(sizeof(int32_t) * plan_ints(p.tiles, 0));
+    p.off_dplan = o, o += up256(sizeof(int32_t) * plan_ints(p.dtiles, p.dsplit));
     p.off_xs = o, o += up256(sizeof(float) * (size_t)(B * d));
     p.off_qs = o, o += up256(sizeof(float) * (size_t)(B * d));
     p.off_occ = o, o += up256(sizeof(float) * (size_t)(2 * B * d));
-    p.off_part_e = o, o += up256(sizeof(float) * (size_t)(ceil_div(2 * B, 32) * 2 * d));
-    p.off_part_r = o, o += up256(sizeof(float) * (size_t)(ceil_div(B, 32) * 2 * d));
+    p.off_part_e = o, o += up256(sizeof(float) * (size_t)seg_partial_floats(2 * B, d));
+    p.off_part_r = o, o += up256(sizeof(float) * (size_t)seg_partial_floats(B, d));
+    p.off_dpart = o, o += up256(sizeof(float) * (size_t)(p.dslots * d * d));
     p.total = o;
     return p;
 }
 
-static TilePlan plan_at(void *base, int64_t tiles)
+static TilePlan plan_at(void *base, int64_t tiles, int64_t split)
 {
     int32_t *q = static_cast<int32_t *>(base);
-    return TilePlan{q, q + 64, q + 64 + tiles};
+    TilePlan p{q, q + 64, q + 64 + tiles, nullptr, nullptr, nullptr, nullptr, nullptr};
+    if (split > 0) {
+        p.tile_part = q + 64 + 2 * tiles;
+        p.num_split = q + 32;
+        p.split_seg = q + 64 + 3 * tiles;
+        p.split_first = p.split_seg + split;
+        p.split_cnt = p.split_first + split;
+    }
+    return p;
 }
 
 size_t transr_fwd_workspace(const kge_tables *tab, const kge_batch *bat)
 {
-    return up256(sizeof(int32_t) * (size_t)(2 * max_tiles(tab, bat) + 64));
+    return up256(sizeof(int32_t) * plan_ints(max_tiles(tab, bat), 0));
 }
 
 int launch_transr_fwd(const kge_tables *tab, const kge_batch *bat, float *pos, float *resid, void *workspace,
@@ -454,8 +566,8 @@ int launch_transr_fwd(const kge_tables *tab, const kge_batch *bat, float *pos, f
         return launch_score_pos(tab, bat, pos, resid, nullptr, st);
     const kge_inspection *ri = bat->rel_insp;
     const int64_t tiles = max_tiles(tab, bat);
-    TilePlan plan = plan_at(workspace, tiles);
-    hipLaunchKernelGGL(transr_plan_kernel, dim3(1), dim3(1024), 0, st, ri->num_unique, ri->seg_offsets, plan);
+    TilePlan plan = plan_at(workspace, tiles, 0);
+    hipLaunchKernelGGL(transr_plan_kernel, dim3(1), dim3(1024), 0, st, ri->num_unique, ri->seg_offsets, plan, kTM);
     GemmArgs a{tab->ent, tab->rel, tab->aux, bat->h, bat->r, bat->t, ri->perm, ri->seg_offsets, ri->unique_ids,
                plan, nullptr, pos, resid, nullptr, nullptr, (int)tab->dim, tab->norm_p};
     const size_t lds = gemm_lds_bytes((int)tab->dim);
@@ -468,9 +580,6 @@ int launch_transr_fwd(const kge_tables *tab, const kge_batch *bat, float *pos, f
 }
 
 size_t transr_bwd_workspace(const kge_tables *tab, const kge_batch *bat) { return make_rplan(tab, bat).total; }
-
-int launch_seg_reduce(const float *occ, const kge_inspection *ins, int d, float *out, float *partial,
-                      bool identity_perm, hipStream_t st);
 
 int launch_transr_bwd(const kge_tables *tab, const kge_batch *bat, const kge_saved *saved, const float *dpos,
                       const kge_grads *grads, void *workspace, size_t workspace_bytes, hipStream_t st)
@@ -489,28 +598,33 @@ int launch_transr_bwd(const kge_tables *tab, const kge_batch *bat, const kge_sav
     float *xs = reinterpret_cast<float *>(ws + p.off_xs), *qs = reinterpret_cast<float *>(ws + p.off_qs);
     float *occ = reinterpret_cast<float *>(ws + p.off_occ);
     const kge_inspection *ri = bat->rel_insp;
-    TilePlan plan = plan_at(ws + p.off_plan, p.tiles);
+    TilePlan plan = plan_at(ws + p.off_plan, p.tiles, 0);
+    TilePlan dplan = plan_at(ws + p.off_dplan, p.dtiles, p.dsplit);
 
     PrepArgs pa{tab->ent, bat->h, bat->t, ri->perm, dpos, saved->pos, saved->residual, xs, qs, occ + B * d, B, d,
                 tab->norm_p, rescal ? 1 : 0};
     hipLaunchKernelGGL(transr_prep_kernel, dim3((unsigned)ceil_div(B, 4)), dim3(256), 0, st, pa);
-    hipLaunchKernelGGL(transr_plan_kernel, dim3(1), dim3(1024), 0, st, ri->num_unique, ri->seg_offsets, plan);
+    hipLaunchKernelGGL(transr_plan_kernel, dim3(1), dim3(1024), 0, st, ri->num_unique, ri->seg_offsets, plan, kTM);
+    hipLaunchKernelGGL(transr_plan_kernel, dim3(1), dim3(1024), 0, st, ri->num_unique, ri->seg_offsets, dplan,
+                       kDmChunk);
     // dX = Q M^T -> occurrence rows of h (and -dX for t)
     GemmArgs ga{tab->ent, tab->rel, tab->aux, bat->h, bat->r, bat->t, ri->perm, ri->seg_offsets, ri->unique_ids,
                 plan, qs, nullptr, nullptr, occ, rescal ? nullptr : occ + B * d, d, tab->norm_p};
     hipLaunchKernelGGL(transr_gemm_kernel<2>, dim3((unsigned)p.tiles), dim3(256), gemm_lds_bytes(d), st, ga);
     // dM = X^T Q per relation group
-    const int64_t groups = B < tab->n_rel ? B : tab->n_rel;
-    DmArgs da{xs, qs, ri->num_unique, ri->seg_offsets, grads->aux_rows, d};
-    hipLaunchKernelGGL(transr_dm_kernel, dim3((unsigned)(ceil_div(d, 32) * groups)), dim3(256), 0, st, da);
+    DmArgs da{xs, qs, ri->seg_offsets, dplan, grads->aux_rows, reinterpret_cast<float *>(ws + p.off_dpart), d};
+    hipLaunchKernelGGL(transr_dm_kernel, dim3((unsigned)(ceil_div(d, 32) * p.dtiles)), dim3(256), 0, st, da);
+    hipLaunchKernelGGL(transr_dm_finish_kernel, dim3((unsigned)ceil_div((int64_t)d * d / 4, 256), (unsigned)p.dsplit),
+                       dim3(256), 0, st, da);
     KGE_CHECK_LAUNCH();
     if (bat->insp_ready && hipStreamWaitEvent(st, reinterpret_cast<hipEvent_t>(bat->insp_ready), 0) != hipSuccess)
         return KGE_ELAUNCH;
-    int rc = launch_seg_reduce(occ, bat->ent_insp, d, grads->ent_rows, reinterpret_cast<float *>(ws + p.off_part_e),
-                               false, st);
-    if (rc || rescal) return rc;
-    // dR[g] = sum of the group's q rows (already in sorted order)
-    return launch_seg_reduce(qs, ri, d, grads->rel_rows, reinterpret_cast<float *>(ws + p.off_part_r), true, st);
+    // entity rows from the h / t occurrence rows; dR[g] = sum of the group's q rows, which are
+    // already stored in sorted order
+    const SegJob jobs[2] = {
+        {occ, bat->ent_insp, d, grads->ent_rows, reinterpret_cast<float *>(ws + p.off_part_e), false},
+        {qs, ri, d, grads->rel_rows, reinterpret_cast<float *>(ws + p.off_part_r), true}};
+    return launch_seg_reduce_jobs(jobs, rescal ? 1 : 2, st);
 }
 
 }  // namespace kge

@@ -38,8 +38,10 @@ def build(force: bool = False) -> None:
 _libs: dict[str, ctypes.CDLL] = {}
 
 
-def _lib(fast: bool = False) -> ctypes.CDLL:
-    name = "libkge_oracle_omp.so" if fast else "libkge_oracle.so"
+def _lib(fast=False) -> ctypes.CDLL:
+    """fast: False = the checker (-O2); "o3" = -O3 one thread; True / "omp" = -O3 + OpenMP forward."""
+    name = {False: "libkge_oracle.so", "o3": "libkge_oracle_o3.so", True: "libkge_oracle_omp.so",
+            "omp": "libkge_oracle_omp.so"}[fast]
     if name not in _libs:
         path = os.path.join(_HERE, name)
         if not os.path.exists(path):
@@ -135,7 +137,7 @@ class SparseGrads:
     aux_rows: np.ndarray | None
 
 
-def backward(model, E, R, A, h, r, t, neg=None, chunk=0, dpos=None, dneg=None, p=2) -> SparseGrads:
+def backward(model, E, R, A, h, r, t, neg=None, chunk=0, dpos=None, dneg=None, p=2, fast=False) -> SparseGrads:
     """Sparse row gradients (unique ids ascending, one row per id) per table."""
     E, R, A = _f32(E), _f32(R), _f32(A)
     h, r, t, neg = _i64(h), _i64(r), _i64(t), _i64(neg)
@@ -157,7 +159,7 @@ def backward(model, E, R, A, h, r, t, neg=None, chunk=0, dpos=None, dneg=None, p
     gE = np.zeros((ins_e.unique_ids.shape[0], d), np.float32)
     gR = np.zeros((ins_r.unique_ids.shape[0], rw), np.float32) if rw else None
     gA = np.zeros((ins_r.unique_ids.shape[0], aw), np.float32) if aw else None
-    rc = _lib().orc_backward(
+    rc = _lib(fast).orc_backward(
         ctypes.c_int(MODELS[model]), ctypes.c_int(p), ctypes.c_int64(B), ctypes.c_int64(d),
         _fp(E), _fp(R), _fp(A), _fp(h), _fp(r), _fp(t), _fp(neg),
         ctypes.c_int64(C), ctypes.c_int64(N), _fp(dpos), _fp(dneg),
@@ -195,5 +197,5 @@ def build_index(r, rel_num):
     return uniq, buf, cnt, bool(rc)
 
 
-def threads(fast: bool = True) -> int:
+def threads(fast=True) -> int:
     return int(_lib(fast).orc_threads())
