@@ -230,7 +230,9 @@ def main():
                             ctypes.c_void_p(step.neg.data_ptr()),
                             ctypes.c_void_p(step.side_pos.data_ptr()) if step.side_pos is not None else None,
                             ctypes.c_void_p(step.side_neg.data_ptr()) if step.side_neg is not None else None,
-                            None, None, 0, stc)
+                            # RotatE: the rotated heads the positive kernel left behind (read-only here)
+                            ctypes.c_void_p(step.residual.data_ptr()) if w.model == "RotatE" else None,
+                            None, 0, stc)
         kname = "score_neg_kernel"
         if w.model == "TransH":  # needs w.h from the positive kernel; time the pair and subtract
             t_pair = time_events(lambda: step.forward(stc), 100, torch)

@@ -21,7 +21,7 @@ FLAGS = [
     # packed fp32 VALU forms are kept out of the generated code
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
     "-Wall", "-Wno-unused-function", "-Wno-unknown-attributes",
-]
+] + os.environ.get("KGE_EXTRA_HIPCC_FLAGS", "").split()
 
 
 def sources() -> list[str]:

@@ -3,7 +3,7 @@
 
 namespace kge {
 int launch_score_pos(const kge_tables *, const kge_batch *, float *, float *, float *, hipStream_t);
-int launch_score_neg(const kge_tables *, const kge_batch *, const float *, float *, float *,
+int launch_score_neg(const kge_tables *, const kge_batch *, const float *, const float *, float *, float *,
                      hipStream_t);
 int launch_transr_fwd(const kge_tables *, const kge_batch *, float *, float *, void *, size_t, hipStream_t);
 size_t transr_fwd_workspace(const kge_tables *, const kge_batch *);
@@ -102,7 +102,8 @@ int kge_score_fwd(const kge_tables *tab, const kge_batch *bat, float *pos, float
             rc = launch_score_pos(tab, bat, pos, residual, side_pos, st);
         if (rc) return rc;
     }
-    if (want_neg) return launch_score_neg(tab, bat, side_pos, neg, side_neg, st);
+    if (want_neg)
+        return launch_score_neg(tab, bat, side_pos, tab->model == KGE_ROTATE ? residual : nullptr, neg, side_neg, st);
     return KGE_OK;
 }
 

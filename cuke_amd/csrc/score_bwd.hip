@@ -30,6 +30,7 @@ struct TileArgs {
     const float *sneg;      // [B, N] forward scores (L2 normalisation)
     const float *side_pos;  // TransH: w.h per positive
     const float *side_neg;  // TransH: [2, B, N]
+    const float *query;     // RotatE: rotated heads [B, d] saved by the forward pass, or null
     float *out0, *out1;
     int64_t plane;  // B * N
     int C, N, d, rel_dim, vec, vecn, n_chunks;
@@ -40,7 +41,7 @@ constexpr int kKL = 32;       // looper rows staged per step
 constexpr int kLP = kTI + 4;  // LDS pitch of a staged row
 
 template <int MODEL, int P, bool OWNER_POS, int RO>
-__global__ __launch_bounds__(256) void bwd_tile_kernel(TileArgs a)
+__global__ __launch_bounds__(256, KGE_TILE_OCC) void bwd_tile_kernel(TileArgs a)
 {
     constexpr int TO = 16 * RO;
     constexpr bool kRot = MODEL == KGE_ROTATE, kTH = MODEL == KGE_TRANSH;
@@ -84,7 +85,7 @@ __global__ __launch_bounds__(256) void bwd_tile_kernel(TileArgs a)
             if constexpr (!kDot)
                 load_query<MODEL>(a.ent + a.h[b] * (int64_t)d, a.rel + rid * (int64_t)a.rel_dim,
                                   kTH ? a.aux + rid * (int64_t)d : nullptr, alo[o], col, lim, half, vec, q0,
-                                  q1);
+                                  q1, (kRot && a.query) ? a.query + b * (int64_t)d : nullptr);
             own[0][o] = q0;
             if constexpr (NPO == 2) own[1][o] = q1;
         } else {
@@ -121,7 +122,7 @@ __global__ __launch_bounds__(256) void bwd_tile_kernel(TileArgs a)
                 float4 q0, q1;
                 load_query<MODEL>(a.ent + a.h[b] * (int64_t)d, a.rel + rid * (int64_t)a.rel_dim,
                                   kTH ? a.aux + rid * (int64_t)d : nullptr, kTH ? a.side_pos[b] : 0.0f, col,
-                                  lim, half, vec, q0, q1);
+                                  lim, half, vec, q0, q1, (kRot && a.query) ? a.query + b * (int64_t)d : nullptr);
                 rl[0][s] = q0;
                 if constexpr (NPL == 2) rl[1][s] = q1;
             }
@@ -598,7 +599,7 @@ int kge_score_bwd(const kge_tables *tab, const kge_batch *bat, const kge_saved *
         const bool vecn = bat->n_neg % 4 == 0 && aligned16(dneg) && (!saved->neg || aligned16(saved->neg)) &&
                           (!saved->side_neg || aligned16(saved->side_neg));
         TileArgs a{tab->ent, tab->rel, tab->aux, bat->h, bat->r, bat->neg, dneg, saved->neg, saved->side_pos,
-                   saved->side_neg, nullptr, nullptr, B * bat->n_neg, (int)bat->chunk, (int)bat->n_neg, (int)d,
+                   saved->side_neg, model == KGE_ROTATE ? saved->residual : nullptr, nullptr, nullptr, B * bat->n_neg, (int)bat->chunk, (int)bat->n_neg, (int)d,
                    (int)tab->rel_dim, vec ? 1 : 0, vecn ? 1 : 0, (int)n_chunks};
         float *occ_neg = occ_e + 2 * B * d;
         switch (model) {

@@ -18,6 +18,7 @@ struct NegArgs {
     const float *ent, *rel, *aux;
     const int64_t *h, *r, *neg;
     const float *side_pos;  // TransH: w_b . h_b
+    const float *query;     // RotatE: rotated heads [B, d] from the positive kernel, or null
     float *out;             // [B, N]
     float *side_neg;        // TransH save-for-backward [2, B, N] (optional):
                             //   plane 0: c = w_b . t'_k ; plane 1: sum_i phi(u_i) w_i with
@@ -56,7 +57,7 @@ __device__ __forceinline__ void pair_elem(float &acc, float &acc2, float a0, flo
 }
 
 template <int MODEL, int P, int RB, int RK, bool SAVE>
-__global__ __launch_bounds__(256) void score_neg_kernel(NegArgs a)
+__global__ __launch_bounds__(256, KGE_TILE_OCC) void score_neg_kernel(NegArgs a)
 {
     constexpr int TB = 16 * RB, TN = 16 * RK;
     constexpr int NPA = (MODEL == KGE_ROTATE || MODEL == KGE_TRANSH) ? 2 : 1;
@@ -78,7 +79,7 @@ __global__ __launch_bounds__(256) void score_neg_kernel(NegArgs a)
     const bool vec = a.vec != 0;
 
     // rows this thread stages
-    const float *ph[SB], *pr[SB], *pw[SB];
+    const float *ph[SB], *pr[SB], *pw[SB], *pq[SB];
     float pa[SB];
     bool okb[SB];
 #pragma unroll
@@ -91,6 +92,7 @@ __global__ __launch_bounds__(256) void score_neg_kernel(NegArgs a)
         pr[s] = a.rel + rid * (int64_t)a.rel_dim;
         pw[s] = MODEL == KGE_TRANSH ? a.aux + rid * (int64_t)d : nullptr;
         pa[s] = MODEL == KGE_TRANSH ? a.side_pos[b] : 0.0f;
+        pq[s] = (MODEL == KGE_ROTATE && a.query) ? a.query + b * (int64_t)d : nullptr;
     }
     const float *pt[SN];
     bool okk[SN];
@@ -110,7 +112,7 @@ __global__ __launch_bounds__(256) void score_neg_kernel(NegArgs a)
         for (int s = 0; s < SB; ++s) {
             const int lim = okb[s] ? klen : 0;
             float4 q0, q1;
-            load_query<MODEL>(ph[s], pr[s], pw[s], pa[s], j, lim, half, vec, q0, q1);
+            load_query<MODEL>(ph[s], pr[s], pw[s], pa[s], j, lim, half, vec, q0, q1, pq[s]);
             ra[0][s] = q0;
             if constexpr (NPA == 2) ra[1][s] = q1;
         }
@@ -238,14 +240,14 @@ static int launch_neg_mp(const NegArgs &a, int64_t n_chunks, hipStream_t st)
     return KGE_OK;
 }
 
-int launch_score_neg(const kge_tables *tab, const kge_batch *bat, const float *side_pos, float *out,
-                     float *side_neg, hipStream_t st)
+int launch_score_neg(const kge_tables *tab, const kge_batch *bat, const float *side_pos, const float *query,
+                     float *out, float *side_neg, hipStream_t st)
 {
     if (bat->batch == 0) return KGE_OK;
     const int64_t n_chunks = bat->batch / bat->chunk;
     if (n_chunks >= (1 << 24) || bat->chunk >= (1 << 30) || bat->n_neg >= (1 << 30)) return KGE_ESHAPE;
     const bool vec = rows_vectorizable(tab);
-    NegArgs a{tab->ent, tab->rel, tab->aux, bat->h, bat->r, bat->neg, side_pos, out, side_neg,
+    NegArgs a{tab->ent, tab->rel, tab->aux, bat->h, bat->r, bat->neg, side_pos, query, out, side_neg,
               bat->batch * bat->n_neg, (int)bat->chunk, (int)bat->n_neg, (int)tab->dim, (int)tab->rel_dim, tab->gamma, vec ? 1 : 0, (int)n_chunks};
     const int p = tab->norm_p;
     switch (tab->model) {

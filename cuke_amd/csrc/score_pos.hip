@@ -14,7 +14,8 @@ struct PosArgs {
     int d, rel_dim;
     float gamma;
     float *pos;       // [B] scores or nullptr
-    float *resid;     // [B, d] residual rows or nullptr (TransE / TransH / TransR)
+    float *resid;     // [B, d] or nullptr: residual rows (TransE / TransH / TransR) or, for RotatE,
+                      // the rotated heads h e^{i theta} laid out [re | im]
     float *side_pos;  // [B] TransH: w.h (used by the shared-negative kernels)
 };
 
@@ -147,14 +148,17 @@ __global__ __launch_bounds__(kPosWaves *kWave) void score_pos_kernel(PosArgs a)
             const Vec<V> hr = Vec<V>::load(eh + j), hi = Vec<V>::load(eh + half + j);
             const Vec<V> tr = Vec<V>::load(et + j), ti = Vec<V>::load(et + half + j);
             const Vec<V> th = Vec<V>::load(rr + j);
+            Vec<V> ar, ai;
 #pragma unroll
             for (int e = 0; e < V; ++e) {
                 float sn, c;
                 sincosf(th.v[e], &sn, &c);
-                const float ur = (hr.v[e] * c - hi.v[e] * sn) - tr.v[e];
-                const float ui = (hr.v[e] * sn + hi.v[e] * c) - ti.v[e];
+                ar.v[e] = hr.v[e] * c - hi.v[e] * sn;
+                ai.v[e] = hr.v[e] * sn + hi.v[e] * c;
+                const float ur = ar.v[e] - tr.v[e], ui = ai.v[e] - ti.v[e];
                 acc += sqrtf(ur * ur + ui * ui);
             }
+            if (out && valid) ar.store(out + j), ai.store(out + half + j);  // rotated head, reused downstream
         }
     }
 

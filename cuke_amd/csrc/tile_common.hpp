@@ -5,6 +5,10 @@
 
 #include "common.hpp"
 
+#ifndef KGE_TILE_OCC
+#define KGE_TILE_OCC 3  // minimum workgroups per CU the tile kernels are compiled for
+#endif
+
 namespace kge {
 
 __device__ __forceinline__ float4 ld4(const float *p, int j, int lim, bool vec)
@@ -59,11 +63,21 @@ __device__ __forceinline__ int pair_len(int d)
 //   TransE    q0 = h+r                   RotatE   q0 = Re(h e^{i theta}), q1 = Im(...)
 //   TransH    q0 = h + r - al*w (al = w.h), q1 = w
 // lim == 0 yields zeros (row outside the tile).
+// pq != nullptr: the row was already formed by the positive kernel (RotatE: rotating h costs a
+// sincos per element, far more than re-reading the stored result) and is simply loaded.
 template <int MODEL>
 __device__ __forceinline__ void load_query(const float *ph, const float *pr, const float *pw, float al,
-                                           int j, int lim, int half, bool vec, float4 &q0, float4 &q1)
+                                           int j, int lim, int half, bool vec, float4 &q0, float4 &q1,
+                                           const float *pq = nullptr)
 {
     q1 = zero4();
+    if constexpr (MODEL == KGE_ROTATE) {
+        if (pq) {
+            q0 = ld4(pq, j, lim, vec);
+            q1 = ld4(pq + half, j, lim, vec);
+            return;
+        }
+    }
     if constexpr (MODEL == KGE_DISTMULT) {
         q0 = mul4(ld4(ph, j, lim, vec), ld4(pr, j, lim, vec));
     } else if constexpr (MODEL == KGE_TRANSE) {
@@ -119,23 +133,29 @@ __device__ __forceinline__ void load_query(const float *ph, const float *pr, con
 
 // XCD-aware tile placement.  The 256 CUs sit in 8 XCDs with one L2 each, and consecutive
 // workgroup ids of a 1-D grid go to consecutive XCDs.  All tiles of one chunk share that
-// chunk's positive and negative rows, so they are steered to one XCD (chunk c -> XCD c % 8):
-// every gathered row is then fetched from HBM by a single L2 instead of by up to eight.
-// Grid: 8 * ceil(n_chunks / 8) * tiles_per_chunk workgroups; returns false for padding ids.
+// chunk's positive and negative rows, so they are steered to one XCD: every gathered row is
+// then fetched from HBM by a single L2 instead of by up to eight.  With fewer than 8 chunks a
+// chunk's tiles are dealt round-robin to 8 / n_chunks XCDs so that no XCD stays idle.
+// Returns false for the padding ids of the grid (see xcd_grid).
 constexpr int kXcds = 8;
+__host__ __device__ inline int xcd_split(int n_chunks) { return n_chunks >= kXcds ? 1 : kXcds / n_chunks; }
 __device__ __forceinline__ bool xcd_tile(int tiles_x, int tiles_y, int n_chunks, int &c, int &ty, int &tx)
 {
     const int lid = blockIdx.x, per = tiles_x * tiles_y;
+    const int split = xcd_split(n_chunks);
+    const int per_v = (per + split - 1) / split;  // tiles of one virtual chunk
     const int xcd = lid % kXcds, k = lid / kXcds;
-    c = (k / per) * kXcds + xcd;
-    const int t = k % per;
+    const int vc = (k / per_v) * kXcds + xcd;      // virtual chunk = (chunk, residue of the tile id)
+    c = vc / split;
+    const int t = (k % per_v) * split + vc % split;
     ty = t / tiles_x;
     tx = t % tiles_x;
-    return c < n_chunks;
+    return c < n_chunks && t < per;
 }
 inline unsigned xcd_grid(int64_t tiles_x, int64_t tiles_y, int64_t n_chunks)
 {
-    return (unsigned)(kXcds * ceil_div(n_chunks, kXcds) * tiles_x * tiles_y);
+    const int64_t split = xcd_split((int)n_chunks), per = tiles_x * tiles_y;
+    return (unsigned)(kXcds * ceil_div(n_chunks * split, kXcds) * ceil_div(per, split));
 }
 
 inline bool rows_vectorizable(const kge_tables *tab)

@@ -224,7 +224,7 @@ class KGEModel:
             fw.side_pos = torch.empty(B, **f32)
             if neg is not None:
                 fw.side_neg = torch.empty((2, B, N), **f32)
-        if self.model in ("TransR", "RESCAL"):
+        if self.model in ("TransR", "RESCAL", "RotatE"):
             fw.residual = torch.empty((B, self.dim), **f32)
         ws, nb = self._fwd_workspace(bat)
         _lib.check(_lib.lib().kge_score_fwd(C.byref(self._tab), C.byref(bat), _ptr(fw.pos),
@@ -406,7 +406,8 @@ class TrainStep:
         self.neg = torch.empty((B, N), **f32) if neg is not None else None
         self.side_pos = torch.empty(B, **f32) if model.model == "TransH" else None
         self.side_neg = torch.empty((2, B, N), **f32) if (model.model == "TransH" and neg is not None) else None
-        self.residual = torch.empty((B, model.dim), **f32) if model.model in ("TransR", "RESCAL") else None
+        self.residual = torch.empty((B, model.dim), **f32) if model.model in ("TransR", "RESCAL", "RotatE") \
+            else None
         self._ws_f_bytes = int(L.kge_score_fwd_workspace(C.byref(model._tab), C.byref(self.bat)))
         self._ws_f = torch.empty(max(self._ws_f_bytes, 1), dtype=torch.uint8, device=dev)
         self.loss = torch.zeros(1, **f32)
