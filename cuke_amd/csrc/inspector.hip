@@ -28,12 +28,14 @@ struct Parts {
     int n_parts;
 };
 
+// Key i of the concatenation.  Branch-free address selection (unused parts have end == n, so
+// they are never chosen): a loop here would keep the compiler from batching the callers' loads.
 __device__ __forceinline__ uint32_t load_key(const Parts &parts, int64_t i)
 {
-    int q = 0;
-    while (q + 1 < parts.n_parts && i >= parts.end[q]) ++q;
-    const int64_t begin = q ? parts.end[q - 1] : 0;
-    return (uint32_t)parts.p[q][i - begin];
+    const int64_t e0 = parts.end[0], e1 = parts.end[1], e2 = parts.end[2];
+    const int64_t *p = i < e0 ? parts.p[0] : (i < e1 ? parts.p[1] : (i < e2 ? parts.p[2] : parts.p[3]));
+    const int64_t begin = i < e0 ? 0 : (i < e1 ? e0 : (i < e2 ? e1 : e2));
+    return (uint32_t)p[i - begin];
 }
 
 // ---- pass step 1: per-block digit histogram --------------------------------------------
@@ -283,144 +285,182 @@ __global__ __launch_bounds__(kSortThreads) void finalize_kernel(const uint32_t *
     }
 }
 
-// ---- small inputs: the whole inspection in one workgroup ------------------------------------
-// Up to 32768 ids: one 1024-thread workgroup runs every radix pass and the dedup with
-// workgroup barriers only (keys ping-pong through L2, digit counters in LDS), so an
-// inspection is one launch instead of 2 per pass + 2; several index sets are inspected by
-// the same launch, one workgroup each.
-constexpr int kSmallThreads = 1024;
-constexpr int kSmallWaves = kSmallThreads / kWave;  // 16
-constexpr int kSmallMaxBits = 10;
-constexpr int kSmallMaxBins = 1 << kSmallMaxBits;
-constexpr int64_t kSmallMaxN = 32768;
+// ---- small and medium inputs: one launch per digit pass ------------------------------------
+// Up to 65536 ids.  A block owns 1024 consecutive keys.  Instead of a separate histogram
+// kernel and scan, every block counts the digits of ALL keys itself (LDS atomics; the keys are
+// a few hundred KB at most and sit in L2), which gives it the global bin starts and the number
+// of same-digit keys in the blocks before it; it then ranks its own keys stably with wave
+// ballots and scatters them.  A pass is therefore ONE launch with no inter-block dependency,
+// the dedup a second one that counts the run heads before the block the same way.  Several
+// index sets share the launches (blockIdx.y).
+constexpr int kMidThreads = 256;
+constexpr int kMidWaves = kMidThreads / kWave;
+constexpr int kMidKeys = 1024;  // keys per block: 4 rounds of 64 per wave
+constexpr int kMidRounds = kMidKeys / kMidThreads;
+constexpr int64_t kMidMaxN = 65536;
 
-struct SmallJob {
+struct MidJob {
     Parts parts;
     int64_t n;
-    int bits;
+    int npass, db;
     kge_inspection out;
     uint32_t *keys_final, *keys_tmp;
     int32_t *vals_tmp;
 };
-struct SmallJobs {
-    SmallJob j[4];
+struct MidJobs {
+    MidJob j[4];
 };
 
-template <int KPT>
-__global__ __launch_bounds__(kSmallThreads) void inspect_small_kernel(SmallJobs jobs)
+template <bool FIRST>
+__global__ __launch_bounds__(kMidThreads) void inspect_mid_pass_kernel(MidJobs jobs, int pass)
 {
-    __shared__ unsigned short s_cnt[kSmallWaves][kSmallMaxBins];  // 32 KB
-    __shared__ uint32_t s_tot[kSmallMaxBins];
-    __shared__ uint32_t s_w[kSmallWaves];
-    const SmallJob &J = jobs.j[blockIdx.x];
-    const int tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid >> 6;
+    __shared__ uint32_t s_tot[kMaxBins];             // digit totals -> global bin starts
+    __shared__ uint32_t s_bef[kMaxBins];             // same digit, earlier blocks
+    __shared__ uint32_t s_cnt[kMidWaves][kMaxBins];  // per-wave running counts
+    __shared__ uint32_t s_w[kMidWaves];
+    const MidJob &J = jobs.j[blockIdx.y];
     const int n = (int)J.n;
-    const int npass = (J.bits + kSmallMaxBits - 1) / kSmallMaxBits;
-    const int db = (J.bits + npass - 1) / npass;
-    const int bins = 1 << db;
+    if (pass >= J.npass || (int)blockIdx.x * kMidKeys >= n) return;
+    const int tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid >> 6;
+    const int bins = 1 << J.db;
     const uint32_t mask = (uint32_t)bins - 1;
-    // wave w owns the contiguous keys [w*m, (w+1)*m), m a multiple of 64
-    const int m = ((n + kSmallWaves * kWave - 1) / (kSmallWaves * kWave)) * kWave;
-    const int nr = m / kWave;  // rounds per wave, <= KPT
-    const int wbase = wave * m;
-    const uint64_t lt_mask = lane ? (~0ull >> (kWave - lane)) : 0ull;
+    const int shift = pass * J.db;
+    const bool to_final = ((J.npass - 1 - pass) & 1) == 0;
+    const uint32_t *kin = to_final ? J.keys_tmp : J.keys_final;  // (unused in the first pass)
+    const int32_t *vin = to_final ? J.vals_tmp : J.out.perm;
+    uint32_t *kout = to_final ? J.keys_final : J.keys_tmp;
+    int32_t *vout = to_final ? J.out.perm : J.vals_tmp;
+    const int my0 = blockIdx.x * kMidKeys;
 
-    const uint32_t *kin = nullptr;
-    const int32_t *vin = nullptr;
-    for (int pass = 0; pass < npass; ++pass) {
-        const bool to_final = ((npass - 1 - pass) & 1) == 0;
-        uint32_t *kout = to_final ? J.keys_final : J.keys_tmp;
-        int32_t *vout = to_final ? J.out.perm : J.vals_tmp;
-        const int shift = pass * db;
-        for (int i = tid; i < kSmallWaves * kSmallMaxBins / 2; i += kSmallThreads)
-            reinterpret_cast<uint32_t *>(&s_cnt[0][0])[i] = 0;
-        uint32_t key[KPT];
-        int32_t val[KPT];
-        uint32_t lrank[KPT];
+    for (int i = tid; i < bins; i += kMidThreads) {
+        s_tot[i] = 0, s_bef[i] = 0;
 #pragma unroll
-        for (int j = 0; j < KPT; ++j) {
-            const int i = wbase + j * kWave + lane;
-            const bool ok = j < nr && i < n;
-            key[j] = ok ? (kin ? kin[i] : load_key(J.parts, i)) : 0u;
-            val[j] = ok ? (vin ? vin[i] : i) : 0;
-        }
-        __syncthreads();
-#pragma unroll
-        for (int j = 0; j < KPT; ++j) {
-            if (j < nr) {  // uniform across the workgroup
-                const int i = wbase + j * kWave + lane;
-                const bool ok = i < n;
-                const uint32_t dg = (key[j] >> shift) & mask;
-                uint64_t peers = __ballot(ok);
-                for (int bit = 0; bit < db; ++bit) {
-                    const bool one = (dg >> bit) & 1u;
-                    const uint64_t mm = __ballot(one);
-                    peers &= one ? mm : ~mm;
-                }
-                const int leader = __ffsll((unsigned long long)peers) - 1;
-                uint32_t old = 0;
-                if (ok && lane == leader) {
-                    old = s_cnt[wave][dg];
-                    s_cnt[wave][dg] = (unsigned short)(old + __popcll(peers));
-                }
-                old = __shfl(old, leader < 0 ? 0 : leader, kWave);
-                lrank[j] = old + __popcll(peers & lt_mask);
-                __builtin_amdgcn_wave_barrier();
-            }
-        }
-        __syncthreads();
-        // per bin: exclusive prefix over the waves, total into s_tot
-        uint32_t tot = 0;
-        if (tid < bins) {
-#pragma unroll
-            for (int w = 0; w < kSmallWaves; ++w) {
-                const uint32_t c = s_cnt[w][tid];
-                s_cnt[w][tid] = (unsigned short)tot;
-                tot += c;
-            }
-        }
-        // exclusive scan of the bin totals over the 1024 threads
-        uint32_t inc = tot;
-#pragma unroll
-        for (int o = 1; o < kWave; o <<= 1) {
-            const uint32_t up = __shfl_up(inc, o, kWave);
-            if (lane >= o) inc += up;
-        }
-        if (lane == kWave - 1) s_w[wave] = inc;
-        __syncthreads();
-        uint32_t woff = 0;
-        for (int w = 0; w < wave; ++w) woff += s_w[w];
-        if (tid < bins) s_tot[tid] = woff + inc - tot;
-        __syncthreads();
-#pragma unroll
-        for (int j = 0; j < KPT; ++j) {
-            const int i = wbase + j * kWave + lane;
-            if (j < nr && i < n) {
-                const uint32_t dg = (key[j] >> shift) & mask;
-                const uint32_t pos = s_tot[dg] + s_cnt[wave][dg] + lrank[j];
-                kout[pos] = key[j];
-                vout[pos] = val[j];
-            }
-        }
-        __threadfence_block();
-        __syncthreads();
-        kin = kout;
-        vin = vout;
+        for (int w = 0; w < kMidWaves; ++w) s_cnt[w][i] = 0;
     }
-
-    // dedup: thread t owns the sorted positions [t*q, (t+1)*q)
-    const int q = (n + kSmallThreads - 1) / kSmallThreads;  // <= KPT
-    const int lo = tid * q;
-    uint32_t k[KPT];
-    bool head[KPT];
-    uint32_t mine = 0;
-    uint32_t prev = (lo > 0 && lo < n) ? J.keys_final[lo - 1] : 0;
+    // own keys first (their loads overlap the counting loop)
+    uint32_t key[kMidRounds];
+    int32_t val[kMidRounds];
 #pragma unroll
-    for (int j = 0; j < KPT; ++j) {
+    for (int j = 0; j < kMidRounds; ++j) {
+        const int i = my0 + wave * (kMidRounds * kWave) + j * kWave + lane;
+        const bool ok = i < n;
+        if constexpr (FIRST) key[j] = ok ? load_key(J.parts, i) : 0u, val[j] = i;
+        else key[j] = ok ? kin[i] : 0u, val[j] = ok ? vin[i] : 0;
+    }
+    __syncthreads();
+    constexpr int kBatch = 16;  // loads in flight per thread: the loop is latency-bound otherwise
+    for (int i0 = 0; i0 < n; i0 += kBatch * kMidThreads) {
+        uint32_t kb[kBatch];
+#pragma unroll
+        for (int u = 0; u < kBatch; ++u) {
+            const int i = i0 + u * kMidThreads + tid;
+            if constexpr (FIRST) kb[u] = i < n ? load_key(J.parts, i) : 0u;
+            else kb[u] = i < n ? kin[i] : 0u;
+        }
+#pragma unroll
+        for (int u = 0; u < kBatch; ++u) {
+            const int i = i0 + u * kMidThreads + tid;
+            if (i < n) {
+                const uint32_t dg = (kb[u] >> shift) & mask;
+                atomicAdd(&s_tot[dg], 1u);
+                if (i < my0) atomicAdd(&s_bef[dg], 1u);
+            }
+        }
+    }
+    __syncthreads();
+    block_exclusive_scan(s_tot, bins, s_w);  // s_tot[bin] = first position of the bin
+
+    const uint64_t lt_mask = lane ? (~0ull >> (kWave - lane)) : 0ull;
+    uint32_t lrank[kMidRounds];
+#pragma unroll
+    for (int j = 0; j < kMidRounds; ++j) {
+        const int i = my0 + wave * (kMidRounds * kWave) + j * kWave + lane;
+        const bool ok = i < n;
+        const uint32_t dg = (key[j] >> shift) & mask;
+        uint64_t peers = __ballot(ok);
+        for (int bit = 0; bit < J.db; ++bit) {
+            const bool one = (dg >> bit) & 1u;
+            const uint64_t mm = __ballot(one);
+            peers &= one ? mm : ~mm;
+        }
+        const int leader = __ffsll((unsigned long long)peers) - 1;
+        uint32_t old = 0;
+        if (ok && lane == leader) {
+            old = s_cnt[wave][dg];
+            s_cnt[wave][dg] = old + __popcll(peers);
+        }
+        old = __shfl(old, leader < 0 ? 0 : leader, kWave);
+        lrank[j] = old + __popcll(peers & lt_mask);
+        __builtin_amdgcn_wave_barrier();
+    }
+    __syncthreads();
+    for (int bin = tid; bin < bins; bin += kMidThreads) {
+        uint32_t run = s_tot[bin] + s_bef[bin];
+#pragma unroll
+        for (int w = 0; w < kMidWaves; ++w) {
+            const uint32_t c = s_cnt[w][bin];
+            s_cnt[w][bin] = run;
+            run += c;
+        }
+    }
+    __syncthreads();
+#pragma unroll
+    for (int j = 0; j < kMidRounds; ++j) {
+        const int i = my0 + wave * (kMidRounds * kWave) + j * kWave + lane;
+        if (i < n) {
+            const uint32_t dg = (key[j] >> shift) & mask;
+            const uint32_t pos = s_cnt[wave][dg] + lrank[j];
+            kout[pos] = key[j];
+            vout[pos] = val[j];
+        }
+    }
+}
+
+__global__ __launch_bounds__(kMidThreads) void inspect_mid_dedup_kernel(MidJobs jobs)
+{
+    __shared__ uint32_t s_red[kMidWaves], s_scan[kMidWaves];
+    const MidJob &J = jobs.j[blockIdx.y];
+    const int n = (int)J.n;
+    const int nblk = n > 0 ? (n + kMidKeys - 1) / kMidKeys : 1;
+    if ((int)blockIdx.x >= nblk) return;
+    const int tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid >> 6;
+    const uint32_t *keys = J.keys_final;
+    const int my0 = blockIdx.x * kMidKeys;
+    // run heads before this block
+    // (my0 is a multiple of 1024: every thread takes whole groups of four keys with one 128-bit
+    // load, plus the key in front of the group; eight groups in flight)
+    uint32_t before = 0;
+    for (int g0 = 0; g0 < my0 / 4; g0 += 8 * kMidThreads) {
+        uint4 q[8];
+        uint32_t pv[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+            const int g = g0 + u * kMidThreads + tid;
+            const bool ok = g < my0 / 4;
+            q[u] = ok ? reinterpret_cast<const uint4 *>(keys)[g] : make_uint4(0, 0, 0, 0);
+            pv[u] = (ok && g > 0) ? keys[4 * g - 1] : 0u;
+        }
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+            const int g = g0 + u * kMidThreads + tid;
+            if (g < my0 / 4)
+                before += ((g == 0 || q[u].x != pv[u]) ? 1 : 0) + (q[u].y != q[u].x ? 1 : 0) +
+                          (q[u].z != q[u].y ? 1 : 0) + (q[u].w != q[u].z ? 1 : 0);
+        }
+    }
+    before = (uint32_t)wave_sum_i((int)before);
+    if (lane == 0) s_red[wave] = before;
+    // thread owns 4 consecutive sorted positions
+    const int lo = my0 + tid * kMidRounds;
+    uint32_t k[kMidRounds];
+    bool head[kMidRounds];
+    uint32_t mine = 0;
+    uint32_t prev = (lo > 0 && lo < n) ? keys[lo - 1] : 0;
+#pragma unroll
+    for (int j = 0; j < kMidRounds; ++j) {
         const int i = lo + j;
-        const bool ok = j < q && i < n;
-        k[j] = ok ? J.keys_final[i] : 0;
-        head[j] = ok && (i == 0 || k[j] != prev);
+        k[j] = i < n ? keys[i] : 0;
+        head[j] = i < n && (i == 0 || k[j] != prev);
         prev = k[j];
         mine += head[j] ? 1 : 0;
     }
@@ -430,21 +470,21 @@ __global__ __launch_bounds__(kSmallThreads) void inspect_small_kernel(SmallJobs 
         const uint32_t up = __shfl_up(inc, o, kWave);
         if (lane >= o) inc += up;
     }
-    if (lane == kWave - 1) s_w[wave] = inc;
+    if (lane == kWave - 1) s_scan[wave] = inc;
     __syncthreads();
-    uint32_t run = inc - mine, all = 0;
-    for (int w = 0; w < kSmallWaves; ++w) {
-        run += w < wave ? s_w[w] : 0;
-        all += s_w[w];
-    }
-    if (tid == 0) {
-        J.out.num_unique[0] = (int32_t)all;
-        J.out.seg_offsets[all] = n;
+    before = 0;
+    uint32_t here = 0;
+    for (int w = 0; w < kMidWaves; ++w) before += s_red[w], here += s_scan[w];
+    uint32_t run = before + inc - mine;
+    for (int w = 0; w < wave; ++w) run += s_scan[w];
+    if ((int)blockIdx.x == nblk - 1 && tid == 0) {
+        J.out.num_unique[0] = (int32_t)(before + here);
+        J.out.seg_offsets[before + here] = n;
     }
 #pragma unroll
-    for (int j = 0; j < KPT; ++j) {
+    for (int j = 0; j < kMidRounds; ++j) {
         const int i = lo + j;
-        if (j < q && i < n) {
+        if (i < n) {
             if (head[j]) {
                 J.out.unique_ids[run] = (int64_t)k[j];
                 J.out.seg_offsets[run] = i;
@@ -517,6 +557,7 @@ static int validate_job(const kge_inspect_job *job, Parts *parts, int64_t *n_out
         parts->p[q] = job->parts[q];
         parts->end[q] = n;
     }
+    for (int q = job->n_parts; q < 4; ++q) parts->p[q] = job->parts[job->n_parts - 1], parts->end[q] = n;
     const kge_inspection *out = &job->out;
     if (n != out->n || n >= (int64_t(1) << 31)) return KGE_ESHAPE;
     if (!out->num_unique || !out->seg_offsets) return KGE_EINVAL;
@@ -578,35 +619,37 @@ int kge_inspect_batch(const kge_inspect_job *jobs, int n_jobs, void *stream)
         const int rc = validate_job(&jobs[q], &parts[q], &n[q]);
         if (rc) return rc;
     }
-    SmallJobs small{};
-    int n_small = 0;
-    int64_t small_max = 0;
+    MidJobs mid{};
+    int n_mid = 0, max_pass = 0;
+    int64_t mid_max = 0;
     for (int q = 0; q < n_jobs; ++q) {
-        if (n[q] > kSmallMaxN) {
+        if (n[q] > kMidMaxN) {
             const int rc = inspect_large(parts[q], n[q], jobs[q].n_rows, &jobs[q].out, jobs[q].workspace, st);
             if (rc) return rc;
             continue;
         }
         const SortPlan p = make_plan(n[q], jobs[q].n_rows);
         char *ws = static_cast<char *>(jobs[q].workspace);
-        SmallJob &J = small.j[n_small++];
+        MidJob &J = mid.j[n_mid++];
         J.parts = parts[q];
         J.n = n[q];
-        J.bits = p.bits;
+        J.npass = p.npass;
+        J.db = p.digit_bits;
         J.out = jobs[q].out;
         J.keys_final = reinterpret_cast<uint32_t *>(ws + p.off_keys0);
         J.keys_tmp = reinterpret_cast<uint32_t *>(ws + p.off_keys1);
         J.vals_tmp = reinterpret_cast<int32_t *>(ws + p.off_vals);
-        small_max = n[q] > small_max ? n[q] : small_max;
+        mid_max = n[q] > mid_max ? n[q] : mid_max;
+        max_pass = p.npass > max_pass ? p.npass : max_pass;
     }
-    if (n_small > 0) {
-        const dim3 grid(n_small), block(kSmallThreads);
-        if (small_max <= 8 * kSmallThreads)
-            hipLaunchKernelGGL(inspect_small_kernel<8>, grid, block, 0, st, small);
-        else if (small_max <= 16 * kSmallThreads)
-            hipLaunchKernelGGL(inspect_small_kernel<16>, grid, block, 0, st, small);
-        else
-            hipLaunchKernelGGL(inspect_small_kernel<32>, grid, block, 0, st, small);
+    if (n_mid > 0) {
+        const dim3 grid((unsigned)(mid_max > 0 ? ceil_div(mid_max, kMidKeys) : 1), (unsigned)n_mid), block(kMidThreads);
+        if (mid_max > 0)
+            for (int pass = 0; pass < max_pass; ++pass) {
+                if (pass == 0) hipLaunchKernelGGL(inspect_mid_pass_kernel<true>, grid, block, 0, st, mid, pass);
+                else hipLaunchKernelGGL(inspect_mid_pass_kernel<false>, grid, block, 0, st, mid, pass);
+            }
+        hipLaunchKernelGGL(inspect_mid_dedup_kernel, grid, block, 0, st, mid);
         KGE_CHECK_LAUNCH();
     }
     return KGE_OK;

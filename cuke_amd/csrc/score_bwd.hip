@@ -40,8 +40,18 @@ constexpr int kTI = 64;       // columns of the row per workgroup
 constexpr int kKL = 32;       // looper rows staged per step
 constexpr int kLP = kTI + 4;  // LDS pitch of a staged row
 
+template <int MODEL, bool OWNER_POS, int RO>
+struct TileShape {
+    static constexpr bool kRot = MODEL == KGE_ROTATE, kTH = MODEL == KGE_TRANSH;
+    static constexpr int TO = 16 * RO;
+    static constexpr int NPL = (kRot || (kTH && !OWNER_POS)) ? 2 : 1;
+    static constexpr int NC = kTH ? 3 : 1;
+    static constexpr int PG = TO + 4;
+    static constexpr int kLdsFloats = NPL * kKL * kLP + NC * kKL * PG;
+};
+
 template <int MODEL, int P, bool OWNER_POS, int RO>
-__global__ __launch_bounds__(256, KGE_TILE_OCC) void bwd_tile_kernel(TileArgs a)
+__device__ __forceinline__ void bwd_tile_body(const TileArgs &a, int lid, float *smem)
 {
     constexpr int TO = 16 * RO;
     constexpr bool kRot = MODEL == KGE_ROTATE, kTH = MODEL == KGE_TRANSH;
@@ -55,15 +65,15 @@ __global__ __launch_bounds__(256, KGE_TILE_OCC) void bwd_tile_kernel(TileArgs a)
     constexpr int SL = kKL / 16;                        // looper float4 per thread per plane
     constexpr int CPT = (TO * kKL / 4 + 255) / 256;     // coefficient float4 per thread per plane
 
-    __shared__ __align__(16) float sL[NPL][kKL][kLP];
-    __shared__ __align__(16) float sG[NC][kKL][PG];
+    float(*sL)[kKL][kLP] = reinterpret_cast<float(*)[kKL][kLP]>(smem);
+    float(*sG)[kKL][PG] = reinterpret_cast<float(*)[kKL][PG]>(smem + NPL * kKL * kLP);
 
     const int tid = threadIdx.x, tx = tid & 15, ty = tid >> 4;
     const int d = a.d, half = d >> 1;
     const int klen = pair_len<MODEL>(d);
     const int n_own = OWNER_POS ? a.C : a.N, n_loop = OWNER_POS ? a.N : a.C;
     int c, tile_y, tile_x;
-    if (!xcd_tile((klen + kTI - 1) / kTI, (n_own + TO - 1) / TO, a.n_chunks, c, tile_y, tile_x)) return;
+    if (!xcd_tile(lid, (klen + kTI - 1) / kTI, (n_own + TO - 1) / TO, a.n_chunks, c, tile_y, tile_x)) return;
     const int col = tile_x * kTI + tx * 4;
     const int ot0 = tile_y * TO;
     const bool vec = a.vec != 0;
@@ -280,32 +290,41 @@ __global__ __launch_bounds__(256, KGE_TILE_OCC) void bwd_tile_kernel(TileArgs a)
     }
 }
 
-template <int MODEL, int P, bool OWNER_POS>
-static int launch_tile_o(const TileArgs &a, int64_t n_chunks, hipStream_t st)
+// Both orientations in ONE launch: the first `grid_head` workgroups own positives (outputs
+// g0 / g1), the rest own negatives (output occ_neg).  The two halves are independent, and
+// together they fill the GPU better than either alone when the batch is small.
+template <int MODEL, int P, int RO>
+__global__ __launch_bounds__(256, KGE_TILE_OCC) void bwd_tile_kernel(TileArgs a, float *g0, float *g1, float *occ_neg,
+                                                                     int grid_head)
 {
-    const int n_own = OWNER_POS ? a.C : a.N;
-    const int klen = MODEL == KGE_ROTATE ? a.d / 2 : a.d;
-    const unsigned gx = (unsigned)ceil_div(klen, kTI);
-    const int64_t big = (int64_t)gx * ceil_div(n_own, 64) * n_chunks;
-    if (big >= 1024) {
-        hipLaunchKernelGGL((bwd_tile_kernel<MODEL, P, OWNER_POS, 4>),
-                           dim3(xcd_grid(gx, ceil_div(n_own, 64), n_chunks)), dim3(256), 0, st, a);
+    constexpr int kFloats = TileShape<MODEL, true, RO>::kLdsFloats > TileShape<MODEL, false, RO>::kLdsFloats
+                                ? TileShape<MODEL, true, RO>::kLdsFloats
+                                : TileShape<MODEL, false, RO>::kLdsFloats;
+    __shared__ __align__(16) float smem[kFloats];
+    if ((int)blockIdx.x < grid_head) {
+        a.out0 = g0, a.out1 = g1;
+        bwd_tile_body<MODEL, P, true, RO>(a, blockIdx.x, smem);
     } else {
-        hipLaunchKernelGGL((bwd_tile_kernel<MODEL, P, OWNER_POS, 2>),
-                           dim3(xcd_grid(gx, ceil_div(n_own, 32), n_chunks)), dim3(256), 0, st, a);
+        a.out0 = occ_neg, a.out1 = nullptr;
+        bwd_tile_body<MODEL, P, false, RO>(a, blockIdx.x - grid_head, smem);
     }
-    KGE_CHECK_LAUNCH();
-    return KGE_OK;
 }
 
 template <int MODEL, int P>
 static int launch_tiles(TileArgs a, float *g0, float *g1, float *occ_neg, int64_t n_chunks, hipStream_t st)
 {
-    a.out0 = g0, a.out1 = g1;
-    int rc = launch_tile_o<MODEL, P, true>(a, n_chunks, st);
-    if (rc) return rc;
-    a.out0 = occ_neg, a.out1 = nullptr;
-    return launch_tile_o<MODEL, P, false>(a, n_chunks, st);
+    const int klen = MODEL == KGE_ROTATE ? a.d / 2 : a.d;
+    const int64_t gx = ceil_div(klen, kTI);
+    const int64_t big = gx * (ceil_div(a.C, 64) + ceil_div(a.N, 64)) * n_chunks;
+    if (big >= 1024) {
+        const unsigned gh = xcd_grid(gx, ceil_div(a.C, 64), n_chunks), gn = xcd_grid(gx, ceil_div(a.N, 64), n_chunks);
+        hipLaunchKernelGGL((bwd_tile_kernel<MODEL, P, 4>), dim3(gh + gn), dim3(256), 0, st, a, g0, g1, occ_neg, (int)gh);
+    } else {
+        const unsigned gh = xcd_grid(gx, ceil_div(a.C, 32), n_chunks), gn = xcd_grid(gx, ceil_div(a.N, 32), n_chunks);
+        hipLaunchKernelGGL((bwd_tile_kernel<MODEL, P, 2>), dim3(gh + gn), dim3(256), 0, st, a, g0, g1, occ_neg, (int)gh);
+    }
+    KGE_CHECK_LAUNCH();
+    return KGE_OK;
 }
 
 // ---------------------------------------------------------------------------------------

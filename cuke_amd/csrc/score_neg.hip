@@ -72,7 +72,7 @@ __global__ __launch_bounds__(256, KGE_TILE_OCC) void score_neg_kernel(NegArgs a)
     const int tid = threadIdx.x, tx = tid & 15, ty = tid >> 4;
     const int srow = tid >> 3, scol = (tid & 7) * 4;
     int c, tile_y, tile_x;
-    if (!xcd_tile((a.N + TN - 1) / TN, (a.C + TB - 1) / TB, a.n_chunks, c, tile_y, tile_x)) return;
+    if (!xcd_tile(blockIdx.x, (a.N + TN - 1) / TN, (a.C + TB - 1) / TB, a.n_chunks, c, tile_y, tile_x)) return;
     const int bt0 = tile_y * TB, kt0 = tile_x * TN;
     const int d = a.d, half = d >> 1;
     const int klen = MODEL == KGE_ROTATE ? half : d;

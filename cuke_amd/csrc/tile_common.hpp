@@ -139,9 +139,9 @@ __device__ __forceinline__ void load_query(const float *ph, const float *pr, con
 // Returns false for the padding ids of the grid (see xcd_grid).
 constexpr int kXcds = 8;
 __host__ __device__ inline int xcd_split(int n_chunks) { return n_chunks >= kXcds ? 1 : kXcds / n_chunks; }
-__device__ __forceinline__ bool xcd_tile(int tiles_x, int tiles_y, int n_chunks, int &c, int &ty, int &tx)
+__device__ __forceinline__ bool xcd_tile(int lid, int tiles_x, int tiles_y, int n_chunks, int &c, int &ty, int &tx)
 {
-    const int lid = blockIdx.x, per = tiles_x * tiles_y;
+    const int per = tiles_x * tiles_y;
     const int split = xcd_split(n_chunks);
     const int per_v = (per + split - 1) / split;  // tiles of one virtual chunk
     const int xcd = lid % kXcds, k = lid / kXcds;

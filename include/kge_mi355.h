@@ -176,9 +176,9 @@ int kge_inspect(const int64_t *const *parts, const int64_t *part_len, int n_part
                 size_t workspace_bytes, void *stream);
 
 /*
- * Several inspections in one call (at most 4 jobs).  Index sets of up to 32768 ids are each
- * handled by a single workgroup and all of them share ONE kernel launch; larger sets run the
- * multi-block sort.  Same outputs as kge_inspect.  A training step inspects concat(h, t, neg)
+ * Several inspections in one call (at most 4 jobs).  Index sets of up to 65536 ids share
+ * their kernel launches (one per radix digit pass plus one for the dedup); larger sets run
+ * the multi-block sort one after the other.  Same outputs as kge_inspect.  A training step inspects concat(h, t, neg)
  * and r together this way.
  */
 typedef struct kge_inspect_job {
