@@ -22,7 +22,13 @@ namespace kge {
 typedef float floatx4 __attribute__((ext_vector_type(4)));
 
 constexpr int kTM = 32;          // triples per tile
-constexpr int kRing = 2;         // supersteps of B operands kept in flight per wave
+#ifndef KGE_TR_RING
+#define KGE_TR_RING 2
+#endif
+#ifndef KGE_TR_OCC
+#define KGE_TR_OCC 3
+#endif
+constexpr int kRing = KGE_TR_RING;  // supersteps of B operands kept in flight per wave
 constexpr int kMaxDimMfma = 1024;
 
 int launch_score_pos(const kge_tables *, const kge_batch *, float *, float *, float *, hipStream_t);
@@ -121,7 +127,7 @@ struct GemmArgs {
 // MODE 1: forward RESCAL   x = E[h],      y = x M,        score = y . E[t]
 // MODE 2: backward dX      x = xs rows,   y = x M^T -> occ_h = y, occ_t = -y (when occ_t is set)
 template <int MODE>
-__global__ __launch_bounds__(256, 3) void transr_gemm_kernel(GemmArgs a)
+__global__ __launch_bounds__(256, KGE_TR_OCC) void transr_gemm_kernel(GemmArgs a)
 {
     extern __shared__ __align__(16) float lds[];
     const int tile = blockIdx.x;
@@ -138,28 +144,55 @@ __global__ __launch_bounds__(256, 3) void transr_gemm_kernel(GemmArgs a)
     const int64_t rid = a.unique_ids[g];
     const float *M = a.proj + rid * (int64_t)d * d;
 
-    // stage the left operand: 8 lanes per row, float4 along k
-    for (int f = tid; f < kTM * (kpad / 4); f += 256) {
-        const int row = f / (kpad / 4), k4 = (f % (kpad / 4)) * 4;
-        float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
-        if (row < rows && k4 < d) {
-            if constexpr (MODE == 2) {
-                v = *reinterpret_cast<const float4 *>(a.xs + (int64_t)(p0 + row) * d + k4);
-            } else {
-                const int b = a.perm[p0 + row];
-                v = *reinterpret_cast<const float4 *>(a.ent + a.h[b] * (int64_t)d + k4);
-                if constexpr (MODE == 0) {
-                    const float4 u = *reinterpret_cast<const float4 *>(a.ent + a.t[b] * (int64_t)d + k4);
-                    v = make_float4(v.x - u.x, v.y - u.y, v.z - u.z, v.w - u.w);
+    // triple ids of the tile first (one dependent-load chain per row instead of one per element)
+    __shared__ int s_b[kTM];
+    __shared__ int64_t s_h[kTM], s_t[kTM];
+    if (tid < kTM) {
+        const int b = tid < rows ? a.perm[p0 + tid] : 0;
+        s_b[tid] = b;
+        if constexpr (MODE != 2) {
+            s_h[tid] = a.h[b];
+            s_t[tid] = a.t[b];
+        }
+    }
+    __syncthreads();
+    // stage the left operand with all loads of a thread in flight together
+    {
+        const int per_row = kpad / 4;
+        constexpr int kStageBatch = 4;
+        for (int f0 = tid; f0 < kTM * per_row; f0 += 256 * kStageBatch) {
+            float4 v[kStageBatch], u[kStageBatch];
+#pragma unroll
+            for (int q = 0; q < kStageBatch; ++q) {
+                const int f = f0 + 256 * q;
+                const int row = f / per_row, k4 = (f % per_row) * 4;
+                v[q] = make_float4(0.f, 0.f, 0.f, 0.f), u[q] = v[q];
+                if (f < kTM * per_row && row < rows && k4 < d) {
+                    if constexpr (MODE == 2) {
+                        v[q] = *reinterpret_cast<const float4 *>(a.xs + (int64_t)(p0 + row) * d + k4);
+                    } else {
+                        v[q] = *reinterpret_cast<const float4 *>(a.ent + s_h[row] * (int64_t)d + k4);
+                        if constexpr (MODE == 0)
+                            u[q] = *reinterpret_cast<const float4 *>(a.ent + s_t[row] * (int64_t)d + k4);
+                    }
+                }
+            }
+#pragma unroll
+            for (int q = 0; q < kStageBatch; ++q) {
+                const int f = f0 + 256 * q;
+                if (f < kTM * per_row) {
+                    const int row = f / per_row, k4 = (f % per_row) * 4;
+                    *reinterpret_cast<float4 *>(&sX[row * pitch + k4]) =
+                        make_float4(v[q].x - u[q].x, v[q].y - u[q].y, v[q].z - u[q].z, v[q].w - u[q].w);
                 }
             }
         }
-        *reinterpret_cast<float4 *>(&sX[row * pitch + k4]) = v;
     }
     __syncthreads();
 
     const int li = lane & 15, kk = lane >> 4;
     const bool two_blocks = rows > 16;
+    const bool tiny = rows <= 4;
     float rowsum[8];  // norm / dot partials for rows 4*kk + r (+16)
 #pragma unroll
     for (int r = 0; r < 8; ++r) rowsum[r] = 0.0f;
@@ -199,6 +232,25 @@ __global__ __launch_bounds__(256, 3) void transr_gemm_kernel(GemmArgs a)
                         for (int s = 0; s < 4; ++s) bc[s] = ring[u][s];
                         if (q + u + kRing < nq) loadb(q + u + kRing, ring[u]);
                         const int qq = q + u;
+                        if (tiny) {
+                            // <= 4 triples: plain FMAs beat a 16-row MFMA block that is 3/4 padding.
+                            // Lane group kk covers its four k of the superstep; the groups are summed
+                            // after the loop.  acc_lo[e][r] = row r, column n0 + 4 li + e.
+#pragma unroll
+                            for (int r = 0; r < 4; ++r) {
+                                if (r >= rows) break;
+                                const float4 xr = *reinterpret_cast<const float4 *>(&sX[r * pitch + 16 * qq + 4 * kk]);
+                                const float xs4[4] = {xr.x, xr.y, xr.z, xr.w};
+#pragma unroll
+                                for (int s = 0; s < 4; ++s) {
+                                    acc_lo[0][r] = fmaf(xs4[s], bc[s].x, acc_lo[0][r]);
+                                    acc_lo[1][r] = fmaf(xs4[s], bc[s].y, acc_lo[1][r]);
+                                    acc_lo[2][r] = fmaf(xs4[s], bc[s].z, acc_lo[2][r]);
+                                    acc_lo[3][r] = fmaf(xs4[s], bc[s].w, acc_lo[3][r]);
+                                }
+                            }
+                            continue;
+                        }
                         const float4 alo = *reinterpret_cast<const float4 *>(&sX[li * pitch + 16 * qq + 4 * kk]);
                         const float4 ahi = *reinterpret_cast<const float4 *>(&sX[(16 + li) * pitch + 16 * qq + 4 * kk]);
                         const float al[4] = {alo.x, alo.y, alo.z, alo.w}, ah[4] = {ahi.x, ahi.y, ahi.z, ahi.w};
@@ -239,6 +291,18 @@ __global__ __launch_bounds__(256, 3) void transr_gemm_kernel(GemmArgs a)
                         for (int e = 0; e < 4; ++e) bc[e] = ring[u][e];
                         if (q + u + kRing < nq) loadb(q + u + kRing, ring[u]);
                         const int qq = q + u;
+                        if (tiny) {  // acc_lo[e][r] = row r, column n0 + 16 e + li
+#pragma unroll
+                            for (int r = 0; r < 4; ++r) {
+                                if (r >= rows) break;
+                                const float4 xr = *reinterpret_cast<const float4 *>(&sX[r * pitch + 16 * qq + 4 * kk]);
+#pragma unroll
+                                for (int e = 0; e < 4; ++e)
+                                    acc_lo[e][r] = fmaf(xr.x, bc[e].x, fmaf(xr.y, bc[e].y,
+                                                   fmaf(xr.z, bc[e].z, fmaf(xr.w, bc[e].w, acc_lo[e][r]))));
+                            }
+                            continue;
+                        }
                         const float4 alo = *reinterpret_cast<const float4 *>(&sX[li * pitch + 16 * qq + 4 * kk]);
                         const float4 ahi = *reinterpret_cast<const float4 *>(&sX[(16 + li) * pitch + 16 * qq + 4 * kk]);
                         const float al[4] = {alo.x, alo.y, alo.z, alo.w}, ah[4] = {ahi.x, ahi.y, ahi.z, ahi.w};
@@ -257,6 +321,17 @@ __global__ __launch_bounds__(256, 3) void transr_gemm_kernel(GemmArgs a)
             }
         }
 
+        if (tiny) {  // sum the four k-slices; every lane group then holds rows 0..3 (group 0 writes)
+#pragma unroll
+            for (int e = 0; e < 4; ++e)
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    float v = acc_lo[e][r];
+                    v += __shfl_xor(v, 16, kWave);
+                    v += __shfl_xor(v, 32, kWave);
+                    acc_lo[e][r] = v;
+                }
+        }
         // epilogue for this sweep: lane holds rows 4 kk + r (and +16), columns per the mode
 #pragma unroll
         for (int blk = 0; blk < 2; ++blk) {
@@ -265,7 +340,7 @@ __global__ __launch_bounds__(256, 3) void transr_gemm_kernel(GemmArgs a)
             for (int r = 0; r < 4; ++r) {
                 const int row = 16 * blk + 4 * kk + r;
                 if (row >= rows) continue;
-                const int b = a.perm[p0 + row];
+                const int b = s_b[row];
                 float y[4];
 #pragma unroll
                 for (int e = 0; e < 4; ++e) y[e] = blk ? acc_hi[e][r] : acc_lo[e][r];
@@ -280,7 +355,7 @@ __global__ __launch_bounds__(256, 3) void transr_gemm_kernel(GemmArgs a)
                             for (int e = 0; e < 4; ++e) s += a.norm_p == 1 ? fabsf(y[e]) : y[e] * y[e];
                             rowsum[4 * blk + r] += s;
                         } else {
-                            const float4 tv = *reinterpret_cast<const float4 *>(a.ent + a.t[b] * (int64_t)d + col);
+                            const float4 tv = *reinterpret_cast<const float4 *>(a.ent + s_t[row] * (int64_t)d + col);
                             rowsum[4 * blk + r] += y[0] * tv.x + y[1] * tv.y + y[2] * tv.z + y[3] * tv.w;
                         }
                         if (a.resid)
@@ -316,8 +391,7 @@ __global__ __launch_bounds__(256, 3) void transr_gemm_kernel(GemmArgs a)
             __syncthreads();
             if (tid < rows) {
                 const float s = sRed[tid] + sRed[kTM + tid] + sRed[2 * kTM + tid] + sRed[3 * kTM + tid];
-                const int b = a.perm[p0 + tid];
-                a.pos[b] = (MODE == 0 && a.norm_p == 2) ? sqrtf(s) : s;
+                a.pos[s_b[tid]] = (MODE == 0 && a.norm_p == 2) ? sqrtf(s) : s;
             }
         }
     }
@@ -403,7 +477,7 @@ struct DmArgs {
 // of one group, 32 rows i); the four waves split the columns j; K runs over the chunk's triples,
 // operands prefetched four supersteps ahead.  Groups longer than one chunk write per-chunk
 // partial matrices that transr_dm_finish_kernel adds up (keeps the longest K loop at 16 supersteps).
-__global__ __launch_bounds__(256, 3) void transr_dm_kernel(DmArgs a)
+__global__ __launch_bounds__(256, KGE_TR_OCC) void transr_dm_kernel(DmArgs a)
 {
     const int d = a.d;
     const int nib = (d + 31) / 32;
