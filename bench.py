@@ -24,6 +24,19 @@ sys.path.insert(0, ROOT)
 HBM_PEAK_GBS = 8000.0       # MI355X HBM3E, published
 FP32_PEAK_TFLOPS = 157.3    # MI355X fp32 vector / fp32 MFMA, published
 
+# HBM bytes per launch of each workload's roofline kernel, from rocprofv3 --pmc FETCH_SIZE and
+# --pmc WRITE_SIZE runs of this script (KiB per dispatch), each scaled by what the same counter
+# reads for the 256 MiB copy kernel of --calibrate-copy (fetch x2.000, write x1.000).  The
+# summaries the numbers come from are profiles/score_path_kernels_<workload>.txt.
+MEASURED_TRAFFIC_BYTES = {
+    "cfg1_transe": 1_664_838,      # score_pos_kernel
+    "cfg2_distmult": 12_956_644,   # score_neg_kernel
+    "cfg2_complex": 12_989_600,    # score_neg_kernel
+    "cfg3_transr": 163_398_460,    # transr_gemm_kernel<0>
+    "cfg4_rotate": 12_094_015,     # score_neg_kernel
+    "cfg5_transh": 619_524_137,    # score_neg_kernel
+}
+
 
 def device_tables(w, dev):
     """Tables drawn on the GPU (seeded); benchmark-size tables are too large to push through numpy."""
@@ -245,9 +258,12 @@ def main():
             k_ms = time_events(only_neg, 100, torch)
         k_bytes, k_flops = neg_kernel_bytes(w), neg_kernel_flops(w)
     else:
-        kname = "score_pos_kernel" if w.model not in ("TransR",) else "transr_fwd_kernel"
+        # positive-only workloads: the forward call is one kernel (TransR: the tile-plan kernel,
+        # a few microseconds, plus the grouped MFMA kernel)
+        kname = "score_pos_kernel" if w.model != "TransR" else "transr_plan_kernel + transr_gemm_kernel<0>"
         k_ms = time_events(lambda: step.forward(stc), 100, torch)
-        k_bytes, k_flops = fwd_b, 0
+        k_bytes = fwd_b
+        k_flops = 2 * w.batch * w.dim * w.dim if w.model == "TransR" else 3 * w.batch * w.dim
     achieved = k_bytes / (k_ms * 1e-3) / 1e9
 
     out = {
@@ -266,9 +282,10 @@ def main():
         "step": {"algorithmic_bytes": total_b, "hbm_gbs": total_b / (ms * 1e-3) / 1e9,
                  "hbm_frac": total_b / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, "wall_s": wall, **stages},
         "roofline": {"kernel": kname, "bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": achieved / HBM_PEAK_GBS, "traffic": None, "kernel_ms": k_ms,
+                     "frac": achieved / HBM_PEAK_GBS, "traffic": MEASURED_TRAFFIC_BYTES.get(w.name),
+                     "kernel_ms": k_ms,
                      "algorithmic_bytes_per_launch": k_bytes,
-                     "fp32_valu": {"flops_per_launch": k_flops,
+                     ("fp32_mfma" if w.model == "TransR" else "fp32_valu"): {"flops_per_launch": k_flops,
                                    "achieved_tflops": k_flops / (k_ms * 1e-3) / 1e12,
                                    "frac_of_157.3": k_flops / (k_ms * 1e-3) / 1e12 / FP32_PEAK_TFLOPS}},
     }
