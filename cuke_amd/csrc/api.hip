@@ -17,6 +17,20 @@ __global__ void check_indices_kernel(const int64_t *idx, int64_t n, int64_t n_ro
     }
 }
 
+__global__ void flatten_negatives_kernel(const int64_t *h, const int64_t *r, const int64_t *t, const int64_t *neg,
+                                         int64_t B, int64_t C, int64_t N, int64_t *hf, int64_t *rf, int64_t *tf)
+{
+    const int64_t total = B * (1 + N);
+    for (int64_t p = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; p < total; p += (int64_t)gridDim.x * blockDim.x) {
+        if (p < B) {
+            hf[p] = h[p], rf[p] = r[p], tf[p] = t[p];
+        } else {
+            const int64_t q = p - B, b = q / N, k = q % N;
+            hf[p] = h[b], rf[p] = r[b], tf[p] = neg[(b / C) * N + k];
+        }
+    }
+}
+
 static int validate_tables(const kge_tables *tab)
 {
     if (!tab || !tab->ent) return KGE_EINVAL;
@@ -104,6 +118,23 @@ int kge_score_fwd(const kge_tables *tab, const kge_batch *bat, float *pos, float
     }
     if (want_neg)
         return launch_score_neg(tab, bat, side_pos, tab->model == KGE_ROTATE ? residual : nullptr, neg, side_neg, st);
+    return KGE_OK;
+}
+
+int kge_flatten_negatives(const kge_batch *bat, int64_t *h_flat, int64_t *r_flat, int64_t *t_flat, void *stream)
+{
+    const int rc = validate_batch(bat);
+    if (rc) return rc;
+    if (!bat->neg) return KGE_EINVAL;
+    if (bat->batch == 0) return KGE_OK;
+    if (!h_flat || !r_flat || !t_flat) return KGE_EINVAL;
+    const int64_t total = bat->batch * (1 + bat->n_neg);
+    if (total >= (int64_t(1) << 31)) return KGE_ESHAPE;
+    const int64_t blocks = ceil_div(total, 256);
+    hipLaunchKernelGGL(flatten_negatives_kernel, dim3((unsigned)(blocks < 4096 ? blocks : 4096)), dim3(256), 0,
+                       as_stream(stream), bat->h, bat->r, bat->t, bat->neg, bat->batch, bat->chunk, bat->n_neg,
+                       h_flat, r_flat, t_flat);
+    KGE_CHECK_LAUNCH();
     return KGE_OK;
 }
 

@@ -121,6 +121,7 @@ class Forward:
     side_pos: torch.Tensor | None = None
     side_neg: torch.Tensor | None = None
     residual: torch.Tensor | None = None
+    flat_pos: torch.Tensor | None = None   # TransR / RESCAL with negatives: scores of the flattened batch
     batch: tuple = ()
     ent_insp: Inspection | None = None
     rel_insp: Inspection | None = None
@@ -215,6 +216,8 @@ class KGEModel:
     # -- scalar scores ---------------------------------------------------------------------
     def score(self, h, r, t, neg=None, chunk=None, ent_insp=None, rel_insp=None) -> Forward:
         """pos[B] and, with shared negatives, neg[B, N] scores."""
+        if neg is not None and self.model in ("TransR", "RESCAL"):
+            return self._score_projected_negatives(h, r, t, neg, chunk)
         bat, keep = self._batch(h, r, t, neg, chunk, ent_insp, rel_insp)
         B, N = bat.batch, bat.n_neg
         f32 = dict(dtype=torch.float32, device=self.dev)
@@ -232,6 +235,23 @@ class KGEModel:
                                             _ptr(fw.residual), _ptr(ws), nb, _stream()), "kge_score_fwd")
         return fw
 
+    def _score_projected_negatives(self, h, r, t, neg, chunk) -> Forward:
+        """TransR / RESCAL with shared negatives: the projection depends on the positive's relation,
+        so (as in the reference's neg_transR, examples.py:1447-1480) the B x N pairs are written out
+        as explicit triples behind the B positives and scored by the grouped per-relation kernels."""
+        bat, (h, r, t, neg, C_, N) = self._batch(h, r, t, neg, chunk)
+        B = bat.batch
+        total = B * (1 + N)
+        flat = [torch.empty(total, dtype=torch.int64, device=self.dev) for _ in range(3)]
+        _lib.check(_lib.lib().kge_flatten_negatives(C.byref(bat), *[_ptr(x) for x in flat], _stream()),
+                   "kge_flatten_negatives")
+        hf, rf, tf = flat
+        fw = self.score(hf, rf, tf, rel_insp=inspect([rf], self.n_rel))
+        fw.flat_pos = fw.pos
+        fw.neg = fw.pos[B:].view(B, N)
+        fw.pos = fw.pos[:B]
+        return fw
+
     def inspect_batch(self, h, r, t, neg=None):
         """Inspections of concat(h, t, neg) over the entity table and of r over the relations."""
         parts = [h, t] + ([neg.reshape(-1)] if neg is not None else [])
@@ -240,6 +260,17 @@ class KGEModel:
     # -- gradients ---------------------------------------------------------------------------
     def backward(self, fw: Forward, dpos=None, dneg=None) -> SparseGrads:
         """Sparse row gradients of sum(dpos * pos) + sum(dneg * neg)."""
+        if getattr(fw, "flat_pos", None) is not None:  # TransR / RESCAL negatives: one flat batch
+            B, N = fw.neg.shape
+            f32 = dict(dtype=torch.float32, device=self.dev)
+            g = torch.zeros(B * (1 + N), **f32)
+            if dpos is not None:
+                g[:B] = dpos.to(**f32)
+            if dneg is not None:
+                g[B:] = dneg.to(**f32).reshape(-1)
+            flat = Forward(fw.flat_pos, None, residual=fw.residual, batch=fw.batch, ent_insp=fw.ent_insp,
+                           rel_insp=fw.rel_insp)
+            return self.backward(flat, g)
         h, r, t, neg, C_, N = fw.batch
         if fw.ent_insp is None or fw.rel_insp is None:
             fw.ent_insp, fw.rel_insp = self.inspect_batch(h, r, t, neg)

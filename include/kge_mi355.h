@@ -224,6 +224,17 @@ int kge_score_bwd(const kge_tables *tab, const kge_batch *bat, const kge_saved *
 int kge_build_index(const int64_t *r, int64_t *uniq, int64_t *buf, int64_t *cnt, int64_t batch,
                     int64_t rel_num, void *stream);
 
+/*
+ * Shared negatives written out as explicit triples, the way the reference's neg_transR defines
+ * them (apps/examples/examples.py:1447-1480: every view is flattened to batch * blocksize rows).
+ * Outputs have B * (1 + n_neg) entries: the B positives first, then row B + b * n_neg + k =
+ * (h[b], r[b], neg[(b / chunk) * n_neg + k]).  TransR / RESCAL score shared negatives through
+ * this list and the grouped per-relation kernels (their projection depends on the positive's
+ * relation, so a negative row cannot be staged once per chunk as for the other models).
+ */
+int kge_flatten_negatives(const kge_batch *bat, int64_t *h_flat, int64_t *r_flat, int64_t *t_flat,
+                          void *stream);
+
 /* Sets flag[0] (int32, caller-zeroed) to 1 if any idx[i] is outside [0, n_rows). */
 int kge_check_indices(const int64_t *idx, int64_t n, int64_t n_rows, int32_t *flag, void *stream);
 

@@ -95,3 +95,31 @@ def test_proj_identity_reduces_to_transe(oracle):
     fw, _ = grouped_forward(m, ix)
     te, _ = oracle.score("TransE", a["E"], a["R"], None, a["h"], a["r"], a["t"], p=2)
     assert_close(fw.pos.cpu().numpy(), te, what="Proj = I")
+
+
+@pytest.mark.parametrize("model", ["TransR", "RESCAL"])
+def test_shared_negatives_through_flattened_triples(oracle, model):
+    # neg_transR (examples.py:1447-1480): out[b * bs + k] = (E[h[b]] - E[t'[k]]) Proj[r[b]] + R[r[b]]
+    w = synth.custom_workload(model, n_ent=200, n_rel=6, dim=40, batch=48, chunk=16, n_neg=12, sigma=0.2,
+                              rel_zipf=1.1, ent_zipf=1.1, seed=5)
+    a = w.arrays
+    m, ix = gpu_model(w)
+    fw = m.score(ix["h"], ix["r"], ix["t"], ix["neg"], w.chunk)
+    pos, negs = oracle.score(model, a["E"], a["R"], a["A"], a["h"], a["r"], a["t"], a["neg"], w.chunk, p=2)
+    assert_close(fw.pos.cpu().numpy(), pos, what="pos")
+    assert_close(fw.neg.cpu().numpy(), negs, what="neg")
+    if model == "TransR":  # the reference's output: one residual row per (b, k), b-major
+        fh = np.repeat(a["h"], w.n_neg); fr = np.repeat(a["r"], w.n_neg)
+        ft = np.array([a["neg"][(b // w.chunk) * w.n_neg + k] for b in range(w.batch) for k in range(w.n_neg)])
+        want = oracle.residual("TransR", a["E"], a["R"], a["A"], fh, fr, ft)
+        assert_close(fw.residual[w.batch:].cpu().numpy(), want, what="neg_transR residual rows")
+    rng = np.random.default_rng(3)
+    dpos = rng.standard_normal(w.batch).astype(np.float32)
+    dneg = rng.standard_normal((w.batch, w.n_neg)).astype(np.float32)
+    g = m.backward(fw, torch.from_numpy(dpos).cuda(), torch.from_numpy(dneg).cuda())
+    ref = oracle.backward(model, a["E"], a["R"], a["A"], a["h"], a["r"], a["t"], a["neg"], w.chunk, dpos, dneg, p=2)
+    assert np.array_equal(g.ent_ids.cpu().numpy(), ref.ent_ids)
+    assert_close(g.ent_rows.cpu().numpy(), ref.ent_rows, what="entity rows", rows=True)
+    if model == "TransR":
+        assert_close(g.rel_rows.cpu().numpy(), ref.rel_rows, what="relation rows", rows=True)
+    assert_close(g.aux_rows.cpu().numpy(), ref.aux_rows, what="projection gradients", rows=True)
