@@ -22,7 +22,7 @@ from . import _lib
 from ._lib import KgeError, MODELS
 
 __all__ = ["KGEModel", "TrainStep", "Inspection", "Forward", "SparseGrads", "inspect", "inspector", "transE",
-           "transH", "transR", "transF", "RESCAL", "margin_loss", "KgeError"]
+           "transH", "transR", "transF", "RESCAL", "margin_loss", "sparse_sgd", "sparse_adagrad", "KgeError"]
 
 
 def _stream() -> C.c_void_p:
@@ -315,6 +315,22 @@ def margin_loss(pos: torch.Tensor, neg: torch.Tensor, margin: float, sign: float
                                  _ptr(dpos), _ptr(dneg), _ptr(ws), ws_bytes, _stream()),
                "kge_margin_loss")
     return loss, dpos, dneg
+
+
+def sparse_sgd(table: torch.Tensor, insp: Inspection, rows: torch.Tensor, lr: float) -> None:
+    """table[id] -= lr * rows[u] for the inspection's unique ids (in place, no host sync)."""
+    t = _table(table, "table", table.dim())
+    _lib.check(_lib.lib().kge_sparse_sgd(_ptr(t), int(rows.shape[1]), _ptr(insp.unique_ids), _ptr(insp.num_unique_dev),
+                                         int(rows.shape[0]), _ptr(rows), float(lr), _stream()), "kge_sparse_sgd")
+
+
+def sparse_adagrad(table: torch.Tensor, state: torch.Tensor, insp: Inspection, rows: torch.Tensor, lr: float,
+                   eps: float = 1e-10) -> None:
+    """Row-wise Adagrad: state[id] += mean(g^2); table[id] -= lr * g / (sqrt(state[id]) + eps)."""
+    t = _table(table, "table", table.dim())
+    _lib.check(_lib.lib().kge_sparse_adagrad(_ptr(t), _ptr(state), int(rows.shape[1]), _ptr(insp.unique_ids),
+                                             _ptr(insp.num_unique_dev), int(rows.shape[0]), _ptr(rows), float(lr),
+                                             float(eps), _stream()), "kge_sparse_adagrad")
 
 
 # ---- the reference's positional call shapes --------------------------------------------------

@@ -235,6 +235,19 @@ int kge_build_index(const int64_t *r, int64_t *uniq, int64_t *buf, int64_t *cnt,
 int kge_flatten_negatives(const kge_batch *bat, int64_t *h_flat, int64_t *r_flat, int64_t *t_flat,
                           void *stream);
 
+/*
+ * Sparse optimizer step on one table from (unique ids, gradient rows) as kge_score_bwd leaves
+ * them: the step after backward.  The reference has no optimizer; these are the two row-wise
+ * rules of the DGL-KE lineage its data layer comes from.  ids are distinct, so rows never collide.
+ *   SGD      table[id] -= lr * g
+ *   Adagrad  state[id] += mean(g^2);  table[id] -= lr * g / (sqrt(state[id]) + eps)
+ * num_unique is the device scalar of the inspection; capacity = rows allocated behind ids/rows.
+ */
+int kge_sparse_sgd(float *table, int64_t dim, const int64_t *ids, const int32_t *num_unique, int64_t capacity,
+                   const float *rows, float lr, void *stream);
+int kge_sparse_adagrad(float *table, float *state, int64_t dim, const int64_t *ids, const int32_t *num_unique,
+                       int64_t capacity, const float *rows, float lr, float eps, void *stream);
+
 /* Sets flag[0] (int32, caller-zeroed) to 1 if any idx[i] is outside [0, n_rows). */
 int kge_check_indices(const int64_t *idx, int64_t n, int64_t n_rows, int32_t *flag, void *stream);
 

@@ -197,5 +197,21 @@ def build_index(r, rel_num):
     return uniq, buf, cnt, bool(rc)
 
 
+def sparse_sgd(table, ids, rows, lr):
+    """Returns the updated copy of ``table``."""
+    table, rows, ids = _f32(table).copy(), _f32(rows), _i64(ids)
+    _lib().orc_sparse_sgd(_fp(table), ctypes.c_int64(table.shape[1]), _fp(ids), ctypes.c_int64(ids.shape[0]),
+                          _fp(rows), ctypes.c_float(lr))
+    return table
+
+
+def sparse_adagrad(table, state, ids, rows, lr, eps=1e-10):
+    """Returns the updated copies of (table, state)."""
+    table, state, rows, ids = _f32(table).copy(), _f32(state).copy(), _f32(rows), _i64(ids)
+    _lib().orc_sparse_adagrad(_fp(table), _fp(state), ctypes.c_int64(table.shape[1]), _fp(ids),
+                              ctypes.c_int64(ids.shape[0]), _fp(rows), ctypes.c_float(lr), ctypes.c_float(eps))
+    return table, state
+
+
 def threads(fast=True) -> int:
     return int(_lib(fast).orc_threads())

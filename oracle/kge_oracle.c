@@ -544,6 +544,30 @@ int orc_build_index(const int64_t *r, int64_t batch, int64_t rel_num, int64_t *u
     return any_undefined;
 }
 
+/*
+ * Sparse optimizer steps (not in the reference; DGL-KE's row-wise rules, see the C header of the
+ * library).  ids are distinct.  Pinned in the tests against numpy fancy-indexing formulas.
+ */
+int orc_sparse_sgd(float *table, int64_t d, const int64_t *ids, int64_t n, const float *rows, float lr)
+{
+    for (int64_t u = 0; u < n; ++u)
+        for (int64_t j = 0; j < d; ++j) table[ids[u] * d + j] -= lr * rows[u * d + j];
+    return 0;
+}
+
+int orc_sparse_adagrad(float *table, float *state, int64_t d, const int64_t *ids, int64_t n, const float *rows,
+                       float lr, float eps)
+{
+    for (int64_t u = 0; u < n; ++u) {
+        float sq = 0.0f;
+        for (int64_t j = 0; j < d; ++j) sq += rows[u * d + j] * rows[u * d + j];
+        state[ids[u]] += sq / (float)d;
+        const float scale = lr / (sqrtf(state[ids[u]]) + eps);
+        for (int64_t j = 0; j < d; ++j) table[ids[u] * d + j] -= scale * rows[u * d + j];
+    }
+    return 0;
+}
+
 int orc_threads(void)
 {
 #ifdef _OPENMP

@@ -60,3 +60,27 @@ def test_check_indices():
     assert int(flag.item()) == 0
     assert L.kge_check_indices(C.c_void_p(idx.data_ptr()), 3, 9, C.c_void_p(flag.data_ptr()), st) == 0
     assert int(flag.item()) == 1
+
+
+@pytest.mark.parametrize("dim", [64, 22, 400])
+def test_sparse_optimizer_steps(oracle, dim):
+    """SGD / row-wise Adagrad on (unique ids, gradient rows) exactly as backward leaves them."""
+    from cuke_amd.kge import inspect, sparse_sgd, sparse_adagrad
+    rng = np.random.default_rng(dim)
+    n_rows = 3000
+    table = rng.standard_normal((n_rows, dim)).astype(np.float32)
+    state = rng.random(n_rows).astype(np.float32)
+    idx = rng.integers(0, n_rows, 1500)
+    ins = inspect([torch.from_numpy(idx).to(DEV)], n_rows)
+    U = ins.num_unique
+    rows_full = rng.standard_normal((1500, dim)).astype(np.float32)  # capacity n, first U rows valid
+    rows_dev = torch.from_numpy(rows_full).to(DEV)
+    ids = ins.ids().cpu().numpy()
+    t_dev = torch.from_numpy(table).to(DEV)
+    sparse_sgd(t_dev, ins, rows_dev, 0.05)
+    assert_close(t_dev.cpu().numpy(), oracle.sparse_sgd(table, ids, rows_full[:U], 0.05), what="sgd", rows=True)
+    t_dev = torch.from_numpy(table).to(DEV); s_dev = torch.from_numpy(state).to(DEV)
+    sparse_adagrad(t_dev, s_dev, ins, rows_dev, 0.05)
+    want_t, want_s = oracle.sparse_adagrad(table, state, ids, rows_full[:U], 0.05)
+    assert_close(t_dev.cpu().numpy(), want_t, what="adagrad table", rows=True)
+    assert_close(s_dev.cpu().numpy(), want_s, what="adagrad state")

@@ -335,3 +335,19 @@ def test_build_index_flags_sixteen_distinct(oracle):
     r = np.arange(16, dtype=np.int64)
     *_, undefined = oracle.build_index(r, 100)
     assert undefined
+
+
+def test_sparse_optimizer_steps_vs_numpy(oracle):
+    rng = np.random.default_rng(12)
+    table = rng.standard_normal((50, 12)).astype(np.float32)
+    state = rng.random(50).astype(np.float32)
+    ids = np.sort(rng.choice(50, 17, replace=False)).astype(np.int64)
+    rows = rng.standard_normal((17, 12)).astype(np.float32)
+    want = table.astype(np.float64).copy(); want[ids] -= 0.1 * rows
+    close(oracle.sparse_sgd(table, ids, rows, 0.1), want)
+    st = state.astype(np.float64).copy(); st[ids] += (rows.astype(np.float64) ** 2).mean(1)
+    want = table.astype(np.float64).copy(); want[ids] -= 0.1 * rows / (np.sqrt(st[ids])[:, None] + 1e-10)
+    got_t, got_s = oracle.sparse_adagrad(table, state, ids, rows, 0.1)
+    close(got_s, st); close(got_t, want)
+    untouched = np.setdiff1d(np.arange(50), ids)
+    assert np.array_equal(got_t[untouched], table[untouched])
