@@ -81,6 +81,7 @@ EXPORTS = {
                                  C.c_void_p]),
     "kge_sparse_adagrad": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int64, C.c_void_p, C.c_void_p, C.c_int64,
                                      C.c_void_p, C.c_float, C.c_float, C.c_void_p]),
+    "kge_sample_negatives": (C.c_int, [C.c_void_p, C.c_int64, C.c_int64, C.c_uint64, C.c_uint64, C.c_void_p]),
     "kge_check_indices": (C.c_int, [C.c_void_p, C.c_int64, C.c_int64, C.c_void_p, C.c_void_p]),
 }
 

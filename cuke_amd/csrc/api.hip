@@ -31,6 +31,23 @@ __global__ void flatten_negatives_kernel(const int64_t *h, const int64_t *r, con
     }
 }
 
+__device__ __forceinline__ uint64_t splitmix64(uint64_t z)
+{
+    z += 0x9E3779B97F4A7C15ull;
+    z = (z ^ (z >> 30)) * 0xBF58476D1CE4E5B9ull;
+    z = (z ^ (z >> 27)) * 0x94D049BB133111EBull;
+    return z ^ (z >> 31);
+}
+
+__global__ void sample_negatives_kernel(int64_t *out, int64_t count, uint64_t n_ent, uint64_t seed, uint64_t step)
+{
+    const uint64_t base = seed ^ splitmix64(step);
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < count; i += (int64_t)gridDim.x * blockDim.x) {
+        const uint64_t x = splitmix64(base ^ ((uint64_t)i * 0x9E3779B97F4A7C15ull));
+        out[i] = (int64_t)__umul64hi(x, n_ent);  // uniform over [0, n_ent)
+    }
+}
+
 static int validate_tables(const kge_tables *tab)
 {
     if (!tab || !tab->ent) return KGE_EINVAL;
@@ -134,6 +151,18 @@ int kge_flatten_negatives(const kge_batch *bat, int64_t *h_flat, int64_t *r_flat
     hipLaunchKernelGGL(flatten_negatives_kernel, dim3((unsigned)(blocks < 4096 ? blocks : 4096)), dim3(256), 0,
                        as_stream(stream), bat->h, bat->r, bat->t, bat->neg, bat->batch, bat->chunk, bat->n_neg,
                        h_flat, r_flat, t_flat);
+    KGE_CHECK_LAUNCH();
+    return KGE_OK;
+}
+
+int kge_sample_negatives(int64_t *out, int64_t count, int64_t n_ent, uint64_t seed, uint64_t step, void *stream)
+{
+    if (count < 0 || n_ent <= 0) return KGE_ESHAPE;
+    if (count == 0) return KGE_OK;
+    if (!out) return KGE_EINVAL;
+    const int64_t blocks = ceil_div(count, 256);
+    hipLaunchKernelGGL(sample_negatives_kernel, dim3((unsigned)(blocks < 2048 ? blocks : 2048)), dim3(256), 0,
+                       as_stream(stream), out, count, (uint64_t)n_ent, seed, step);
     KGE_CHECK_LAUNCH();
     return KGE_OK;
 }

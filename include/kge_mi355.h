@@ -248,6 +248,16 @@ int kge_sparse_sgd(float *table, int64_t dim, const int64_t *ids, const int32_t 
 int kge_sparse_adagrad(float *table, float *state, int64_t dim, const int64_t *ids, const int32_t *num_unique,
                        int64_t capacity, const float *rows, float lr, float eps, void *stream);
 
+/*
+ * Uniform negative entity ids for one batch, drawn on the device: out[i] for i < count is
+ *   mulhi64(splitmix64(seed ^ splitmix64(step) ^ (i * 0x9E3779B97F4A7C15)), n_ent)
+ * with splitmix64 the usual 64-bit finaliser.  Deterministic in (seed, step, i), no state, no
+ * exclusion of true positives (the reference's sampler is created with exclude_positive=False,
+ * apps/kge/data/data_init.py:26-43).  Stands where the reference calls the DGL EdgeSampler
+ * (apps/kge/data/sampler.py:342-353) for the chunked negative tails.
+ */
+int kge_sample_negatives(int64_t *out, int64_t count, int64_t n_ent, uint64_t seed, uint64_t step, void *stream);
+
 /* Sets flag[0] (int32, caller-zeroed) to 1 if any idx[i] is outside [0, n_rows). */
 int kge_check_indices(const int64_t *idx, int64_t n, int64_t n_rows, int32_t *flag, void *stream);
 

@@ -213,5 +213,25 @@ def sparse_adagrad(table, state, ids, rows, lr, eps=1e-10):
     return table, state
 
 
+def _splitmix64(z):
+    """splitmix64 finaliser on uint64 scalars or arrays (wrap-around arithmetic intended)."""
+    with np.errstate(over="ignore"):
+        z = np.asarray(z, dtype=np.uint64)
+        z = (z + np.uint64(0x9E3779B97F4A7C15))
+        z = (z ^ (z >> np.uint64(30))) * np.uint64(0xBF58476D1CE4E5B9)
+        z = (z ^ (z >> np.uint64(27))) * np.uint64(0x94D049BB133111EB)
+        return z ^ (z >> np.uint64(31))
+
+
+def sample_negatives(count, n_ent, seed, step):
+    """numpy restatement of the device negative sampler (see kge_sample_negatives in the C header)."""
+    with np.errstate(over="ignore"):
+        i = np.arange(count, dtype=np.uint64)
+        base = np.uint64(seed) ^ _splitmix64(np.uint64(step))
+        x = _splitmix64(base ^ (i * np.uint64(0x9E3779B97F4A7C15)))
+    # 64 x 64 -> high 64 bits, with Python integers (exact)
+    return np.array([(int(v) * int(n_ent)) >> 64 for v in x], dtype=np.int64)
+
+
 def threads(fast=True) -> int:
     return int(_lib(fast).orc_threads())
