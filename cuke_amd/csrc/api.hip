@@ -126,6 +126,7 @@ int kge_score_fwd(const kge_tables *tab, const kge_batch *bat, float *pos, float
     hipStream_t st = as_stream(stream);
     const bool want_neg = neg && bat->neg;
     if (want_neg && tab->model == KGE_TRANSH && !side_pos) return KGE_EINVAL;
+    if (want_neg && tab->model == KGE_ROTATE && !residual) return KGE_EINVAL;  // rotated heads buffer
     if (pos || side_pos || residual) {
         if ((tab->model == KGE_TRANSR || tab->model == KGE_RESCAL) && bat->rel_insp)
             rc = launch_transr_fwd(tab, bat, pos, residual, workspace, workspace_bytes, st);

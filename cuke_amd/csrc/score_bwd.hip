@@ -13,6 +13,8 @@
 //      (inspection perm / seg_offsets); every output row is written exactly once.
 #include <stdlib.h>
 
+#include <type_traits>
+
 #include "seg_reduce.hpp"
 #include "tile_common.hpp"
 
@@ -81,6 +83,8 @@ __device__ __forceinline__ void bwd_tile_body(const TileArgs &a, int lid, float 
     // ---- owners: registers -----------------------------------------------------------
     float4 own[NPO][RO];
     float alo[RO];
+    auto load_owners = [&](auto vtag) {
+    constexpr bool VEC = decltype(vtag)::value;
 #pragma unroll
     for (int o = 0; o < RO; ++o) {
         const int ol = ot0 + ty * RO + o;
@@ -93,17 +97,20 @@ __device__ __forceinline__ void bwd_tile_body(const TileArgs &a, int lid, float 
             if constexpr (kTH) alo[o] = a.side_pos[b];
             float4 q0 = zero4(), q1 = zero4();
             if constexpr (!kDot)
-                load_query<MODEL>(a.ent + a.h[b] * (int64_t)d, a.rel + rid * (int64_t)a.rel_dim,
-                                  kTH ? a.aux + rid * (int64_t)d : nullptr, alo[o], col, lim, half, vec, q0,
-                                  q1, (kRot && a.query) ? a.query + b * (int64_t)d : nullptr);
+                load_query<MODEL, VEC>(a.ent + a.h[b] * (int64_t)d, a.rel + rid * (int64_t)a.rel_dim,
+                                  kTH ? a.aux + rid * (int64_t)d : nullptr, alo[o], col, lim, half, q0,
+                                  q1, kRot ? a.query + b * (int64_t)d : nullptr);
             own[0][o] = q0;
             if constexpr (NPO == 2) own[1][o] = q1;
         } else {
             const float *pt = a.ent + a.neg[(int64_t)c * a.N + oc] * (int64_t)d;
-            own[0][o] = kDot ? zero4() : ld4(pt, col, lim, vec);
-            if constexpr (NPO == 2) own[1][o] = ld4(pt + half, col, lim, vec);
+            own[0][o] = kDot ? zero4() : ld4<VEC>(pt, col, lim);
+            if constexpr (NPO == 2) own[1][o] = ld4<VEC>(pt + half, col, lim);
         }
     }
+    };
+    if (vec) load_owners(std::true_type{});
+    else load_owners(std::false_type{});
 
     float4 acc[NOUT][RO];
 #pragma unroll
@@ -115,7 +122,8 @@ __device__ __forceinline__ void bwd_tile_body(const TileArgs &a, int lid, float 
     float4 rl[NPL][SL];
     float4 rc[NC][CPT];
 
-    auto load_step = [&](int l0) {
+    auto load_step_v = [&](auto vtag, auto ntag, int l0) {
+        constexpr bool VEC = decltype(vtag)::value, VECN = decltype(ntag)::value;
         // looper rows: thread stages rows ty + 16*s, columns col..col+3
 #pragma unroll
         for (int s = 0; s < SL; ++s) {
@@ -124,15 +132,15 @@ __device__ __forceinline__ void bwd_tile_body(const TileArgs &a, int lid, float 
             const int lc = ll < n_loop ? ll : n_loop - 1;
             if constexpr (OWNER_POS) {
                 const float *pt = a.ent + a.neg[(int64_t)c * a.N + lc] * (int64_t)d;
-                rl[0][s] = ld4(pt, col, lim, vec);
-                if constexpr (NPL == 2) rl[1][s] = ld4(pt + half, col, lim, vec);
+                rl[0][s] = ld4<VEC>(pt, col, lim);
+                if constexpr (NPL == 2) rl[1][s] = ld4<VEC>(pt + half, col, lim);
             } else {
                 const int64_t b = (int64_t)c * a.C + lc;
                 const int64_t rid = a.r[b];
                 float4 q0, q1;
-                load_query<MODEL>(a.ent + a.h[b] * (int64_t)d, a.rel + rid * (int64_t)a.rel_dim,
+                load_query<MODEL, VEC>(a.ent + a.h[b] * (int64_t)d, a.rel + rid * (int64_t)a.rel_dim,
                                   kTH ? a.aux + rid * (int64_t)d : nullptr, kTH ? a.side_pos[b] : 0.0f, col,
-                                  lim, half, vec, q0, q1, (kRot && a.query) ? a.query + b * (int64_t)d : nullptr);
+                                  lim, half, q0, q1, kRot ? a.query + b * (int64_t)d : nullptr);
                 rl[0][s] = q0;
                 if constexpr (NPL == 2) rl[1][s] = q1;
             }
@@ -154,9 +162,9 @@ __device__ __forceinline__ void bwd_tile_body(const TileArgs &a, int lid, float 
             }
             const int lim = inside ? a.N : 0;
             const int64_t off = ((int64_t)c * a.C + (inside ? bl : 0)) * a.N;
-            float4 g = ld4(a.dneg + off, kl, lim, a.vecn);
+            float4 g = ld4<VECN>(a.dneg + off, kl, lim);
             if constexpr (kL2) {
-                const float4 sc = ld4(a.sneg + off, kl, lim, a.vecn);
+                const float4 sc = ld4<VECN>(a.sneg + off, kl, lim);
                 g.x = sc.x > 0.0f ? g.x / sc.x : 0.0f;
                 g.y = sc.y > 0.0f ? g.y / sc.y : 0.0f;
                 g.z = sc.z > 0.0f ? g.z / sc.z : 0.0f;
@@ -164,10 +172,20 @@ __device__ __forceinline__ void bwd_tile_body(const TileArgs &a, int lid, float 
             }
             rc[0][s] = g;
             if constexpr (kTH) {
-                const float4 graw = ld4(a.dneg + off, kl, lim, a.vecn);
-                rc[1][s] = ld4(a.side_neg + off, kl, lim, a.vecn);
-                rc[2][s] = mul4(graw, ld4(a.side_neg + a.plane + off, kl, lim, a.vecn));
+                const float4 graw = ld4<VECN>(a.dneg + off, kl, lim);
+                rc[1][s] = ld4<VECN>(a.side_neg + off, kl, lim);
+                rc[2][s] = mul4(graw, ld4<VECN>(a.side_neg + a.plane + off, kl, lim));
             }
+        }
+    };
+
+    auto load_step = [&](int l0) {  // one uniform dispatch per step, no branch per load
+        if (vec) {
+            if (a.vecn) load_step_v(std::true_type{}, std::true_type{}, l0);
+            else load_step_v(std::true_type{}, std::false_type{}, l0);
+        } else {
+            if (a.vecn) load_step_v(std::false_type{}, std::true_type{}, l0);
+            else load_step_v(std::false_type{}, std::false_type{}, l0);
         }
     };
 
@@ -599,6 +617,7 @@ int kge_score_bwd(const kge_tables *tab, const kge_batch *bat, const kge_saved *
         if (model == KGE_TRANSF) return KGE_EUNSUPPORTED;
         if (normed && P == 2 && !saved->neg) return KGE_EINVAL;
         if (model == KGE_TRANSH && (!saved->side_pos || !saved->side_neg)) return KGE_EINVAL;
+        if (model == KGE_ROTATE && !saved->residual) return KGE_EINVAL;  // rotated heads from the forward pass
     }
     if (model == KGE_TRANSH && !grads->aux_rows) return KGE_EINVAL;
 

@@ -10,6 +10,8 @@
 // fp32 VALU; no matrix cores.
 #include <stdlib.h>
 
+#include <type_traits>
+
 #include "tile_common.hpp"
 
 namespace kge {
@@ -18,7 +20,7 @@ struct NegArgs {
     const float *ent, *rel, *aux;
     const int64_t *h, *r, *neg;
     const float *side_pos;  // TransH: w_b . h_b
-    const float *query;     // RotatE: rotated heads [B, d] from the positive kernel, or null
+    const float *query;     // RotatE: rotated heads [B, d] from the positive kernel (required)
     float *out;             // [B, N]
     float *side_neg;        // TransH save-for-backward [2, B, N] (optional):
                             //   plane 0: c = w_b . t'_k ; plane 1: sum_i phi(u_i) w_i with
@@ -92,7 +94,7 @@ __global__ __launch_bounds__(256, KGE_TILE_OCC) void score_neg_kernel(NegArgs a)
         pr[s] = a.rel + rid * (int64_t)a.rel_dim;
         pw[s] = MODEL == KGE_TRANSH ? a.aux + rid * (int64_t)d : nullptr;
         pa[s] = MODEL == KGE_TRANSH ? a.side_pos[b] : 0.0f;
-        pq[s] = (MODEL == KGE_ROTATE && a.query) ? a.query + b * (int64_t)d : nullptr;
+        pq[s] = MODEL == KGE_ROTATE ? a.query + b * (int64_t)d : nullptr;
     }
     const float *pt[SN];
     bool okk[SN];
@@ -105,23 +107,28 @@ __global__ __launch_bounds__(256, KGE_TILE_OCC) void score_neg_kernel(NegArgs a)
 
     float4 ra[NPA][SB], rt[NPT][SN];
 
-    auto load_slice = [&](int j0, int pass) {
+    auto load_slice_v = [&](auto vtag, int j0) {
+        constexpr bool VEC = decltype(vtag)::value;
         const int j = j0 + scol;
-        (void)pass;
 #pragma unroll
         for (int s = 0; s < SB; ++s) {
             const int lim = okb[s] ? klen : 0;
             float4 q0, q1;
-            load_query<MODEL>(ph[s], pr[s], pw[s], pa[s], j, lim, half, vec, q0, q1, pq[s]);
+            load_query<MODEL, VEC>(ph[s], pr[s], pw[s], pa[s], j, lim, half, q0, q1, pq[s]);
             ra[0][s] = q0;
             if constexpr (NPA == 2) ra[1][s] = q1;
         }
 #pragma unroll
         for (int s = 0; s < SN; ++s) {
             const int lim = okk[s] ? klen : 0;
-            rt[0][s] = ld4(pt[s], j, lim, vec);
-            if constexpr (MODEL == KGE_ROTATE) rt[1][s] = ld4(pt[s] + half, j, lim, vec);
+            rt[0][s] = ld4<VEC>(pt[s], j, lim);
+            if constexpr (MODEL == KGE_ROTATE) rt[1][s] = ld4<VEC>(pt[s] + half, j, lim);
         }
+    };
+
+    auto load_slice = [&](int j0, int) {  // one uniform branch per slice, none per load
+        if (vec) load_slice_v(std::true_type{}, j0);
+        else load_slice_v(std::false_type{}, j0);
     };
 
     float acc[RB][RK], cdot[RB][RK], acc2[RB][RK];

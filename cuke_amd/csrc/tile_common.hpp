@@ -11,15 +11,26 @@
 
 namespace kge {
 
-__device__ __forceinline__ float4 ld4(const float *p, int j, int lim, bool vec)
+// Four consecutive floats p[j .. j+3], zero where j + e >= lim.  Branch-free: an out-of-range
+// request reads p[0] (always a valid row start here) and discards it, so the callers' loads sit
+// in one basic block and the compiler can issue them back to back.
+template <bool VEC>
+__device__ __forceinline__ float4 ld4(const float *p, int j, int lim)
 {
-    if (vec) return j < lim ? *reinterpret_cast<const float4 *>(p + j) : make_float4(0, 0, 0, 0);
-    float4 q;
-    q.x = j + 0 < lim ? p[j + 0] : 0.0f;
-    q.y = j + 1 < lim ? p[j + 1] : 0.0f;
-    q.z = j + 2 < lim ? p[j + 2] : 0.0f;
-    q.w = j + 3 < lim ? p[j + 3] : 0.0f;
-    return q;
+    if constexpr (VEC) {  // rows are 16-byte aligned and lim % 4 == 0
+        const bool ok = j < lim;
+        const float4 v = *reinterpret_cast<const float4 *>(p + (ok ? j : 0));
+        return ok ? v : make_float4(0.f, 0.f, 0.f, 0.f);
+    } else {
+        float4 q;
+        const bool k0 = j + 0 < lim, k1 = j + 1 < lim, k2 = j + 2 < lim, k3 = j + 3 < lim;
+        const float x0 = p[k0 ? j + 0 : 0], x1 = p[k1 ? j + 1 : 0], x2 = p[k2 ? j + 2 : 0], x3 = p[k3 ? j + 3 : 0];
+        q.x = k0 ? x0 : 0.0f;
+        q.y = k1 ? x1 : 0.0f;
+        q.z = k2 ? x2 : 0.0f;
+        q.w = k3 ? x3 : 0.0f;
+        return q;
+    }
 }
 
 __device__ __forceinline__ void st4(float *p, int j, int lim, bool vec, float4 v)
@@ -60,36 +71,28 @@ __device__ __forceinline__ int pair_len(int d)
 
 // Four consecutive elements (index j .. j+3 of the reduction axis) of the query row.
 //   DistMult  q0 = h*r                   ComplEx  q0 = (h o r) laid out [re | im]
-//   TransE    q0 = h+r                   RotatE   q0 = Re(h e^{i theta}), q1 = Im(...)
+//   TransE    q0 = h+r                   RotatE   q0 = Re(h e^{i theta}), q1 = Im(...) (from pq)
 //   TransH    q0 = h + r - al*w (al = w.h), q1 = w
 // lim == 0 yields zeros (row outside the tile).
-// pq != nullptr: the row was already formed by the positive kernel (RotatE: rotating h costs a
-// sincos per element, far more than re-reading the stored result) and is simply loaded.
-template <int MODEL>
+// RotatE takes its query rows from pq, the [B, d] buffer of rotated heads.
+template <int MODEL, bool VEC>
 __device__ __forceinline__ void load_query(const float *ph, const float *pr, const float *pw, float al,
-                                           int j, int lim, int half, bool vec, float4 &q0, float4 &q1,
+                                           int j, int lim, int half, float4 &q0, float4 &q1,
                                            const float *pq = nullptr)
 {
     q1 = zero4();
-    if constexpr (MODEL == KGE_ROTATE) {
-        if (pq) {
-            q0 = ld4(pq, j, lim, vec);
-            q1 = ld4(pq + half, j, lim, vec);
-            return;
-        }
-    }
     if constexpr (MODEL == KGE_DISTMULT) {
-        q0 = mul4(ld4(ph, j, lim, vec), ld4(pr, j, lim, vec));
+        q0 = mul4(ld4<VEC>(ph, j, lim), ld4<VEC>(pr, j, lim));
     } else if constexpr (MODEL == KGE_TRANSE) {
-        q0 = add4(ld4(ph, j, lim, vec), ld4(pr, j, lim, vec));
+        q0 = add4(ld4<VEC>(ph, j, lim), ld4<VEC>(pr, j, lim));
     } else if constexpr (MODEL == KGE_COMPLEX) {
         float q[4];
-        if (vec) {  // half % 4 == 0: the four elements sit on one side of the re|im split
+        if constexpr (VEC) {  // half % 4 == 0: the four elements sit on one side of the re|im split
             const bool re = j < half;
             const int i = re ? j : j - half;
             const int l2 = lim ? half : 0;
-            const float4 hr = ld4(ph, i, l2, true), hi = ld4(ph + half, i, l2, true);
-            const float4 rr = ld4(pr, i, l2, true), ri = ld4(pr + half, i, l2, true);
+            const float4 hr = ld4<true>(ph, i, l2), hi = ld4<true>(ph + half, i, l2);
+            const float4 rr = ld4<true>(pr, i, l2), ri = ld4<true>(pr + half, i, l2);
             q[0] = re ? hr.x * rr.x - hi.x * ri.x : hr.x * ri.x + hi.x * rr.x;
             q[1] = re ? hr.y * rr.y - hi.y * ri.y : hr.y * ri.y + hi.y * rr.y;
             q[2] = re ? hr.z * rr.z - hi.z * ri.z : hr.z * ri.z + hi.z * rr.z;
@@ -98,31 +101,21 @@ __device__ __forceinline__ void load_query(const float *ph, const float *pr, con
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
                 const int jj = j + e;
-                if (jj < lim) {
-                    const int i = jj < half ? jj : jj - half;
-                    const float hr = ph[i], hi = ph[i + half], rr = pr[i], ri = pr[i + half];
-                    q[e] = jj < half ? hr * rr - hi * ri : hr * ri + hi * rr;
-                } else {
-                    q[e] = 0.0f;
-                }
+                const bool ok = jj < lim;
+                const int i = ok ? (jj < half ? jj : jj - half) : 0;
+                const float hr = ph[i], hi = ph[i + half], rr = pr[i], ri = pr[i + half];
+                q[e] = ok ? (jj < half ? hr * rr - hi * ri : hr * ri + hi * rr) : 0.0f;
             }
         }
         q0 = make_float4(q[0], q[1], q[2], q[3]);
     } else if constexpr (MODEL == KGE_ROTATE) {
-        const float4 hr = ld4(ph, j, lim, vec), hi = ld4(ph + half, j, lim, vec);
-        const float4 th = ld4(pr, j, lim, vec);
-        float4 sn, cs;
-        sincosf(th.x, &sn.x, &cs.x);
-        sincosf(th.y, &sn.y, &cs.y);
-        sincosf(th.z, &sn.z, &cs.z);
-        sincosf(th.w, &sn.w, &cs.w);
-        q0 = make_float4(hr.x * cs.x - hi.x * sn.x, hr.y * cs.y - hi.y * sn.y,
-                         hr.z * cs.z - hi.z * sn.z, hr.w * cs.w - hi.w * sn.w);
-        q1 = make_float4(hr.x * sn.x + hi.x * cs.x, hr.y * sn.y + hi.y * cs.y,
-                         hr.z * sn.z + hi.z * cs.z, hr.w * sn.w + hi.w * cs.w);
+        // the rotated head h e^{i theta} was written by the positive kernel ([re | im] row pq):
+        // a plain load here instead of a sincos per element in every tile that needs the row
+        q0 = ld4<VEC>(pq, j, lim);
+        q1 = ld4<VEC>(pq + half, j, lim);
     } else if constexpr (MODEL == KGE_TRANSH) {
-        const float4 vw = ld4(pw, j, lim, vec);
-        const float4 vh = ld4(ph, j, lim, vec), vr = ld4(pr, j, lim, vec);
+        const float4 vw = ld4<VEC>(pw, j, lim);
+        const float4 vh = ld4<VEC>(ph, j, lim), vr = ld4<VEC>(pr, j, lim);
         q1 = vw;
         q0 = make_float4((vh.x + vr.x) - al * vw.x, (vh.y + vr.y) - al * vw.y,
                          (vh.z + vr.z) - al * vw.z, (vh.w + vr.w) - al * vw.w);

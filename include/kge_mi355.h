@@ -120,7 +120,7 @@ typedef struct kge_saved {
     const float *side_neg;  /* [2, B, n_neg]: TransH, plane 0 = w_b . t'_k per pair,
                                plane 1 = sum_i phi(u_i) w_i (phi = sign for L1, u/||u|| for L2) */
     const float *residual;  /* [B, dim]: TransR residual rows / RESCAL E[h] Proj[r] rows;
-                               RotatE (optional): rotated heads h e^{i theta} as [re | im] */
+                               RotatE: rotated heads h e^{i theta} as [re | im] */
 } kge_saved;
 
 /* Sparse row gradients: row u of each array belongs to the u-th unique id of the
@@ -154,8 +154,10 @@ int kge_residual_fwd(const kge_tables *tab, const kge_batch *bat, float *out, vo
  * per-relation MFMA contractions and needs kge_score_fwd_workspace() bytes of workspace;
  * without it every triple streams its own projection.  `residual` [B, dim] receives the
  * projected rows (TransR: the residual, RESCAL: E[h] Proj[r]) that kge_score_bwd consumes.
- * RotatE: when `residual` is given it receives the rotated heads, which the shared-negative
- * kernels (forward and backward) then load instead of recomputing a sincos per element.
+ * RotatE: `residual` [B, dim] receives the rotated heads h e^{i theta}; the shared-negative
+ * kernels (forward and backward) load them instead of recomputing a sincos per element, so it
+ * is required whenever negatives are scored (filled by this call when pos is requested, or
+ * left from an earlier call on the same batch).
  */
 size_t kge_score_fwd_workspace(const kge_tables *tab, const kge_batch *bat);
 int kge_score_fwd(const kge_tables *tab, const kge_batch *bat, float *pos, float *neg,
