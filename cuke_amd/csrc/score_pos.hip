@@ -14,8 +14,8 @@ struct PosArgs {
     int d, rel_dim;
     float gamma;
     float *pos;       // [B] scores or nullptr
-    float *resid;     // [B, d] or nullptr: residual rows (TransE / TransH / TransR) or, for RotatE,
-                      // the rotated heads h e^{i theta} laid out [re | im]
+    float *resid;     // [B, d] or nullptr: residual rows (TransE / TransH / TransR), the projected heads
+                      // E[h] Proj[r] (RESCAL) or, for RotatE, the rotated heads h e^{i theta} laid out [re | im]
     float *side_pos;  // [B] TransH: w.h (used by the shared-negative kernels)
 };
 
@@ -112,6 +112,7 @@ __global__ __launch_bounds__(kPosWaves *kWave) void score_pos_kernel(PosArgs a)
                 const Vec<V> vt = Vec<V>::load(et + j);
 #pragma unroll
                 for (int e = 0; e < V; ++e) acc += s.v[e] * vt.v[e];
+                if (out && valid) s.store(out + j);  // E[h] Proj[r], consumed by the backward pass
             }
         }
     } else if constexpr (MODEL == KGE_DISTMULT) {

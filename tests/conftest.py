@@ -12,6 +12,16 @@ def pytest_configure(config):
     config.addinivalue_line("markers", "gpu: needs a real MI355X (run with -m gpu)")
 
 
+@pytest.fixture(scope="session", autouse=True)
+def hip_library():
+    """The tests load the in-tree library; it is compiled here only if nothing has been built yet."""
+    from cuke_amd import _lib
+    if not os.path.exists(_lib.LIB_PATH):
+        from cuke_amd import build
+        build.build(force=False)
+    return _lib.LIB_PATH
+
+
 @pytest.fixture(scope="session")
 def oracle():
     import oracle as orc

@@ -17,7 +17,12 @@ RTOL = 1e-5
 # implementations, so a few elements per million legitimately differ by more than the bar.
 # `outliers=(fraction, factor)` admits at most that fraction of elements, each within
 # factor x the bound; it is only used by the RotatE gradient tests.
-def assert_close(got, ref, rtol=RTOL, what="", rows=False, outliers=None):
+#
+# `global_floor=f` adds f x rtol x rms(whole array) to the bound.  Rows of 2-6 elements have no
+# usable scale of their own when the row is the nearly cancelling sum of many unit-size terms
+# (the rounding error follows the size of the terms, not of what is left), so the tests over
+# such narrow tables take a tenth of the array's scale as the floor.
+def assert_close(got, ref, rtol=RTOL, what="", rows=False, outliers=None, global_floor=0.0):
     got = np.asarray(got, np.float64)
     ref = np.asarray(ref, np.float64)
     assert got.shape == ref.shape, (what, got.shape, ref.shape)
@@ -29,6 +34,8 @@ def assert_close(got, ref, rtol=RTOL, what="", rows=False, outliers=None):
         rms = float(np.sqrt(np.mean(ref * ref)))
     err = np.abs(got - ref)
     bound = rtol * np.abs(ref) + rtol * rms
+    if global_floor:
+        bound = bound + global_floor * rtol * float(np.sqrt(np.mean(ref * ref)))
     bad = err > bound
     if outliers is not None and bad.any():
         frac, factor = outliers
