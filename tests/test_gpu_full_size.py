@@ -1,0 +1,138 @@
+"""The benchmark configurations at their full sizes.
+
+Every configuration is small enough for the CPU oracle to finish in seconds to a minute, so the
+forward scores and the sparse gradients are compared directly at full size, and on top of that
+through properties that do not need the oracle at all: a shared-negative score must equal the
+per-triple score of the explicit triple (h, r, neg), the backward pass is linear in the upstream
+gradients, and gradient rows are invariant under a permutation of the chunks."""
+import numpy as np
+import pytest
+import torch
+
+from cuke_amd import synth
+from helpers import assert_close, gpu_model
+
+pytestmark = pytest.mark.gpu
+
+FULL = ["cfg1_transe", "cfg2_distmult", "cfg2_complex", "cfg3_transr", "cfg4_rotate", "cfg5_transh"]
+
+
+@pytest.fixture(scope="module", params=FULL)
+def full(request):
+    # cfg5 is scored with the L1 norm: lattice-valued tables keep every residual away from the
+    # sign discontinuity of the L1 gradient
+    w = synth.make_workload(request.param, lattice=(request.param == "cfg5_transh"))
+    m, ix = gpu_model(w)
+    rel = None
+    if w.model == "TransR":
+        from cuke_amd.kge import inspect
+        rel = inspect([ix["r"]], m.n_rel)
+    fw = m.score(ix["h"], ix["r"], ix["t"], ix.get("neg"), w.chunk or None, rel_insp=rel)
+    yield w, m, ix, fw
+    del m, ix, fw
+    torch.cuda.empty_cache()
+
+
+def upstream(w, seed):
+    rng = np.random.default_rng(seed)
+    dpos = rng.standard_normal(w.batch).astype(np.float32)
+    dneg = rng.standard_normal((w.batch, w.n_neg)).astype(np.float32) if w.chunk else None
+    return dpos, dneg
+
+
+def dev(x):
+    return None if x is None else torch.from_numpy(x).cuda()
+
+
+def test_forward_against_oracle(oracle, full):
+    w, m, ix, fw = full
+    a = w.arrays
+    pos, negs = oracle.score(w.model, a["E"], a["R"], a["A"], a["h"], a["r"], a["t"], a.get("neg"), w.chunk,
+                             p=w.norm_p, gamma=w.gamma)
+    assert_close(fw.pos.cpu().numpy(), pos, what=f"{w.name} pos")
+    if w.chunk:
+        assert_close(fw.neg.cpu().numpy(), negs, what=f"{w.name} neg")
+
+
+def test_backward_against_oracle(oracle, full):
+    w, m, ix, fw = full
+    if not w.backward:
+        pytest.skip("forward-only configuration")
+    a = w.arrays
+    dpos, dneg = upstream(w, 11)
+    g = m.backward(fw, dev(dpos), dev(dneg))
+    ref = oracle.backward(w.model, a["E"], a["R"], a["A"], a["h"], a["r"], a["t"], a.get("neg"), w.chunk,
+                          dpos, dneg, p=w.norm_p)
+    assert np.array_equal(g.ent_ids.cpu().numpy(), ref.ent_ids)
+    assert np.array_equal(g.rel_ids.cpu().numpy(), ref.rel_ids)
+    out = (1e-5, 4.0) if w.model == "RotatE" else None
+    assert_close(g.ent_rows.cpu().numpy(), ref.ent_rows, what=f"{w.name} entity rows", rows=True, outliers=out)
+    if ref.rel_rows is not None and ref.rel_rows.size:
+        assert_close(g.rel_rows.cpu().numpy(), ref.rel_rows, what=f"{w.name} relation rows", rows=True,
+                     outliers=out)
+    if ref.aux_rows is not None:
+        assert_close(g.aux_rows.cpu().numpy(), ref.aux_rows, what=f"{w.name} aux rows", rows=True)
+
+
+def test_shared_negative_equals_explicit_triple(full):
+    """neg[b, k] from the tile kernels == the positive-path score of (h[b], r[b], neg[(b / C) * N + k])."""
+    w, m, ix, fw = full
+    if not w.chunk:
+        pytest.skip("no negatives")
+    g = torch.Generator(device="cpu").manual_seed(5)
+    n = 200_000
+    b = torch.randint(0, w.batch, (n,), generator=g).cuda()
+    k = torch.randint(0, w.n_neg, (n,), generator=g).cuda()
+    tails = ix["neg"][(b // w.chunk) * w.n_neg + k]
+    explicit = m.score(ix["h"][b], ix["r"][b], tails).pos
+    assert_close(fw.neg[b, k].cpu().numpy(), explicit.cpu().numpy(), what=f"{w.name} sampled negatives")
+
+
+def test_backward_is_linear_in_upstream_gradients(full):
+    w, m, ix, fw = full
+    if not w.backward:
+        pytest.skip("forward-only configuration")
+    x = upstream(w, 21)
+    y = upstream(w, 22)
+    ca, cb = np.float32(0.75), np.float32(-1.5)
+    mix = tuple(None if u is None else ca * u + cb * v for u, v in zip(x, y))
+    gx = m.backward(fw, dev(x[0]), dev(x[1]))
+    gy = m.backward(fw, dev(y[0]), dev(y[1]))
+    gm = m.backward(fw, dev(mix[0]), dev(mix[1]))
+    assert torch.equal(gx.ent_ids, gm.ent_ids) and torch.equal(gx.rel_ids, gm.rel_ids)
+    for name in ("ent_rows", "rel_rows", "aux_rows"):
+        rx, ry, rm = getattr(gx, name), getattr(gy, name), getattr(gm, name)
+        if rm is None or rm.numel() == 0:
+            continue
+        want = float(ca) * rx.double() + float(cb) * ry.double()
+        # Three fp32 evaluations are compared with each other, and the combination may cancel, so
+        # the error scale is that of the two terms (element and row rms), at 3 x the parity bar.
+        size = abs(float(ca)) * rx.double().abs() + abs(float(cb)) * ry.double().abs()
+        bound = 3e-5 * (size + size.pow(2).mean(dim=-1, keepdim=True).sqrt())
+        bad = (rm.double() - want).abs() > bound
+        assert not bool(bad.any()), f"{w.name} linearity of {name}: {int(bad.sum())}/{bad.numel()} outside tolerance"
+
+
+def test_gradients_invariant_under_chunk_permutation(full):
+    """Reordering whole chunks (with their negatives and upstream gradients) permutes the triples
+    but not the set of contributions to any table row; only the fp32 summation order changes."""
+    w, m, ix, fw = full
+    if not w.backward or not w.chunk:
+        pytest.skip("needs shared negatives and a backward pass")
+    C, N, nc = w.chunk, w.n_neg, w.n_chunks
+    perm = torch.randperm(nc, generator=torch.Generator().manual_seed(9)).cuda()
+    rows = (perm[:, None] * C + torch.arange(C, device="cuda")[None, :]).reshape(-1)
+    nrows = (perm[:, None] * N + torch.arange(N, device="cuda")[None, :]).reshape(-1)
+    dpos, dneg = (dev(u) for u in upstream(w, 31))
+    g0 = m.backward(fw, dpos, dneg)
+    fw2 = m.score(ix["h"][rows], ix["r"][rows], ix["t"][rows], ix["neg"][nrows], C)
+    assert torch.equal(fw2.pos, fw.pos[rows]) and torch.equal(fw2.neg, fw.neg[rows])
+    g1 = m.backward(fw2, dpos[rows].contiguous(), dneg[rows].contiguous())
+    assert torch.equal(g0.ent_ids, g1.ent_ids) and torch.equal(g0.rel_ids, g1.rel_ids)
+    out = (1e-5, 4.0) if w.model == "RotatE" else None
+    for name in ("ent_rows", "rel_rows", "aux_rows"):
+        r0, r1 = getattr(g0, name), getattr(g1, name)
+        if r0 is None or r0.numel() == 0:
+            continue
+        assert_close(r1.cpu().numpy(), r0.cpu().numpy(), rtol=2e-5, what=f"{w.name} {name} after permutation",
+                     rows=True, outliers=out)

@@ -24,7 +24,10 @@ def check(oracle, parts, n_rows):
 
 @pytest.mark.parametrize("n,n_rows", [(0, 10), (1, 10), (37, 1), (64, 64), (2048, 2000), (2049, 5),
                                       (5000, 1 << 11), (5000, (1 << 11) + 1), (12288, 1_000_000),
-                                      (49152, 4_000_000), (70000, 1 << 22), (300_000, 40_000)])
+                                      (49152, 4_000_000), (70000, 1 << 22), (300_000, 40_000),
+                                      # block size (1024 keys) and the mid / large path switch (65536 keys)
+                                      (1023, 50), (1024, 50), (1025, 50), (65535, 70_000), (65536, 1000),
+                                      (65537, 1000), (65537, 1 << 30)])
 def test_inspect_uniform(oracle, n, n_rows):
     rng = np.random.default_rng(n + n_rows)
     check(oracle, [rng.integers(0, n_rows, n, dtype=np.int64)], n_rows)
