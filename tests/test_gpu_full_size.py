@@ -136,3 +136,46 @@ def test_gradients_invariant_under_chunk_permutation(full):
             continue
         assert_close(r1.cpu().numpy(), r0.cpu().numpy(), rtol=2e-5, what=f"{w.name} {name} after permutation",
                      rows=True, outliers=out)
+
+
+@pytest.mark.parametrize("model,p", [("DistMult", 2), ("TransE", 2)])
+def test_more_than_2_to_31_scores(model, p):
+    """262144 x 8192 negatives = 2^31 scores per call: element offsets into the score and upstream
+    gradient arrays pass the 32-bit range.  Forward: sampled (b, k) against the per-triple path.
+    Backward: the whole batch against the sum of its two halves run as separate calls."""
+    C, N, nc, d = 1024, 8192, 256, 32
+    w = synth.custom_workload(model, n_ent=100_000, n_rel=100, dim=d, batch=C * nc, chunk=C, n_neg=N, norm_p=p,
+                              sigma=0.3, seed=77)
+    m, ix = gpu_model(w)
+    fw = m.score(ix["h"], ix["r"], ix["t"], ix["neg"], C)
+    assert fw.neg.numel() == 1 << 31
+    gen = torch.Generator(device="cpu").manual_seed(6)
+    b = torch.randint(0, w.batch, (300_000,), generator=gen).cuda()
+    k = torch.randint(0, N, (300_000,), generator=gen).cuda()
+    b[:4] = w.batch - 1  # the last rows sit at the top of the offset range
+    k[:4] = torch.tensor([N - 1, N - 2, 0, 1])
+    explicit = m.score(ix["h"][b], ix["r"][b], ix["neg"][(b // C) * N + k]).pos
+    assert_close(fw.neg[b, k].cpu().numpy(), explicit.cpu().numpy(), what=f"{model} sampled negatives")
+
+    dpos = torch.randn(w.batch, device="cuda", generator=torch.Generator(device="cuda").manual_seed(1))
+    dneg = torch.randn(w.batch, N, device="cuda", generator=torch.Generator(device="cuda").manual_seed(2))
+    g = m.backward(fw, dpos, dneg)
+    want_e = torch.zeros(w.n_ent, d, dtype=torch.float64, device="cuda")
+    want_r = torch.zeros(w.n_rel, d, dtype=torch.float64, device="cuda")
+    half = w.batch // 2
+    for lo in (0, half):
+        rows = slice(lo, lo + half)
+        nrows = slice(lo // C * N, (lo + half) // C * N)
+        fh = m.score(ix["h"][rows], ix["r"][rows], ix["t"][rows], ix["neg"][nrows], C)
+        assert torch.equal(fh.neg, fw.neg[rows])
+        gh = m.backward(fh, dpos[rows], dneg[rows])
+        want_e.index_add_(0, gh.ent_ids, gh.ent_rows.double())
+        want_r.index_add_(0, gh.rel_ids, gh.rel_rows.double())
+        del fh, gh
+    assert_close(g.ent_rows.cpu().numpy(), want_e[g.ent_ids].cpu().numpy(), rtol=2e-5, what=f"{model} entity rows",
+                 rows=True)
+    assert_close(g.rel_rows.cpu().numpy(), want_r[g.rel_ids].cpu().numpy(), rtol=2e-5, what=f"{model} relation rows",
+                 rows=True)
+    touched = torch.zeros(w.n_ent, dtype=torch.bool, device="cuda")
+    touched[g.ent_ids] = True
+    assert not bool(want_e[~touched].any())
