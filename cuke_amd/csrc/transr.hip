@@ -23,12 +23,18 @@ typedef float floatx4 __attribute__((ext_vector_type(4)));
 
 constexpr int kTM = 32;          // triples per tile
 #ifndef KGE_TR_RING
-#define KGE_TR_RING 2
+#define KGE_TR_RING 3
 #endif
 #ifndef KGE_TR_OCC
 #define KGE_TR_OCC 3
 #endif
 constexpr int kRing = KGE_TR_RING;  // supersteps of B operands kept in flight per wave
+#ifndef KGE_TR_DM_RING
+#define KGE_TR_DM_RING 2
+#endif
+constexpr int kDmRing = KGE_TR_DM_RING;  // the same for the dM kernel's operand stages
+constexpr int kThin = 4;            // a group's last tile with at most this many triples takes the thin path
+constexpr int kThinRing = 8;        // 128-bit projection loads in flight per thread on the thin path
 constexpr int kMaxDimMfma = 1024;
 
 int launch_score_pos(const kge_tables *, const kge_batch *, float *, float *, float *, hipStream_t);
@@ -47,19 +53,23 @@ struct TilePlan {
     int32_t *split_cnt;   // [max_split] number of partial slots
 };
 
+// Inclusive scan over the 1024 threads of the block: shuffle scan inside each wave, then the 16
+// wave totals are scanned by every wave for itself (two barriers in all).
 __device__ int block_inclusive_scan_1024(int v, int *s_scan)
 {
-    s_scan[threadIdx.x] = v;
-    __syncthreads();
-    for (int o = 1; o < 1024; o <<= 1) {  // Hillis-Steele
-        const int u = (int)threadIdx.x >= o ? s_scan[threadIdx.x - o] : 0;
-        __syncthreads();
-        s_scan[threadIdx.x] += u;
-        __syncthreads();
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+#pragma unroll
+    for (int o = 1; o < 64; o <<= 1) {
+        const int u = __shfl_up(v, o, kWave);
+        if (lane >= o) v += u;
     }
-    const int r = s_scan[threadIdx.x];
+    __syncthreads();  // s_scan may still be read from the previous call
+    if (lane == 63) s_scan[wave] = v;
     __syncthreads();
-    return r;
+    int before = 0;
+#pragma unroll
+    for (int w = 0; w < 16; ++w) before += w < wave ? s_scan[w] : 0;
+    return v + before;
 }
 
 __global__ __launch_bounds__(1024) void transr_plan_kernel(const int32_t *num_unique, const int32_t *seg_offsets,
@@ -113,7 +123,7 @@ __global__ __launch_bounds__(1024) void transr_plan_kernel(const int32_t *num_un
 struct GemmArgs {
     const float *ent, *rel, *proj;
     const int64_t *h, *r, *t;
-    const int32_t *perm, *seg_offsets;
+    const int32_t *perm, *seg_offsets, *num_unique;
     const int64_t *unique_ids;
     TilePlan plan;
     const float *xs;  // TRANSPOSED pass: left operand rows in sorted order [B, d]
@@ -121,7 +131,322 @@ struct GemmArgs {
     float *resid;     // forward: [B, d] rows y (nullable)
     float *occ_h, *occ_t;  // backward-dX: [B, d] each (occ_t nullable)
     int d, norm_p;
+    int thin_groups;       // upper bound of the number of relation groups = trailing thin workgroups
+    int max_tiles;         // leading workgroups: planned tiles
 };
+
+// ---- thin path: the last <= kThin triples of a relation group ---------------------------------
+// More than half of the distinct relations of a Zipf-distributed batch occur only a few times.
+// Such a tile is a matrix-vector product that streams the whole 4*d*d-byte projection for a
+// handful of rows: what matters is the number of bytes in flight, not the matrix cores.  The
+// thin kernels walk the projection as one contiguous array of 128-bit loads with kThinRing loads
+// per thread in flight and keep the (up to four) left-hand rows in LDS / registers.
+
+struct ThinTile {
+    int rows, p0;
+};
+
+// workgroup g looks at group g; returns rows == 0 when the group has no thin tail tile
+__device__ __forceinline__ ThinTile thin_tile_of_group(const int32_t *num_unique, const int32_t *seg_offsets, int g)
+{
+    ThinTile t{0, 0};
+    if (g >= num_unique[0]) return t;
+    const int s0 = seg_offsets[g], s1 = seg_offsets[g + 1];
+    const int rows = (s1 - s0 - 1) % kTM + 1;
+    if (rows > kThin) return t;
+    t.rows = rows;
+    t.p0 = s1 - rows;
+    return t;
+}
+
+// Y[r][:] = X[r][:] * M for the r < rows <= 4 triples of the tile (MODE 0 TransR, MODE 1 RESCAL).
+// Thread (phase, cq) owns the four columns 4 cq .. 4 cq + 3 and the projection rows
+// k = phase, phase + P, ... (P = 256 / (d / 4) phases): consecutive threads read consecutive
+// 16-byte pieces of the projection.  The phases are summed through LDS in a fixed order.
+template <int MODE>
+__device__ __forceinline__ void transr_thin_fwd_body(const GemmArgs &a, float *lds, int g)
+{
+    const ThinTile tt = thin_tile_of_group(a.num_unique, a.seg_offsets, g);
+    const int rows = tt.rows;
+    if (rows == 0) return;
+    const int d = a.d, nq4 = d >> 2, tid = threadIdx.x;
+    const int P = 256 / nq4;
+    const int kcap = ((d + P - 1) / P + kThinRing) * P;  // k range the prefetch can name
+    float4 *sXT = reinterpret_cast<float4 *>(lds);        // [kcap] x[0..3][k]
+    float4 *sRed = sXT + kcap;                             // [P][4][nq4]
+    float *sPart = reinterpret_cast<float *>(sRed + P * 4 * nq4);  // [4][nq4]
+    __shared__ int s_b[kThin];
+    __shared__ int64_t s_h[kThin], s_t[kThin];
+    const int64_t rid = a.unique_ids[g];
+    const float4 *M4 = reinterpret_cast<const float4 *>(a.proj + rid * (int64_t)d * d);
+    if (tid < kThin) {
+        const int b = tid < rows ? a.perm[tt.p0 + tid] : 0;
+        s_b[tid] = b;
+        s_h[tid] = a.h[b];
+        s_t[tid] = a.t[b];
+    }
+    for (int k = tid; k < kcap; k += 256) sXT[k] = make_float4(0.f, 0.f, 0.f, 0.f);
+    __syncthreads();
+    for (int f = tid; f < rows * nq4; f += 256) {
+        const int r = f / nq4, k4 = (f % nq4) * 4;
+        float4 v = *reinterpret_cast<const float4 *>(a.ent + s_h[r] * (int64_t)d + k4);
+        if constexpr (MODE == 0) {
+            const float4 u = *reinterpret_cast<const float4 *>(a.ent + s_t[r] * (int64_t)d + k4);
+            v = make_float4(v.x - u.x, v.y - u.y, v.z - u.z, v.w - u.w);
+        }
+        float *col = reinterpret_cast<float *>(sXT + k4) + r;
+        col[0] = v.x, col[4] = v.y, col[8] = v.z, col[12] = v.w;
+    }
+    __syncthreads();
+
+    const int cq = tid % nq4, ph = tid / nq4;
+    const bool active = ph < P;
+    float4 acc[4];
+#pragma unroll
+    for (int r = 0; r < 4; ++r) acc[r] = make_float4(0.f, 0.f, 0.f, 0.f);
+    if (active) {
+        // x is zero for k >= d, so a clamped (always valid) address needs no branch
+        auto loadm = [&](int k) { return M4[(int64_t)(k < d ? k : d - 1) * nq4 + cq]; };
+        float4 ring[kThinRing];
+#pragma unroll
+        for (int u = 0; u < kThinRing; ++u) ring[u] = loadm(ph + P * u);
+        for (int k0 = ph; k0 < d; k0 += P * kThinRing) {
+#pragma unroll
+            for (int u = 0; u < kThinRing; ++u) {
+                const int k = k0 + P * u;
+                float4 m = ring[u];
+                ring[u] = loadm(k + P * kThinRing);
+                const float4 x = sXT[k];  // zero beyond d
+                if (k >= d) m = make_float4(0.f, 0.f, 0.f, 0.f);  // keeps 0 * inf out
+                const float xr[4] = {x.x, x.y, x.z, x.w};
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    acc[r].x = fmaf(xr[r], m.x, acc[r].x);
+                    acc[r].y = fmaf(xr[r], m.y, acc[r].y);
+                    acc[r].z = fmaf(xr[r], m.z, acc[r].z);
+                    acc[r].w = fmaf(xr[r], m.w, acc[r].w);
+                }
+            }
+        }
+#pragma unroll
+        for (int r = 0; r < 4; ++r) sRed[(ph * 4 + r) * nq4 + cq] = acc[r];
+    }
+    __syncthreads();
+    for (int f = tid; f < rows * nq4; f += 256) {
+        const int r = f / nq4, q = f % nq4;
+        float4 y = sRed[r * nq4 + q];
+        for (int pp = 1; pp < P; ++pp) {
+            const float4 v = sRed[(pp * 4 + r) * nq4 + q];
+            y.x += v.x, y.y += v.y, y.z += v.z, y.w += v.w;
+        }
+        float sum;
+        if constexpr (MODE == 0) {
+            const float4 rv = *reinterpret_cast<const float4 *>(a.rel + rid * (int64_t)d + 4 * q);
+            y.x += rv.x, y.y += rv.y, y.z += rv.z, y.w += rv.w;
+            sum = a.norm_p == 1 ? fabsf(y.x) + fabsf(y.y) + fabsf(y.z) + fabsf(y.w)
+                                : y.x * y.x + y.y * y.y + y.z * y.z + y.w * y.w;
+        } else {
+            const float4 tv = *reinterpret_cast<const float4 *>(a.ent + s_t[r] * (int64_t)d + 4 * q);
+            sum = y.x * tv.x + y.y * tv.y + y.z * tv.z + y.w * tv.w;
+        }
+        if (a.resid) *reinterpret_cast<float4 *>(a.resid + (int64_t)s_b[r] * d + 4 * q) = y;
+        sPart[r * nq4 + q] = sum;
+    }
+    if (!a.pos) return;
+    __syncthreads();
+    const int wave = tid >> 6, lane = tid & 63;
+    if (wave < rows) {  // wave r adds row r's column sums in a fixed order
+        float s = 0.0f;
+        for (int q = lane; q < nq4; q += kWave) s += sPart[wave * nq4 + q];
+        s = wave_sum(s);
+        if (lane == 0) a.pos[s_b[wave]] = (MODE == 0 && a.norm_p == 2) ? sqrtf(s) : s;
+    }
+}
+
+static size_t thin_fwd_lds_bytes(int d)
+{
+    const int nq4 = d / 4, P = 256 / nq4;
+    const int kcap = ((d + P - 1) / P + kThinRing) * P;
+    return sizeof(float4) * ((size_t)kcap + (size_t)P * 4 * nq4) + sizeof(float) * 4 * (size_t)nq4;
+}
+
+// Sum over the 16 lanes of a DPP row; every lane of the row ends up with the total.
+__device__ __forceinline__ float row16_sum(float v)
+{
+    v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0xB1, 0xF, 0xF, true));   // quad_perm [1,0,3,2]
+    v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x4E, 0xF, 0xF, true));   // quad_perm [2,3,0,1]
+    v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x141, 0xF, 0xF, true));  // row_half_mirror
+    v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x140, 0xF, 0xF, true));  // row_mirror
+    return v;
+}
+
+// dX for a thin tile: Y[r][j] = sum_k Q[r][k] M[j][k].  Sixteen lanes share one projection row j:
+// lane i of the group reads the k-quads i, i + 16, ... (each load instruction covers 256
+// contiguous bytes of the row) against its quads of the (up to four) Q rows held in registers,
+// and the sixteen partial sums are added with four DPP steps, no LDS and no barrier in the loop.
+// A wave works on four rows at a time, the four waves interleave; NS = quads per lane.  Rows wider
+// than 64 NS floats are covered in several passes over k-chunks that add into the staged result.
+template <int NS>
+__device__ __forceinline__ void transr_thin_dx_body(const GemmArgs &a, float *sY, int g)  // sY: [4][d]
+{
+    const ThinTile tt = thin_tile_of_group(a.num_unique, a.seg_offsets, g);
+    const int rows = tt.rows;
+    if (rows == 0) return;
+    constexpr int R = 8 / NS;  // row groups in flight per wave: R * NS loads per lane
+    const int d = a.d, nq4 = d >> 2, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int li = lane & 15, sub = lane >> 4;
+    __shared__ int s_b[kThin];
+    if (tid < kThin) s_b[tid] = tid < rows ? a.perm[tt.p0 + tid] : 0;
+    const int64_t rid = a.unique_ids[g];
+    const float4 *M4 = reinterpret_cast<const float4 *>(a.proj + rid * (int64_t)d * d);
+    const int jfirst = 4 * wave + sub;  // row of (step i, wave, sub): j = 16 i + 4 wave + sub
+    for (int c0 = 0; c0 < nq4; c0 += 16 * NS) {  // k-chunk of 16 NS quads
+        float4 q[NS][4];
+        int qc[NS];
+#pragma unroll
+        for (int s = 0; s < NS; ++s) {
+            const int c = c0 + li + 16 * s;
+            qc[s] = c < nq4 ? c : 0;
+#pragma unroll
+            for (int r = 0; r < 4; ++r)  // zero beyond the row and beyond `rows`: clamped loads then add nothing
+                q[s][r] = (c < nq4 && r < rows)
+                              ? *reinterpret_cast<const float4 *>(a.xs + (int64_t)(tt.p0 + r) * d + 4 * c)
+                              : make_float4(0.f, 0.f, 0.f, 0.f);
+        }
+        auto loadrow = [&](int j, float4 *dst) {
+            const int64_t base = (int64_t)(j < d ? j : d - 1) * nq4;
+#pragma unroll
+            for (int s = 0; s < NS; ++s) dst[s] = M4[base + qc[s]];
+        };
+        float4 ring[R][NS];
+#pragma unroll
+        for (int u = 0; u + 1 < R || u == 0; ++u) loadrow(jfirst + 16 * u, ring[u]);
+        for (int j0 = jfirst; j0 < d + 16 * R; j0 += 16 * R) {  // uniform trip count over the workgroup
+#pragma unroll
+            for (int u = 0; u < R; ++u) {
+                const int j = j0 + 16 * u;
+                if constexpr (R > 1) {
+                    loadrow(j + 16 * (R - 1), ring[(u + R - 1) % R]);
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+                float p[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                for (int s = 0; s < NS; ++s) {
+                    const float4 m = ring[u][s];
+#pragma unroll
+                    for (int r = 0; r < 4; ++r)
+                        p[r] = fmaf(q[s][r].x, m.x, fmaf(q[s][r].y, m.y, fmaf(q[s][r].z, m.z, fmaf(q[s][r].w, m.w, p[r]))));
+                }
+                if constexpr (R == 1) loadrow(j + 16, ring[0]);
+#pragma unroll
+                for (int r = 0; r < 4; ++r) p[r] = row16_sum(p[r]);
+                if (li < 4 && j < d) {
+                    const float v = li == 0 ? p[0] : (li == 1 ? p[1] : (li == 2 ? p[2] : p[3]));
+                    sY[li * d + j] = c0 == 0 ? v : sY[li * d + j] + v;  // same lane owns (li, j) in every pass
+                }
+            }
+        }
+    }
+    __syncthreads();
+    for (int f = tid; f < rows * nq4; f += 256) {
+        const int r = f / nq4, c = f % nq4;
+        const float4 y = *reinterpret_cast<const float4 *>(&sY[r * d + 4 * c]);
+        const int64_t o = (int64_t)s_b[r] * d + 4 * c;
+        *reinterpret_cast<float4 *>(a.occ_h + o) = y;
+        if (a.occ_t) *reinterpret_cast<float4 *>(a.occ_t + o) = make_float4(-y.x, -y.y, -y.z, -y.w);
+    }
+}
+
+static size_t thin_dx_lds_bytes(int d) { return sizeof(float) * 4 * (size_t)d; }
+
+// One sweep of a tile: acc (+)= X[32 x d] * B over all supersteps for this wave's columns
+// [n0, n0 + wcols).  Everything inside the loop is free of branches: addresses are clamped
+// into the projection instead of predicating the loads (the staged X is zero for k >= d, and a
+// lane beyond wcols computes columns nobody stores), the prefetch of a superstep past the end
+// re-reads the last one, and the superstep count is rounded up to whole ring turns with the X
+// operand selected to zero.  A branch around a load makes the compiler wait for every load
+// in flight at each step, which turns the prefetch ring into a depth of one.
+//   MODE 0/1: B[k][j] = M[k][n0 + 4 li + e], one float4 per k row per lane;
+//   MODE 2:   B[k][j] = M[n0 + 16 e + li][k], a lane's float4 along k serves the four steps.
+template <int MODE, bool TWO>
+__device__ __forceinline__ void gemm_sweep(const float *M, const float *sX, int pitch, int d, int nq, int n0,
+                                           int wcols, int li, int kk, floatx4 (&acc_lo)[4], floatx4 (&acc_hi)[4])
+{
+    const float *base[4];
+    if constexpr (MODE != 2) {
+        const int col = n0 + (4 * li < wcols ? 4 * li : 0);
+#pragma unroll
+        for (int s = 0; s < 4; ++s) base[s] = M + col;
+    } else {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            const int col = 16 * e + li;
+            base[e] = M + (int64_t)(n0 + (col < wcols ? col : 0)) * d;
+        }
+    }
+    auto loadb = [&](int q, float4 *dst) {
+        q = q < nq ? q : nq - 1;
+        if constexpr (MODE != 2) {
+#pragma unroll
+            for (int s = 0; s < 4; ++s) {
+                const int k = 16 * q + 4 * kk + s;
+                dst[s] = *reinterpret_cast<const float4 *>(base[s] + (int64_t)(k < d ? k : d - 1) * d);
+            }
+        } else {
+            const int k = 16 * q + 4 * kk;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) dst[e] = *reinterpret_cast<const float4 *>(base[e] + (k < d ? k : d - 4));
+        }
+    };
+    // Ring of kRing slots: step qq consumes slot qq % kRing and first refills the slot consumed one
+    // step earlier with superstep qq + kRing - 1, so kRing - 1 supersteps are always in flight and
+    // the loads are issued ahead of the matrix-core work of the step (pinned by the scheduling
+    // barrier; left alone the compiler sinks them below it and the ring degenerates to depth 1).
+    float4 ring[kRing][4];
+#pragma unroll
+    for (int u = 0; u + 1 < kRing; ++u) loadb(u, ring[u]);
+    const float *xlo = sX + li * pitch + 4 * kk, *xhi = sX + (16 + li) * pitch + 4 * kk;
+    for (int q = 0; q < nq; q += kRing) {
+#pragma unroll
+        for (int u = 0; u < kRing; ++u) {
+            const int qq = q + u;
+            loadb(qq + kRing - 1, ring[(u + kRing - 1) % kRing]);
+            __builtin_amdgcn_sched_barrier(0);
+            float4 bc[4];
+#pragma unroll
+            for (int s = 0; s < 4; ++s) bc[s] = ring[u][s];
+            const bool live = qq < nq;
+            const int qc = live ? qq : nq - 1;
+            float4 alo = *reinterpret_cast<const float4 *>(xlo + 16 * qc);
+            float4 ahi = TWO ? *reinterpret_cast<const float4 *>(xhi + 16 * qc) : make_float4(0.f, 0.f, 0.f, 0.f);
+            if (!live) alo = make_float4(0.f, 0.f, 0.f, 0.f), ahi = alo;
+            const float al[4] = {alo.x, alo.y, alo.z, alo.w}, ah[4] = {ahi.x, ahi.y, ahi.z, ahi.w};
+            if constexpr (MODE != 2) {
+#pragma unroll
+                for (int s = 0; s < 4; ++s) {
+                    const float bv[4] = {bc[s].x, bc[s].y, bc[s].z, bc[s].w};
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        acc_lo[e] = __builtin_amdgcn_mfma_f32_16x16x4f32(al[s], bv[e], acc_lo[e], 0, 0, 0);
+                        if constexpr (TWO)
+                            acc_hi[e] = __builtin_amdgcn_mfma_f32_16x16x4f32(ah[s], bv[e], acc_hi[e], 0, 0, 0);
+                    }
+                }
+            } else {
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    const float bv[4] = {bc[e].x, bc[e].y, bc[e].z, bc[e].w};
+#pragma unroll
+                    for (int s = 0; s < 4; ++s) {
+                        acc_lo[e] = __builtin_amdgcn_mfma_f32_16x16x4f32(al[s], bv[s], acc_lo[e], 0, 0, 0);
+                        if constexpr (TWO)
+                            acc_hi[e] = __builtin_amdgcn_mfma_f32_16x16x4f32(ah[s], bv[s], acc_hi[e], 0, 0, 0);
+                    }
+                }
+            }
+        }
+    }
+}
 
 // MODE 0: forward TransR   x = E[h]-E[t], y = x M + R[r], score = ||y||_p
 // MODE 1: forward RESCAL   x = E[h],      y = x M,        score = y . E[t]
@@ -130,6 +455,21 @@ template <int MODE>
 __global__ __launch_bounds__(256, KGE_TR_OCC) void transr_gemm_kernel(GemmArgs a)
 {
     extern __shared__ __align__(16) float lds[];
+    // Workgroups [0, max_tiles) take the planned 32-triple tiles, the following `thin_groups`
+    // stream the thin group tails.  The tiles come first because each is one long chain of
+    // dependent loads and matrix-core steps (about 20 us whatever else runs); the thin
+    // workgroups then fill the remaining slots and the memory bandwidth.
+    if ((int)blockIdx.x >= a.max_tiles) {
+        if constexpr (MODE == 2) {
+            const int ns = (a.d / 4 + 15) / 16;  // k-quads per lane of a 16-lane row group
+            if (ns <= 1) transr_thin_dx_body<1>(a, lds, blockIdx.x - a.max_tiles);
+            else if (ns <= 2) transr_thin_dx_body<2>(a, lds, blockIdx.x - a.max_tiles);
+            else transr_thin_dx_body<4>(a, lds, blockIdx.x - a.max_tiles);
+        } else {
+            transr_thin_fwd_body<MODE>(a, lds, blockIdx.x - a.max_tiles);
+        }
+        return;
+    }
     const int tile = blockIdx.x;
     if (tile >= a.plan.num_tiles[0]) return;
     const int d = a.d;
@@ -141,6 +481,7 @@ __global__ __launch_bounds__(256, KGE_TR_OCC) void transr_gemm_kernel(GemmArgs a
     const int g = a.plan.tile_seg[tile], p0 = a.plan.tile_p0[tile];
     const int seg_end = a.seg_offsets[g + 1];
     const int rows = seg_end - p0 < kTM ? seg_end - p0 : kTM;
+    if (rows <= kThin) return;  // streamed by a thin workgroup
     const int64_t rid = a.unique_ids[g];
     const float *M = a.proj + rid * (int64_t)d * d;
 
@@ -192,7 +533,6 @@ __global__ __launch_bounds__(256, KGE_TR_OCC) void transr_gemm_kernel(GemmArgs a
 
     const int li = lane & 15, kk = lane >> 4;
     const bool two_blocks = rows > 16;
-    const bool tiny = rows <= 4;
     float rowsum[8];  // norm / dot partials for rows 4*kk + r (+16)
 #pragma unroll
     for (int r = 0; r < 8; ++r) rowsum[r] = 0.0f;
@@ -207,131 +547,10 @@ __global__ __launch_bounds__(256, KGE_TR_OCC) void transr_gemm_kernel(GemmArgs a
         for (int e = 0; e < 4; ++e) acc_lo[e] = floatx4{0.f, 0.f, 0.f, 0.f}, acc_hi[e] = floatx4{0.f, 0.f, 0.f, 0.f};
 
         if (wcols > 0) {
-            const int nq = kpad / 16;
-            if constexpr (MODE != 2) {
-                // B[k][j] = M[k][n0 + 4 li + e]: one float4 per (k) row per lane
-                const bool colok = 4 * li < wcols;
-                auto loadb = [&](int q, float4 *dst) {
-#pragma unroll
-                    for (int s = 0; s < 4; ++s) {
-                        const int k = 16 * q + 4 * kk + s;
-                        dst[s] = (colok && k < d) ? *reinterpret_cast<const float4 *>(M + (int64_t)k * d + n0 + 4 * li)
-                                                  : make_float4(0.f, 0.f, 0.f, 0.f);
-                    }
-                };
-                float4 ring[kRing][4];  // supersteps of B in flight
-#pragma unroll
-                for (int u = 0; u < kRing; ++u)
-                    if (u < nq) loadb(u, ring[u]);
-                for (int q = 0; q < nq; q += kRing) {
-#pragma unroll
-                    for (int u = 0; u < kRing; ++u) {
-                        if (q + u >= nq) break;
-                        float4 bc[4];
-#pragma unroll
-                        for (int s = 0; s < 4; ++s) bc[s] = ring[u][s];
-                        if (q + u + kRing < nq) loadb(q + u + kRing, ring[u]);
-                        const int qq = q + u;
-                        if (tiny) {
-                            // <= 4 triples: plain FMAs beat a 16-row MFMA block that is 3/4 padding.
-                            // Lane group kk covers its four k of the superstep; the groups are summed
-                            // after the loop.  acc_lo[e][r] = row r, column n0 + 4 li + e.
-#pragma unroll
-                            for (int r = 0; r < 4; ++r) {
-                                if (r >= rows) break;
-                                const float4 xr = *reinterpret_cast<const float4 *>(&sX[r * pitch + 16 * qq + 4 * kk]);
-                                const float xs4[4] = {xr.x, xr.y, xr.z, xr.w};
-#pragma unroll
-                                for (int s = 0; s < 4; ++s) {
-                                    acc_lo[0][r] = fmaf(xs4[s], bc[s].x, acc_lo[0][r]);
-                                    acc_lo[1][r] = fmaf(xs4[s], bc[s].y, acc_lo[1][r]);
-                                    acc_lo[2][r] = fmaf(xs4[s], bc[s].z, acc_lo[2][r]);
-                                    acc_lo[3][r] = fmaf(xs4[s], bc[s].w, acc_lo[3][r]);
-                                }
-                            }
-                            continue;
-                        }
-                        const float4 alo = *reinterpret_cast<const float4 *>(&sX[li * pitch + 16 * qq + 4 * kk]);
-                        const float4 ahi = *reinterpret_cast<const float4 *>(&sX[(16 + li) * pitch + 16 * qq + 4 * kk]);
-                        const float al[4] = {alo.x, alo.y, alo.z, alo.w}, ah[4] = {ahi.x, ahi.y, ahi.z, ahi.w};
-#pragma unroll
-                        for (int s = 0; s < 4; ++s) {
-                            const float bv[4] = {bc[s].x, bc[s].y, bc[s].z, bc[s].w};
-#pragma unroll
-                            for (int e = 0; e < 4; ++e) {
-                                acc_lo[e] = __builtin_amdgcn_mfma_f32_16x16x4f32(al[s], bv[e], acc_lo[e], 0, 0, 0);
-                                if (two_blocks)
-                                    acc_hi[e] = __builtin_amdgcn_mfma_f32_16x16x4f32(ah[s], bv[e], acc_hi[e], 0, 0, 0);
-                            }
-                        }
-                    }
-                }
-            } else {
-                // B[k][j] = M[j][k] (transposed): MFMA e owns output columns n0 + 16 e + li, and a
-                // lane's float4 along k of row (n0 + 16 e + li) serves the four steps
-                auto loadb = [&](int q, float4 *dst) {
-#pragma unroll
-                    for (int e = 0; e < 4; ++e) {
-                        const int col = 16 * e + li, k = 16 * q + 4 * kk;
-                        dst[e] = (col < wcols && k < d)
-                                     ? *reinterpret_cast<const float4 *>(M + (int64_t)(n0 + col) * d + k)
-                                     : make_float4(0.f, 0.f, 0.f, 0.f);
-                    }
-                };
-                float4 ring[kRing][4];
-#pragma unroll
-                for (int u = 0; u < kRing; ++u)
-                    if (u < nq) loadb(u, ring[u]);
-                for (int q = 0; q < nq; q += kRing) {
-#pragma unroll
-                    for (int u = 0; u < kRing; ++u) {
-                        if (q + u >= nq) break;
-                        float4 bc[4];
-#pragma unroll
-                        for (int e = 0; e < 4; ++e) bc[e] = ring[u][e];
-                        if (q + u + kRing < nq) loadb(q + u + kRing, ring[u]);
-                        const int qq = q + u;
-                        if (tiny) {  // acc_lo[e][r] = row r, column n0 + 16 e + li
-#pragma unroll
-                            for (int r = 0; r < 4; ++r) {
-                                if (r >= rows) break;
-                                const float4 xr = *reinterpret_cast<const float4 *>(&sX[r * pitch + 16 * qq + 4 * kk]);
-#pragma unroll
-                                for (int e = 0; e < 4; ++e)
-                                    acc_lo[e][r] = fmaf(xr.x, bc[e].x, fmaf(xr.y, bc[e].y,
-                                                   fmaf(xr.z, bc[e].z, fmaf(xr.w, bc[e].w, acc_lo[e][r]))));
-                            }
-                            continue;
-                        }
-                        const float4 alo = *reinterpret_cast<const float4 *>(&sX[li * pitch + 16 * qq + 4 * kk]);
-                        const float4 ahi = *reinterpret_cast<const float4 *>(&sX[(16 + li) * pitch + 16 * qq + 4 * kk]);
-                        const float al[4] = {alo.x, alo.y, alo.z, alo.w}, ah[4] = {ahi.x, ahi.y, ahi.z, ahi.w};
-#pragma unroll
-                        for (int e = 0; e < 4; ++e) {
-                            const float bv[4] = {bc[e].x, bc[e].y, bc[e].z, bc[e].w};
-#pragma unroll
-                            for (int s = 0; s < 4; ++s) {
-                                acc_lo[e] = __builtin_amdgcn_mfma_f32_16x16x4f32(al[s], bv[s], acc_lo[e], 0, 0, 0);
-                                if (two_blocks)
-                                    acc_hi[e] = __builtin_amdgcn_mfma_f32_16x16x4f32(ah[s], bv[s], acc_hi[e], 0, 0, 0);
-                            }
-                        }
-                    }
-                }
-            }
+            if (two_blocks) gemm_sweep<MODE, true>(M, sX, pitch, d, kpad / 16, n0, wcols, li, kk, acc_lo, acc_hi);
+            else gemm_sweep<MODE, false>(M, sX, pitch, d, kpad / 16, n0, wcols, li, kk, acc_lo, acc_hi);
         }
 
-        if (tiny) {  // sum the four k-slices; every lane group then holds rows 0..3 (group 0 writes)
-#pragma unroll
-            for (int e = 0; e < 4; ++e)
-#pragma unroll
-                for (int r = 0; r < 4; ++r) {
-                    float v = acc_lo[e][r];
-                    v += __shfl_xor(v, 16, kWave);
-                    v += __shfl_xor(v, 32, kWave);
-                    acc_lo[e][r] = v;
-                }
-        }
         // epilogue for this sweep: lane holds rows 4 kk + r (and +16), columns per the mode
 #pragma unroll
         for (int blk = 0; blk < 2; ++blk) {
@@ -397,10 +616,17 @@ __global__ __launch_bounds__(256, KGE_TR_OCC) void transr_gemm_kernel(GemmArgs a
     }
 }
 
-static size_t gemm_lds_bytes(int d)
+static size_t gemm_lds_bytes(int d)  // the larger of the tile layout and the thin layouts
 {
     const int kpad = (d + 15) & ~15;
-    return sizeof(float) * ((size_t)kTM * (kpad + 4) + 4 * kTM);
+    const size_t tile = sizeof(float) * ((size_t)kTM * (kpad + 4) + 4 * kTM);
+    const size_t thin = thin_fwd_lds_bytes(d) > thin_dx_lds_bytes(d) ? thin_fwd_lds_bytes(d) : thin_dx_lds_bytes(d);
+    return tile > thin ? tile : thin;
+}
+
+static int thin_groups(const kge_tables *tab, const kge_batch *bat)
+{
+    return (int)(bat->batch < tab->n_rel ? bat->batch : tab->n_rel);
 }
 
 static int64_t max_tiles(const kge_tables *tab, const kge_batch *bat)
@@ -471,7 +697,47 @@ struct DmArgs {
     float *dm;       // [U, d, d]
     float *part;     // [max_slots, d, d] partial results of split groups
     int d;
+    const int32_t *num_unique;
+    int max_items;   // leading workgroups: (tile, 32-row block) items; the rest: one thin group each
 };
+
+// dM of a group of at most kThin triples: four outer products written as one contiguous stream.
+// Thread (phase, cq) keeps its column quad of the Q rows in registers and walks the rows
+// k = phase, phase + P, ... of the output, so consecutive threads write consecutive 16 bytes.
+__device__ __forceinline__ void transr_thin_dm_body(const DmArgs &a, float *lds, int g)
+{
+    if (g >= a.num_unique[0]) return;
+    const int s0 = a.seg_offsets[g], rows = a.seg_offsets[g + 1] - s0;
+    if (rows > kThin) return;
+    const int d = a.d, nq4 = d >> 2, tid = threadIdx.x;
+    const int P = 256 / nq4;
+    float4 *sXT = reinterpret_cast<float4 *>(lds);  // [d] x[0..3][k]
+    for (int f = tid; f < 4 * nq4; f += 256) {
+        const int r = f / nq4, k4 = (f % nq4) * 4;
+        const float4 v = r < rows ? *reinterpret_cast<const float4 *>(a.xs + (int64_t)(s0 + r) * d + k4)
+                                  : make_float4(0.f, 0.f, 0.f, 0.f);
+        float *col = reinterpret_cast<float *>(sXT + k4) + r;
+        col[0] = v.x, col[4] = v.y, col[8] = v.z, col[12] = v.w;
+    }
+    const int cq = tid % nq4, ph = tid / nq4;
+    float4 q[4];
+#pragma unroll
+    for (int r = 0; r < 4; ++r)
+        q[r] = r < rows ? *reinterpret_cast<const float4 *>(a.qs + (int64_t)(s0 + r) * d + 4 * cq)
+                        : make_float4(0.f, 0.f, 0.f, 0.f);
+    __syncthreads();
+    if (ph >= P) return;
+    float4 *out = reinterpret_cast<float4 *>(a.dm + (int64_t)g * d * d);
+    for (int k = ph; k < d; k += P) {
+        const float4 x = sXT[k];
+        float4 o;
+        o.x = fmaf(x.w, q[3].x, fmaf(x.z, q[2].x, fmaf(x.y, q[1].x, x.x * q[0].x)));
+        o.y = fmaf(x.w, q[3].y, fmaf(x.z, q[2].y, fmaf(x.y, q[1].y, x.x * q[0].y)));
+        o.z = fmaf(x.w, q[3].z, fmaf(x.z, q[2].z, fmaf(x.y, q[1].z, x.x * q[0].z)));
+        o.w = fmaf(x.w, q[3].w, fmaf(x.z, q[2].w, fmaf(x.y, q[1].w, x.x * q[0].w)));
+        out[(int64_t)k * nq4 + cq] = o;
+    }
+}
 
 // dM[g][i][j] = sum_{p in group g} xs[p][i] * qs[p][j].  A work item is (chunk of <= 256 triples
 // of one group, 32 rows i); the four waves split the columns j; K runs over the chunk's triples,
@@ -479,6 +745,11 @@ struct DmArgs {
 // partial matrices that transr_dm_finish_kernel adds up (keeps the longest K loop at 16 supersteps).
 __global__ __launch_bounds__(256, KGE_TR_OCC) void transr_dm_kernel(DmArgs a)
 {
+    extern __shared__ __align__(16) float lds[];  // thin groups only: d float4
+    if ((int)blockIdx.x >= a.max_items) {
+        transr_thin_dm_body(a, lds, blockIdx.x - a.max_items);
+        return;
+    }
     const int d = a.d;
     const int nib = (d + 31) / 32;
     const int tile = blockIdx.x / nib;
@@ -487,6 +758,7 @@ __global__ __launch_bounds__(256, KGE_TR_OCC) void transr_dm_kernel(DmArgs a)
     const int g = a.plan.tile_seg[tile];
     const int s0 = a.plan.tile_p0[tile];
     const int seg_end = a.seg_offsets[g + 1];
+    if (seg_end - a.seg_offsets[g] <= kThin) return;  // written by a thin workgroup
     const int s1 = s0 + kDmChunk < seg_end ? s0 + kDmChunk : seg_end;
     const int slot = a.plan.tile_part[tile];
     float *dst = slot >= 0 ? a.part + (int64_t)slot * d * d : a.dm + (int64_t)g * d * d;
@@ -523,16 +795,16 @@ __global__ __launch_bounds__(256, KGE_TR_OCC) void transr_dm_kernel(DmArgs a)
                                          : make_float4(0.f, 0.f, 0.f, 0.f);
             }
         };
-        Stage ring[kRing];
+        Stage ring[kDmRing];
 #pragma unroll
-        for (int u = 0; u < kRing; ++u)
+        for (int u = 0; u < kDmRing; ++u)
             if (u < nq) load_stage(u, ring[u]);
-        for (int q = 0; q < nq; q += kRing) {
+        for (int q = 0; q < nq; q += kDmRing) {
 #pragma unroll
-            for (int u = 0; u < kRing; ++u) {
+            for (int u = 0; u < kDmRing; ++u) {
                 if (q + u >= nq) break;
                 const Stage cur = ring[u];
-                if (q + u + kRing < nq) load_stage(q + u + kRing, ring[u]);
+                if (q + u + kDmRing < nq) load_stage(q + u + kDmRing, ring[u]);
 #pragma unroll
                 for (int s = 0; s < 4; ++s) {
                     const float b4[4] = {cur.bv[s].x, cur.bv[s].y, cur.bv[s].z, cur.bv[s].w};
@@ -642,13 +914,14 @@ int launch_transr_fwd(const kge_tables *tab, const kge_batch *bat, float *pos, f
     const int64_t tiles = max_tiles(tab, bat);
     TilePlan plan = plan_at(workspace, tiles, 0);
     hipLaunchKernelGGL(transr_plan_kernel, dim3(1), dim3(1024), 0, st, ri->num_unique, ri->seg_offsets, plan, kTM);
-    GemmArgs a{tab->ent, tab->rel, tab->aux, bat->h, bat->r, bat->t, ri->perm, ri->seg_offsets, ri->unique_ids,
-               plan, nullptr, pos, resid, nullptr, nullptr, (int)tab->dim, tab->norm_p};
+    GemmArgs a{tab->ent, tab->rel, tab->aux, bat->h, bat->r, bat->t, ri->perm, ri->seg_offsets, ri->num_unique, ri->unique_ids,
+               plan, nullptr, pos, resid, nullptr, nullptr, (int)tab->dim, tab->norm_p, thin_groups(tab, bat), (int)tiles};
     const size_t lds = gemm_lds_bytes((int)tab->dim);
+    const dim3 grid((unsigned)(tiles + a.thin_groups));
     if (rescal)
-        hipLaunchKernelGGL(transr_gemm_kernel<1>, dim3((unsigned)tiles), dim3(256), lds, st, a);
+        hipLaunchKernelGGL(transr_gemm_kernel<1>, grid, dim3(256), lds, st, a);
     else
-        hipLaunchKernelGGL(transr_gemm_kernel<0>, dim3((unsigned)tiles), dim3(256), lds, st, a);
+        hipLaunchKernelGGL(transr_gemm_kernel<0>, grid, dim3(256), lds, st, a);
     KGE_CHECK_LAUNCH();
     return KGE_OK;
 }
@@ -682,12 +955,16 @@ int launch_transr_bwd(const kge_tables *tab, const kge_batch *bat, const kge_sav
     hipLaunchKernelGGL(transr_plan_kernel, dim3(1), dim3(1024), 0, st, ri->num_unique, ri->seg_offsets, dplan,
                        kDmChunk);
     // dX = Q M^T -> occurrence rows of h (and -dX for t)
-    GemmArgs ga{tab->ent, tab->rel, tab->aux, bat->h, bat->r, bat->t, ri->perm, ri->seg_offsets, ri->unique_ids,
-                plan, qs, nullptr, nullptr, occ, rescal ? nullptr : occ + B * d, d, tab->norm_p};
-    hipLaunchKernelGGL(transr_gemm_kernel<2>, dim3((unsigned)p.tiles), dim3(256), gemm_lds_bytes(d), st, ga);
+    GemmArgs ga{tab->ent, tab->rel, tab->aux, bat->h, bat->r, bat->t, ri->perm, ri->seg_offsets, ri->num_unique, ri->unique_ids,
+                plan, qs, nullptr, nullptr, occ, rescal ? nullptr : occ + B * d, d, tab->norm_p, thin_groups(tab, bat), (int)p.tiles};
+    hipLaunchKernelGGL(transr_gemm_kernel<2>, dim3((unsigned)(p.tiles + ga.thin_groups)), dim3(256), gemm_lds_bytes(d),
+                       st, ga);
     // dM = X^T Q per relation group
-    DmArgs da{xs, qs, ri->seg_offsets, dplan, grads->aux_rows, reinterpret_cast<float *>(ws + p.off_dpart), d};
-    hipLaunchKernelGGL(transr_dm_kernel, dim3((unsigned)(ceil_div(d, 32) * p.dtiles)), dim3(256), 0, st, da);
+    const int dm_items = (int)(ceil_div(d, 32) * p.dtiles);
+    DmArgs da{xs, qs, ri->seg_offsets, dplan, grads->aux_rows, reinterpret_cast<float *>(ws + p.off_dpart), d,
+              ri->num_unique, dm_items};
+    hipLaunchKernelGGL(transr_dm_kernel, dim3((unsigned)(dm_items + thin_groups(tab, bat))), dim3(256),
+                       sizeof(float) * 4 * (size_t)d, st, da);
     hipLaunchKernelGGL(transr_dm_finish_kernel, dim3((unsigned)ceil_div((int64_t)d * d / 4, 256), (unsigned)p.dsplit),
                        dim3(256), 0, st, da);
     KGE_CHECK_LAUNCH();
