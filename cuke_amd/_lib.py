@@ -42,7 +42,7 @@ class Batch(C.Structure):
     _fields_ = [("batch", C.c_int64), ("h", C.c_void_p), ("r", C.c_void_p), ("t", C.c_void_p),
                 ("neg", C.c_void_p), ("chunk", C.c_int64), ("n_neg", C.c_int64),
                 ("ent_insp", C.POINTER(Inspection)), ("rel_insp", C.POINTER(Inspection)),
-                ("insp_ready", C.c_void_p)]
+                ("insp_ready", C.c_void_p), ("neg_mode", C.c_int32), ("reserved", C.c_int32)]
 
 
 class Saved(C.Structure):

@@ -18,7 +18,8 @@ __global__ void check_indices_kernel(const int64_t *idx, int64_t n, int64_t n_ro
 }
 
 __global__ void flatten_negatives_kernel(const int64_t *h, const int64_t *r, const int64_t *t, const int64_t *neg,
-                                         int64_t B, int64_t C, int64_t N, int64_t *hf, int64_t *rf, int64_t *tf)
+                                         int64_t B, int64_t C, int64_t N, int head, int64_t *hf, int64_t *rf,
+                                         int64_t *tf)
 {
     const int64_t total = B * (1 + N);
     for (int64_t p = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; p < total; p += (int64_t)gridDim.x * blockDim.x) {
@@ -26,7 +27,8 @@ __global__ void flatten_negatives_kernel(const int64_t *h, const int64_t *r, con
             hf[p] = h[p], rf[p] = r[p], tf[p] = t[p];
         } else {
             const int64_t q = p - B, b = q / N, k = q % N;
-            hf[p] = h[b], rf[p] = r[b], tf[p] = neg[(b / C) * N + k];
+            const int64_t e = neg[(b / C) * N + k];
+            hf[p] = head ? e : h[b], rf[p] = r[b], tf[p] = head ? t[b] : e;
         }
     }
 }
@@ -71,6 +73,7 @@ static int validate_batch(const kge_batch *bat)
     if (bat->neg) {
         if (bat->chunk <= 0 || bat->n_neg <= 0) return KGE_ESHAPE;
         if (bat->batch % bat->chunk != 0) return KGE_ESHAPE;
+        if (bat->neg_mode != KGE_NEG_TAIL && bat->neg_mode != KGE_NEG_HEAD) return KGE_EINVAL;
     }
     return KGE_OK;
 }
@@ -93,7 +96,7 @@ const char *kge_strerror(int status)
     }
 }
 
-int kge_abi_version(void) { return 1; }
+int kge_abi_version(void) { return 2; }
 
 size_t kge_score_fwd_workspace(const kge_tables *tab, const kge_batch *bat)
 {
@@ -151,7 +154,7 @@ int kge_flatten_negatives(const kge_batch *bat, int64_t *h_flat, int64_t *r_flat
     const int64_t blocks = ceil_div(total, 256);
     hipLaunchKernelGGL(flatten_negatives_kernel, dim3((unsigned)(blocks < 4096 ? blocks : 4096)), dim3(256), 0,
                        as_stream(stream), bat->h, bat->r, bat->t, bat->neg, bat->batch, bat->chunk, bat->n_neg,
-                       h_flat, r_flat, t_flat);
+                       bat->neg_mode == KGE_NEG_HEAD ? 1 : 0, h_flat, r_flat, t_flat);
     KGE_CHECK_LAUNCH();
     return KGE_OK;
 }

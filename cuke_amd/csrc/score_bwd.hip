@@ -36,6 +36,7 @@ struct TileArgs {
     float *out0, *out1;
     int64_t plane;  // B * N
     int C, N, d, rel_dim, vec, vecn, n_chunks;
+    float rsign;    // +1: negatives replace the tail; -1: the head (h then holds the tails; see load_query)
 };
 
 constexpr int kTI = 64;       // columns of the row per workgroup
@@ -99,7 +100,7 @@ __device__ __forceinline__ void bwd_tile_body(const TileArgs &a, int lid, float 
             if constexpr (!kDot)
                 load_query<MODEL, VEC>(a.ent + a.h[b] * (int64_t)d, a.rel + rid * (int64_t)a.rel_dim,
                                   kTH ? a.aux + rid * (int64_t)d : nullptr, alo[o], col, lim, half, q0,
-                                  q1, kRot ? a.query + b * (int64_t)d : nullptr);
+                                  q1, kRot ? a.query + b * (int64_t)d : nullptr, a.rsign);
             own[0][o] = q0;
             if constexpr (NPO == 2) own[1][o] = q1;
         } else {
@@ -140,7 +141,7 @@ __device__ __forceinline__ void bwd_tile_body(const TileArgs &a, int lid, float 
                 float4 q0, q1;
                 load_query<MODEL, VEC>(a.ent + a.h[b] * (int64_t)d, a.rel + rid * (int64_t)a.rel_dim,
                                   kTH ? a.aux + rid * (int64_t)d : nullptr, kTH ? a.side_pos[b] : 0.0f, col,
-                                  lim, half, q0, q1, kRot ? a.query + b * (int64_t)d : nullptr);
+                                  lim, half, q0, q1, kRot ? a.query + b * (int64_t)d : nullptr, a.rsign);
                 rl[0][s] = q0;
                 if constexpr (NPL == 2) rl[1][s] = q1;
             }
@@ -370,7 +371,11 @@ __device__ __forceinline__ Vec<V> ldz(const float *p, int j)
     return z;
 }
 
-template <int MODEL, int P, int V>
+// G (g0) is the gradient with respect to the query row a_b accumulated over the chunk's negatives.
+// With negatives that replace the tail the query is built from (h, r); with HEAD it is built from
+// (x, rho) = (t, -r) [TransE, TransH], (t, conj r) [ComplEx], (t, -theta) [RotatE], (t, r) [DistMult],
+// so G chains into the t and r rows instead and the positive triple's own term is kept apart.
+template <int MODEL, int P, int V, bool HEAD>
 __global__ __launch_bounds__(256) void bwd_pos_kernel(PosBwdArgs a)
 {
     const int lane = threadIdx.x & (kWave - 1);
@@ -400,10 +405,18 @@ __global__ __launch_bounds__(256) void bwd_pos_kernel(PosBwdArgs a)
             for (int e = 0; e < V; ++e) {
                 const float u = (vh.v[e] - vt.v[e]) + vr.v[e];
                 const float q = gs * (P == 1 ? sgn(u) : u);
-                dh.v[e] = q + G.v[e];
-                dt.v[e] = -q;
+                dh.v[e] = HEAD ? q : q + G.v[e];
+                dt.v[e] = HEAD ? G.v[e] - q : -q;
             }
-            dh.store(oh + j), dh.store(orr + j), dt.store(ot + j);
+            if constexpr (HEAD) {
+                Vec<V> dr;
+#pragma unroll
+                for (int e = 0; e < V; ++e) dr.v[e] = dh.v[e] - G.v[e];
+                dr.store(orr + j);
+            } else {
+                dh.store(orr + j);
+            }
+            dh.store(oh + j), dt.store(ot + j);
         }
     } else if constexpr (MODEL == KGE_DISTMULT) {
         for (int j = lane * V; j < d; j += kWave * V) {
@@ -412,10 +425,17 @@ __global__ __launch_bounds__(256) void bwd_pos_kernel(PosBwdArgs a)
             Vec<V> dh, dr, dt;
 #pragma unroll
             for (int e = 0; e < V; ++e) {
-                const float Q = fmaf(g, vt.v[e], G.v[e]);
-                dh.v[e] = vr.v[e] * Q;
-                dr.v[e] = vh.v[e] * Q;
-                dt.v[e] = g * (vh.v[e] * vr.v[e]);
+                if constexpr (HEAD) {  // a = t * r
+                    const float Q = fmaf(g, vh.v[e], G.v[e]);
+                    dt.v[e] = vr.v[e] * Q;
+                    dr.v[e] = vt.v[e] * Q;
+                    dh.v[e] = g * (vt.v[e] * vr.v[e]);
+                } else {
+                    const float Q = fmaf(g, vt.v[e], G.v[e]);
+                    dh.v[e] = vr.v[e] * Q;
+                    dr.v[e] = vh.v[e] * Q;
+                    dt.v[e] = g * (vh.v[e] * vr.v[e]);
+                }
             }
             dh.store(oh + j), dr.store(orr + j), dt.store(ot + j);
         }
@@ -440,13 +460,24 @@ __global__ __launch_bounds__(256) void bwd_pos_kernel(PosBwdArgs a)
             Vec<V> dhr, dhi, drr, dri, dtr, dti;
 #pragma unroll
             for (int e = 0; e < V; ++e) {
-                const float Qr = fmaf(g, tr.v[e], Gr.v[e]), Qi = fmaf(g, ti.v[e], Gi.v[e]);
-                dhr.v[e] = Qr * qr.v[e] + Qi * qi.v[e];
-                dhi.v[e] = Qi * qr.v[e] - Qr * qi.v[e];
-                drr.v[e] = Qr * hr.v[e] + Qi * hi.v[e];
-                dri.v[e] = Qi * hr.v[e] - Qr * hi.v[e];
-                dtr.v[e] = g * (hr.v[e] * qr.v[e] - hi.v[e] * qi.v[e]);
-                dti.v[e] = g * (hr.v[e] * qi.v[e] + hi.v[e] * qr.v[e]);
+                if constexpr (HEAD) {
+                    // s = Re<n, r, conj t> = n . (conj(r) o t): a = conj(r) o t, Q = g h + G
+                    const float Qr = fmaf(g, hr.v[e], Gr.v[e]), Qi = fmaf(g, hi.v[e], Gi.v[e]);
+                    dtr.v[e] = Qr * qr.v[e] - Qi * qi.v[e];
+                    dti.v[e] = Qi * qr.v[e] + Qr * qi.v[e];
+                    drr.v[e] = Qr * tr.v[e] + Qi * ti.v[e];
+                    dri.v[e] = Qr * ti.v[e] - Qi * tr.v[e];
+                    dhr.v[e] = g * (qr.v[e] * tr.v[e] + qi.v[e] * ti.v[e]);
+                    dhi.v[e] = g * (qr.v[e] * ti.v[e] - qi.v[e] * tr.v[e]);
+                } else {
+                    const float Qr = fmaf(g, tr.v[e], Gr.v[e]), Qi = fmaf(g, ti.v[e], Gi.v[e]);
+                    dhr.v[e] = Qr * qr.v[e] + Qi * qi.v[e];
+                    dhi.v[e] = Qi * qr.v[e] - Qr * qi.v[e];
+                    drr.v[e] = Qr * hr.v[e] + Qi * hi.v[e];
+                    dri.v[e] = Qi * hr.v[e] - Qr * hi.v[e];
+                    dtr.v[e] = g * (hr.v[e] * qr.v[e] - hi.v[e] * qi.v[e]);
+                    dti.v[e] = g * (hr.v[e] * qi.v[e] + hi.v[e] * qr.v[e]);
+                }
             }
             dhr.store(oh + j), dhi.store(oh + half + j);
             drr.store(orr + j), dri.store(orr + half + j);
@@ -468,12 +499,22 @@ __global__ __launch_bounds__(256) void bwd_pos_kernel(PosBwdArgs a)
                 const float m = sqrtf(ur * ur + ui * ui);
                 const float k = m > 0.0f ? -g / m : 0.0f;  // s = gamma - sum m
                 const float qpr = k * ur, qpi = k * ui;
-                const float Qr = qpr + Gr.v[e], Qi = qpi + Gi.v[e];
-                dhr.v[e] = Qr * cs + Qi * sn;
-                dhi.v[e] = Qi * cs - Qr * sn;
-                dth.v[e] = Qi * ar - Qr * ai;
-                dtr.v[e] = -qpr;
-                dti.v[e] = -qpi;
+                if constexpr (HEAD) {
+                    // negatives: a' = t e^{-i theta}, G = dL/da'; positive term as in the tail form
+                    const float br = tr.v[e] * cs + ti.v[e] * sn, bi = ti.v[e] * cs - tr.v[e] * sn;
+                    dhr.v[e] = qpr * cs + qpi * sn;
+                    dhi.v[e] = qpi * cs - qpr * sn;
+                    dtr.v[e] = (Gr.v[e] * cs - Gi.v[e] * sn) - qpr;
+                    dti.v[e] = (Gi.v[e] * cs + Gr.v[e] * sn) - qpi;
+                    dth.v[e] = (qpi * ar - qpr * ai) - (Gi.v[e] * br - Gr.v[e] * bi);
+                } else {
+                    const float Qr = qpr + Gr.v[e], Qi = qpi + Gi.v[e];
+                    dhr.v[e] = Qr * cs + Qi * sn;
+                    dhi.v[e] = Qi * cs - Qr * sn;
+                    dth.v[e] = Qi * ar - Qr * ai;
+                    dtr.v[e] = -qpr;
+                    dti.v[e] = -qpi;
+                }
             }
             dhr.store(oh + j), dhi.store(oh + half + j);
             dth.store(orr + j);
@@ -514,11 +555,18 @@ __global__ __launch_bounds__(256) void bwd_pos_kernel(PosBwdArgs a)
                 const float d0 = vh.v[e] - vt.v[e];
                 const float u = (d0 + vr.v[e]) - sd * vw.v[e];
                 const float q = gs * (P == 1 ? sgn(u) : u);
-                const float Q = q + G.v[e];
-                dr.v[e] = Q;
-                dh.v[e] = Q - (qw + gw) * vw.v[e];
-                dt.v[e] = -(q - qw * vw.v[e]);
-                dw.v[e] = Gw.v[e] - (qw * d0 + sd * q) - gw * vh.v[e];
+                if constexpr (HEAD) {  // G chains through a = t - r - (w.t) w
+                    dr.v[e] = q - G.v[e];
+                    dh.v[e] = q - qw * vw.v[e];
+                    dt.v[e] = (G.v[e] - gw * vw.v[e]) - (q - qw * vw.v[e]);
+                    dw.v[e] = Gw.v[e] - (qw * d0 + sd * q) - gw * vt.v[e];
+                } else {
+                    const float Q = q + G.v[e];
+                    dr.v[e] = Q;
+                    dh.v[e] = Q - (qw + gw) * vw.v[e];
+                    dt.v[e] = -(q - qw * vw.v[e]);
+                    dw.v[e] = Gw.v[e] - (qw * d0 + sd * q) - gw * vh.v[e];
+                }
             }
             dh.store(oh + j), dt.store(ot + j), dr.store(orr + j), dw.store(ow + j);
         }
@@ -526,11 +574,16 @@ __global__ __launch_bounds__(256) void bwd_pos_kernel(PosBwdArgs a)
 }
 
 template <int MODEL, int P>
-static int launch_pos_bwd(const PosBwdArgs &a, bool vec4, hipStream_t st)
+static int launch_pos_bwd(const PosBwdArgs &a, bool vec4, bool head, hipStream_t st)
 {
     const dim3 grid((unsigned)ceil_div(a.B, 4)), block(256);
-    if (vec4) hipLaunchKernelGGL((bwd_pos_kernel<MODEL, P, 4>), grid, block, 0, st, a);
-    else hipLaunchKernelGGL((bwd_pos_kernel<MODEL, P, 1>), grid, block, 0, st, a);
+    if (head) {
+        if (vec4) hipLaunchKernelGGL((bwd_pos_kernel<MODEL, P, 4, true>), grid, block, 0, st, a);
+        else hipLaunchKernelGGL((bwd_pos_kernel<MODEL, P, 1, true>), grid, block, 0, st, a);
+    } else {
+        if (vec4) hipLaunchKernelGGL((bwd_pos_kernel<MODEL, P, 4, false>), grid, block, 0, st, a);
+        else hipLaunchKernelGGL((bwd_pos_kernel<MODEL, P, 1, false>), grid, block, 0, st, a);
+    }
     KGE_CHECK_LAUNCH();
     return KGE_OK;
 }
@@ -613,6 +666,8 @@ int kge_score_bwd(const kge_tables *tab, const kge_batch *bat, const kge_saved *
     if (tab->rel_dim > 0 && !grads->rel_rows) return KGE_EINVAL;
     if (normed && P == 2 && dpos && !saved->pos) return KGE_EINVAL;
     const bool have_neg = bat->neg && dneg;
+    if (bat->neg && bat->neg_mode != KGE_NEG_TAIL && bat->neg_mode != KGE_NEG_HEAD) return KGE_EINVAL;
+    const bool head = have_neg && bat->neg_mode == KGE_NEG_HEAD;
     if (have_neg) {
         if (model == KGE_TRANSF) return KGE_EUNSUPPORTED;
         if (normed && P == 2 && !saved->neg) return KGE_EINVAL;
@@ -636,9 +691,10 @@ int kge_score_bwd(const kge_tables *tab, const kge_batch *bat, const kge_saved *
         if (n_chunks >= (1 << 24)) return KGE_ESHAPE;
         const bool vecn = bat->n_neg % 4 == 0 && aligned16(dneg) && (!saved->neg || aligned16(saved->neg)) &&
                           (!saved->side_neg || aligned16(saved->side_neg));
-        TileArgs a{tab->ent, tab->rel, tab->aux, bat->h, bat->r, bat->neg, dneg, saved->neg, saved->side_pos,
-                   saved->side_neg, model == KGE_ROTATE ? saved->residual : nullptr, nullptr, nullptr, B * bat->n_neg, (int)bat->chunk, (int)bat->n_neg, (int)d,
-                   (int)tab->rel_dim, vec ? 1 : 0, vecn ? 1 : 0, (int)n_chunks};
+        TileArgs a{tab->ent, tab->rel, tab->aux, head ? bat->t : bat->h, bat->r, bat->neg, dneg, saved->neg,
+                   saved->side_pos, saved->side_neg, model == KGE_ROTATE ? saved->residual : nullptr, nullptr, nullptr,
+                   B * bat->n_neg, (int)bat->chunk, (int)bat->n_neg, (int)d, (int)tab->rel_dim, vec ? 1 : 0,
+                   vecn ? 1 : 0, (int)n_chunks, head ? -1.0f : 1.0f};
         float *occ_neg = occ_e + 2 * B * d;
         switch (model) {
         case KGE_TRANSE:
@@ -663,15 +719,15 @@ int kge_score_bwd(const kge_tables *tab, const kge_batch *bat, const kge_saved *
                   g0, g1, occ_e, occ_e + B * d, occ_r, occ_w, B, (int)d, (int)tab->rel_dim};
     switch (model) {
     case KGE_TRANSE:
-        rc = P == 1 ? launch_pos_bwd<KGE_TRANSE, 1>(pa, vec, st) : launch_pos_bwd<KGE_TRANSE, 2>(pa, vec, st);
+        rc = P == 1 ? launch_pos_bwd<KGE_TRANSE, 1>(pa, vec, head, st) : launch_pos_bwd<KGE_TRANSE, 2>(pa, vec, head, st);
         break;
     case KGE_TRANSH:
-        rc = P == 1 ? launch_pos_bwd<KGE_TRANSH, 1>(pa, vec, st) : launch_pos_bwd<KGE_TRANSH, 2>(pa, vec, st);
+        rc = P == 1 ? launch_pos_bwd<KGE_TRANSH, 1>(pa, vec, head, st) : launch_pos_bwd<KGE_TRANSH, 2>(pa, vec, head, st);
         break;
-    case KGE_DISTMULT: rc = launch_pos_bwd<KGE_DISTMULT, 2>(pa, vec, st); break;
-    case KGE_COMPLEX: rc = launch_pos_bwd<KGE_COMPLEX, 2>(pa, vec, st); break;
-    case KGE_ROTATE: rc = launch_pos_bwd<KGE_ROTATE, 2>(pa, vec, st); break;
-    case KGE_TRANSF: rc = launch_pos_bwd<KGE_TRANSF, 2>(pa, vec, st); break;
+    case KGE_DISTMULT: rc = launch_pos_bwd<KGE_DISTMULT, 2>(pa, vec, head, st); break;
+    case KGE_COMPLEX: rc = launch_pos_bwd<KGE_COMPLEX, 2>(pa, vec, head, st); break;
+    case KGE_ROTATE: rc = launch_pos_bwd<KGE_ROTATE, 2>(pa, vec, head, st); break;
+    case KGE_TRANSF: rc = launch_pos_bwd<KGE_TRANSF, 2>(pa, vec, head, st); break;
     default: return KGE_EUNSUPPORTED;
     }
     if (rc) return rc;

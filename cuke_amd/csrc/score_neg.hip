@@ -18,7 +18,7 @@ namespace kge {
 
 struct NegArgs {
     const float *ent, *rel, *aux;
-    const int64_t *h, *r, *neg;
+    const int64_t *h, *r, *neg;  // h: the side of the positive that is kept (tails with head negatives)
     const float *side_pos;  // TransH: w_b . h_b
     const float *query;     // RotatE: rotated heads [B, d] from the positive kernel (required)
     float *out;             // [B, N]
@@ -29,6 +29,7 @@ struct NegArgs {
     int C, N, d, rel_dim;
     float gamma;
     int vec, n_chunks;
+    float rsign;            // +1: negatives replace the tail; -1: the head (see load_query)
 };
 
 constexpr int kKD = 32;        // floats of each row staged per step
@@ -114,7 +115,7 @@ __global__ __launch_bounds__(256, KGE_TILE_OCC) void score_neg_kernel(NegArgs a)
         for (int s = 0; s < SB; ++s) {
             const int lim = okb[s] ? klen : 0;
             float4 q0, q1;
-            load_query<MODEL, VEC>(ph[s], pr[s], pw[s], pa[s], j, lim, half, q0, q1, pq[s]);
+            load_query<MODEL, VEC>(ph[s], pr[s], pw[s], pa[s], j, lim, half, q0, q1, pq[s], a.rsign);
             ra[0][s] = q0;
             if constexpr (NPA == 2) ra[1][s] = q1;
         }
@@ -254,8 +255,10 @@ int launch_score_neg(const kge_tables *tab, const kge_batch *bat, const float *s
     const int64_t n_chunks = bat->batch / bat->chunk;
     if (n_chunks >= (1 << 24) || bat->chunk >= (1 << 30) || bat->n_neg >= (1 << 30)) return KGE_ESHAPE;
     const bool vec = rows_vectorizable(tab);
-    NegArgs a{tab->ent, tab->rel, tab->aux, bat->h, bat->r, bat->neg, side_pos, query, out, side_neg,
-              bat->batch * bat->n_neg, (int)bat->chunk, (int)bat->n_neg, (int)tab->dim, (int)tab->rel_dim, tab->gamma, vec ? 1 : 0, (int)n_chunks};
+    const bool head = bat->neg_mode == KGE_NEG_HEAD;
+    NegArgs a{tab->ent, tab->rel, tab->aux, head ? bat->t : bat->h, bat->r, bat->neg, side_pos, query, out, side_neg,
+              bat->batch * bat->n_neg, (int)bat->chunk, (int)bat->n_neg, (int)tab->dim, (int)tab->rel_dim, tab->gamma,
+              vec ? 1 : 0, (int)n_chunks, head ? -1.0f : 1.0f};
     const int p = tab->norm_p;
     switch (tab->model) {
     case KGE_TRANSE:

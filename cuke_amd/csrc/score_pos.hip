@@ -17,6 +17,7 @@ struct PosArgs {
     float *resid;     // [B, d] or nullptr: residual rows (TransE / TransH / TransR), the projected heads
                       // E[h] Proj[r] (RESCAL) or, for RotatE, the rotated heads h e^{i theta} laid out [re | im]
     float *side_pos;  // [B] TransH: w.h (used by the shared-negative kernels)
+    int head;         // negatives replace the head: side_pos = w.t, RotatE resid = t e^{-i theta}
 };
 
 constexpr int kPosWaves = 4;
@@ -65,7 +66,7 @@ __global__ __launch_bounds__(kPosWaves *kWave) void score_pos_kernel(PosArgs a)
 #pragma unroll
             for (int e = 0; e < V; ++e) {
                 sd += vw.v[e] * (vh.v[e] - vt.v[e]);
-                wh += vw.v[e] * vh.v[e];
+                wh += vw.v[e] * (a.head ? vt.v[e] : vh.v[e]);
             }
         }
         sd = wave_sum(sd);
@@ -158,8 +159,12 @@ __global__ __launch_bounds__(kPosWaves *kWave) void score_pos_kernel(PosArgs a)
                 ai.v[e] = hr.v[e] * sn + hi.v[e] * c;
                 const float ur = ar.v[e] - tr.v[e], ui = ai.v[e] - ti.v[e];
                 acc += sqrtf(ur * ur + ui * ui);
+                if (a.head) {  // the kept side is the tail: t e^{-i theta}
+                    ar.v[e] = tr.v[e] * c + ti.v[e] * sn;
+                    ai.v[e] = ti.v[e] * c - tr.v[e] * sn;
+                }
             }
-            if (out && valid) ar.store(out + j), ai.store(out + half + j);  // rotated head, reused downstream
+            if (out && valid) ar.store(out + j), ai.store(out + half + j);  // rotated row, reused downstream
         }
     }
 
@@ -194,7 +199,8 @@ int launch_score_pos(const kge_tables *tab, const kge_batch *bat, float *pos, fl
 {
     if (bat->batch == 0) return KGE_OK;
     PosArgs a{tab->ent, tab->rel,      tab->aux,          bat->h,     bat->r, bat->t, bat->batch,
-              (int)tab->dim, (int)tab->rel_dim, tab->gamma, pos, resid, side_pos};
+              (int)tab->dim, (int)tab->rel_dim, tab->gamma, pos, resid, side_pos,
+              (bat->neg && bat->neg_mode == KGE_NEG_HEAD) ? 1 : 0};
     const bool complex_rows = tab->model == KGE_COMPLEX || tab->model == KGE_ROTATE;
     const bool vec4 = tab->dim % (complex_rows ? 8 : 4) == 0 && aligned16(tab->ent) &&
                       (!tab->rel || aligned16(tab->rel)) && (!tab->aux || aligned16(tab->aux)) &&

@@ -75,16 +75,23 @@ __device__ __forceinline__ int pair_len(int d)
 //   TransH    q0 = h + r - al*w (al = w.h), q1 = w
 // lim == 0 yields zeros (row outside the tile).
 // RotatE takes its query rows from pq, the [B, d] buffer of rotated heads.
+//
+// Negatives that replace the HEAD use the same pair kernels: score(n, r, t) is the tail-mode
+// function of (x, rho, n) with x = t and rho = -r (TransE, TransH), conj(r) (ComplEx), -theta
+// (RotatE, already applied in pq) or r (DistMult).  The caller passes the tail row as `ph` and
+// rs = -1; rs multiplies r (its imaginary half for ComplEx), which is exact, so rs = +1
+// reproduces the tail-mode arithmetic bit for bit.
 template <int MODEL, bool VEC>
 __device__ __forceinline__ void load_query(const float *ph, const float *pr, const float *pw, float al,
                                            int j, int lim, int half, float4 &q0, float4 &q1,
-                                           const float *pq = nullptr)
+                                           const float *pq = nullptr, float rs = 1.0f)
 {
     q1 = zero4();
     if constexpr (MODEL == KGE_DISTMULT) {
         q0 = mul4(ld4<VEC>(ph, j, lim), ld4<VEC>(pr, j, lim));
     } else if constexpr (MODEL == KGE_TRANSE) {
-        q0 = add4(ld4<VEC>(ph, j, lim), ld4<VEC>(pr, j, lim));
+        const float4 vh = ld4<VEC>(ph, j, lim), vr = ld4<VEC>(pr, j, lim);
+        q0 = make_float4(fmaf(rs, vr.x, vh.x), fmaf(rs, vr.y, vh.y), fmaf(rs, vr.z, vh.z), fmaf(rs, vr.w, vh.w));
     } else if constexpr (MODEL == KGE_COMPLEX) {
         float q[4];
         if constexpr (VEC) {  // half % 4 == 0: the four elements sit on one side of the re|im split
@@ -92,7 +99,9 @@ __device__ __forceinline__ void load_query(const float *ph, const float *pr, con
             const int i = re ? j : j - half;
             const int l2 = lim ? half : 0;
             const float4 hr = ld4<true>(ph, i, l2), hi = ld4<true>(ph + half, i, l2);
-            const float4 rr = ld4<true>(pr, i, l2), ri = ld4<true>(pr + half, i, l2);
+            const float4 rr = ld4<true>(pr, i, l2);
+            float4 ri = ld4<true>(pr + half, i, l2);
+            ri = make_float4(rs * ri.x, rs * ri.y, rs * ri.z, rs * ri.w);
             q[0] = re ? hr.x * rr.x - hi.x * ri.x : hr.x * ri.x + hi.x * rr.x;
             q[1] = re ? hr.y * rr.y - hi.y * ri.y : hr.y * ri.y + hi.y * rr.y;
             q[2] = re ? hr.z * rr.z - hi.z * ri.z : hr.z * ri.z + hi.z * rr.z;
@@ -103,7 +112,7 @@ __device__ __forceinline__ void load_query(const float *ph, const float *pr, con
                 const int jj = j + e;
                 const bool ok = jj < lim;
                 const int i = ok ? (jj < half ? jj : jj - half) : 0;
-                const float hr = ph[i], hi = ph[i + half], rr = pr[i], ri = pr[i + half];
+                const float hr = ph[i], hi = ph[i + half], rr = pr[i], ri = rs * pr[i + half];
                 q[e] = ok ? (jj < half ? hr * rr - hi * ri : hr * ri + hi * rr) : 0.0f;
             }
         }
@@ -117,8 +126,8 @@ __device__ __forceinline__ void load_query(const float *ph, const float *pr, con
         const float4 vw = ld4<VEC>(pw, j, lim);
         const float4 vh = ld4<VEC>(ph, j, lim), vr = ld4<VEC>(pr, j, lim);
         q1 = vw;
-        q0 = make_float4((vh.x + vr.x) - al * vw.x, (vh.y + vr.y) - al * vw.y,
-                         (vh.z + vr.z) - al * vw.z, (vh.w + vr.w) - al * vw.w);
+        q0 = make_float4(fmaf(rs, vr.x, vh.x) - al * vw.x, fmaf(rs, vr.y, vh.y) - al * vw.y,
+                         fmaf(rs, vr.z, vh.z) - al * vw.z, fmaf(rs, vr.w, vh.w) - al * vw.w);
     } else {
         q0 = zero4();
     }

@@ -5,8 +5,9 @@ Mirrors the reference's data layer where it can be mirrored offline:
 dictionaries, ``head\\trel\\ttail`` triples; it does not download anything), and ``TrainSampler``
 plays the role of ``TrainDataset.create_sampler`` (apps/kge/data/sampler.py:304-353): batches of
 positives plus, per chunk of ``neg_chunk_size`` positives, ``neg_sample_size`` shared negative
-tails drawn uniformly (exclude_positive=False) -- drawn on the GPU by ``kge_sample_negatives``.
-Only tail corruption is produced: the score kernels share negative TAILS per chunk.
+entities drawn uniformly (exclude_positive=False) -- drawn on the GPU by ``kge_sample_negatives``.
+The negatives replace the tail, the head, or alternate between the two from batch to batch, as the
+reference's head / tail samplers do (apps/kge/data/sampler.py:287-353, 451-487).
 """
 from __future__ import annotations
 
@@ -62,11 +63,20 @@ class KGDataset:
 
 class TrainSampler:
     """Iterates over (h, r, t, neg) device tensors: ``batch_size`` positives (a seeded shuffle of the
-    training triples, reshuffled every epoch) and ``neg_sample_size`` shared negative tails for
-    every chunk of ``neg_chunk_size`` positives."""
+    training triples, reshuffled every epoch) and ``neg_sample_size`` shared negative entities for
+    every chunk of ``neg_chunk_size`` positives.
+
+    ``mode`` says which side the negatives replace: ``'tail'``, ``'head'``, or ``'both'``, which
+    alternates like the reference's NewBidirectionalOneShotIterator (apps/kge/data/sampler.py:481-487:
+    first batch tail, second head, ...).  ``neg_mode`` holds the mode of the batch returned last; pass
+    it to ``KGEModel.score(..., neg_mode=sampler.neg_mode)``."""
 
     def __init__(self, triples, n_entities, batch_size, neg_sample_size, neg_chunk_size=None, shuffle=True,
-                 seed=0, device="cuda:0"):
+                 seed=0, device="cuda:0", mode="tail"):
+        if mode not in ("tail", "head", "both"):
+            raise ValueError("mode is 'tail', 'head' or 'both'")
+        self.mode = mode
+        self.neg_mode = "head" if mode == "head" else "tail"
         self.h, self.r, self.t = (np.asarray(x, dtype=np.int64) for x in triples)
         self.n_entities, self.batch = int(n_entities), int(batch_size)
         self.n_neg = int(neg_sample_size)
@@ -102,5 +112,7 @@ class TrainSampler:
                                                    self.seed, self.step,
                                                    C.c_void_p(torch.cuda.current_stream().cuda_stream)),
                    "kge_sample_negatives")
+        if self.mode == "both":
+            self.neg_mode = "head" if self.step % 2 else "tail"
         self.step += 1
         return h, r, t, neg

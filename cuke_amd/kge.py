@@ -25,6 +25,9 @@ __all__ = ["KGEModel", "TrainStep", "Inspection", "Forward", "SparseGrads", "ins
            "transH", "transR", "transF", "RESCAL", "margin_loss", "sparse_sgd", "sparse_adagrad", "KgeError"]
 
 
+NEG_MODES = {"tail": 0, "head": 1}  # KGE_NEG_TAIL / KGE_NEG_HEAD
+
+
 def _stream() -> C.c_void_p:
     return C.c_void_p(torch.cuda.current_stream().cuda_stream)
 
@@ -123,6 +126,7 @@ class Forward:
     residual: torch.Tensor | None = None
     flat_pos: torch.Tensor | None = None   # TransR / RESCAL with negatives: scores of the flattened batch
     batch: tuple = ()
+    neg_mode: str = "tail"
     ent_insp: Inspection | None = None
     rel_insp: Inspection | None = None
 
@@ -178,7 +182,9 @@ class KGEModel:
                                 self.A.data_ptr() if self.A is not None else None)
 
     # -- helpers ---------------------------------------------------------------------------
-    def _batch(self, h, r, t, neg=None, chunk=None, ent_insp=None, rel_insp=None):
+    def _batch(self, h, r, t, neg=None, chunk=None, ent_insp=None, rel_insp=None, neg_mode="tail"):
+        if neg_mode not in NEG_MODES:
+            raise ValueError("neg_mode is 'tail' or 'head'")
         h, r, t = (_index(x, n, self.dev) for x, n in ((h, "h"), (r, "r"), (t, "t")))
         B = int(h.numel())
         if int(r.numel()) != B or int(t.numel()) != B:
@@ -196,7 +202,7 @@ class KGEModel:
         bat = _lib.Batch(B, h.data_ptr(), r.data_ptr(), t.data_ptr(),
                          neg.data_ptr() if neg is not None else None, C_, N,
                          C.pointer(ent_insp._c) if ent_insp is not None else None,
-                         C.pointer(rel_insp._c) if rel_insp is not None else None, None)
+                         C.pointer(rel_insp._c) if rel_insp is not None else None, None, NEG_MODES[neg_mode], 0)
         return bat, (h, r, t, neg, C_, N)
 
     # -- reference-shaped output -------------------------------------------------------------
@@ -214,15 +220,19 @@ class KGEModel:
         return torch.empty(max(nb, 1), dtype=torch.uint8, device=self.dev), nb
 
     # -- scalar scores ---------------------------------------------------------------------
-    def score(self, h, r, t, neg=None, chunk=None, ent_insp=None, rel_insp=None) -> Forward:
-        """pos[B] and, with shared negatives, neg[B, N] scores."""
+    def score(self, h, r, t, neg=None, chunk=None, ent_insp=None, rel_insp=None, neg_mode="tail") -> Forward:
+        """pos[B] and, with shared negatives, neg[B, N] scores.
+
+        ``neg_mode='tail'``: neg[b, k] scores (h_b, r_b, neg_k), the reference's shared-negative layout
+        (apps/examples/examples.py:1404-1444); ``'head'``: (neg_k, r_b, t_b), the head-corrupted batches of
+        the reference's sampler (apps/kge/data/sampler.py:287-353)."""
         if neg is not None and self.model in ("TransR", "RESCAL"):
-            return self._score_projected_negatives(h, r, t, neg, chunk)
-        bat, keep = self._batch(h, r, t, neg, chunk, ent_insp, rel_insp)
+            return self._score_projected_negatives(h, r, t, neg, chunk, neg_mode)
+        bat, keep = self._batch(h, r, t, neg, chunk, ent_insp, rel_insp, neg_mode)
         B, N = bat.batch, bat.n_neg
         f32 = dict(dtype=torch.float32, device=self.dev)
         fw = Forward(torch.empty(B, **f32), torch.empty((B, N), **f32) if neg is not None else None,
-                     batch=keep, ent_insp=ent_insp, rel_insp=rel_insp)
+                     batch=keep, ent_insp=ent_insp, rel_insp=rel_insp, neg_mode=neg_mode)
         if self.model == "TransH":
             fw.side_pos = torch.empty(B, **f32)
             if neg is not None:
@@ -235,11 +245,11 @@ class KGEModel:
                                             _ptr(fw.residual), _ptr(ws), nb, _stream()), "kge_score_fwd")
         return fw
 
-    def _score_projected_negatives(self, h, r, t, neg, chunk) -> Forward:
+    def _score_projected_negatives(self, h, r, t, neg, chunk, neg_mode="tail") -> Forward:
         """TransR / RESCAL with shared negatives: the projection depends on the positive's relation,
         so (as in the reference's neg_transR, examples.py:1447-1480) the B x N pairs are written out
         as explicit triples behind the B positives and scored by the grouped per-relation kernels."""
-        bat, (h, r, t, neg, C_, N) = self._batch(h, r, t, neg, chunk)
+        bat, (h, r, t, neg, C_, N) = self._batch(h, r, t, neg, chunk, neg_mode=neg_mode)
         B = bat.batch
         total = B * (1 + N)
         flat = [torch.empty(total, dtype=torch.int64, device=self.dev) for _ in range(3)]
@@ -274,7 +284,7 @@ class KGEModel:
         h, r, t, neg, C_, N = fw.batch
         if fw.ent_insp is None or fw.rel_insp is None:
             fw.ent_insp, fw.rel_insp = self.inspect_batch(h, r, t, neg)
-        bat, _ = self._batch(h, r, t, neg, C_ or None, fw.ent_insp, fw.rel_insp)
+        bat, _ = self._batch(h, r, t, neg, C_ or None, fw.ent_insp, fw.rel_insp, fw.neg_mode)
         B = bat.batch
         f32 = dict(dtype=torch.float32, device=self.dev)
         if dpos is not None:
@@ -408,13 +418,13 @@ class TrainStep:
     """
 
     def __init__(self, model: KGEModel, h, r, t, neg=None, chunk=None, loss="sum", margin=1.0,
-                 sign=1.0, dpos=None, dneg=None):
+                 sign=1.0, dpos=None, dneg=None, neg_mode="tail"):
         self.m = model
         dev = model.dev
         L = self.L = _lib.lib()
         f32 = dict(dtype=torch.float32, device=dev)
         i32 = dict(dtype=torch.int32, device=dev)
-        _, (h, r, t, neg, C_, N) = model._batch(h, r, t, neg, chunk)
+        _, (h, r, t, neg, C_, N) = model._batch(h, r, t, neg, chunk, neg_mode=neg_mode)
         self.idx = (h, r, t, neg)
         B = self.B = int(h.numel())
         self.N, self.C = N, C_
@@ -446,7 +456,7 @@ class TrainStep:
 
         self.bat = _lib.Batch(B, h.data_ptr(), r.data_ptr(), t.data_ptr(),
                               neg.data_ptr() if neg is not None else None, C_, N,
-                              C.pointer(self.ent_insp._c), C.pointer(self.rel_insp._c), None)
+                              C.pointer(self.ent_insp._c), C.pointer(self.rel_insp._c), None, NEG_MODES[neg_mode], 0)
         self.side = torch.cuda.Stream(device=dev)  # default priority
         self.insp_event = torch.cuda.Event()
         self.pos = torch.empty(B, **f32)

@@ -89,13 +89,15 @@ typedef struct kge_inspection {
     int32_t *sorted_seg;   /* capacity n */
 } kge_inspection;
 
+enum { KGE_NEG_TAIL = 0, KGE_NEG_HEAD = 1 };
+
 /* One batch of triples.  neg == NULL: positives only. */
 typedef struct kge_batch {
     int64_t batch;       /* B positives */
     const int64_t *h;    /* [B] head entity ids */
     const int64_t *r;    /* [B] relation ids */
     const int64_t *t;    /* [B] tail entity ids */
-    const int64_t *neg;  /* [B / chunk * n_neg] shared negative tail ids, chunk-major */
+    const int64_t *neg;  /* [B / chunk * n_neg] shared negative entity ids, chunk-major */
     int64_t chunk;       /* positives per chunk; B % chunk == 0 */
     int64_t n_neg;       /* negatives per chunk: positive b is scored against
                             neg[(b / chunk) * n_neg + k], k < n_neg
@@ -110,17 +112,24 @@ typedef struct kge_batch {
        concurrently with the forward pass and the gradient tile kernels.  rel_insp is NOT
        covered when the model is TransR / RESCAL (their forward already consumed it). */
     void *insp_ready;
+    /* Which side of the positive the shared negatives replace: KGE_NEG_TAIL scores
+       (h_b, r_b, neg_k), the layout of apps/examples/examples.py:1404-1444; KGE_NEG_HEAD scores
+       (neg_k, r_b, t_b), the head-corrupted batches of apps/kge/data/sampler.py:287-353
+       (neg_head).  Zero-initialised structs get KGE_NEG_TAIL. */
+    int32_t neg_mode;
+    int32_t reserved;
 } kge_batch;
 
 /* Forward outputs that backward consumes. */
 typedef struct kge_saved {
     const float *pos;       /* [B] positive scores */
     const float *neg;       /* [B, n_neg] negative scores (NULL without negatives) */
-    const float *side_pos;  /* [B]: TransH w.h per positive; TransR: unused */
-    const float *side_neg;  /* [2, B, n_neg]: TransH, plane 0 = w_b . t'_k per pair,
+    const float *side_pos;  /* [B]: TransH w.h per positive (w.t with KGE_NEG_HEAD); TransR: unused */
+    const float *side_neg;  /* [2, B, n_neg]: TransH, plane 0 = w_b . e_k per pair (e_k the negative),
                                plane 1 = sum_i phi(u_i) w_i (phi = sign for L1, u/||u|| for L2) */
     const float *residual;  /* [B, dim]: TransR residual rows / RESCAL E[h] Proj[r] rows;
-                               RotatE: rotated heads h e^{i theta} as [re | im] */
+                               RotatE: rotated heads h e^{i theta} as [re | im]
+                               (with KGE_NEG_HEAD: counter-rotated tails t e^{-i theta}) */
 } kge_saved;
 
 /* Sparse row gradients: row u of each array belongs to the u-th unique id of the

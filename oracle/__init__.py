@@ -85,9 +85,16 @@ def residual(model, E, R, A, h, r, t):
     return out
 
 
+def _neg_head(neg_mode) -> int:
+    if neg_mode not in ("tail", "head"):
+        raise ValueError("neg_mode is 'tail' or 'head'")
+    return 1 if neg_mode == "head" else 0
+
+
 def score(model, E, R, A, h, r, t, neg=None, chunk=0, p=2, gamma=0.0, fast=False,
-          want_pos=True):
-    """pos[B] and (when ``neg`` is given) negs[B, N] scores."""
+          want_pos=True, neg_mode="tail"):
+    """pos[B] and (when ``neg`` is given) negs[B, N] scores; the shared negatives replace the
+    tail (``neg_mode='tail'``) or the head (``'head'``) of every positive of their chunk."""
     E, R, A = _f32(E), _f32(R), _f32(A)
     h, r, t, neg = _i64(h), _i64(r), _i64(t), _i64(neg)
     B, d = h.shape[0], E.shape[1]
@@ -104,7 +111,7 @@ def score(model, E, R, A, h, r, t, neg=None, chunk=0, p=2, gamma=0.0, fast=False
         ctypes.c_int(MODELS[model]), ctypes.c_int(p), ctypes.c_float(gamma),
         ctypes.c_int64(B), ctypes.c_int64(d), _fp(E), _fp(R), _fp(A),
         _fp(h), _fp(r), _fp(t), _fp(neg), ctypes.c_int64(C), ctypes.c_int64(N),
-        _fp(pos), _fp(negs))
+        ctypes.c_int(_neg_head(neg_mode)), _fp(pos), _fp(negs))
     assert rc == 0
     return pos, negs
 
@@ -137,7 +144,8 @@ class SparseGrads:
     aux_rows: np.ndarray | None
 
 
-def backward(model, E, R, A, h, r, t, neg=None, chunk=0, dpos=None, dneg=None, p=2, fast=False) -> SparseGrads:
+def backward(model, E, R, A, h, r, t, neg=None, chunk=0, dpos=None, dneg=None, p=2, fast=False,
+             neg_mode="tail") -> SparseGrads:
     """Sparse row gradients (unique ids ascending, one row per id) per table."""
     E, R, A = _f32(E), _f32(R), _f32(A)
     h, r, t, neg = _i64(h), _i64(r), _i64(t), _i64(neg)
@@ -162,7 +170,7 @@ def backward(model, E, R, A, h, r, t, neg=None, chunk=0, dpos=None, dneg=None, p
     rc = _lib(fast).orc_backward(
         ctypes.c_int(MODELS[model]), ctypes.c_int(p), ctypes.c_int64(B), ctypes.c_int64(d),
         _fp(E), _fp(R), _fp(A), _fp(h), _fp(r), _fp(t), _fp(neg),
-        ctypes.c_int64(C), ctypes.c_int64(N), _fp(dpos), _fp(dneg),
+        ctypes.c_int64(C), ctypes.c_int64(N), ctypes.c_int(_neg_head(neg_mode)), _fp(dpos), _fp(dneg),
         _fp(slot_h), _fp(slot_t), _fp(slot_n), _fp(slot_r),
         ctypes.c_int64(gE.shape[0]), ctypes.c_int64(ins_r.unique_ids.shape[0]),
         _fp(gE), _fp(gR), _fp(gA))

@@ -188,10 +188,12 @@ static float score_one(int model, int p, float gamma, int64_t d, const float *eh
 }
 
 /* pos[B]; negs[B*N] when neg != NULL: positive b of chunk c = b / C is scored
- * against the N tails neg[c*N .. c*N+N-1] (examples.py:1404-1444 layout). */
+ * against the N entities neg[c*N .. c*N+N-1] (examples.py:1404-1444 layout), which replace the
+ * tail (neg_head == 0: triple (h_b, r_b, neg_k), the reference's layout) or the head
+ * (neg_head != 0: triple (neg_k, r_b, t_b), the head batches of apps/kge/data/sampler.py). */
 int orc_score(int model, int p, float gamma, int64_t B, int64_t d, const float *E, const float *R,
               const float *A, const int64_t *h, const int64_t *r, const int64_t *t,
-              const int64_t *neg, int64_t C, int64_t N, float *pos, float *negs)
+              const int64_t *neg, int64_t C, int64_t N, int neg_head, float *pos, float *negs)
 {
     const int64_t rw = rel_width(model, d), aw = aux_width(model, d);
     float *tmp = (float *)malloc(sizeof(float) * (size_t)(d > 0 ? d : 1));
@@ -207,9 +209,11 @@ int orc_score(int model, int p, float gamma, int64_t B, int64_t d, const float *
             if (pos) pos[b] = score_one(model, p, gamma, d, eh, rr, E + t[b] * d, ax, ltmp);
             if (neg) {
                 const int64_t c = b / C;
-                for (int64_t k = 0; k < N; ++k)
-                    negs[b * N + k] =
-                        score_one(model, p, gamma, d, eh, rr, E + neg[c * N + k] * d, ax, ltmp);
+                for (int64_t k = 0; k < N; ++k) {
+                    const float *en = E + neg[c * N + k] * d;
+                    negs[b * N + k] = neg_head ? score_one(model, p, gamma, d, en, rr, E + t[b] * d, ax, ltmp)
+                                               : score_one(model, p, gamma, d, eh, rr, en, ax, ltmp);
+                }
             }
         }
         free(ltmp);
@@ -221,9 +225,11 @@ int orc_score(int model, int p, float gamma, int64_t B, int64_t d, const float *
         if (pos) pos[b] = score_one(model, p, gamma, d, eh, rr, E + t[b] * d, ax, tmp);
         if (neg) {
             const int64_t c = b / C;
-            for (int64_t k = 0; k < N; ++k)
-                negs[b * N + k] =
-                    score_one(model, p, gamma, d, eh, rr, E + neg[c * N + k] * d, ax, tmp);
+            for (int64_t k = 0; k < N; ++k) {
+                const float *en = E + neg[c * N + k] * d;
+                negs[b * N + k] = neg_head ? score_one(model, p, gamma, d, en, rr, E + t[b] * d, ax, tmp)
+                                           : score_one(model, p, gamma, d, eh, rr, en, ax, tmp);
+            }
         }
     }
 #endif
@@ -380,7 +386,7 @@ static void add_row(double *acc, const float *src, int64_t n)
 
 int orc_backward(int model, int p, int64_t B, int64_t d, const float *E, const float *R,
                  const float *A, const int64_t *h, const int64_t *r, const int64_t *t,
-                 const int64_t *neg, int64_t C, int64_t N, const float *dpos, const float *dneg,
+                 const int64_t *neg, int64_t C, int64_t N, int neg_head, const float *dpos, const float *dneg,
                  const int64_t *slot_h, const int64_t *slot_t, const int64_t *slot_neg,
                  const int64_t *slot_r, int64_t n_slots_e, int64_t n_slots_r, float *gE, float *gR,
                  float *gA)
@@ -400,18 +406,20 @@ int orc_backward(int model, int p, int64_t B, int64_t d, const float *E, const f
         const int64_t c = C > 0 ? b / C : 0;
         for (int64_t q = 0; q < n_t; ++q) {
             float g;
-            const float *et;
-            int64_t slot_tail;
+            const float *ehead = eh, *et = E + t[b] * d;
+            int64_t slot_head = slot_h[b], slot_tail = slot_t[b];
             if (q == 0) {
                 if (!dpos) continue;
-                g = dpos[b], et = E + t[b] * d, slot_tail = slot_t[b];
-            } else {
+                g = dpos[b];
+            } else {  /* the negative replaces the tail, or the head when neg_head is set */
                 const int64_t k = q - 1;
-                g = dneg[b * N + k], et = E + neg[c * N + k] * d, slot_tail = slot_neg[c * N + k];
+                g = dneg[b * N + k];
+                if (neg_head) ehead = E + neg[c * N + k] * d, slot_head = slot_neg[c * N + k];
+                else et = E + neg[c * N + k] * d, slot_tail = slot_neg[c * N + k];
             }
             memset(one, 0, sizeof(float) * (size_t)(3 * d + aw));
-            bwd_one(model, p, d, eh, rr, et, ax, g, dh, dr, dt, da, tmp);
-            add_row(aE + slot_h[b] * d, dh, d);
+            bwd_one(model, p, d, ehead, rr, et, ax, g, dh, dr, dt, da, tmp);
+            add_row(aE + slot_head * d, dh, d);
             add_row(aE + slot_tail * d, dt, d);
             if (rw) add_row(aR + slot_r[b] * rw, dr, rw);
             if (aw) add_row(aA + slot_r[b] * aw, da, aw);

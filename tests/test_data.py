@@ -58,3 +58,28 @@ def test_device_sampler_bit_exact_and_feeds_a_step(oracle, tmp_path):
     E = torch.randn(4, 8, device="cuda:0"); R = torch.randn(2, 8, device="cuda:0")
     fw = KGEModel("DistMult", E, R).score(h, r, t, neg, chunk=2)
     assert fw.neg.shape == (4, 3)
+
+
+@pytest.mark.gpu
+def test_sampler_alternates_head_and_tail_batches(oracle, tmp_path):
+    # apps/kge/data/sampler.py:481-487: odd steps tail, even steps head, starting with tail
+    import torch
+    from cuke_amd.data import KGDataset, TrainSampler
+    from cuke_amd.kge import KGEModel
+    d = write_dataset(tmp_path)
+    ds = KGDataset(d / "entities.dict", d / "relations.dict", d / "train.txt")
+    s = TrainSampler(ds.train, ds.n_entities, batch_size=4, neg_sample_size=3, neg_chunk_size=2, seed=3, mode="both")
+    E = torch.randn(4, 8, device="cuda:0"); R = torch.randn(2, 8, device="cuda:0")
+    m = KGEModel("TransE", E, R)
+    modes = []
+    for _ in range(4):
+        h, r, t, neg = next(s)
+        modes.append(s.neg_mode)
+        fw = m.score(h, r, t, neg, chunk=2, neg_mode=s.neg_mode)
+        _, want = oracle.score("TransE", E.cpu().numpy(), R.cpu().numpy(), None, h.cpu().numpy(), r.cpu().numpy(),
+                               t.cpu().numpy(), neg.cpu().numpy(), 2, neg_mode=s.neg_mode)
+        np.testing.assert_allclose(fw.neg.cpu().numpy(), want, rtol=1e-5, atol=1e-6)
+    assert modes == ["tail", "head", "tail", "head"]
+    assert TrainSampler(ds.train, ds.n_entities, 4, 3, 2, mode="head").neg_mode == "head"
+    with pytest.raises(ValueError):
+        TrainSampler(ds.train, ds.n_entities, 4, 3, 2, mode="sideways")

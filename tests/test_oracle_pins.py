@@ -138,6 +138,42 @@ def test_shared_negatives_equal_flattened_triples(oracle, model):
     assert np.array_equal(negs.reshape(-1), flat)
 
 
+@pytest.mark.parametrize("model", ALL)
+def test_head_mode_negatives_equal_flattened_triples(oracle, model):
+    # negatives that replace the head: out[b][k] = f(E[neg[(b / C) * N + k]], R[r[b]], E[t[b]]),
+    # scores and sparse gradients, against the positive-only oracle on the explicit triples
+    w = small(model, seed=6)
+    a = w.arrays
+    B, N, C = w.batch, w.n_neg, w.chunk
+    _, negs = oracle.score(model, a["E"], a["R"], a["A"], a["h"], a["r"], a["t"], a["neg"], C, gamma=w.gamma,
+                           neg_mode="head")
+    fh = np.array([a["neg"][(b // C) * N + k] for b in range(B) for k in range(N)])
+    fr, ft = np.repeat(a["r"], N), np.repeat(a["t"], N)
+    flat, _ = oracle.score(model, a["E"], a["R"], a["A"], fh, fr, ft, gamma=w.gamma)
+    assert np.array_equal(negs.reshape(-1), flat)
+
+    rng = np.random.default_rng(0)
+    dpos = rng.standard_normal(B).astype(np.float32)
+    dneg = rng.standard_normal((B, N)).astype(np.float32)
+    g = oracle.backward(model, a["E"], a["R"], a["A"], a["h"], a["r"], a["t"], a["neg"], C, dpos, dneg,
+                        neg_mode="head")
+    gp = oracle.backward(model, a["E"], a["R"], a["A"], a["h"], a["r"], a["t"], dpos=dpos)
+    gn = oracle.backward(model, a["E"], a["R"], a["A"], fh, fr, ft, dpos=dneg.reshape(-1))
+
+    def dense(ids, rows, n):
+        out = np.zeros((n,) + rows.shape[1:], np.float64)
+        out[ids] = rows
+        return out
+    close(dense(g.ent_ids, g.ent_rows, w.n_ent),
+          dense(gp.ent_ids, gp.ent_rows, w.n_ent) + dense(gn.ent_ids, gn.ent_rows, w.n_ent))
+    if g.rel_rows is not None:
+        close(dense(g.rel_ids, g.rel_rows, w.n_rel),
+              dense(gp.rel_ids, gp.rel_rows, w.n_rel) + dense(gn.rel_ids, gn.rel_rows, w.n_rel))
+    if g.aux_rows is not None:
+        close(dense(g.rel_ids, g.aux_rows, w.n_rel),
+              dense(gp.rel_ids, gp.aux_rows, w.n_rel) + dense(gn.rel_ids, gn.aux_rows, w.n_rel))
+
+
 def test_reference_view_layout_is_the_special_case_neg_equals_tails(oracle):
     # examples.py:1404-1444: with N == C and neg == t every positive is scored against the
     # tails of its own chunk: out[b][k] = E[h[b]] - E[t[(b / bs) * bs + k]] + R[r[b]]
