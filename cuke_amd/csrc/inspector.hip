@@ -38,6 +38,33 @@ __device__ __forceinline__ uint32_t load_key(const Parts &parts, int64_t i)
     return (uint32_t)p[i - begin];
 }
 
+// The same with the part table held in registers and the index clamped by the caller: the load
+// is unconditional (a branch or a select around a load makes the compiler wait for it on the
+// spot, which serialises a batch of loads into one memory round trip each).
+struct KeySrc {
+    // byte address of key i = base_k + 8 i for the part k that holds position i; the bases are
+    // plain integers so that the choice is a per-lane select (choosing among pointer VALUES makes
+    // the compiler loop over the distinct pointers of a wave, one waited load per turn)
+    uint64_t b0, b1, b2, b3;
+    int64_t e0, e1, e2;
+    __device__ explicit KeySrc(const Parts &parts)
+        : e0(parts.end[0]), e1(parts.end[1]), e2(parts.end[2])
+    {
+        b0 = reinterpret_cast<uint64_t>(parts.p[0]);
+        b1 = reinterpret_cast<uint64_t>(parts.p[1]) - 8u * (uint64_t)e0;
+        b2 = reinterpret_cast<uint64_t>(parts.p[2]) - 8u * (uint64_t)e1;
+        b3 = reinterpret_cast<uint64_t>(parts.p[3]) - 8u * (uint64_t)e2;
+    }
+    __device__ __forceinline__ uint32_t operator()(int64_t i) const  // i must be a valid position
+    {
+        const uint64_t base = i < e0 ? b0 : (i < e1 ? b1 : (i < e2 ? b2 : b3));
+        // low word of the int64 id; the address-space-1 pointer makes this a global (not flat) load,
+        // which leaves the LDS counter alone so that the histogram atomics need not drain per key
+        typedef const uint32_t __attribute__((address_space(1))) *global_u32;
+        return *reinterpret_cast<global_u32>(base + 8u * (uint64_t)i);
+    }
+};
+
 // ---- pass step 1: per-block digit histogram --------------------------------------------
 __global__ __launch_bounds__(kSortThreads) void radix_hist_kernel(Parts parts, const uint32_t *keys_in,
                                                                   int64_t n, int shift, int bins,
@@ -337,25 +364,29 @@ __global__ __launch_bounds__(kMidThreads) void inspect_mid_pass_kernel(MidJobs j
 #pragma unroll
         for (int w = 0; w < kMidWaves; ++w) s_cnt[w][i] = 0;
     }
-    // own keys first (their loads overlap the counting loop)
+    // own keys first (their loads overlap the counting loop); positions past n are clamped and
+    // masked at their use
+    const KeySrc src(J.parts);
+    const int last = n - 1;
     uint32_t key[kMidRounds];
     int32_t val[kMidRounds];
 #pragma unroll
     for (int j = 0; j < kMidRounds; ++j) {
         const int i = my0 + wave * (kMidRounds * kWave) + j * kWave + lane;
-        const bool ok = i < n;
-        if constexpr (FIRST) key[j] = ok ? load_key(J.parts, i) : 0u, val[j] = i;
-        else key[j] = ok ? kin[i] : 0u, val[j] = ok ? vin[i] : 0;
+        const int ic = i < n ? i : last;
+        if constexpr (FIRST) key[j] = src(ic), val[j] = i;
+        else key[j] = kin[ic], val[j] = vin[ic];
     }
     __syncthreads();
-    constexpr int kBatch = 16;  // loads in flight per thread: the loop is latency-bound otherwise
+    constexpr int kBatch = 32;  // unconditional loads in flight per thread
     for (int i0 = 0; i0 < n; i0 += kBatch * kMidThreads) {
         uint32_t kb[kBatch];
 #pragma unroll
         for (int u = 0; u < kBatch; ++u) {
             const int i = i0 + u * kMidThreads + tid;
-            if constexpr (FIRST) kb[u] = i < n ? load_key(J.parts, i) : 0u;
-            else kb[u] = i < n ? kin[i] : 0u;
+            const int ic = i < n ? i : last;
+            if constexpr (FIRST) kb[u] = src(ic);
+            else kb[u] = kin[ic];
         }
 #pragma unroll
         for (int u = 0; u < kBatch; ++u) {
@@ -436,9 +467,9 @@ __global__ __launch_bounds__(kMidThreads) void inspect_mid_dedup_kernel(MidJobs 
 #pragma unroll
         for (int u = 0; u < 8; ++u) {
             const int g = g0 + u * kMidThreads + tid;
-            const bool ok = g < my0 / 4;
-            q[u] = ok ? reinterpret_cast<const uint4 *>(keys)[g] : make_uint4(0, 0, 0, 0);
-            pv[u] = (ok && g > 0) ? keys[4 * g - 1] : 0u;
+            const int gc = g < my0 / 4 ? g : my0 / 4 - 1;  // clamped: unconditional loads, masked below
+            q[u] = reinterpret_cast<const uint4 *>(keys)[gc];
+            pv[u] = keys[gc > 0 ? 4 * gc - 1 : 0];
         }
 #pragma unroll
         for (int u = 0; u < 8; ++u) {
