@@ -139,8 +139,11 @@ __global__ __launch_bounds__(256, KGE_TILE_OCC) void score_neg_kernel(NegArgs a)
         for (int k = 0; k < RK; ++k) acc[i][k] = 0.0f, cdot[i][k] = 0.0f, acc2[i][k] = 0.0f;
 
     const int nslice = (klen + kKD - 1) / kKD;
-#pragma unroll 1
-    for (int pass = 0; pass < NPASS; ++pass) {
+    // One sweep over the reduction axis.  `pass` is a compile-time tag: TransH's first sweep (the
+    // w . t' dot products) and second sweep (the norm) get their own straight-line inner loops; as a
+    // run-time value it put a branch around every pair of the micro-tile.
+    auto sweep = [&](auto pass_tag) {
+        constexpr int pass = decltype(pass_tag)::value;
         load_slice(0, pass);
 #pragma unroll 1
         for (int s = 0; s < nslice; ++s) {
@@ -175,7 +178,7 @@ __global__ __launch_bounds__(256, KGE_TILE_OCC) void score_neg_kernel(NegArgs a)
                     for (int k = 0; k < RK; ++k) {
                         const float4 a0 = av[0][i], a1 = av[NPA - 1][i];
                         const float4 t0 = tv[0][k], t1 = tv[NPT - 1][k];
-                        if (MODEL == KGE_TRANSH && pass == 0) {
+                        if constexpr (MODEL == KGE_TRANSH && pass == 0) {
                             float &cc = cdot[i][k];
                             cc = fmaf(a1.x, t0.x, cc);
                             cc = fmaf(a1.y, t0.y, cc);
@@ -192,7 +195,9 @@ __global__ __launch_bounds__(256, KGE_TILE_OCC) void score_neg_kernel(NegArgs a)
             }
             __syncthreads();
         }
-    }
+    };
+    sweep(std::integral_constant<int, 0>{});
+    if constexpr (NPASS == 2) sweep(std::integral_constant<int, 1>{});
 
 #pragma unroll
     for (int i = 0; i < RB; ++i) {
