@@ -119,31 +119,57 @@ __device__ __forceinline__ void bwd_tile_body(const TileArgs &a, int lid, float 
 #pragma unroll
         for (int o = 0; o < RO; ++o) acc[q][o] = zero4();
 
-    // ---- staging registers -------------------------------------------------------------
-    float4 rl[NPL][SL];
-    float4 rc[NC][CPT];
+    // ---- staging: a three-deep software pipeline --------------------------------------------
+    // While step st is computed, the rows and coefficients of step st+1 are in flight and so are
+    // the looper INDICES of step st+2 (h / r / neg ids, TransH w.h): the dependent chain
+    // "index -> row address -> row" never stalls a step.  The prefetch registers hold raw loads
+    // (load_query_raw); they are combined into query rows / scaled coefficients only when the
+    // step is written to LDS, so nothing waits on them before the compute.  TransH keeps the
+    // combine at load time: its register budget has no room for the raw operands.
+    constexpr bool kDefer = !kTH;
+    constexpr int NRAW = OWNER_POS ? NPL : (kDefer ? query_raw_count<MODEL>() : NPL);
+    constexpr int NCR = kTH ? 3 : (kL2 ? 2 : 1);  // raw coefficient planes: dneg, (sneg | side_neg x 2)
+    float4 rraw[SL][NRAW];
+    float4 craw[NCR][CPT];
+    int64_t li0[SL], li1[SL];  // looper ids: negative entity, or (kept entity, relation) of a positive
+    float lal[SL];             // TransH: w . x of a looper positive
 
-    auto load_step_v = [&](auto vtag, auto ntag, int l0) {
+    auto load_idx = [&](int l0) {
+#pragma unroll
+        for (int s = 0; s < SL; ++s) {
+            const int ll = l0 + ty + 16 * s;
+            const int lc = ll < n_loop ? ll : n_loop - 1;
+            if constexpr (OWNER_POS) {
+                li0[s] = a.neg[(int64_t)c * a.N + lc];
+            } else {
+                const int64_t b = (int64_t)c * a.C + lc;
+                li0[s] = a.h[b], li1[s] = a.r[b];
+                if constexpr (kTH) lal[s] = a.side_pos[b];
+            }
+        }
+    };
+
+    auto load_rows_v = [&](auto vtag, auto ntag, int l0) {
         constexpr bool VEC = decltype(vtag)::value, VECN = decltype(ntag)::value;
         // looper rows: thread stages rows ty + 16*s, columns col..col+3
 #pragma unroll
         for (int s = 0; s < SL; ++s) {
             const int ll = l0 + ty + 16 * s;
             const int lim = ll < n_loop ? klen : 0;
-            const int lc = ll < n_loop ? ll : n_loop - 1;
             if constexpr (OWNER_POS) {
-                const float *pt = a.ent + a.neg[(int64_t)c * a.N + lc] * (int64_t)d;
-                rl[0][s] = ld4<VEC>(pt, col, lim);
-                if constexpr (NPL == 2) rl[1][s] = ld4<VEC>(pt + half, col, lim);
+                const float *pt = a.ent + li0[s] * (int64_t)d;
+                rraw[s][0] = ld4_raw<VEC>(pt, col, lim);
+                if constexpr (NPL == 2) rraw[s][1] = ld4_raw<VEC>(pt + half, col, lim);
             } else {
-                const int64_t b = (int64_t)c * a.C + lc;
-                const int64_t rid = a.r[b];
-                float4 q0, q1;
-                load_query<MODEL, VEC>(a.ent + a.h[b] * (int64_t)d, a.rel + rid * (int64_t)a.rel_dim,
-                                  kTH ? a.aux + rid * (int64_t)d : nullptr, kTH ? a.side_pos[b] : 0.0f, col,
-                                  lim, half, q0, q1, kRot ? a.query + b * (int64_t)d : nullptr, a.rsign);
-                rl[0][s] = q0;
-                if constexpr (NPL == 2) rl[1][s] = q1;
+                const int64_t b = (int64_t)c * a.C + (ll < n_loop ? ll : n_loop - 1);
+                const float *ph = a.ent + li0[s] * (int64_t)d, *pr = a.rel + li1[s] * (int64_t)a.rel_dim;
+                const float *pw = kTH ? a.aux + li1[s] * (int64_t)d : nullptr;
+                const float *pq = kRot ? a.query + b * (int64_t)d : nullptr;
+                if constexpr (kDefer) {
+                    load_query_raw<MODEL, VEC>(ph, pr, pw, pq, col, lim, half, rraw[s]);
+                } else {
+                    load_query<MODEL, VEC>(ph, pr, pw, lal[s], col, lim, half, rraw[s][0], rraw[s][NRAW - 1], pq, a.rsign);
+                }
             }
         }
         // coefficients of the (TO owners x kKL loopers) block, read along k (contiguous)
@@ -163,45 +189,67 @@ __device__ __forceinline__ void bwd_tile_body(const TileArgs &a, int lid, float 
             }
             const int lim = inside ? a.N : 0;
             const int64_t off = ((int64_t)c * a.C + (inside ? bl : 0)) * a.N;
-            float4 g = ld4<VECN>(a.dneg + off, kl, lim);
-            if constexpr (kL2) {
-                const float4 sc = ld4<VECN>(a.sneg + off, kl, lim);
-                g.x = sc.x > 0.0f ? g.x / sc.x : 0.0f;
-                g.y = sc.y > 0.0f ? g.y / sc.y : 0.0f;
-                g.z = sc.z > 0.0f ? g.z / sc.z : 0.0f;
-                g.w = sc.w > 0.0f ? g.w / sc.w : 0.0f;
-            }
-            rc[0][s] = g;
+            craw[0][s] = ld4<VECN>(a.dneg + off, kl, lim);
+            if constexpr (kL2 && !kTH) craw[1][s] = ld4<VECN>(a.sneg + off, kl, lim);
             if constexpr (kTH) {
-                const float4 graw = ld4<VECN>(a.dneg + off, kl, lim);
-                rc[1][s] = ld4<VECN>(a.side_neg + off, kl, lim);
-                rc[2][s] = mul4(graw, ld4<VECN>(a.side_neg + a.plane + off, kl, lim));
+                craw[1][s] = ld4<VECN>(a.side_neg + off, kl, lim);
+                craw[2][s] = ld4<VECN>(a.side_neg + a.plane + off, kl, lim);
+                if constexpr (kL2) {  // fold the norm in now (TransH does not defer)
+                    const float4 sc = ld4<VECN>(a.sneg + off, kl, lim);
+                    float4 &g = craw[0][s];
+                    craw[2][s] = mul4(g, craw[2][s]);
+                    g.x = sc.x > 0.0f ? g.x / sc.x : 0.0f;
+                    g.y = sc.y > 0.0f ? g.y / sc.y : 0.0f;
+                    g.z = sc.z > 0.0f ? g.z / sc.z : 0.0f;
+                    g.w = sc.w > 0.0f ? g.w / sc.w : 0.0f;
+                } else {
+                    craw[2][s] = mul4(craw[0][s], craw[2][s]);
+                }
             }
         }
     };
 
-    auto load_step = [&](int l0) {  // one uniform dispatch per step, no branch per load
+    auto load_rows = [&](int l0) {  // one uniform dispatch per step, no branch per load
         if (vec) {
-            if (a.vecn) load_step_v(std::true_type{}, std::true_type{}, l0);
-            else load_step_v(std::true_type{}, std::false_type{}, l0);
+            if (a.vecn) load_rows_v(std::true_type{}, std::true_type{}, l0);
+            else load_rows_v(std::true_type{}, std::false_type{}, l0);
         } else {
-            if (a.vecn) load_step_v(std::false_type{}, std::true_type{}, l0);
-            else load_step_v(std::false_type{}, std::false_type{}, l0);
+            if (a.vecn) load_rows_v(std::false_type{}, std::true_type{}, l0);
+            else load_rows_v(std::false_type{}, std::false_type{}, l0);
         }
     };
 
-    auto store_step = [&]() {
+    auto store_step_v = [&](auto vtag, int l0) {
+        constexpr bool VEC = decltype(vtag)::value;
 #pragma unroll
-        for (int s = 0; s < SL; ++s)
-#pragma unroll
-            for (int pl = 0; pl < NPL; ++pl)
-                *reinterpret_cast<float4 *>(&sL[pl][ty + 16 * s][tx * 4]) = rl[pl][s];
+        for (int s = 0; s < SL; ++s) {
+            float4 q0, q1 = zero4();
+            if constexpr (OWNER_POS || !kDefer) {
+                q0 = rraw[s][0];
+                if constexpr (NPL == 2) q1 = rraw[s][NRAW - 1];
+            } else {
+                const int ll = l0 + ty + 16 * s;
+                combine_query<MODEL, VEC>(rraw[s], 0.0f, col, ll < n_loop ? klen : 0, half, a.rsign, q0, q1);
+            }
+            *reinterpret_cast<float4 *>(&sL[0][ty + 16 * s][tx * 4]) = q0;
+            if constexpr (NPL == 2) *reinterpret_cast<float4 *>(&sL[1][ty + 16 * s][tx * 4]) = q1;
+        }
 #pragma unroll
         for (int s = 0; s < CPT; ++s) {
             const int f = tid + 256 * s;
+            float4 cv[NC];
+            cv[0] = craw[0][s];
+            if constexpr (kL2 && !kTH) {
+                const float4 sc = craw[1][s];
+                cv[0].x = sc.x > 0.0f ? cv[0].x / sc.x : 0.0f;
+                cv[0].y = sc.y > 0.0f ? cv[0].y / sc.y : 0.0f;
+                cv[0].z = sc.z > 0.0f ? cv[0].z / sc.z : 0.0f;
+                cv[0].w = sc.w > 0.0f ? cv[0].w / sc.w : 0.0f;
+            }
+            if constexpr (kTH) cv[1] = craw[1][s], cv[2] = craw[2][s];
 #pragma unroll
             for (int pl = 0; pl < NC; ++pl) {
-                const float4 v = rc[pl][s];
+                const float4 v = cv[pl];
                 if constexpr (OWNER_POS) {
                     const int orow = f >> 3, l = (f & 7) * 4;
                     if (orow < TO) {
@@ -217,14 +265,23 @@ __device__ __forceinline__ void bwd_tile_body(const TileArgs &a, int lid, float 
             }
         }
     };
+    auto store_step = [&](int l0) {
+        if (vec) store_step_v(std::true_type{}, l0);
+        else store_step_v(std::false_type{}, l0);
+    };
 
     const int nstep = (n_loop + kKL - 1) / kKL;
-    load_step(0);
+    load_idx(0);
+    load_rows(0);
+    load_idx(kKL);  // clamped inside: harmless past the end
 #pragma unroll 1
     for (int st = 0; st < nstep; ++st) {
-        store_step();
+        store_step(st * kKL);
         __syncthreads();
-        if (st + 1 < nstep) load_step((st + 1) * kKL);
+        if (st + 1 < nstep) {
+            load_rows((st + 1) * kKL);
+            load_idx((st + 2) * kKL);
+        }
         // two-level sum: the kKL loopers of a step go into a fresh accumulator that is folded
         // into the running one per step, so rounding grows with sqrt(steps) of the large partial
         // sums instead of sqrt(loopers)

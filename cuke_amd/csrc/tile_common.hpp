@@ -133,6 +133,111 @@ __device__ __forceinline__ void load_query(const float *ph, const float *pr, con
     }
 }
 
+// ---- the same in two steps ---------------------------------------------------------------------
+// A tile kernel that prefetches the next block of rows while it computes on the current one only
+// overlaps the two if nothing touches the loaded registers before the compute: any arithmetic
+// on them (h * r, the zero fill of a tail) makes the compiler wait for the loads where they are
+// issued.  load_query_raw() therefore only loads -- clamped to a valid address, no select, no
+// arithmetic -- and combine_query() forms the query row when the block is written to LDS.
+template <bool VEC>
+__device__ __forceinline__ float4 ld4_raw(const float *p, int j, int lim)
+{
+    if constexpr (VEC) {  // rows are 16-byte aligned and lim % 4 == 0
+        return *reinterpret_cast<const float4 *>(p + (j < lim ? j : 0));
+    } else {
+        return make_float4(p[j + 0 < lim ? j + 0 : 0], p[j + 1 < lim ? j + 1 : 0], p[j + 2 < lim ? j + 2 : 0],
+                           p[j + 3 < lim ? j + 3 : 0]);
+    }
+}
+
+// zero the elements at or beyond lim (the whole quad when VEC)
+template <bool VEC>
+__device__ __forceinline__ float4 mask4(float4 v, int j, int lim)
+{
+    if constexpr (VEC) return j < lim ? v : make_float4(0.f, 0.f, 0.f, 0.f);
+    return make_float4(j + 0 < lim ? v.x : 0.0f, j + 1 < lim ? v.y : 0.0f, j + 2 < lim ? v.z : 0.0f,
+                       j + 3 < lim ? v.w : 0.0f);
+}
+
+template <int MODEL>
+constexpr int query_raw_count()
+{
+    return MODEL == KGE_COMPLEX ? 4 : (MODEL == KGE_TRANSH ? 3 : 2);
+}
+
+template <int MODEL, bool VEC, int N>
+__device__ __forceinline__ void load_query_raw(const float *ph, const float *pr, const float *pw, const float *pq,
+                                               int j, int lim, int half, float4 (&raw)[N])
+{
+    static_assert(N == query_raw_count<MODEL>(), "raw operand count");
+    if constexpr (MODEL == KGE_DISTMULT || MODEL == KGE_TRANSE) {
+        raw[0] = ld4_raw<VEC>(ph, j, lim);
+        raw[1] = ld4_raw<VEC>(pr, j, lim);
+    } else if constexpr (MODEL == KGE_COMPLEX) {
+        if constexpr (VEC) {  // half % 4 == 0: the four elements sit on one side of the re|im split
+            const int i = j < half ? j : j - half;
+            const int l2 = lim ? half : 0;
+            raw[0] = ld4_raw<true>(ph, i, l2), raw[1] = ld4_raw<true>(ph + half, i, l2);
+            raw[2] = ld4_raw<true>(pr, i, l2), raw[3] = ld4_raw<true>(pr + half, i, l2);
+        } else {
+            float v[4][4];
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                const int jj = j + e;
+                const int i = jj < lim ? (jj < half ? jj : jj - half) : 0;
+                v[0][e] = ph[i], v[1][e] = ph[i + half], v[2][e] = pr[i], v[3][e] = pr[i + half];
+            }
+#pragma unroll
+            for (int n = 0; n < 4; ++n) raw[n] = make_float4(v[n][0], v[n][1], v[n][2], v[n][3]);
+        }
+    } else if constexpr (MODEL == KGE_ROTATE) {
+        raw[0] = ld4_raw<VEC>(pq, j, lim);
+        raw[1] = ld4_raw<VEC>(pq + half, j, lim);
+    } else if constexpr (MODEL == KGE_TRANSH) {
+        raw[0] = ld4_raw<VEC>(pw, j, lim);
+        raw[1] = ld4_raw<VEC>(ph, j, lim);
+        raw[2] = ld4_raw<VEC>(pr, j, lim);
+    }
+}
+
+// The query row from its raw operands (same j, lim, half, rs as load_query; same arithmetic).
+template <int MODEL, bool VEC, int N>
+__device__ __forceinline__ void combine_query(const float4 (&raw)[N], float al, int j, int lim, int half, float rs,
+                                              float4 &q0, float4 &q1)
+{
+    q1 = zero4();
+    if constexpr (MODEL == KGE_DISTMULT) {
+        q0 = mask4<VEC>(mul4(raw[0], raw[1]), j, lim);
+    } else if constexpr (MODEL == KGE_TRANSE) {
+        const float4 vh = raw[0], vr = raw[1];
+        q0 = mask4<VEC>(make_float4(fmaf(rs, vr.x, vh.x), fmaf(rs, vr.y, vh.y), fmaf(rs, vr.z, vh.z), fmaf(rs, vr.w, vh.w)),
+                        j, lim);
+    } else if constexpr (MODEL == KGE_COMPLEX) {
+        const float hr[4] = {raw[0].x, raw[0].y, raw[0].z, raw[0].w}, hi[4] = {raw[1].x, raw[1].y, raw[1].z, raw[1].w};
+        const float rr[4] = {raw[2].x, raw[2].y, raw[2].z, raw[2].w};
+        const float ri[4] = {rs * raw[3].x, rs * raw[3].y, rs * raw[3].z, rs * raw[3].w};
+        float q[4];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            const int jj = VEC ? j : j + e;  // VEC: one side of the split for the whole quad
+            const float v = jj < half ? hr[e] * rr[e] - hi[e] * ri[e] : hr[e] * ri[e] + hi[e] * rr[e];
+            q[e] = jj < lim ? v : 0.0f;
+        }
+        q0 = make_float4(q[0], q[1], q[2], q[3]);
+    } else if constexpr (MODEL == KGE_ROTATE) {
+        q0 = mask4<VEC>(raw[0], j, lim);
+        q1 = mask4<VEC>(raw[1], j, lim);
+    } else if constexpr (MODEL == KGE_TRANSH) {
+        const float4 vw = raw[0], vh = raw[1], vr = raw[2];
+        q1 = mask4<VEC>(vw, j, lim);
+        q0 = mask4<VEC>(make_float4(fmaf(rs, vr.x, vh.x) - al * vw.x, fmaf(rs, vr.y, vh.y) - al * vw.y,
+                                    fmaf(rs, vr.z, vh.z) - al * vw.z, fmaf(rs, vr.w, vh.w) - al * vw.w),
+                        j, lim);
+    } else {
+        q0 = zero4();
+    }
+}
+
 // XCD-aware tile placement.  The 256 CUs sit in 8 XCDs with one L2 each, and consecutive
 // workgroup ids of a 1-D grid go to consecutive XCDs.  All tiles of one chunk share that
 // chunk's positive and negative rows, so they are steered to one XCD: every gathered row is
