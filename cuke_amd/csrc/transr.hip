@@ -739,6 +739,62 @@ __device__ __forceinline__ void transr_thin_dm_body(const DmArgs &a, float *lds,
     }
 }
 
+// K loop of a dM work item: acc (+)= X[p, i0 .. i0+31]^T Q[p, n0 .. n0+wcols) over the positions
+// p in [s0, s1).  As in gemm_sweep the loads of a superstep are free of branches: addresses are
+// clamped (a position past s1 re-reads s1 - 1 and its X value is selected to zero, a lane outside
+// the row / column range reads column i0 / n0 and produces values nobody stores), the issue
+// order of the prefetch is pinned, and the 16- or 32-row variant is a template parameter.
+template <bool TWO>
+__device__ __forceinline__ void dm_sweep(const float *xs, const float *qs, int d, int s0, int s1, int nq, int i0,
+                                         int n0, int wcols, int li, int kk, floatx4 (&acc_lo)[4], floatx4 (&acc_hi)[4])
+{
+    struct Stage {
+        float al[4], ah[4];
+        float4 bv[4];
+    };
+    const bool ilo = i0 + li < d, ihi = i0 + 16 + li < d;
+    const float *xlo = xs + i0 + (ilo ? li : 0), *xhi = xs + i0 + (ihi ? 16 + li : 0);
+    const float *qb = qs + n0 + (4 * li < wcols ? 4 * li : 0);
+    auto load_stage = [&](int q, Stage &st) {
+#pragma unroll
+        for (int s = 0; s < 4; ++s) {
+            const int p = s0 + 16 * q + 4 * kk + s;
+            const int64_t row = (int64_t)(p < s1 ? p : s1 - 1) * d;
+            st.al[s] = xlo[row];
+            if constexpr (TWO) st.ah[s] = xhi[row];
+            st.bv[s] = *reinterpret_cast<const float4 *>(qb + row);
+        }
+    };
+    // Most work items are short (a group of 5..16 triples is a single superstep), so unlike in
+    // gemm_sweep the prefetch is skipped past the end: a uniform branch per superstep, none per load.
+    Stage ring[kDmRing];
+#pragma unroll
+    for (int u = 0; u + 1 < kDmRing; ++u)
+        if (u < nq) load_stage(u, ring[u]);
+    for (int q = 0; q < nq; q += kDmRing) {
+#pragma unroll
+        for (int u = 0; u < kDmRing; ++u) {
+            const int qq = q + u;
+            if (qq >= nq) break;
+            if (qq + kDmRing - 1 < nq) load_stage(qq + kDmRing - 1, ring[(u + kDmRing - 1) % kDmRing]);
+            __builtin_amdgcn_sched_barrier(0);
+            const Stage &cur = ring[u];
+#pragma unroll
+            for (int s = 0; s < 4; ++s) {
+                const bool live = s0 + 16 * qq + 4 * kk + s < s1;
+                const float al = (live && ilo) ? cur.al[s] : 0.0f;
+                const float ah = (TWO && live && ihi) ? cur.ah[s] : 0.0f;
+                const float b4[4] = {cur.bv[s].x, cur.bv[s].y, cur.bv[s].z, cur.bv[s].w};
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    acc_lo[e] = __builtin_amdgcn_mfma_f32_16x16x4f32(al, b4[e], acc_lo[e], 0, 0, 0);
+                    if constexpr (TWO) acc_hi[e] = __builtin_amdgcn_mfma_f32_16x16x4f32(ah, b4[e], acc_hi[e], 0, 0, 0);
+                }
+            }
+        }
+    }
+}
+
 // dM[g][i][j] = sum_{p in group g} xs[p][i] * qs[p][j].  A work item is (chunk of <= 256 triples
 // of one group, 32 rows i); the four waves split the columns j; K runs over the chunk's triples,
 // operands prefetched four supersteps ahead.  Groups longer than one chunk write per-chunk
@@ -765,7 +821,6 @@ __global__ __launch_bounds__(256, KGE_TR_OCC) void transr_dm_kernel(DmArgs a)
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int li = lane & 15, kk = lane >> 4;
     const bool two_blocks = i0 + 16 < d;
-    const bool ilo = i0 + li < d, ihi = i0 + 16 + li < d;
     const int nq = (s1 - s0 + 15) / 16;
 
     for (int c0 = 0; c0 < d; c0 += 256) {
@@ -779,44 +834,8 @@ __global__ __launch_bounds__(256, KGE_TR_OCC) void transr_dm_kernel(DmArgs a)
 #pragma unroll
         for (int e = 0; e < 4; ++e) acc_lo[e] = floatx4{0.f, 0.f, 0.f, 0.f}, acc_hi[e] = floatx4{0.f, 0.f, 0.f, 0.f};
 
-        struct Stage {
-            float al[4], ah[4];
-            float4 bv[4];
-        };
-        auto load_stage = [&](int q, Stage &st) {
-#pragma unroll
-            for (int s = 0; s < 4; ++s) {
-                const int p = s0 + 16 * q + 4 * kk + s;
-                const bool ok = p < s1;
-                const float *xr = a.xs + (int64_t)p * d + i0;
-                st.al[s] = (ok && ilo) ? xr[li] : 0.0f;
-                st.ah[s] = (ok && ihi) ? xr[16 + li] : 0.0f;
-                st.bv[s] = (ok && colok) ? *reinterpret_cast<const float4 *>(a.qs + (int64_t)p * d + n0 + 4 * li)
-                                         : make_float4(0.f, 0.f, 0.f, 0.f);
-            }
-        };
-        Stage ring[kDmRing];
-#pragma unroll
-        for (int u = 0; u < kDmRing; ++u)
-            if (u < nq) load_stage(u, ring[u]);
-        for (int q = 0; q < nq; q += kDmRing) {
-#pragma unroll
-            for (int u = 0; u < kDmRing; ++u) {
-                if (q + u >= nq) break;
-                const Stage cur = ring[u];
-                if (q + u + kDmRing < nq) load_stage(q + u + kDmRing, ring[u]);
-#pragma unroll
-                for (int s = 0; s < 4; ++s) {
-                    const float b4[4] = {cur.bv[s].x, cur.bv[s].y, cur.bv[s].z, cur.bv[s].w};
-#pragma unroll
-                    for (int e = 0; e < 4; ++e) {
-                        acc_lo[e] = __builtin_amdgcn_mfma_f32_16x16x4f32(cur.al[s], b4[e], acc_lo[e], 0, 0, 0);
-                        if (two_blocks)
-                            acc_hi[e] = __builtin_amdgcn_mfma_f32_16x16x4f32(cur.ah[s], b4[e], acc_hi[e], 0, 0, 0);
-                    }
-                }
-            }
-        }
+        if (two_blocks) dm_sweep<true>(a.xs, a.qs, d, s0, s1, nq, i0, n0, wcols, li, kk, acc_lo, acc_hi);
+        else dm_sweep<false>(a.xs, a.qs, d, s0, s1, nq, i0, n0, wcols, li, kk, acc_lo, acc_hi);
         if (colok) {
 #pragma unroll
             for (int blk = 0; blk < 2; ++blk)
