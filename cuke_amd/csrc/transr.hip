@@ -72,9 +72,13 @@ __device__ int block_inclusive_scan_1024(int v, int *s_scan)
     return v + before;
 }
 
+// One workgroup per plan: block 0 builds `plan0` with tiles of `tile0` positions, block 1 (when
+// launched) `plan1` with `tile1`.
 __global__ __launch_bounds__(1024) void transr_plan_kernel(const int32_t *num_unique, const int32_t *seg_offsets,
-                                                          TilePlan plan, int tile)
+                                                          TilePlan plan0, int tile0, TilePlan plan1, int tile1)
 {
+    const TilePlan &plan = blockIdx.x == 0 ? plan0 : plan1;
+    const int tile = blockIdx.x == 0 ? tile0 : tile1;
     __shared__ int s_scan[1024];
     __shared__ int s_carry[3];
     const int U = num_unique[0];
@@ -932,7 +936,8 @@ int launch_transr_fwd(const kge_tables *tab, const kge_batch *bat, float *pos, f
     const kge_inspection *ri = bat->rel_insp;
     const int64_t tiles = max_tiles(tab, bat);
     TilePlan plan = plan_at(workspace, tiles, 0);
-    hipLaunchKernelGGL(transr_plan_kernel, dim3(1), dim3(1024), 0, st, ri->num_unique, ri->seg_offsets, plan, kTM);
+    hipLaunchKernelGGL(transr_plan_kernel, dim3(1), dim3(1024), 0, st, ri->num_unique, ri->seg_offsets, plan, kTM,
+                       plan, kTM);
     GemmArgs a{tab->ent, tab->rel, tab->aux, bat->h, bat->r, bat->t, ri->perm, ri->seg_offsets, ri->num_unique, ri->unique_ids,
                plan, nullptr, pos, resid, nullptr, nullptr, (int)tab->dim, tab->norm_p, thin_groups(tab, bat), (int)tiles};
     const size_t lds = gemm_lds_bytes((int)tab->dim);
@@ -970,9 +975,8 @@ int launch_transr_bwd(const kge_tables *tab, const kge_batch *bat, const kge_sav
     PrepArgs pa{tab->ent, bat->h, bat->t, ri->perm, dpos, saved->pos, saved->residual, xs, qs, occ + B * d, B, d,
                 tab->norm_p, rescal ? 1 : 0};
     hipLaunchKernelGGL(transr_prep_kernel, dim3((unsigned)ceil_div(B, 4)), dim3(256), 0, st, pa);
-    hipLaunchKernelGGL(transr_plan_kernel, dim3(1), dim3(1024), 0, st, ri->num_unique, ri->seg_offsets, plan, kTM);
-    hipLaunchKernelGGL(transr_plan_kernel, dim3(1), dim3(1024), 0, st, ri->num_unique, ri->seg_offsets, dplan,
-                       kDmChunk);
+    hipLaunchKernelGGL(transr_plan_kernel, dim3(2), dim3(1024), 0, st, ri->num_unique, ri->seg_offsets, plan, kTM,
+                       dplan, kDmChunk);
     // dX = Q M^T -> occurrence rows of h (and -dX for t)
     GemmArgs ga{tab->ent, tab->rel, tab->aux, bat->h, bat->r, bat->t, ri->perm, ri->seg_offsets, ri->num_unique, ri->unique_ids,
                 plan, qs, nullptr, nullptr, occ, rescal ? nullptr : occ + B * d, d, tab->norm_p, thin_groups(tab, bat), (int)p.tiles};
