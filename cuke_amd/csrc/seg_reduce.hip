@@ -39,44 +39,57 @@ __global__ __launch_bounds__(256) void seg_reduce_l1(SegArgs3 jobs)
     const int cnt = (int)((a.n - p0) < kSegL ? (a.n - p0) : kSegL);
     const bool active = colv < d;
 
-    int seg[kSegL];
+    // Everything the walk needs is loaded up front in batches of unconditional loads (positions
+    // past the end re-read the last valid one, an inactive lane reads column 0, both are masked
+    // afterwards): a branch or a select around a load would make the compiler wait for each load
+    // on the spot and turn the eight rows into eight serial round trips.
+    int64_t pc[kSegL];
+#pragma unroll
+    for (int q = 0; q < kSegL; ++q) pc[q] = p0 + (q < cnt ? q : cnt - 1);
+    int src[kSegL], seg[kSegL];
+    if (a.perm) {  // uniform
+#pragma unroll
+        for (int q = 0; q < kSegL; ++q) src[q] = a.perm[pc[q]];
+    } else {
+#pragma unroll
+        for (int q = 0; q < kSegL; ++q) src[q] = (int)pc[q];
+    }
+#pragma unroll
+    for (int q = 0; q < kSegL; ++q) seg[q] = a.sorted_seg[pc[q]];
+    const int cc = active ? colv : 0;
     Vec<V> v[kSegL];
 #pragma unroll
-    for (int q = 0; q < kSegL; ++q) {
-        const bool ok = q < cnt;
-        const int64_t p = p0 + (ok ? q : 0);
-        const int src = a.perm ? a.perm[p] : (int)p;
-        seg[q] = ok ? a.sorted_seg[p] : -1;
-        if (ok && active) v[q] = Vec<V>::load(a.occ + (int64_t)src * d + colv);
-        else
-#pragma unroll
-            for (int e = 0; e < V; ++e) v[q].v[e] = 0.0f;
-    }
+    for (int q = 0; q < kSegL; ++q) v[q] = Vec<V>::load(a.occ + (int64_t)src[q] * d + cc);
+    // A run starts before this block iff it shares its id with the position in front of the block,
+    // and runs on past it iff it shares it with the position behind: two loads instead of the run
+    // bounds of every position.
+    const int seg_before = a.sorted_seg[p0 > 0 ? p0 - 1 : 0], seg_after = a.sorted_seg[p0 + cnt < a.n ? p0 + cnt : p0];
+    const int prev_id = p0 > 0 ? seg_before : -1;
+    const int next_id = p0 + cnt < a.n ? seg_after : -1;
+
     Vec<V> acc;
 #pragma unroll
     for (int e = 0; e < V; ++e) acc.v[e] = 0.0f;
-    int cur = seg[0];
     auto flush = [&](int sg) {
-        const int s0 = a.seg_offsets[sg], s1 = a.seg_offsets[sg + 1];
         float *dst;
-        if (s0 >= p0 && s1 <= p0 + kSegL) dst = a.out + (int64_t)sg * d;
-        else dst = a.partial + (j * 2 + (s0 < p0 ? 0 : 1)) * (int64_t)d;
+        if (sg == prev_id) dst = a.partial + (j * 2 + 0) * (int64_t)d;       // began in an earlier block
+        else if (sg == next_id) dst = a.partial + (j * 2 + 1) * (int64_t)d;  // continues in a later block
+        else dst = a.out + (int64_t)sg * d;                                   // wholly inside: final
         if (active) acc.store(dst + colv);
     };
 #pragma unroll
     for (int q = 0; q < kSegL; ++q) {
         if (q < cnt) {
-            if (seg[q] != cur) {
-                flush(cur);
+            if (q > 0 && seg[q] != seg[q - 1]) {
+                flush(seg[q - 1]);
 #pragma unroll
                 for (int e = 0; e < V; ++e) acc.v[e] = 0.0f;
-                cur = seg[q];
             }
 #pragma unroll
             for (int e = 0; e < V; ++e) acc.v[e] += v[q].v[e];
         }
     }
-    flush(cur);
+    flush(seg[cnt - 1]);
 }
 
 template <int V>
@@ -105,11 +118,14 @@ __global__ __launch_bounds__(256) void seg_reduce_l2(SegArgs3 jobs)
 #pragma unroll
             for (int u = 0; u < 4; ++u) {
                 const int64_t jb = jj + 4 * u;
-                if (active && jb <= je) t[u] = Vec<V>::load(a.partial + (jb * 2) * (int64_t)d + colv);
-                else
+                t[u] = Vec<V>::load(a.partial + ((jb <= je ? jb : je) * 2) * (int64_t)d + (active ? colv : 0));
+            }
+#pragma unroll
+            for (int u = 0; u < 4; ++u)
+                if (jj + 4 * u > je) {
 #pragma unroll
                     for (int e = 0; e < V; ++e) t[u].v[e] = 0.0f;
-            }
+                }
 #pragma unroll
             for (int u = 0; u < 4; ++u)
 #pragma unroll
