@@ -29,12 +29,12 @@ FP32_PEAK_TFLOPS = 157.3    # MI355X fp32 vector / fp32 MFMA, published
 # reads for the 256 MiB copy kernel of --calibrate-copy (fetch x2.000, write x1.000).  The
 # summaries the numbers come from are profiles/score_path_kernels_<workload>.txt.
 MEASURED_TRAFFIC_BYTES = {
-    "cfg1_transe": 1_664_838,      # score_pos_kernel
-    "cfg2_distmult": 12_956_644,   # score_neg_kernel
-    "cfg2_complex": 12_989_600,    # score_neg_kernel
-    "cfg3_transr": 163_398_460,    # transr_gemm_kernel<0>
-    "cfg4_rotate": 12_094_015,     # score_neg_kernel
-    "cfg5_transh": 619_524_137,    # score_neg_kernel
+    "cfg1_transe": 1_664_794,      # score_pos_kernel
+    "cfg2_distmult": 12_965_862,   # score_neg_kernel
+    "cfg2_complex": 12_999_779,    # score_neg_kernel
+    "cfg3_transr": 164_185_957,    # transr_gemm_kernel<0>
+    "cfg4_rotate": 12_029_140,     # score_neg_kernel
+    "cfg5_transh": 530_065_844,    # score_neg_kernel
 }
 
 

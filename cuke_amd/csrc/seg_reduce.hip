@@ -113,21 +113,22 @@ __global__ __launch_bounds__(256) void seg_reduce_l2(SegArgs3 jobs)
         Vec<V> acc;
 #pragma unroll
         for (int e = 0; e < V; ++e) acc.v[e] = 0.0f;
-        for (int64_t jj = j + 1 + wave; jj <= je; jj += 16) {  // four loads in flight per wave
-            Vec<V> t[4];
+        constexpr int kFly = 8;  // partial rows in flight per wave: the hottest row's chain is the long pole
+        for (int64_t jj = j + 1 + wave; jj <= je; jj += 4 * kFly) {
+            Vec<V> t[kFly];
 #pragma unroll
-            for (int u = 0; u < 4; ++u) {
+            for (int u = 0; u < kFly; ++u) {
                 const int64_t jb = jj + 4 * u;
                 t[u] = Vec<V>::load(a.partial + ((jb <= je ? jb : je) * 2) * (int64_t)d + (active ? colv : 0));
             }
 #pragma unroll
-            for (int u = 0; u < 4; ++u)
+            for (int u = 0; u < kFly; ++u)
                 if (jj + 4 * u > je) {
 #pragma unroll
                     for (int e = 0; e < V; ++e) t[u].v[e] = 0.0f;
                 }
 #pragma unroll
-            for (int u = 0; u < 4; ++u)
+            for (int u = 0; u < kFly; ++u)
 #pragma unroll
                 for (int e = 0; e < V; ++e) acc.v[e] += t[u].v[e];
         }
