@@ -88,6 +88,9 @@ EXPORTS = {
 _lib = None
 
 
+ABI_VERSION = 2  # layout of the ctypes structures above; must match kge_abi_version()
+
+
 def lib() -> C.CDLL:
     global _lib
     if _lib is None:
@@ -99,6 +102,9 @@ def lib() -> C.CDLL:
         for name, (res, args) in EXPORTS.items():
             fn = getattr(handle, name)
             fn.restype, fn.argtypes = res, args
+        if handle.kge_abi_version() != ABI_VERSION:
+            raise KgeError(f"{LIB_PATH} has ABI version {handle.kge_abi_version()}, this package expects "
+                           f"{ABI_VERSION}: rebuild it with `python -m cuke_amd.build`")
         _lib = handle
     return _lib
 
