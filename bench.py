@@ -273,7 +273,7 @@ def main():
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": ms,
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32",
         "data": "synthetic (seeded N(0,sigma) tables, Zipf/uniform indices, shared negatives per chunk)",
-        "config": {"workload": w.name, "model": w.model, "n_ent": w.n_ent, "n_rel": w.n_rel, "dim": w.dim,
+        "config": {"workload": w.name, "score_function": w.model, "n_ent": w.n_ent, "n_rel": w.n_rel, "dim": w.dim,
                    "batch": w.batch, "chunk": w.chunk, "n_neg": w.n_neg, "norm_p": w.norm_p,
                    "backward": do_bwd, "loss": w.loss, "hip_graph": use_graph,
                    "ms_per_step_direct": ms_direct, "ms_per_step_graph": ms_graph,
