@@ -345,6 +345,10 @@ __global__ __launch_bounds__(kMidThreads) void inspect_mid_pass_kernel(MidJobs j
     __shared__ uint32_t s_bef[kMaxBins];             // same digit, earlier blocks
     __shared__ uint32_t s_cnt[kMidWaves][kMaxBins];  // per-wave running counts
     __shared__ uint32_t s_w[kMidWaves];
+    // The inspection usually runs on its own stream next to the score kernels, whose waves fill
+    // every SIMD; without a raised wave priority these few workgroups get a fraction of the issue
+    // slots and the step waits for them at the join.
+    __builtin_amdgcn_s_setprio(3);
     const MidJob &J = jobs.j[blockIdx.y];
     const int n = (int)J.n;
     if (pass >= J.npass || (int)blockIdx.x * kMidKeys >= n) return;
@@ -450,6 +454,7 @@ __global__ __launch_bounds__(kMidThreads) void inspect_mid_pass_kernel(MidJobs j
 __global__ __launch_bounds__(kMidThreads) void inspect_mid_dedup_kernel(MidJobs jobs)
 {
     __shared__ uint32_t s_red[kMidWaves], s_scan[kMidWaves];
+    __builtin_amdgcn_s_setprio(3);
     const MidJob &J = jobs.j[blockIdx.y];
     const int n = (int)J.n;
     const int nblk = n > 0 ? (n + kMidKeys - 1) / kMidKeys : 1;

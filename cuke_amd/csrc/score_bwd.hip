@@ -392,7 +392,9 @@ static int launch_tiles(TileArgs a, float *g0, float *g1, float *occ_neg, int64_
     const int klen = MODEL == KGE_ROTATE ? a.d / 2 : a.d;
     const int64_t gx = ceil_div(klen, kTI);
     const int64_t big = gx * (ceil_div(a.C, 64) + ceil_div(a.N, 64)) * n_chunks;
-    if (big >= 1024) {
+    static const int knob = [] { const char *e = getenv("KGE_BWD_TILE"); return e ? atoi(e) : 0; }();
+    // KGE_BWD_TILE is a development knob; the size rule follows launch_neg_mp (see there)
+    if (knob == 4 || (knob != 2 && big >= 1024)) {
         const unsigned gh = xcd_grid(gx, ceil_div(a.C, 64), n_chunks), gn = xcd_grid(gx, ceil_div(a.N, 64), n_chunks);
         hipLaunchKernelGGL((bwd_tile_kernel<MODEL, P, 4>), dim3(gh + gn), dim3(256), 0, st, a, g0, g1, occ_neg, (int)gh);
     } else {
