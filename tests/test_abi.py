@@ -47,3 +47,63 @@ def test_host_side_rejects_cpu_tensors():
         KGEModel("TransE", torch.zeros(4, 8), torch.zeros(2, 8))
     with pytest.raises(ValueError):
         KGEModel("NoSuchModel", torch.zeros(4, 8), torch.zeros(2, 8))
+
+
+def test_argument_validation_returns_status_codes_without_touching_the_gpu():
+    """Every entry point validates before it launches: wrong arguments come back as status codes
+    (the reference raises c10::Error from tensor accessors instead, pycuke1/codegen/cpu.py:9-13).
+    The pointers below are never dereferenced on the host and no kernel is launched."""
+    import ctypes as C
+    from cuke_amd import _lib
+    L = _lib.lib()
+    EINVAL, ESHAPE, EWORKSPACE = -1, -2, -4
+    fake = C.c_void_p(0x1000)  # stands for a device pointer; validation must reject before any use
+
+    def tables(model=0, dim=16, rel_dim=16, n_ent=10, n_rel=3, p=2, ent=fake, rel=fake, aux=None):
+        return _lib.Tables(model, p, 0.0, 0, dim, rel_dim, n_ent, n_rel, ent, rel, aux)
+
+    def batch(B=8, h=fake, r=fake, t=fake, neg=None, chunk=0, n_neg=0, mode=0):
+        return _lib.Batch(B, h, r, t, neg, chunk, n_neg, None, None, None, mode, 0)
+
+    out = fake
+    # null descriptors / tables
+    assert L.kge_residual_fwd(None, C.byref(batch()), out, None, 0, None) == EINVAL
+    assert L.kge_score_fwd(C.byref(tables(ent=None)), C.byref(batch()), out, None, None, None, None, None, 0,
+                           None) == EINVAL
+    # unknown model, bad norm order, odd complex dimension, wrong relation width
+    assert L.kge_score_fwd(C.byref(tables(model=99)), C.byref(batch()), out, None, None, None, None, None, 0,
+                           None) == EINVAL
+    assert L.kge_score_fwd(C.byref(tables(p=3)), C.byref(batch()), out, None, None, None, None, None, 0,
+                           None) == EINVAL
+    assert L.kge_score_fwd(C.byref(tables(model=_lib.MODELS["ComplEx"], dim=15, rel_dim=15)), C.byref(batch()), out,
+                           None, None, None, None, None, 0, None) == ESHAPE
+    assert L.kge_score_fwd(C.byref(tables(rel_dim=8)), C.byref(batch()), out, None, None, None, None, None, 0,
+                           None) == ESHAPE
+    # TransH without its normals
+    assert L.kge_score_fwd(C.byref(tables(model=_lib.MODELS["TransH"])), C.byref(batch()), out, None, None, None,
+                           None, None, 0, None) == EINVAL
+    # batch: missing index arrays, batch not a whole number of chunks, unknown negative mode
+    assert L.kge_score_fwd(C.byref(tables()), C.byref(batch(h=None)), out, None, None, None, None, None, 0,
+                           None) == EINVAL
+    assert L.kge_score_fwd(C.byref(tables()), C.byref(batch(B=10, neg=fake, chunk=4, n_neg=2)), out, fake, None,
+                           None, None, None, 0, None) == ESHAPE
+    assert L.kge_score_fwd(C.byref(tables()), C.byref(batch(neg=fake, chunk=4, n_neg=2, mode=7)), out, fake, None,
+                           None, None, None, 0, None) == EINVAL
+    # backward: inspections are mandatory
+    saved, grads = _lib.Saved(fake, None, None, None, None), _lib.Grads(fake, fake, None)
+    assert L.kge_score_bwd(C.byref(tables()), C.byref(batch()), C.byref(saved), fake, None, C.byref(grads), fake,
+                           1 << 20, None) == EINVAL
+    # inspector: part count, row range, workspace
+    assert L.kge_inspect(None, None, 1, 10, None, None, 0, None) == EINVAL
+    assert L.kge_inspect_batch(None, 1, None) == EINVAL
+    assert L.kge_inspect_workspace(-1, 10) == 0 and L.kge_inspect_workspace(100, 0) == 0
+    # loss: workspace too small
+    assert L.kge_margin_loss(fake, fake, 8, 4, 1.0, 1.0, fake, None, None, fake, 8, None) == EWORKSPACE
+    # build_index / sampler / index check
+    assert L.kge_sample_negatives(fake, 10, 0, 1, 0, None) == ESHAPE
+    assert L.kge_sample_negatives(None, 10, 5, 1, 0, None) == EINVAL
+    assert L.kge_check_indices(fake, 10, 5, None, None) == EINVAL
+    # empty work is not an error and launches nothing
+    assert L.kge_score_fwd(C.byref(tables()), C.byref(batch(B=0, h=None, r=None, t=None)), None, None, None, None,
+                           None, None, 0, None) == 0
+    assert L.kge_sample_negatives(None, 0, 5, 1, 0, None) == 0
