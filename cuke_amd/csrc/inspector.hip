@@ -70,6 +70,7 @@ __global__ __launch_bounds__(kSortThreads) void radix_hist_kernel(Parts parts, c
                                                                   int64_t n, int shift, int bins,
                                                                   uint32_t *hist)
 {
+    __builtin_amdgcn_s_setprio(3);  // see inspect_mid_pass_kernel
     __shared__ uint32_t sh[kMaxBins];
     for (int i = threadIdx.x; i < bins; i += kSortThreads) sh[i] = 0;
     __syncthreads();
@@ -90,6 +91,7 @@ __global__ __launch_bounds__(kSortThreads) void radix_hist_kernel(Parts parts, c
 // ---- pass step 2 (many blocks only): exclusive scan down each histogram column ---------
 __global__ void radix_colscan_kernel(uint32_t *hist, uint32_t *totals, int bins, int nblocks)
 {
+    __builtin_amdgcn_s_setprio(3);  // see inspect_mid_pass_kernel
     const int bin = blockIdx.x * blockDim.x + threadIdx.x;
     if (bin >= bins) return;
     uint32_t run = 0;
@@ -137,6 +139,7 @@ __global__ __launch_bounds__(kSortThreads) void radix_scatter_kernel(
     const uint32_t *hist, const uint32_t *totals, int nblocks, int fused_scan, uint32_t *keys_out,
     int32_t *vals_out)
 {
+    __builtin_amdgcn_s_setprio(3);  // see inspect_mid_pass_kernel
     __shared__ uint32_t s_base[kMaxBins];               // global start of (bin, this block)
     __shared__ uint32_t s_cnt[kSortWaves][kMaxBins];    // per-wave running digit counts
     __shared__ uint32_t s_wtot[kSortWaves];
@@ -231,6 +234,7 @@ __global__ __launch_bounds__(kSortThreads) void radix_scatter_kernel(
 __global__ __launch_bounds__(kSortThreads) void count_heads_kernel(const uint32_t *keys, int64_t n,
                                                                    uint32_t *block_heads)
 {
+    __builtin_amdgcn_s_setprio(3);  // see inspect_mid_pass_kernel
     __shared__ uint32_t s_w[kSortWaves];
     const int64_t base = (int64_t)blockIdx.x * kKeysPerBlock;
     int c = 0;
@@ -253,6 +257,7 @@ __global__ __launch_bounds__(kSortThreads) void finalize_kernel(const uint32_t *
                                                                 int64_t n, const uint32_t *block_heads,
                                                                 int nblocks, kge_inspection out)
 {
+    __builtin_amdgcn_s_setprio(3);  // see inspect_mid_pass_kernel
     __shared__ uint32_t s_red[kSortWaves], s_all[kSortWaves], s_scan[kSortWaves];
     const int tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid >> 6;
     const int me = blockIdx.x;
