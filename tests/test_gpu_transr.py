@@ -22,6 +22,8 @@ def grouped_forward(m, ix):
     dict(dim=256, batch=1000, n_rel=400),    # mostly singletons
     dict(dim=64, batch=257, n_rel=1),        # one group, many tiles
     dict(dim=36, batch=130, n_rel=9),        # K tail (36 = 2 * 16 + 4)
+    dict(dim=400, batch=60, n_rel=40),       # wide rows: two column sweeps, thin tails in two k-chunks
+    dict(dim=496, batch=24, n_rel=20),       # the widest row the LDS tile takes
 ])
 @pytest.mark.parametrize("p", [1, 2])
 def test_grouped_forward(oracle, model, shape, p):
@@ -48,6 +50,8 @@ def test_grouped_forward(oracle, model, shape, p):
     dict(dim=200, batch=300, n_rel=7),
     dict(dim=36, batch=130, n_rel=9),
     dict(dim=64, batch=257, n_rel=1),
+    dict(dim=400, batch=60, n_rel=40),
+    dict(dim=496, batch=24, n_rel=20),
 ])
 @pytest.mark.parametrize("p", [1, 2])
 def test_grouped_backward(oracle, model, shape, p):
@@ -65,7 +69,13 @@ def test_grouped_backward(oracle, model, shape, p):
     ref = oracle.backward(model, a["E"], a["R"], a["A"], a["h"], a["r"], a["t"], dpos=dpos, p=p)
     assert np.array_equal(g.ent_ids.cpu().numpy(), ref.ent_ids)
     assert np.array_equal(g.rel_ids.cpu().numpy(), ref.rel_ids)
-    assert_close(g.ent_rows.cpu().numpy(), ref.ent_rows, what="entity rows", rows=True)
+    # dX = Q M^T sums `dim` products per element.  With the L1 norm every q_j is +-g, so a row of dX is
+    # g times an alternating sum of projection entries: the partial sums are an order of magnitude above
+    # the result, and fp32 accumulation (GPU) differs from the oracle's double accumulation by
+    # eps * sqrt(dim) * sum|terms|, not by eps * |result|.  For the wide rows the floor is therefore the
+    # scale of the whole array rather than of the (cancelled) row.
+    floor = 2.0 if (p == 1 and shape["dim"] >= 400) else 0.0
+    assert_close(g.ent_rows.cpu().numpy(), ref.ent_rows, what="entity rows", rows=True, global_floor=floor)
     if model == "TransR":
         assert_close(g.rel_rows.cpu().numpy(), ref.rel_rows, what="relation rows", rows=True)
     assert_close(g.aux_rows.cpu().numpy(), ref.aux_rows, what="projection gradients", rows=True)
