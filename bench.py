@@ -29,12 +29,12 @@ FP32_PEAK_TFLOPS = 157.3    # MI355X fp32 vector / fp32 MFMA, published
 # reads for the 256 MiB copy kernel of --calibrate-copy (fetch x2.000, write x1.000).  The
 # summaries the numbers come from are profiles/score_path_kernels_<workload>.txt.
 MEASURED_TRAFFIC_BYTES = {
-    "cfg1_transe": 1_664_794,      # score_pos_kernel
-    "cfg2_distmult": 12_965_862,   # score_neg_kernel
-    "cfg2_complex": 12_999_779,    # score_neg_kernel
-    "cfg3_transr": 164_185_957,    # transr_gemm_kernel<0>
-    "cfg4_rotate": 12_029_140,     # score_neg_kernel
-    "cfg5_transh": 530_065_844,    # score_neg_kernel
+    "cfg1_transe": 1_664_832,      # score_pos_kernel
+    "cfg2_distmult": 12_964_826,   # score_neg_kernel
+    "cfg2_complex": 12_999_689,    # score_neg_kernel
+    "cfg3_transr": 164_198_860,    # transr_gemm_kernel<0>
+    "cfg4_rotate": 12_029_161,     # score_neg_kernel
+    "cfg5_transh": 530_513_415,    # score_neg_kernel
 }
 
 
