@@ -28,17 +28,7 @@ struct Parts {
     int n_parts;
 };
 
-// Key i of the concatenation.  Branch-free address selection (unused parts have end == n, so
-// they are never chosen): a loop here would keep the compiler from batching the callers' loads.
-__device__ __forceinline__ uint32_t load_key(const Parts &parts, int64_t i)
-{
-    const int64_t e0 = parts.end[0], e1 = parts.end[1], e2 = parts.end[2];
-    const int64_t *p = i < e0 ? parts.p[0] : (i < e1 ? parts.p[1] : (i < e2 ? parts.p[2] : parts.p[3]));
-    const int64_t begin = i < e0 ? 0 : (i < e1 ? e0 : (i < e2 ? e1 : e2));
-    return (uint32_t)p[i - begin];
-}
-
-// The same with the part table held in registers and the index clamped by the caller: the load
+// Key i of the concatenation, with the part table held in registers and the index clamped by the caller: the load
 // is unconditional (a branch or a select around a load makes the compiler wait for it on the
 // spot, which serialises a batch of loads into one memory round trip each).
 struct KeySrc {
@@ -76,14 +66,25 @@ __global__ __launch_bounds__(kSortThreads) void radix_hist_kernel(Parts parts, c
     __syncthreads();
     const int64_t base = (int64_t)blockIdx.x * kKeysPerBlock;
     const uint32_t mask = (uint32_t)bins - 1;
+    // all loads first (clamped, unconditional), then the counting
+    const KeySrc src(parts);
+    uint32_t kb[kKeysPerThread];
+    if (keys_in) {  // uniform
 #pragma unroll
-    for (int j = 0; j < kKeysPerThread; ++j) {
-        const int64_t i = base + j * kSortThreads + threadIdx.x;
-        if (i < n) {
-            const uint32_t k = keys_in ? keys_in[i] : load_key(parts, i);
-            atomicAdd(&sh[(k >> shift) & mask], 1u);
+        for (int j = 0; j < kKeysPerThread; ++j) {
+            const int64_t i = base + j * kSortThreads + threadIdx.x;
+            kb[j] = keys_in[i < n ? i : n - 1];
+        }
+    } else {
+#pragma unroll
+        for (int j = 0; j < kKeysPerThread; ++j) {
+            const int64_t i = base + j * kSortThreads + threadIdx.x;
+            kb[j] = src(i < n ? i : n - 1);
         }
     }
+#pragma unroll
+    for (int j = 0; j < kKeysPerThread; ++j)
+        if (base + j * kSortThreads + threadIdx.x < n) atomicAdd(&sh[(kb[j] >> shift) & mask], 1u);
     __syncthreads();
     for (int i = threadIdx.x; i < bins; i += kSortThreads) hist[(int64_t)blockIdx.x * bins + i] = sh[i];
 }
@@ -181,12 +182,27 @@ __global__ __launch_bounds__(kSortThreads) void radix_scatter_kernel(
     uint32_t key[kKeysPerThread], lrank[kKeysPerThread];
     int32_t val[kKeysPerThread];
     const uint64_t lt_mask = lane ? (~0ull >> (kWave - lane)) : 0ull;
+    {  // all key / value loads of the thread in one batch (clamped, unconditional)
+        const KeySrc src(parts);
+        if (keys_in) {  // uniform: later passes read the previous pass's output
+#pragma unroll
+            for (int j = 0; j < kKeysPerThread; ++j) {
+                const int64_t i = wbase + j * kWave + lane;
+                const int64_t ic = i < n ? i : n - 1;
+                key[j] = keys_in[ic], val[j] = vals_in[ic];
+            }
+        } else {
+#pragma unroll
+            for (int j = 0; j < kKeysPerThread; ++j) {
+                const int64_t i = wbase + j * kWave + lane;
+                key[j] = src(i < n ? i : n - 1), val[j] = (int32_t)i;
+            }
+        }
+    }
 #pragma unroll
     for (int j = 0; j < kKeysPerThread; ++j) {
         const int64_t i = wbase + j * kWave + lane;
         const bool ok = i < n;
-        key[j] = ok ? (keys_in ? keys_in[i] : load_key(parts, i)) : 0u;
-        val[j] = ok ? (vals_in ? vals_in[i] : (int32_t)i) : 0;
         const uint32_t dg = (key[j] >> shift) & mask;
         uint64_t peers = __ballot(ok);
         for (int bit = 0; bit < digit_bits; ++bit) {
