@@ -320,7 +320,9 @@ __device__ __forceinline__ void bwd_tile_body(const TileArgs &a, int lid, float 
                         const float ur = OWNER_POS ? o0p[e] - lvp[e] : lvp[e] - o0p[e];
                         const float ui = OWNER_POS ? o1p[e] - lv1p[e] : lv1p[e] - o1p[e];
                         const float m2 = fmaf(ur, ur, ui * ui);
-                        const float rs = m2 > 0.0f ? __builtin_amdgcn_rsqf(m2) : 0.0f;
+                        // u == 0 contributes k * 0 = 0 whatever k is: clamping m2 away from zero (one max)
+                        // replaces the compare-and-select that would force rs = 0 there
+                        const float rs = __builtin_amdgcn_rsqf(fmaxf(m2, 1e-37f));
                         const float k = OWNER_POS ? -g * rs : g * rs;  // d/da = -g u/|u| ; d/dt' = +g u/|u|
                         a0p[e] = fmaf(k, ur, a0p[e]);
                         a1p[e] = fmaf(k, ui, a1p[e]);
