@@ -1,0 +1,58 @@
+"""A few complete training steps -- sampler, scores, margin loss, sparse gradients, optimizer -- on the
+GPU and with the oracle, from the same start: the tables must stay together, and every update must lower
+the loss of the batch it was computed on."""
+import numpy as np
+import pytest
+import torch
+
+from cuke_amd import synth
+from helpers import assert_close
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.mark.parametrize("model,p", [("DistMult", 2), ("TransE", 2), ("RotatE", 2)])
+@pytest.mark.parametrize("opt", ["sgd", "adagrad"])
+def test_training_steps_track_the_oracle(oracle, model, p, opt):
+    from cuke_amd.data import TrainSampler
+    from cuke_amd.kge import KGEModel, margin_loss, sparse_adagrad, sparse_sgd
+    w = synth.custom_workload(model, n_ent=300, n_rel=7, dim=32, batch=2048, norm_p=p, sigma=0.3, gamma=6.0, seed=3)
+    a = w.arrays
+    dev = torch.device("cuda:0")
+    E, R = torch.from_numpy(a["E"]).to(dev), torch.from_numpy(a["R"]).to(dev)
+    Eo, Ro = a["E"].copy(), a["R"].copy()
+    sE, sR = torch.zeros(E.shape[0], device=dev), torch.zeros(R.shape[0], device=dev)
+    sEo, sRo = np.zeros(E.shape[0], np.float32), np.zeros(R.shape[0], np.float32)
+    m = KGEModel(model, E, R, norm_p=p, gamma=w.gamma)
+    sampler = TrainSampler((a["h"], a["r"], a["t"]), w.n_ent, batch_size=128, neg_sample_size=16, neg_chunk_size=32,
+                           seed=5, mode="both")
+    sign = 1.0 if model in ("DistMult", "RotatE") else -1.0  # distances: smaller is better
+    lr, losses = 0.05, []
+    for step in range(6):
+        h, r, t, neg = next(sampler)
+        mode = sampler.neg_mode
+        fw = m.score(h, r, t, neg, chunk=32, neg_mode=mode)
+        loss, dpos, dneg = margin_loss(fw.pos, fw.neg, margin=1.0, sign=sign)
+        g = m.backward(fw, dpos, dneg)
+        if opt == "sgd":
+            sparse_sgd(E, fw.ent_insp, g.ent_rows, lr), sparse_sgd(R, fw.rel_insp, g.rel_rows, lr)
+        else:
+            sparse_adagrad(E, sE, fw.ent_insp, g.ent_rows, lr)
+            sparse_adagrad(R, sR, fw.rel_insp, g.rel_rows, lr)
+        again = m.score(h, r, t, neg, chunk=32, neg_mode=mode)
+        after, _, _ = margin_loss(again.pos, again.neg, margin=1.0, sign=sign)
+        losses.append((float(loss), float(after)))
+        # the same step with the oracle on its own copies
+        hn, rn, tn, nn = (x.cpu().numpy() for x in (h, r, t, neg))
+        pos, negs = oracle.score(model, Eo, Ro, None, hn, rn, tn, nn, 32, p=p, gamma=w.gamma, neg_mode=mode)
+        lo, dpo, dno = oracle.margin_loss(pos, negs, 1.0, sign)
+        go = oracle.backward(model, Eo, Ro, None, hn, rn, tn, nn, 32, dpo, dno, p=p, neg_mode=mode)
+        if opt == "sgd":
+            Eo, Ro = oracle.sparse_sgd(Eo, go.ent_ids, go.ent_rows, lr), oracle.sparse_sgd(Ro, go.rel_ids, go.rel_rows, lr)
+        else:
+            Eo, sEo = oracle.sparse_adagrad(Eo, sEo, go.ent_ids, go.ent_rows, lr)
+            Ro, sRo = oracle.sparse_adagrad(Ro, sRo, go.rel_ids, go.rel_rows, lr)
+        assert abs(float(loss) - lo) <= 1e-5 * max(1.0, abs(lo)), (step, float(loss), lo)
+    assert_close(E.cpu().numpy(), Eo, rtol=1e-4, what=f"{model} {opt} entity table after 6 steps")
+    assert_close(R.cpu().numpy(), Ro, rtol=1e-4, what=f"{model} {opt} relation table after 6 steps")
+    assert all(after < before for before, after in losses), losses
