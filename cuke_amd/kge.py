@@ -13,6 +13,7 @@ of libkge_mi355.so reached through the C ABI.
 """
 from __future__ import annotations
 
+import collections
 import ctypes as C
 from dataclasses import dataclass
 
@@ -407,6 +408,10 @@ def inspector(r: torch.Tensor, rel_num: int, C_: int = 16):
     return uniq, buf, cnt
 
 
+class _InspSet:
+    """Per-batch state of a TrainStep: index tensors, both inspections, their jobs and events."""
+
+
 class TrainStep:
     """One forward + backward pass over a fixed-shape batch with every buffer allocated up front.
 
@@ -417,6 +422,8 @@ class TrainStep:
     loss = "margin": margin-ranking loss with ``margin`` and ``sign``
     """
 
+    kPipelineSets = 3  # one running, one being inspected, one being refilled
+
     def __init__(self, model: KGEModel, h, r, t, neg=None, chunk=None, loss="sum", margin=1.0,
                  sign=1.0, dpos=None, dneg=None, neg_mode="tail"):
         self.m = model
@@ -425,40 +432,20 @@ class TrainStep:
         f32 = dict(dtype=torch.float32, device=dev)
         i32 = dict(dtype=torch.int32, device=dev)
         _, (h, r, t, neg, C_, N) = model._batch(h, r, t, neg, chunk, neg_mode=neg_mode)
-        self.idx = (h, r, t, neg)
+        idx0 = (h, r, t, neg)
         B = self.B = int(h.numel())
         self.N, self.C = N, C_
         self.loss_kind, self.margin, self.sign = loss, float(margin), float(sign)
 
-        def make_insp(n, n_rows):
-            ins = Inspection(n, n_rows, torch.zeros(1, **i32), torch.empty(max(n, 1), dtype=torch.int64, device=dev),
-                             torch.empty(n + 1, **i32), torch.empty(max(n, 1), **i32),
-                             torch.empty(max(n, 1), **i32), torch.empty(max(n, 1), **i32))
-            ins._c = _lib.Inspection(n, n_rows, ins.num_unique_dev.data_ptr(), ins.unique_ids.data_ptr(),
-                                     ins.seg_offsets.data_ptr(), ins.perm.data_ptr(), ins.inverse.data_ptr(),
-                                     ins.sorted_seg.data_ptr())
-            ws = torch.empty(max(int(L.kge_inspect_workspace(n, n_rows)), 1), dtype=torch.uint8, device=dev)
-            return ins, ws
-
-        parts = [h, t] + ([neg] if neg is not None else [])
-        n_occ = sum(int(p.numel()) for p in parts)
-        self.ent_insp, self._ws_e = make_insp(n_occ, int(model.E.shape[0]))
-        self.rel_insp, self._ws_r = make_insp(B, max(model.n_rel, 1))
-        jobs = (_lib.InspectJob * 2)()
-        for job, ps, ins, ws in ((jobs[0], parts, self.ent_insp, self._ws_e), (jobs[1], [r], self.rel_insp, self._ws_r)):
-            for q, p_ in enumerate(ps):
-                job.parts[q], job.part_len[q] = p_.data_ptr(), int(p_.numel())
-            job.n_parts, job.n_rows, job.out = len(ps), ins.n_rows, ins._c
-            job.workspace, job.workspace_bytes = ws.data_ptr(), ws.numel()
-        self._jobs = jobs
+        self._parts = lambda ix: [ix[0], ix[2]] + ([ix[3]] if ix[3] is not None else [])
+        self.n_occ = n_occ = sum(int(p.numel()) for p in self._parts(idx0))
+        self._neg_mode = neg_mode
         # forward-only scoring needs no inspection unless the relation groups drive TransR / RESCAL
         self.needs_rel_groups = model.model in ("TransR", "RESCAL")
-
-        self.bat = _lib.Batch(B, h.data_ptr(), r.data_ptr(), t.data_ptr(),
-                              neg.data_ptr() if neg is not None else None, C_, N,
-                              C.pointer(self.ent_insp._c), C.pointer(self.rel_insp._c), None, NEG_MODES[neg_mode], 0)
+        self._sets = [self._make_set(idx0)]
+        self._cur = 0
+        self._staged, self._stage_at = collections.deque(), 0
         self.side = torch.cuda.Stream(device=dev)  # default priority
-        self.insp_event = torch.cuda.Event()
         self.pos = torch.empty(B, **f32)
         self.neg = torch.empty((B, N), **f32) if neg is not None else None
         self.side_pos = torch.empty(B, **f32) if model.model == "TransH" else None
@@ -490,6 +477,49 @@ class TrainStep:
         self._ws_b = torch.empty(max(self._ws_b_bytes, 1), dtype=torch.uint8, device=dev)
         self.graph = None
 
+    def _make_set(self, idx):
+        """Index tensors plus everything the inspector writes for them: one set per batch in flight."""
+        m, L, dev = self.m, self.L, self.m.dev
+        i32 = dict(dtype=torch.int32, device=dev)
+        h, r, t, neg = idx
+
+        def make_insp(n, n_rows):
+            ins = Inspection(n, n_rows, torch.zeros(1, **i32), torch.empty(max(n, 1), dtype=torch.int64, device=dev),
+                             torch.empty(n + 1, **i32), torch.empty(max(n, 1), **i32),
+                             torch.empty(max(n, 1), **i32), torch.empty(max(n, 1), **i32))
+            ins._c = _lib.Inspection(n, n_rows, ins.num_unique_dev.data_ptr(), ins.unique_ids.data_ptr(),
+                                     ins.seg_offsets.data_ptr(), ins.perm.data_ptr(), ins.inverse.data_ptr(),
+                                     ins.sorted_seg.data_ptr())
+            ws = torch.empty(max(int(L.kge_inspect_workspace(n, n_rows)), 1), dtype=torch.uint8, device=dev)
+            return ins, ws
+
+        s = _InspSet()
+        s.idx = idx
+        parts = self._parts(idx)
+        s.ent_insp, s.ws_e = make_insp(self.n_occ, int(m.E.shape[0]))
+        s.rel_insp, s.ws_r = make_insp(self.B, max(m.n_rel, 1))
+        s.jobs = (_lib.InspectJob * 2)()
+        for job, ps, ins, ws in ((s.jobs[0], parts, s.ent_insp, s.ws_e), (s.jobs[1], [r], s.rel_insp, s.ws_r)):
+            for q, p_ in enumerate(ps):
+                job.parts[q], job.part_len[q] = p_.data_ptr(), int(p_.numel())
+            job.n_parts, job.n_rows, job.out = len(ps), ins.n_rows, ins._c
+            job.workspace, job.workspace_bytes = ws.data_ptr(), ws.numel()
+        s.bat = _lib.Batch(self.B, h.data_ptr(), r.data_ptr(), t.data_ptr(),
+                           neg.data_ptr() if neg is not None else None, self.C, self.N,
+                           C.pointer(s.ent_insp._c), C.pointer(s.rel_insp._c), None, NEG_MODES[self._neg_mode], 0)
+        s.insp_event = torch.cuda.Event()
+        s.done_event = None  # recorded on the main stream after the last pipelined step that used this set
+        s.inputs_ready = None
+        return s
+
+    # the set of the step enqueued last (the only set unless run(pipeline=True) is used)
+    idx = property(lambda self: self._sets[self._cur].idx)
+    ent_insp = property(lambda self: self._sets[self._cur].ent_insp)
+    rel_insp = property(lambda self: self._sets[self._cur].rel_insp)
+    bat = property(lambda self: self._sets[self._cur].bat)
+    _jobs = property(lambda self: self._sets[self._cur].jobs)
+    insp_event = property(lambda self: self._sets[self._cur].insp_event)
+
     # the individual stages, each one C call
     def inspect(self, st, backward=True):
         """Both inspections in one call; forward-only steps inspect r alone, and only if needed."""
@@ -514,11 +544,62 @@ class TrainStep:
                                         _ptr(self.dpos), _ptr(self.dneg), C.byref(self.grads), _ptr(self._ws_b),
                                         self._ws_b_bytes, st), "kge_score_bwd")
 
-    def run(self, backward=True, overlap=True):
+    # ---- pipelined issue: index tensors and inspections in a ring of sets ----
+    def _ring(self):
+        """Grow to kPipelineSets sets on first use (copies of the construction-time indices)."""
+        if len(self._sets) < self.kPipelineSets:
+            first = self._sets[0].idx
+            while len(self._sets) < self.kPipelineSets:
+                self._sets.append(self._make_set(tuple(x.clone() if x is not None else None for x in first)))
+            torch.cuda.current_stream().synchronize()  # once: the copies are read from other streams
+            self._stage_at = (self._cur + 1) % len(self._sets)
+        return self._sets
+
+    def next_inputs(self, stream=None):
+        """The index tensors (h, r, t, neg) that the next ``stage()`` will hand to the inspector.
+        ``stream`` (default: the current one) is made to wait until the last step that read them has
+        finished, so the caller can refill them in place on that stream."""
+        nxt = self._ring()[self._stage_at]
+        if nxt.done_event is not None:
+            (stream or torch.cuda.current_stream()).wait_event(nxt.done_event)
+        return nxt.idx
+
+    def stage(self, inputs_ready=None):
+        """Declare the tensors of ``next_inputs()`` final -- complete once ``inputs_ready`` (a
+        torch.cuda.Event; None = already complete) has fired -- and start their inspection on the
+        side stream.  ``run(pipeline=True)`` consumes staged batches oldest first.  Staging one
+        batch ahead of the step that is about to run lets the inspector finish before backward asks
+        for it, which also keeps the host off the slow path of waiting on a pending event."""
+        sets = self._ring()
+        at = self._stage_at
+        if len(self._staged) >= len(sets) - 1:
+            raise KgeError(f"at most {len(sets) - 1} batches can be staged ahead of run()")
+        s, side = sets[at], self.side
+        if s.done_event is not None:
+            side.wait_event(s.done_event)  # its inspection may still be read by an earlier step
+        if inputs_ready is not None:
+            side.wait_event(inputs_ready)
+        s.inputs_ready = inputs_ready
+        sst = C.c_void_p(side.cuda_stream)
+        if self.needs_rel_groups:  # the relation groups drive the forward pass: inspected in run()
+            _lib.check(self.L.kge_inspect_batch(C.byref(s.jobs[0]), 1, sst), "kge_inspect_batch(entities)")
+        else:
+            _lib.check(self.L.kge_inspect_batch(s.jobs, 2, sst), "kge_inspect_batch")
+        s.insp_event.record(side)
+        self._staged.append(at)
+        self._stage_at = (at + 1) % len(sets)
+
+    def run(self, backward=True, overlap=True, pipeline=False, inputs_ready=None):
         """Enqueue one step.  With overlap (default) the inspector runs on a side stream while
         the main stream computes scores and per-occurrence gradients; backward waits for it
         right before its segmented reduction.  TransR / RESCAL need the relation groups in the
-        forward pass, so their relation inspection stays on the main stream."""
+        forward pass, so their relation inspection stays on the main stream.
+
+        pipeline=True runs the oldest batch handed over with ``stage()`` (staging the tensors of
+        ``next_inputs()`` first, with ``inputs_ready``, if none is waiting).  Index tensors and
+        inspections live in a ring of sets, so the side stream never waits for the step before.
+        Results (``sparse_grads()``, ``pos`` ...) are those of the step enqueued last.  Not
+        capturable into one graph: the dependencies cross steps."""
         main = torch.cuda.current_stream()
         st = C.c_void_p(main.cuda_stream)
         if not (backward and overlap):
@@ -529,19 +610,35 @@ class TrainStep:
                 self.loss_grad(st)
                 self.backward(st)
             return
-        side = self.side
-        sst = C.c_void_p(side.cuda_stream)
-        side.wait_stream(main)
-        if self.needs_rel_groups:
-            _lib.check(self.L.kge_inspect_batch(C.byref(self._jobs[1]), 1, st), "kge_inspect_batch(relations)")
-            _lib.check(self.L.kge_inspect_batch(C.byref(self._jobs[0]), 1, sst), "kge_inspect_batch(entities)")
+        if pipeline:
+            if not self._staged:
+                self.stage(inputs_ready)
+            self._cur = self._staged.popleft()
+            cur = self._sets[self._cur]
+            if cur.inputs_ready is not None:
+                main.wait_event(cur.inputs_ready)  # the score kernels read the index tensors too
+            if self.needs_rel_groups:
+                _lib.check(self.L.kge_inspect_batch(C.byref(cur.jobs[1]), 1, st), "kge_inspect_batch(relations)")
         else:
-            _lib.check(self.L.kge_inspect_batch(self._jobs, 2, sst), "kge_inspect_batch")
-        self.insp_event.record(side)
-        self.bat.insp_ready = self.insp_event.cuda_event
+            if self._staged:
+                raise KgeError("staged batches are waiting: use run(pipeline=True)")
+            cur, side = self._sets[self._cur], self.side
+            sst = C.c_void_p(side.cuda_stream)
+            side.wait_stream(main)
+            if self.needs_rel_groups:
+                _lib.check(self.L.kge_inspect_batch(C.byref(cur.jobs[1]), 1, st), "kge_inspect_batch(relations)")
+                _lib.check(self.L.kge_inspect_batch(C.byref(cur.jobs[0]), 1, sst), "kge_inspect_batch(entities)")
+            else:
+                _lib.check(self.L.kge_inspect_batch(cur.jobs, 2, sst), "kge_inspect_batch")
+            cur.insp_event.record(side)
+        cur.bat.insp_ready = cur.insp_event.cuda_event
         self.forward(st)
         self.loss_grad(st)
         self.backward(st)
+        if pipeline or (len(self._sets) > 1 and not torch.cuda.is_current_stream_capturing()):
+            if cur.done_event is None:
+                cur.done_event = torch.cuda.Event()
+            cur.done_event.record(main)
 
     def capture(self, backward=True):
         """Record run() into a HIP graph; replay() then launches the whole step at once."""

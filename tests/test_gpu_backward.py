@@ -164,3 +164,77 @@ def test_train_step_eager_overlapped_and_graph_replays(oracle, name, over):
     for i in range(3):
         step.replay()
         check(f"graph replay {i}")
+
+
+@pytest.mark.parametrize("name,over", [
+    ("cfg2_distmult", dict(n_ent=50_000, batch=512)),
+    ("cfg4_rotate", dict(batch=256)),
+    ("cfg3_transr", dict(batch=1024)),
+    # L1 norm: lattice-valued tables keep every residual element away from the sign ambiguity at zero
+    ("cfg5_transh", dict(n_ent=20_000, batch=512, n_neg=64, chunk=64, lattice=True)),
+])
+@pytest.mark.parametrize("ahead", [0, 1])
+def test_train_step_pipelined_inspections(oracle, name, over, ahead):
+    """run(pipeline=True): index tensors and inspections live in a ring of sets, so the inspector of a
+    batch overlaps the steps before it.  Six steps are enqueued without any synchronisation, each on new
+    indices that a loader stream writes into next_inputs() and hands over with stage() -- `ahead` batches
+    before the step that consumes them -- and each step's gradients are copied out on the main stream.
+    After one synchronisation at the end every step must match the oracle on its own batch."""
+    from cuke_amd.kge import SparseGrads, TrainStep
+    w = synth.make_workload(name, **over)
+    a = w.arrays
+    m, ix = gpu_model(w)
+    sign = -1.0 if w.model in ("TransR", "TransH") else 1.0
+    step = TrainStep(m, ix["h"], ix["r"], ix["t"], ix.get("neg"), w.chunk or None, loss=w.loss,
+                     margin=w.margin, sign=sign)
+    rng = np.random.default_rng(11)
+    loader = torch.cuda.Stream()
+    n_steps = 6
+    batches, staged_host, kept = [], [], []
+
+    def hand_over(i):
+        new = {k: rng.integers(0, w.n_rel if k == "r" else w.n_ent, size=a[k].shape).astype(np.int64)
+               for k in ("h", "r", "t", "neg") if a.get(k) is not None}
+        if i == 3:  # a batch with heavy repetition: few distinct rows
+            new = {k: v % 7 for k, v in new.items()}
+        host = {k: torch.from_numpy(v).pin_memory() for k, v in new.items()}
+        with torch.cuda.stream(loader):
+            bufs = dict(zip(("h", "r", "t", "neg"), step.next_inputs(loader)))
+            for k, v in host.items():
+                bufs[k].copy_(v, non_blocking=True)
+            ready = torch.cuda.Event()
+            ready.record(loader)
+        step.stage(ready)
+        batches.append(new)
+        staged_host.append(host)  # pinned buffers stay alive until the copies have run
+
+    for i in range(ahead):
+        hand_over(i)
+    for i in range(n_steps):
+        if i + ahead < n_steps:
+            hand_over(i + ahead)
+        step.run(pipeline=True)
+        ins_e, ins_r = step.ent_insp, step.rel_insp
+        kept.append(dict(ne=ins_e.num_unique_dev.clone(), nr=ins_r.num_unique_dev.clone(),
+                         eid=ins_e.unique_ids.clone(), rid=ins_r.unique_ids.clone(), erows=step.ent_rows.clone(),
+                         rrows=step.rel_rows.clone() if step.rel_rows is not None else None,
+                         arows=step.aux_rows.clone() if step.aux_rows is not None else None,
+                         dpos=step.dpos.clone(), dneg=step.dneg.clone() if step.dneg is not None else None))
+    torch.cuda.synchronize()
+    for i, (new, k) in enumerate(zip(batches, kept)):
+        ref = oracle.backward(w.model, a["E"], a["R"], a["A"], new["h"], new["r"], new["t"], new.get("neg"), w.chunk,
+                              k["dpos"].cpu().numpy(), k["dneg"].cpu().numpy() if k["dneg"] is not None else None,
+                              p=w.norm_p)
+        ue, ur = int(k["ne"]), int(k["nr"])
+        got = SparseGrads(k["eid"][:ue], k["erows"][:ue], k["rid"][:ur],
+                          k["rrows"][:ur] if k["rrows"] is not None else None,
+                          k["arows"][:ur] if k["arows"] is not None else None)
+        compare(got, ref, f"{name} pipelined step {i}", outliers=(1e-5, 4.0) if w.model == "RotatE" else None)
+    # the plain mode still works afterwards, on the set of the step run last
+    step.run()
+    torch.cuda.synchronize()
+    ref = oracle.backward(w.model, a["E"], a["R"], a["A"], batches[-1]["h"], batches[-1]["r"], batches[-1]["t"],
+                          batches[-1].get("neg"), w.chunk, step.dpos.cpu().numpy(),
+                          step.dneg.cpu().numpy() if step.dneg is not None else None, p=w.norm_p)
+    compare(step.sparse_grads(), ref, f"{name} plain run after the pipelined ones",
+            outliers=(1e-5, 4.0) if w.model == "RotatE" else None)
