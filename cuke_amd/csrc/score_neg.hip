@@ -220,11 +220,147 @@ __global__ __launch_bounds__(256, KGE_TILE_OCC) void score_neg_kernel(NegArgs a)
     }
 }
 
+// DistMult / ComplEx: the pair scores of a tile are a plain matrix product, query rows (TB x d)
+// times negative rows (TN x d) transposed, so the inner loop runs on the matrix cores
+// (v_mfma_f32_16x16x4_f32, fp32 in, fp32 accumulate).  Staging is the same as above; the four
+// waves tile the workgroup 2 x 2 and each owns (TB/2) x (TN/2) scores as 16 x 16 blocks.
+// Operand layout: lane l supplies A[i = l % 16][k = l / 16] and B[k = l / 16][j = l % 16] and
+// receives D[i = 4 * (l / 16) + v][j = l % 16], v = 0..3.  Inside 16 consecutive k the MFMA step
+// s pairs lane group g = l / 16 with k = 4 g + s (any pairing works as long as both operands use
+// it), so a lane's values for four steps are one 128-bit LDS read of its row.
+typedef float v4f __attribute__((ext_vector_type(4)));
+
+template <int MODEL, int RB, int RK>
+__global__ __launch_bounds__(256, KGE_TILE_OCC) void score_neg_mfma_kernel(NegArgs a)
+{
+    static_assert(MODEL == KGE_DISTMULT || MODEL == KGE_COMPLEX, "dot-product scores only");
+    constexpr int TB = 16 * RB, TN = 16 * RK;
+    constexpr int SB = TB / 32, SN = TN / 32;
+    constexpr int MB = RB / 2, NB = RK / 2;  // 16 x 16 blocks per wave
+    static_assert(TB % 32 == 0 && TN % 32 == 0, "tile rows are staged 32 at a time");
+
+    __shared__ __align__(16) float sA[TB][kLDW];
+    __shared__ __align__(16) float sT[TN][kLDW];
+
+    const int tid = threadIdx.x;
+    const int srow = tid >> 3, scol = (tid & 7) * 4;
+    const int lane = tid & 63, wave = tid >> 6;
+    const int fr = lane & 15, fg = lane >> 4;
+    const int wrow = (wave >> 1) * (TB / 2), wcol = (wave & 1) * (TN / 2);
+    int c, tile_y, tile_x;
+    if (!xcd_tile(blockIdx.x, (a.N + TN - 1) / TN, (a.C + TB - 1) / TB, a.n_chunks, c, tile_y, tile_x)) return;
+    const int bt0 = tile_y * TB, kt0 = tile_x * TN;
+    const int d = a.d, half = d >> 1;
+    const bool vec = a.vec != 0;
+
+    const float *ph[SB], *pr[SB];
+    bool okb[SB];
+#pragma unroll
+    for (int s = 0; s < SB; ++s) {
+        const int bl = bt0 + srow + 32 * s;
+        okb[s] = bl < a.C;
+        const int64_t b = (int64_t)c * a.C + (okb[s] ? bl : a.C - 1);
+        ph[s] = a.ent + a.h[b] * (int64_t)d;
+        pr[s] = a.rel + a.r[b] * (int64_t)a.rel_dim;
+    }
+    const float *pt[SN];
+    bool okk[SN];
+#pragma unroll
+    for (int s = 0; s < SN; ++s) {
+        const int kl = kt0 + srow + 32 * s;
+        okk[s] = kl < a.N;
+        pt[s] = a.ent + a.neg[(int64_t)c * a.N + (okk[s] ? kl : a.N - 1)] * (int64_t)d;
+    }
+
+    float4 ra[SB], rt[SN];
+    auto load_slice_v = [&](auto vtag, int j0) {
+        constexpr bool VEC = decltype(vtag)::value;
+        const int j = j0 + scol;
+#pragma unroll
+        for (int s = 0; s < SB; ++s) {
+            float4 q1;
+            load_query<MODEL, VEC>(ph[s], pr[s], nullptr, 0.0f, j, okb[s] ? d : 0, half, ra[s], q1, nullptr, a.rsign);
+        }
+#pragma unroll
+        for (int s = 0; s < SN; ++s) rt[s] = ld4<VEC>(pt[s], j, okk[s] ? d : 0);
+    };
+    auto load_slice = [&](int j0) {
+        if (vec) load_slice_v(std::true_type{}, j0);
+        else load_slice_v(std::false_type{}, j0);
+    };
+
+    // two accumulators per block (one per half of the slice) keep consecutive MFMAs independent
+    v4f acc[2][MB][NB];
+#pragma unroll
+    for (int g = 0; g < 2; ++g)
+#pragma unroll
+        for (int m = 0; m < MB; ++m)
+#pragma unroll
+            for (int n = 0; n < NB; ++n) acc[g][m][n] = v4f{0.0f, 0.0f, 0.0f, 0.0f};
+
+    const int nslice = (d + kKD - 1) / kKD;
+    load_slice(0);
+#pragma unroll 1
+    for (int s = 0; s < nslice; ++s) {
+#pragma unroll
+        for (int q = 0; q < SB; ++q) *reinterpret_cast<float4 *>(&sA[srow + 32 * q][scol]) = ra[q];
+#pragma unroll
+        for (int q = 0; q < SN; ++q) *reinterpret_cast<float4 *>(&sT[srow + 32 * q][scol]) = rt[q];
+        __syncthreads();
+        if (s + 1 < nslice) load_slice((s + 1) * kKD);
+#pragma unroll
+        for (int g = 0; g < kKD / 16; ++g) {
+            float4 av[MB], tv[NB];
+#pragma unroll
+            for (int m = 0; m < MB; ++m)
+                av[m] = *reinterpret_cast<const float4 *>(&sA[wrow + 16 * m + fr][16 * g + 4 * fg]);
+#pragma unroll
+            for (int n = 0; n < NB; ++n)
+                tv[n] = *reinterpret_cast<const float4 *>(&sT[wcol + 16 * n + fr][16 * g + 4 * fg]);
+#pragma unroll
+            for (int e = 0; e < 4; ++e)
+#pragma unroll
+                for (int m = 0; m < MB; ++m)
+#pragma unroll
+                    for (int n = 0; n < NB; ++n) {
+                        const float x = e == 0 ? av[m].x : e == 1 ? av[m].y : e == 2 ? av[m].z : av[m].w;
+                        const float y = e == 0 ? tv[n].x : e == 1 ? tv[n].y : e == 2 ? tv[n].z : tv[n].w;
+                        acc[g & 1][m][n] = __builtin_amdgcn_mfma_f32_16x16x4f32(x, y, acc[g & 1][m][n], 0, 0, 0);
+                    }
+        }
+        __syncthreads();
+    }
+
+#pragma unroll
+    for (int m = 0; m < MB; ++m)
+#pragma unroll
+        for (int v = 0; v < 4; ++v) {
+            const int bl = bt0 + wrow + 16 * m + 4 * fg + v;
+            if (bl >= a.C) continue;
+            const int64_t rowoff = ((int64_t)c * a.C + bl) * a.N;
+#pragma unroll
+            for (int n = 0; n < NB; ++n) {
+                const int kl = kt0 + wcol + 16 * n + fr;
+                if (kl < a.N) a.out[rowoff + kl] = acc[0][m][n][v] + acc[1][m][n][v];
+            }
+        }
+}
+
 // 0: choose by size, 2: 32x32 tiles, 3: 32x64, 4: 64x64 (development knob)
 static int neg_tile_override()
 {
     static const int v = [] {
         const char *e = getenv("KGE_NEG_TILE");
+        return e ? atoi(e) : 0;
+    }();
+    return v;
+}
+
+// 1: keep DistMult / ComplEx on the vector ALUs (development knob)
+static int neg_valu_override()
+{
+    static const int v = [] {
+        const char *e = getenv("KGE_NEG_VALU");
         return e ? atoi(e) : 0;
     }();
     return v;
@@ -240,6 +376,22 @@ static int launch_neg_mp(const NegArgs &a, int64_t n_chunks, hipStream_t st)
     // starve an inspection running next to it on another stream; the inspector kernels raise their
     // wave priority for that reason.
     if (tile != 2 && tile != 4 && tile != 3) tile = big_tiles >= 1024 ? 4 : 2;
+    if constexpr (MODEL == KGE_DISTMULT || MODEL == KGE_COMPLEX) {
+        if (!neg_valu_override()) {
+            if (tile == 4) {
+                const dim3 grid(xcd_grid(ceil_div(a.N, 64), ceil_div(a.C, 64), n_chunks));
+                hipLaunchKernelGGL((score_neg_mfma_kernel<MODEL, 4, 4>), grid, dim3(256), 0, st, a);
+            } else if (tile == 3) {
+                const dim3 grid(xcd_grid(ceil_div(a.N, 64), ceil_div(a.C, 32), n_chunks));
+                hipLaunchKernelGGL((score_neg_mfma_kernel<MODEL, 2, 4>), grid, dim3(256), 0, st, a);
+            } else {
+                const dim3 grid(xcd_grid(ceil_div(a.N, 32), ceil_div(a.C, 32), n_chunks));
+                hipLaunchKernelGGL((score_neg_mfma_kernel<MODEL, 2, 2>), grid, dim3(256), 0, st, a);
+            }
+            KGE_CHECK_LAUNCH();
+            return KGE_OK;
+        }
+    }
     if (tile == 3) {  // 32 positives x 64 negatives
         const dim3 grid(xcd_grid(ceil_div(a.N, 64), ceil_div(a.C, 32), n_chunks));
         if (MODEL == KGE_TRANSH && a.side_neg)
