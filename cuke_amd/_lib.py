@@ -42,7 +42,8 @@ class Batch(C.Structure):
     _fields_ = [("batch", C.c_int64), ("h", C.c_void_p), ("r", C.c_void_p), ("t", C.c_void_p),
                 ("neg", C.c_void_p), ("chunk", C.c_int64), ("n_neg", C.c_int64),
                 ("ent_insp", C.POINTER(Inspection)), ("rel_insp", C.POINTER(Inspection)),
-                ("insp_ready", C.c_void_p), ("neg_mode", C.c_int32), ("reserved", C.c_int32)]
+                ("insp_ready", C.c_void_p), ("neg_mode", C.c_int32), ("fuse_inspection", C.c_int32),
+                ("insp_jobs", C.c_void_p)]
 
 
 class Saved(C.Structure):
@@ -67,6 +68,7 @@ EXPORTS = {
     "kge_inspect": (C.c_int, [C.POINTER(C.c_void_p), C.POINTER(C.c_int64), C.c_int, C.c_int64,
                               C.POINTER(Inspection), C.c_void_p, C.c_size_t, C.c_void_p]),
     "kge_inspect_batch": (C.c_int, [C.POINTER(InspectJob), C.c_int, C.c_void_p]),
+    "kge_fused_inspection_ok": (C.c_int, [C.POINTER(Tables), C.POINTER(Batch), C.POINTER(InspectJob)]),
     "kge_margin_loss_workspace": (C.c_size_t, [C.c_int64, C.c_int64]),
     "kge_margin_loss": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int64, C.c_int64, C.c_float,
                                   C.c_float, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p,
@@ -88,7 +90,7 @@ EXPORTS = {
 _lib = None
 
 
-ABI_VERSION = 2  # layout of the ctypes structures above; must match kge_abi_version()
+ABI_VERSION = 3  # layout of the ctypes structures above; must match kge_abi_version()
 
 
 def lib() -> C.CDLL:

@@ -1,10 +1,12 @@
 // extern "C" entry points: argument validation and kernel dispatch.
-#include "common.hpp"
+#include "inspector_mid.hpp"
 
 namespace kge {
 int launch_score_pos(const kge_tables *, const kge_batch *, float *, float *, float *, hipStream_t);
+int launch_score_pos_fused(const kge_tables *, const kge_batch *, float *, float *, float *, const FusedInsp *,
+                           hipStream_t);
 int launch_score_neg(const kge_tables *, const kge_batch *, const float *, const float *, float *, float *,
-                     hipStream_t);
+                     const FusedInsp *, hipStream_t);
 int launch_transr_fwd(const kge_tables *, const kge_batch *, float *, float *, void *, size_t, hipStream_t);
 size_t transr_fwd_workspace(const kge_tables *, const kge_batch *);
 
@@ -96,7 +98,7 @@ const char *kge_strerror(int status)
     }
 }
 
-int kge_abi_version(void) { return 2; }
+int kge_abi_version(void) { return 3; }
 
 size_t kge_score_fwd_workspace(const kge_tables *tab, const kge_batch *bat)
 {
@@ -130,15 +132,24 @@ int kge_score_fwd(const kge_tables *tab, const kge_batch *bat, float *pos, float
     const bool want_neg = neg && bat->neg;
     if (want_neg && tab->model == KGE_TRANSH && !side_pos) return KGE_EINVAL;
     if (want_neg && tab->model == KGE_ROTATE && !residual) return KGE_EINVAL;  // rotated heads buffer
+    // fused inspection: first digit pass with the per-positive kernel, second with the tile kernel
+    const bool fuse = bat->fuse_inspection != 0;
+    FusedInsp fi0{}, fi1{};
+    if (fuse) {
+        if (!want_neg || !bat->insp_jobs || !(pos || side_pos || residual) || bat->batch == 0) return KGE_EINVAL;
+        if ((rc = plan_fused_inspection(bat->insp_jobs, 0, &fi0))) return rc;
+        if ((rc = plan_fused_inspection(bat->insp_jobs, 1, &fi1))) return rc;
+    }
     if (pos || side_pos || residual) {
         if ((tab->model == KGE_TRANSR || tab->model == KGE_RESCAL) && bat->rel_insp)
             rc = launch_transr_fwd(tab, bat, pos, residual, workspace, workspace_bytes, st);
         else
-            rc = launch_score_pos(tab, bat, pos, residual, side_pos, st);
+            rc = launch_score_pos_fused(tab, bat, pos, residual, side_pos, fuse ? &fi0 : nullptr, st);
         if (rc) return rc;
     }
     if (want_neg)
-        return launch_score_neg(tab, bat, side_pos, tab->model == KGE_ROTATE ? residual : nullptr, neg, side_neg, st);
+        return launch_score_neg(tab, bat, side_pos, tab->model == KGE_ROTATE ? residual : nullptr, neg, side_neg,
+                                fuse ? &fi1 : nullptr, st);
     return KGE_OK;
 }
 

@@ -9,51 +9,15 @@
 // histogram -> column scan -> stable scatter.  Stability inside a block comes from
 // wave-level peer matching (ballots), not from atomics, so the result is
 // deterministic and equals a stable argsort.
-#include "common.hpp"
+#include "inspector_mid.hpp"
 
 namespace kge {
 
-constexpr int kSortThreads = 256;
 constexpr int kSortWaves = kSortThreads / kWave;
 constexpr int kKeysPerThread = 8;
 constexpr int kKeysPerBlock = kSortThreads * kKeysPerThread;  // 2048
-constexpr int kMaxDigitBits = 11;
-constexpr int kMaxBins = 1 << kMaxDigitBits;
 constexpr int kFusedScanBlocks = 32;  // up to this many blocks the scatter kernel scans the
                                       // histogram columns itself (one launch less per pass)
-
-struct Parts {
-    const int64_t *p[4];
-    int64_t end[4];  // exclusive end offset of each part in the concatenation
-    int n_parts;
-};
-
-// Key i of the concatenation, with the part table held in registers and the index clamped by the caller: the load
-// is unconditional (a branch or a select around a load makes the compiler wait for it on the
-// spot, which serialises a batch of loads into one memory round trip each).
-struct KeySrc {
-    // byte address of key i = base_k + 8 i for the part k that holds position i; the bases are
-    // plain integers so that the choice is a per-lane select (choosing among pointer VALUES makes
-    // the compiler loop over the distinct pointers of a wave, one waited load per turn)
-    uint64_t b0, b1, b2, b3;
-    int64_t e0, e1, e2;
-    __device__ explicit KeySrc(const Parts &parts)
-        : e0(parts.end[0]), e1(parts.end[1]), e2(parts.end[2])
-    {
-        b0 = reinterpret_cast<uint64_t>(parts.p[0]);
-        b1 = reinterpret_cast<uint64_t>(parts.p[1]) - 8u * (uint64_t)e0;
-        b2 = reinterpret_cast<uint64_t>(parts.p[2]) - 8u * (uint64_t)e1;
-        b3 = reinterpret_cast<uint64_t>(parts.p[3]) - 8u * (uint64_t)e2;
-    }
-    __device__ __forceinline__ uint32_t operator()(int64_t i) const  // i must be a valid position
-    {
-        const uint64_t base = i < e0 ? b0 : (i < e1 ? b1 : (i < e2 ? b2 : b3));
-        // low word of the int64 id; the address-space-1 pointer makes this a global (not flat) load,
-        // which leaves the LDS counter alone so that the histogram atomics need not drain per key
-        typedef const uint32_t __attribute__((address_space(1))) *global_u32;
-        return *reinterpret_cast<global_u32>(base + 8u * (uint64_t)i);
-    }
-};
 
 // ---- pass step 1: per-block digit histogram --------------------------------------------
 __global__ __launch_bounds__(kSortThreads) void radix_hist_kernel(Parts parts, const uint32_t *keys_in,
@@ -102,36 +66,6 @@ __global__ void radix_colscan_kernel(uint32_t *hist, uint32_t *totals, int bins,
         run += v;
     }
     totals[bin] = run;
-}
-
-// exclusive scan of s[0..bins) in place (bins <= 2048, 256 threads)
-__device__ void block_exclusive_scan(uint32_t *s, int bins, uint32_t *wave_tot)
-{
-    const int per = (bins + kSortThreads - 1) / kSortThreads;  // <= 8
-    const int lo = threadIdx.x * per;
-    uint32_t loc[kMaxBins / kSortThreads];
-    uint32_t sum = 0;
-    for (int i = 0; i < per; ++i) {
-        const uint32_t v = lo + i < bins ? s[lo + i] : 0;
-        loc[i] = sum;
-        sum += v;
-    }
-    // inclusive scan of `sum` across the wave, then across the waves
-    const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x >> 6;
-    uint32_t inc = sum;
-#pragma unroll
-    for (int o = 1; o < kWave; o <<= 1) {
-        const uint32_t up = __shfl_up(inc, o, kWave);
-        if (lane >= o) inc += up;
-    }
-    if (lane == kWave - 1) wave_tot[wave] = inc;
-    __syncthreads();
-    uint32_t woff = 0;
-    for (int w = 0; w < wave; ++w) woff += wave_tot[w];
-    const uint32_t excl = woff + inc - sum;
-    for (int i = 0; i < per; ++i)
-        if (lo + i < bins) s[lo + i] = excl + loc[i];
-    __syncthreads();
 }
 
 // ---- pass step 3: stable scatter ---------------------------------------------------------
@@ -333,225 +267,24 @@ __global__ __launch_bounds__(kSortThreads) void finalize_kernel(const uint32_t *
     }
 }
 
-// ---- small and medium inputs: one launch per digit pass ------------------------------------
-// Up to 65536 ids.  A block owns 1024 consecutive keys.  Instead of a separate histogram
-// kernel and scan, every block counts the digits of ALL keys itself (LDS atomics; the keys are
-// a few hundred KB at most and sit in L2), which gives it the global bin starts and the number
-// of same-digit keys in the blocks before it; it then ranks its own keys stably with wave
-// ballots and scatters them.  A pass is therefore ONE launch with no inter-block dependency,
-// the dedup a second one that counts the run heads before the block the same way.  Several
-// index sets share the launches (blockIdx.y).
-constexpr int kMidThreads = 256;
-constexpr int kMidWaves = kMidThreads / kWave;
-constexpr int kMidKeys = 1024;  // keys per block: 4 rounds of 64 per wave
-constexpr int kMidRounds = kMidKeys / kMidThreads;
-constexpr int64_t kMidMaxN = 65536;
-
-struct MidJob {
-    Parts parts;
-    int64_t n;
-    int npass, db;
-    kge_inspection out;
-    uint32_t *keys_final, *keys_tmp;
-    int32_t *vals_tmp;
-};
-struct MidJobs {
-    MidJob j[4];
-};
+// ---- small and medium inputs: the mid-path bodies as kernels of their own -------------------
+__global__ __launch_bounds__(kMidThreads) void inspect_mid_hist_kernel(MidJobs jobs)
+{
+    __shared__ uint32_t smem[kMaxBins];
+    mid_hist_body(jobs.j[blockIdx.y], blockIdx.x, smem);
+}
 
 template <bool FIRST>
-__global__ __launch_bounds__(kMidThreads) void inspect_mid_pass_kernel(MidJobs jobs, int pass)
+__global__ __launch_bounds__(kMidThreads) void inspect_mid_scatter_kernel(MidJobs jobs, int pass)
 {
-    __shared__ uint32_t s_tot[kMaxBins];             // digit totals -> global bin starts
-    __shared__ uint32_t s_bef[kMaxBins];             // same digit, earlier blocks
-    __shared__ uint32_t s_cnt[kMidWaves][kMaxBins];  // per-wave running counts
-    __shared__ uint32_t s_w[kMidWaves];
-    // The inspection usually runs on its own stream next to the score kernels, whose waves fill
-    // every SIMD; without a raised wave priority these few workgroups get a fraction of the issue
-    // slots and the step waits for them at the join.
-    __builtin_amdgcn_s_setprio(3);
-    const MidJob &J = jobs.j[blockIdx.y];
-    const int n = (int)J.n;
-    if (pass >= J.npass || (int)blockIdx.x * kMidKeys >= n) return;
-    const int tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid >> 6;
-    const int bins = 1 << J.db;
-    const uint32_t mask = (uint32_t)bins - 1;
-    const int shift = pass * J.db;
-    const bool to_final = ((J.npass - 1 - pass) & 1) == 0;
-    const uint32_t *kin = to_final ? J.keys_tmp : J.keys_final;  // (unused in the first pass)
-    const int32_t *vin = to_final ? J.vals_tmp : J.out.perm;
-    uint32_t *kout = to_final ? J.keys_final : J.keys_tmp;
-    int32_t *vout = to_final ? J.out.perm : J.vals_tmp;
-    const int my0 = blockIdx.x * kMidKeys;
-
-    for (int i = tid; i < bins; i += kMidThreads) {
-        s_tot[i] = 0, s_bef[i] = 0;
-#pragma unroll
-        for (int w = 0; w < kMidWaves; ++w) s_cnt[w][i] = 0;
-    }
-    // own keys first (their loads overlap the counting loop); positions past n are clamped and
-    // masked at their use
-    const KeySrc src(J.parts);
-    const int last = n - 1;
-    uint32_t key[kMidRounds];
-    int32_t val[kMidRounds];
-#pragma unroll
-    for (int j = 0; j < kMidRounds; ++j) {
-        const int i = my0 + wave * (kMidRounds * kWave) + j * kWave + lane;
-        const int ic = i < n ? i : last;
-        if constexpr (FIRST) key[j] = src(ic), val[j] = i;
-        else key[j] = kin[ic], val[j] = vin[ic];
-    }
-    __syncthreads();
-    constexpr int kBatch = 32;  // unconditional loads in flight per thread
-    for (int i0 = 0; i0 < n; i0 += kBatch * kMidThreads) {
-        uint32_t kb[kBatch];
-#pragma unroll
-        for (int u = 0; u < kBatch; ++u) {
-            const int i = i0 + u * kMidThreads + tid;
-            const int ic = i < n ? i : last;
-            if constexpr (FIRST) kb[u] = src(ic);
-            else kb[u] = kin[ic];
-        }
-#pragma unroll
-        for (int u = 0; u < kBatch; ++u) {
-            const int i = i0 + u * kMidThreads + tid;
-            if (i < n) {
-                const uint32_t dg = (kb[u] >> shift) & mask;
-                atomicAdd(&s_tot[dg], 1u);
-                if (i < my0) atomicAdd(&s_bef[dg], 1u);
-            }
-        }
-    }
-    __syncthreads();
-    block_exclusive_scan(s_tot, bins, s_w);  // s_tot[bin] = first position of the bin
-
-    const uint64_t lt_mask = lane ? (~0ull >> (kWave - lane)) : 0ull;
-    uint32_t lrank[kMidRounds];
-#pragma unroll
-    for (int j = 0; j < kMidRounds; ++j) {
-        const int i = my0 + wave * (kMidRounds * kWave) + j * kWave + lane;
-        const bool ok = i < n;
-        const uint32_t dg = (key[j] >> shift) & mask;
-        uint64_t peers = __ballot(ok);
-        for (int bit = 0; bit < J.db; ++bit) {
-            const bool one = (dg >> bit) & 1u;
-            const uint64_t mm = __ballot(one);
-            peers &= one ? mm : ~mm;
-        }
-        const int leader = __ffsll((unsigned long long)peers) - 1;
-        uint32_t old = 0;
-        if (ok && lane == leader) {
-            old = s_cnt[wave][dg];
-            s_cnt[wave][dg] = old + __popcll(peers);
-        }
-        old = __shfl(old, leader < 0 ? 0 : leader, kWave);
-        lrank[j] = old + __popcll(peers & lt_mask);
-        __builtin_amdgcn_wave_barrier();
-    }
-    __syncthreads();
-    for (int bin = tid; bin < bins; bin += kMidThreads) {
-        uint32_t run = s_tot[bin] + s_bef[bin];
-#pragma unroll
-        for (int w = 0; w < kMidWaves; ++w) {
-            const uint32_t c = s_cnt[w][bin];
-            s_cnt[w][bin] = run;
-            run += c;
-        }
-    }
-    __syncthreads();
-#pragma unroll
-    for (int j = 0; j < kMidRounds; ++j) {
-        const int i = my0 + wave * (kMidRounds * kWave) + j * kWave + lane;
-        if (i < n) {
-            const uint32_t dg = (key[j] >> shift) & mask;
-            const uint32_t pos = s_cnt[wave][dg] + lrank[j];
-            kout[pos] = key[j];
-            vout[pos] = val[j];
-        }
-    }
+    __shared__ uint32_t smem[mid_pass_lds_words(kMaxBins)];
+    mid_scatter_body<FIRST>(jobs.j[blockIdx.y], pass, blockIdx.x, smem);
 }
 
 __global__ __launch_bounds__(kMidThreads) void inspect_mid_dedup_kernel(MidJobs jobs)
 {
-    __shared__ uint32_t s_red[kMidWaves], s_scan[kMidWaves];
-    __builtin_amdgcn_s_setprio(3);
-    const MidJob &J = jobs.j[blockIdx.y];
-    const int n = (int)J.n;
-    const int nblk = n > 0 ? (n + kMidKeys - 1) / kMidKeys : 1;
-    if ((int)blockIdx.x >= nblk) return;
-    const int tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid >> 6;
-    const uint32_t *keys = J.keys_final;
-    const int my0 = blockIdx.x * kMidKeys;
-    // run heads before this block
-    // (my0 is a multiple of 1024: every thread takes whole groups of four keys with one 128-bit
-    // load, plus the key in front of the group; eight groups in flight)
-    uint32_t before = 0;
-    for (int g0 = 0; g0 < my0 / 4; g0 += 8 * kMidThreads) {
-        uint4 q[8];
-        uint32_t pv[8];
-#pragma unroll
-        for (int u = 0; u < 8; ++u) {
-            const int g = g0 + u * kMidThreads + tid;
-            const int gc = g < my0 / 4 ? g : my0 / 4 - 1;  // clamped: unconditional loads, masked below
-            q[u] = reinterpret_cast<const uint4 *>(keys)[gc];
-            pv[u] = keys[gc > 0 ? 4 * gc - 1 : 0];
-        }
-#pragma unroll
-        for (int u = 0; u < 8; ++u) {
-            const int g = g0 + u * kMidThreads + tid;
-            if (g < my0 / 4)
-                before += ((g == 0 || q[u].x != pv[u]) ? 1 : 0) + (q[u].y != q[u].x ? 1 : 0) +
-                          (q[u].z != q[u].y ? 1 : 0) + (q[u].w != q[u].z ? 1 : 0);
-        }
-    }
-    before = (uint32_t)wave_sum_i((int)before);
-    if (lane == 0) s_red[wave] = before;
-    // thread owns 4 consecutive sorted positions
-    const int lo = my0 + tid * kMidRounds;
-    uint32_t k[kMidRounds];
-    bool head[kMidRounds];
-    uint32_t mine = 0;
-    uint32_t prev = (lo > 0 && lo < n) ? keys[lo - 1] : 0;
-#pragma unroll
-    for (int j = 0; j < kMidRounds; ++j) {
-        const int i = lo + j;
-        k[j] = i < n ? keys[i] : 0;
-        head[j] = i < n && (i == 0 || k[j] != prev);
-        prev = k[j];
-        mine += head[j] ? 1 : 0;
-    }
-    uint32_t inc = mine;
-#pragma unroll
-    for (int o = 1; o < kWave; o <<= 1) {
-        const uint32_t up = __shfl_up(inc, o, kWave);
-        if (lane >= o) inc += up;
-    }
-    if (lane == kWave - 1) s_scan[wave] = inc;
-    __syncthreads();
-    before = 0;
-    uint32_t here = 0;
-    for (int w = 0; w < kMidWaves; ++w) before += s_red[w], here += s_scan[w];
-    uint32_t run = before + inc - mine;
-    for (int w = 0; w < wave; ++w) run += s_scan[w];
-    if ((int)blockIdx.x == nblk - 1 && tid == 0) {
-        J.out.num_unique[0] = (int32_t)(before + here);
-        J.out.seg_offsets[before + here] = n;
-    }
-#pragma unroll
-    for (int j = 0; j < kMidRounds; ++j) {
-        const int i = lo + j;
-        if (i < n) {
-            if (head[j]) {
-                J.out.unique_ids[run] = (int64_t)k[j];
-                J.out.seg_offsets[run] = i;
-                ++run;
-            }
-            const int32_t seg = (int32_t)run - 1;
-            J.out.sorted_seg[i] = seg;
-            J.out.inverse[J.out.perm[i]] = seg;
-        }
-    }
+    __shared__ uint32_t smem[kMidDedupLdsWords];
+    mid_dedup_body(jobs.j[blockIdx.y], blockIdx.x, smem);
 }
 
 // ---- host side ---------------------------------------------------------------------------
@@ -577,29 +310,20 @@ static SortPlan make_plan(int64_t n, int64_t n_rows)
     p.bits = bits;
     p.npass = (bits + kMaxDigitBits - 1) / kMaxDigitBits;
     p.digit_bits = (bits + p.npass - 1) / p.npass;
+    if (p.digit_bits < 2) p.digit_bits = 2;  // the scatter step reads histogram bins four at a time
     p.nblocks = n > 0 ? ceil_div(n, kKeysPerBlock) : 1;
     size_t o = 0;
     const size_t n4 = align_up(sizeof(uint32_t) * (size_t)(n > 0 ? n : 1));
     p.off_keys0 = o, o += n4;
     p.off_keys1 = o, o += n4;
     p.off_vals = o, o += n4;
-    p.off_hist = o, o += align_up(sizeof(uint32_t) * (size_t)p.nblocks * kMaxBins);
+    // per-block digit histograms: one table (multi-block sort) or one per pass (up to 65536 ids)
+    const size_t hist_rows = n <= kMidMaxN ? (size_t)kMidMaxPass * mid_blocks(n) : (size_t)p.nblocks;
+    p.off_hist = o, o += align_up(sizeof(uint32_t) * hist_rows * kMaxBins);
     p.off_totals = o, o += align_up(sizeof(uint32_t) * kMaxBins);
     p.off_heads = o, o += align_up(sizeof(uint32_t) * (size_t)p.nblocks);
     p.total = o;
     return p;
-}
-
-}  // namespace kge
-
-using namespace kge;
-
-extern "C" {
-
-size_t kge_inspect_workspace(int64_t n, int64_t n_rows)
-{
-    if (n < 0 || n_rows <= 0) return 0;
-    return make_plan(n, n_rows).total;
 }
 
 static int validate_job(const kge_inspect_job *job, Parts *parts, int64_t *n_out)
@@ -622,6 +346,60 @@ static int validate_job(const kge_inspect_job *job, Parts *parts, int64_t *n_out
     if (!job->workspace || job->workspace_bytes < make_plan(n, job->n_rows).total) return KGE_EWORKSPACE;
     *n_out = n;
     return KGE_OK;
+}
+
+int plan_fused_inspection(const kge_inspect_job *jobs, int slot, FusedInsp *out)
+{
+    if (!jobs || !out || slot < 0 || slot >= kFusedSlots) return KGE_EINVAL;
+    FusedInsp f{};
+    int words = kMidDedupLdsWords;
+    int blocks[2];
+    for (int q = 0; q < 2; ++q) {
+        Parts parts;
+        int64_t n;
+        const int rc = validate_job(&jobs[q], &parts, &n);
+        if (rc) return rc;
+        if (n < 1 || n > kMidMaxN) return KGE_EUNSUPPORTED;
+        const int bits = key_bits(jobs[q].n_rows);
+        if (bits > 2 * kMaxDigitBits) return KGE_EUNSUPPORTED;
+        // two narrow digits rather than one wide one: the second pass hides inside its host kernel,
+        // and the LDS a pass needs grows with the number of bins
+        const SortPlan p = make_plan(n, jobs[q].n_rows);
+        char *ws = static_cast<char *>(jobs[q].workspace);
+        MidJob &J = f.j[q];
+        J.parts = parts;
+        J.n = n;
+        J.npass = bits <= 6 ? 1 : 2;
+        J.db = (bits + J.npass - 1) / J.npass;
+        if (J.db < 2) J.db = 2;
+        J.out = jobs[q].out;
+        J.keys_final = reinterpret_cast<uint32_t *>(ws + p.off_keys0);
+        J.keys_tmp = reinterpret_cast<uint32_t *>(ws + p.off_keys1);
+        J.vals_tmp = reinterpret_cast<int32_t *>(ws + p.off_vals);
+        J.hist = reinterpret_cast<uint32_t *>(ws + p.off_hist);
+        blocks[q] = (int)ceil_div(n, kMidKeys);
+        const int step = slot - (kFusedSlots - 2 - J.npass);
+        const int w = step == 0 ? (1 << J.db) : (step >= 1 && step <= J.npass ? mid_pass_lds_words(1 << J.db) : 0);
+        words = w > words ? w : words;
+    }
+    f.split = blocks[0];
+    f.blocks = (blocks[0] + blocks[1] + 7) / 8 * 8;
+    f.slot = slot;
+    f.lds_bytes = words * (int)sizeof(uint32_t);
+    *out = f;
+    return KGE_OK;
+}
+
+}  // namespace kge
+
+using namespace kge;
+
+extern "C" {
+
+size_t kge_inspect_workspace(int64_t n, int64_t n_rows)
+{
+    if (n < 0 || n_rows <= 0) return 0;
+    return make_plan(n, n_rows).total;
 }
 
 // multi-block path: 2-3 launches per digit pass + 2
@@ -696,20 +474,34 @@ int kge_inspect_batch(const kge_inspect_job *jobs, int n_jobs, void *stream)
         J.keys_final = reinterpret_cast<uint32_t *>(ws + p.off_keys0);
         J.keys_tmp = reinterpret_cast<uint32_t *>(ws + p.off_keys1);
         J.vals_tmp = reinterpret_cast<int32_t *>(ws + p.off_vals);
+        J.hist = reinterpret_cast<uint32_t *>(ws + p.off_hist);
         mid_max = n[q] > mid_max ? n[q] : mid_max;
         max_pass = p.npass > max_pass ? p.npass : max_pass;
     }
     if (n_mid > 0) {
         const dim3 grid((unsigned)(mid_max > 0 ? ceil_div(mid_max, kMidKeys) : 1), (unsigned)n_mid), block(kMidThreads);
-        if (mid_max > 0)
+        if (mid_max > 0) {
+            hipLaunchKernelGGL(inspect_mid_hist_kernel, grid, block, 0, st, mid);
             for (int pass = 0; pass < max_pass; ++pass) {
-                if (pass == 0) hipLaunchKernelGGL(inspect_mid_pass_kernel<true>, grid, block, 0, st, mid, pass);
-                else hipLaunchKernelGGL(inspect_mid_pass_kernel<false>, grid, block, 0, st, mid, pass);
+                if (pass == 0) hipLaunchKernelGGL(inspect_mid_scatter_kernel<true>, grid, block, 0, st, mid, pass);
+                else hipLaunchKernelGGL(inspect_mid_scatter_kernel<false>, grid, block, 0, st, mid, pass);
             }
+        }
         hipLaunchKernelGGL(inspect_mid_dedup_kernel, grid, block, 0, st, mid);
         KGE_CHECK_LAUNCH();
     }
     return KGE_OK;
+}
+
+int kge_fused_inspection_ok(const kge_tables *tab, const kge_batch *bat, const kge_inspect_job *jobs)
+{
+    if (!tab || !bat || !jobs || !bat->neg || bat->batch <= 0) return 0;
+    switch (tab->model) {
+    case KGE_TRANSE: case KGE_TRANSH: case KGE_DISTMULT: case KGE_COMPLEX: case KGE_ROTATE: break;
+    default: return 0;  // no shared-negative kernels to ride with
+    }
+    FusedInsp f;
+    return plan_fused_inspection(jobs, 0, &f) == KGE_OK ? 1 : 0;
 }
 
 int kge_inspect(const int64_t *const *parts_in, const int64_t *part_len, int n_parts, int64_t n_rows,

@@ -15,10 +15,13 @@
 
 #include <type_traits>
 
+#include "inspector_mid.hpp"
 #include "seg_reduce.hpp"
 #include "tile_common.hpp"
 
 namespace kge {
+
+typedef float v4f __attribute__((ext_vector_type(4)));
 
 // ---------------------------------------------------------------------------------------
 // 1 + 2: tile kernel.  "Owners" keep their slice of the row in registers and accumulate
@@ -118,6 +121,21 @@ __device__ __forceinline__ void bwd_tile_body(const TileArgs &a, int lid, float 
     for (int q = 0; q < NOUT; ++q)
 #pragma unroll
         for (int o = 0; o < RO; ++o) acc[q][o] = zero4();
+
+    // DistMult / ComplEx: the sum over loopers is a plain matrix product, coefficients (owners x
+    // loopers) times looper rows (loopers x columns), so it runs on the matrix cores
+    // (v_mfma_f32_16x16x4_f32).  Lane l supplies A[i = l % 16][k = l / 16] and B[k][j = l % 16] and
+    // receives D[i = 4 (l / 16) + v][j].  Inside 16 loopers the MFMA step s pairs lane group
+    // g = l / 16 with looper 4 g + s; a lane's 128-bit read of four consecutive columns of that
+    // looper's row feeds four MFMAs, so MFMA e owns the columns 4 j + e.  A wave owns 16 owners and
+    // all 64 columns (64-owner tiles), or 16 owners and the columns 4 j + {0,1} / {2,3} (32-owner tiles).
+    constexpr int OB = TO / 16, EW = OB;  // owner blocks; MFMAs (columns per lane) per wave
+    static_assert(!kDot || OB == 4 || OB == 2, "MFMA tiling written for 32- and 64-owner tiles");
+    const int mlane = tid & 63, mwave = tid >> 6, fj = mlane & 15, fg = mlane >> 4;
+    const int ob = mwave % OB, e0 = (mwave / OB) * EW;
+    v4f macc[EW];
+#pragma unroll
+    for (int e = 0; e < EW; ++e) macc[e] = v4f{0.0f, 0.0f, 0.0f, 0.0f};
 
     // ---- staging: a three-deep software pipeline --------------------------------------------
     // While step st is computed, the rows and coefficients of step st+1 are in flight and so are
@@ -285,13 +303,33 @@ __device__ __forceinline__ void bwd_tile_body(const TileArgs &a, int lid, float 
         // two-level sum: the kKL loopers of a step go into a fresh accumulator that is folded
         // into the running one per step, so rounding grows with sqrt(steps) of the large partial
         // sums instead of sqrt(loopers)
+        if constexpr (kDot) {
+#pragma unroll
+            for (int q = 0; q < kKL / 16; ++q)
+#pragma unroll
+                for (int ms = 0; ms < 4; ++ms) {
+                    const int l = 16 * q + 4 * fg + ms;
+                    const float av = sG[0][l][ob * 16 + fj];
+                    float bv[EW];
+                    if constexpr (EW == 4) {
+                        const float4 b4 = *reinterpret_cast<const float4 *>(&sL[0][l][4 * fj]);
+                        bv[0] = b4.x, bv[1] = b4.y, bv[2] = b4.z, bv[3] = b4.w;
+                    } else {
+                        const float2 b2 = *reinterpret_cast<const float2 *>(&sL[0][l][4 * fj + e0]);
+                        bv[0] = b2.x, bv[1] = b2.y;
+                    }
+#pragma unroll
+                    for (int e = 0; e < EW; ++e)
+                        macc[e] = __builtin_amdgcn_mfma_f32_16x16x4f32(av, bv[e], macc[e], 0, 0, 0);
+                }
+        }
         float4 sacc[NOUT][RO];
 #pragma unroll
         for (int q = 0; q < NOUT; ++q)
 #pragma unroll
             for (int o = 0; o < RO; ++o) sacc[q][o] = zero4();
 #pragma unroll 4
-        for (int l = 0; l < kKL; ++l) {
+        for (int l = 0; l < (kDot ? 0 : kKL); ++l) {
             float4 lv[NPL];
 #pragma unroll
             for (int pl = 0; pl < NPL; ++pl) lv[pl] = *reinterpret_cast<const float4 *>(&sL[pl][l][tx * 4]);
@@ -356,6 +394,27 @@ __device__ __forceinline__ void bwd_tile_body(const TileArgs &a, int lid, float 
         __syncthreads();
     }
 
+    if constexpr (kDot) {
+#pragma unroll
+        for (int v = 0; v < 4; ++v) {
+            const int ol = ot0 + ob * 16 + 4 * fg + v;
+            if (ol >= n_own) continue;
+            const int64_t row = OWNER_POS ? (int64_t)c * a.C + ol : (int64_t)c * a.N + ol;
+            float *dst = a.out0 + row * (int64_t)d;
+            const int c0 = tile_x * kTI + 4 * fj + e0;
+            if (vec && c0 + EW <= klen) {  // rows 16-byte aligned and d % 4 == 0: whole group inside
+                if constexpr (EW == 4)
+                    *reinterpret_cast<float4 *>(dst + c0) = make_float4(macc[0][v], macc[1][v], macc[2][v], macc[3][v]);
+                else
+                    *reinterpret_cast<float2 *>(dst + c0) = make_float2(macc[0][v], macc[1][v]);
+            } else {
+#pragma unroll
+                for (int e = 0; e < EW; ++e)
+                    if (c0 + e < klen) dst[c0 + e] = macc[e][v];
+            }
+        }
+        return;
+    }
 #pragma unroll
     for (int o = 0; o < RO; ++o) {
         const int ol = ot0 + ty * RO + o;
@@ -373,35 +432,53 @@ __device__ __forceinline__ void bwd_tile_body(const TileArgs &a, int lid, float 
 // together they fill the GPU better than either alone when the batch is small.
 template <int MODEL, int P, int RO>
 __global__ __launch_bounds__(256, KGE_TILE_OCC) void bwd_tile_kernel(TileArgs a, float *g0, float *g1, float *occ_neg,
-                                                                     int grid_head)
+                                                                     int grid_head, FusedInsp fi)
+{
+    extern __shared__ __align__(16) char dyn_smem[];  // tile_lds_bytes<MODEL, RO>() or the inspector's need
+    if (fused_insp_block(fi, reinterpret_cast<uint32_t *>(dyn_smem))) return;
+    float *smem = reinterpret_cast<float *>(dyn_smem);
+    const int lid = (int)blockIdx.x - fi.blocks;
+    if (lid < grid_head) {
+        a.out0 = g0, a.out1 = g1;
+        bwd_tile_body<MODEL, P, true, RO>(a, lid, smem);
+    } else {
+        a.out0 = occ_neg, a.out1 = nullptr;
+        bwd_tile_body<MODEL, P, false, RO>(a, lid - grid_head, smem);
+    }
+}
+
+template <int MODEL, int RO>
+static size_t tile_lds_bytes(const FusedInsp &fi)
 {
     constexpr int kFloats = TileShape<MODEL, true, RO>::kLdsFloats > TileShape<MODEL, false, RO>::kLdsFloats
                                 ? TileShape<MODEL, true, RO>::kLdsFloats
                                 : TileShape<MODEL, false, RO>::kLdsFloats;
-    __shared__ __align__(16) float smem[kFloats];
-    if ((int)blockIdx.x < grid_head) {
-        a.out0 = g0, a.out1 = g1;
-        bwd_tile_body<MODEL, P, true, RO>(a, blockIdx.x, smem);
-    } else {
-        a.out0 = occ_neg, a.out1 = nullptr;
-        bwd_tile_body<MODEL, P, false, RO>(a, blockIdx.x - grid_head, smem);
-    }
+    const size_t own = sizeof(float) * kFloats;
+    return fi.blocks > 0 && (size_t)fi.lds_bytes > own ? (size_t)fi.lds_bytes : own;
 }
 
 template <int MODEL, int P>
-static int launch_tiles(TileArgs a, float *g0, float *g1, float *occ_neg, int64_t n_chunks, hipStream_t st)
+static int launch_tiles(TileArgs a, float *g0, float *g1, float *occ_neg, int64_t n_chunks, const FusedInsp &fi,
+                        hipStream_t st)
 {
     const int klen = MODEL == KGE_ROTATE ? a.d / 2 : a.d;
     const int64_t gx = ceil_div(klen, kTI);
     const int64_t big = gx * (ceil_div(a.C, 64) + ceil_div(a.N, 64)) * n_chunks;
     static const int knob = [] { const char *e = getenv("KGE_BWD_TILE"); return e ? atoi(e) : 0; }();
     // KGE_BWD_TILE is a development knob; the size rule follows launch_neg_mp (see there)
-    if (knob == 4 || (knob != 2 && big >= 1024)) {
+    // (the matrix-core inner loop of DistMult / ComplEx gives a wave all 64 columns of its 16 owners
+    // with 64-owner tiles and half of them with 32-owner tiles: the large tile wins at every size)
+    constexpr bool kDotModel = MODEL == KGE_DISTMULT || MODEL == KGE_COMPLEX;
+    if (knob == 4 || (knob != 2 && (kDotModel || big >= 1024))) {
         const unsigned gh = xcd_grid(gx, ceil_div(a.C, 64), n_chunks), gn = xcd_grid(gx, ceil_div(a.N, 64), n_chunks);
-        hipLaunchKernelGGL((bwd_tile_kernel<MODEL, P, 4>), dim3(gh + gn), dim3(256), 0, st, a, g0, g1, occ_neg, (int)gh);
+        const size_t lds = tile_lds_bytes<MODEL, 4>(fi);
+        hipLaunchKernelGGL((bwd_tile_kernel<MODEL, P, 4>), dim3(gh + gn + fi.blocks), dim3(256), lds, st, a, g0, g1,
+                           occ_neg, (int)gh, fi);
     } else {
         const unsigned gh = xcd_grid(gx, ceil_div(a.C, 32), n_chunks), gn = xcd_grid(gx, ceil_div(a.N, 32), n_chunks);
-        hipLaunchKernelGGL((bwd_tile_kernel<MODEL, P, 2>), dim3(gh + gn), dim3(256), 0, st, a, g0, g1, occ_neg, (int)gh);
+        const size_t lds = tile_lds_bytes<MODEL, 2>(fi);
+        hipLaunchKernelGGL((bwd_tile_kernel<MODEL, P, 2>), dim3(gh + gn + fi.blocks), dim3(256), lds, st, a, g0, g1,
+                           occ_neg, (int)gh, fi);
     }
     KGE_CHECK_LAUNCH();
     return KGE_OK;
@@ -437,10 +514,12 @@ __device__ __forceinline__ Vec<V> ldz(const float *p, int j)
 // (x, rho) = (t, -r) [TransE, TransH], (t, conj r) [ComplEx], (t, -theta) [RotatE], (t, r) [DistMult],
 // so G chains into the t and r rows instead and the positive triple's own term is kept apart.
 template <int MODEL, int P, int V, bool HEAD>
-__global__ __launch_bounds__(256) void bwd_pos_kernel(PosBwdArgs a)
+__global__ __launch_bounds__(256) void bwd_pos_kernel(PosBwdArgs a, FusedInsp fi)
 {
+    extern __shared__ __align__(16) char dyn_smem[];  // inspector workgroups only
+    if (fused_insp_block(fi, reinterpret_cast<uint32_t *>(dyn_smem))) return;
     const int lane = threadIdx.x & (kWave - 1);
-    const int64_t b = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    const int64_t b = (int64_t)((int)blockIdx.x - fi.blocks) * 4 + (threadIdx.x >> 6);
     if (b >= a.B) return;  // whole waves leave together; no block-level sync below
     const int d = a.d, half = d >> 1;
     const int64_t rid = a.r[b];
@@ -635,15 +714,16 @@ __global__ __launch_bounds__(256) void bwd_pos_kernel(PosBwdArgs a)
 }
 
 template <int MODEL, int P>
-static int launch_pos_bwd(const PosBwdArgs &a, bool vec4, bool head, hipStream_t st)
+static int launch_pos_bwd(const PosBwdArgs &a, bool vec4, bool head, const FusedInsp &fi, hipStream_t st)
 {
-    const dim3 grid((unsigned)ceil_div(a.B, 4)), block(256);
+    const dim3 grid((unsigned)ceil_div(a.B, 4) + (unsigned)fi.blocks), block(256);
+    const size_t lds = fi.blocks > 0 ? (size_t)fi.lds_bytes : 0;
     if (head) {
-        if (vec4) hipLaunchKernelGGL((bwd_pos_kernel<MODEL, P, 4, true>), grid, block, 0, st, a);
-        else hipLaunchKernelGGL((bwd_pos_kernel<MODEL, P, 1, true>), grid, block, 0, st, a);
+        if (vec4) hipLaunchKernelGGL((bwd_pos_kernel<MODEL, P, 4, true>), grid, block, lds, st, a, fi);
+        else hipLaunchKernelGGL((bwd_pos_kernel<MODEL, P, 1, true>), grid, block, lds, st, a, fi);
     } else {
-        if (vec4) hipLaunchKernelGGL((bwd_pos_kernel<MODEL, P, 4, false>), grid, block, 0, st, a);
-        else hipLaunchKernelGGL((bwd_pos_kernel<MODEL, P, 1, false>), grid, block, 0, st, a);
+        if (vec4) hipLaunchKernelGGL((bwd_pos_kernel<MODEL, P, 4, false>), grid, block, lds, st, a, fi);
+        else hipLaunchKernelGGL((bwd_pos_kernel<MODEL, P, 1, false>), grid, block, lds, st, a, fi);
     }
     KGE_CHECK_LAUNCH();
     return KGE_OK;
@@ -746,6 +826,15 @@ int kge_score_bwd(const kge_tables *tab, const kge_batch *bat, const kge_saved *
     float *g1 = have_neg && model == KGE_TRANSH ? reinterpret_cast<float *>(ws + p.off_g1) : nullptr;
     const bool vec = rows_vectorizable(tab);
     int rc = KGE_OK;
+    // inspection fused into the score kernels' launches: the histogram and the first digit pass
+    // rode with the two forward kernels; the last pass rides with the gradient tile kernel, the
+    // dedup with the per-positive kernel
+    FusedInsp fi_pass{}, fi_dedup{};
+    if (bat->fuse_inspection) {
+        if (!have_neg || !bat->insp_jobs) return KGE_EINVAL;
+        if ((rc = plan_fused_inspection(bat->insp_jobs, 2, &fi_pass))) return rc;
+        if ((rc = plan_fused_inspection(bat->insp_jobs, 3, &fi_dedup))) return rc;
+    }
 
     if (have_neg) {
         const int64_t n_chunks = B / bat->chunk;
@@ -759,16 +848,16 @@ int kge_score_bwd(const kge_tables *tab, const kge_batch *bat, const kge_saved *
         float *occ_neg = occ_e + 2 * B * d;
         switch (model) {
         case KGE_TRANSE:
-            rc = P == 1 ? launch_tiles<KGE_TRANSE, 1>(a, g0, g1, occ_neg, n_chunks, st)
-                        : launch_tiles<KGE_TRANSE, 2>(a, g0, g1, occ_neg, n_chunks, st);
+            rc = P == 1 ? launch_tiles<KGE_TRANSE, 1>(a, g0, g1, occ_neg, n_chunks, fi_pass, st)
+                        : launch_tiles<KGE_TRANSE, 2>(a, g0, g1, occ_neg, n_chunks, fi_pass, st);
             break;
         case KGE_TRANSH:
-            rc = P == 1 ? launch_tiles<KGE_TRANSH, 1>(a, g0, g1, occ_neg, n_chunks, st)
-                        : launch_tiles<KGE_TRANSH, 2>(a, g0, g1, occ_neg, n_chunks, st);
+            rc = P == 1 ? launch_tiles<KGE_TRANSH, 1>(a, g0, g1, occ_neg, n_chunks, fi_pass, st)
+                        : launch_tiles<KGE_TRANSH, 2>(a, g0, g1, occ_neg, n_chunks, fi_pass, st);
             break;
-        case KGE_DISTMULT: rc = launch_tiles<KGE_DISTMULT, 2>(a, g0, g1, occ_neg, n_chunks, st); break;
-        case KGE_COMPLEX: rc = launch_tiles<KGE_COMPLEX, 2>(a, g0, g1, occ_neg, n_chunks, st); break;
-        case KGE_ROTATE: rc = launch_tiles<KGE_ROTATE, 2>(a, g0, g1, occ_neg, n_chunks, st); break;
+        case KGE_DISTMULT: rc = launch_tiles<KGE_DISTMULT, 2>(a, g0, g1, occ_neg, n_chunks, fi_pass, st); break;
+        case KGE_COMPLEX: rc = launch_tiles<KGE_COMPLEX, 2>(a, g0, g1, occ_neg, n_chunks, fi_pass, st); break;
+        case KGE_ROTATE: rc = launch_tiles<KGE_ROTATE, 2>(a, g0, g1, occ_neg, n_chunks, fi_pass, st); break;
         default: return KGE_EUNSUPPORTED;
         }
         if (rc) return rc;
@@ -780,15 +869,15 @@ int kge_score_bwd(const kge_tables *tab, const kge_batch *bat, const kge_saved *
                   g0, g1, occ_e, occ_e + B * d, occ_r, occ_w, B, (int)d, (int)tab->rel_dim};
     switch (model) {
     case KGE_TRANSE:
-        rc = P == 1 ? launch_pos_bwd<KGE_TRANSE, 1>(pa, vec, head, st) : launch_pos_bwd<KGE_TRANSE, 2>(pa, vec, head, st);
+        rc = P == 1 ? launch_pos_bwd<KGE_TRANSE, 1>(pa, vec, head, fi_dedup, st) : launch_pos_bwd<KGE_TRANSE, 2>(pa, vec, head, fi_dedup, st);
         break;
     case KGE_TRANSH:
-        rc = P == 1 ? launch_pos_bwd<KGE_TRANSH, 1>(pa, vec, head, st) : launch_pos_bwd<KGE_TRANSH, 2>(pa, vec, head, st);
+        rc = P == 1 ? launch_pos_bwd<KGE_TRANSH, 1>(pa, vec, head, fi_dedup, st) : launch_pos_bwd<KGE_TRANSH, 2>(pa, vec, head, fi_dedup, st);
         break;
-    case KGE_DISTMULT: rc = launch_pos_bwd<KGE_DISTMULT, 2>(pa, vec, head, st); break;
-    case KGE_COMPLEX: rc = launch_pos_bwd<KGE_COMPLEX, 2>(pa, vec, head, st); break;
-    case KGE_ROTATE: rc = launch_pos_bwd<KGE_ROTATE, 2>(pa, vec, head, st); break;
-    case KGE_TRANSF: rc = launch_pos_bwd<KGE_TRANSF, 2>(pa, vec, head, st); break;
+    case KGE_DISTMULT: rc = launch_pos_bwd<KGE_DISTMULT, 2>(pa, vec, head, fi_dedup, st); break;
+    case KGE_COMPLEX: rc = launch_pos_bwd<KGE_COMPLEX, 2>(pa, vec, head, fi_dedup, st); break;
+    case KGE_ROTATE: rc = launch_pos_bwd<KGE_ROTATE, 2>(pa, vec, head, fi_dedup, st); break;
+    case KGE_TRANSF: rc = launch_pos_bwd<KGE_TRANSF, 2>(pa, vec, head, fi_dedup, st); break;
     default: return KGE_EUNSUPPORTED;
     }
     if (rc) return rc;

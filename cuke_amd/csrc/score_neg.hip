@@ -12,6 +12,7 @@
 
 #include <type_traits>
 
+#include "inspector_mid.hpp"
 #include "tile_common.hpp"
 
 namespace kge {
@@ -60,8 +61,10 @@ __device__ __forceinline__ void pair_elem(float &acc, float &acc2, float a0, flo
 }
 
 template <int MODEL, int P, int RB, int RK, bool SAVE>
-__global__ __launch_bounds__(256, KGE_TILE_OCC) void score_neg_kernel(NegArgs a)
+__global__ __launch_bounds__(256, KGE_TILE_OCC) void score_neg_kernel(NegArgs a, FusedInsp fi)
 {
+    extern __shared__ __align__(16) char dyn_smem[];
+    if (fused_insp_block(fi, reinterpret_cast<uint32_t *>(dyn_smem))) return;
     constexpr int TB = 16 * RB, TN = 16 * RK;
     constexpr int NPA = (MODEL == KGE_ROTATE || MODEL == KGE_TRANSH) ? 2 : 1;
     constexpr int NPT = MODEL == KGE_ROTATE ? 2 : 1;
@@ -69,13 +72,13 @@ __global__ __launch_bounds__(256, KGE_TILE_OCC) void score_neg_kernel(NegArgs a)
     constexpr int NPASS = MODEL == KGE_TRANSH ? 2 : 1;
     static_assert(TB % 32 == 0 && TN % 32 == 0, "tile rows are staged 32 at a time");
 
-    __shared__ __align__(16) float sA[NPA][TB][kLDW];
-    __shared__ __align__(16) float sT[NPT][TN][kLDW];
+    float(*sA)[TB][kLDW] = reinterpret_cast<float(*)[TB][kLDW]>(dyn_smem);
+    float(*sT)[TN][kLDW] = reinterpret_cast<float(*)[TN][kLDW]>(dyn_smem + sizeof(float) * NPA * TB * kLDW);
 
     const int tid = threadIdx.x, tx = tid & 15, ty = tid >> 4;
     const int srow = tid >> 3, scol = (tid & 7) * 4;
     int c, tile_y, tile_x;
-    if (!xcd_tile(blockIdx.x, (a.N + TN - 1) / TN, (a.C + TB - 1) / TB, a.n_chunks, c, tile_y, tile_x)) return;
+    if (!xcd_tile(blockIdx.x - fi.blocks, (a.N + TN - 1) / TN, (a.C + TB - 1) / TB, a.n_chunks, c, tile_y, tile_x)) return;
     const int bt0 = tile_y * TB, kt0 = tile_x * TN;
     const int d = a.d, half = d >> 1;
     const int klen = MODEL == KGE_ROTATE ? half : d;
@@ -231,16 +234,18 @@ __global__ __launch_bounds__(256, KGE_TILE_OCC) void score_neg_kernel(NegArgs a)
 typedef float v4f __attribute__((ext_vector_type(4)));
 
 template <int MODEL, int RB, int RK>
-__global__ __launch_bounds__(256, KGE_TILE_OCC) void score_neg_mfma_kernel(NegArgs a)
+__global__ __launch_bounds__(256, KGE_TILE_OCC) void score_neg_mfma_kernel(NegArgs a, FusedInsp fi)
 {
+    extern __shared__ __align__(16) char dyn_smem[];
+    if (fused_insp_block(fi, reinterpret_cast<uint32_t *>(dyn_smem))) return;
     static_assert(MODEL == KGE_DISTMULT || MODEL == KGE_COMPLEX, "dot-product scores only");
     constexpr int TB = 16 * RB, TN = 16 * RK;
     constexpr int SB = TB / 32, SN = TN / 32;
     constexpr int MB = RB / 2, NB = RK / 2;  // 16 x 16 blocks per wave
     static_assert(TB % 32 == 0 && TN % 32 == 0, "tile rows are staged 32 at a time");
 
-    __shared__ __align__(16) float sA[TB][kLDW];
-    __shared__ __align__(16) float sT[TN][kLDW];
+    float(*sA)[kLDW] = reinterpret_cast<float(*)[kLDW]>(dyn_smem);
+    float(*sT)[kLDW] = reinterpret_cast<float(*)[kLDW]>(dyn_smem + sizeof(float) * TB * kLDW);
 
     const int tid = threadIdx.x;
     const int srow = tid >> 3, scol = (tid & 7) * 4;
@@ -248,7 +253,7 @@ __global__ __launch_bounds__(256, KGE_TILE_OCC) void score_neg_mfma_kernel(NegAr
     const int fr = lane & 15, fg = lane >> 4;
     const int wrow = (wave >> 1) * (TB / 2), wcol = (wave & 1) * (TN / 2);
     int c, tile_y, tile_x;
-    if (!xcd_tile(blockIdx.x, (a.N + TN - 1) / TN, (a.C + TB - 1) / TB, a.n_chunks, c, tile_y, tile_x)) return;
+    if (!xcd_tile(blockIdx.x - fi.blocks, (a.N + TN - 1) / TN, (a.C + TB - 1) / TB, a.n_chunks, c, tile_y, tile_x)) return;
     const int bt0 = tile_y * TB, kt0 = tile_x * TN;
     const int d = a.d, half = d >> 1;
     const bool vec = a.vec != 0;
@@ -366,9 +371,17 @@ static int neg_valu_override()
     return v;
 }
 
-template <int MODEL, int P>
-static int launch_neg_mp(const NegArgs &a, int64_t n_chunks, hipStream_t st)
+// LDS bytes of a launch: the tile's staging buffers, or what the inspector workgroups need if more
+static size_t neg_lds(int planes, int TB, int TN, int planes_t, const FusedInsp &fi)
 {
+    const size_t own = sizeof(float) * kLDW * ((size_t)planes * TB + (size_t)planes_t * TN);
+    return fi.blocks > 0 && (size_t)fi.lds_bytes > own ? (size_t)fi.lds_bytes : own;
+}
+
+template <int MODEL, int P>
+static int launch_neg_mp(const NegArgs &a, int64_t n_chunks, const FusedInsp &fi, hipStream_t st)
+{
+    constexpr int NPA = (MODEL == KGE_ROTATE || MODEL == KGE_TRANSH) ? 2 : 1, NPT = MODEL == KGE_ROTATE ? 2 : 1;
     const int64_t big_tiles = ceil_div(a.C, 64) * ceil_div(a.N, 64) * n_chunks;
     int tile = neg_tile_override();
     // 32x32 tiles up to about 1024 big tiles: more waves to hide latency (~20 % faster than 64x64
@@ -376,48 +389,38 @@ static int launch_neg_mp(const NegArgs &a, int64_t n_chunks, hipStream_t st)
     // starve an inspection running next to it on another stream; the inspector kernels raise their
     // wave priority for that reason.
     if (tile != 2 && tile != 4 && tile != 3) tile = big_tiles >= 1024 ? 4 : 2;
+    const int TB = tile == 4 ? 64 : 32, TN = tile == 2 ? 32 : 64;
+    const dim3 grid(xcd_grid(ceil_div(a.N, TN), ceil_div(a.C, TB), n_chunks) + (unsigned)fi.blocks);
     if constexpr (MODEL == KGE_DISTMULT || MODEL == KGE_COMPLEX) {
         if (!neg_valu_override()) {
-            if (tile == 4) {
-                const dim3 grid(xcd_grid(ceil_div(a.N, 64), ceil_div(a.C, 64), n_chunks));
-                hipLaunchKernelGGL((score_neg_mfma_kernel<MODEL, 4, 4>), grid, dim3(256), 0, st, a);
-            } else if (tile == 3) {
-                const dim3 grid(xcd_grid(ceil_div(a.N, 64), ceil_div(a.C, 32), n_chunks));
-                hipLaunchKernelGGL((score_neg_mfma_kernel<MODEL, 2, 4>), grid, dim3(256), 0, st, a);
-            } else {
-                const dim3 grid(xcd_grid(ceil_div(a.N, 32), ceil_div(a.C, 32), n_chunks));
-                hipLaunchKernelGGL((score_neg_mfma_kernel<MODEL, 2, 2>), grid, dim3(256), 0, st, a);
-            }
+            const size_t lds = neg_lds(1, TB, TN, 1, fi);
+            if (tile == 4) hipLaunchKernelGGL((score_neg_mfma_kernel<MODEL, 4, 4>), grid, dim3(256), lds, st, a, fi);
+            else if (tile == 3) hipLaunchKernelGGL((score_neg_mfma_kernel<MODEL, 2, 4>), grid, dim3(256), lds, st, a, fi);
+            else hipLaunchKernelGGL((score_neg_mfma_kernel<MODEL, 2, 2>), grid, dim3(256), lds, st, a, fi);
             KGE_CHECK_LAUNCH();
             return KGE_OK;
         }
     }
+    const size_t lds = neg_lds(NPA, TB, TN, NPT, fi);
+    const bool save = MODEL == KGE_TRANSH && a.side_neg;
     if (tile == 3) {  // 32 positives x 64 negatives
-        const dim3 grid(xcd_grid(ceil_div(a.N, 64), ceil_div(a.C, 32), n_chunks));
-        if (MODEL == KGE_TRANSH && a.side_neg)
-            hipLaunchKernelGGL((score_neg_kernel<MODEL, P, 2, 4, true>), grid, dim3(256), 0, st, a);
-        else
-            hipLaunchKernelGGL((score_neg_kernel<MODEL, P, 2, 4, false>), grid, dim3(256), 0, st, a);
+        if (save) hipLaunchKernelGGL((score_neg_kernel<MODEL, P, 2, 4, true>), grid, dim3(256), lds, st, a, fi);
+        else hipLaunchKernelGGL((score_neg_kernel<MODEL, P, 2, 4, false>), grid, dim3(256), lds, st, a, fi);
     } else if (tile == 4) {
-        const dim3 grid(xcd_grid(ceil_div(a.N, 64), ceil_div(a.C, 64), n_chunks));
-        if (MODEL == KGE_TRANSH && a.side_neg)
-            hipLaunchKernelGGL((score_neg_kernel<MODEL, P, 4, 4, true>), grid, dim3(256), 0, st, a);
-        else
-            hipLaunchKernelGGL((score_neg_kernel<MODEL, P, 4, 4, false>), grid, dim3(256), 0, st, a);
+        if (save) hipLaunchKernelGGL((score_neg_kernel<MODEL, P, 4, 4, true>), grid, dim3(256), lds, st, a, fi);
+        else hipLaunchKernelGGL((score_neg_kernel<MODEL, P, 4, 4, false>), grid, dim3(256), lds, st, a, fi);
     } else {
-        const dim3 grid(xcd_grid(ceil_div(a.N, 32), ceil_div(a.C, 32), n_chunks));
-        if (MODEL == KGE_TRANSH && a.side_neg)
-            hipLaunchKernelGGL((score_neg_kernel<MODEL, P, 2, 2, true>), grid, dim3(256), 0, st, a);
-        else
-            hipLaunchKernelGGL((score_neg_kernel<MODEL, P, 2, 2, false>), grid, dim3(256), 0, st, a);
+        if (save) hipLaunchKernelGGL((score_neg_kernel<MODEL, P, 2, 2, true>), grid, dim3(256), lds, st, a, fi);
+        else hipLaunchKernelGGL((score_neg_kernel<MODEL, P, 2, 2, false>), grid, dim3(256), lds, st, a, fi);
     }
     KGE_CHECK_LAUNCH();
     return KGE_OK;
 }
 
 int launch_score_neg(const kge_tables *tab, const kge_batch *bat, const float *side_pos, const float *query,
-                     float *out, float *side_neg, hipStream_t st)
+                     float *out, float *side_neg, const FusedInsp *fused, hipStream_t st)
 {
+    const FusedInsp fi = fused ? *fused : FusedInsp{};
     if (bat->batch == 0) return KGE_OK;
     const int64_t n_chunks = bat->batch / bat->chunk;
     if (n_chunks >= (1 << 24) || bat->chunk >= (1 << 30) || bat->n_neg >= (1 << 30)) return KGE_ESHAPE;
@@ -429,14 +432,14 @@ int launch_score_neg(const kge_tables *tab, const kge_batch *bat, const float *s
     const int p = tab->norm_p;
     switch (tab->model) {
     case KGE_TRANSE:
-        return p == 1 ? launch_neg_mp<KGE_TRANSE, 1>(a, n_chunks, st)
-                      : launch_neg_mp<KGE_TRANSE, 2>(a, n_chunks, st);
+        return p == 1 ? launch_neg_mp<KGE_TRANSE, 1>(a, n_chunks, fi, st)
+                      : launch_neg_mp<KGE_TRANSE, 2>(a, n_chunks, fi, st);
     case KGE_TRANSH:
-        return p == 1 ? launch_neg_mp<KGE_TRANSH, 1>(a, n_chunks, st)
-                      : launch_neg_mp<KGE_TRANSH, 2>(a, n_chunks, st);
-    case KGE_DISTMULT: return launch_neg_mp<KGE_DISTMULT, 2>(a, n_chunks, st);
-    case KGE_COMPLEX: return launch_neg_mp<KGE_COMPLEX, 2>(a, n_chunks, st);
-    case KGE_ROTATE: return launch_neg_mp<KGE_ROTATE, 2>(a, n_chunks, st);
+        return p == 1 ? launch_neg_mp<KGE_TRANSH, 1>(a, n_chunks, fi, st)
+                      : launch_neg_mp<KGE_TRANSH, 2>(a, n_chunks, fi, st);
+    case KGE_DISTMULT: return launch_neg_mp<KGE_DISTMULT, 2>(a, n_chunks, fi, st);
+    case KGE_COMPLEX: return launch_neg_mp<KGE_COMPLEX, 2>(a, n_chunks, fi, st);
+    case KGE_ROTATE: return launch_neg_mp<KGE_ROTATE, 2>(a, n_chunks, fi, st);
     default: return KGE_EUNSUPPORTED;  // TransR / TransF / RESCAL: positives only
     }
 }

@@ -507,6 +507,8 @@ class TrainStep:
         s.bat = _lib.Batch(self.B, h.data_ptr(), r.data_ptr(), t.data_ptr(),
                            neg.data_ptr() if neg is not None else None, self.C, self.N,
                            C.pointer(s.ent_insp._c), C.pointer(s.rel_insp._c), None, NEG_MODES[self._neg_mode], 0)
+        s.bat.insp_jobs = C.addressof(s.jobs)
+        s.fusable = bool(L.kge_fused_inspection_ok(C.byref(m._tab), C.byref(s.bat), s.jobs))
         s.insp_event = torch.cuda.Event()
         s.done_event = None  # recorded on the main stream after the last pipelined step that used this set
         s.inputs_ready = None
@@ -589,11 +591,23 @@ class TrainStep:
         self._staged.append(at)
         self._stage_at = (at + 1) % len(sets)
 
-    def run(self, backward=True, overlap=True, pipeline=False, inputs_ready=None):
-        """Enqueue one step.  With overlap (default) the inspector runs on a side stream while
-        the main stream computes scores and per-occurrence gradients; backward waits for it
-        right before its segmented reduction.  TransR / RESCAL need the relation groups in the
-        forward pass, so their relation inspection stays on the main stream.
+    @property
+    def fusable(self):
+        """True if the inspections of this batch shape can ride inside the score kernels' launches."""
+        return self._sets[self._cur].fusable
+
+    def run(self, backward=True, overlap=True, pipeline=False, inputs_ready=None, fused=None):
+        """Enqueue one step.
+
+        fused (default whenever the batch qualifies: shared negatives, index sets of at most 65536
+        ids): no inspector kernels at all -- the inspector's workgroups ride in front of the
+        score kernels' own workgroups in the same launches, so the whole step is one chain of
+        kernels on one stream with the inspection off its critical path.
+
+        Otherwise, with overlap, the inspector runs on a side stream while the main stream
+        computes scores and per-occurrence gradients; backward waits for it right before its
+        segmented reduction.  TransR / RESCAL need the relation groups in the forward pass, so
+        their relation inspection stays on the main stream.
 
         pipeline=True runs the oldest batch handed over with ``stage()`` (staging the tensors of
         ``next_inputs()`` first, with ``inputs_ready``, if none is waiting).  Index tensors and
@@ -602,6 +616,22 @@ class TrainStep:
         capturable into one graph: the dependencies cross steps."""
         main = torch.cuda.current_stream()
         st = C.c_void_p(main.cuda_stream)
+        if fused is None:
+            fused = backward and not pipeline and self.fusable
+        if fused:
+            if not (backward and self.fusable) or pipeline or self._staged:
+                raise KgeError("fused inspection needs a backward step over a batch that qualifies "
+                               "(TrainStep.fusable), outside the staged pipeline")
+            bat = self.bat
+            bat.insp_ready, bat.fuse_inspection = None, 1
+            try:
+                self.forward(st)
+                self.loss_grad(st)
+                self.backward(st)
+            finally:
+                bat.fuse_inspection = 0
+            self._record_done(main)
+            return
         if not (backward and overlap):
             self.bat.insp_ready = None
             self.inspect(st, backward)
@@ -635,7 +665,12 @@ class TrainStep:
         self.forward(st)
         self.loss_grad(st)
         self.backward(st)
-        if pipeline or (len(self._sets) > 1 and not torch.cuda.is_current_stream_capturing()):
+        self._record_done(main, pipeline)
+
+    def _record_done(self, main, force=False):
+        """Marks the end of the step that read the current set, for the ring's reuse check."""
+        cur = self._sets[self._cur]
+        if force or (len(self._sets) > 1 and not torch.cuda.is_current_stream_capturing()):
             if cur.done_event is None:
                 cur.done_event = torch.cuda.Event()
             cur.done_event.record(main)

@@ -117,7 +117,18 @@ typedef struct kge_batch {
        (neg_k, r_b, t_b), the head-corrupted batches of apps/kge/data/sampler.py:287-353
        (neg_head).  Zero-initialised structs get KGE_NEG_TAIL. */
     int32_t neg_mode;
-    int32_t reserved;
+    /* Non-zero: the inspections are not run by kge_inspect* at all; their workgroups ride in
+       front of the score kernels' own in the same launches (histogram and first digit pass
+       with the two forward kernels of kge_score_fwd, last pass and dedup with the two gradient
+       kernels of kge_score_bwd), which takes them off the critical path without a second stream.  insp_jobs then points to two jobs, [0] for concat(h, t, neg) and [1] for
+       r, whose `out` are the structs ent_insp / rel_insp point to.  Requirements: shared
+       negatives, each index set at most 65536 ids, tables of at most 2^22 rows
+       (kge_fused_inspection_ok says whether a batch qualifies); kge_score_fwd (with pos and
+       neg scores requested) and kge_score_bwd must both be called, in this order, on one stream,
+       and ent_insp / rel_insp hold the result only after kge_score_bwd.  No counterpart in the
+       reference, whose inspector is a separate call (apps/kge/kge.py:249-271). */
+    int32_t fuse_inspection;
+    const struct kge_inspect_job *insp_jobs;
 } kge_batch;
 
 /* Forward outputs that backward consumes. */
@@ -203,6 +214,9 @@ typedef struct kge_inspect_job {
     size_t workspace_bytes;
 } kge_inspect_job;
 int kge_inspect_batch(const kge_inspect_job *jobs, int n_jobs, void *stream);
+/* 1 if a batch with these two jobs (see kge_batch.fuse_inspection) can have its inspection fused
+   into the score kernels, else 0. */
+int kge_fused_inspection_ok(const kge_tables *tab, const kge_batch *bat, const kge_inspect_job *jobs);
 
 /*
  * Margin-ranking loss over score pairs and its gradient:

@@ -135,8 +135,9 @@ def test_transh_l1_generic_floats_differ_only_by_sign_flips(oracle):
     ("cfg3_transr", dict(batch=1024)),
 ])
 def test_train_step_eager_overlapped_and_graph_replays(oracle, name, over):
-    """The preallocated step: plain order, inspector overlapped on a side stream, and HIP-graph
-    replays (several, with eager work and synchronisation in between) all give the oracle's gradients."""
+    """The preallocated step: plain order, inspector overlapped on a side stream, inspector fused into
+    the score kernels' launches, and HIP-graph replays (several, with eager work and synchronisation in
+    between) all give the oracle's gradients."""
     from cuke_amd.kge import TrainStep
     w = synth.make_workload(name, **over)
     a = w.arrays
@@ -156,10 +157,13 @@ def test_train_step_eager_overlapped_and_graph_replays(oracle, name, over):
         compare(step.sparse_grads(), ref, f"{name} {tag}", outliers=(1e-5, 4.0) if w.model == "RotatE" else None)
         step.ent_rows.zero_()  # eager work between runs; also proves the next run rewrites everything
 
-    step.run(overlap=False)
+    step.run(overlap=False, fused=False)
     check("in order")
-    step.run(overlap=True)
+    step.run(overlap=True, fused=False)
     check("overlapped")
+    assert step.fusable == (w.chunk is not None and w.chunk > 0)
+    step.run()  # inspection fused into the score kernels' launches where the batch qualifies
+    check("fused" if step.fusable else "default")
     step.capture()
     for i in range(3):
         step.replay()
@@ -231,10 +235,42 @@ def test_train_step_pipelined_inspections(oracle, name, over, ahead):
                           k["arows"][:ur] if k["arows"] is not None else None)
         compare(got, ref, f"{name} pipelined step {i}", outliers=(1e-5, 4.0) if w.model == "RotatE" else None)
     # the plain mode still works afterwards, on the set of the step run last
-    step.run()
+    step.run(fused=False)
     torch.cuda.synchronize()
     ref = oracle.backward(w.model, a["E"], a["R"], a["A"], batches[-1]["h"], batches[-1]["r"], batches[-1]["t"],
                           batches[-1].get("neg"), w.chunk, step.dpos.cpu().numpy(),
                           step.dneg.cpu().numpy() if step.dneg is not None else None, p=w.norm_p)
     compare(step.sparse_grads(), ref, f"{name} plain run after the pipelined ones",
             outliers=(1e-5, 4.0) if w.model == "RotatE" else None)
+
+
+@pytest.mark.parametrize("model,p", [("DistMult", 2), ("ComplEx", 2), ("TransE", 1), ("TransH", 2), ("RotatE", 2)])
+@pytest.mark.parametrize("shape", [
+    dict(n_ent=50, n_rel=3, dim=24, batch=96, chunk=24, n_neg=40),              # one digit pass for both tables
+    dict(n_ent=70_000, n_rel=300, dim=32, batch=1100, chunk=100, n_neg=37),     # ragged block edges, two passes
+    dict(n_ent=3_000_000, n_rel=5000, dim=16, batch=4096, chunk=512, n_neg=512),  # 22-bit ids, several workgroups
+])
+@pytest.mark.parametrize("neg_mode", ["tail", "head"])
+def test_fused_inspection_matches_the_separate_inspector(oracle, model, p, shape, neg_mode):
+    """run(fused=True): the inspector's workgroups ride in the score kernels' launches.  Its outputs must
+    be bit-identical to the stand-alone inspector's, and the gradients must match the oracle."""
+    from cuke_amd.kge import TrainStep, inspect
+    w = synth.custom_workload(model, norm_p=p, sigma=0.2, gamma=4.0, ent_zipf=1.1, seed=7, lattice=(p == 1), **shape)
+    a = w.arrays
+    m, ix = gpu_model(w)
+    step = TrainStep(m, ix["h"], ix["r"], ix["t"], ix["neg"], w.chunk, neg_mode=neg_mode)
+    assert step.fusable
+    step.run(fused=True)
+    torch.cuda.synchronize()
+    want_e = inspect([ix["h"], ix["t"], ix["neg"]], w.n_ent)
+    want_r = inspect([ix["r"]], w.n_rel)
+    for got, want, what in ((step.ent_insp, want_e, "entities"), (step.rel_insp, want_r, "relations")):
+        u = want.num_unique
+        assert got.num_unique == u, what
+        for f in ("unique_ids", "seg_offsets"):
+            assert torch.equal(getattr(got, f)[:u + (f == "seg_offsets")], getattr(want, f)[:u + (f == "seg_offsets")]), (what, f)
+        for f in ("perm", "inverse", "sorted_seg"):
+            assert torch.equal(getattr(got, f), getattr(want, f)), (what, f)
+    ref = oracle.backward(w.model, a["E"], a["R"], a["A"], a["h"], a["r"], a["t"], a["neg"], w.chunk,
+                          step.dpos.cpu().numpy(), step.dneg.cpu().numpy(), p=p, neg_mode=neg_mode)
+    compare(step.sparse_grads(), ref, f"{model} fused {neg_mode}", outliers=(1e-5, 4.0) if model == "RotatE" else None)
