@@ -29,12 +29,12 @@ FP32_PEAK_TFLOPS = 157.3    # MI355X fp32 vector / fp32 MFMA, published
 # reads for the 256 MiB copy kernel of --calibrate-copy (fetch x2.000, write x1.000).  The
 # summaries the numbers come from are profiles/score_path_kernels_<workload>.txt.
 MEASURED_TRAFFIC_BYTES = {
-    "cfg1_transe": 1_664_832,      # score_pos_kernel
-    "cfg2_distmult": 12_964_826,   # score_neg_kernel
-    "cfg2_complex": 12_999_689,    # score_neg_kernel
-    "cfg3_transr": 164_198_860,    # transr_gemm_kernel<0>
-    "cfg4_rotate": 12_029_161,     # score_neg_kernel
-    "cfg5_transh": 530_513_415,    # score_neg_kernel
+    "cfg1_transe": 1_695_564,      # score_pos_kernel
+    "cfg2_distmult": 13_077_412,   # score_neg_mfma_kernel
+    "cfg2_complex": 13_099_832,    # score_neg_mfma_kernel
+    "cfg3_transr": 164_192_487,    # transr_plan_kernel + transr_gemm_kernel<0>
+    "cfg4_rotate": 12_060_452,     # score_neg_kernel
+    "cfg5_transh": 593_910_021,    # score_neg_kernel
 }
 
 
@@ -261,7 +261,7 @@ def main():
                             # RotatE: the rotated heads the positive kernel left behind (read-only here)
                             ctypes.c_void_p(step.residual.data_ptr()) if w.model == "RotatE" else None,
                             None, 0, stc)
-        kname = "score_neg_kernel"
+        kname = "score_neg_mfma_kernel" if w.model in ("DistMult", "ComplEx") else "score_neg_kernel"
         if w.model == "TransH":  # needs w.h from the positive kernel; time the pair and subtract
             t_pair = time_events(lambda: step.forward(stc), 100, torch)
             t_pos = time_events(lambda: L.kge_score_fwd(ctypes.byref(model._tab), ctypes.byref(step.bat),
@@ -301,7 +301,7 @@ def main():
                      "frac": achieved / HBM_PEAK_GBS, "traffic": MEASURED_TRAFFIC_BYTES.get(w.name),
                      "kernel_ms": k_ms,
                      "algorithmic_bytes_per_launch": k_bytes,
-                     ("fp32_mfma" if w.model == "TransR" else "fp32_valu"): {"flops_per_launch": k_flops,
+                     ("fp32_mfma" if w.model in ("TransR", "DistMult", "ComplEx") else "fp32_valu"): {"flops_per_launch": k_flops,
                                    "achieved_tflops": k_flops / (k_ms * 1e-3) / 1e12,
                                    "frac_of_157.3": k_flops / (k_ms * 1e-3) / 1e12 / FP32_PEAK_TFLOPS}},
     }
