@@ -270,7 +270,7 @@ __global__ __launch_bounds__(kSortThreads) void finalize_kernel(const uint32_t *
 // ---- small and medium inputs: the mid-path bodies as kernels of their own -------------------
 __global__ __launch_bounds__(kMidThreads) void inspect_mid_hist_kernel(MidJobs jobs)
 {
-    __shared__ uint32_t smem[kMaxBins];
+    __shared__ uint32_t smem[mid_hist_lds_words(kMaxBins, kMidMaxPass)];
     mid_hist_body(jobs.j[blockIdx.y], blockIdx.x, smem);
 }
 
@@ -379,7 +379,8 @@ int plan_fused_inspection(const kge_inspect_job *jobs, int slot, FusedInsp *out)
         J.hist = reinterpret_cast<uint32_t *>(ws + p.off_hist);
         blocks[q] = (int)ceil_div(n, kMidKeys);
         const int step = slot - (kFusedSlots - 2 - J.npass);
-        const int w = step == 0 ? (1 << J.db) : (step >= 1 && step <= J.npass ? mid_pass_lds_words(1 << J.db) : 0);
+        const int w = step == 0 ? mid_hist_lds_words(1 << J.db, J.npass)
+                                : (step >= 1 && step <= J.npass ? mid_pass_lds_words(1 << J.db) : 0);
         words = w > words ? w : words;
     }
     f.split = blocks[0];

@@ -127,8 +127,10 @@ __device__ __forceinline__ uint32_t *mid_hist(const MidJob &J, int pass)
     return J.hist + (size_t)pass * mid_blocks(J.n) * (1u << J.db);
 }
 
-// Step 0 of a job: digit histogram of this workgroup's own keys for the first pass; also clears
-// the workgroup's rows for the later passes, which the scatter steps fill through atomics.
+// Step 0 of a job: the digit histograms of this workgroup's own keys, one per pass (a histogram
+// does not depend on the order of the keys, so all passes' totals are known before any sorting).
+__host__ __device__ constexpr int mid_hist_lds_words(int bins, int npass) { return bins * npass; }
+
 __device__ __forceinline__ void mid_hist_body(const MidJob &J, int bx, uint32_t *smem)
 {
     __builtin_amdgcn_s_setprio(3);  // see mid_scatter_body
@@ -145,24 +147,24 @@ __device__ __forceinline__ void mid_hist_body(const MidJob &J, int bx, uint32_t 
         const int i = my0 + j * kMidThreads + tid;
         key[j] = src(i < n ? i : n - 1);
     }
-    for (int i = tid; i < bins; i += kMidThreads) smem[i] = 0;
+    for (int i = tid; i < bins * J.npass; i += kMidThreads) smem[i] = 0;
     __syncthreads();
 #pragma unroll
     for (int j = 0; j < kMidRounds; ++j)
-        if (my0 + j * kMidThreads + tid < n) atomicAdd(&smem[key[j] & mask], 1u);
+        if (my0 + j * kMidThreads + tid < n)
+            for (int p = 0; p < J.npass; ++p) atomicAdd(&smem[p * bins + ((key[j] >> (p * J.db)) & mask)], 1u);
     __syncthreads();
     const size_t row = (size_t)bx * bins;
-    for (int i = tid; i < bins; i += kMidThreads) {
-        mid_hist(J, 0)[row + i] = smem[i];
-        for (int p = 1; p < J.npass; ++p) mid_hist(J, p)[row + i] = 0;
-    }
+    for (int p = 0; p < J.npass; ++p)
+        for (int i = tid; i < bins; i += kMidThreads) mid_hist(J, p)[row + i] = smem[p * bins + i];
 }
 
-// One digit pass of job J for the keys [bx * kMidKeys, (bx + 1) * kMidKeys): bin starts and the
-// same-digit counts of the workgroups before this one come from the per-workgroup histograms (a
-// few coalesced loads per thread), the workgroup's own keys are ranked stably with wave ballots
-// and scattered; while scattering, every key is also counted into the next pass's histogram of
-// the workgroup its new position falls in (integer atomics: the counts do not depend on order).
+// One digit pass of job J for the keys [bx * kMidKeys, (bx + 1) * kMidKeys).  Bin starts come from
+// the column sums of the per-workgroup histograms (a few coalesced loads per thread).  The number
+// of same-digit keys in front of this workgroup comes from the same histograms in the first pass
+// (the keys are still in input order, workgroup by workgroup); in a later pass the workgroup counts
+// the digits of the sorted keys in front of it itself (batched loads, LDS atomics).  Its own keys
+// are ranked stably with wave ballots and scattered.
 template <bool FIRST>
 __device__ __forceinline__ void mid_scatter_body(const MidJob &J, int pass, int bx, uint32_t *smem)
 {
@@ -227,6 +229,23 @@ __device__ __forceinline__ void mid_scatter_body(const MidJob &J, int pass, int 
         for (int w = 0; w < kMidWaves; ++w) reinterpret_cast<uint4 *>(s_cnt + w * bins)[q] = make_uint4(0, 0, 0, 0);
     }
     __syncthreads();
+    if (pass > 0) {  // s_bef held the histogram-order count, which only the first pass can use
+        for (int i = tid; i < bins; i += kMidThreads) s_bef[i] = 0;
+        __syncthreads();
+        constexpr int kBatch = 16;  // unconditional loads in flight per thread
+        for (int i0 = 0; i0 < my0; i0 += kBatch * kMidThreads) {
+            uint32_t kb[kBatch];
+#pragma unroll
+            for (int u = 0; u < kBatch; ++u) {
+                const int i = i0 + u * kMidThreads + tid;
+                kb[u] = kin[i < my0 ? i : my0 - 1];
+            }
+#pragma unroll
+            for (int u = 0; u < kBatch; ++u)
+                if (i0 + u * kMidThreads + tid < my0) atomicAdd(&s_bef[(kb[u] >> shift) & mask], 1u);
+        }
+        __syncthreads();
+    }
     block_exclusive_scan(s_tot, bins, s_w);  // s_tot[bin] = first position of the bin
 
     const uint64_t lt_mask = lane ? (~0ull >> (kWave - lane)) : 0ull;
@@ -263,19 +282,15 @@ __device__ __forceinline__ void mid_scatter_body(const MidJob &J, int pass, int 
         }
     }
     __syncthreads();
-    uint32_t *Hn = pass + 1 < J.npass ? mid_hist(J, pass + 1) : nullptr;
 #pragma unroll
     for (int j = 0; j < kMidRounds; ++j) {
         const int i = my0 + wave * (kMidRounds * kWave) + j * kWave + lane;
-        const bool ok = i < n;
-        const uint32_t dg = (key[j] >> shift) & mask;
-        const uint32_t pos = ok ? s_cnt[wave * bins + dg] + lrank[j] : 0u;
-        if (ok) {
+        if (i < n) {
+            const uint32_t dg = (key[j] >> shift) & mask;
+            const uint32_t pos = s_cnt[wave * bins + dg] + lrank[j];
             kout[pos] = key[j];
             vout[pos] = val[j];
         }
-        // count the key into the next pass's histogram of the workgroup it lands in
-        if (Hn && ok) atomicAdd(&Hn[(pos / kMidKeys) * (uint32_t)bins + ((key[j] >> (shift + J.db)) & mask)], 1u);
     }
 }
 
