@@ -384,11 +384,12 @@ static int launch_neg_mp(const NegArgs &a, int64_t n_chunks, const FusedInsp &fi
     constexpr int NPA = (MODEL == KGE_ROTATE || MODEL == KGE_TRANSH) ? 2 : 1, NPT = MODEL == KGE_ROTATE ? 2 : 1;
     const int64_t big_tiles = ceil_div(a.C, 64) * ceil_div(a.N, 64) * n_chunks;
     int tile = neg_tile_override();
-    // 32x32 tiles up to about 1024 big tiles: more waves to hide latency (~20 % faster than 64x64
-    // on the 256-big-tile DistMult workload).  A launch that fills every slot of every CU would
-    // starve an inspection running next to it on another stream; the inspector kernels raise their
-    // wave priority for that reason.
-    if (tile != 2 && tile != 4 && tile != 3) tile = big_tiles >= 1024 ? 4 : 2;
+    // Small tiles up to about 1024 big tiles: more waves to hide latency (32x32 is ~20 % faster than
+    // 64x64 on a 256-big-tile workload with the vector-ALU loop; the matrix-core loop, whose
+    // launches are bound by the rows its workgroups pull from L2, does best with 32x64).  The
+    // inspector workgroups that share the machine with these launches raise their wave priority.
+    constexpr bool kDotModel = MODEL == KGE_DISTMULT || MODEL == KGE_COMPLEX;
+    if (tile != 2 && tile != 4 && tile != 3) tile = big_tiles >= 1024 ? 4 : (kDotModel ? 3 : 2);
     const int TB = tile == 4 ? 64 : 32, TN = tile == 2 ? 32 : 64;
     const dim3 grid(xcd_grid(ceil_div(a.N, TN), ceil_div(a.C, TB), n_chunks) + (unsigned)fi.blocks);
     if constexpr (MODEL == KGE_DISTMULT || MODEL == KGE_COMPLEX) {

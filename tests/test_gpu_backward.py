@@ -274,3 +274,23 @@ def test_fused_inspection_matches_the_separate_inspector(oracle, model, p, shape
     ref = oracle.backward(w.model, a["E"], a["R"], a["A"], a["h"], a["r"], a["t"], a["neg"], w.chunk,
                           step.dpos.cpu().numpy(), step.dneg.cpu().numpy(), p=p, neg_mode=neg_mode)
     compare(step.sparse_grads(), ref, f"{model} fused {neg_mode}", outliers=(1e-5, 4.0) if model == "RotatE" else None)
+
+
+def test_train_step_falls_back_to_the_stream_inspector_for_large_index_sets(oracle):
+    """More than 65536 ids in concat(h, t, neg): the batch does not qualify for the fused inspection, the
+    default run() uses the multi-block inspector on the side stream, and asking for fused=True is an error."""
+    from cuke_amd import KgeError
+    from cuke_amd.kge import TrainStep
+    w = synth.custom_workload("DistMult", n_ent=5000, n_rel=40, dim=8, batch=32768, chunk=4096, n_neg=512,
+                              sigma=0.2, ent_zipf=1.1, seed=2)
+    a = w.arrays
+    m, ix = gpu_model(w)
+    step = TrainStep(m, ix["h"], ix["r"], ix["t"], ix["neg"], w.chunk)
+    assert step.n_occ > 65536 and not step.fusable
+    with pytest.raises(KgeError):
+        step.run(fused=True)
+    step.run()
+    torch.cuda.synchronize()
+    ref = oracle.backward(w.model, a["E"], a["R"], a["A"], a["h"], a["r"], a["t"], a["neg"], w.chunk,
+                          step.dpos.cpu().numpy(), step.dneg.cpu().numpy())
+    compare(step.sparse_grads(), ref, "large index set, stream inspector")
