@@ -133,12 +133,14 @@ int kge_score_fwd(const kge_tables *tab, const kge_batch *bat, float *pos, float
     if (want_neg && tab->model == KGE_TRANSH && !side_pos) return KGE_EINVAL;
     if (want_neg && tab->model == KGE_ROTATE && !residual) return KGE_EINVAL;  // rotated heads buffer
     // fused inspection: first digit pass with the per-positive kernel, second with the tile kernel
-    const bool fuse = bat->fuse_inspection != 0;
+    const bool grouped_model = tab->model == KGE_TRANSR || tab->model == KGE_RESCAL;
+    const bool fuse = bat->fuse_inspection != 0 && !grouped_model;  // (the grouped kernels plan their own riders)
+    if (bat->fuse_inspection && grouped_model && !(bat->rel_insp && (pos || residual))) return KGE_EINVAL;
     FusedInsp fi0{}, fi1{};
     if (fuse) {
         if (!want_neg || !bat->insp_jobs || !(pos || side_pos || residual) || bat->batch == 0) return KGE_EINVAL;
-        if ((rc = plan_fused_inspection(bat->insp_jobs, 0, &fi0))) return rc;
-        if ((rc = plan_fused_inspection(bat->insp_jobs, 1, &fi1))) return rc;
+        if ((rc = plan_fused_inspection(bat->insp_jobs, 2, 0, &fi0))) return rc;
+        if ((rc = plan_fused_inspection(bat->insp_jobs, 2, 1, &fi1))) return rc;
     }
     if (pos || side_pos || residual) {
         if ((tab->model == KGE_TRANSR || tab->model == KGE_RESCAL) && bat->rel_insp)

@@ -326,6 +326,8 @@ static SortPlan make_plan(int64_t n, int64_t n_rows)
     return p;
 }
 
+bool transr_grouped_path_ok(const kge_tables *tab, const kge_batch *bat);  // transr.hip
+
 static int validate_job(const kge_inspect_job *job, Parts *parts, int64_t *n_out)
 {
     if (job->n_parts < 1 || job->n_parts > 4) return KGE_EINVAL;
@@ -348,13 +350,14 @@ static int validate_job(const kge_inspect_job *job, Parts *parts, int64_t *n_out
     return KGE_OK;
 }
 
-int plan_fused_inspection(const kge_inspect_job *jobs, int slot, FusedInsp *out)
+int plan_fused_inspection(const kge_inspect_job *jobs, int n_jobs, int slot, FusedInsp *out)
 {
-    if (!jobs || !out || slot < 0 || slot >= kFusedSlots) return KGE_EINVAL;
+    if (!jobs || !out || slot < 0 || slot >= kFusedSlots || n_jobs < 1 || n_jobs > 2) return KGE_EINVAL;
     FusedInsp f{};
+    f.n_jobs = n_jobs;
     int words = kMidDedupLdsWords;
-    int blocks[2];
-    for (int q = 0; q < 2; ++q) {
+    int blocks[2] = {0, 0};
+    for (int q = 0; q < n_jobs; ++q) {
         Parts parts;
         int64_t n;
         const int rc = validate_job(&jobs[q], &parts, &n);
@@ -488,7 +491,11 @@ int kge_inspect_batch(const kge_inspect_job *jobs, int n_jobs, void *stream)
                 else hipLaunchKernelGGL(inspect_mid_scatter_kernel<false>, grid, block, 0, st, mid, pass);
             }
         }
-        hipLaunchKernelGGL(inspect_mid_dedup_kernel, grid, block, 0, st, mid);
+        // (jobs with a single digit pass are finished by their scatter step; empty jobs still need
+        // the dedup step to write their zero counts)
+        bool need_dedup = false;
+        for (int q = 0; q < n_mid; ++q) need_dedup = need_dedup || mid.j[q].npass > 1 || mid.j[q].n == 0;
+        if (need_dedup) hipLaunchKernelGGL(inspect_mid_dedup_kernel, grid, block, 0, st, mid);
         KGE_CHECK_LAUNCH();
     }
     return KGE_OK;
@@ -496,13 +503,18 @@ int kge_inspect_batch(const kge_inspect_job *jobs, int n_jobs, void *stream)
 
 int kge_fused_inspection_ok(const kge_tables *tab, const kge_batch *bat, const kge_inspect_job *jobs)
 {
-    if (!tab || !bat || !jobs || !bat->neg || bat->batch <= 0) return 0;
+    if (!tab || !bat || !jobs || bat->batch <= 0) return 0;
     switch (tab->model) {
-    case KGE_TRANSE: case KGE_TRANSH: case KGE_DISTMULT: case KGE_COMPLEX: case KGE_ROTATE: break;
-    default: return 0;  // no shared-negative kernels to ride with
+    case KGE_TRANSE: case KGE_TRANSH: case KGE_DISTMULT: case KGE_COMPLEX: case KGE_ROTATE:
+        if (!bat->neg) return 0;  // the shared-negative kernels are the hosts
+        break;
+    case KGE_TRANSR: case KGE_RESCAL:
+        if (bat->neg || !transr_grouped_path_ok(tab, bat)) return 0;  // the grouped MFMA kernels are the hosts
+        break;
+    default: return 0;
     }
     FusedInsp f;
-    return plan_fused_inspection(jobs, 0, &f) == KGE_OK ? 1 : 0;
+    return plan_fused_inspection(jobs, fused_job_count(tab->model), 0, &f) == KGE_OK ? 1 : 0;
 }
 
 int kge_inspect(const int64_t *const *parts_in, const int64_t *part_len, int n_parts, int64_t n_rows,

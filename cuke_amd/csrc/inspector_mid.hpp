@@ -107,9 +107,11 @@ struct MidJobs {
 // has np + 2 steps (histogram, np scatters, dedup), one per launch; the four hosts of a
 // shared-negative training step are, in order, the per-positive forward kernel, the forward tile
 // kernel, the gradient tile kernel and the per-positive gradient kernel (slot 0..3), and a job
-// uses the last np + 2 of them.  Workgroup b < blocks belongs to job 0 if b < split, else job 1.
+// uses the last np + 2 of them (grouped TransR / RESCAL steps: forward GEMM, prep, dX GEMM, dM).
+// Workgroup b < blocks belongs to job 0 if b < split, else job 1.
 struct FusedInsp {
     MidJob j[2];
+    int n_jobs;  // 1 or 2
     int blocks;  // a multiple of 8, so the host's own workgroups keep their XCD (0: nothing fused)
     int split;   // workgroups of job 0
     int slot;
@@ -117,7 +119,7 @@ struct FusedInsp {
 };
 
 // LDS words a digit pass with `bins` bins needs
-__host__ __device__ constexpr int mid_pass_lds_words(int bins) { return (2 + kMidWaves) * bins + kMidWaves; }
+__host__ __device__ constexpr int mid_pass_lds_words(int bins) { return (3 + kMidWaves) * bins + kMidWaves; }
 
 // Workgroups of a job, and the per-workgroup digit histograms of pass p in the job's workspace
 // (kMidMaxPass tables of [workgroups][bins] counters).
@@ -246,7 +248,33 @@ __device__ __forceinline__ void mid_scatter_body(const MidJob &J, int pass, int 
         }
         __syncthreads();
     }
+    // A job with a single pass sorts by the whole key, so every non-empty bin is one distinct id:
+    // the run structure falls out of the histogram and no dedup step is needed.
+    const bool finish = J.npass == 1;
+    uint32_t *s_u = s_w + kMidWaves;  // finish: number of non-empty bins below this one
+    uint32_t nonempty = 0, n_unique = 0;  // bit u of nonempty: bin tid + 256 u has keys
+    if (finish) {
+        for (int u = 0, bin = tid; bin < bins; ++u, bin += kMidThreads) {
+            const uint32_t f = s_tot[bin] > 0 ? 1u : 0u;
+            nonempty |= f << u;
+            s_u[bin] = f;
+        }
+        __syncthreads();
+        block_exclusive_scan(s_u, bins, s_w);
+        n_unique = s_u[bins - 1] + (s_tot[bins - 1] > 0 ? 1u : 0u);
+    }
     block_exclusive_scan(s_tot, bins, s_w);  // s_tot[bin] = first position of the bin
+    if (finish && bx == 0) {
+        for (int u = 0, bin = tid; bin < bins; ++u, bin += kMidThreads)
+            if ((nonempty >> u) & 1u) {
+                J.out.unique_ids[s_u[bin]] = (int64_t)bin;
+                J.out.seg_offsets[s_u[bin]] = (int32_t)s_tot[bin];
+            }
+        if (tid == 0) {
+            J.out.num_unique[0] = (int32_t)n_unique;
+            J.out.seg_offsets[n_unique] = n;
+        }
+    }
 
     const uint64_t lt_mask = lane ? (~0ull >> (kWave - lane)) : 0ull;
     uint32_t lrank[kMidRounds];
@@ -290,6 +318,10 @@ __device__ __forceinline__ void mid_scatter_body(const MidJob &J, int pass, int 
             const uint32_t pos = s_cnt[wave * bins + dg] + lrank[j];
             kout[pos] = key[j];
             vout[pos] = val[j];
+            if (finish) {
+                J.out.sorted_seg[pos] = (int32_t)s_u[dg];
+                J.out.inverse[val[j]] = (int32_t)s_u[dg];
+            }
         }
     }
 }
@@ -303,7 +335,7 @@ __device__ __forceinline__ void mid_dedup_body(const MidJob &J, int bx, uint32_t
     __builtin_amdgcn_s_setprio(3);
     const int n = (int)J.n;
     const int nblk = n > 0 ? (n + kMidKeys - 1) / kMidKeys : 1;
-    if (bx >= nblk) return;
+    if (bx >= nblk || (J.npass == 1 && n > 0)) return;  // single pass: finished by the scatter step
     const int tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid >> 6;
     const uint32_t *keys = J.keys_final;
     const int my0 = bx * kMidKeys;
@@ -386,6 +418,7 @@ __device__ __forceinline__ bool fused_insp_block(const FusedInsp &f, uint32_t *s
 {
     const int b = blockIdx.x;
     if (b >= f.blocks) return false;
+    if (b >= f.split && f.n_jobs < 2) return true;  // padding up to a multiple of 8 workgroups
     const MidJob &J = f.j[b < f.split ? 0 : 1];
     const int bx = b < f.split ? b : b - f.split;
     const int step = f.slot - (kFusedSlots - 2 - J.npass);  // 0: histogram, 1..np: scatter, np + 1: dedup
@@ -396,8 +429,14 @@ __device__ __forceinline__ bool fused_insp_block(const FusedInsp &f, uint32_t *s
     return true;
 }
 
-// host side (inspector.hip): fills `out` for one slot from two inspection jobs; KGE_EUNSUPPORTED
-// when a job is too large or its table needs more than two digit passes of kMaxDigitBits bits
-int plan_fused_inspection(const kge_inspect_job *jobs, int slot, FusedInsp *out);
+// host side (inspector.hip): fills `out` for one slot from one or two inspection jobs;
+// KGE_EUNSUPPORTED when a job is too large or its table needs more than two digit passes of
+// kMaxDigitBits bits
+int plan_fused_inspection(const kge_inspect_job *jobs, int n_jobs, int slot, FusedInsp *out);
+
+// Jobs that ride with a model's kernels: both index sets with the shared-negative kernels, the
+// entity set alone with the grouped TransR / RESCAL kernels (their relation groups must exist
+// before the forward pass starts).
+inline int fused_job_count(int model) { return model == KGE_TRANSR || model == KGE_RESCAL ? 1 : 2; }
 
 }  // namespace kge

@@ -832,8 +832,8 @@ int kge_score_bwd(const kge_tables *tab, const kge_batch *bat, const kge_saved *
     FusedInsp fi_pass{}, fi_dedup{};
     if (bat->fuse_inspection) {
         if (!have_neg || !bat->insp_jobs) return KGE_EINVAL;
-        if ((rc = plan_fused_inspection(bat->insp_jobs, 2, &fi_pass))) return rc;
-        if ((rc = plan_fused_inspection(bat->insp_jobs, 3, &fi_dedup))) return rc;
+        if ((rc = plan_fused_inspection(bat->insp_jobs, 2, 2, &fi_pass))) return rc;
+        if ((rc = plan_fused_inspection(bat->insp_jobs, 2, 3, &fi_dedup))) return rc;
     }
 
     if (have_neg) {

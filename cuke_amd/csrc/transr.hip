@@ -14,7 +14,7 @@
 //     float4 of the staged row;
 //   * j: a lane's float4 of four consecutive matrix columns feeds four MFMAs (one per element),
 //     so MFMA e owns columns n0 + 4 (l % 16) + e.
-#include "common.hpp"
+#include "inspector_mid.hpp"
 #include "seg_reduce.hpp"
 
 namespace kge {
@@ -456,25 +456,27 @@ __device__ __forceinline__ void gemm_sweep(const float *M, const float *sX, int 
 // MODE 1: forward RESCAL   x = E[h],      y = x M,        score = y . E[t]
 // MODE 2: backward dX      x = xs rows,   y = x M^T -> occ_h = y, occ_t = -y (when occ_t is set)
 template <int MODE>
-__global__ __launch_bounds__(256, KGE_TR_OCC) void transr_gemm_kernel(GemmArgs a)
+__global__ __launch_bounds__(256, KGE_TR_OCC) void transr_gemm_kernel(GemmArgs a, FusedInsp fi)
 {
     extern __shared__ __align__(16) float lds[];
+    if (fused_insp_block(fi, reinterpret_cast<uint32_t *>(lds))) return;  // an inspector workgroup riding along
+    const int bid = (int)blockIdx.x - fi.blocks;
     // Workgroups [0, max_tiles) take the planned 32-triple tiles, the following `thin_groups`
     // stream the thin group tails.  The tiles come first because each is one long chain of
     // dependent loads and matrix-core steps (about 20 us whatever else runs); the thin
     // workgroups then fill the remaining slots and the memory bandwidth.
-    if ((int)blockIdx.x >= a.max_tiles) {
+    if (bid >= a.max_tiles) {
         if constexpr (MODE == 2) {
             const int ns = (a.d / 4 + 15) / 16;  // k-quads per lane of a 16-lane row group
-            if (ns <= 1) transr_thin_dx_body<1>(a, lds, blockIdx.x - a.max_tiles);
-            else if (ns <= 2) transr_thin_dx_body<2>(a, lds, blockIdx.x - a.max_tiles);
-            else transr_thin_dx_body<4>(a, lds, blockIdx.x - a.max_tiles);
+            if (ns <= 1) transr_thin_dx_body<1>(a, lds, bid - a.max_tiles);
+            else if (ns <= 2) transr_thin_dx_body<2>(a, lds, bid - a.max_tiles);
+            else transr_thin_dx_body<4>(a, lds, bid - a.max_tiles);
         } else {
-            transr_thin_fwd_body<MODE>(a, lds, blockIdx.x - a.max_tiles);
+            transr_thin_fwd_body<MODE>(a, lds, bid - a.max_tiles);
         }
         return;
     }
-    const int tile = blockIdx.x;
+    const int tile = bid;
     if (tile >= a.plan.num_tiles[0]) return;
     const int d = a.d;
     const int kpad = (d + 15) & ~15;
@@ -645,6 +647,11 @@ static bool mfma_path_ok(const kge_tables *tab, const kge_batch *bat)
            aligned16(tab->aux) && (!tab->rel || aligned16(tab->rel)) && bat->rel_insp->n == bat->batch;
 }
 
+bool transr_grouped_path_ok(const kge_tables *tab, const kge_batch *bat)
+{
+    return mfma_path_ok(tab, bat) && gemm_lds_bytes((int)tab->dim) <= 64 * 1024;
+}
+
 // ---- backward kernels ----------------------------------------------------------------------
 struct PrepArgs {
     const float *ent;
@@ -659,10 +666,12 @@ struct PrepArgs {
 
 // One wave per sorted position p (triple b = perm[p]):
 //   TransR: xs[p] = E[h]-E[t], qs[p] = g * d||e||/de     RESCAL: xs[p] = E[h], qs[p] = g * E[t], occ_t[b] = g * v
-__global__ __launch_bounds__(256) void transr_prep_kernel(PrepArgs a)
+__global__ __launch_bounds__(256) void transr_prep_kernel(PrepArgs a, FusedInsp fi)
 {
+    extern __shared__ __align__(16) float lds[];  // inspector workgroups only
+    if (fused_insp_block(fi, reinterpret_cast<uint32_t *>(lds))) return;
     const int lane = threadIdx.x & 63;
-    const int64_t p = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    const int64_t p = (int64_t)((int)blockIdx.x - fi.blocks) * 4 + (threadIdx.x >> 6);
     if (p >= a.B) return;
     const int b = a.perm[p];
     const int d = a.d;
@@ -803,18 +812,20 @@ __device__ __forceinline__ void dm_sweep(const float *xs, const float *qs, int d
 // of one group, 32 rows i); the four waves split the columns j; K runs over the chunk's triples,
 // operands prefetched four supersteps ahead.  Groups longer than one chunk write per-chunk
 // partial matrices that transr_dm_finish_kernel adds up (keeps the longest K loop at 16 supersteps).
-__global__ __launch_bounds__(256, KGE_TR_OCC) void transr_dm_kernel(DmArgs a)
+__global__ __launch_bounds__(256, KGE_TR_OCC) void transr_dm_kernel(DmArgs a, FusedInsp fi)
 {
-    extern __shared__ __align__(16) float lds[];  // thin groups only: d float4
-    if ((int)blockIdx.x >= a.max_items) {
-        transr_thin_dm_body(a, lds, blockIdx.x - a.max_items);
+    extern __shared__ __align__(16) float lds[];  // thin groups: d float4; inspector workgroups: their own need
+    if (fused_insp_block(fi, reinterpret_cast<uint32_t *>(lds))) return;
+    const int bid = (int)blockIdx.x - fi.blocks;
+    if (bid >= a.max_items) {
+        transr_thin_dm_body(a, lds, bid - a.max_items);
         return;
     }
     const int d = a.d;
     const int nib = (d + 31) / 32;
-    const int tile = blockIdx.x / nib;
+    const int tile = bid / nib;
     if (tile >= a.plan.num_tiles[0]) return;
-    const int i0 = (blockIdx.x % nib) * 32;
+    const int i0 = (bid % nib) * 32;
     const int g = a.plan.tile_seg[tile];
     const int s0 = a.plan.tile_p0[tile];
     const int seg_end = a.seg_offsets[g + 1];
@@ -925,14 +936,26 @@ size_t transr_fwd_workspace(const kge_tables *tab, const kge_batch *bat)
     return up256(sizeof(int32_t) * plan_ints(max_tiles(tab, bat), 0));
 }
 
+static size_t lds_with(const FusedInsp &fi, size_t own)
+{
+    return fi.blocks > 0 && (size_t)fi.lds_bytes > own ? (size_t)fi.lds_bytes : own;
+}
+
 int launch_transr_fwd(const kge_tables *tab, const kge_batch *bat, float *pos, float *resid, void *workspace,
                       size_t workspace_bytes, hipStream_t st)
 {
     if (bat->batch == 0) return KGE_OK;
     const bool rescal = tab->model == KGE_RESCAL;
-    if (!mfma_path_ok(tab, bat) || !workspace || workspace_bytes < transr_fwd_workspace(tab, bat) ||
-        gemm_lds_bytes((int)tab->dim) > 64 * 1024)
-        return launch_score_pos(tab, bat, pos, resid, nullptr, st);
+    const bool grouped = mfma_path_ok(tab, bat) && workspace && workspace_bytes >= transr_fwd_workspace(tab, bat) &&
+                         gemm_lds_bytes((int)tab->dim) <= 64 * 1024;
+    // fused entity inspection: its histogram step rides with the forward GEMM
+    FusedInsp fi{};
+    if (bat->fuse_inspection) {
+        if (!grouped || !bat->insp_jobs || bat->neg) return KGE_EINVAL;
+        const int rc = plan_fused_inspection(bat->insp_jobs, 1, 0, &fi);
+        if (rc) return rc;
+    }
+    if (!grouped) return launch_score_pos(tab, bat, pos, resid, nullptr, st);
     const kge_inspection *ri = bat->rel_insp;
     const int64_t tiles = max_tiles(tab, bat);
     TilePlan plan = plan_at(workspace, tiles, 0);
@@ -940,12 +963,12 @@ int launch_transr_fwd(const kge_tables *tab, const kge_batch *bat, float *pos, f
                        plan, kTM);
     GemmArgs a{tab->ent, tab->rel, tab->aux, bat->h, bat->r, bat->t, ri->perm, ri->seg_offsets, ri->num_unique, ri->unique_ids,
                plan, nullptr, pos, resid, nullptr, nullptr, (int)tab->dim, tab->norm_p, thin_groups(tab, bat), (int)tiles};
-    const size_t lds = gemm_lds_bytes((int)tab->dim);
-    const dim3 grid((unsigned)(tiles + a.thin_groups));
+    const size_t lds = lds_with(fi, gemm_lds_bytes((int)tab->dim));
+    const dim3 grid((unsigned)(tiles + a.thin_groups + fi.blocks));
     if (rescal)
-        hipLaunchKernelGGL(transr_gemm_kernel<1>, grid, dim3(256), lds, st, a);
+        hipLaunchKernelGGL(transr_gemm_kernel<1>, grid, dim3(256), lds, st, a, fi);
     else
-        hipLaunchKernelGGL(transr_gemm_kernel<0>, grid, dim3(256), lds, st, a);
+        hipLaunchKernelGGL(transr_gemm_kernel<0>, grid, dim3(256), lds, st, a, fi);
     KGE_CHECK_LAUNCH();
     return KGE_OK;
 }
@@ -974,20 +997,30 @@ int launch_transr_bwd(const kge_tables *tab, const kge_batch *bat, const kge_sav
 
     PrepArgs pa{tab->ent, bat->h, bat->t, ri->perm, dpos, saved->pos, saved->residual, xs, qs, occ + B * d, B, d,
                 tab->norm_p, rescal ? 1 : 0};
-    hipLaunchKernelGGL(transr_prep_kernel, dim3((unsigned)ceil_div(B, 4)), dim3(256), 0, st, pa);
+    // fused entity inspection: first digit pass with prep, second with the dX GEMM, dedup with dM
+    FusedInsp f1{}, f2{}, f3{};
+    if (bat->fuse_inspection) {
+        if (!bat->insp_jobs) return KGE_EINVAL;
+        int rc;
+        if ((rc = plan_fused_inspection(bat->insp_jobs, 1, 1, &f1))) return rc;
+        if ((rc = plan_fused_inspection(bat->insp_jobs, 1, 2, &f2))) return rc;
+        if ((rc = plan_fused_inspection(bat->insp_jobs, 1, 3, &f3))) return rc;
+    }
+    hipLaunchKernelGGL(transr_prep_kernel, dim3((unsigned)(ceil_div(B, 4) + f1.blocks)), dim3(256), lds_with(f1, 0), st, pa,
+                       f1);
     hipLaunchKernelGGL(transr_plan_kernel, dim3(2), dim3(1024), 0, st, ri->num_unique, ri->seg_offsets, plan, kTM,
                        dplan, kDmChunk);
     // dX = Q M^T -> occurrence rows of h (and -dX for t)
     GemmArgs ga{tab->ent, tab->rel, tab->aux, bat->h, bat->r, bat->t, ri->perm, ri->seg_offsets, ri->num_unique, ri->unique_ids,
                 plan, qs, nullptr, nullptr, occ, rescal ? nullptr : occ + B * d, d, tab->norm_p, thin_groups(tab, bat), (int)p.tiles};
-    hipLaunchKernelGGL(transr_gemm_kernel<2>, dim3((unsigned)(p.tiles + ga.thin_groups)), dim3(256), gemm_lds_bytes(d),
-                       st, ga);
+    hipLaunchKernelGGL(transr_gemm_kernel<2>, dim3((unsigned)(p.tiles + ga.thin_groups + f2.blocks)), dim3(256),
+                       lds_with(f2, gemm_lds_bytes(d)), st, ga, f2);
     // dM = X^T Q per relation group
     const int dm_items = (int)(ceil_div(d, 32) * p.dtiles);
     DmArgs da{xs, qs, ri->seg_offsets, dplan, grads->aux_rows, reinterpret_cast<float *>(ws + p.off_dpart), d,
               ri->num_unique, dm_items};
-    hipLaunchKernelGGL(transr_dm_kernel, dim3((unsigned)(dm_items + thin_groups(tab, bat))), dim3(256),
-                       sizeof(float) * 4 * (size_t)d, st, da);
+    hipLaunchKernelGGL(transr_dm_kernel, dim3((unsigned)(dm_items + thin_groups(tab, bat) + f3.blocks)), dim3(256),
+                       lds_with(f3, sizeof(float) * 4 * (size_t)d), st, da, f3);
     hipLaunchKernelGGL(transr_dm_finish_kernel, dim3((unsigned)ceil_div((int64_t)d * d / 4, 256), (unsigned)p.dsplit),
                        dim3(256), 0, st, da);
     KGE_CHECK_LAUNCH();

@@ -599,10 +599,12 @@ class TrainStep:
     def run(self, backward=True, overlap=True, pipeline=False, inputs_ready=None, fused=None):
         """Enqueue one step.
 
-        fused (default whenever the batch qualifies: shared negatives, index sets of at most 65536
-        ids): no inspector kernels at all -- the inspector's workgroups ride in front of the
-        score kernels' own workgroups in the same launches, so the whole step is one chain of
-        kernels on one stream with the inspection off its critical path.
+        fused (default whenever the batch qualifies: index sets of at most 65536 ids; shared
+        negatives, or TransR / RESCAL on their grouped path): the inspector's workgroups ride in
+        front of the score kernels' own workgroups in the same launches, so the whole step is one
+        chain of kernels on one stream with the inspection off its critical path.  TransR /
+        RESCAL inspect the relations first (the forward pass is planned from their groups); only
+        the entity inspection rides.
 
         Otherwise, with overlap, the inspector runs on a side stream while the main stream
         computes scores and per-occurrence gradients; backward waits for it right before its
@@ -625,6 +627,8 @@ class TrainStep:
             bat = self.bat
             bat.insp_ready, bat.fuse_inspection = None, 1
             try:
+                if self.needs_rel_groups:  # the forward pass is planned from the relation groups
+                    _lib.check(self.L.kge_inspect_batch(C.byref(self._jobs[1]), 1, st), "kge_inspect_batch(relations)")
                 self.forward(st)
                 self.loss_grad(st)
                 self.backward(st)

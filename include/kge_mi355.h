@@ -117,16 +117,21 @@ typedef struct kge_batch {
        (neg_k, r_b, t_b), the head-corrupted batches of apps/kge/data/sampler.py:287-353
        (neg_head).  Zero-initialised structs get KGE_NEG_TAIL. */
     int32_t neg_mode;
-    /* Non-zero: the inspections are not run by kge_inspect* at all; their workgroups ride in
-       front of the score kernels' own in the same launches (histogram and first digit pass
-       with the two forward kernels of kge_score_fwd, last pass and dedup with the two gradient
-       kernels of kge_score_bwd), which takes them off the critical path without a second stream.  insp_jobs then points to two jobs, [0] for concat(h, t, neg) and [1] for
-       r, whose `out` are the structs ent_insp / rel_insp point to.  Requirements: shared
-       negatives, each index set at most 65536 ids, tables of at most 2^22 rows
-       (kge_fused_inspection_ok says whether a batch qualifies); kge_score_fwd (with pos and
-       neg scores requested) and kge_score_bwd must both be called, in this order, on one stream,
-       and ent_insp / rel_insp hold the result only after kge_score_bwd.  No counterpart in the
-       reference, whose inspector is a separate call (apps/kge/kge.py:249-271). */
+    /* Non-zero: the inspector's workgroups ride in front of the score kernels' own in the same
+       launches, which takes the inspection off the critical path without a second stream.
+       insp_jobs points to two jobs, [0] for the entity index set (concat(h, t, neg)) and [1] for r,
+       whose `out` are the structs ent_insp / rel_insp point to.
+       - Shared negatives (TransE, TransH, DistMult, ComplEx, RotatE): both jobs ride; histogram
+         and first digit pass with the two forward kernels of kge_score_fwd (pos and neg scores
+         must be requested), last pass and dedup with the two gradient kernels of kge_score_bwd.
+       - TransR / RESCAL on their grouped path (no negatives, rel_insp complete before
+         kge_score_fwd): job [0] rides with the forward GEMM, then with the prep, dX and dM kernels
+         of kge_score_bwd; job [1] is not used.
+       Requirements: each riding index set at most 65536 ids, tables of at most 2^22 rows
+       (kge_fused_inspection_ok says whether a batch qualifies); kge_score_fwd and kge_score_bwd
+       must both be called, in this order, on one stream, and the riding inspections hold their
+       result only after kge_score_bwd.  No counterpart in the reference, whose inspector is a
+       separate call (apps/kge/kge.py:249-271). */
     int32_t fuse_inspection;
     const struct kge_inspect_job *insp_jobs;
 } kge_batch;

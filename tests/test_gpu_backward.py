@@ -161,7 +161,7 @@ def test_train_step_eager_overlapped_and_graph_replays(oracle, name, over):
     check("in order")
     step.run(overlap=True, fused=False)
     check("overlapped")
-    assert step.fusable == (w.chunk is not None and w.chunk > 0)
+    assert step.fusable
     step.run()  # inspection fused into the score kernels' launches where the batch qualifies
     check("fused" if step.fusable else "default")
     step.capture()
@@ -294,3 +294,31 @@ def test_train_step_falls_back_to_the_stream_inspector_for_large_index_sets(orac
     ref = oracle.backward(w.model, a["E"], a["R"], a["A"], a["h"], a["r"], a["t"], a["neg"], w.chunk,
                           step.dpos.cpu().numpy(), step.dneg.cpu().numpy())
     compare(step.sparse_grads(), ref, "large index set, stream inspector")
+
+
+@pytest.mark.parametrize("model", ["TransR", "RESCAL"])
+@pytest.mark.parametrize("shape", [
+    dict(n_ent=900, n_rel=37, dim=32, batch=3001),        # ragged last workgroup, two digit passes
+    dict(n_ent=60, n_rel=5, dim=16, batch=700),           # one digit pass: finished by the scatter step
+    dict(n_ent=2_000_000, n_rel=700, dim=8, batch=20000),  # 21-bit ids, 40 inspector workgroups
+])
+def test_fused_entity_inspection_with_the_grouped_projection_kernels(oracle, model, shape):
+    """TransR / RESCAL: the relation inspection runs first, the entity inspection rides with the forward GEMM,
+    prep, dX GEMM and dM kernels.  Bit-identical to the stand-alone inspector; gradients vs the oracle."""
+    from cuke_amd.kge import TrainStep, inspect
+    w = synth.custom_workload(model, norm_p=2, sigma=0.2, rel_zipf=1.1, seed=5, **shape)
+    a = w.arrays
+    m, ix = gpu_model(w)
+    step = TrainStep(m, ix["h"], ix["r"], ix["t"])
+    assert step.fusable
+    step.run(fused=True)
+    torch.cuda.synchronize()
+    want = inspect([ix["h"], ix["t"]], w.n_ent)
+    got, u = step.ent_insp, want.num_unique
+    assert got.num_unique == u
+    assert torch.equal(got.unique_ids[:u], want.unique_ids[:u]) and torch.equal(got.seg_offsets[:u + 1], want.seg_offsets[:u + 1])
+    for f in ("perm", "inverse", "sorted_seg"):
+        assert torch.equal(getattr(got, f), getattr(want, f)), f
+    ref = oracle.backward(w.model, a["E"], a["R"], a["A"], a["h"], a["r"], a["t"], None, 0,
+                          step.dpos.cpu().numpy(), None, p=2)
+    compare(step.sparse_grads(), ref, f"{model} fused entity inspection")
