@@ -48,7 +48,8 @@ class Batch(C.Structure):
 
 class Saved(C.Structure):
     _fields_ = [("pos", C.c_void_p), ("neg", C.c_void_p), ("side_pos", C.c_void_p),
-                ("side_neg", C.c_void_p), ("residual", C.c_void_p)]
+                ("side_neg", C.c_void_p), ("residual", C.c_void_p),
+                ("fwd_workspace", C.c_void_p), ("fwd_workspace_bytes", C.c_size_t)]
 
 
 class Grads(C.Structure):

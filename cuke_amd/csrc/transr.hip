@@ -931,9 +931,18 @@ static TilePlan plan_at(void *base, int64_t tiles, int64_t split)
     return p;
 }
 
-size_t transr_fwd_workspace(const kge_tables *tab, const kge_batch *bat)
+// The forward workspace holds both tile plans of the batch: the 32-triple tiles of the GEMM kernels
+// and the chunked plan of the dM kernel.  A backward pass that is handed this workspace
+// (kge_saved.fwd_workspace) finds its plans there and launches no plan kernel of its own.
+static size_t fwd_plan_bytes(const kge_tables *tab, const kge_batch *bat)
 {
     return up256(sizeof(int32_t) * plan_ints(max_tiles(tab, bat), 0));
+}
+
+size_t transr_fwd_workspace(const kge_tables *tab, const kge_batch *bat)
+{
+    const RPlan p = make_rplan(tab, bat);
+    return fwd_plan_bytes(tab, bat) + up256(sizeof(int32_t) * plan_ints(p.dtiles, p.dsplit));
 }
 
 static size_t lds_with(const FusedInsp &fi, size_t own)
@@ -959,8 +968,10 @@ int launch_transr_fwd(const kge_tables *tab, const kge_batch *bat, float *pos, f
     const kge_inspection *ri = bat->rel_insp;
     const int64_t tiles = max_tiles(tab, bat);
     TilePlan plan = plan_at(workspace, tiles, 0);
-    hipLaunchKernelGGL(transr_plan_kernel, dim3(1), dim3(1024), 0, st, ri->num_unique, ri->seg_offsets, plan, kTM,
-                       plan, kTM);
+    const RPlan rp = make_rplan(tab, bat);
+    TilePlan dplan = plan_at(static_cast<char *>(workspace) + fwd_plan_bytes(tab, bat), rp.dtiles, rp.dsplit);
+    hipLaunchKernelGGL(transr_plan_kernel, dim3(2), dim3(1024), 0, st, ri->num_unique, ri->seg_offsets, plan, kTM,
+                       dplan, kDmChunk);
     GemmArgs a{tab->ent, tab->rel, tab->aux, bat->h, bat->r, bat->t, ri->perm, ri->seg_offsets, ri->num_unique, ri->unique_ids,
                plan, nullptr, pos, resid, nullptr, nullptr, (int)tab->dim, tab->norm_p, thin_groups(tab, bat), (int)tiles};
     const size_t lds = lds_with(fi, gemm_lds_bytes((int)tab->dim));
@@ -992,8 +1003,12 @@ int launch_transr_bwd(const kge_tables *tab, const kge_batch *bat, const kge_sav
     float *xs = reinterpret_cast<float *>(ws + p.off_xs), *qs = reinterpret_cast<float *>(ws + p.off_qs);
     float *occ = reinterpret_cast<float *>(ws + p.off_occ);
     const kge_inspection *ri = bat->rel_insp;
-    TilePlan plan = plan_at(ws + p.off_plan, p.tiles, 0);
-    TilePlan dplan = plan_at(ws + p.off_dplan, p.dtiles, p.dsplit);
+    // the plans: left behind by the forward pass, or built here
+    const bool have_plans = saved->fwd_workspace && saved->fwd_workspace_bytes >= transr_fwd_workspace(tab, bat);
+    char *pbase = have_plans ? static_cast<char *>(const_cast<void *>(saved->fwd_workspace)) : nullptr;
+    TilePlan plan = have_plans ? plan_at(pbase, p.tiles, 0) : plan_at(ws + p.off_plan, p.tiles, 0);
+    TilePlan dplan = have_plans ? plan_at(pbase + fwd_plan_bytes(tab, bat), p.dtiles, p.dsplit)
+                                : plan_at(ws + p.off_dplan, p.dtiles, p.dsplit);
 
     PrepArgs pa{tab->ent, bat->h, bat->t, ri->perm, dpos, saved->pos, saved->residual, xs, qs, occ + B * d, B, d,
                 tab->norm_p, rescal ? 1 : 0};
@@ -1008,8 +1023,9 @@ int launch_transr_bwd(const kge_tables *tab, const kge_batch *bat, const kge_sav
     }
     hipLaunchKernelGGL(transr_prep_kernel, dim3((unsigned)(ceil_div(B, 4) + f1.blocks)), dim3(256), lds_with(f1, 0), st, pa,
                        f1);
-    hipLaunchKernelGGL(transr_plan_kernel, dim3(2), dim3(1024), 0, st, ri->num_unique, ri->seg_offsets, plan, kTM,
-                       dplan, kDmChunk);
+    if (!have_plans)
+        hipLaunchKernelGGL(transr_plan_kernel, dim3(2), dim3(1024), 0, st, ri->num_unique, ri->seg_offsets, plan, kTM,
+                           dplan, kDmChunk);
     // dX = Q M^T -> occurrence rows of h (and -dX for t)
     GemmArgs ga{tab->ent, tab->rel, tab->aux, bat->h, bat->r, bat->t, ri->perm, ri->seg_offsets, ri->num_unique, ri->unique_ids,
                 plan, qs, nullptr, nullptr, occ, rescal ? nullptr : occ + B * d, d, tab->norm_p, thin_groups(tab, bat), (int)p.tiles};

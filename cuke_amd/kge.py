@@ -465,6 +465,8 @@ class TrainStep:
                 self.dneg = torch.ones((B, N), **f32) if dneg is None else dneg.to(**f32).contiguous()
         self.saved = _lib.Saved(*[(x.data_ptr() if x is not None else None) for x in
                                   (self.pos, self.neg, self.side_pos, self.side_neg, self.residual)])
+        if self.needs_rel_groups and self._ws_f_bytes:  # backward reuses the forward pass's tile plans
+            self.saved.fwd_workspace, self.saved.fwd_workspace_bytes = self._ws_f.data_ptr(), self._ws_f_bytes
         self.ent_rows = torch.empty((n_occ, model.dim), **f32)
         self.rel_rows = torch.empty((B, model.rel_dim), **f32) if model.rel_dim else None
         self.aux_rows = None

@@ -146,6 +146,11 @@ typedef struct kge_saved {
     const float *residual;  /* [B, dim]: TransR residual rows / RESCAL E[h] Proj[r] rows;
                                RotatE: rotated heads h e^{i theta} as [re | im]
                                (with KGE_NEG_HEAD: counter-rotated tails t e^{-i theta}) */
+    /* TransR / RESCAL, optional: the workspace the forward call of this batch was given (it
+       holds the tile plans of the relation groups); kge_score_bwd then reuses them instead of
+       building its own.  NULL / 0: backward plans for itself. */
+    const void *fwd_workspace;
+    size_t fwd_workspace_bytes;
 } kge_saved;
 
 /* Sparse row gradients: row u of each array belongs to the u-th unique id of the
