@@ -277,7 +277,7 @@ __global__ __launch_bounds__(kMidThreads) void inspect_mid_hist_kernel(MidJobs j
 template <bool FIRST>
 __global__ __launch_bounds__(kMidThreads) void inspect_mid_scatter_kernel(MidJobs jobs, int pass)
 {
-    __shared__ uint32_t smem[mid_pass_lds_words(kMaxBins)];
+    __shared__ uint32_t smem[mid_pass_lds_words(kMaxBins, 1)];
     mid_scatter_body<FIRST>(jobs.j[blockIdx.y], pass, blockIdx.x, smem);
 }
 
@@ -383,7 +383,7 @@ int plan_fused_inspection(const kge_inspect_job *jobs, int n_jobs, int slot, Fus
         blocks[q] = (int)ceil_div(n, kMidKeys);
         const int step = slot - (kFusedSlots - 2 - J.npass);
         const int w = step == 0 ? mid_hist_lds_words(1 << J.db, J.npass)
-                                : (step >= 1 && step <= J.npass ? mid_pass_lds_words(1 << J.db) : 0);
+                                : (step >= 1 && step <= J.npass ? mid_pass_lds_words(1 << J.db, J.npass) : 0);
         words = w > words ? w : words;
     }
     f.split = blocks[0];

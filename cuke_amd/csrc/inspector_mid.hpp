@@ -119,7 +119,11 @@ struct FusedInsp {
 };
 
 // LDS words a digit pass with `bins` bins needs
-__host__ __device__ constexpr int mid_pass_lds_words(int bins) { return (3 + kMidWaves) * bins + kMidWaves; }
+// (a job with a single pass also keeps the index of every non-empty bin: one more array)
+__host__ __device__ constexpr int mid_pass_lds_words(int bins, int npass)
+{
+    return (2 + kMidWaves + (npass == 1 ? 1 : 0)) * bins + kMidWaves;
+}
 
 // Workgroups of a job, and the per-workgroup digit histograms of pass p in the job's workspace
 // (kMidMaxPass tables of [workgroups][bins] counters).
