@@ -80,9 +80,13 @@ def algorithmic_bytes(w, u_ent, u_rel):
 
 def neg_kernel_bytes(w):
     """Algorithmic bytes of ONE launch of the shared-negative forward kernel: the h and r (and w)
-    rows of every positive, every negative row once per chunk, the indices, the scores out."""
+    rows of every positive (RotatE: its one rotated-head row), every negative row once per chunk,
+    the indices, the scores out."""
     B, d, rd, N = w.batch, w.dim, w.rel_dim, w.n_neg
     nn = w.n_chunks * N
+    if w.model == "RotatE":
+        # one rotated-head row per positive (written by the positive kernel of the same call), no h / r gathers
+        return 4 * (B * d + nn * d) + 8 * nn + 4 * B * N
     aux_row = d if w.model == "TransH" else 0
     out_planes = 3 if w.model == "TransH" else 1
     return 4 * (B * (d + rd + aux_row) + nn * d) + 8 * (2 * B + nn) + 4 * out_planes * B * N
@@ -253,24 +257,20 @@ def main():
     from cuke_amd import _lib
     L = _lib.lib()
     if w.chunk:
-        def only_neg():
-            L.kge_score_fwd(ctypes.byref(model._tab), ctypes.byref(step.bat), None,
-                            ctypes.c_void_p(step.neg.data_ptr()),
-                            ctypes.c_void_p(step.side_pos.data_ptr()) if step.side_pos is not None else None,
-                            ctypes.c_void_p(step.side_neg.data_ptr()) if step.side_neg is not None else None,
-                            # RotatE: the rotated heads the positive kernel left behind (read-only here)
-                            ctypes.c_void_p(step.residual.data_ptr()) if w.model == "RotatE" else None,
-                            None, 0, stc)
+        P = lambda t: ctypes.c_void_p(t.data_ptr()) if t is not None else None
         kname = "score_neg_mfma_kernel" if w.model in ("DistMult", "ComplEx") else "score_neg_kernel"
-        if w.model == "TransH":  # needs w.h from the positive kernel; time the pair and subtract
+        if w.model in ("TransH", "RotatE"):
+            # the tile kernel reads what the positive kernel of the same call leaves behind (w.h, the
+            # rotated heads): time the forward call and the positive kernel alone, report the
+            # difference
             t_pair = time_events(lambda: step.forward(stc), 100, torch)
-            t_pos = time_events(lambda: L.kge_score_fwd(ctypes.byref(model._tab), ctypes.byref(step.bat),
-                                                        ctypes.c_void_p(step.pos.data_ptr()), None,
-                                                        ctypes.c_void_p(step.side_pos.data_ptr()), None, None,
-                                                        None, 0, stc), 100, torch)
+            t_pos = time_events(lambda: L.kge_score_fwd(ctypes.byref(model._tab), ctypes.byref(step.bat), P(step.pos),
+                                                        None, P(step.side_pos), None, P(step.residual), None, 0, stc),
+                                100, torch)
             k_ms = t_pair - t_pos
         else:
-            k_ms = time_events(only_neg, 100, torch)
+            k_ms = time_events(lambda: L.kge_score_fwd(ctypes.byref(model._tab), ctypes.byref(step.bat), None,
+                                                       P(step.neg), None, None, None, None, 0, stc), 100, torch)
         k_bytes, k_flops = neg_kernel_bytes(w), neg_kernel_flops(w)
     else:
         # positive-only workloads: the forward call is one kernel (TransR: the tile-plan kernel,
