@@ -291,6 +291,9 @@ def main():
         "config": {"workload": w.name, "score_function": w.model, "n_ent": w.n_ent, "n_rel": w.n_rel, "dim": w.dim,
                    "batch": w.batch, "chunk": w.chunk, "n_neg": w.n_neg, "norm_p": w.norm_p,
                    "backward": do_bwd, "loss": w.loss, "hip_graph": use_graph, "issue": issue,
+                   "pair_sums": ("vector ALUs (KGE_DOT_VALU=1)" if os.environ.get("KGE_DOT_VALU", "0") not in ("", "0")
+                                 else "matrix cores, fp32") if w.model in ("DistMult", "ComplEx") and w.chunk
+                   else "vector ALUs",
                    "ms_per_step_direct": ms_direct, "ms_per_step_pipelined": ms_pipe,
                    "ms_per_step_graph": ms_graph,
                    "scores_per_step": scores, "positives_per_s": w.batch / (ms * 1e-3),

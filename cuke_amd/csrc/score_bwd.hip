@@ -56,12 +56,13 @@ struct TileShape {
     static constexpr int kLdsFloats = NPL * kKL * kLP + NC * kKL * PG;
 };
 
-template <int MODEL, int P, bool OWNER_POS, int RO>
+template <int MODEL, int P, bool OWNER_POS, int RO, bool MF>
 __device__ __forceinline__ void bwd_tile_body(const TileArgs &a, int lid, float *smem)
 {
     constexpr int TO = 16 * RO;
     constexpr bool kRot = MODEL == KGE_ROTATE, kTH = MODEL == KGE_TRANSH;
     constexpr bool kDot = MODEL == KGE_DISTMULT || MODEL == KGE_COMPLEX;
+    constexpr bool kMf = kDot && MF;  // the sum over loopers on the matrix cores (else on the vector ALUs)
     constexpr bool kL2 = (MODEL == KGE_TRANSE || kTH) && P == 2;
     constexpr int NPL = (kRot || (kTH && !OWNER_POS)) ? 2 : 1;  // looper planes in LDS
     constexpr int NPO = (kRot || (kTH && OWNER_POS)) ? 2 : 1;   // owner planes in registers
@@ -130,7 +131,7 @@ __device__ __forceinline__ void bwd_tile_body(const TileArgs &a, int lid, float 
     // looper's row feeds four MFMAs, so MFMA e owns the columns 4 j + e.  A wave owns 16 owners and
     // all 64 columns (64-owner tiles), or 16 owners and the columns 4 j + {0,1} / {2,3} (32-owner tiles).
     constexpr int OB = TO / 16, EW = OB;  // owner blocks; MFMAs (columns per lane) per wave
-    static_assert(!kDot || OB == 4 || OB == 2, "MFMA tiling written for 32- and 64-owner tiles");
+    static_assert(!kMf || OB == 4 || OB == 2, "MFMA tiling written for 32- and 64-owner tiles");
     const int mlane = tid & 63, mwave = tid >> 6, fj = mlane & 15, fg = mlane >> 4;
     const int ob = mwave % OB, e0 = (mwave / OB) * EW;
     v4f macc[EW];
@@ -303,7 +304,7 @@ __device__ __forceinline__ void bwd_tile_body(const TileArgs &a, int lid, float 
         // two-level sum: the kKL loopers of a step go into a fresh accumulator that is folded
         // into the running one per step, so rounding grows with sqrt(steps) of the large partial
         // sums instead of sqrt(loopers)
-        if constexpr (kDot) {
+        if constexpr (kMf) {
 #pragma unroll
             for (int q = 0; q < kKL / 16; ++q)
 #pragma unroll
@@ -329,7 +330,7 @@ __device__ __forceinline__ void bwd_tile_body(const TileArgs &a, int lid, float 
 #pragma unroll
             for (int o = 0; o < RO; ++o) sacc[q][o] = zero4();
 #pragma unroll 4
-        for (int l = 0; l < (kDot ? 0 : kKL); ++l) {
+        for (int l = 0; l < (kMf ? 0 : kKL); ++l) {
             float4 lv[NPL];
 #pragma unroll
             for (int pl = 0; pl < NPL; ++pl) lv[pl] = *reinterpret_cast<const float4 *>(&sL[pl][l][tx * 4]);
@@ -394,7 +395,7 @@ __device__ __forceinline__ void bwd_tile_body(const TileArgs &a, int lid, float 
         __syncthreads();
     }
 
-    if constexpr (kDot) {
+    if constexpr (kMf) {
 #pragma unroll
         for (int v = 0; v < 4; ++v) {
             const int ol = ot0 + ob * 16 + 4 * fg + v;
@@ -430,7 +431,7 @@ __device__ __forceinline__ void bwd_tile_body(const TileArgs &a, int lid, float 
 // Both orientations in ONE launch: the first `grid_head` workgroups own positives (outputs
 // g0 / g1), the rest own negatives (output occ_neg).  The two halves are independent, and
 // together they fill the GPU better than either alone when the batch is small.
-template <int MODEL, int P, int RO>
+template <int MODEL, int P, int RO, bool MF>
 __global__ __launch_bounds__(256, KGE_TILE_OCC) void bwd_tile_kernel(TileArgs a, float *g0, float *g1, float *occ_neg,
                                                                      int grid_head, FusedInsp fi)
 {
@@ -440,10 +441,10 @@ __global__ __launch_bounds__(256, KGE_TILE_OCC) void bwd_tile_kernel(TileArgs a,
     const int lid = (int)blockIdx.x - fi.blocks;
     if (lid < grid_head) {
         a.out0 = g0, a.out1 = g1;
-        bwd_tile_body<MODEL, P, true, RO>(a, lid, smem);
+        bwd_tile_body<MODEL, P, true, RO, MF>(a, lid, smem);
     } else {
         a.out0 = occ_neg, a.out1 = nullptr;
-        bwd_tile_body<MODEL, P, false, RO>(a, lid - grid_head, smem);
+        bwd_tile_body<MODEL, P, false, RO, MF>(a, lid - grid_head, smem);
     }
 }
 
@@ -457,6 +458,17 @@ static size_t tile_lds_bytes(const FusedInsp &fi)
     return fi.blocks > 0 && (size_t)fi.lds_bytes > own ? (size_t)fi.lds_bytes : own;
 }
 
+// 1: DistMult / ComplEx pair sums on the vector ALUs instead of the matrix cores (the forward tile
+// kernel reads the same variable)
+static int dot_valu_override()
+{
+    static const int v = [] {
+        const char *e = getenv("KGE_DOT_VALU");
+        return e ? atoi(e) : 0;
+    }();
+    return v;
+}
+
 template <int MODEL, int P>
 static int launch_tiles(TileArgs a, float *g0, float *g1, float *occ_neg, int64_t n_chunks, const FusedInsp &fi,
                         hipStream_t st)
@@ -466,18 +478,36 @@ static int launch_tiles(TileArgs a, float *g0, float *g1, float *occ_neg, int64_
     const int64_t big = gx * (ceil_div(a.C, 64) + ceil_div(a.N, 64)) * n_chunks;
     static const int knob = [] { const char *e = getenv("KGE_BWD_TILE"); return e ? atoi(e) : 0; }();
     // KGE_BWD_TILE is a development knob; the size rule follows launch_neg_mp (see there)
-    // (the matrix-core inner loop of DistMult / ComplEx gives a wave all 64 columns of its 16 owners
-    // with 64-owner tiles and half of them with 32-owner tiles: the large tile wins at every size)
     constexpr bool kDotModel = MODEL == KGE_DISTMULT || MODEL == KGE_COMPLEX;
-    if (knob == 4 || (knob != 2 && (kDotModel || big >= 1024))) {
+    if constexpr (kDotModel) {
+        // matrix-core inner loop (KGE_DOT_VALU=1 keeps the vector-ALU loop): a wave gets all 64
+        // columns of its 16 owners with 64-owner tiles and half of them with 32-owner tiles, and the
+        // large tile wins at every size
+        if (!dot_valu_override()) {
+            if (knob == 2) {
+                const unsigned gh = xcd_grid(gx, ceil_div(a.C, 32), n_chunks), gn = xcd_grid(gx, ceil_div(a.N, 32), n_chunks);
+                const size_t lds = tile_lds_bytes<MODEL, 2>(fi);
+                hipLaunchKernelGGL((bwd_tile_kernel<MODEL, P, 2, true>), dim3(gh + gn + fi.blocks), dim3(256), lds, st, a,
+                                   g0, g1, occ_neg, (int)gh, fi);
+            } else {
+                const unsigned gh = xcd_grid(gx, ceil_div(a.C, 64), n_chunks), gn = xcd_grid(gx, ceil_div(a.N, 64), n_chunks);
+                const size_t lds = tile_lds_bytes<MODEL, 4>(fi);
+                hipLaunchKernelGGL((bwd_tile_kernel<MODEL, P, 4, true>), dim3(gh + gn + fi.blocks), dim3(256), lds, st, a,
+                                   g0, g1, occ_neg, (int)gh, fi);
+            }
+            KGE_CHECK_LAUNCH();
+            return KGE_OK;
+        }
+    }
+    if (knob == 4 || (knob != 2 && big >= 1024)) {
         const unsigned gh = xcd_grid(gx, ceil_div(a.C, 64), n_chunks), gn = xcd_grid(gx, ceil_div(a.N, 64), n_chunks);
         const size_t lds = tile_lds_bytes<MODEL, 4>(fi);
-        hipLaunchKernelGGL((bwd_tile_kernel<MODEL, P, 4>), dim3(gh + gn + fi.blocks), dim3(256), lds, st, a, g0, g1,
+        hipLaunchKernelGGL((bwd_tile_kernel<MODEL, P, 4, false>), dim3(gh + gn + fi.blocks), dim3(256), lds, st, a, g0, g1,
                            occ_neg, (int)gh, fi);
     } else {
         const unsigned gh = xcd_grid(gx, ceil_div(a.C, 32), n_chunks), gn = xcd_grid(gx, ceil_div(a.N, 32), n_chunks);
         const size_t lds = tile_lds_bytes<MODEL, 2>(fi);
-        hipLaunchKernelGGL((bwd_tile_kernel<MODEL, P, 2>), dim3(gh + gn + fi.blocks), dim3(256), lds, st, a, g0, g1,
+        hipLaunchKernelGGL((bwd_tile_kernel<MODEL, P, 2, false>), dim3(gh + gn + fi.blocks), dim3(256), lds, st, a, g0, g1,
                            occ_neg, (int)gh, fi);
     }
     KGE_CHECK_LAUNCH();

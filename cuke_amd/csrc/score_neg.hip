@@ -361,11 +361,12 @@ static int neg_tile_override()
     return v;
 }
 
-// 1: keep DistMult / ComplEx on the vector ALUs (development knob)
+// 1: keep DistMult / ComplEx on the vector ALUs instead of the matrix cores (the gradient tile
+// kernel reads the same variable)
 static int neg_valu_override()
 {
     static const int v = [] {
-        const char *e = getenv("KGE_NEG_VALU");
+        const char *e = getenv("KGE_DOT_VALU");
         return e ? atoi(e) : 0;
     }();
     return v;
@@ -389,7 +390,7 @@ static int launch_neg_mp(const NegArgs &a, int64_t n_chunks, const FusedInsp &fi
     // launches are bound by the rows its workgroups pull from L2, does best with 32x64).  The
     // inspector workgroups that share the machine with these launches raise their wave priority.
     constexpr bool kDotModel = MODEL == KGE_DISTMULT || MODEL == KGE_COMPLEX;
-    if (tile != 2 && tile != 4 && tile != 3) tile = big_tiles >= 1024 ? 4 : (kDotModel ? 3 : 2);
+    if (tile != 2 && tile != 4 && tile != 3) tile = big_tiles >= 1024 ? 4 : (kDotModel && !neg_valu_override() ? 3 : 2);
     const int TB = tile == 4 ? 64 : 32, TN = tile == 2 ? 32 : 64;
     const dim3 grid(xcd_grid(ceil_div(a.N, TN), ceil_div(a.C, TB), n_chunks) + (unsigned)fi.blocks);
     if constexpr (MODEL == KGE_DISTMULT || MODEL == KGE_COMPLEX) {
