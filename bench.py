@@ -272,6 +272,24 @@ def main():
             k_ms = time_events(lambda: L.kge_score_fwd(ctypes.byref(model._tab), ctypes.byref(step.bat), None,
                                                        P(step.neg), None, None, None, None, 0, stc), 100, torch)
         k_bytes, k_flops = neg_kernel_bytes(w), neg_kernel_flops(w)
+        # the two memory-bound pieces of a shared-negative step, on their own: the per-positive
+        # gather kernel and the inspection of concat(h, t, neg) and r
+        if w.model not in ("TransH", "RotatE"):
+            t_pos = time_events(lambda: L.kge_score_fwd(ctypes.byref(model._tab), ctypes.byref(step.bat), P(step.pos),
+                                                        None, P(step.side_pos), None, P(step.residual), None, 0, stc),
+                                100, torch)
+        aux_row = w.dim if w.model == "TransH" else 0
+        pos_bytes = 4 * w.batch * (2 * w.dim + w.rel_dim + aux_row) + 8 * 3 * w.batch + 4 * w.batch \
+            + (4 * w.batch * w.dim if w.model == "RotatE" else 0) + (4 * w.batch if w.model == "TransH" else 0)
+        n_ids = step.n_occ + w.batch
+        insp_bytes = n_ids * (8 + 3 * 4) + (u_ent + u_rel) * (8 + 4)  # ids in; perm, inverse, segment per id; unique ids, offsets
+        extra = {"positive_gather": {"kernel": "score_pos_kernel", "ms": t_pos, "algorithmic_bytes": pos_bytes,
+                                     "gbs": pos_bytes / (t_pos * 1e-3) / 1e9,
+                                     "hbm_frac": pos_bytes / (t_pos * 1e-3) / 1e9 / HBM_PEAK_GBS},
+                 "inspection": {"ids": n_ids, "ms": stages["inspect_ms"], "algorithmic_bytes": insp_bytes,
+                                "ids_per_s": n_ids / (stages["inspect_ms"] * 1e-3),
+                                "note": "stand-alone inspector launches; in the timed step its workgroups ride with the "
+                                        "score kernels where the batch qualifies"}}
     else:
         # positive-only workloads: the forward call is one kernel (TransR: the tile-plan kernel,
         # a few microseconds, plus the grouped MFMA kernel)
@@ -279,6 +297,7 @@ def main():
         k_ms = time_events(lambda: step.forward(stc), 100, torch)
         k_bytes = fwd_b
         k_flops = 2 * w.batch * w.dim * w.dim if w.model == "TransR" else 3 * w.batch * w.dim
+        extra = {}
     achieved = k_bytes / (k_ms * 1e-3) / 1e9
 
     out = {
@@ -299,7 +318,7 @@ def main():
                    "scores_per_step": scores, "positives_per_s": w.batch / (ms * 1e-3),
                    "unique_entity_rows": u_ent, "unique_relation_rows": u_rel},
         "step": {"algorithmic_bytes": total_b, "hbm_gbs": total_b / (ms * 1e-3) / 1e9,
-                 "hbm_frac": total_b / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, "wall_s": wall, **stages},
+                 "hbm_frac": total_b / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, "wall_s": wall, **stages, **extra},
         "roofline": {"kernel": kname, "bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": achieved / HBM_PEAK_GBS, "traffic": MEASURED_TRAFFIC_BYTES.get(w.name),
                      "kernel_ms": k_ms,
