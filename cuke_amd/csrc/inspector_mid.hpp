@@ -75,14 +75,20 @@ __device__ inline void block_exclusive_scan(uint32_t *s, int bins, uint32_t *wav
     __syncthreads();
 }
 
-// ---- small and medium inputs: one launch per digit pass ------------------------------------
-// Up to 65536 ids.  A block owns 1024 consecutive keys.  Instead of a separate histogram
-// kernel and scan, every block counts the digits of ALL keys itself (LDS atomics; the keys are
-// a few hundred KB at most and sit in L2), which gives it the global bin starts and the number
-// of same-digit keys in the blocks before it; it then ranks its own keys stably with wave
-// ballots and scatters them.  A pass is therefore ONE launch with no inter-block dependency,
-// the dedup a second one that counts the run heads before the block the same way.  Several
-// index sets share the launches.
+// ---- small and medium inputs (up to 65536 ids) ---------------------------------------------------
+// A workgroup owns 1024 consecutive keys.  The steps of a job are
+//   histogram: every workgroup writes the digit histograms of its own keys, one per pass, to the
+//              job's workspace (a histogram does not depend on key order, so all passes' bin totals
+//              are known before anything is sorted);
+//   scatter p: bin starts = column sums of pass p's histograms; the same-digit keys in front of the
+//              workgroup come from those histograms too in the first pass, and from a recount of
+//              the sorted keys in front of it in a later pass; the workgroup's own keys are ranked
+//              stably with wave ballots and scattered.  A job with a single pass is finished here
+//              (every non-empty bin is one distinct id);
+//   dedup:     run detection over the sorted keys.
+// No step depends on another workgroup of the same launch, only on the launch before, so the steps
+// run as launches of their own (several index sets sharing them) or as extra workgroups in front
+// of another kernel's grid (FusedInsp).
 constexpr int kMidThreads = 256;
 constexpr int kMidWaves = kMidThreads / kWave;
 constexpr int kMidKeys = 1024;  // keys per block: 4 rounds of 64 per wave
