@@ -346,6 +346,7 @@ static int validate_job(const kge_inspect_job *job, Parts *parts, int64_t *n_out
     if (!out->num_unique || !out->seg_offsets) return KGE_EINVAL;
     if (n > 0 && (!out->unique_ids || !out->perm || !out->inverse || !out->sorted_seg)) return KGE_EINVAL;
     if (!job->workspace || job->workspace_bytes < make_plan(n, job->n_rows).total) return KGE_EWORKSPACE;
+    if (!aligned16(job->workspace)) return KGE_EWORKSPACE;  // the key buffers are read with 128-bit loads
     *n_out = n;
     return KGE_OK;
 }

@@ -244,17 +244,26 @@ __device__ __forceinline__ void mid_scatter_body(const MidJob &J, int pass, int 
     if (pass > 0) {  // s_bef held the histogram-order count, which only the first pass can use
         for (int i = tid; i < bins; i += kMidThreads) s_bef[i] = 0;
         __syncthreads();
-        constexpr int kBatch = 16;  // unconditional loads in flight per thread
-        for (int i0 = 0; i0 < my0; i0 += kBatch * kMidThreads) {
-            uint32_t kb[kBatch];
+        // (my0 is a multiple of 1024 and the key buffers are 256-byte aligned: whole groups of four
+        // keys per 128-bit load, sixteen groups per thread in flight)
+        constexpr int kBatch = 16;
+        const uint4 *kin4 = reinterpret_cast<const uint4 *>(kin);
+        const int groups = my0 >> 2;
+        for (int g0 = 0; g0 < groups; g0 += kBatch * kMidThreads) {
+            uint4 kb[kBatch];
 #pragma unroll
             for (int u = 0; u < kBatch; ++u) {
-                const int i = i0 + u * kMidThreads + tid;
-                kb[u] = kin[i < my0 ? i : my0 - 1];
+                const int g = g0 + u * kMidThreads + tid;
+                kb[u] = kin4[g < groups ? g : groups - 1];  // clamped: unconditional loads, masked below
             }
 #pragma unroll
             for (int u = 0; u < kBatch; ++u)
-                if (i0 + u * kMidThreads + tid < my0) atomicAdd(&s_bef[(kb[u] >> shift) & mask], 1u);
+                if (g0 + u * kMidThreads + tid < groups) {
+                    atomicAdd(&s_bef[(kb[u].x >> shift) & mask], 1u);
+                    atomicAdd(&s_bef[(kb[u].y >> shift) & mask], 1u);
+                    atomicAdd(&s_bef[(kb[u].z >> shift) & mask], 1u);
+                    atomicAdd(&s_bef[(kb[u].w >> shift) & mask], 1u);
+                }
         }
         __syncthreads();
     }

@@ -220,7 +220,7 @@ typedef struct kge_inspect_job {
     int32_t reserved;
     int64_t n_rows;
     kge_inspection out;
-    void *workspace;          /* kge_inspect_workspace(n, n_rows) bytes */
+    void *workspace;          /* kge_inspect_workspace(n, n_rows) bytes, 16-byte aligned */
     size_t workspace_bytes;
 } kge_inspect_job;
 int kge_inspect_batch(const kge_inspect_job *jobs, int n_jobs, void *stream);
