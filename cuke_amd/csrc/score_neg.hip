@@ -33,6 +33,8 @@ struct NegArgs {
     float rsign;            // +1: negatives replace the tail; -1: the head (see load_query)
 };
 
+typedef float v4f __attribute__((ext_vector_type(4)));
+
 constexpr int kKD = 32;        // floats of each row staged per step
 constexpr int kLDW = kKD + 4;  // LDS row pitch: +4 floats keeps 128-bit reads of
                                // 8 consecutive rows on distinct banks
@@ -199,8 +201,86 @@ __global__ __launch_bounds__(256, KGE_TILE_OCC) void score_neg_kernel(NegArgs a,
             __syncthreads();
         }
     };
-    sweep(std::integral_constant<int, 0>{});
-    if constexpr (NPASS == 2) sweep(std::integral_constant<int, 1>{});
+    if constexpr (MODEL == KGE_TRANSH) {
+        // TransH, first sweep: c[b][k] = w_b . t'_k for the whole tile is a matrix product (normal
+        // rows x negative rows), run on the matrix cores (v_mfma_f32_16x16x4_f32; operand layout
+        // and k relabelling as in score_neg_mfma_kernel below).  Only the w and t' rows are staged.
+        // The four waves tile the workgroup 2 x 2; the products then go through LDS into the
+        // (ty + 16 i, tx + 16 k) layout of the second sweep's micro-tiles.
+        constexpr int MB = RB / 2, NB = RK / 2;
+        const int lane = tid & 63, wave = tid >> 6, fr = lane & 15, fg = lane >> 4;
+        const int wrow = (wave >> 1) * (TB / 2), wcol = (wave & 1) * (TN / 2);
+        v4f macc[MB][NB];
+#pragma unroll
+        for (int m = 0; m < MB; ++m)
+#pragma unroll
+            for (int n = 0; n < NB; ++n) macc[m][n] = v4f{0.0f, 0.0f, 0.0f, 0.0f};
+        float4 rw[SB];
+        auto load_w = [&](int j0) {  // one uniform branch per slice, none per load
+            const int j = j0 + scol;
+            if (vec) {
+#pragma unroll
+                for (int q = 0; q < SB; ++q) rw[q] = ld4<true>(pw[q], j, okb[q] ? d : 0);
+#pragma unroll
+                for (int q = 0; q < SN; ++q) rt[0][q] = ld4<true>(pt[q], j, okk[q] ? d : 0);
+            } else {
+#pragma unroll
+                for (int q = 0; q < SB; ++q) rw[q] = ld4<false>(pw[q], j, okb[q] ? d : 0);
+#pragma unroll
+                for (int q = 0; q < SN; ++q) rt[0][q] = ld4<false>(pt[q], j, okk[q] ? d : 0);
+            }
+        };
+        load_w(0);
+#pragma unroll 1
+        for (int s = 0; s < nslice; ++s) {
+#pragma unroll
+            for (int q = 0; q < SB; ++q) *reinterpret_cast<float4 *>(&sA[1][srow + 32 * q][scol]) = rw[q];
+#pragma unroll
+            for (int q = 0; q < SN; ++q) *reinterpret_cast<float4 *>(&sT[0][srow + 32 * q][scol]) = rt[0][q];
+            __syncthreads();
+            if (s + 1 < nslice) load_w((s + 1) * kKD);
+#pragma unroll
+            for (int g = 0; g < kKD / 16; ++g) {
+                float4 av[MB], tv[NB];
+#pragma unroll
+                for (int m = 0; m < MB; ++m)
+                    av[m] = *reinterpret_cast<const float4 *>(&sA[1][wrow + 16 * m + fr][16 * g + 4 * fg]);
+#pragma unroll
+                for (int n = 0; n < NB; ++n)
+                    tv[n] = *reinterpret_cast<const float4 *>(&sT[0][wcol + 16 * n + fr][16 * g + 4 * fg]);
+#pragma unroll
+                for (int e = 0; e < 4; ++e)
+#pragma unroll
+                    for (int m = 0; m < MB; ++m)
+#pragma unroll
+                        for (int n = 0; n < NB; ++n) {
+                            const float x = e == 0 ? av[m].x : e == 1 ? av[m].y : e == 2 ? av[m].z : av[m].w;
+                            const float y = e == 0 ? tv[n].x : e == 1 ? tv[n].y : e == 2 ? tv[n].z : tv[n].w;
+                            macc[m][n] = __builtin_amdgcn_mfma_f32_16x16x4f32(x, y, macc[m][n], 0, 0, 0);
+                        }
+            }
+            __syncthreads();
+        }
+        // D[i = 4 (l / 16) + v][j = l % 16] of block (m, n) -> sC[row][col] -> cdot of the micro-tiles
+        float(*sC)[TN + 1] = reinterpret_cast<float(*)[TN + 1]>(dyn_smem);  // TB x (TN + 1) floats fit in plane 0 + 1 of sA
+        static_assert(sizeof(float) * TB * (TN + 1) <= sizeof(float) * NPA * TB * kLDW + sizeof(float) * NPT * TN * kLDW,
+                      "the product tile reuses the staging buffers");
+#pragma unroll
+        for (int m = 0; m < MB; ++m)
+#pragma unroll
+            for (int n = 0; n < NB; ++n)
+#pragma unroll
+                for (int v = 0; v < 4; ++v) sC[wrow + 16 * m + 4 * fg + v][wcol + 16 * n + fr] = macc[m][n][v];
+        __syncthreads();
+#pragma unroll
+        for (int i = 0; i < RB; ++i)
+#pragma unroll
+            for (int k = 0; k < RK; ++k) cdot[i][k] = sC[ty + 16 * i][tx + 16 * k];
+        __syncthreads();
+        sweep(std::integral_constant<int, 1>{});
+    } else {
+        sweep(std::integral_constant<int, 0>{});
+    }
 
 #pragma unroll
     for (int i = 0; i < RB; ++i) {
@@ -231,7 +311,6 @@ __global__ __launch_bounds__(256, KGE_TILE_OCC) void score_neg_kernel(NegArgs a,
 // receives D[i = 4 * (l / 16) + v][j = l % 16], v = 0..3.  Inside 16 consecutive k the MFMA step
 // s pairs lane group g = l / 16 with k = 4 g + s (any pairing works as long as both operands use
 // it), so a lane's values for four steps are one 128-bit LDS read of its row.
-typedef float v4f __attribute__((ext_vector_type(4)));
 
 template <int MODEL, int RB, int RK>
 __global__ __launch_bounds__(256, KGE_TILE_OCC) void score_neg_mfma_kernel(NegArgs a, FusedInsp fi)
