@@ -29,12 +29,12 @@ FP32_PEAK_TFLOPS = 157.3    # MI355X fp32 vector / fp32 MFMA, published
 # reads for the 256 MiB copy kernel of --calibrate-copy (fetch x2.000, write x1.000).  The
 # summaries the numbers come from are profiles/score_path_kernels_<workload>.txt.
 MEASURED_TRAFFIC_BYTES = {
-    "cfg1_transe": 1_698_632,      # score_pos_kernel
-    "cfg2_distmult": 13_062_824,   # score_neg_mfma_kernel
-    "cfg2_complex": 13_072_108,    # score_neg_mfma_kernel
-    "cfg3_transr": 164_370_338,    # transr_plan_kernel + transr_gemm_kernel<0>
-    "cfg4_rotate": 12_056_141,     # score_neg_kernel
-    "cfg5_transh": 550_556_038,    # score_neg_kernel
+    "cfg1_transe": 1_687_370,      # score_pos_kernel
+    "cfg2_distmult": 13_060_992,   # score_neg_mfma_kernel
+    "cfg2_complex": 13_093_719,    # score_neg_mfma_kernel
+    "cfg3_transr": 164_398_014,    # transr_plan_kernel + transr_gemm_kernel<0>
+    "cfg4_rotate": 12_060_695,     # score_neg_kernel
+    "cfg5_transh": 531_454_520,    # score_neg_kernel
 }
 
 
