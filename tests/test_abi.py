@@ -107,3 +107,43 @@ def test_argument_validation_returns_status_codes_without_touching_the_gpu():
     assert L.kge_score_fwd(C.byref(tables()), C.byref(batch(B=0, h=None, r=None, t=None)), None, None, None, None,
                            None, None, 0, None) == 0
     assert L.kge_sample_negatives(None, 0, 5, 1, 0, None) == 0
+
+
+def test_fused_inspection_eligibility_is_decided_on_the_host():
+    """kge_fused_inspection_ok only reads the descriptors: shared negatives, index sets of at most 65536 ids and
+    tables of at most 2^22 rows qualify; TransF (no shared-negative kernels), larger sets and larger tables do not,
+    and asking the score calls for a fused inspection without the jobs is an argument error."""
+    import ctypes as C
+    from cuke_amd import _lib
+    L = _lib.lib()
+    fake = 0x10000  # stands for a 16-byte aligned device pointer; nothing is dereferenced or launched
+
+    def jobs(n_ent_ids, n_rel_ids, n_ent_rows, n_rel_rows=100):
+        js = (_lib.InspectJob * 2)()
+        for j, n, rows in ((js[0], n_ent_ids, n_ent_rows), (js[1], n_rel_ids, n_rel_rows)):
+            j.parts[0], j.part_len[0], j.n_parts, j.n_rows = fake, n, 1, rows
+            j.out = _lib.Inspection(n, rows, fake, fake, fake, fake, fake, fake)
+            j.workspace, j.workspace_bytes = fake, int(L.kge_inspect_workspace(n, rows))
+        return js
+
+    def tables(model, dim=16):
+        rel_dim = {"RotatE": dim // 2, "RESCAL": 0}.get(model, dim)
+        aux = fake if model in ("TransH", "TransR", "RESCAL") else None
+        return _lib.Tables(_lib.MODELS[model], 2, 0.0, 0, dim, rel_dim, 1000, 100, fake, fake if rel_dim else None, aux)
+
+    def batch(B=1024, neg=True):
+        return _lib.Batch(B, fake, fake, fake, fake if neg else None, 256 if neg else 0, 256 if neg else 0,
+                          None, None, None, 0, 0, None)
+
+    ok = lambda model, bat, js: L.kge_fused_inspection_ok(C.byref(tables(model)), C.byref(bat), js)
+    assert ok("DistMult", batch(), jobs(3072, 1024, 1000)) == 1
+    assert ok("RotatE", batch(), jobs(3072, 1024, 1 << 22)) == 1
+    assert ok("TransE", batch(), jobs(3072, 1024, (1 << 22) + 1)) == 0      # needs a third digit pass
+    assert ok("TransH", batch(), jobs(65537, 1024, 1000)) == 0              # multi-block sort territory
+    assert ok("TransF", batch(), jobs(3072, 1024, 1000)) == 0               # no tile kernels to ride with
+    assert ok("DistMult", batch(neg=False), jobs(2048, 1024, 1000)) == 0
+    assert ok("TransR", batch(neg=False), jobs(2048, 1024, 1000)) == 0      # no relation groups given
+    # the flag without the jobs
+    bat = batch()
+    bat.fuse_inspection = 1
+    assert L.kge_score_fwd(C.byref(tables("DistMult")), C.byref(bat), fake, fake, None, None, None, None, 0, None) == -1
