@@ -179,3 +179,27 @@ def test_more_than_2_to_31_scores(model, p):
     touched = torch.zeros(w.n_ent, dtype=torch.bool, device="cuda")
     touched[g.ent_ids] = True
     assert not bool(want_e[~touched].any())
+
+
+def test_preallocated_step_with_riding_inspection_equals_the_eager_path_bit_for_bit(full):
+    """TrainStep.run() at full size (inspection riding inside the score kernels' launches, tile plans
+    reused by backward) must give exactly the bits of KGEModel.score + backward with the stand-alone
+    inspector: the same kernels do the arithmetic, only where the inspector's workgroups run differs."""
+    from cuke_amd.kge import TrainStep
+    w, m, ix, fw = full
+    if not w.backward:
+        pytest.skip("forward-only configuration")
+    dpos, dneg = upstream(w, 5)
+    g = m.backward(fw, dev(dpos), dev(dneg))
+    step = TrainStep(m, ix["h"], ix["r"], ix["t"], ix.get("neg"), w.chunk or None, dpos=dev(dpos), dneg=dev(dneg))
+    assert step.fusable
+    step.run()
+    torch.cuda.synchronize()
+    s = step.sparse_grads()
+    assert torch.equal(step.pos, fw.pos) and (fw.neg is None or torch.equal(step.neg, fw.neg))
+    assert torch.equal(s.ent_ids, g.ent_ids) and torch.equal(s.rel_ids, g.rel_ids)
+    assert torch.equal(s.ent_rows, g.ent_rows)
+    for a_, b_ in ((s.rel_rows, g.rel_rows), (s.aux_rows, g.aux_rows)):
+        assert (a_ is None) == (b_ is None)
+        if a_ is not None:
+            assert torch.equal(a_, b_)
