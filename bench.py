@@ -237,6 +237,17 @@ def main():
             ms, wall, issue = ms_graph, wall_g, "graph"
     use_graph = issue == "graph"
 
+    # DistMult / ComplEx: the same step with the pair sums of the tile kernels on the other unit
+    # (matrix cores <-> vector ALUs), direct launches, for comparison; the setting is restored
+    ms_forms = None
+    if w.model in ("DistMult", "ComplEx") and w.chunk and do_bwd:
+        from cuke_amd import _lib as _l
+        was = _l.lib().kge_set_pair_sum_unit(0)
+        _l.lib().kge_set_pair_sum_unit(1 - was)
+        ms_other, _ = timed(lambda: step.run(do_bwd))
+        _l.lib().kge_set_pair_sum_unit(was)
+        ms_forms = {"matrix_cores": ms_other if was else ms_direct, "vector_alus": ms_direct if was else ms_other}
+
     u_ent, u_rel = step.ent_insp.num_unique, step.rel_insp.num_unique
     fwd_b, bwd_b = algorithmic_bytes(w, u_ent, u_rel)
     total_b = fwd_b + (bwd_b if do_bwd else 0)
@@ -311,10 +322,10 @@ def main():
                    "batch": w.batch, "chunk": w.chunk, "n_neg": w.n_neg, "norm_p": w.norm_p,
                    "backward": do_bwd, "loss": w.loss, "hip_graph": use_graph, "issue": issue,
                    "pair_sums": ("vector ALUs (KGE_DOT_VALU=1)" if os.environ.get("KGE_DOT_VALU", "0") not in ("", "0")
-                                 else "matrix cores, fp32") if w.model in ("DistMult", "ComplEx") and w.chunk
+                                 else "matrix cores, fp32 (default)") if w.model in ("DistMult", "ComplEx") and w.chunk
                    else "vector ALUs",
                    "ms_per_step_direct": ms_direct, "ms_per_step_pipelined": ms_pipe,
-                   "ms_per_step_graph": ms_graph,
+                   "ms_per_step_graph": ms_graph, "ms_per_step_direct_by_pair_sum_unit": ms_forms,
                    "scores_per_step": scores, "positives_per_s": w.batch / (ms * 1e-3),
                    "unique_entity_rows": u_ent, "unique_relation_rows": u_rel},
         "step": {"algorithmic_bytes": total_b, "hbm_gbs": total_b / (ms * 1e-3) / 1e9,

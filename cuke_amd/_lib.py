@@ -60,6 +60,7 @@ EXPORTS = {
     # name: (restype, argtypes)
     "kge_strerror": (C.c_char_p, [C.c_int]),
     "kge_abi_version": (C.c_int, []),
+    "kge_set_pair_sum_unit": (C.c_int, [C.c_int]),
     "kge_residual_fwd": (C.c_int, [C.POINTER(Tables), C.POINTER(Batch), C.c_void_p, C.c_void_p, C.c_size_t,
                                    C.c_void_p]),
     "kge_score_fwd_workspace": (C.c_size_t, [C.POINTER(Tables), C.POINTER(Batch)]),

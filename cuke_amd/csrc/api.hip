@@ -1,7 +1,19 @@
 // extern "C" entry points: argument validation and kernel dispatch.
+#include <stdlib.h>
+
 #include "inspector_mid.hpp"
 
 namespace kge {
+static int g_dot_valu = -1;  // -1: not read from the environment yet
+int dot_valu_option()
+{
+    if (g_dot_valu < 0) {
+        const char *e = getenv("KGE_DOT_VALU");
+        g_dot_valu = e && atoi(e) != 0 ? 1 : 0;
+    }
+    return g_dot_valu;
+}
+
 int launch_score_pos(const kge_tables *, const kge_batch *, float *, float *, float *, hipStream_t);
 int launch_score_pos_fused(const kge_tables *, const kge_batch *, float *, float *, float *, const FusedInsp *,
                            hipStream_t);
@@ -99,6 +111,13 @@ const char *kge_strerror(int status)
 }
 
 int kge_abi_version(void) { return 3; }
+
+int kge_set_pair_sum_unit(int vector_alu)
+{
+    const int before = dot_valu_option();
+    g_dot_valu = vector_alu ? 1 : 0;
+    return before;
+}
 
 size_t kge_score_fwd_workspace(const kge_tables *tab, const kge_batch *bat)
 {

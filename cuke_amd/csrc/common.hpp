@@ -61,6 +61,10 @@ inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 
 
 inline hipStream_t as_stream(void *s) { return reinterpret_cast<hipStream_t>(s); }
 
+// DistMult / ComplEx pair sums: 0 = matrix cores (default), 1 = vector ALUs.  Starts from the
+// environment variable KGE_DOT_VALU; kge_set_pair_sum_unit() changes it at run time (api.hip).
+int dot_valu_option();
+
 // floats per relation / auxiliary row for a model with entity width d
 inline int64_t rel_width(int model, int64_t d)
 {

@@ -458,16 +458,7 @@ static size_t tile_lds_bytes(const FusedInsp &fi)
     return fi.blocks > 0 && (size_t)fi.lds_bytes > own ? (size_t)fi.lds_bytes : own;
 }
 
-// 1: DistMult / ComplEx pair sums on the vector ALUs instead of the matrix cores (the forward tile
-// kernel reads the same variable)
-static int dot_valu_override()
-{
-    static const int v = [] {
-        const char *e = getenv("KGE_DOT_VALU");
-        return e ? atoi(e) : 0;
-    }();
-    return v;
-}
+static int dot_valu_override() { return dot_valu_option(); }
 
 template <int MODEL, int P>
 static int launch_tiles(TileArgs a, float *g0, float *g1, float *occ_neg, int64_t n_chunks, const FusedInsp &fi,

@@ -440,16 +440,7 @@ static int neg_tile_override()
     return v;
 }
 
-// 1: keep DistMult / ComplEx on the vector ALUs instead of the matrix cores (the gradient tile
-// kernel reads the same variable)
-static int neg_valu_override()
-{
-    static const int v = [] {
-        const char *e = getenv("KGE_DOT_VALU");
-        return e ? atoi(e) : 0;
-    }();
-    return v;
-}
+static int neg_valu_override() { return dot_valu_option(); }
 
 // LDS bytes of a launch: the tile's staging buffers, or what the inspector workgroups need if more
 static size_t neg_lds(int planes, int TB, int TN, int planes_t, const FusedInsp &fi)

@@ -164,6 +164,13 @@ typedef struct kge_grads {
 const char *kge_strerror(int status);
 int kge_abi_version(void);
 
+/* The shared-negative tile kernels of DistMult / ComplEx sum their pair products either on the
+   matrix cores (0, the default: fp32 MFMA, fp32 accumulate) or on the vector ALUs (1).  Both
+   meet the same tolerance; the switch exists so that the two forms can be compared in one
+   process.  Initial value: environment variable KGE_DOT_VALU.  Returns the previous setting.
+   Not thread-safe against concurrent launches.  No counterpart in the reference. */
+int kge_set_pair_sum_unit(int vector_alu);
+
 /*
  * Residual vectors, the reference's output for TransE / TransH / TransR:
  *   out[b][:] = (E[h]-E[t]) + R[r]                       (kge.py:290)

@@ -322,3 +322,21 @@ def test_fused_entity_inspection_with_the_grouped_projection_kernels(oracle, mod
     ref = oracle.backward(w.model, a["E"], a["R"], a["A"], a["h"], a["r"], a["t"], None, 0,
                           step.dpos.cpu().numpy(), None, p=2)
     compare(step.sparse_grads(), ref, f"{model} fused entity inspection")
+
+
+@pytest.mark.parametrize("model", ["DistMult", "ComplEx"])
+def test_pair_sums_on_matrix_cores_and_on_vector_alus_agree(oracle, model):
+    """kge_set_pair_sum_unit switches the DistMult / ComplEx tile kernels between the fp32 matrix-core form
+    (default) and the vector-ALU form in one process: both must meet the oracle's tolerance."""
+    from cuke_amd import _lib
+    w = synth.custom_workload(model, n_ent=400, n_rel=9, dim=72, batch=320, chunk=160, n_neg=130, sigma=0.2,
+                              ent_zipf=1.1, seed=4)
+    L = _lib.lib()
+    was = L.kge_set_pair_sum_unit(0)
+    try:
+        for unit in (0, 1):
+            L.kge_set_pair_sum_unit(unit)
+            g, ref = run_both(oracle, w, seed=3)
+            compare(g, ref, f"{model} pair sums on unit {unit}")
+    finally:
+        L.kge_set_pair_sum_unit(was)
