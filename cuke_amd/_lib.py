@@ -75,6 +75,8 @@ EXPORTS = {
     "kge_margin_loss": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int64, C.c_int64, C.c_float,
                                   C.c_float, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p,
                                   C.c_size_t, C.c_void_p]),
+    "kge_margin_loss_static": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int64, C.c_int64, C.c_float,
+                                         C.c_float, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p]),
     "kge_score_bwd_workspace": (C.c_size_t, [C.POINTER(Tables), C.POINTER(Batch)]),
     "kge_score_bwd": (C.c_int, [C.POINTER(Tables), C.POINTER(Batch), C.POINTER(Saved), C.c_void_p,
                                 C.c_void_p, C.POINTER(Grads), C.c_void_p, C.c_size_t, C.c_void_p]),

@@ -1,6 +1,8 @@
 // Margin-ranking loss over (positive, shared-negative) score pairs and its gradient.
 // Not part of the reference (it has no loss); defined as
 //   L = mean_{b,k} max(0, margin - sign * (pos[b] - neg[b][k])).
+#include <mutex>
+
 #include "common.hpp"
 
 namespace kge {
@@ -47,6 +49,30 @@ __global__ __launch_bounds__(256) void margin_total_kernel(const double *row_los
     if (threadIdx.x == 0) loss[0] = (float)(s[0] * scale);
 }
 
+// Scratch of kge_margin_loss_static: the per-row partial losses, one double per positive.  Every
+// GPU the library runs on holds its own copy of this array (512 KiB) until the process ends.
+constexpr int64_t kStaticLossRows = KGE_MARGIN_LOSS_STATIC_MAX_BATCH;
+static __device__ __align__(256) double scratch[kStaticLossRows];
+
+constexpr int kMaxDevices = 64;
+static std::mutex g_scratch_mutex;
+static double *g_scratch_ptr[kMaxDevices];  // device address of `scratch` on each device, once looked up
+
+// Device address of `scratch` on the current device (the array's name is only a host-side handle).
+static int static_scratch(double **out)
+{
+    int dev = -1;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return KGE_ELAUNCH;
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    if (!g_scratch_ptr[dev]) {
+        void *p = nullptr;
+        if (hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)) != hipSuccess || !p) return KGE_ELAUNCH;
+        g_scratch_ptr[dev] = static_cast<double *>(p);
+    }
+    *out = g_scratch_ptr[dev];
+    return KGE_OK;
+}
+
 }  // namespace kge
 
 using namespace kge;
@@ -78,6 +104,19 @@ int kge_margin_loss(const float *pos, const float *neg, int64_t batch, int64_t n
                        count > 0 ? 1.0 / count : 0.0, loss);
     KGE_CHECK_LAUNCH();
     return KGE_OK;
+}
+
+int kge_margin_loss_static(const float *pos, const float *neg, int64_t batch, int64_t n_neg, float margin,
+                           float sign, float *loss, float *dpos, float *dneg, void *stream)
+{
+    if (batch > kStaticLossRows) return KGE_EWORKSPACE;  // more rows than the built-in scratch holds
+    double *rows = nullptr;
+    const int rc = static_scratch(&rows);
+    if (rc) return rc;
+    // every row slot the total kernel reads is written by the row kernel of the same call first,
+    // so nothing left behind by an earlier call needs clearing
+    return kge_margin_loss(pos, neg, batch, n_neg, margin, sign, loss, dpos, dneg, rows,
+                           sizeof(double) * (size_t)kStaticLossRows, stream);
 }
 
 }  // extern "C"

@@ -246,6 +246,21 @@ int kge_margin_loss(const float *pos, const float *neg, int64_t batch, int64_t n
                     void *workspace, size_t workspace_bytes, void *stream);
 
 /*
+ * kge_margin_loss for callers that cannot allocate device memory (code under HIP graph capture,
+ * tight serving loops, harnesses that forbid hipMalloc): same arguments and results, but the
+ * per-row partial losses live in a device array built into the library (8 bytes per row,
+ * KGE_MARGIN_LOSS_STATIC_MAX_BATCH rows = 512 KiB held on every GPU the library runs on until the
+ * process ends) instead of a caller-provided workspace.  Allocates nothing.  batch above the
+ * limit returns KGE_EWORKSPACE.  All calls on one GPU share that array: calls that overlap on one
+ * GPU (different streams or threads) race; calls on one stream do not.  No counterpart in the
+ * reference.
+ */
+#define KGE_MARGIN_LOSS_STATIC_MAX_BATCH 65536
+int kge_margin_loss_static(const float *pos, const float *neg, int64_t batch, int64_t n_neg,
+                           float margin, float sign, float *loss, float *dpos, float *dneg,
+                           void *stream);
+
+/*
  * Backward of kge_score_fwd: upstream dpos[B] (may be NULL = 0), dneg[B, n_neg]
  * -> one gradient row per unique table row, written once, no atomics.
  * The reference only prints per-triple dense gradient kernels
