@@ -6,11 +6,23 @@ array already resident in HBM: index inspection (radix sort + dedup of the entit
 and relation ids) -> scores of the positives and of the shared negatives ->
 (margin loss) -> sparse row gradients.  Prints ONE JSON line.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload cfg2_distmult]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload all|cfg2_distmult|...]
+
+With no --workload every benchmark configuration is timed in the one run: the headline fields
+of the line are those of the largest single-GPU configuration (cfg5_transh) and `per_workload`
+holds the same fields for the other five.  Per workload:
+  * the timed loop rotates over --batches distinct seeded batches (index sets), so the gathered
+    rows of a step are not left in the caches by the step before; the same loop over one batch
+    is reported beside it (`ms_per_step_same_batch`);
+  * before anything is timed the step's own inputs are spot-checked against the CPU oracle
+    (sampled pair scores, positive scores and whole gradient rows); a mismatch aborts the run;
+  * `roofline` describes the kernel with the largest share of the step, timed live with HIP
+    events recorded behind every kernel on the stream the kernels run on.
 """
 from __future__ import annotations
 
 import argparse
+import ctypes
 import json
 import os
 import sys
@@ -24,17 +36,16 @@ sys.path.insert(0, ROOT)
 HBM_PEAK_GBS = 8000.0       # MI355X HBM3E, published
 FP32_PEAK_TFLOPS = 157.3    # MI355X fp32 vector / fp32 MFMA, published
 
-# HBM bytes per launch of each workload's roofline kernel, from rocprofv3 --pmc FETCH_SIZE and
-# --pmc WRITE_SIZE runs of this script (KiB per dispatch), each scaled by what the same counter
-# reads for the 256 MiB copy kernel of --calibrate-copy (fetch x2.000, write x1.000).  The
-# summaries the numbers come from are profiles/score_path_kernels_<workload>.txt.
+ALL_WORKLOADS = ["cfg5_transh", "cfg1_transe", "cfg2_distmult", "cfg2_complex", "cfg3_transr", "cfg4_rotate"]
+# which roof binds a workload by arithmetic (flop per algorithmic byte against the ridge of 19.7)
+BOUND = {"cfg1_transe": "hbm", "cfg2_distmult": "fp32", "cfg2_complex": "fp32", "cfg3_transr": "hbm",
+         "cfg4_rotate": "fp32", "cfg5_transh": "fp32", "ref_transr_8192x512": "hbm"}
+
+# HBM bytes per launch of a workload's dominant kernel, from rocprofv3 --pmc FETCH_SIZE and --pmc
+# WRITE_SIZE runs of this script (KiB per dispatch), each scaled by what the same counter reads
+# for the 256 MiB copy kernel of --calibrate-copy.  The summaries the numbers come from are
+# profiles/score_path_kernels_<workload>.txt; a pair that has not been measured reports null.
 MEASURED_TRAFFIC_BYTES = {
-    "cfg1_transe": 1_687_370,      # score_pos_kernel
-    "cfg2_distmult": 13_060_992,   # score_neg_mfma_kernel
-    "cfg2_complex": 13_093_719,    # score_neg_mfma_kernel
-    "cfg3_transr": 164_398_014,    # transr_plan_kernel + transr_gemm_kernel<0>
-    "cfg4_rotate": 12_060_695,     # score_neg_kernel
-    "cfg5_transh": 531_454_520,    # score_neg_kernel
 }
 
 
@@ -57,6 +68,7 @@ def device_tables(w, dev):
     return E, R, A
 
 
+# ---- algorithmic bytes and flops ---------------------------------------------------------------
 def algorithmic_bytes(w, u_ent, u_rel):
     """Bytes the step has to move by the problem statement alone: every gathered row once per
     gather (h, r, t [, w] per positive; negatives once per chunk), 8 B per index, 4 B per score;
@@ -78,26 +90,70 @@ def algorithmic_bytes(w, u_ent, u_rel):
     return fwd, bwd
 
 
-def neg_kernel_bytes(w):
-    """Algorithmic bytes of ONE launch of the shared-negative forward kernel: the h and r (and w)
-    rows of every positive (RotatE: its one rotated-head row), every negative row once per chunk,
-    the indices, the scores out."""
+# flop per (pair, element of the reduction axis) of the forward pass: multiply-add for the dot
+# products; sub, fma with w.t', abs/accumulate and the w.t' multiply-add for TransH (6); the
+# complex difference, modulus and accumulate for RotatE (7 per complex element, its square root
+# not counted).  Backward does the same pair work in both orientations: twice the forward count.
+PAIR_FLOPS = {"DistMult": 2, "ComplEx": 2, "TransE": 3, "TransH": 6, "RotatE": 7, "TransF": 2}
+
+
+def algorithmic_flops(w):
+    klen = w.dim // 2 if w.model == "RotatE" else w.dim
+    if w.model in ("TransR", "RESCAL"):
+        f = 2 * w.batch * w.dim * w.dim
+        return f, 2 * f
+    f = PAIR_FLOPS[w.model] * w.batch * (1 + w.n_neg) * klen
+    return f, 2 * f
+
+
+def kernel_model(w, label, u_ent, u_rel):
+    """(algorithmic bytes, algorithmic flops, arithmetic unit) of ONE launch of the kernel `label`."""
     B, d, rd, N = w.batch, w.dim, w.rel_dim, w.n_neg
     nn = w.n_chunks * N
-    if w.model == "RotatE":
-        # one rotated-head row per positive (written by the positive kernel of the same call), no h / r gathers
-        return 4 * (B * d + nn * d) + 8 * nn + 4 * B * N
+    klen = d // 2 if w.model == "RotatE" else d
     aux_row = d if w.model == "TransH" else 0
-    out_planes = 3 if w.model == "TransH" else 1
-    return 4 * (B * (d + rd + aux_row) + nn * d) + 8 * (2 * B + nn) + 4 * out_planes * B * N
+    dot = w.model in ("DistMult", "ComplEx")
+    pair_flops = PAIR_FLOPS.get(w.model, 0) * B * N * klen
+    l2 = w.model in ("TransE", "TransH") and w.norm_p == 2
+    if label == "score_pos_kernel":
+        by = 4 * B * (2 * d + rd + aux_row) + 8 * 3 * B + 4 * B
+        by += 4 * B * d if w.model == "RotatE" else 0
+        by += 4 * B if w.model == "TransH" else 0
+        return by, PAIR_FLOPS.get(w.model, 2) * B * klen, "valu"
+    if label == "score_neg_kernel":
+        if w.model == "RotatE":  # one rotated-head row per positive, written by the positive kernel of the same call
+            by = 4 * (B * d + nn * d) + 8 * nn + 4 * B * N
+        else:
+            out_planes = 3 if w.model == "TransH" else 1
+            by = 4 * (B * (d + rd + aux_row) + nn * d) + 8 * (2 * B + nn) + 4 * out_planes * B * N
+        return by, pair_flops, "mfma" if dot else "valu"
+    if label == "bwd_tile_kernel":
+        planes_in = 1 + (1 if l2 else 0) + (2 if w.model == "TransH" else 0)   # dneg, scores, TransH side planes
+        rows_in = B * (d if w.model == "RotatE" else d + rd + aux_row) + nn * d
+        rows_out = B * d * (2 if w.model == "TransH" else 1) + nn * d
+        by = 4 * (rows_in + rows_out) + 8 * (2 * B + nn) + 4 * planes_in * B * N
+        return by, 2 * pair_flops, "mfma" if dot else "valu"
+    if label == "bwd_pos_kernel":
+        g_rows = (B * d * (2 if w.model == "TransH" else 1)) if N else 0
+        by = 4 * (B * (2 * d + rd + aux_row) + g_rows + B * (2 * d + rd + aux_row)) + 8 * 3 * B + 8 * B
+        return by, 6 * B * klen, "valu"
+    if label == "seg_reduce_l1":
+        n_occ = 2 * B + nn
+        by = 4 * (n_occ * d + B * (rd + aux_row)) + 8 * (n_occ + B) + 4 * (u_ent * d + u_rel * (rd + aux_row))
+        return by, n_occ * d, "valu"
+    if label == "seg_reduce_l2":
+        return 4 * (u_ent * d) // 8, 0, "valu"
+    if label.startswith("transr_plan_kernel") or label == "transr_gemm_kernel<dX>":
+        by = 4 * (u_rel * d * d + 3 * B * d + u_rel * d) + 8 * 3 * B
+        return by, 2 * B * d * d, "mfma"
+    if label == "transr_dm_kernel":
+        return 4 * (u_rel * d * d + 2 * B * d), 2 * B * d * d, "mfma"
+    if label == "transr_prep_kernel":
+        return 4 * 5 * B * d, 3 * B * d, "valu"
+    return 0, 0, "valu"
 
 
-def neg_kernel_flops(w):
-    per_elem = {"DistMult": 2, "ComplEx": 2, "TransE": 2, "TransH": 9, "RotatE": 8}[w.model]
-    klen = w.dim // 2 if w.model == "RotatE" else w.dim
-    return per_elem * w.batch * w.n_neg * klen
-
-
+# ---- timing ------------------------------------------------------------------------------------
 def time_events(fn, iters, torch):
     """Average milliseconds per call of fn over `iters` back-to-back calls, by HIP events on the
     stream the kernels are launched on (torch's current stream)."""
@@ -111,18 +167,210 @@ def time_events(fn, iters, torch):
     return a.elapsed_time(b) / iters
 
 
-def cpu_baseline(w, target_s=12.0, cap_s=40.0):
-    """The oracle's loops (the restatement of cuke's generated CPU code; gcc -O3, ONE thread)
-    timed on this host over a bounded sample of the same workload: whole chunks of the batch
-    (same dim, chunk size, negatives and index distributions; entity table cut to 200k rows to
-    bound host memory), forward + backward, repeated until about `target_s` seconds of CPU
-    work have been spent.  Beside it: the forward pass alone with OpenMP over all host cores."""
+# ---- parity spot check of the inputs that are timed ----------------------------------------------
+class SpotCheckError(RuntimeError):
+    pass
+
+
+def _tol_ok(got, ref, rows, rtol=1e-5):
+    got, ref = np.asarray(got, np.float64), np.asarray(ref, np.float64)
+    rms = np.sqrt(np.mean(ref * ref, axis=-1, keepdims=True)) if rows else float(np.sqrt(np.mean(ref * ref)))
+    err = np.abs(got - ref)
+    bound = rtol * np.abs(ref) + rtol * rms
+    return err, bound
+
+
+def spot_check(w, model, step, ix, n_pairs=4096, n_pos=512, n_rows=64, n_rel_rows=8, max_triples=40_000, seed=7):
+    """Runs one step on the device and compares, against the CPU oracle evaluated on rows copied
+    back from the device tables: `n_pairs` sampled (positive, negative) pair scores, `n_pos`
+    positive scores and the complete gradient rows of `n_rows` sampled entity ids and `n_rel_rows`
+    relation ids.  A gradient row is checked exactly: the oracle differentiates every triple and
+    pair of the batch that touches the row, written out as explicit triples.  Bar: |got - ref| <=
+    1e-5 |ref| + 1e-5 rms(ref) (rms per gradient row).  L1 gradients are sums of signs of
+    residual elements, and an element within an ulp of zero may take either sign: up to 0.5 % of
+    the elements of the sampled rows may differ, each by at most two flips of the largest
+    upstream gradient.  RotatE unit vectors u/|u| with tiny |u| admit 1e-4 of the elements within
+    4x the bound.  Raises SpotCheckError on a mismatch."""
+    import torch
+    import oracle
+    oracle.build()
+    rng = np.random.default_rng(seed)
+    h, r, t = (ix[k].cpu().numpy() for k in ("h", "r", "t"))
+    neg = ix["neg"].cpu().numpy() if "neg" in ix else None
+    B, N, C = w.batch, w.n_neg, w.chunk
+    do_bwd = w.backward
+    step.select(0)
+    step.run(do_bwd)
+    torch.cuda.synchronize()
+    pos_dev = step.pos.cpu().numpy()
+    neg_dev = step.neg.cpu().numpy() if step.neg is not None else None
+    report = {}
+
+    def gathered(ent_ids, rel_ids):
+        """Compact host copies of the device rows for these ids + the id -> compact index maps."""
+        ue, ur = np.unique(ent_ids), np.unique(rel_ids)
+        dev = model.E.device
+        E = model.E[torch.from_numpy(ue).to(dev)].cpu().numpy()
+        R = model.R[torch.from_numpy(ur).to(dev)].cpu().numpy() if model.R is not None and model.rel_dim else None
+        A = model.A[torch.from_numpy(ur).to(dev)].cpu().numpy() if model.A is not None else None
+        return E, R, A, (lambda x: np.searchsorted(ue, x)), (lambda x: np.searchsorted(ur, x))
+
+    # -- scores
+    bs = rng.choice(B, size=min(n_pos, B), replace=False)
+    fh, fr, ft, want = [h[bs]], [r[bs]], [t[bs]], [pos_dev[bs]]
+    if neg is not None:
+        pb = rng.integers(0, B, n_pairs)
+        pk = rng.integers(0, N, n_pairs)
+        fh.append(h[pb]), fr.append(r[pb]), ft.append(neg[(pb // C) * N + pk]), want.append(neg_dev[pb, pk])
+    fh, fr, ft, want = (np.concatenate(x) for x in (fh, fr, ft, want))
+    E, R, A, me, mr = gathered(np.concatenate([fh, ft]), fr)
+    ref, _ = oracle.score(w.model, E, R, A, me(fh), mr(fr), me(ft), p=w.norm_p, gamma=w.gamma)
+    err, bound = _tol_ok(want, ref, rows=False)
+    if (err > bound).any():
+        i = int(np.argmax(err - bound))
+        raise SpotCheckError(f"{w.name}: {int((err > bound).sum())}/{ref.size} sampled scores differ from the oracle; "
+                             f"worst: device {want[i]!r} oracle {ref[i]!r}")
+    report["scores_checked"] = int(ref.size)
+    if not do_bwd:
+        return report
+
+    # -- upstream gradients as the device step used them
+    if w.loss == "margin":
+        sign = step.sign
+        loss_ref, _, _ = oracle.margin_loss(pos_dev, neg_dev, w.margin, sign)
+        loss_dev = float(step.loss.item())
+        if abs(loss_dev - loss_ref) > 1e-5 * max(1.0, abs(loss_ref)):
+            raise SpotCheckError(f"{w.name}: margin loss {loss_dev!r} differs from the oracle's {loss_ref!r}")
+    dpos = step.dpos.cpu().numpy() if step.dpos is not None else np.zeros(B, np.float32)
+    dneg = step.dneg.cpu().numpy() if step.dneg is not None else None
+    g = step.sparse_grads()
+    ent_ids, rel_ids = g.ent_ids.cpu().numpy(), g.rel_ids.cpu().numpy()
+    occ = np.concatenate([h, t] + ([neg] if neg is not None else []))
+    if not np.array_equal(ent_ids, np.unique(occ)) or not np.array_equal(rel_ids, np.unique(r)):
+        raise SpotCheckError(f"{w.name}: unique ids of the sparse gradients differ from numpy.unique")
+    l1 = w.model in ("TransE", "TransH") and w.norm_p == 1
+    gmax = float(max(np.abs(dpos).max(), np.abs(dneg).max() if dneg is not None else 0.0))
+
+    def explicit_triples(mask_b_full, neg_slots):
+        """Every triple / pair of the batch named by: positives whose whole row set is wanted
+        (mask over b: the positive and all its pairs) and negative slots (chunk, k): all pairs of
+        the chunk with that negative.  Returned as flat (h, r, t, g) without duplicates."""
+        items = set()
+        for b in np.flatnonzero(mask_b_full):
+            items.add((int(b), -1))
+            for k in range(N if neg is not None else 0):
+                items.add((int(b), k))
+        for (c, k) in neg_slots:
+            for b in range(c * C, (c + 1) * C):
+                items.add((b, int(k)))
+        it = np.array(sorted(items), dtype=np.int64).reshape(-1, 2)
+        b_, k_ = it[:, 0], it[:, 1]
+        is_pos = k_ < 0
+        tt = np.where(is_pos, t[b_], neg[(b_ // C) * N + np.maximum(k_, 0)] if neg is not None else t[b_])
+        gg = np.where(is_pos, dpos[b_], dneg[b_, np.maximum(k_, 0)] if dneg is not None else 0.0).astype(np.float32)
+        return h[b_], r[b_], tt, gg
+
+    def check_rows(kind, ids, dev_rows_of, ref_rows_of):
+        bad_total = checked = flips = 0
+        for e in ids:
+            got, ref = dev_rows_of(e), ref_rows_of(e)
+            if ref is None:
+                continue
+            err, bound = _tol_ok(got, ref, rows=True)
+            bad = err > bound
+            checked += ref.size
+            if bad.any():
+                if l1 and (err[bad] <= 4.0 * gmax * (1 + 1e-5)).all():
+                    flips += int(bad.sum())
+                elif w.model == "RotatE" and (err <= 4 * bound).all():
+                    bad_total += int(bad.sum())
+                else:
+                    i = np.unravel_index(np.argmax(err - bound), err.shape)
+                    raise SpotCheckError(f"{w.name}: gradient row of {kind} {int(e)} differs from the oracle at {i}: "
+                                         f"device {np.asarray(got)[i]!r} oracle {np.asarray(ref)[i]!r}")
+        if checked and flips > 5e-3 * checked:
+            raise SpotCheckError(f"{w.name}: {flips}/{checked} L1 gradient elements of {kind} rows differ by sign flips")
+        if checked and bad_total > 1e-4 * checked + 1:
+            raise SpotCheckError(f"{w.name}: {bad_total}/{checked} RotatE gradient elements of {kind} rows outside the bound")
+        return checked, flips
+
+    ent_rows_dev, rel_rows_dev, aux_rows_dev = g.ent_rows, g.rel_rows, g.aux_rows
+
+    def oracle_rows(fh, fr, ft, fg):
+        E, R, A, me, mr = gathered(np.concatenate([fh, ft]), fr)
+        ref = oracle.backward(w.model, E, R, A, me(fh), mr(fr), me(ft), None, 0, fg, None, p=w.norm_p)
+        return ref, np.unique(np.concatenate([fh, ft])), np.unique(fr)
+
+    # -- entity rows
+    def ent_ref(e):
+        mb = (h == e) | (t == e)
+        slots = [(int(s // N), int(s % N)) for s in np.flatnonzero(neg == e)] if neg is not None else []
+        n_tr = int(mb.sum()) * (1 + (N if neg is not None else 0)) + len(slots) * C
+        if n_tr > max_triples:
+            return None
+        fh, fr, ft, fg = explicit_triples(mb, slots)
+        ref, ue, _ = oracle_rows(fh, fr, ft, fg)
+        return ref.ent_rows[int(np.searchsorted(ue, e))]
+
+    pick = rng.permutation(ent_ids)[: 4 * n_rows]
+    done = []
+
+    def ent_ref_capped(e):
+        if len(done) >= n_rows:
+            return None
+        ref = ent_ref(e)
+        if ref is not None:
+            done.append(e)
+        return ref
+
+    pos_of = {int(e): i for i, e in enumerate(ent_ids)}
+    n_e, f_e = check_rows("entity", pick, lambda e: ent_rows_dev[pos_of[int(e)]].cpu().numpy(), ent_ref_capped)
+
+    # -- relation (and auxiliary) rows
+    rpos_of = {int(e): i for i, e in enumerate(rel_ids)}
+    done_r = []
+
+    def rel_ref(rid, aux):
+        mb = r == rid
+        if int(mb.sum()) * (1 + (N if neg is not None else 0)) > max_triples or len(done_r) >= 2 * n_rel_rows:
+            return None
+        fh, fr, ft, fg = explicit_triples(mb, [])
+        ref, _, ur = oracle_rows(fh, fr, ft, fg)
+        done_r.append(rid)
+        rows = ref.aux_rows if aux else ref.rel_rows
+        return rows[int(np.searchsorted(ur, rid))]
+
+    rpick = rng.permutation(rel_ids)[: 4 * n_rel_rows]
+    n_r = f_r = 0
+    if rel_rows_dev is not None:
+        n_r, f_r = check_rows("relation", rpick, lambda e: rel_rows_dev[rpos_of[int(e)]].cpu().numpy(),
+                              lambda e: rel_ref(e, False))
+    n_a = f_a = 0
+    if aux_rows_dev is not None:
+        done_r.clear()
+        n_a, f_a = check_rows("relation (aux table)", rpick[: n_rel_rows],
+                              lambda e: aux_rows_dev[rpos_of[int(e)]].cpu().numpy(), lambda e: rel_ref(e, True))
+    report.update({"entity_rows_checked": len(done), "gradient_elements_checked": int(n_e + n_r + n_a),
+                   "l1_sign_flips": int(f_e + f_r + f_a)})
+    return report
+
+
+# ---- CPU baseline ------------------------------------------------------------------------------
+def cpu_baseline(w, target_s=4.0):
+    """The oracle's loops (the restatement of cuke's generated CPU code) timed on this host over a
+    bounded sample of the same workload: whole chunks of the batch (same dim, chunk size, negatives
+    and index distributions; entity table cut to 200k rows to bound host memory), forward +
+    backward, repeated until about `target_s` seconds of CPU work have been spent on one thread
+    (gcc -O3), then the same with OpenMP over the batch on all host cores for about half as long."""
     import oracle
     from cuke_amd import synth
     oracle.build()
     n_ent = min(w.n_ent, 200_000)
     unit = w.chunk if w.chunk else min(w.batch, 1024)
-    s = synth.make_workload(w.name, seed=w.seed, n_ent=n_ent)
+    base, over = (w.name, {}) if w.name in synth.CONFIGS else ("cfg3_transr", dict(dim=w.dim))
+    s = synth.make_workload(base, seed=w.seed, n_ent=n_ent, **over)
+    if s.model in ("TransR", "RESCAL") and s.dim >= 512:
+        unit = 256  # bounds the per-thread d x d gradient accumulators of the OpenMP leg
     a = s.arrays
 
     def run(b0, b1, fast):
@@ -133,44 +381,200 @@ def cpu_baseline(w, target_s=12.0, cap_s=40.0):
                                  s.chunk, p=s.norm_p, gamma=s.gamma, fast=fast)
         tf = time.perf_counter() - t0
         tb = 0.0
-        if s.backward and fast == "o3":
+        if s.backward:
             dneg = np.ones_like(negs) if negs is not None else None
             t0 = time.perf_counter()
             oracle.backward(s.model, a["E"], a["R"], a["A"], a["h"][sl], a["r"][sl], a["t"][sl], neg, s.chunk,
-                            np.ones_like(pos), dneg, p=s.norm_p, fast="o3")
+                            np.ones_like(pos), dneg, p=s.norm_p, fast=fast)
             tb = time.perf_counter() - t0
         return tf, tb
 
-    t_fwd = t_bwd = 0.0
-    scored = 0
-    done = 0
-    while True:
-        b0 = (done * unit) % s.batch
-        tf, tb = run(b0, b0 + unit, "o3")
-        t_fwd, t_bwd, done = t_fwd + tf, t_bwd + tb, done + 1
-        scored += unit * (1 + s.n_neg)
-        spent = t_fwd + t_bwd
-        if spent >= target_s or spent + spent / done > cap_s:
-            break
+    def leg(fast, budget):
+        t_fwd = t_bwd = 0.0
+        scored = done = 0
+        while True:
+            b0 = (done * unit) % s.batch
+            tf, tb = run(b0, b0 + unit, fast)
+            t_fwd, t_bwd, done = t_fwd + tf, t_bwd + tb, done + 1
+            scored += unit * (1 + s.n_neg)
+            spent = t_fwd + t_bwd
+            if spent >= budget or spent + spent / done > 2.5 * budget:
+                return scored, t_fwd, t_bwd, done
+
+    scored, t_fwd, t_bwd, done = leg("o3", target_s)
     run(0, unit, "omp")  # first call starts the OpenMP thread pool
-    tf_omp, _ = run(0, unit, "omp")
-    return {"value": scored / (t_fwd + t_bwd), "unit": "triples scored/s", "cores": 1, "kind": "port",
-            "sample": f"{s.model} dim={s.dim} n_ent={s.n_ent}: {done} x (B={unit}, N={s.n_neg}) = {scored} scores, "
-                      f"fwd {t_fwd:.2f}s + bwd {t_bwd:.2f}s, gcc -O3 -march=x86-64-v3, 1 thread",
-            "fwd_s": t_fwd, "bwd_s": t_bwd,
-            "forward_only_openmp": {"value": unit * (1 + s.n_neg) / tf_omp, "unit": "triples scored/s",
-                                    "cores": oracle.threads("omp")}}
+    scored_m, tf_m, tb_m, done_m = leg("omp", target_s / 2)
+    what = "fwd+bwd" if s.backward else "fwd"
+    out = {"value": scored / (t_fwd + t_bwd), "unit": "triples scored/s", "cores": 1, "kind": "port",
+           "sample": f"{s.model} dim={s.dim} n_ent={s.n_ent}: {done} x (B={unit}, N={s.n_neg}) = {scored} scores {what}, "
+                     f"fwd {t_fwd:.2f}s + bwd {t_bwd:.2f}s, gcc -O3 -march=x86-64-v3, 1 thread",
+           "fwd_s": t_fwd, "bwd_s": t_bwd,
+           "all_cores": {"value": scored_m / (tf_m + tb_m), "unit": "triples scored/s", "cores": oracle.threads("omp"),
+                         "sample": f"{done_m} x (B={unit}, N={s.n_neg}) {what}, OpenMP over the batch, "
+                                   f"fwd {tf_m:.2f}s + bwd {tb_m:.2f}s"}}
+    if not s.chunk and not s.backward:
+        # the flags the reference's own JIT build of its generated C++ gets: no optimisation flag, one thread
+        sc0, tf0, tb0, d0 = leg("o0", 1.0)
+        out["as_the_reference_builds_it"] = {"value": sc0 / (tf0 + tb0), "unit": "triples scored/s", "cores": 1,
+                                             "sample": f"{d0} x B={unit} fwd, gcc -O0, 1 thread"}
+    return out
+
+
+# ---- one workload ------------------------------------------------------------------------------
+def make_named_workload(name, seed):
+    from cuke_amd import synth
+    if name == "ref_transr_8192x512":
+        # the TransR shape of the reference's own sweep scripts (apps/kge/scripts/test_fig9c_cuke.sh:
+        # batch 8192, dim 512); tables and relation distribution as in the TransR benchmark configuration
+        w = synth.make_workload("cfg3_transr", seed=seed, tables=False, dim=512)
+        w.name = name
+        return w
+    return synth.make_workload(name, seed=seed, tables=False)
+
+
+def run_workload(name, args, torch):
+    from cuke_amd.kge import KGEModel, TrainStep
+    dev = torch.device("cuda:0")
+    w = make_named_workload(name, args.seed)
+    E, R, A = device_tables(w, dev)
+    model = KGEModel(w.model, E, R, A, norm_p=w.norm_p, gamma=w.gamma)
+    nb = max(1, args.batches)
+    sets = [w] + [make_named_workload(name, args.seed + 1 + i) for i in range(nb - 1)]
+    ixs = [{k: torch.from_numpy(v).to(dev) for k, v in s.arrays.items() if v is not None} for s in sets]
+    sign = 1.0 if w.model in ("DistMult", "ComplEx", "RotatE", "TransF", "RESCAL") else -1.0
+    ix = ixs[0]
+    step = TrainStep(model, ix["h"], ix["r"], ix["t"], ix.get("neg"), w.chunk or None, loss=w.loss,
+                     margin=w.margin, sign=sign)
+    for o in ixs[1:]:
+        step.add_batch(o["h"], o["r"], o["t"], o.get("neg"))
+    do_bwd = w.backward
+
+    check = {"parity_spot_check": "skipped (--no-check)"}
+    if not args.no_check:
+        t0 = time.perf_counter()
+        check = {"parity_spot_check": "ok", **spot_check(w, model, step, ix), "seconds": None}
+        check["seconds"] = round(time.perf_counter() - t0, 2)
+
+    def timed(one):
+        for _ in range(args.warmup):
+            one()
+        torch.cuda.synchronize()
+        return time_events(one, args.steps, torch)
+
+    counter = [0]
+
+    def rotating(run_one):
+        def f():
+            i = counter[0] % nb
+            counter[0] += 1
+            run_one(i)
+        return f
+
+    def direct(i):
+        step.select(i)
+        step.run(do_bwd)
+
+    step.select(0)
+    ms_same = timed(lambda: step.run(do_bwd))
+    ms_rot = timed(rotating(direct))
+    ms_graph = None
+    issue, ms = "direct", ms_rot
+    if not args.no_graph:
+        graphs = []
+        for i in range(nb):
+            step.select(i)
+            graphs.append(step.capture(do_bwd))
+        ms_graph = timed(rotating(lambda i: graphs[i].replay()))
+        if ms_graph < ms:
+            issue, ms = "graph", ms_graph
+        del graphs
+        step.graph = None
+
+    # DistMult / ComplEx: the same rotating loop with the pair sums of the tile kernels on the vector ALUs
+    ms_forms = None
+    if w.model in ("DistMult", "ComplEx") and w.chunk and do_bwd:
+        model.pair_sums = "vector_alus"
+        ms_valu = timed(rotating(direct))
+        model.pair_sums = "matrix_cores"
+        ms_forms = {"matrix_cores": ms_rot, "vector_alus": ms_valu}
+
+    step.select(0)
+    u_ent, u_rel = step.ent_insp.num_unique, step.rel_insp.num_unique
+    if not do_bwd:
+        occ = torch.cat([ix["h"], ix["t"]] + ([ix["neg"]] if "neg" in ix else []))
+        u_ent, u_rel = int(torch.unique(occ).numel()), int(torch.unique(ix["r"]).numel())
+    fwd_b, bwd_b = algorithmic_bytes(w, u_ent, u_rel)
+    fwd_f, bwd_f = algorithmic_flops(w)
+    total_b = fwd_b + (bwd_b if do_bwd else 0)
+    total_f = fwd_f + (bwd_f if do_bwd else 0)
+    scores = w.scores_per_step
+
+    # per-kernel durations, live: an event behind every kernel, rotating batches; a long fill kernel
+    # in front of each step lets the host enqueue the whole step before the device starts it
+    lead = torch.empty(128 * 1024 * 1024, dtype=torch.float32, device=dev)
+    kt = step.kernel_times(steps=max(8, min(32, args.steps)), backward=do_bwd, batches=list(range(nb)), lead=lead)
+    del lead
+    kt_sum = sum(ms_k for _, ms_k in kt)
+    kname, k_ms = max(kt, key=lambda x: x[1])
+    k_bytes, k_flops, k_unit = kernel_model(w, kname, u_ent, u_rel)
+    bound = BOUND.get(name, "hbm")
+    gbs = k_bytes / (k_ms * 1e-3) / 1e9
+    tfs = k_flops / (k_ms * 1e-3) / 1e12
+    hbm_roof = {"achieved": gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": gbs / HBM_PEAK_GBS}
+    fp32_roof = {"achieved": tfs, "peak": FP32_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": tfs / FP32_PEAK_TFLOPS,
+                 "arithmetic_unit": "fp32 MFMA" if k_unit == "mfma" else "fp32 vector ALUs"}
+    main_roof, other = (hbm_roof, fp32_roof) if bound == "hbm" else (fp32_roof, hbm_roof)
+    step_gbs = total_b / (ms * 1e-3) / 1e9
+    step_tfs = total_f / (ms * 1e-3) / 1e12
+    roofline = {"kernel": kname, "bound": "hbm" if bound == "hbm" else "mfma" if k_unit == "mfma" else "fp32_valu",
+                "achieved": main_roof["achieved"], "peak": main_roof["peak"], "unit": main_roof["unit"],
+                "frac": main_roof["frac"], "traffic": MEASURED_TRAFFIC_BYTES.get((name, kname)),
+                "kernel_ms": k_ms, "kernel_share_of_step": k_ms / kt_sum if kt_sum else None,
+                "algorithmic_bytes_per_launch": k_bytes, "algorithmic_flops_per_launch": k_flops,
+                "other_roof": {"bound": "fp32" if bound == "hbm" else "hbm", **other},
+                "step": {"bound": bound, "frac": (step_gbs / HBM_PEAK_GBS) if bound == "hbm" else (step_tfs / FP32_PEAK_TFLOPS),
+                         "hbm_gbs": step_gbs, "hbm_frac": step_gbs / HBM_PEAK_GBS, "fp32_tflops": step_tfs,
+                         "fp32_frac": step_tfs / FP32_PEAK_TFLOPS, "algorithmic_bytes": total_b,
+                         "algorithmic_flops": total_f}}
+
+    out = {
+        "metric": "triples scored/sec fwd+bwd per KGE model; % of HBM (or MFMA) roofline",
+        "value": scores / (ms * 1e-3),
+        "unit": "triples scored/s",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": ms,
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32",
+        "data": "synthetic (seeded N(0,sigma) tables, Zipf/uniform indices, shared negatives per chunk)",
+        "config": {"workload": w.name, "score_function": w.model, "n_ent": w.n_ent, "n_rel": w.n_rel, "dim": w.dim,
+                   "batch": w.batch, "chunk": w.chunk, "n_neg": w.n_neg, "norm_p": w.norm_p,
+                   "backward": do_bwd, "loss": w.loss, "issue": issue, "rotating_batches": nb,
+                   "pair_sums": "matrix cores, fp32" if w.model in ("DistMult", "ComplEx") and w.chunk else "vector ALUs",
+                   "ms_per_step_rotating_direct": ms_rot, "ms_per_step_rotating_graph": ms_graph,
+                   "ms_per_step_same_batch": ms_same, "ms_per_step_by_pair_sum_unit": ms_forms,
+                   "scores_per_step": scores, "positives_per_s": w.batch / (ms * 1e-3),
+                   "unique_entity_rows": u_ent, "unique_relation_rows": u_rel},
+        "kernels_ms": [[n_, round(m_, 6)] for n_, m_ in kt],
+        "roofline": roofline,
+        **check,
+    }
+    if not args.no_cpu:
+        out["cpu_baseline"] = cpu_baseline(w, args.cpu_seconds)
+    del step, model, E, R, A, ixs
+    torch.cuda.empty_cache()
+    return out
 
 
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=200)
-    ap.add_argument("--warmup", type=int, default=20)
-    ap.add_argument("--workload", default="cfg2_distmult")
-    ap.add_argument("--no-graph", action="store_true", help="launch kernels one by one instead of a HIP graph")
-    ap.add_argument("--no-pipeline", action="store_true", help="do not try the double-buffered inspector")
-    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--steps", type=int, default=100)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--workload", default="all",
+                    help="all (default), one of " + ", ".join(ALL_WORKLOADS) + ", or ref_transr_8192x512")
+    ap.add_argument("--batches", type=int, default=8, help="distinct seeded batches the timed loop rotates over")
+    ap.add_argument("--no-graph", action="store_true", help="do not also time HIP-graph replays of the step")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline legs")
+    ap.add_argument("--no-check", action="store_true", help="skip the parity spot check (profiling runs)")
+    ap.add_argument("--cpu-seconds", type=float, default=4.0, help="one-thread CPU work per workload")
     ap.add_argument("--seed", type=int, default=0)
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run one 256 MiB device-to-device copy kernel (a known-traffic reference "
@@ -182,8 +586,6 @@ def main():
         sys.exit(2)
 
     import torch
-    from cuke_amd import synth
-    from cuke_amd.kge import KGEModel, TrainStep
 
     dev = torch.device("cuda:0")
     if args.calibrate_copy:
@@ -192,154 +594,23 @@ def main():
         dst.copy_(src)  # one elementwise copy kernel: reads 256 MiB, writes 256 MiB
         torch.cuda.synchronize()
         del src, dst
-    w = synth.make_workload(args.workload, seed=args.seed, tables=False)
-    E, R, A = device_tables(w, dev)
-    model = KGEModel(w.model, E, R, A, norm_p=w.norm_p, gamma=w.gamma)
-    ix = {k: torch.from_numpy(v).to(dev) for k, v in w.arrays.items() if v is not None}
-    sign = 1.0 if w.model in ("DistMult", "ComplEx", "RotatE", "TransF", "RESCAL") else -1.0
-    step = TrainStep(model, ix["h"], ix["r"], ix["t"], ix.get("neg"), w.chunk or None, loss=w.loss,
-                     margin=w.margin, sign=sign)
-    do_bwd = w.backward
-
-    # Three ways to issue the same step: kernel by kernel from the host; kernel by kernel with the
-    # index tensors and inspections in a ring of sets, so the inspector of batch i+1 (side stream)
-    # is enqueued before step i and neither stream waits for the other on the critical path (every
-    # timed step still enqueues exactly one inspection and one forward / loss / backward); or as
-    # one HIP graph replay.  All are warmed up and timed
-    # over exactly --steps steps, every step doing its own inspection, forward, loss and backward;
-    # the fastest is the reported configuration (a graph replay has a fixed host cost that only
-    # pays off when the step has many kernels).
-    def timed(one):
-        for _ in range(args.warmup):
-            one()
-        torch.cuda.synchronize()
+    names = ALL_WORKLOADS if args.workload == "all" else [args.workload]
+    results = []
+    for n in names:
         t0 = time.perf_counter()
-        ms_ = time_events(one, args.steps, torch)
-        return ms_, time.perf_counter() - t0
-
-    ms_direct, wall = timed(lambda: step.run(do_bwd))
-    ms_graph = ms_pipe = None
-    issue = "direct"
-    ms = ms_direct
-    if do_bwd and not args.no_pipeline:
-        def one_pipelined():
-            step.stage()  # inspector of the batch after the one that runs now (side stream)
-            step.run(do_bwd, pipeline=True)
-        step.stage()  # primes the ring: from here on one batch is always inspected ahead
-        ms_pipe, wall_p = timed(one_pipelined)
-        step.run(do_bwd, pipeline=True)  # drains the batch staged last
-        if ms_pipe < ms:
-            ms, wall, issue = ms_pipe, wall_p, "pipelined"
-    if not args.no_graph:
-        step.capture(do_bwd)
-        ms_graph, wall_g = timed(step.replay)
-        if ms_graph < ms:
-            ms, wall, issue = ms_graph, wall_g, "graph"
-    use_graph = issue == "graph"
-
-    # DistMult / ComplEx: the same step with the pair sums of the tile kernels on the other unit
-    # (matrix cores <-> vector ALUs), direct launches, for comparison; the setting is restored
-    ms_forms = None
-    if w.model in ("DistMult", "ComplEx") and w.chunk and do_bwd:
-        from cuke_amd import _lib as _l
-        was = _l.lib().kge_set_pair_sum_unit(0)
-        _l.lib().kge_set_pair_sum_unit(1 - was)
-        ms_other, _ = timed(lambda: step.run(do_bwd))
-        _l.lib().kge_set_pair_sum_unit(was)
-        ms_forms = {"matrix_cores": ms_other if was else ms_direct, "vector_alus": ms_direct if was else ms_other}
-
-    u_ent, u_rel = step.ent_insp.num_unique, step.rel_insp.num_unique
-    fwd_b, bwd_b = algorithmic_bytes(w, u_ent, u_rel)
-    total_b = fwd_b + (bwd_b if do_bwd else 0)
-    scores = w.scores_per_step
-
-    # per-stage times, un-graphed, each stage launched back to back
-    st = torch.cuda.current_stream().cuda_stream
-    import ctypes
-    stc = ctypes.c_void_p(st)
-    stages = {"inspect_ms": time_events(lambda: step.inspect(stc), 50, torch),
-              "forward_ms": time_events(lambda: step.forward(stc), 50, torch)}
-    if do_bwd:
-        stages["loss_ms"] = time_events(lambda: step.loss_grad(stc), 50, torch)
-        stages["backward_ms"] = time_events(lambda: step.backward(stc), 50, torch)
-
-    # dominant kernel in isolation: the shared-negative forward tile kernel (or, for
-    # positive-only workloads, the per-triple kernel), K launches between two events
-    from cuke_amd import _lib
-    L = _lib.lib()
-    if w.chunk:
-        P = lambda t: ctypes.c_void_p(t.data_ptr()) if t is not None else None
-        kname = "score_neg_mfma_kernel" if w.model in ("DistMult", "ComplEx") else "score_neg_kernel"
-        if w.model in ("TransH", "RotatE"):
-            # the tile kernel reads what the positive kernel of the same call leaves behind (w.h, the
-            # rotated heads): time the forward call and the positive kernel alone, report the
-            # difference
-            t_pair = time_events(lambda: step.forward(stc), 100, torch)
-            t_pos = time_events(lambda: L.kge_score_fwd(ctypes.byref(model._tab), ctypes.byref(step.bat), P(step.pos),
-                                                        None, P(step.side_pos), None, P(step.residual), None, 0, stc),
-                                100, torch)
-            k_ms = t_pair - t_pos
-        else:
-            k_ms = time_events(lambda: L.kge_score_fwd(ctypes.byref(model._tab), ctypes.byref(step.bat), None,
-                                                       P(step.neg), None, None, None, None, 0, stc), 100, torch)
-        k_bytes, k_flops = neg_kernel_bytes(w), neg_kernel_flops(w)
-        # the two memory-bound pieces of a shared-negative step, on their own: the per-positive
-        # gather kernel and the inspection of concat(h, t, neg) and r
-        if w.model not in ("TransH", "RotatE"):
-            t_pos = time_events(lambda: L.kge_score_fwd(ctypes.byref(model._tab), ctypes.byref(step.bat), P(step.pos),
-                                                        None, P(step.side_pos), None, P(step.residual), None, 0, stc),
-                                100, torch)
-        aux_row = w.dim if w.model == "TransH" else 0
-        pos_bytes = 4 * w.batch * (2 * w.dim + w.rel_dim + aux_row) + 8 * 3 * w.batch + 4 * w.batch \
-            + (4 * w.batch * w.dim if w.model == "RotatE" else 0) + (4 * w.batch if w.model == "TransH" else 0)
-        n_ids = step.n_occ + w.batch
-        insp_bytes = n_ids * (8 + 3 * 4) + (u_ent + u_rel) * (8 + 4)  # ids in; perm, inverse, segment per id; unique ids, offsets
-        extra = {"positive_gather": {"kernel": "score_pos_kernel", "ms": t_pos, "algorithmic_bytes": pos_bytes,
-                                     "gbs": pos_bytes / (t_pos * 1e-3) / 1e9,
-                                     "hbm_frac": pos_bytes / (t_pos * 1e-3) / 1e9 / HBM_PEAK_GBS},
-                 "inspection": {"ids": n_ids, "ms": stages["inspect_ms"], "algorithmic_bytes": insp_bytes,
-                                "ids_per_s": n_ids / (stages["inspect_ms"] * 1e-3),
-                                "note": "stand-alone inspector launches; in the timed step its workgroups ride with the "
-                                        "score kernels where the batch qualifies"}}
-    else:
-        # positive-only workloads: the forward call is one kernel (TransR: the tile-plan kernel,
-        # a few microseconds, plus the grouped MFMA kernel)
-        kname = "score_pos_kernel" if w.model != "TransR" else "transr_plan_kernel + transr_gemm_kernel<0>"
-        k_ms = time_events(lambda: step.forward(stc), 100, torch)
-        k_bytes = fwd_b
-        k_flops = 2 * w.batch * w.dim * w.dim if w.model == "TransR" else 3 * w.batch * w.dim
-        extra = {}
-    achieved = k_bytes / (k_ms * 1e-3) / 1e9
-
-    out = {
-        "metric": "triples scored/sec fwd+bwd per KGE model; % of HBM (or MFMA) roofline",
-        "value": scores / (ms * 1e-3),
-        "unit": "triples scored/s",
-        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": ms,
-        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32",
-        "data": "synthetic (seeded N(0,sigma) tables, Zipf/uniform indices, shared negatives per chunk)",
-        "config": {"workload": w.name, "score_function": w.model, "n_ent": w.n_ent, "n_rel": w.n_rel, "dim": w.dim,
-                   "batch": w.batch, "chunk": w.chunk, "n_neg": w.n_neg, "norm_p": w.norm_p,
-                   "backward": do_bwd, "loss": w.loss, "hip_graph": use_graph, "issue": issue,
-                   "pair_sums": ("vector ALUs (KGE_DOT_VALU=1)" if os.environ.get("KGE_DOT_VALU", "0") not in ("", "0")
-                                 else "matrix cores, fp32 (default)") if w.model in ("DistMult", "ComplEx") and w.chunk
-                   else "vector ALUs",
-                   "ms_per_step_direct": ms_direct, "ms_per_step_pipelined": ms_pipe,
-                   "ms_per_step_graph": ms_graph, "ms_per_step_direct_by_pair_sum_unit": ms_forms,
-                   "scores_per_step": scores, "positives_per_s": w.batch / (ms * 1e-3),
-                   "unique_entity_rows": u_ent, "unique_relation_rows": u_rel},
-        "step": {"algorithmic_bytes": total_b, "hbm_gbs": total_b / (ms * 1e-3) / 1e9,
-                 "hbm_frac": total_b / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, "wall_s": wall, **stages, **extra},
-        "roofline": {"kernel": kname, "bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": achieved / HBM_PEAK_GBS, "traffic": MEASURED_TRAFFIC_BYTES.get(w.name),
-                     "kernel_ms": k_ms,
-                     "algorithmic_bytes_per_launch": k_bytes,
-                     ("fp32_mfma" if w.model in ("TransR", "DistMult", "ComplEx") else "fp32_valu"): {"flops_per_launch": k_flops,
-                                   "achieved_tflops": k_flops / (k_ms * 1e-3) / 1e12,
-                                   "frac_of_157.3": k_flops / (k_ms * 1e-3) / 1e12 / FP32_PEAK_TFLOPS}},
-    }
-    if not args.no_cpu:
-        out["cpu_baseline"] = cpu_baseline(w)
+        try:
+            res = run_workload(n, args, torch)
+        except SpotCheckError as e:
+            print(f"bench.py: parity spot check failed, nothing is reported: {e}", file=sys.stderr)
+            sys.exit(1)
+        res["bench_seconds"] = round(time.perf_counter() - t0, 1)
+        results.append(res)
+        print(f"[bench] {n}: {res['ms_per_step']:.4f} ms/step, {res['value']:.3e} scores/s, dominant "
+              f"{res['roofline']['kernel']} {res['roofline']['frac']:.3f} of {res['roofline']['bound']}",
+              file=sys.stderr, flush=True)
+    out = results[0]
+    if len(results) > 1:
+        out["per_workload"] = results[1:]
     print(json.dumps(out))
 
 

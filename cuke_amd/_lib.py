@@ -21,7 +21,7 @@ class KgeError(RuntimeError):
 
 class Tables(C.Structure):
     _fields_ = [("model", C.c_int32), ("norm_p", C.c_int32), ("gamma", C.c_float),
-                ("reserved", C.c_int32), ("dim", C.c_int64), ("rel_dim", C.c_int64),
+                ("flags", C.c_int32), ("dim", C.c_int64), ("rel_dim", C.c_int64),
                 ("n_ent", C.c_int64), ("n_rel", C.c_int64),
                 ("ent", C.c_void_p), ("rel", C.c_void_p), ("aux", C.c_void_p)]
 
@@ -38,12 +38,20 @@ class InspectJob(C.Structure):
                 ("workspace", C.c_void_p), ("workspace_bytes", C.c_size_t)]
 
 
+class Timeline(C.Structure):
+    _fields_ = [("begin", C.c_void_p), ("events", C.POINTER(C.c_void_p)), ("labels", C.POINTER(C.c_char_p)),
+                ("capacity", C.c_int32), ("count", C.c_int32)]
+
+
+PAIR_SUMS_VALU = 1  # kge_tables.flags
+
+
 class Batch(C.Structure):
     _fields_ = [("batch", C.c_int64), ("h", C.c_void_p), ("r", C.c_void_p), ("t", C.c_void_p),
                 ("neg", C.c_void_p), ("chunk", C.c_int64), ("n_neg", C.c_int64),
                 ("ent_insp", C.POINTER(Inspection)), ("rel_insp", C.POINTER(Inspection)),
                 ("insp_ready", C.c_void_p), ("neg_mode", C.c_int32), ("fuse_inspection", C.c_int32),
-                ("insp_jobs", C.c_void_p)]
+                ("insp_jobs", C.c_void_p), ("timeline", C.POINTER(Timeline))]
 
 
 class Saved(C.Structure):
@@ -60,7 +68,11 @@ EXPORTS = {
     # name: (restype, argtypes)
     "kge_strerror": (C.c_char_p, [C.c_int]),
     "kge_abi_version": (C.c_int, []),
-    "kge_set_pair_sum_unit": (C.c_int, [C.c_int]),
+    "kge_timeline_create": (C.POINTER(Timeline), [C.c_int32]),
+    "kge_timeline_destroy": (None, [C.POINTER(Timeline)]),
+    "kge_timeline_begin": (C.c_int, [C.POINTER(Timeline), C.c_void_p]),
+    "kge_timeline_mark": (C.c_int, [C.POINTER(Timeline), C.c_char_p, C.c_void_p]),
+    "kge_timeline_elapsed": (C.c_int, [C.POINTER(Timeline), C.POINTER(C.c_float)]),
     "kge_residual_fwd": (C.c_int, [C.POINTER(Tables), C.POINTER(Batch), C.c_void_p, C.c_void_p, C.c_size_t,
                                    C.c_void_p]),
     "kge_score_fwd_workspace": (C.c_size_t, [C.POINTER(Tables), C.POINTER(Batch)]),
@@ -94,7 +106,7 @@ EXPORTS = {
 _lib = None
 
 
-ABI_VERSION = 3  # layout of the ctypes structures above; must match kge_abi_version()
+ABI_VERSION = 4  # layout of the ctypes structures above; must match kge_abi_version()
 
 
 def lib() -> C.CDLL:

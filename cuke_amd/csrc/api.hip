@@ -4,16 +4,6 @@
 #include "inspector_mid.hpp"
 
 namespace kge {
-static int g_dot_valu = -1;  // -1: not read from the environment yet
-int dot_valu_option()
-{
-    if (g_dot_valu < 0) {
-        const char *e = getenv("KGE_DOT_VALU");
-        g_dot_valu = e && atoi(e) != 0 ? 1 : 0;
-    }
-    return g_dot_valu;
-}
-
 int launch_score_pos(const kge_tables *, const kge_batch *, float *, float *, float *, hipStream_t);
 int launch_score_pos_fused(const kge_tables *, const kge_batch *, float *, float *, float *, const FusedInsp *,
                            hipStream_t);
@@ -74,6 +64,7 @@ static int validate_tables(const kge_tables *tab)
     if (tab->rel_dim != rel_width(tab->model, tab->dim)) return KGE_ESHAPE;
     if (tab->rel_dim > 0 && (!tab->rel || tab->n_rel <= 0)) return KGE_EINVAL;
     if (aux_width(tab->model, tab->dim) > 0 && !tab->aux) return KGE_EINVAL;
+    if (tab->flags & ~KGE_PAIR_SUMS_VALU) return KGE_EINVAL;
     const bool normed = tab->model == KGE_TRANSE || tab->model == KGE_TRANSH || tab->model == KGE_TRANSR;
     if (normed && tab->norm_p != 1 && tab->norm_p != 2) return KGE_EINVAL;
     return KGE_OK;
@@ -110,13 +101,68 @@ const char *kge_strerror(int status)
     }
 }
 
-int kge_abi_version(void) { return 3; }
+int kge_abi_version(void) { return 4; }
 
-int kge_set_pair_sum_unit(int vector_alu)
+kge_timeline *kge_timeline_create(int32_t capacity)
 {
-    const int before = dot_valu_option();
-    g_dot_valu = vector_alu ? 1 : 0;
-    return before;
+    if (capacity <= 0 || capacity > 4096) return nullptr;
+    kge_timeline *tl = static_cast<kge_timeline *>(calloc(1, sizeof(kge_timeline)));
+    if (!tl) return nullptr;
+    tl->events = static_cast<void **>(calloc((size_t)capacity, sizeof(void *)));
+    tl->labels = static_cast<const char **>(calloc((size_t)capacity, sizeof(char *)));
+    tl->capacity = capacity;
+    bool ok = tl->events && tl->labels;
+    hipEvent_t ev;
+    if (ok && hipEventCreate(&ev) == hipSuccess) tl->begin = ev;
+    else ok = false;
+    for (int i = 0; ok && i < capacity; ++i) {
+        if (hipEventCreate(&ev) == hipSuccess) tl->events[i] = ev;
+        else ok = false;
+    }
+    if (!ok) {
+        kge_timeline_destroy(tl);
+        return nullptr;
+    }
+    return tl;
+}
+
+void kge_timeline_destroy(kge_timeline *tl)
+{
+    if (!tl) return;
+    if (tl->begin) (void)hipEventDestroy(reinterpret_cast<hipEvent_t>(tl->begin));
+    for (int i = 0; tl->events && i < tl->capacity; ++i)
+        if (tl->events[i]) (void)hipEventDestroy(reinterpret_cast<hipEvent_t>(tl->events[i]));
+    free(tl->events);
+    free(const_cast<char **>(tl->labels));
+    free(tl);
+}
+
+int kge_timeline_begin(kge_timeline *tl, void *stream)
+{
+    if (!tl || !tl->begin) return KGE_EINVAL;
+    tl->count = 0;
+    return hipEventRecord(reinterpret_cast<hipEvent_t>(tl->begin), as_stream(stream)) == hipSuccess ? KGE_OK : KGE_ELAUNCH;
+}
+
+int kge_timeline_mark(kge_timeline *tl, const char *label, void *stream)
+{
+    if (!tl || !label) return KGE_EINVAL;
+    if (tl->count >= tl->capacity) return KGE_EWORKSPACE;
+    const int before = tl->count;
+    timeline_mark(tl, as_stream(stream), label);
+    return tl->count == before + 1 ? KGE_OK : KGE_ELAUNCH;
+}
+
+int kge_timeline_elapsed(const kge_timeline *tl, float *ms)
+{
+    if (!tl || !ms || !tl->begin) return KGE_EINVAL;
+    hipEvent_t prev = reinterpret_cast<hipEvent_t>(tl->begin);
+    for (int i = 0; i < tl->count; ++i) {
+        hipEvent_t cur = reinterpret_cast<hipEvent_t>(tl->events[i]);
+        if (hipEventElapsedTime(&ms[i], prev, cur) != hipSuccess) return KGE_ELAUNCH;
+        prev = cur;
+    }
+    return tl->count;
 }
 
 size_t kge_score_fwd_workspace(const kge_tables *tab, const kge_batch *bat)
@@ -135,6 +181,7 @@ int kge_residual_fwd(const kge_tables *tab, const kge_batch *bat, float *out, vo
     if (!out && bat->batch > 0) return KGE_EINVAL;
     if (tab->model != KGE_TRANSE && tab->model != KGE_TRANSH && tab->model != KGE_TRANSR)
         return KGE_EUNSUPPORTED;  // the other models have scalar outputs only
+    KGE_CLEAR_LAUNCH_ERRORS();
     if (tab->model == KGE_TRANSR && bat->rel_insp)
         return launch_transr_fwd(tab, bat, nullptr, out, workspace, workspace_bytes, as_stream(stream));
     return launch_score_pos(tab, bat, nullptr, out, nullptr, as_stream(stream));
@@ -148,6 +195,7 @@ int kge_score_fwd(const kge_tables *tab, const kge_batch *bat, float *pos, float
     if (rc) return rc;
     if ((rc = validate_batch(bat))) return rc;
     hipStream_t st = as_stream(stream);
+    KGE_CLEAR_LAUNCH_ERRORS();
     const bool want_neg = neg && bat->neg;
     if (want_neg && tab->model == KGE_TRANSH && !side_pos) return KGE_EINVAL;
     if (want_neg && tab->model == KGE_ROTATE && !residual) return KGE_EINVAL;  // rotated heads buffer
@@ -164,13 +212,18 @@ int kge_score_fwd(const kge_tables *tab, const kge_batch *bat, float *pos, float
     if (pos || side_pos || residual) {
         if ((tab->model == KGE_TRANSR || tab->model == KGE_RESCAL) && bat->rel_insp)
             rc = launch_transr_fwd(tab, bat, pos, residual, workspace, workspace_bytes, st);
-        else
+        else {
             rc = launch_score_pos_fused(tab, bat, pos, residual, side_pos, fuse ? &fi0 : nullptr, st);
+            timeline_mark(bat->timeline, st, "score_pos_kernel");
+        }
         if (rc) return rc;
     }
-    if (want_neg)
-        return launch_score_neg(tab, bat, side_pos, tab->model == KGE_ROTATE ? residual : nullptr, neg, side_neg,
-                                fuse ? &fi1 : nullptr, st);
+    if (want_neg) {
+        rc = launch_score_neg(tab, bat, side_pos, tab->model == KGE_ROTATE ? residual : nullptr, neg, side_neg,
+                              fuse ? &fi1 : nullptr, st);
+        timeline_mark(bat->timeline, st, "score_neg_kernel");
+        return rc;
+    }
     return KGE_OK;
 }
 

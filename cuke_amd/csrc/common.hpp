@@ -10,6 +10,10 @@ namespace kge {
 
 constexpr int kWave = 64;
 
+// Launch errors are sticky per host thread: an entry point clears whatever another library left
+// behind (KGE_CLEAR_LAUNCH_ERRORS) before its first launch, so that KGE_CHECK_LAUNCH reports only
+// this library's own launches.
+#define KGE_CLEAR_LAUNCH_ERRORS() ((void)hipGetLastError())
 #define KGE_CHECK_LAUNCH()                                   \
     do {                                                     \
         if (hipGetLastError() != hipSuccess) return KGE_ELAUNCH; \
@@ -61,9 +65,16 @@ inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 
 
 inline hipStream_t as_stream(void *s) { return reinterpret_cast<hipStream_t>(s); }
 
-// DistMult / ComplEx pair sums: 0 = matrix cores (default), 1 = vector ALUs.  Starts from the
-// environment variable KGE_DOT_VALU; kge_set_pair_sum_unit() changes it at run time (api.hip).
-int dot_valu_option();
+// DistMult / ComplEx pair sums on the vector ALUs instead of the matrix cores (kge_tables.flags)
+inline bool pair_sums_valu(const kge_tables *tab) { return (tab->flags & KGE_PAIR_SUMS_VALU) != 0; }
+
+// One entry of the caller's timeline (kge_batch.timeline): the kernel launched last ends here.
+inline void timeline_mark(kge_timeline *tl, hipStream_t st, const char *label)
+{
+    if (!tl || !tl->events || !tl->labels || tl->count < 0 || tl->count >= tl->capacity) return;
+    if (hipEventRecord(reinterpret_cast<hipEvent_t>(tl->events[tl->count]), st) != hipSuccess) return;
+    tl->labels[tl->count++] = label;
+}
 
 // floats per relation / auxiliary row for a model with entity width d
 inline int64_t rel_width(int model, int64_t d)

@@ -11,8 +11,6 @@
 //      the positive triple's own term; writes the h / t / r (/ w) occurrence rows
 //   4. seg_reduce: occurrence rows are summed per distinct id in sorted order
 //      (inspection perm / seg_offsets); every output row is written exactly once.
-#include <stdlib.h>
-
 #include <type_traits>
 
 #include "inspector_mid.hpp"
@@ -458,39 +456,28 @@ static size_t tile_lds_bytes(const FusedInsp &fi)
     return fi.blocks > 0 && (size_t)fi.lds_bytes > own ? (size_t)fi.lds_bytes : own;
 }
 
-static int dot_valu_override() { return dot_valu_option(); }
-
 template <int MODEL, int P>
-static int launch_tiles(TileArgs a, float *g0, float *g1, float *occ_neg, int64_t n_chunks, const FusedInsp &fi,
-                        hipStream_t st)
+static int launch_tiles(TileArgs a, float *g0, float *g1, float *occ_neg, int64_t n_chunks, bool dot_valu,
+                        const FusedInsp &fi, hipStream_t st)
 {
     const int klen = MODEL == KGE_ROTATE ? a.d / 2 : a.d;
     const int64_t gx = ceil_div(klen, kTI);
     const int64_t big = gx * (ceil_div(a.C, 64) + ceil_div(a.N, 64)) * n_chunks;
-    static const int knob = [] { const char *e = getenv("KGE_BWD_TILE"); return e ? atoi(e) : 0; }();
-    // KGE_BWD_TILE is a development knob; the size rule follows launch_neg_mp (see there)
+    // the size rule follows launch_neg_mp (see there)
     constexpr bool kDotModel = MODEL == KGE_DISTMULT || MODEL == KGE_COMPLEX;
     if constexpr (kDotModel) {
-        // matrix-core inner loop (KGE_DOT_VALU=1 keeps the vector-ALU loop): a wave gets all 64
-        // columns of its 16 owners with 64-owner tiles and half of them with 32-owner tiles, and the
-        // large tile wins at every size
-        if (!dot_valu_override()) {
-            if (knob == 2) {
-                const unsigned gh = xcd_grid(gx, ceil_div(a.C, 32), n_chunks), gn = xcd_grid(gx, ceil_div(a.N, 32), n_chunks);
-                const size_t lds = tile_lds_bytes<MODEL, 2>(fi);
-                hipLaunchKernelGGL((bwd_tile_kernel<MODEL, P, 2, true>), dim3(gh + gn + fi.blocks), dim3(256), lds, st, a,
-                                   g0, g1, occ_neg, (int)gh, fi);
-            } else {
-                const unsigned gh = xcd_grid(gx, ceil_div(a.C, 64), n_chunks), gn = xcd_grid(gx, ceil_div(a.N, 64), n_chunks);
-                const size_t lds = tile_lds_bytes<MODEL, 4>(fi);
-                hipLaunchKernelGGL((bwd_tile_kernel<MODEL, P, 4, true>), dim3(gh + gn + fi.blocks), dim3(256), lds, st, a,
-                                   g0, g1, occ_neg, (int)gh, fi);
-            }
+        // matrix-core inner loop (KGE_PAIR_SUMS_VALU keeps the vector-ALU loop): a wave gets all 64
+        // columns of its 16 owners with 64-owner tiles, which win at every size
+        if (!dot_valu) {
+            const unsigned gh = xcd_grid(gx, ceil_div(a.C, 64), n_chunks), gn = xcd_grid(gx, ceil_div(a.N, 64), n_chunks);
+            const size_t lds = tile_lds_bytes<MODEL, 4>(fi);
+            hipLaunchKernelGGL((bwd_tile_kernel<MODEL, P, 4, true>), dim3(gh + gn + fi.blocks), dim3(256), lds, st, a,
+                               g0, g1, occ_neg, (int)gh, fi);
             KGE_CHECK_LAUNCH();
             return KGE_OK;
         }
     }
-    if (knob == 4 || (knob != 2 && big >= 1024)) {
+    if (big >= 1024) {
         const unsigned gh = xcd_grid(gx, ceil_div(a.C, 64), n_chunks), gn = xcd_grid(gx, ceil_div(a.N, 64), n_chunks);
         const size_t lds = tile_lds_bytes<MODEL, 4>(fi);
         hipLaunchKernelGGL((bwd_tile_kernel<MODEL, P, 4, false>), dim3(gh + gn + fi.blocks), dim3(256), lds, st, a, g0, g1,
@@ -816,6 +803,7 @@ int kge_score_bwd(const kge_tables *tab, const kge_batch *bat, const kge_saved *
     if (!bat->h || !bat->r || !bat->t || !bat->ent_insp || !bat->rel_insp || !grads->ent_rows) return KGE_EINVAL;
     if (bat->neg && (bat->chunk <= 0 || bat->n_neg <= 0 || bat->batch % bat->chunk)) return KGE_ESHAPE;
     hipStream_t st = as_stream(stream);
+    KGE_CLEAR_LAUNCH_ERRORS();
     if (tab->model == KGE_TRANSR || tab->model == KGE_RESCAL)
         return launch_transr_bwd(tab, bat, saved, dpos, grads, workspace, workspace_bytes, st);
 
@@ -867,20 +855,22 @@ int kge_score_bwd(const kge_tables *tab, const kge_batch *bat, const kge_saved *
                    B * bat->n_neg, (int)bat->chunk, (int)bat->n_neg, (int)d, (int)tab->rel_dim, vec ? 1 : 0,
                    vecn ? 1 : 0, (int)n_chunks, head ? -1.0f : 1.0f};
         float *occ_neg = occ_e + 2 * B * d;
+        const bool dv = pair_sums_valu(tab);
         switch (model) {
         case KGE_TRANSE:
-            rc = P == 1 ? launch_tiles<KGE_TRANSE, 1>(a, g0, g1, occ_neg, n_chunks, fi_pass, st)
-                        : launch_tiles<KGE_TRANSE, 2>(a, g0, g1, occ_neg, n_chunks, fi_pass, st);
+            rc = P == 1 ? launch_tiles<KGE_TRANSE, 1>(a, g0, g1, occ_neg, n_chunks, dv, fi_pass, st)
+                        : launch_tiles<KGE_TRANSE, 2>(a, g0, g1, occ_neg, n_chunks, dv, fi_pass, st);
             break;
         case KGE_TRANSH:
-            rc = P == 1 ? launch_tiles<KGE_TRANSH, 1>(a, g0, g1, occ_neg, n_chunks, fi_pass, st)
-                        : launch_tiles<KGE_TRANSH, 2>(a, g0, g1, occ_neg, n_chunks, fi_pass, st);
+            rc = P == 1 ? launch_tiles<KGE_TRANSH, 1>(a, g0, g1, occ_neg, n_chunks, dv, fi_pass, st)
+                        : launch_tiles<KGE_TRANSH, 2>(a, g0, g1, occ_neg, n_chunks, dv, fi_pass, st);
             break;
-        case KGE_DISTMULT: rc = launch_tiles<KGE_DISTMULT, 2>(a, g0, g1, occ_neg, n_chunks, fi_pass, st); break;
-        case KGE_COMPLEX: rc = launch_tiles<KGE_COMPLEX, 2>(a, g0, g1, occ_neg, n_chunks, fi_pass, st); break;
-        case KGE_ROTATE: rc = launch_tiles<KGE_ROTATE, 2>(a, g0, g1, occ_neg, n_chunks, fi_pass, st); break;
+        case KGE_DISTMULT: rc = launch_tiles<KGE_DISTMULT, 2>(a, g0, g1, occ_neg, n_chunks, dv, fi_pass, st); break;
+        case KGE_COMPLEX: rc = launch_tiles<KGE_COMPLEX, 2>(a, g0, g1, occ_neg, n_chunks, dv, fi_pass, st); break;
+        case KGE_ROTATE: rc = launch_tiles<KGE_ROTATE, 2>(a, g0, g1, occ_neg, n_chunks, dv, fi_pass, st); break;
         default: return KGE_EUNSUPPORTED;
         }
+        timeline_mark(bat->timeline, st, "bwd_tile_kernel");
         if (rc) return rc;
     } else if (p.nn > 0) {
         hipLaunchKernelGGL(fill_zero_kernel, dim3(1024), dim3(256), 0, st, occ_e + 2 * B * d, p.nn * d);
@@ -901,6 +891,7 @@ int kge_score_bwd(const kge_tables *tab, const kge_batch *bat, const kge_saved *
     case KGE_TRANSF: rc = launch_pos_bwd<KGE_TRANSF, 2>(pa, vec, head, fi_dedup, st); break;
     default: return KGE_EUNSUPPORTED;
     }
+    timeline_mark(bat->timeline, st, "bwd_pos_kernel");
     if (rc) return rc;
 
     if (bat->insp_ready && hipStreamWaitEvent(st, reinterpret_cast<hipEvent_t>(bat->insp_ready), 0) != hipSuccess)
@@ -909,7 +900,7 @@ int kge_score_bwd(const kge_tables *tab, const kge_batch *bat, const kge_saved *
         {occ_e, bat->ent_insp, (int)d, grads->ent_rows, reinterpret_cast<float *>(ws + p.off_part_e), false},
         {occ_r, bat->rel_insp, (int)tab->rel_dim, grads->rel_rows, reinterpret_cast<float *>(ws + p.off_part_r), false},
         {occ_w, bat->rel_insp, (int)d, grads->aux_rows, reinterpret_cast<float *>(ws + p.off_part_w), false}};
-    return launch_seg_reduce_jobs(jobs, model == KGE_TRANSH ? 3 : 2, st);
+    return launch_seg_reduce_jobs(jobs, model == KGE_TRANSH ? 3 : 2, st, bat->timeline);
 }
 
 }  // extern "C"

@@ -6,10 +6,10 @@
 // "query" rows a_b = f(h_b, r_b) are formed while staging (the gathers of h and r
 // are fused into the staging loads) and the negative rows are gathered straight
 // into LDS, KD floats of the row at a time; each thread then accumulates an
-// RB x RK block of pair scores from LDS with 128-bit reads.  All arithmetic is
-// fp32 VALU; no matrix cores.
-#include <stdlib.h>
-
+// RB x RK block of pair scores from LDS with 128-bit reads (score_neg_kernel, fp32 vector
+// ALUs).  Where the pair scores are plain dot products (DistMult, ComplEx, and the w . t'
+// sweep of TransH) the tile is a matrix product and runs on the matrix cores
+// (score_neg_mfma_kernel, fp32 MFMA with fp32 accumulation).
 #include <type_traits>
 
 #include "inspector_mid.hpp"
@@ -430,18 +430,6 @@ __global__ __launch_bounds__(256, KGE_TILE_OCC) void score_neg_mfma_kernel(NegAr
         }
 }
 
-// 0: choose by size, 2: 32x32 tiles, 3: 32x64, 4: 64x64 (development knob)
-static int neg_tile_override()
-{
-    static const int v = [] {
-        const char *e = getenv("KGE_NEG_TILE");
-        return e ? atoi(e) : 0;
-    }();
-    return v;
-}
-
-static int neg_valu_override() { return dot_valu_option(); }
-
 // LDS bytes of a launch: the tile's staging buffers, or what the inspector workgroups need if more
 static size_t neg_lds(int planes, int TB, int TN, int planes_t, const FusedInsp &fi)
 {
@@ -450,21 +438,20 @@ static size_t neg_lds(int planes, int TB, int TN, int planes_t, const FusedInsp 
 }
 
 template <int MODEL, int P>
-static int launch_neg_mp(const NegArgs &a, int64_t n_chunks, const FusedInsp &fi, hipStream_t st)
+static int launch_neg_mp(const NegArgs &a, int64_t n_chunks, bool dot_valu, const FusedInsp &fi, hipStream_t st)
 {
     constexpr int NPA = (MODEL == KGE_ROTATE || MODEL == KGE_TRANSH) ? 2 : 1, NPT = MODEL == KGE_ROTATE ? 2 : 1;
     const int64_t big_tiles = ceil_div(a.C, 64) * ceil_div(a.N, 64) * n_chunks;
-    int tile = neg_tile_override();
     // Small tiles up to about 1024 big tiles: more waves to hide latency (32x32 is ~20 % faster than
     // 64x64 on a 256-big-tile workload with the vector-ALU loop; the matrix-core loop, whose
     // launches are bound by the rows its workgroups pull from L2, does best with 32x64).  The
     // inspector workgroups that share the machine with these launches raise their wave priority.
     constexpr bool kDotModel = MODEL == KGE_DISTMULT || MODEL == KGE_COMPLEX;
-    if (tile != 2 && tile != 4 && tile != 3) tile = big_tiles >= 1024 ? 4 : (kDotModel && !neg_valu_override() ? 3 : 2);
+    const int tile = big_tiles >= 1024 ? 4 : (kDotModel && !dot_valu ? 3 : 2);  // 2: 32x32, 3: 32x64, 4: 64x64
     const int TB = tile == 4 ? 64 : 32, TN = tile == 2 ? 32 : 64;
     const dim3 grid(xcd_grid(ceil_div(a.N, TN), ceil_div(a.C, TB), n_chunks) + (unsigned)fi.blocks);
     if constexpr (MODEL == KGE_DISTMULT || MODEL == KGE_COMPLEX) {
-        if (!neg_valu_override()) {
+        if (!dot_valu) {
             const size_t lds = neg_lds(1, TB, TN, 1, fi);
             if (tile == 4) hipLaunchKernelGGL((score_neg_mfma_kernel<MODEL, 4, 4>), grid, dim3(256), lds, st, a, fi);
             else if (tile == 3) hipLaunchKernelGGL((score_neg_mfma_kernel<MODEL, 2, 4>), grid, dim3(256), lds, st, a, fi);
@@ -502,16 +489,17 @@ int launch_score_neg(const kge_tables *tab, const kge_batch *bat, const float *s
               bat->batch * bat->n_neg, (int)bat->chunk, (int)bat->n_neg, (int)tab->dim, (int)tab->rel_dim, tab->gamma,
               vec ? 1 : 0, (int)n_chunks, head ? -1.0f : 1.0f};
     const int p = tab->norm_p;
+    const bool dv = pair_sums_valu(tab);
     switch (tab->model) {
     case KGE_TRANSE:
-        return p == 1 ? launch_neg_mp<KGE_TRANSE, 1>(a, n_chunks, fi, st)
-                      : launch_neg_mp<KGE_TRANSE, 2>(a, n_chunks, fi, st);
+        return p == 1 ? launch_neg_mp<KGE_TRANSE, 1>(a, n_chunks, dv, fi, st)
+                      : launch_neg_mp<KGE_TRANSE, 2>(a, n_chunks, dv, fi, st);
     case KGE_TRANSH:
-        return p == 1 ? launch_neg_mp<KGE_TRANSH, 1>(a, n_chunks, fi, st)
-                      : launch_neg_mp<KGE_TRANSH, 2>(a, n_chunks, fi, st);
-    case KGE_DISTMULT: return launch_neg_mp<KGE_DISTMULT, 2>(a, n_chunks, fi, st);
-    case KGE_COMPLEX: return launch_neg_mp<KGE_COMPLEX, 2>(a, n_chunks, fi, st);
-    case KGE_ROTATE: return launch_neg_mp<KGE_ROTATE, 2>(a, n_chunks, fi, st);
+        return p == 1 ? launch_neg_mp<KGE_TRANSH, 1>(a, n_chunks, dv, fi, st)
+                      : launch_neg_mp<KGE_TRANSH, 2>(a, n_chunks, dv, fi, st);
+    case KGE_DISTMULT: return launch_neg_mp<KGE_DISTMULT, 2>(a, n_chunks, dv, fi, st);
+    case KGE_COMPLEX: return launch_neg_mp<KGE_COMPLEX, 2>(a, n_chunks, dv, fi, st);
+    case KGE_ROTATE: return launch_neg_mp<KGE_ROTATE, 2>(a, n_chunks, dv, fi, st);
     default: return KGE_EUNSUPPORTED;  // TransR / TransF / RESCAL: positives only
     }
 }

@@ -147,7 +147,7 @@ __global__ __launch_bounds__(256) void seg_reduce_l2(SegArgs3 jobs)
     }
 }
 
-int launch_seg_reduce_jobs(const SegJob *jobs, int n_jobs, hipStream_t st)
+int launch_seg_reduce_jobs(const SegJob *jobs, int n_jobs, hipStream_t st, kge_timeline *timeline)
 {
     SegArgs3 args{};
     int m = 0;
@@ -173,11 +173,14 @@ int launch_seg_reduce_jobs(const SegJob *jobs, int n_jobs, hipStream_t st)
     const dim3 g1((unsigned)ceil_div(max_waves, 4), (unsigned)m), g2((unsigned)max_blocks, (unsigned)m), block(256);
     if (v4) {
         hipLaunchKernelGGL(seg_reduce_l1<4>, g1, block, 0, st, args);
+        timeline_mark(timeline, st, "seg_reduce_l1");
         hipLaunchKernelGGL(seg_reduce_l2<4>, g2, block, 0, st, args);
     } else {
         hipLaunchKernelGGL(seg_reduce_l1<1>, g1, block, 0, st, args);
+        timeline_mark(timeline, st, "seg_reduce_l1");
         hipLaunchKernelGGL(seg_reduce_l2<1>, g2, block, 0, st, args);
     }
+    timeline_mark(timeline, st, "seg_reduce_l2");
     KGE_CHECK_LAUNCH();
     return KGE_OK;
 }

@@ -19,6 +19,6 @@ struct SegJob {
 inline int64_t seg_partial_floats(int64_t n, int64_t d) { return ceil_div(n > 0 ? n : 1, kSegL) * 2 * d; }
 
 // Up to three jobs share the same two launches.
-int launch_seg_reduce_jobs(const SegJob *jobs, int n_jobs, hipStream_t st);
+int launch_seg_reduce_jobs(const SegJob *jobs, int n_jobs, hipStream_t st, kge_timeline *timeline = nullptr);
 
 }  // namespace kge

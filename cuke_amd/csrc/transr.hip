@@ -964,7 +964,11 @@ int launch_transr_fwd(const kge_tables *tab, const kge_batch *bat, float *pos, f
         const int rc = plan_fused_inspection(bat->insp_jobs, 1, 0, &fi);
         if (rc) return rc;
     }
-    if (!grouped) return launch_score_pos(tab, bat, pos, resid, nullptr, st);
+    if (!grouped) {
+        const int rc = launch_score_pos(tab, bat, pos, resid, nullptr, st);
+        timeline_mark(bat->timeline, st, "score_pos_kernel");
+        return rc;
+    }
     const kge_inspection *ri = bat->rel_insp;
     const int64_t tiles = max_tiles(tab, bat);
     TilePlan plan = plan_at(workspace, tiles, 0);
@@ -980,6 +984,7 @@ int launch_transr_fwd(const kge_tables *tab, const kge_batch *bat, float *pos, f
         hipLaunchKernelGGL(transr_gemm_kernel<1>, grid, dim3(256), lds, st, a, fi);
     else
         hipLaunchKernelGGL(transr_gemm_kernel<0>, grid, dim3(256), lds, st, a, fi);
+    timeline_mark(bat->timeline, st, "transr_plan_kernel + transr_gemm_kernel<fwd>");
     KGE_CHECK_LAUNCH();
     return KGE_OK;
 }
@@ -1023,6 +1028,7 @@ int launch_transr_bwd(const kge_tables *tab, const kge_batch *bat, const kge_sav
     }
     hipLaunchKernelGGL(transr_prep_kernel, dim3((unsigned)(ceil_div(B, 4) + f1.blocks)), dim3(256), lds_with(f1, 0), st, pa,
                        f1);
+    timeline_mark(bat->timeline, st, "transr_prep_kernel");
     if (!have_plans)
         hipLaunchKernelGGL(transr_plan_kernel, dim3(2), dim3(1024), 0, st, ri->num_unique, ri->seg_offsets, plan, kTM,
                            dplan, kDmChunk);
@@ -1031,14 +1037,17 @@ int launch_transr_bwd(const kge_tables *tab, const kge_batch *bat, const kge_sav
                 plan, qs, nullptr, nullptr, occ, rescal ? nullptr : occ + B * d, d, tab->norm_p, thin_groups(tab, bat), (int)p.tiles};
     hipLaunchKernelGGL(transr_gemm_kernel<2>, dim3((unsigned)(p.tiles + ga.thin_groups + f2.blocks)), dim3(256),
                        lds_with(f2, gemm_lds_bytes(d)), st, ga, f2);
+    timeline_mark(bat->timeline, st, "transr_gemm_kernel<dX>");
     // dM = X^T Q per relation group
     const int dm_items = (int)(ceil_div(d, 32) * p.dtiles);
     DmArgs da{xs, qs, ri->seg_offsets, dplan, grads->aux_rows, reinterpret_cast<float *>(ws + p.off_dpart), d,
               ri->num_unique, dm_items};
     hipLaunchKernelGGL(transr_dm_kernel, dim3((unsigned)(dm_items + thin_groups(tab, bat) + f3.blocks)), dim3(256),
                        lds_with(f3, sizeof(float) * 4 * (size_t)d), st, da, f3);
+    timeline_mark(bat->timeline, st, "transr_dm_kernel");
     hipLaunchKernelGGL(transr_dm_finish_kernel, dim3((unsigned)ceil_div((int64_t)d * d / 4, 256), (unsigned)p.dsplit),
                        dim3(256), 0, st, da);
+    timeline_mark(bat->timeline, st, "transr_dm_finish_kernel");
     KGE_CHECK_LAUNCH();
     if (bat->insp_ready && hipStreamWaitEvent(st, reinterpret_cast<hipEvent_t>(bat->insp_ready), 0) != hipSuccess)
         return KGE_ELAUNCH;
@@ -1047,7 +1056,7 @@ int launch_transr_bwd(const kge_tables *tab, const kge_batch *bat, const kge_sav
     const SegJob jobs[2] = {
         {occ, bat->ent_insp, d, grads->ent_rows, reinterpret_cast<float *>(ws + p.off_part_e), false},
         {qs, ri, d, grads->rel_rows, reinterpret_cast<float *>(ws + p.off_part_r), true}};
-    return launch_seg_reduce_jobs(jobs, rescal ? 1 : 2, st);
+    return launch_seg_reduce_jobs(jobs, rescal ? 1 : 2, st, bat->timeline);
 }
 
 }  // namespace kge

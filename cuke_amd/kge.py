@@ -150,9 +150,12 @@ class KGEModel:
     Remb   [n_rel, dim] float32 (RotatE: [n_rel, dim/2] phases; RESCAL: None)
     aux    TransH: hyperplane normals [n_rel, dim] (the reference's Pemb);
            TransR / RESCAL: projections [n_rel, dim, dim] (the reference's Proj)
+    pair_sums  "matrix_cores" (default) or "vector_alus": where the shared-negative tile kernels of
+           DistMult / ComplEx sum their pair products (``pair_sums`` can be reassigned between calls)
     """
 
-    def __init__(self, model: str, Eemb, Remb=None, aux=None, norm_p: int = 2, gamma: float = 0.0):
+    def __init__(self, model: str, Eemb, Remb=None, aux=None, norm_p: int = 2, gamma: float = 0.0,
+                 pair_sums: str = "matrix_cores"):
         if model not in MODELS:
             raise ValueError(f"unknown model {model!r}; expected one of {sorted(MODELS)}")
         self.model = model
@@ -177,10 +180,23 @@ class KGEModel:
             if tuple(self.A.shape) != want:
                 raise ValueError(f"aux has shape {tuple(self.A.shape)}, {model} needs {want}")
         self.norm_p, self.gamma = int(norm_p), float(gamma)
-        self._tab = _lib.Tables(MODELS[model], self.norm_p, self.gamma, 0, self.dim, self.rel_dim,
+        if pair_sums not in ("matrix_cores", "vector_alus"):
+            raise ValueError("pair_sums is 'matrix_cores' or 'vector_alus'")
+        self._tab = _lib.Tables(MODELS[model], self.norm_p, self.gamma,
+                                _lib.PAIR_SUMS_VALU if pair_sums == "vector_alus" else 0, self.dim, self.rel_dim,
                                 int(self.E.shape[0]), self.n_rel, self.E.data_ptr(),
                                 self.R.data_ptr() if (self.R is not None and self.rel_dim) else None,
                                 self.A.data_ptr() if self.A is not None else None)
+
+    @property
+    def pair_sums(self) -> str:
+        return "vector_alus" if self._tab.flags & _lib.PAIR_SUMS_VALU else "matrix_cores"
+
+    @pair_sums.setter
+    def pair_sums(self, unit: str) -> None:
+        if unit not in ("matrix_cores", "vector_alus"):
+            raise ValueError("pair_sums is 'matrix_cores' or 'vector_alus'")
+        self._tab.flags = _lib.PAIR_SUMS_VALU if unit == "vector_alus" else 0
 
     # -- helpers ---------------------------------------------------------------------------
     def _batch(self, h, r, t, neg=None, chunk=None, ent_insp=None, rel_insp=None, neg_mode="tail"):
@@ -328,9 +344,17 @@ def margin_loss(pos: torch.Tensor, neg: torch.Tensor, margin: float, sign: float
     return loss, dpos, dneg
 
 
+def _inplace_table(table):
+    """A table that is updated in place must be the caller's own memory, not a contiguous copy of it."""
+    t = _table(table, "table", table.dim())
+    if t.data_ptr() != table.data_ptr() or not table.is_contiguous():
+        raise ValueError("table must be contiguous: it is updated in place")
+    return t
+
+
 def sparse_sgd(table: torch.Tensor, insp: Inspection, rows: torch.Tensor, lr: float) -> None:
     """table[id] -= lr * rows[u] for the inspection's unique ids (in place, no host sync)."""
-    t = _table(table, "table", table.dim())
+    t = _inplace_table(table)
     _lib.check(_lib.lib().kge_sparse_sgd(_ptr(t), int(rows.shape[1]), _ptr(insp.unique_ids), _ptr(insp.num_unique_dev),
                                          int(rows.shape[0]), _ptr(rows), float(lr), _stream()), "kge_sparse_sgd")
 
@@ -338,7 +362,9 @@ def sparse_sgd(table: torch.Tensor, insp: Inspection, rows: torch.Tensor, lr: fl
 def sparse_adagrad(table: torch.Tensor, state: torch.Tensor, insp: Inspection, rows: torch.Tensor, lr: float,
                    eps: float = 1e-10) -> None:
     """Row-wise Adagrad: state[id] += mean(g^2); table[id] -= lr * g / (sqrt(state[id]) + eps)."""
-    t = _table(table, "table", table.dim())
+    t = _inplace_table(table)
+    if not state.is_contiguous():
+        raise ValueError("state must be contiguous: it is updated in place")
     _lib.check(_lib.lib().kge_sparse_adagrad(_ptr(t), _ptr(state), int(rows.shape[1]), _ptr(insp.unique_ids),
                                              _ptr(insp.num_unique_dev), int(rows.shape[0]), _ptr(rows), float(lr),
                                              float(eps), _stream()), "kge_sparse_adagrad")
@@ -445,6 +471,8 @@ class TrainStep:
         self._sets = [self._make_set(idx0)]
         self._cur = 0
         self._staged, self._stage_at = collections.deque(), 0
+        self._pipelined = False   # the ring of run(pipeline=True) has been set up
+        self._timeline = None     # set by kernel_times()
         self.side = torch.cuda.Stream(device=dev)  # default priority
         self.pos = torch.empty(B, **f32)
         self.neg = torch.empty((B, N), **f32) if neg is not None else None
@@ -516,6 +544,77 @@ class TrainStep:
         s.inputs_ready = None
         return s
 
+    def add_batch(self, h, r, t, neg=None) -> int:
+        """Another batch of the same shape, with index tensors and inspections of its own (scores, gradients
+        and workspaces are shared).  Returns its number for ``select()``; the batch given to the
+        constructor is number 0."""
+        if self._staged or self._pipelined:
+            raise KgeError("add_batch() cannot be mixed with the staged pipeline")
+        _, (h, r, t, neg, C_, N) = self.m._batch(h, r, t, neg, self.C or None, neg_mode=self._neg_mode)
+        if int(h.numel()) != self.B or N != self.N or (neg is None) != (self.neg is None):
+            raise ValueError("every batch of a TrainStep has the shape of the first one")
+        self._sets.append(self._make_set((h, r, t, neg)))
+        return len(self._sets) - 1
+
+    def select(self, i: int) -> None:
+        """Make batch ``i`` (see ``add_batch``) the one the next ``run()`` processes."""
+        if self._staged or self._pipelined:
+            raise KgeError("select() cannot be mixed with the staged pipeline")
+        if not 0 <= i < len(self._sets):
+            raise IndexError(i)
+        self._cur = i
+
+    # -- per-kernel timing ----------------------------------------------------------------------------
+    _LABELS = {k: k.encode() for k in ("inspect", "inspect(relations)", "margin_loss")}
+
+    def _mark(self, label: str, st) -> None:
+        if self._timeline is not None:
+            _lib.check(self.L.kge_timeline_mark(self._timeline, self._LABELS[label], st), "kge_timeline_mark")
+
+    def kernel_times(self, steps: int = 10, backward: bool = True, batches=None, lead=None):
+        """[(kernel name, mean milliseconds)] of one step, in launch order: ``steps`` steps are run with an
+        event recorded behind every kernel (kge_batch.timeline) and read back after each step.  Event
+        records between the kernels cost a little themselves, so the sum is an upper bound of the
+        step time that ``run()`` alone takes.  ``batches``: batch numbers to rotate over.  ``lead``: a
+        large tensor that is zero-filled on the stream in front of every step, so that the host has
+        enqueued the whole step before the device starts on it and the intervals hold no launch gaps."""
+        L = self.L
+        tl = L.kge_timeline_create(64)
+        if not tl:
+            raise KgeError("kge_timeline_create failed")
+        main = torch.cuda.current_stream()
+        st = C.c_void_p(main.cuda_stream)
+        sums, names = None, None
+        ms = (C.c_float * 64)()
+        self._timeline = tl
+        try:
+            for i in range(steps):
+                if batches:
+                    self.select(batches[i % len(batches)])
+                self.bat.timeline = tl
+                if lead is not None:
+                    lead.zero_()
+                _lib.check(L.kge_timeline_begin(tl, st), "kge_timeline_begin")
+                try:
+                    self.run(backward, overlap=False)
+                finally:
+                    self.bat.timeline = None
+                main.synchronize()
+                n = L.kge_timeline_elapsed(tl, ms)
+                if n < 0:
+                    _lib.check(n, "kge_timeline_elapsed")
+                cur = [tl.contents.labels[k].decode() for k in range(n)]
+                if names is None:
+                    names, sums = cur, [0.0] * n
+                elif cur != names:
+                    raise KgeError(f"the kernel sequence changed between steps: {names} vs {cur}")
+                for k in range(n):
+                    sums[k] += ms[k]
+        finally:
+            self._timeline = None
+            L.kge_timeline_destroy(tl)
+        return [(nm, s / steps) for nm, s in zip(names or [], sums or [])]
+
     # the set of the step enqueued last (the only set unless run(pipeline=True) is used)
     idx = property(lambda self: self._sets[self._cur].idx)
     ent_insp = property(lambda self: self._sets[self._cur].ent_insp)
@@ -542,6 +641,7 @@ class TrainStep:
             _lib.check(self.L.kge_margin_loss(_ptr(self.pos), _ptr(self.neg), self.B, self.N, self.margin,
                                               self.sign, _ptr(self.loss), _ptr(self.dpos), _ptr(self.dneg),
                                               _ptr(self._ws_l), self._ws_l.numel(), st), "kge_margin_loss")
+            self._mark("margin_loss", st)
 
     def backward(self, st):
         _lib.check(self.L.kge_score_bwd(C.byref(self.m._tab), C.byref(self.bat), C.byref(self.saved),
@@ -551,6 +651,7 @@ class TrainStep:
     # ---- pipelined issue: index tensors and inspections in a ring of sets ----
     def _ring(self):
         """Grow to kPipelineSets sets on first use (copies of the construction-time indices)."""
+        self._pipelined = True
         if len(self._sets) < self.kPipelineSets:
             first = self._sets[0].idx
             while len(self._sets) < self.kPipelineSets:
@@ -620,6 +721,8 @@ class TrainStep:
         capturable into one graph: the dependencies cross steps."""
         main = torch.cuda.current_stream()
         st = C.c_void_p(main.cuda_stream)
+        for s_ in self._sets:  # cached unique counts belong to the batches of earlier steps
+            s_.ent_insp._u = s_.rel_insp._u = None
         if fused is None:
             fused = backward and not pipeline and self.fusable
         if fused:
@@ -631,6 +734,7 @@ class TrainStep:
             try:
                 if self.needs_rel_groups:  # the forward pass is planned from the relation groups
                     _lib.check(self.L.kge_inspect_batch(C.byref(self._jobs[1]), 1, st), "kge_inspect_batch(relations)")
+                    self._mark("inspect(relations)", st)
                 self.forward(st)
                 self.loss_grad(st)
                 self.backward(st)
@@ -641,6 +745,8 @@ class TrainStep:
         if not (backward and overlap):
             self.bat.insp_ready = None
             self.inspect(st, backward)
+            if backward or self.needs_rel_groups:
+                self._mark("inspect", st)
             self.forward(st)
             if backward:
                 self.loss_grad(st)
@@ -696,7 +802,6 @@ class TrainStep:
 
     def sparse_grads(self) -> SparseGrads:
         ue, ur = self.ent_insp.num_unique, self.rel_insp.num_unique
-        self.ent_insp._u = self.rel_insp._u = None  # counts belong to the batch just run
         return SparseGrads(self.ent_insp.unique_ids[:ue], self.ent_rows[:ue], self.rel_insp.unique_ids[:ur],
                            self.rel_rows[:ur] if self.rel_rows is not None else None,
                            self.aux_rows[:ur] if self.aux_rows is not None else None)

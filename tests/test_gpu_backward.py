@@ -11,13 +11,14 @@ pytestmark = pytest.mark.gpu
 NEG_MODELS = ["TransE", "TransH", "DistMult", "ComplEx", "RotatE"]
 
 
-def run_both(oracle, w, seed=0, use_pos=True, use_neg=True):
+def run_both(oracle, w, seed=0, use_pos=True, use_neg=True, pair_sums="matrix_cores"):
     a = w.arrays
     rng = np.random.default_rng(seed)
     dpos = rng.standard_normal(w.batch).astype(np.float32) if use_pos else None
     has_neg = "neg" in a
     dneg = rng.standard_normal((w.batch, w.n_neg)).astype(np.float32) if (has_neg and use_neg) else None
     m, ix = gpu_model(w)
+    m.pair_sums = pair_sums
     fw = m.score(ix["h"], ix["r"], ix["t"], ix.get("neg"), w.chunk or None)
     dev = fw.pos.device
     g = m.backward(fw, None if dpos is None else torch.from_numpy(dpos).to(dev),
@@ -326,17 +327,10 @@ def test_fused_entity_inspection_with_the_grouped_projection_kernels(oracle, mod
 
 @pytest.mark.parametrize("model", ["DistMult", "ComplEx"])
 def test_pair_sums_on_matrix_cores_and_on_vector_alus_agree(oracle, model):
-    """kge_set_pair_sum_unit switches the DistMult / ComplEx tile kernels between the fp32 matrix-core form
-    (default) and the vector-ALU form in one process: both must meet the oracle's tolerance."""
-    from cuke_amd import _lib
+    """kge_tables.flags (KGEModel.pair_sums) switches the DistMult / ComplEx tile kernels between the fp32
+    matrix-core form (default) and the vector-ALU form per call: both must meet the oracle's tolerance."""
     w = synth.custom_workload(model, n_ent=400, n_rel=9, dim=72, batch=320, chunk=160, n_neg=130, sigma=0.2,
                               ent_zipf=1.1, seed=4)
-    L = _lib.lib()
-    was = L.kge_set_pair_sum_unit(0)
-    try:
-        for unit in (0, 1):
-            L.kge_set_pair_sum_unit(unit)
-            g, ref = run_both(oracle, w, seed=3)
-            compare(g, ref, f"{model} pair sums on unit {unit}")
-    finally:
-        L.kge_set_pair_sum_unit(was)
+    for unit in ("matrix_cores", "vector_alus"):
+        g, ref = run_both(oracle, w, seed=3, pair_sums=unit)
+        compare(g, ref, f"{model} pair sums on the {unit}")
