@@ -49,25 +49,6 @@ MEASURED_TRAFFIC_BYTES = {
 }
 
 
-def device_tables(w, dev):
-    """Tables drawn on the GPU (seeded); benchmark-size tables are too large to push through numpy."""
-    import torch
-    g = torch.Generator(device=dev)
-    g.manual_seed(1000 + w.seed)
-    E = torch.randn((w.n_ent, w.dim), generator=g, device=dev, dtype=torch.float32) * w.sigma
-    if w.model == "RotatE":
-        R = (torch.rand((w.n_rel, w.rel_dim), generator=g, device=dev, dtype=torch.float32) * 2 - 1) * np.pi
-    else:
-        R = torch.randn((w.n_rel, w.rel_dim), generator=g, device=dev, dtype=torch.float32) * w.sigma
-    A = None
-    if w.model == "TransH":
-        A = torch.randn((w.n_rel, w.dim), generator=g, device=dev, dtype=torch.float32)
-        A = A / A.norm(dim=1, keepdim=True)
-    elif w.model in ("TransR", "RESCAL"):
-        A = torch.randn((w.n_rel, w.dim, w.dim), generator=g, device=dev, dtype=torch.float32) * w.sigma
-    return E, R, A
-
-
 # ---- algorithmic bytes and flops ---------------------------------------------------------------
 def algorithmic_bytes(w, u_ent, u_rel):
     """Bytes the step has to move by the problem statement alone: every gathered row once per
@@ -436,7 +417,8 @@ def run_workload(name, args, torch):
     from cuke_amd.kge import KGEModel, TrainStep
     dev = torch.device("cuda:0")
     w = make_named_workload(name, args.seed)
-    E, R, A = device_tables(w, dev)
+    from cuke_amd import synth
+    E, R, A = synth.device_tables(w, dev)
     model = KGEModel(w.model, E, R, A, norm_p=w.norm_p, gamma=w.gamma)
     nb = max(1, args.batches)
     sets = [w] + [make_named_workload(name, args.seed + 1 + i) for i in range(nb - 1)]

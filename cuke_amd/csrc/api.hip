@@ -197,7 +197,7 @@ int kge_score_fwd(const kge_tables *tab, const kge_batch *bat, float *pos, float
     hipStream_t st = as_stream(stream);
     KGE_CLEAR_LAUNCH_ERRORS();
     const bool want_neg = neg && bat->neg;
-    if (want_neg && tab->model == KGE_TRANSH && !side_pos) return KGE_EINVAL;
+    if (want_neg && (tab->model == KGE_TRANSH || tab->model == KGE_TRANSF) && !side_pos) return KGE_EINVAL;
     if (want_neg && tab->model == KGE_ROTATE && !residual) return KGE_EINVAL;  // rotated heads buffer
     // fused inspection: first digit pass with the per-positive kernel, second with the tile kernel
     const bool grouped_model = tab->model == KGE_TRANSR || tab->model == KGE_RESCAL;

@@ -506,7 +506,7 @@ int kge_fused_inspection_ok(const kge_tables *tab, const kge_batch *bat, const k
 {
     if (!tab || !bat || !jobs || bat->batch <= 0) return 0;
     switch (tab->model) {
-    case KGE_TRANSE: case KGE_TRANSH: case KGE_DISTMULT: case KGE_COMPLEX: case KGE_ROTATE:
+    case KGE_TRANSE: case KGE_TRANSH: case KGE_DISTMULT: case KGE_COMPLEX: case KGE_ROTATE: case KGE_TRANSF:
         if (!bat->neg) return 0;  // the shared-negative kernels are the hosts
         break;
     case KGE_TRANSR: case KGE_RESCAL:

@@ -59,7 +59,7 @@ __device__ __forceinline__ void bwd_tile_body(const TileArgs &a, int lid, float 
 {
     constexpr int TO = 16 * RO;
     constexpr bool kRot = MODEL == KGE_ROTATE, kTH = MODEL == KGE_TRANSH;
-    constexpr bool kDot = MODEL == KGE_DISTMULT || MODEL == KGE_COMPLEX;
+    constexpr bool kDot = MODEL == KGE_DISTMULT || MODEL == KGE_COMPLEX || MODEL == KGE_TRANSF;  // score = query . t' (+ const)
     constexpr bool kMf = kDot && MF;  // the sum over loopers on the matrix cores (else on the vector ALUs)
     constexpr bool kL2 = (MODEL == KGE_TRANSE || kTH) && P == 2;
     constexpr int NPL = (kRot || (kTH && !OWNER_POS)) ? 2 : 1;  // looper planes in LDS
@@ -464,7 +464,7 @@ static int launch_tiles(TileArgs a, float *g0, float *g1, float *occ_neg, int64_
     const int64_t gx = ceil_div(klen, kTI);
     const int64_t big = gx * (ceil_div(a.C, 64) + ceil_div(a.N, 64)) * n_chunks;
     // the size rule follows launch_neg_mp (see there)
-    constexpr bool kDotModel = MODEL == KGE_DISTMULT || MODEL == KGE_COMPLEX;
+    constexpr bool kDotModel = MODEL == KGE_DISTMULT || MODEL == KGE_COMPLEX || MODEL == KGE_TRANSF;
     if constexpr (kDotModel) {
         // matrix-core inner loop (KGE_PAIR_SUMS_VALU keeps the vector-ALU loop): a wave gets all 64
         // columns of its 16 owners with 64-owner tiles, which win at every size
@@ -500,6 +500,8 @@ struct PosBwdArgs {
     const int64_t *h, *r, *t;
     const float *dpos, *spos, *side_pos;
     const float *g0, *g1;  // [B, d] accumulations over the negatives (may be null)
+    const float *dneg;     // TransF with negatives: [B, N] upstream gradient (its row sums scale the constant's gradient)
+    int64_t N;
     float *occ_h, *occ_t;  // [B, d] each
     float *occ_r;          // [B, rel_dim]
     float *occ_w;          // [B, d] TransH
@@ -588,14 +590,30 @@ __global__ __launch_bounds__(256) void bwd_pos_kernel(PosBwdArgs a, FusedInsp fi
             dh.store(oh + j), dr.store(orr + j), dt.store(ot + j);
         }
     } else if constexpr (MODEL == KGE_TRANSF) {
+        // pair score (2x + rs r).n - rs r.x with x the kept side (h; t with HEAD, rs = -1): G = sum_k dneg n_k
+        // chains with 2 into x and rs into r; the constant's gradient is -rs S r (to x) and -rs S x (to r),
+        // S = sum_k dneg[b][k]
+        float S = 0.0f;
+        if (a.dneg && g0) {  // uniform
+            for (int64_t k = lane; k < a.N; k += kWave) S += a.dneg[b * a.N + k];
+            S = wave_sum(S);
+        }
         for (int j = lane * V; j < d; j += kWave * V) {
             const Vec<V> vh = Vec<V>::load(eh + j), vt = Vec<V>::load(et + j), vr = Vec<V>::load(rr + j);
+            const Vec<V> G = ldz<V>(g0, j);
             Vec<V> dh, dr, dt;
 #pragma unroll
             for (int e = 0; e < V; ++e) {
                 dh.v[e] = g * (2.0f * vt.v[e] - vr.v[e]);
                 dt.v[e] = g * (2.0f * vh.v[e] + vr.v[e]);
                 dr.v[e] = g * (vt.v[e] - vh.v[e]);
+                if constexpr (HEAD) {
+                    dt.v[e] += fmaf(S, vr.v[e], 2.0f * G.v[e]);
+                    dr.v[e] += fmaf(S, vt.v[e], -G.v[e]);
+                } else {
+                    dh.v[e] += fmaf(-S, vr.v[e], 2.0f * G.v[e]);
+                    dr.v[e] += fmaf(-S, vh.v[e], G.v[e]);
+                }
             }
             dh.store(oh + j), dr.store(orr + j), dt.store(ot + j);
         }
@@ -819,7 +837,6 @@ int kge_score_bwd(const kge_tables *tab, const kge_batch *bat, const kge_saved *
     if (bat->neg && bat->neg_mode != KGE_NEG_TAIL && bat->neg_mode != KGE_NEG_HEAD) return KGE_EINVAL;
     const bool head = have_neg && bat->neg_mode == KGE_NEG_HEAD;
     if (have_neg) {
-        if (model == KGE_TRANSF) return KGE_EUNSUPPORTED;
         if (normed && P == 2 && !saved->neg) return KGE_EINVAL;
         if (model == KGE_TRANSH && (!saved->side_pos || !saved->side_neg)) return KGE_EINVAL;
         if (model == KGE_ROTATE && !saved->residual) return KGE_EINVAL;  // rotated heads from the forward pass
@@ -868,6 +885,7 @@ int kge_score_bwd(const kge_tables *tab, const kge_batch *bat, const kge_saved *
         case KGE_DISTMULT: rc = launch_tiles<KGE_DISTMULT, 2>(a, g0, g1, occ_neg, n_chunks, dv, fi_pass, st); break;
         case KGE_COMPLEX: rc = launch_tiles<KGE_COMPLEX, 2>(a, g0, g1, occ_neg, n_chunks, dv, fi_pass, st); break;
         case KGE_ROTATE: rc = launch_tiles<KGE_ROTATE, 2>(a, g0, g1, occ_neg, n_chunks, dv, fi_pass, st); break;
+        case KGE_TRANSF: rc = launch_tiles<KGE_TRANSF, 2>(a, g0, g1, occ_neg, n_chunks, dv, fi_pass, st); break;
         default: return KGE_EUNSUPPORTED;
         }
         timeline_mark(bat->timeline, st, "bwd_tile_kernel");
@@ -877,7 +895,8 @@ int kge_score_bwd(const kge_tables *tab, const kge_batch *bat, const kge_saved *
     }
 
     PosBwdArgs pa{tab->ent, tab->rel, tab->aux, bat->h, bat->r, bat->t, dpos, saved->pos, saved->side_pos,
-                  g0, g1, occ_e, occ_e + B * d, occ_r, occ_w, B, (int)d, (int)tab->rel_dim};
+                  g0, g1, have_neg ? dneg : nullptr, bat->n_neg, occ_e, occ_e + B * d, occ_r, occ_w, B, (int)d,
+                  (int)tab->rel_dim};
     switch (model) {
     case KGE_TRANSE:
         rc = P == 1 ? launch_pos_bwd<KGE_TRANSE, 1>(pa, vec, head, fi_dedup, st) : launch_pos_bwd<KGE_TRANSE, 2>(pa, vec, head, fi_dedup, st);

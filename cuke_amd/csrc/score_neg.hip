@@ -20,7 +20,7 @@ namespace kge {
 struct NegArgs {
     const float *ent, *rel, *aux;
     const int64_t *h, *r, *neg;  // h: the side of the positive that is kept (tails with head negatives)
-    const float *side_pos;  // TransH: w_b . h_b
+    const float *side_pos;  // TransH: w_b . h_b; TransF: r_b . h_b (the kept side: t_b with head negatives)
     const float *query;     // RotatE: rotated heads [B, d] from the positive kernel (required)
     float *out;             // [B, N]
     float *side_neg;        // TransH save-for-backward [2, B, N] (optional):
@@ -44,7 +44,7 @@ template <int MODEL, int P, bool SAVE>
 __device__ __forceinline__ void pair_elem(float &acc, float &acc2, float a0, float a1, float t0, float t1,
                                           float c)
 {
-    if constexpr (MODEL == KGE_DISTMULT || MODEL == KGE_COMPLEX) {
+    if constexpr (MODEL == KGE_DISTMULT || MODEL == KGE_COMPLEX || MODEL == KGE_TRANSF) {
         acc = fmaf(a0, t0, acc);
     } else if constexpr (MODEL == KGE_TRANSE) {
         const float u = a0 - t0;
@@ -294,6 +294,7 @@ __global__ __launch_bounds__(256, KGE_TILE_OCC) void score_neg_kernel(NegArgs a,
             float s = acc[i][k];
             if constexpr (MODEL == KGE_TRANSE || MODEL == KGE_TRANSH) s = P == 2 ? sqrtf(s) : s;
             if constexpr (MODEL == KGE_ROTATE) s = a.gamma - s;
+            if constexpr (MODEL == KGE_TRANSF) s -= a.rsign * a.side_pos[(int64_t)c * a.C + bl];
             a.out[rowoff + kl] = s;
             if constexpr (MODEL == KGE_TRANSH && SAVE) {
                 a.side_neg[rowoff + kl] = cdot[i][k];
@@ -317,7 +318,7 @@ __global__ __launch_bounds__(256, KGE_TILE_OCC) void score_neg_mfma_kernel(NegAr
 {
     extern __shared__ __align__(16) char dyn_smem[];
     if (fused_insp_block(fi, reinterpret_cast<uint32_t *>(dyn_smem))) return;
-    static_assert(MODEL == KGE_DISTMULT || MODEL == KGE_COMPLEX, "dot-product scores only");
+    static_assert(MODEL == KGE_DISTMULT || MODEL == KGE_COMPLEX || MODEL == KGE_TRANSF, "dot-product scores only");
     constexpr int TB = 16 * RB, TN = 16 * RK;
     constexpr int SB = TB / 32, SN = TN / 32;
     constexpr int MB = RB / 2, NB = RK / 2;  // 16 x 16 blocks per wave
@@ -422,10 +423,12 @@ __global__ __launch_bounds__(256, KGE_TILE_OCC) void score_neg_mfma_kernel(NegAr
             const int bl = bt0 + wrow + 16 * m + 4 * fg + v;
             if (bl >= a.C) continue;
             const int64_t rowoff = ((int64_t)c * a.C + bl) * a.N;
+            float shift = 0.0f;  // TransF: the per-positive constant -r.h (+r.t with head negatives)
+            if constexpr (MODEL == KGE_TRANSF) shift = -a.rsign * a.side_pos[(int64_t)c * a.C + bl];
 #pragma unroll
             for (int n = 0; n < NB; ++n) {
                 const int kl = kt0 + wcol + 16 * n + fr;
-                if (kl < a.N) a.out[rowoff + kl] = acc[0][m][n][v] + acc[1][m][n][v];
+                if (kl < a.N) a.out[rowoff + kl] = (acc[0][m][n][v] + acc[1][m][n][v]) + shift;
             }
         }
 }
@@ -446,11 +449,11 @@ static int launch_neg_mp(const NegArgs &a, int64_t n_chunks, bool dot_valu, cons
     // 64x64 on a 256-big-tile workload with the vector-ALU loop; the matrix-core loop, whose
     // launches are bound by the rows its workgroups pull from L2, does best with 32x64).  The
     // inspector workgroups that share the machine with these launches raise their wave priority.
-    constexpr bool kDotModel = MODEL == KGE_DISTMULT || MODEL == KGE_COMPLEX;
+    constexpr bool kDotModel = MODEL == KGE_DISTMULT || MODEL == KGE_COMPLEX || MODEL == KGE_TRANSF;
     const int tile = big_tiles >= 1024 ? 4 : (kDotModel && !dot_valu ? 3 : 2);  // 2: 32x32, 3: 32x64, 4: 64x64
     const int TB = tile == 4 ? 64 : 32, TN = tile == 2 ? 32 : 64;
     const dim3 grid(xcd_grid(ceil_div(a.N, TN), ceil_div(a.C, TB), n_chunks) + (unsigned)fi.blocks);
-    if constexpr (MODEL == KGE_DISTMULT || MODEL == KGE_COMPLEX) {
+    if constexpr (kDotModel) {
         if (!dot_valu) {
             const size_t lds = neg_lds(1, TB, TN, 1, fi);
             if (tile == 4) hipLaunchKernelGGL((score_neg_mfma_kernel<MODEL, 4, 4>), grid, dim3(256), lds, st, a, fi);
@@ -500,7 +503,8 @@ int launch_score_neg(const kge_tables *tab, const kge_batch *bat, const float *s
     case KGE_DISTMULT: return launch_neg_mp<KGE_DISTMULT, 2>(a, n_chunks, dv, fi, st);
     case KGE_COMPLEX: return launch_neg_mp<KGE_COMPLEX, 2>(a, n_chunks, dv, fi, st);
     case KGE_ROTATE: return launch_neg_mp<KGE_ROTATE, 2>(a, n_chunks, dv, fi, st);
-    default: return KGE_EUNSUPPORTED;  // TransR / TransF / RESCAL: positives only
+    case KGE_TRANSF: return launch_neg_mp<KGE_TRANSF, 2>(a, n_chunks, dv, fi, st);
+    default: return KGE_EUNSUPPORTED;  // TransR / RESCAL: their projection depends on the positive's relation
     }
 }
 

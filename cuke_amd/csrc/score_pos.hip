@@ -16,8 +16,8 @@ struct PosArgs {
     float *pos;       // [B] scores or nullptr
     float *resid;     // [B, d] or nullptr: residual rows (TransE / TransH / TransR), the projected heads
                       // E[h] Proj[r] (RESCAL) or, for RotatE, the rotated heads h e^{i theta} laid out [re | im]
-    float *side_pos;  // [B] TransH: w.h (used by the shared-negative kernels)
-    int head;         // negatives replace the head: side_pos = w.t, RotatE resid = t e^{-i theta}
+    float *side_pos;  // [B] TransH: w.h; TransF: r.h (used by the shared-negative kernels)
+    int head;         // negatives replace the head: side_pos = w.t / r.t, RotatE resid = t e^{-i theta}
 };
 
 constexpr int kPosWaves = 4;
@@ -125,12 +125,19 @@ __global__ __launch_bounds__(kPosWaves *kWave) void score_pos_kernel(PosArgs a, 
             for (int e = 0; e < V; ++e) acc += (vh.v[e] * vr.v[e]) * vt.v[e];
         }
     } else if constexpr (MODEL == KGE_TRANSF) {
+        float rx = 0.0f;  // r . (the side the shared negatives keep)
         for (int j = lane * V; j < d; j += kWave * V) {
             const Vec<V> vh = Vec<V>::load(eh + j), vt = Vec<V>::load(et + j),
                          vr = Vec<V>::load(rr + j);
 #pragma unroll
-            for (int e = 0; e < V; ++e)
+            for (int e = 0; e < V; ++e) {
                 acc += (vh.v[e] + vr.v[e]) * vt.v[e] + (vt.v[e] - vr.v[e]) * vh.v[e];
+                rx += vr.v[e] * (a.head ? vt.v[e] : vh.v[e]);
+            }
+        }
+        if (a.side_pos) {  // uniform
+            rx = wave_sum(rx);
+            if (valid && lane == 0) a.side_pos[b] = rx;
         }
     } else if constexpr (MODEL == KGE_COMPLEX) {
         const int half = d / 2;

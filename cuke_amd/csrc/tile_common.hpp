@@ -73,11 +73,13 @@ __device__ __forceinline__ int pair_len(int d)
 //   DistMult  q0 = h*r                   ComplEx  q0 = (h o r) laid out [re | im]
 //   TransE    q0 = h+r                   RotatE   q0 = Re(h e^{i theta}), q1 = Im(...) (from pq)
 //   TransH    q0 = h + r - al*w (al = w.h), q1 = w
+//   TransF    q0 = 2h + r: score = (h + r).t' + (t' - r).h = (2h + r).t' - r.h, a dot product with
+//             the query plus a constant per positive
 // lim == 0 yields zeros (row outside the tile).
 // RotatE takes its query rows from pq, the [B, d] buffer of rotated heads.
 //
 // Negatives that replace the HEAD use the same pair kernels: score(n, r, t) is the tail-mode
-// function of (x, rho, n) with x = t and rho = -r (TransE, TransH), conj(r) (ComplEx), -theta
+// function of (x, rho, n) with x = t and rho = -r (TransE, TransH, TransF), conj(r) (ComplEx), -theta
 // (RotatE, already applied in pq) or r (DistMult).  The caller passes the tail row as `ph` and
 // rs = -1; rs multiplies r (its imaginary half for ComplEx), which is exact, so rs = +1
 // reproduces the tail-mode arithmetic bit for bit.
@@ -92,6 +94,10 @@ __device__ __forceinline__ void load_query(const float *ph, const float *pr, con
     } else if constexpr (MODEL == KGE_TRANSE) {
         const float4 vh = ld4<VEC>(ph, j, lim), vr = ld4<VEC>(pr, j, lim);
         q0 = make_float4(fmaf(rs, vr.x, vh.x), fmaf(rs, vr.y, vh.y), fmaf(rs, vr.z, vh.z), fmaf(rs, vr.w, vh.w));
+    } else if constexpr (MODEL == KGE_TRANSF) {
+        const float4 vh = ld4<VEC>(ph, j, lim), vr = ld4<VEC>(pr, j, lim);
+        q0 = make_float4(fmaf(rs, vr.x, 2.0f * vh.x), fmaf(rs, vr.y, 2.0f * vh.y), fmaf(rs, vr.z, 2.0f * vh.z),
+                         fmaf(rs, vr.w, 2.0f * vh.w));
     } else if constexpr (MODEL == KGE_COMPLEX) {
         float q[4];
         if constexpr (VEC) {  // half % 4 == 0: the four elements sit on one side of the re|im split
@@ -170,7 +176,7 @@ __device__ __forceinline__ void load_query_raw(const float *ph, const float *pr,
                                                int j, int lim, int half, float4 (&raw)[N])
 {
     static_assert(N == query_raw_count<MODEL>(), "raw operand count");
-    if constexpr (MODEL == KGE_DISTMULT || MODEL == KGE_TRANSE) {
+    if constexpr (MODEL == KGE_DISTMULT || MODEL == KGE_TRANSE || MODEL == KGE_TRANSF) {
         raw[0] = ld4_raw<VEC>(ph, j, lim);
         raw[1] = ld4_raw<VEC>(pr, j, lim);
     } else if constexpr (MODEL == KGE_COMPLEX) {
@@ -211,6 +217,11 @@ __device__ __forceinline__ void combine_query(const float4 (&raw)[N], float al, 
     } else if constexpr (MODEL == KGE_TRANSE) {
         const float4 vh = raw[0], vr = raw[1];
         q0 = mask4<VEC>(make_float4(fmaf(rs, vr.x, vh.x), fmaf(rs, vr.y, vh.y), fmaf(rs, vr.z, vh.z), fmaf(rs, vr.w, vh.w)),
+                        j, lim);
+    } else if constexpr (MODEL == KGE_TRANSF) {
+        const float4 vh = raw[0], vr = raw[1];
+        q0 = mask4<VEC>(make_float4(fmaf(rs, vr.x, 2.0f * vh.x), fmaf(rs, vr.y, 2.0f * vh.y), fmaf(rs, vr.z, 2.0f * vh.z),
+                                    fmaf(rs, vr.w, 2.0f * vh.w)),
                         j, lim);
     } else if constexpr (MODEL == KGE_COMPLEX) {
         const float hr[4] = {raw[0].x, raw[0].y, raw[0].z, raw[0].w}, hi[4] = {raw[1].x, raw[1].y, raw[1].z, raw[1].w};

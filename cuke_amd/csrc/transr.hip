@@ -36,6 +36,10 @@ constexpr int kDmRing = KGE_TR_DM_RING;  // the same for the dM kernel's operand
 constexpr int kThin = 4;            // a group's last tile with at most this many triples takes the thin path
 constexpr int kThinRing = 8;        // 128-bit projection loads in flight per thread on the thin path
 constexpr int kMaxDimMfma = 1024;
+// Dynamic LDS a grouped kernel may ask for: a CU of gfx950 has 160 KB, a few hundred bytes of
+// which the kernels' static arrays take.  The 32 x d left-operand tile needs 66.5 KB at d = 512
+// and 129 KB at d = 1024 (then one workgroup per CU).
+constexpr size_t kMaxGemmLds = 158 * 1024;
 
 int launch_score_pos(const kge_tables *, const kge_batch *, float *, float *, float *, hipStream_t);
 
@@ -649,7 +653,7 @@ static bool mfma_path_ok(const kge_tables *tab, const kge_batch *bat)
 
 bool transr_grouped_path_ok(const kge_tables *tab, const kge_batch *bat)
 {
-    return mfma_path_ok(tab, bat) && gemm_lds_bytes((int)tab->dim) <= 64 * 1024;
+    return mfma_path_ok(tab, bat) && gemm_lds_bytes((int)tab->dim) <= kMaxGemmLds;
 }
 
 // ---- backward kernels ----------------------------------------------------------------------
@@ -945,6 +949,17 @@ size_t transr_fwd_workspace(const kge_tables *tab, const kge_batch *bat)
     return fwd_plan_bytes(tab, bat) + up256(sizeof(int32_t) * plan_ints(p.dtiles, p.dsplit));
 }
 
+// A launch with more than 64 KB of dynamic LDS has to be allowed per kernel first.
+template <int MODE>
+static int allow_lds(size_t bytes)
+{
+    if (bytes <= 64 * 1024) return KGE_OK;
+    return hipFuncSetAttribute(reinterpret_cast<const void *>(&transr_gemm_kernel<MODE>),
+                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)kMaxGemmLds) == hipSuccess
+               ? KGE_OK
+               : KGE_ELAUNCH;
+}
+
 static size_t lds_with(const FusedInsp &fi, size_t own)
 {
     return fi.blocks > 0 && (size_t)fi.lds_bytes > own ? (size_t)fi.lds_bytes : own;
@@ -956,7 +971,7 @@ int launch_transr_fwd(const kge_tables *tab, const kge_batch *bat, float *pos, f
     if (bat->batch == 0) return KGE_OK;
     const bool rescal = tab->model == KGE_RESCAL;
     const bool grouped = mfma_path_ok(tab, bat) && workspace && workspace_bytes >= transr_fwd_workspace(tab, bat) &&
-                         gemm_lds_bytes((int)tab->dim) <= 64 * 1024;
+                         gemm_lds_bytes((int)tab->dim) <= kMaxGemmLds;
     // fused entity inspection: its histogram step rides with the forward GEMM
     FusedInsp fi{};
     if (bat->fuse_inspection) {
@@ -980,6 +995,7 @@ int launch_transr_fwd(const kge_tables *tab, const kge_batch *bat, float *pos, f
                plan, nullptr, pos, resid, nullptr, nullptr, (int)tab->dim, tab->norm_p, thin_groups(tab, bat), (int)tiles};
     const size_t lds = lds_with(fi, gemm_lds_bytes((int)tab->dim));
     const dim3 grid((unsigned)(tiles + a.thin_groups + fi.blocks));
+    if (const int rc = rescal ? allow_lds<1>(lds) : allow_lds<0>(lds)) return rc;
     if (rescal)
         hipLaunchKernelGGL(transr_gemm_kernel<1>, grid, dim3(256), lds, st, a, fi);
     else
@@ -996,7 +1012,7 @@ int launch_transr_bwd(const kge_tables *tab, const kge_batch *bat, const kge_sav
 {
     const bool rescal = tab->model == KGE_RESCAL;
     if (bat->neg) return KGE_EUNSUPPORTED;  // positives only for the projection models
-    if (!mfma_path_ok(tab, bat) || gemm_lds_bytes((int)tab->dim) > 64 * 1024) return KGE_EUNSUPPORTED;
+    if (!mfma_path_ok(tab, bat) || gemm_lds_bytes((int)tab->dim) > kMaxGemmLds) return KGE_EUNSUPPORTED;
     if (!saved->residual || !grads->aux_rows || !grads->ent_rows) return KGE_EINVAL;
     if (!rescal && (!grads->rel_rows || (tab->norm_p == 2 && !saved->pos))) return KGE_EINVAL;
     const RPlan p = make_rplan(tab, bat);
@@ -1035,6 +1051,7 @@ int launch_transr_bwd(const kge_tables *tab, const kge_batch *bat, const kge_sav
     // dX = Q M^T -> occurrence rows of h (and -dX for t)
     GemmArgs ga{tab->ent, tab->rel, tab->aux, bat->h, bat->r, bat->t, ri->perm, ri->seg_offsets, ri->num_unique, ri->unique_ids,
                 plan, qs, nullptr, nullptr, occ, rescal ? nullptr : occ + B * d, d, tab->norm_p, thin_groups(tab, bat), (int)p.tiles};
+    if (const int rc = allow_lds<2>(lds_with(f2, gemm_lds_bytes(d)))) return rc;
     hipLaunchKernelGGL(transr_gemm_kernel<2>, dim3((unsigned)(p.tiles + ga.thin_groups + f2.blocks)), dim3(256),
                        lds_with(f2, gemm_lds_bytes(d)), st, ga, f2);
     timeline_mark(bat->timeline, st, "transr_gemm_kernel<dX>");

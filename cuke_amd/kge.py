@@ -250,9 +250,9 @@ class KGEModel:
         f32 = dict(dtype=torch.float32, device=self.dev)
         fw = Forward(torch.empty(B, **f32), torch.empty((B, N), **f32) if neg is not None else None,
                      batch=keep, ent_insp=ent_insp, rel_insp=rel_insp, neg_mode=neg_mode)
-        if self.model == "TransH":
+        if self.model == "TransH" or (self.model == "TransF" and neg is not None):
             fw.side_pos = torch.empty(B, **f32)
-            if neg is not None:
+            if neg is not None and self.model == "TransH":
                 fw.side_neg = torch.empty((2, B, N), **f32)
         if self.model in ("TransR", "RESCAL", "RotatE"):
             fw.residual = torch.empty((B, self.dim), **f32)
@@ -476,7 +476,8 @@ class TrainStep:
         self.side = torch.cuda.Stream(device=dev)  # default priority
         self.pos = torch.empty(B, **f32)
         self.neg = torch.empty((B, N), **f32) if neg is not None else None
-        self.side_pos = torch.empty(B, **f32) if model.model == "TransH" else None
+        self.side_pos = torch.empty(B, **f32) if (model.model == "TransH" or
+                                                  (model.model == "TransF" and neg is not None)) else None
         self.side_neg = torch.empty((2, B, N), **f32) if (model.model == "TransH" and neg is not None) else None
         self.residual = torch.empty((B, model.dim), **f32) if model.model in ("TransR", "RESCAL", "RotatE") \
             else None

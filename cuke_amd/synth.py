@@ -130,6 +130,27 @@ def make_tables(w: Workload) -> None:
             a["A"] = (np.clip(np.rint(a["A"] * 4 * 3), -4, 4) / 4).astype(np.float32)
 
 
+def device_tables(w: Workload, dev):
+    """The workload's tables drawn on the GPU from its seed (same distributions as make_tables): tables of
+    benchmark size are too large to push through numpy.  Returns torch tensors (E, R, A)."""
+    import torch
+    g = torch.Generator(device=dev)
+    g.manual_seed(1000 + w.seed)
+    f32 = dict(generator=g, device=dev, dtype=torch.float32)
+    E = torch.randn((w.n_ent, w.dim), **f32) * w.sigma
+    if w.model == "RotatE":
+        R = (torch.rand((w.n_rel, w.rel_dim), **f32) * 2 - 1) * np.pi
+    else:
+        R = torch.randn((w.n_rel, w.rel_dim), **f32) * w.sigma
+    A = None
+    if w.model == "TransH":
+        A = torch.randn((w.n_rel, w.dim), **f32)
+        A = A / A.norm(dim=1, keepdim=True)
+    elif w.model in ("TransR", "RESCAL"):
+        A = torch.randn((w.n_rel, w.dim, w.dim), **f32) * w.sigma
+    return E, R, A
+
+
 def make_workload(name: str, seed: int = 0, tables: bool = True, **override) -> Workload:
     """Build a named configuration; keyword overrides shrink it for tests."""
     spec = dict(CONFIGS[name])

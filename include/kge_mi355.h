@@ -173,7 +173,8 @@ typedef struct kge_batch {
 typedef struct kge_saved {
     const float *pos;       /* [B] positive scores */
     const float *neg;       /* [B, n_neg] negative scores (NULL without negatives) */
-    const float *side_pos;  /* [B]: TransH w.h per positive (w.t with KGE_NEG_HEAD); TransR: unused */
+    const float *side_pos;  /* [B]: TransH w.h per positive (w.t with KGE_NEG_HEAD); TransF with
+                               negatives r.h (r.t); TransR: unused */
     const float *side_neg;  /* [2, B, n_neg]: TransH, plane 0 = w_b . e_k per pair (e_k the negative),
                                plane 1 = sum_i phi(u_i) w_i (phi = sign for L1, u/||u|| for L2) */
     const float *residual;  /* [B, dim]: TransR residual rows / RESCAL E[h] Proj[r] rows;
@@ -211,7 +212,8 @@ int kge_residual_fwd(const kge_tables *tab, const kge_batch *bat, float *out, vo
 /*
  * Scalar scores.  pos[B]; neg[B, n_neg] when bat->neg is set (either may be
  * NULL to skip).  side_pos / side_neg are optional save-for-backward outputs
- * (see kge_saved; required later by kge_score_bwd for TransH).
+ * (see kge_saved; required later by kge_score_bwd for TransH; side_pos is also required when
+ * TransF scores shared negatives: the pair kernel reads r.h from it).
  * Scalar-score models of the reference: TransF / RESCAL (kge.py:363,387).
  * TransR / RESCAL: with bat->rel_insp (relation groups) the projection runs as grouped
  * per-relation MFMA contractions and needs kge_score_fwd_workspace() bytes of workspace;

@@ -503,6 +503,58 @@ int orc_backward(int model, int p, int64_t B, int64_t d, const float *E, const f
 }
 
 /*
+ * Which gradient rows an L1 sign ambiguity can reach.  The L1 gradient of TransE / TransH is a
+ * sum of signs of residual elements; an element within rounding of zero may get either sign
+ * from two correct fp32 implementations, and (TransH) one flipped sign moves every column of
+ * the rows of that triple through q.w.  For every triple and pair of the batch whose residual
+ * holds an element with |u_j| <= eps this marks the slots of its head, tail / negative and
+ * relation rows in flagE[n_slots_e] / flagR[n_slots_r] (bytes, caller-zeroed; writes of 1
+ * only, so threads may race on them).  Returns the number of such elements, -1 for a model
+ * without an L1 form.
+ */
+int64_t orc_l1_ambiguous(int model, int64_t B, int64_t d, const float *E, const float *R, const float *A,
+                         const int64_t *h, const int64_t *r, const int64_t *t, const int64_t *neg, int64_t C,
+                         int64_t N, int neg_head, float eps, const int64_t *slot_h, const int64_t *slot_t,
+                         const int64_t *slot_neg, const int64_t *slot_r, unsigned char *flagE,
+                         unsigned char *flagR)
+{
+    if (model != ORC_TRANSE && model != ORC_TRANSH) return -1;
+    int64_t total = 0;
+#ifdef _OPENMP
+#pragma omp parallel reduction(+ : total)
+#endif
+    {
+        float *u = (float *)malloc(sizeof(float) * (size_t)(d + 1));
+#ifdef _OPENMP
+#pragma omp for schedule(static)
+#endif
+        for (int64_t b = 0; b < B; ++b) {
+            const float *rr = R + r[b] * d, *ax = A ? A + r[b] * d : NULL;
+            const int64_t c = C > 0 ? b / C : 0;
+            for (int64_t q = 0; q < 1 + (neg ? N : 0); ++q) {
+                const float *eh = E + h[b] * d, *et = E + t[b] * d;
+                int64_t sh = slot_h[b], st = slot_t[b];
+                if (q > 0) {
+                    const int64_t k = q - 1;
+                    if (neg_head) eh = E + neg[c * N + k] * d, sh = slot_neg[c * N + k];
+                    else et = E + neg[c * N + k] * d, st = slot_neg[c * N + k];
+                }
+                if (model == ORC_TRANSE) residual_transe(d, eh, rr, et, u);
+                else (void)residual_transh(d, eh, rr, et, ax, u);
+                int64_t n = 0;
+                for (int64_t j = 0; j < d; ++j) n += fabsf(u[j]) <= eps;
+                if (n) {
+                    flagE[sh] = 1, flagE[st] = 1, flagR[slot_r[b]] = 1;
+                    total += n;
+                }
+            }
+        }
+        free(u);
+    }
+    return total;
+}
+
+/*
  * Margin-ranking loss over positive/negative score pairs,
  *   L = mean_{b,k} max(0, margin - sign * (pos[b] - neg[b,k])),
  * sign = +1 when larger scores are better (== torch margin_ranking_loss with

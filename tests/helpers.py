@@ -58,3 +58,22 @@ def gpu_model(w, device="cuda:0"):
     m = KGEModel(w.model, E, R, A, norm_p=w.norm_p, gamma=w.gamma)
     idx = {k: torch.from_numpy(a[k]).to(dev) for k in ("h", "r", "t", "neg") if k in a}
     return m, idx
+
+
+def compare_l1_generic(oracle, w, a, g, ref, dmax, what, fast=False):
+    """L1 gradients on generic floats.  A residual element within rounding of zero may take either sign in
+    two correct fp32 evaluations, and one flipped sign moves every column of the rows of that pair (through
+    q.w).  The oracle names the rows such an element can reach (|u| <= 6e-8, a few ulps of the operands);
+    every other row must meet the ordinary bar, and a reachable row may be off by at most its flips."""
+    amb_e, amb_r, n_amb = oracle.l1_ambiguous_rows(w.model, a["E"], a["R"], a["A"], a["h"], a["r"], a["t"],
+                                                   a.get("neg"), w.chunk, eps=6e-8, fast=fast)
+    assert np.array_equal(g.ent_ids.cpu().numpy(), ref.ent_ids) and np.array_equal(g.rel_ids.cpu().numpy(), ref.rel_ids)
+    assert amb_e.mean() < 0.5, f"{what}: the mask must leave most rows to the ordinary bar ({amb_e.mean():.2f} masked)"
+    for name, amb in (("ent_rows", amb_e), ("rel_rows", amb_r), ("aux_rows", amb_r)):
+        got, want = getattr(g, name).cpu().numpy(), getattr(ref, name)
+        assert_close(got[~amb], want[~amb], what=f"{what} {name} clear of sign ambiguity", rows=True)
+        # a masked row: each flip changes a pair's q_j by 2|g| and, through (q.w) w and (q.w) d0, the
+        # other columns by less; bound the row by the flips that can reach it
+        err = np.abs(got[amb].astype(np.float64) - want[amb])
+        assert (err <= 2.0 * dmax * n_amb * (1 + 1e-3)).all() if err.size else True
+    return int(amb_e.sum()), n_amb

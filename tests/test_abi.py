@@ -111,7 +111,7 @@ def test_argument_validation_returns_status_codes_without_touching_the_gpu():
 
 def test_fused_inspection_eligibility_is_decided_on_the_host():
     """kge_fused_inspection_ok only reads the descriptors: shared negatives, index sets of at most 65536 ids and
-    tables of at most 2^22 rows qualify; TransF (no shared-negative kernels), larger sets and larger tables do not,
+    tables of at most 2^22 rows qualify; larger sets and larger tables do not,
     and asking the score calls for a fused inspection without the jobs is an argument error."""
     import ctypes as C
     from cuke_amd import _lib
@@ -140,7 +140,7 @@ def test_fused_inspection_eligibility_is_decided_on_the_host():
     assert ok("RotatE", batch(), jobs(3072, 1024, 1 << 22)) == 1
     assert ok("TransE", batch(), jobs(3072, 1024, (1 << 22) + 1)) == 0      # needs a third digit pass
     assert ok("TransH", batch(), jobs(65537, 1024, 1000)) == 0              # multi-block sort territory
-    assert ok("TransF", batch(), jobs(3072, 1024, 1000)) == 0               # no tile kernels to ride with
+    assert ok("TransF", batch(), jobs(3072, 1024, 1000)) == 1
     assert ok("DistMult", batch(neg=False), jobs(2048, 1024, 1000)) == 0
     assert ok("TransR", batch(neg=False), jobs(2048, 1024, 1000)) == 0      # no relation groups given
     # the flag without the jobs

@@ -59,8 +59,6 @@ def test_hip_path_reproduces_golden_vectors(case, mode):
     from cuke_amd.kge import KGEModel
     get, chunk, n_neg, p, gamma = load(case)
     model = case.split("_")[0]
-    if model == "TransF":
-        pytest.skip("TransF has no shared-negative form in the library (positives are covered elsewhere)")
     dev = torch.device("cuda:0")
     tt = lambda x: None if x is None else torch.from_numpy(np.ascontiguousarray(x)).to(dev)  # noqa: E731
     R = get("R")

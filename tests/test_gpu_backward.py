@@ -4,11 +4,11 @@ import pytest
 import torch
 
 from cuke_amd import synth
-from helpers import assert_close, gpu_model
+from helpers import assert_close, compare_l1_generic, gpu_model
 
 pytestmark = pytest.mark.gpu
 
-NEG_MODELS = ["TransE", "TransH", "DistMult", "ComplEx", "RotatE"]
+NEG_MODELS = ["TransE", "TransH", "DistMult", "ComplEx", "RotatE", "TransF"]
 
 
 def run_both(oracle, w, seed=0, use_pos=True, use_neg=True, pair_sums="matrix_cores"):
@@ -58,7 +58,7 @@ def test_shared_negative_gradients(oracle, model, shape, p):
     compare(g, ref, f"{model} {shape} p={p}")
 
 
-@pytest.mark.parametrize("model", NEG_MODELS + ["TransF"])
+@pytest.mark.parametrize("model", NEG_MODELS)
 def test_positive_only_gradients(oracle, model):
     w = synth.custom_workload(model, n_ent=300, n_rel=9, dim=64, batch=333, sigma=0.2, gamma=4.0,
                               ent_zipf=1.2, seed=3)
@@ -118,16 +118,12 @@ def test_margin_loss_step_rotate(oracle):
 
 
 def test_transh_l1_generic_floats_differ_only_by_sign_flips(oracle):
-    # On generic floats the two implementations may disagree on the sign of residual elements
-    # that are within rounding of zero (about one element in 10^6).  Such a flip moves a few
-    # hundred gradient entries by O(|g| |w|^2); everything else must still agree.
     w = synth.make_workload("cfg5_transh", n_ent=200_000, batch=1024)
     g, ref = run_both(oracle, w, seed=9)
-    got, want = g.ent_rows.cpu().numpy().astype(np.float64), ref.ent_rows.astype(np.float64)
-    rms = np.sqrt(np.mean(want * want, axis=1, keepdims=True))
-    bad = np.abs(got - want) > 1e-5 * np.abs(want) + 1e-5 * rms
-    assert bad.mean() < 5e-3
-    assert np.abs(got - want).max() < 16.0  # a handful of flips, each worth at most 2|g|
+    rng = np.random.default_rng(9)  # the upstream gradients run_both drew
+    dmax = max(np.abs(rng.standard_normal(w.batch)).max(), np.abs(rng.standard_normal((w.batch, w.n_neg))).max())
+    masked, n_amb = compare_l1_generic(oracle, w, w.arrays, g, ref, float(dmax), "cfg5 scaled, generic floats")
+    assert n_amb > 0, "at this size some residual element is expected within 6e-8 of zero"
 
 
 @pytest.mark.parametrize("name,over", [

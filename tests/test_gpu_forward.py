@@ -9,7 +9,7 @@ from helpers import assert_close, gpu_model
 pytestmark = pytest.mark.gpu
 
 RESIDUAL = ["TransE", "TransH", "TransR"]
-NEG_MODELS = ["TransE", "TransH", "DistMult", "ComplEx", "RotatE"]
+NEG_MODELS = ["TransE", "TransH", "DistMult", "ComplEx", "RotatE", "TransF"]
 ALL = ["TransE", "TransH", "TransR", "DistMult", "ComplEx", "RotatE", "TransF", "RESCAL"]
 
 
@@ -43,6 +43,34 @@ def test_reference_shaped_callables(oracle):
             out = kge.transR(w.batch, w.dim, 0, E, h, t, 0, P, r, dummy, dummy, dummy, R)
         want = oracle.residual(model, a["E"], a["R"], a["A"], a["h"], a["r"], a["t"])
         assert_close(out.cpu().numpy(), want, what=f"{model} residual")
+
+
+def test_reference_shaped_scalar_callables(oracle):
+    """kge.transF / kge.RESCAL take the reference's positional lists literally
+    (apps/kge/test_cuke.py:198,244): (batch, dim, nnodes, E, h, nedges, R | Proj, r, uniq, buf, cnt, t) -- the tail
+    ids come LAST, after the three inspector tensors.  h and t are drawn differently, and TransF / RESCAL are not
+    symmetric in them, so a slip in the order changes the scores."""
+    from cuke_amd import kge
+    dev = torch.device("cuda:0")
+    for model in ("TransF", "RESCAL"):
+        w = synth.custom_workload(model, n_ent=300, n_rel=17, dim=64, batch=160, sigma=0.2, seed=9)
+        a = w.arrays
+        E = torch.from_numpy(a["E"]).to(dev)
+        h, r, t = (torch.from_numpy(a[k]).to(dev) for k in "hrt")
+        r_sorted, order = torch.sort(r)  # the reference sorts the batch by relation before its inspector
+        uniq, buf, cnt = kge.inspector(r_sorted, w.n_rel)
+        if model == "TransF":
+            Rm = torch.from_numpy(a["R"]).to(dev)
+            out = kge.transF(w.batch, w.dim, w.n_ent, E, h[order], w.n_rel, Rm, r_sorted, uniq, buf, cnt, t[order])
+        else:
+            Pm = torch.from_numpy(a["A"]).to(dev)
+            out = kge.RESCAL(w.batch, w.dim, w.n_ent, E, h[order], w.n_rel, Pm, r_sorted, uniq, buf, cnt, t[order])
+        o = order.cpu().numpy()
+        want, _ = oracle.score(model, a["E"], a["R"], a["A"], a["h"][o], a["r"][o], a["t"][o])
+        assert out.shape == (w.batch,)
+        assert_close(out.cpu().numpy(), want, what=f"{model} positional call")
+        swapped, _ = oracle.score(model, a["E"], a["R"], a["A"], a["t"][o], a["r"][o], a["h"][o])
+        assert np.abs(swapped - want).max() > 1e-3, "the test inputs must tell h from t"
 
 
 @pytest.mark.parametrize("model", ALL)

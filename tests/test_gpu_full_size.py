@@ -10,7 +10,7 @@ import pytest
 import torch
 
 from cuke_amd import synth
-from helpers import assert_close, gpu_model
+from helpers import assert_close, compare_l1_generic, gpu_model
 
 pytestmark = pytest.mark.gpu
 
@@ -136,6 +136,38 @@ def test_gradients_invariant_under_chunk_permutation(full):
             continue
         assert_close(r1.cpu().numpy(), r0.cpu().numpy(), rtol=2e-5, what=f"{w.name} {name} after permutation",
                      rows=True, outliers=out)
+
+
+def test_cfg5_on_its_stated_inputs_at_full_size(oracle):
+    """Config 5 as it is stated: a 4,000,000 x 400 entity table N(0, 0.05), 10,000 relations with unit
+    normals, 16,384 positives x 1,024 shared negatives, L1 norm.  The tables are drawn on the GPU (as the
+    benchmark draws them); the oracle gets the rows the batch names, copied back from the device, under
+    compact ids.  Scores: ordinary bar (|u| is continuous, no sign ambiguity in the forward pass).
+    Gradients: ordinary bar on every row no sign ambiguity can reach (see compare_l1_generic).  The oracle
+    runs its OpenMP build here (same source and loops; threads split the batch)."""
+    from cuke_amd.kge import KGEModel
+    w = synth.make_workload("cfg5_transh", tables=False)
+    a = w.arrays
+    E, R, A = synth.device_tables(w, torch.device("cuda:0"))
+    assert torch.allclose(A.norm(dim=1), torch.ones(w.n_rel, device=A.device), atol=1e-5)
+    m = KGEModel(w.model, E, R, A, norm_p=1)
+    ix = {k: torch.from_numpy(a[k]).cuda() for k in ("h", "r", "t", "neg")}
+    fw = m.score(ix["h"], ix["r"], ix["t"], ix["neg"], w.chunk)
+    ue, ur = np.unique(np.concatenate([a["h"], a["t"], a["neg"]])), np.unique(a["r"])
+    c = dict(E=E[torch.from_numpy(ue).cuda()].cpu().numpy(), R=R[torch.from_numpy(ur).cuda()].cpu().numpy(),
+             A=A[torch.from_numpy(ur).cuda()].cpu().numpy(), h=np.searchsorted(ue, a["h"]), t=np.searchsorted(ue, a["t"]),
+             r=np.searchsorted(ur, a["r"]), neg=np.searchsorted(ue, a["neg"]))
+    pos, negs = oracle.score("TransH", c["E"], c["R"], c["A"], c["h"], c["r"], c["t"], c["neg"], w.chunk, p=1,
+                             fast="omp")
+    assert_close(fw.pos.cpu().numpy(), pos, what="cfg5 (stated inputs) pos")
+    assert_close(fw.neg.cpu().numpy(), negs, what="cfg5 (stated inputs) neg")
+    dpos, dneg = upstream(w, 13)
+    g = m.backward(fw, dev(dpos), dev(dneg))
+    ref = oracle.backward("TransH", c["E"], c["R"], c["A"], c["h"], c["r"], c["t"], c["neg"], w.chunk, dpos, dneg,
+                          p=1, fast="omp")
+    ref.ent_ids, ref.rel_ids = ue[ref.ent_ids], ur[ref.rel_ids]  # compact ids back to table ids
+    dmax = float(max(np.abs(dpos).max(), np.abs(dneg).max()))
+    compare_l1_generic(oracle, w, c, g, ref, dmax, "cfg5 (stated inputs)", fast="omp")
 
 
 @pytest.mark.parametrize("model,p", [("DistMult", 2), ("TransE", 2)])

@@ -10,7 +10,7 @@ from helpers import assert_close, gpu_model
 
 pytestmark = pytest.mark.gpu
 
-NEG_MODELS = ["TransE", "TransH", "DistMult", "ComplEx", "RotatE"]
+NEG_MODELS = ["TransE", "TransH", "DistMult", "ComplEx", "RotatE", "TransF"]
 
 
 def both(oracle, w, seed=0, neg_mode="head"):

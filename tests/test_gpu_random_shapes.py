@@ -12,7 +12,7 @@ from helpers import assert_close, gpu_model
 
 pytestmark = pytest.mark.gpu
 
-NEG_MODELS = ["TransE", "TransH", "DistMult", "ComplEx", "RotatE"]
+NEG_MODELS = ["TransE", "TransH", "DistMult", "ComplEx", "RotatE", "TransF"]
 
 
 def draw(seed):

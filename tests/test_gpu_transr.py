@@ -23,7 +23,9 @@ def grouped_forward(m, ix):
     dict(dim=64, batch=257, n_rel=1),        # one group, many tiles
     dict(dim=36, batch=130, n_rel=9),        # K tail (36 = 2 * 16 + 4)
     dict(dim=400, batch=60, n_rel=40),       # wide rows: two column sweeps, thin tails in two k-chunks
-    dict(dim=496, batch=24, n_rel=20),       # the widest row the LDS tile takes
+    dict(dim=496, batch=24, n_rel=20),
+    dict(dim=512, batch=4096, n_rel=30),     # the reference's own sweep shapes (apps/kge/scripts/test_fig9c_cuke.sh):
+    dict(dim=1024, batch=1024, n_rel=12),    # left-operand tiles of 66.5 KB and 129 KB in LDS
 ])
 @pytest.mark.parametrize("p", [1, 2])
 def test_grouped_forward(oracle, model, shape, p):
@@ -52,6 +54,8 @@ def test_grouped_forward(oracle, model, shape, p):
     dict(dim=64, batch=257, n_rel=1),
     dict(dim=400, batch=60, n_rel=40),
     dict(dim=496, batch=24, n_rel=20),
+    dict(dim=512, batch=4096, n_rel=30),
+    dict(dim=1024, batch=1024, n_rel=12),
 ])
 @pytest.mark.parametrize("p", [1, 2])
 def test_grouped_backward(oracle, model, shape, p):

@@ -387,3 +387,50 @@ def test_sparse_optimizer_steps_vs_numpy(oracle):
     close(got_s, st); close(got_t, want)
     untouched = np.setdiff1d(np.arange(50), ids)
     assert np.array_equal(got_t[untouched], table[untouched])
+
+
+def test_openmp_build_of_the_oracle_gives_the_checkers_results(oracle):
+    """The OpenMP build (the timed multi-thread leg, and the checker of the full-size config-5 test) is the
+    same source: every score comes from the same serial loop, so scores are bit-identical; gradient rows
+    differ only in the order the per-thread double accumulators are added."""
+    for model, p in (("TransH", 1), ("DistMult", 2), ("RotatE", 2), ("TransR", 2)):
+        kw = dict(chunk=32, n_neg=24) if model != "TransR" else {}
+        w = synth.custom_workload(model, n_ent=300, n_rel=7, dim=24, batch=96, norm_p=p, sigma=0.2, gamma=3.0,
+                                  ent_zipf=1.1, seed=2, **kw)
+        a = w.arrays
+        args = (model, a["E"], a["R"], a["A"], a["h"], a["r"], a["t"], a.get("neg"), w.chunk)
+        pos0, neg0 = oracle.score(*args, p=p, gamma=w.gamma)
+        pos1, neg1 = oracle.score(*args, p=p, gamma=w.gamma, fast="omp")
+        assert np.array_equal(pos0, pos1) and (neg0 is None or np.array_equal(neg0, neg1))
+        rng = np.random.default_rng(1)
+        dpos = rng.standard_normal(w.batch).astype(np.float32)
+        dneg = rng.standard_normal((w.batch, w.n_neg)).astype(np.float32) if w.chunk else None
+        g0 = oracle.backward(*args, dpos, dneg, p=p)
+        g1 = oracle.backward(*args, dpos, dneg, p=p, fast="omp")
+        for x, y in ((g0.ent_rows, g1.ent_rows), (g0.rel_rows, g1.rel_rows), (g0.aux_rows, g1.aux_rows)):
+            if x is not None:
+                assert np.allclose(x, y, rtol=1e-6, atol=1e-9)
+
+
+def test_l1_ambiguity_mask_vs_numpy(oracle):
+    """l1_ambiguous_rows marks exactly the rows of the triples and pairs whose residual has an element with
+    |u| <= eps (brute force in numpy; eps chosen large enough that a fraction of the rows is marked)."""
+    w = synth.custom_workload("TransH", n_ent=60, n_rel=5, dim=8, batch=24, chunk=12, n_neg=6, norm_p=1, sigma=0.2,
+                              seed=4)
+    a = w.arrays
+    eps = 2e-3
+    fe, fr, n = oracle.l1_ambiguous_rows("TransH", a["E"], a["R"], a["A"], a["h"], a["r"], a["t"], a["neg"], w.chunk,
+                                         eps=eps)
+    ue, ur = np.unique(np.concatenate([a["h"], a["t"], a["neg"]])), np.unique(a["r"])
+    we, wr, total = np.zeros(ue.size, bool), np.zeros(ur.size, bool), 0
+    for b in range(w.batch):
+        tails = [a["t"][b]] + list(a["neg"][(b // w.chunk) * w.n_neg:(b // w.chunk + 1) * w.n_neg])
+        for tl in tails:
+            u = oracle.residual("TransH", a["E"], a["R"], a["A"], a["h"][b:b + 1], a["r"][b:b + 1], np.array([tl]))[0]
+            k = int((np.abs(u) <= np.float32(eps)).sum())
+            if k:
+                total += k
+                we[np.searchsorted(ue, [a["h"][b], tl])] = True
+                wr[np.searchsorted(ur, a["r"][b])] = True
+    assert n == total and 0 < we.sum() < we.size
+    assert np.array_equal(fe, we) and np.array_equal(fr, wr)
