@@ -54,10 +54,24 @@ struct TileShape {
     static constexpr int kLdsFloats = NPL * kKL * kLP + NC * kKL * PG;
 };
 
-template <int MODEL, int P, bool OWNER_POS, int RO, bool MF>
-__device__ __forceinline__ void bwd_tile_body(const TileArgs &a, int lid, float *smem)
+// Width of the narrow last column tile: klen % 64 when that is between 1 and 16, else 0 (rows are
+// then covered by 64-column tiles alone).
+__host__ __device__ inline int narrow_cols(int klen)
 {
-    constexpr int TO = 16 * RO;
+    const int rem = klen % kTI;
+    return rem > 0 && rem <= 16 ? rem : 0;
+}
+
+// NARROW: the tile covers the last 16 columns of rows whose width leaves a remainder of at most 16
+// over the 64-column tiles.  A 64-column tile there would keep 12 of its 16 column lanes idle;
+// instead the column lanes are regrouped as 4 column groups x 4 owner sub-tiles and every thread
+// owns one row (RO_ = 1) of its sub-tile, so all 256 threads work on the 64 owners x 16 columns.
+template <int MODEL, int P, bool OWNER_POS, int RO, bool MF, bool NARROW = false>
+__device__ __forceinline__ void bwd_tile_body(const TileArgs &a, int lid, float *smem, int col_base = 0)
+{
+    static_assert(!(NARROW && MF), "the matrix-core loop has no narrow form");
+    constexpr int RO_ = NARROW ? 1 : RO;           // owners per thread
+    constexpr int TO = NARROW ? 64 : 16 * RO;      // owners per tile
     constexpr bool kRot = MODEL == KGE_ROTATE, kTH = MODEL == KGE_TRANSH;
     constexpr bool kDot = MODEL == KGE_DISTMULT || MODEL == KGE_COMPLEX || MODEL == KGE_TRANSF;  // score = query . t' (+ const)
     constexpr bool kMf = kDot && MF;  // the sum over loopers on the matrix cores (else on the vector ALUs)
@@ -69,6 +83,7 @@ __device__ __forceinline__ void bwd_tile_body(const TileArgs &a, int lid, float 
     constexpr int PG = TO + 4;
     constexpr int SL = kKL / 16;                        // looper float4 per thread per plane
     constexpr int CPT = (TO * kKL / 4 + 255) / 256;     // coefficient float4 per thread per plane
+    static_assert(!NARROW || RO == 4, "narrow tiles share the 64-owner LDS layout");
 
     float(*sL)[kKL][kLP] = reinterpret_cast<float(*)[kKL][kLP]>(smem);
     float(*sG)[kKL][PG] = reinterpret_cast<float(*)[kKL][PG]>(smem + NPL * kKL * kLP);
@@ -78,19 +93,25 @@ __device__ __forceinline__ void bwd_tile_body(const TileArgs &a, int lid, float 
     const int klen = pair_len<MODEL>(d);
     const int n_own = OWNER_POS ? a.C : a.N, n_loop = OWNER_POS ? a.N : a.C;
     int c, tile_y, tile_x;
-    if (!xcd_tile(lid, (klen + kTI - 1) / kTI, (n_own + TO - 1) / TO, a.n_chunks, c, tile_y, tile_x)) return;
-    const int col = tile_x * kTI + tx * 4;
+    // wide tiles cover the columns [0, tiles_x * 64); a narrow tile the 16 columns from col_base on
+    constexpr bool kHasNarrow = RO == 4 && !MF;  // launches of this shape hand a short remainder to narrow tiles
+    const int wide_tiles_x = (kHasNarrow && narrow_cols(klen)) ? klen / kTI : (klen + kTI - 1) / kTI;
+    if (!xcd_tile(lid, NARROW ? 1 : wide_tiles_x, (n_own + TO - 1) / TO, a.n_chunks, c, tile_y, tile_x)) return;
+    const int scol = (NARROW ? col_base : tile_x * kTI) + tx * 4;            // columns this thread stages
+    const int ctx = NARROW ? (tx & 3) : tx;                                  // column lane it computes
+    const int col = (NARROW ? col_base : tile_x * kTI) + ctx * 4;            // columns it owns
     const int ot0 = tile_y * TO;
+    auto orow = [&](int o) { return NARROW ? (tx >> 2) * 16 + ty : ty * RO_ + o; };  // owner row inside the tile
     const bool vec = a.vec != 0;
 
     // ---- owners: registers -----------------------------------------------------------
-    float4 own[NPO][RO];
-    float alo[RO];
+    float4 own[NPO][RO_];
+    float alo[RO_];
     auto load_owners = [&](auto vtag) {
     constexpr bool VEC = decltype(vtag)::value;
 #pragma unroll
-    for (int o = 0; o < RO; ++o) {
-        const int ol = ot0 + ty * RO + o;
+    for (int o = 0; o < RO_; ++o) {
+        const int ol = ot0 + orow(o);
         const int lim = ol < n_own ? klen : 0;
         const int oc = ol < n_own ? ol : n_own - 1;
         alo[o] = 0.0f;
@@ -115,11 +136,11 @@ __device__ __forceinline__ void bwd_tile_body(const TileArgs &a, int lid, float 
     if (vec) load_owners(std::true_type{});
     else load_owners(std::false_type{});
 
-    float4 acc[NOUT][RO];
+    float4 acc[NOUT][RO_];
 #pragma unroll
     for (int q = 0; q < NOUT; ++q)
 #pragma unroll
-        for (int o = 0; o < RO; ++o) acc[q][o] = zero4();
+        for (int o = 0; o < RO_; ++o) acc[q][o] = zero4();
 
     // DistMult / ComplEx: the sum over loopers is a plain matrix product, coefficients (owners x
     // loopers) times looper rows (loopers x columns), so it runs on the matrix cores
@@ -175,17 +196,17 @@ __device__ __forceinline__ void bwd_tile_body(const TileArgs &a, int lid, float 
             const int lim = ll < n_loop ? klen : 0;
             if constexpr (OWNER_POS) {
                 const float *pt = a.ent + li0[s] * (int64_t)d;
-                rraw[s][0] = ld4_raw<VEC>(pt, col, lim);
-                if constexpr (NPL == 2) rraw[s][1] = ld4_raw<VEC>(pt + half, col, lim);
+                rraw[s][0] = ld4_raw<VEC>(pt, scol, lim);
+                if constexpr (NPL == 2) rraw[s][1] = ld4_raw<VEC>(pt + half, scol, lim);
             } else {
                 const int64_t b = (int64_t)c * a.C + (ll < n_loop ? ll : n_loop - 1);
                 const float *ph = a.ent + li0[s] * (int64_t)d, *pr = a.rel + li1[s] * (int64_t)a.rel_dim;
                 const float *pw = kTH ? a.aux + li1[s] * (int64_t)d : nullptr;
                 const float *pq = kRot ? a.query + b * (int64_t)d : nullptr;
                 if constexpr (kDefer) {
-                    load_query_raw<MODEL, VEC>(ph, pr, pw, pq, col, lim, half, rraw[s]);
+                    load_query_raw<MODEL, VEC>(ph, pr, pw, pq, scol, lim, half, rraw[s]);
                 } else {
-                    load_query<MODEL, VEC>(ph, pr, pw, lal[s], col, lim, half, rraw[s][0], rraw[s][NRAW - 1], pq, a.rsign);
+                    load_query<MODEL, VEC>(ph, pr, pw, lal[s], scol, lim, half, rraw[s][0], rraw[s][NRAW - 1], pq, a.rsign);
                 }
             }
         }
@@ -246,7 +267,7 @@ __device__ __forceinline__ void bwd_tile_body(const TileArgs &a, int lid, float 
                 if constexpr (NPL == 2) q1 = rraw[s][NRAW - 1];
             } else {
                 const int ll = l0 + ty + 16 * s;
-                combine_query<MODEL, VEC>(rraw[s], 0.0f, col, ll < n_loop ? klen : 0, half, a.rsign, q0, q1);
+                combine_query<MODEL, VEC>(rraw[s], 0.0f, scol, ll < n_loop ? klen : 0, half, a.rsign, q0, q1);
             }
             *reinterpret_cast<float4 *>(&sL[0][ty + 16 * s][tx * 4]) = q0;
             if constexpr (NPL == 2) *reinterpret_cast<float4 *>(&sL[1][ty + 16 * s][tx * 4]) = q1;
@@ -322,19 +343,19 @@ __device__ __forceinline__ void bwd_tile_body(const TileArgs &a, int lid, float 
                         macc[e] = __builtin_amdgcn_mfma_f32_16x16x4f32(av, bv[e], macc[e], 0, 0, 0);
                 }
         }
-        float4 sacc[NOUT][RO];
+        float4 sacc[NOUT][RO_];
 #pragma unroll
         for (int q = 0; q < NOUT; ++q)
 #pragma unroll
-            for (int o = 0; o < RO; ++o) sacc[q][o] = zero4();
+            for (int o = 0; o < RO_; ++o) sacc[q][o] = zero4();
 #pragma unroll 4
         for (int l = 0; l < (kMf ? 0 : kKL); ++l) {
             float4 lv[NPL];
 #pragma unroll
-            for (int pl = 0; pl < NPL; ++pl) lv[pl] = *reinterpret_cast<const float4 *>(&sL[pl][l][tx * 4]);
+            for (int pl = 0; pl < NPL; ++pl) lv[pl] = *reinterpret_cast<const float4 *>(&sL[pl][l][ctx * 4]);
 #pragma unroll
-            for (int o = 0; o < RO; ++o) {
-                const float g = sG[0][l][ty * RO + o];
+            for (int o = 0; o < RO_; ++o) {
+                const float g = sG[0][l][orow(o)];
                 const float *lvp = reinterpret_cast<const float *>(&lv[0]);
                 const float *lv1p = reinterpret_cast<const float *>(&lv[NPL - 1]);
                 const float *o0p = reinterpret_cast<const float *>(&own[0][o]);
@@ -365,15 +386,17 @@ __device__ __forceinline__ void bwd_tile_body(const TileArgs &a, int lid, float 
                         a1p[e] = fmaf(k, ui, a1p[e]);
                     }
                 } else if constexpr (kTH) {
-                    const float cc = sG[1][l][ty * RO + o], ee = sG[2][l][ty * RO + o];
+                    const float cc = sG[1][l][orow(o)], ee = sG[2][l][orow(o)];
                     if constexpr (OWNER_POS) {
-                        const float sdk = alo[o] - cc;  // w.(h - t'_k)
+                        // q = g phi(u) goes into a0 and, times -w.(h - t'_k), into a1: with the two
+                        // coefficients formed once per pair, phi(u) feeds two multiply-adds directly
+                        const float gk = -(alo[o] - cc) * g;
 #pragma unroll
                         for (int e = 0; e < 4; ++e) {
                             const float u = fmaf(cc, o1p[e], o0p[e] - lvp[e]);
-                            const float q = g * (P == 1 ? fast_sgn(u) : u);
-                            a0p[e] += q;
-                            a1p[e] = fmaf(ee, lvp[e], fmaf(-sdk, q, a1p[e]));
+                            const float ph = P == 1 ? fast_sgn(u) : u;
+                            a0p[e] = fmaf(g, ph, a0p[e]);
+                            a1p[e] = fmaf(ee, lvp[e], fmaf(gk, ph, a1p[e]));
                         }
                     } else {
 #pragma unroll
@@ -389,7 +412,7 @@ __device__ __forceinline__ void bwd_tile_body(const TileArgs &a, int lid, float 
 #pragma unroll
         for (int q = 0; q < NOUT; ++q)
 #pragma unroll
-            for (int o = 0; o < RO; ++o) acc[q][o] = add4(acc[q][o], sacc[q][o]);
+            for (int o = 0; o < RO_; ++o) acc[q][o] = add4(acc[q][o], sacc[q][o]);
         __syncthreads();
     }
 
@@ -415,8 +438,8 @@ __device__ __forceinline__ void bwd_tile_body(const TileArgs &a, int lid, float 
         return;
     }
 #pragma unroll
-    for (int o = 0; o < RO; ++o) {
-        const int ol = ot0 + ty * RO + o;
+    for (int o = 0; o < RO_; ++o) {
+        const int ol = ot0 + orow(o);
         if (ol >= n_own) continue;
         const int64_t row = OWNER_POS ? (int64_t)c * a.C + ol : (int64_t)c * a.N + ol;
         float *dst = a.out0 + row * (int64_t)d;
@@ -429,20 +452,43 @@ __device__ __forceinline__ void bwd_tile_body(const TileArgs &a, int lid, float 
 // Both orientations in ONE launch: the first `grid_head` workgroups own positives (outputs
 // g0 / g1), the rest own negatives (output occ_neg).  The two halves are independent, and
 // together they fill the GPU better than either alone when the batch is small.
+// Workgroup ranges of a launch, in order: the inspector's riders, wide tiles owning positives,
+// wide tiles owning negatives, then (64-owner vector-ALU launches only, when the row width leaves
+// a remainder of at most 16 columns) narrow tiles owning positives and narrow tiles owning negatives.
+struct TileGrid {
+    int head, neg, narrow_head, narrow_neg;
+};
+
 template <int MODEL, int P, int RO, bool MF>
 __global__ __launch_bounds__(256, KGE_TILE_OCC) void bwd_tile_kernel(TileArgs a, float *g0, float *g1, float *occ_neg,
-                                                                     int grid_head, FusedInsp fi)
+                                                                     TileGrid grid, FusedInsp fi)
 {
     extern __shared__ __align__(16) char dyn_smem[];  // tile_lds_bytes<MODEL, RO>() or the inspector's need
     if (fused_insp_block(fi, reinterpret_cast<uint32_t *>(dyn_smem))) return;
     float *smem = reinterpret_cast<float *>(dyn_smem);
-    const int lid = (int)blockIdx.x - fi.blocks;
-    if (lid < grid_head) {
+    int lid = (int)blockIdx.x - fi.blocks;
+    if (lid < grid.head) {
         a.out0 = g0, a.out1 = g1;
         bwd_tile_body<MODEL, P, true, RO, MF>(a, lid, smem);
-    } else {
+        return;
+    }
+    lid -= grid.head;
+    if (lid < grid.neg) {
         a.out0 = occ_neg, a.out1 = nullptr;
-        bwd_tile_body<MODEL, P, false, RO, MF>(a, lid - grid_head, smem);
+        bwd_tile_body<MODEL, P, false, RO, MF>(a, lid, smem);
+        return;
+    }
+    if constexpr (RO == 4 && !MF) {
+        lid -= grid.neg;
+        const int klen = pair_len<MODEL>(a.d);
+        const int col_base = (klen / kTI) * kTI;
+        if (lid < grid.narrow_head) {
+            a.out0 = g0, a.out1 = g1;
+            bwd_tile_body<MODEL, P, true, RO, MF, true>(a, lid, smem, col_base);
+        } else {
+            a.out0 = occ_neg, a.out1 = nullptr;
+            bwd_tile_body<MODEL, P, false, RO, MF, true>(a, lid - grid.narrow_head, smem, col_base);
+        }
     }
 }
 
@@ -462,6 +508,8 @@ static int launch_tiles(TileArgs a, float *g0, float *g1, float *occ_neg, int64_
 {
     const int klen = MODEL == KGE_ROTATE ? a.d / 2 : a.d;
     const int64_t gx = ceil_div(klen, kTI);
+    const bool narrow = narrow_cols(klen) > 0;       // the last 1..16 columns go to narrow tiles (64-owner VALU launches)
+    const int64_t gxw = narrow ? klen / kTI : gx;    // wide column tiles of such a launch
     const int64_t big = gx * (ceil_div(a.C, 64) + ceil_div(a.N, 64)) * n_chunks;
     // the size rule follows launch_neg_mp (see there)
     constexpr bool kDotModel = MODEL == KGE_DISTMULT || MODEL == KGE_COMPLEX || MODEL == KGE_TRANSF;
@@ -472,21 +520,23 @@ static int launch_tiles(TileArgs a, float *g0, float *g1, float *occ_neg, int64_
             const unsigned gh = xcd_grid(gx, ceil_div(a.C, 64), n_chunks), gn = xcd_grid(gx, ceil_div(a.N, 64), n_chunks);
             const size_t lds = tile_lds_bytes<MODEL, 4>(fi);
             hipLaunchKernelGGL((bwd_tile_kernel<MODEL, P, 4, true>), dim3(gh + gn + fi.blocks), dim3(256), lds, st, a,
-                               g0, g1, occ_neg, (int)gh, fi);
+                               g0, g1, occ_neg, TileGrid{(int)gh, (int)gn, 0, 0}, fi);
             KGE_CHECK_LAUNCH();
             return KGE_OK;
         }
     }
     if (big >= 1024) {
-        const unsigned gh = xcd_grid(gx, ceil_div(a.C, 64), n_chunks), gn = xcd_grid(gx, ceil_div(a.N, 64), n_chunks);
+        const unsigned gh = xcd_grid(gxw, ceil_div(a.C, 64), n_chunks), gn = xcd_grid(gxw, ceil_div(a.N, 64), n_chunks);
+        const unsigned nh = narrow ? xcd_grid(1, ceil_div(a.C, 64), n_chunks) : 0;
+        const unsigned nn = narrow ? xcd_grid(1, ceil_div(a.N, 64), n_chunks) : 0;
         const size_t lds = tile_lds_bytes<MODEL, 4>(fi);
-        hipLaunchKernelGGL((bwd_tile_kernel<MODEL, P, 4, false>), dim3(gh + gn + fi.blocks), dim3(256), lds, st, a, g0, g1,
-                           occ_neg, (int)gh, fi);
+        hipLaunchKernelGGL((bwd_tile_kernel<MODEL, P, 4, false>), dim3(gh + gn + nh + nn + fi.blocks), dim3(256), lds, st,
+                           a, g0, g1, occ_neg, TileGrid{(int)gh, (int)gn, (int)nh, (int)nn}, fi);
     } else {
         const unsigned gh = xcd_grid(gx, ceil_div(a.C, 32), n_chunks), gn = xcd_grid(gx, ceil_div(a.N, 32), n_chunks);
         const size_t lds = tile_lds_bytes<MODEL, 2>(fi);
         hipLaunchKernelGGL((bwd_tile_kernel<MODEL, P, 2, false>), dim3(gh + gn + fi.blocks), dim3(256), lds, st, a, g0, g1,
-                           occ_neg, (int)gh, fi);
+                           occ_neg, TileGrid{(int)gh, (int)gn, 0, 0}, fi);
     }
     KGE_CHECK_LAUNCH();
     return KGE_OK;

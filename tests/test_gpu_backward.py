@@ -11,7 +11,7 @@ pytestmark = pytest.mark.gpu
 NEG_MODELS = ["TransE", "TransH", "DistMult", "ComplEx", "RotatE", "TransF"]
 
 
-def run_both(oracle, w, seed=0, use_pos=True, use_neg=True, pair_sums="matrix_cores"):
+def run_both(oracle, w, seed=0, use_pos=True, use_neg=True, pair_sums="matrix_cores", fast=False):
     a = w.arrays
     rng = np.random.default_rng(seed)
     dpos = rng.standard_normal(w.batch).astype(np.float32) if use_pos else None
@@ -24,7 +24,7 @@ def run_both(oracle, w, seed=0, use_pos=True, use_neg=True, pair_sums="matrix_co
     g = m.backward(fw, None if dpos is None else torch.from_numpy(dpos).to(dev),
                    None if dneg is None else torch.from_numpy(dneg).to(dev))
     ref = oracle.backward(w.model, a["E"], a["R"], a["A"], a["h"], a["r"], a["t"], a.get("neg"), w.chunk,
-                          dpos, dneg, p=w.norm_p)
+                          dpos, dneg, p=w.norm_p, fast=fast)
     return g, ref
 
 
@@ -64,6 +64,17 @@ def test_positive_only_gradients(oracle, model):
                               ent_zipf=1.2, seed=3)
     g, ref = run_both(oracle, w, seed=2)
     compare(g, ref, f"{model} positives only")
+
+
+@pytest.mark.parametrize("model,p,dim", [("TransE", 1, 72), ("TransH", 2, 80), ("TransH", 1, 76), ("RotatE", 2, 152)])
+def test_row_widths_that_end_in_a_narrow_column_tile(oracle, model, p, dim):
+    """Batches large enough for the 64-owner gradient tiles whose row width leaves 1..16 columns over the
+    64-column tiles (72 = 64 + 8, 80 = 64 + 16, 76 = 64 + 12, RotatE 76 complex elements): those columns are
+    computed by the narrow tiles, every other column by the wide ones."""
+    w = synth.custom_workload(model, n_ent=3000, n_rel=11, dim=dim, batch=128 * 256, chunk=128, n_neg=128, norm_p=p,
+                              sigma=0.2, gamma=4.0, ent_zipf=1.1, seed=dim + p, lattice=(p == 1))
+    g, ref = run_both(oracle, w, seed=5, fast="omp")
+    compare(g, ref, f"{model} p={p} dim={dim}", outliers=(1e-5, 4.0) if model == "RotatE" else None)
 
 
 def test_missing_upstream_gradients_mean_zero(oracle):
