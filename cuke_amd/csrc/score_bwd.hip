@@ -76,6 +76,10 @@ __device__ __forceinline__ void bwd_tile_body(const TileArgs &a, int lid, float 
     constexpr bool kDot = MODEL == KGE_DISTMULT || MODEL == KGE_COMPLEX || MODEL == KGE_TRANSF;  // score = query . t' (+ const)
     constexpr bool kMf = kDot && MF;  // the sum over loopers on the matrix cores (else on the vector ALUs)
     constexpr bool kL2 = (MODEL == KGE_TRANSE || kTH) && P == 2;
+    // L1 translation models: owner and looper rows carry the factor 2^100, so the sign of a residual
+    // element is a single clamp (sgn_of_scaled, tile_common.hpp); the coefficient that multiplies a
+    // scaled row (TransH: e) carries 2^-100
+    constexpr bool kSc = (MODEL == KGE_TRANSE || kTH) && P == 1;
     constexpr int NPL = (kRot || (kTH && !OWNER_POS)) ? 2 : 1;  // looper planes in LDS
     constexpr int NPO = (kRot || (kTH && OWNER_POS)) ? 2 : 1;   // owner planes in registers
     constexpr int NC = kTH ? 3 : 1;                             // coefficient planes: g~, c, e
@@ -130,6 +134,10 @@ __device__ __forceinline__ void bwd_tile_body(const TileArgs &a, int lid, float 
             const float *pt = a.ent + a.neg[(int64_t)c * a.N + oc] * (int64_t)d;
             own[0][o] = kDot ? zero4() : ld4<VEC>(pt, col, lim);
             if constexpr (NPO == 2) own[1][o] = ld4<VEC>(pt + half, col, lim);
+        }
+        if constexpr (kSc) {
+#pragma unroll
+            for (int q = 0; q < NPO; ++q) own[q][o] = scale4(own[q][o], kSgnScale);
         }
     }
     };
@@ -241,7 +249,7 @@ __device__ __forceinline__ void bwd_tile_body(const TileArgs &a, int lid, float 
                     g.z = sc.z > 0.0f ? g.z / sc.z : 0.0f;
                     g.w = sc.w > 0.0f ? g.w / sc.w : 0.0f;
                 } else {
-                    craw[2][s] = mul4(craw[0][s], craw[2][s]);
+                    craw[2][s] = mul4(scale4(craw[0][s], kSgnUnscale), craw[2][s]);  // kSc: multiplies a scaled row
                 }
             }
         }
@@ -269,6 +277,7 @@ __device__ __forceinline__ void bwd_tile_body(const TileArgs &a, int lid, float 
                 const int ll = l0 + ty + 16 * s;
                 combine_query<MODEL, VEC>(rraw[s], 0.0f, scol, ll < n_loop ? klen : 0, half, a.rsign, q0, q1);
             }
+            if constexpr (kSc) q0 = scale4(q0, kSgnScale), q1 = scale4(q1, kSgnScale);
             *reinterpret_cast<float4 *>(&sL[0][ty + 16 * s][tx * 4]) = q0;
             if constexpr (NPL == 2) *reinterpret_cast<float4 *>(&sL[1][ty + 16 * s][tx * 4]) = q1;
         }
@@ -368,8 +377,8 @@ __device__ __forceinline__ void bwd_tile_body(const TileArgs &a, int lid, float 
                 } else if constexpr (MODEL == KGE_TRANSE) {
 #pragma unroll
                     for (int e = 0; e < 4; ++e) {
-                        const float u = OWNER_POS ? o0p[e] - lvp[e] : lvp[e] - o0p[e];  // a - t'
-                        const float ph = P == 1 ? fast_sgn(u) : u;
+                        const float u = OWNER_POS ? o0p[e] - lvp[e] : lvp[e] - o0p[e];  // a - t' (P == 1: times 2^100)
+                        const float ph = P == 1 ? sgn_of_scaled(u) : u;
                         a0p[e] = OWNER_POS ? fmaf(g, ph, a0p[e]) : fmaf(-g, ph, a0p[e]);
                     }
                 } else if constexpr (kRot) {
@@ -394,7 +403,7 @@ __device__ __forceinline__ void bwd_tile_body(const TileArgs &a, int lid, float 
 #pragma unroll
                         for (int e = 0; e < 4; ++e) {
                             const float u = fmaf(cc, o1p[e], o0p[e] - lvp[e]);
-                            const float ph = P == 1 ? fast_sgn(u) : u;
+                            const float ph = P == 1 ? sgn_of_scaled(u) : u;
                             a0p[e] = fmaf(g, ph, a0p[e]);
                             a1p[e] = fmaf(ee, lvp[e], fmaf(gk, ph, a1p[e]));
                         }
@@ -402,8 +411,8 @@ __device__ __forceinline__ void bwd_tile_body(const TileArgs &a, int lid, float 
 #pragma unroll
                         for (int e = 0; e < 4; ++e) {
                             const float u = fmaf(cc, lv1p[e], lvp[e] - o0p[e]);
-                            const float q = g * (P == 1 ? fast_sgn(u) : u);
-                            a0p[e] = fmaf(ee, lv1p[e], a0p[e] - q);
+                            const float ph = P == 1 ? sgn_of_scaled(u) : u;
+                            a0p[e] = fmaf(ee, lv1p[e], fmaf(-g, ph, a0p[e]));
                         }
                     }
                 }

@@ -52,10 +52,11 @@ __device__ __forceinline__ void pair_elem(float &acc, float &acc2, float a0, flo
         else acc = fmaf(u, u, acc);
     } else if constexpr (MODEL == KGE_TRANSH) {
         // a0 = h + r - (w.h) w, a1 = w, c = w . t'
+        // (P == 1 with SAVE: a0, a1 and t0 carry the factor 2^100, see sgn_of_scaled)
         const float u = fmaf(c, a1, a0 - t0);
         if constexpr (P == 1) acc += fabsf(u);
         else acc = fmaf(u, u, acc);
-        if constexpr (SAVE) acc2 = fmaf(P == 1 ? fast_sgn(u) : u, a1, acc2);
+        if constexpr (SAVE) acc2 = fmaf(P == 1 ? sgn_of_scaled(u) : u, a1, acc2);
     } else if constexpr (MODEL == KGE_ROTATE) {
         const float ur = a0 - t0, ui = a1 - t1;
         acc += __builtin_amdgcn_sqrtf(fmaf(ur, ur, ui * ui));
@@ -72,6 +73,9 @@ __global__ __launch_bounds__(256, KGE_TILE_OCC) void score_neg_kernel(NegArgs a,
     constexpr int NPT = MODEL == KGE_ROTATE ? 2 : 1;
     constexpr int SB = TB / 32, SN = TN / 32;  // float4 per thread per plane per step
     constexpr int NPASS = MODEL == KGE_TRANSH ? 2 : 1;
+    // TransH, L1, with the sign sums saved for backward: the second sweep's rows are staged times
+    // 2^100 so that the sign of a residual element is a single clamp (tile_common.hpp)
+    constexpr bool kScaled = MODEL == KGE_TRANSH && P == 1 && SAVE;
     static_assert(TB % 32 == 0 && TN % 32 == 0, "tile rows are staged 32 at a time");
 
     float(*sA)[TB][kLDW] = reinterpret_cast<float(*)[TB][kLDW]>(dyn_smem);
@@ -156,12 +160,14 @@ __global__ __launch_bounds__(256, KGE_TILE_OCC) void score_neg_kernel(NegArgs a,
             for (int q = 0; q < SB; ++q)
 #pragma unroll
                 for (int pl = 0; pl < NPA; ++pl)
-                    *reinterpret_cast<float4 *>(&sA[pl][srow + 32 * q][scol]) = ra[pl][q];
+                    *reinterpret_cast<float4 *>(&sA[pl][srow + 32 * q][scol]) =
+                        kScaled ? scale4(ra[pl][q], kSgnScale) : ra[pl][q];
 #pragma unroll
             for (int q = 0; q < SN; ++q)
 #pragma unroll
                 for (int pl = 0; pl < NPT; ++pl)
-                    *reinterpret_cast<float4 *>(&sT[pl][srow + 32 * q][scol]) = rt[pl][q];
+                    *reinterpret_cast<float4 *>(&sT[pl][srow + 32 * q][scol]) =
+                        kScaled ? scale4(rt[pl][q], kSgnScale) : rt[pl][q];
             __syncthreads();
             if (s + 1 < nslice) load_slice((s + 1) * kKD, pass);
 #pragma unroll
@@ -292,6 +298,7 @@ __global__ __launch_bounds__(256, KGE_TILE_OCC) void score_neg_kernel(NegArgs a,
             const int kl = kt0 + tx + 16 * k;
             if (kl >= a.N) continue;
             float s = acc[i][k];
+            if constexpr (kScaled) s *= kSgnUnscale, acc2[i][k] *= kSgnUnscale;
             if constexpr (MODEL == KGE_TRANSE || MODEL == KGE_TRANSH) s = P == 2 ? sqrtf(s) : s;
             if constexpr (MODEL == KGE_ROTATE) s = a.gamma - s;
             if constexpr (MODEL == KGE_TRANSF) s -= a.rsign * a.side_pos[(int64_t)c * a.C + bl];

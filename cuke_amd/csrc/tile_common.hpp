@@ -69,6 +69,16 @@ __device__ __forceinline__ float fast_sgn(float u)
     return __builtin_amdgcn_fmed3f(u * 0x1p100f, -1.0f, 1.0f);
 }
 
+// The multiply of fast_sgn() can be paid once per staged row element instead of once per pair
+// element: scaling by a power of two commutes with every fp32 rounding (no overflow: table values
+// times 2^100 stay far below 2^127), so a residual formed from rows that carry the factor 2^100 is
+// exactly 2^100 times the residual of the plain rows, and its sign is one clamp away.  The L1 tile
+// kernels of TransE / TransH stage their rows scaled; sums of |U| and of sign(U) * W are scaled
+// back once per pair, and coefficients that multiply a scaled row carry 2^-100.
+constexpr float kSgnScale = 0x1p100f, kSgnUnscale = 0x1p-100f;
+__device__ __forceinline__ float sgn_of_scaled(float U) { return __builtin_amdgcn_fmed3f(U, -1.0f, 1.0f); }
+__device__ __forceinline__ float4 scale4(float4 v, float s) { return make_float4(v.x * s, v.y * s, v.z * s, v.w * s); }
+
 // reduction length of the pair kernels: complex pairs for RotatE, floats otherwise
 template <int MODEL>
 __device__ __forceinline__ int pair_len(int d)
