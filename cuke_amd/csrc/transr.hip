@@ -48,6 +48,8 @@ struct TilePlan {
     int32_t *num_tiles;  // [1]
     int32_t *tile_seg;   // [max_tiles] group (unique-relation index)
     int32_t *tile_p0;    // [max_tiles] first sorted position
+    int32_t *tile_end;   // [max_tiles] end of the tile's group in sorted positions (GEMM plan only, else null)
+    int32_t *tile_rid;   // [max_tiles] relation id of the group (GEMM plan only, else null)
     // groups longer than one tile ("split" groups, used by the dM kernel): every tile of such
     // a group writes a partial result to slot tile_part[tile]; -1 for unsplit groups
     int32_t *tile_part;   // [max_tiles] or null
@@ -79,7 +81,8 @@ __device__ int block_inclusive_scan_1024(int v, int *s_scan)
 // One workgroup per plan: block 0 builds `plan0` with tiles of `tile0` positions, block 1 (when
 // launched) `plan1` with `tile1`.
 __global__ __launch_bounds__(1024) void transr_plan_kernel(const int32_t *num_unique, const int32_t *seg_offsets,
-                                                          TilePlan plan0, int tile0, TilePlan plan1, int tile1)
+                                                          const int64_t *unique_ids, TilePlan plan0, int tile0,
+                                                          TilePlan plan1, int tile1)
 {
     const TilePlan &plan = blockIdx.x == 0 ? plan0 : plan1;
     const int tile = blockIdx.x == 0 ? tile0 : tile1;
@@ -90,10 +93,11 @@ __global__ __launch_bounds__(1024) void transr_plan_kernel(const int32_t *num_un
     __syncthreads();
     for (int base = 0; base < U; base += 1024) {
         const int g = base + threadIdx.x;
-        int s0 = 0, cnt = 0;
+        int s0 = 0, s1 = 0, cnt = 0, rid = 0;
         if (g < U) {
-            s0 = seg_offsets[g];
-            cnt = (seg_offsets[g + 1] - s0 + tile - 1) / tile;
+            s0 = seg_offsets[g], s1 = seg_offsets[g + 1];
+            rid = (int)unique_ids[g];
+            cnt = (s1 - s0 + tile - 1) / tile;
         }
         const int inc_t = block_inclusive_scan_1024(cnt, s_scan);
         const int start = s_carry[0] + inc_t - cnt;
@@ -115,6 +119,7 @@ __global__ __launch_bounds__(1024) void transr_plan_kernel(const int32_t *num_un
         for (int q = 0; q < cnt; ++q) {
             plan.tile_seg[start + q] = g;
             plan.tile_p0[start + q] = s0 + q * tile;
+            if (plan.tile_end) plan.tile_end[start + q] = s1, plan.tile_rid[start + q] = rid;
             if (plan.tile_part) plan.tile_part[start + q] = pstart >= 0 ? pstart + q : -1;
         }
         __syncthreads();
@@ -376,23 +381,27 @@ static size_t thin_dx_lds_bytes(int d) { return sizeof(float) * 4 * (size_t)d; }
 // in flight at each step, which turns the prefetch ring into a depth of one.
 //   MODE 0/1: B[k][j] = M[k][n0 + 4 li + e], one float4 per k row per lane;
 //   MODE 2:   B[k][j] = M[n0 + 16 e + li][k], a lane's float4 along k serves the four steps.
-template <int MODE, bool TWO>
-__device__ __forceinline__ void gemm_sweep(const float *M, const float *sX, int pitch, int d, int nq, int n0,
-                                           int wcols, int li, int kk, floatx4 (&acc_lo)[4], floatx4 (&acc_hi)[4])
-{
+template <int MODE>
+struct BLoader {
     const float *base[4];
-    if constexpr (MODE != 2) {
-        const int col = n0 + (4 * li < wcols ? 4 * li : 0);
+    int d, nq, kk;
+    __device__ __forceinline__ void init(const float *M, int d_, int nq_, int n0, int wcols, int li, int kk_)
+    {
+        d = d_, nq = nq_, kk = kk_;
+        if constexpr (MODE != 2) {
+            const int col = n0 + (4 * li < wcols ? 4 * li : 0);
 #pragma unroll
-        for (int s = 0; s < 4; ++s) base[s] = M + col;
-    } else {
+            for (int s = 0; s < 4; ++s) base[s] = M + col;
+        } else {
 #pragma unroll
-        for (int e = 0; e < 4; ++e) {
-            const int col = 16 * e + li;
-            base[e] = M + (int64_t)(n0 + (col < wcols ? col : 0)) * d;
+            for (int e = 0; e < 4; ++e) {
+                const int col = 16 * e + li;
+                base[e] = M + (int64_t)(n0 + (col < wcols ? col : 0)) * d;
+            }
         }
     }
-    auto loadb = [&](int q, float4 *dst) {
+    __device__ __forceinline__ void load(int q, float4 *dst) const
+    {
         q = q < nq ? q : nq - 1;
         if constexpr (MODE != 2) {
 #pragma unroll
@@ -405,20 +414,34 @@ __device__ __forceinline__ void gemm_sweep(const float *M, const float *sX, int 
 #pragma unroll
             for (int e = 0; e < 4; ++e) dst[e] = *reinterpret_cast<const float4 *>(base[e] + (k < d ? k : d - 4));
         }
-    };
-    // Ring of kRing slots: step qq consumes slot qq % kRing and first refills the slot consumed one
-    // step earlier with superstep qq + kRing - 1, so kRing - 1 supersteps are always in flight and
-    // the loads are issued ahead of the matrix-core work of the step (pinned by the scheduling
-    // barrier; left alone the compiler sinks them below it and the ring degenerates to depth 1).
-    float4 ring[kRing][4];
+    }
+};
+
+// Ring of kRing slots: step qq consumes slot qq % kRing and first refills the slot consumed one
+// step earlier with superstep qq + kRing - 1, so kRing - 1 supersteps are always in flight and
+// the loads are issued ahead of the matrix-core work of the step (pinned by the scheduling
+// barrier; left alone the compiler sinks them below it and the ring degenerates to depth 1).
+// ring_prime() issues the first kRing - 1 supersteps; a tile calls it before it stages its left
+// operand (the projection only depends on the tile's relation), so those loads fly during the
+// index chain and the row gathers of the staging.
+template <int MODE>
+__device__ __forceinline__ void ring_prime(const BLoader<MODE> &bl, float4 (&ring)[kRing][4])
+{
 #pragma unroll
-    for (int u = 0; u + 1 < kRing; ++u) loadb(u, ring[u]);
+    for (int u = 0; u + 1 < kRing; ++u) bl.load(u, ring[u]);
+}
+
+template <int MODE, bool TWO>
+__device__ __forceinline__ void gemm_sweep(const BLoader<MODE> &bl, float4 (&ring)[kRing][4], const float *sX, int pitch,
+                                           int li, int kk, floatx4 (&acc_lo)[4], floatx4 (&acc_hi)[4])
+{
+    const int nq = bl.nq;
     const float *xlo = sX + li * pitch + 4 * kk, *xhi = sX + (16 + li) * pitch + 4 * kk;
     for (int q = 0; q < nq; q += kRing) {
 #pragma unroll
         for (int u = 0; u < kRing; ++u) {
             const int qq = q + u;
-            loadb(qq + kRing - 1, ring[(u + kRing - 1) % kRing]);
+            bl.load(qq + kRing - 1, ring[(u + kRing - 1) % kRing]);
             __builtin_amdgcn_sched_barrier(0);
             float4 bc[4];
 #pragma unroll
@@ -488,12 +511,33 @@ __global__ __launch_bounds__(256, KGE_TR_OCC) void transr_gemm_kernel(GemmArgs a
     float *sX = lds;                 // [kTM][pitch]
     float *sRed = lds + kTM * pitch; // [4][kTM]
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int g = a.plan.tile_seg[tile], p0 = a.plan.tile_p0[tile];
-    const int seg_end = a.seg_offsets[g + 1];
+    // everything the tile needs to know comes from the plan in one round trip
+    const int p0 = a.plan.tile_p0[tile], seg_end = a.plan.tile_end[tile];
+    const int64_t rid = a.plan.tile_rid[tile];
     const int rows = seg_end - p0 < kTM ? seg_end - p0 : kTM;
     if (rows <= kThin) return;  // streamed by a thin workgroup
-    const int64_t rid = a.unique_ids[g];
     const float *M = a.proj + rid * (int64_t)d * d;
+    const int li = lane & 15, kk = lane >> 4;
+
+    // The projection's first supersteps are requested before the left operand is staged: they
+    // depend on the relation only and fly during the index chain and the row gathers below.
+    auto wave_cols = [&](int c0, int &n0, int &wcols) {  // 256 output columns per sweep, split over the waves
+        const int span = d - c0 < 256 ? d - c0 : 256;
+        const int cw = ((span / 4 + 3) / 4) * 4;  // columns per wave, a multiple of 4
+        n0 = c0 + wave * cw;
+        wcols = n0 >= c0 + span ? 0 : (c0 + span - n0 < cw ? c0 + span - n0 : cw);
+    };
+    BLoader<MODE> bl;
+    float4 ring[kRing][4];
+    {
+        int n0, wcols;
+        wave_cols(0, n0, wcols);
+        if (wcols > 0) {  // per wave; a wave without columns (narrow rows) sits the sweep out
+            bl.init(M, d, kpad / 16, n0, wcols, li, kk);
+            ring_prime<MODE>(bl, ring);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+    }
 
     // triple ids of the tile first (one dependent-load chain per row instead of one per element)
     __shared__ int s_b[kTM];
@@ -541,24 +585,37 @@ __global__ __launch_bounds__(256, KGE_TR_OCC) void transr_gemm_kernel(GemmArgs a
     }
     __syncthreads();
 
-    const int li = lane & 15, kk = lane >> 4;
     const bool two_blocks = rows > 16;
     float rowsum[8];  // norm / dot partials for rows 4*kk + r (+16)
 #pragma unroll
     for (int r = 0; r < 8; ++r) rowsum[r] = 0.0f;
 
-    for (int c0 = 0; c0 < d; c0 += 256) {  // 256 output columns per sweep, split over the waves
-        const int span = d - c0 < 256 ? d - c0 : 256;
-        const int cw = ((span / 4 + 3) / 4) * 4;  // columns per wave, a multiple of 4
-        const int n0 = c0 + wave * cw;
-        const int wcols = n0 >= c0 + span ? 0 : (c0 + span - n0 < cw ? c0 + span - n0 : cw);
+    for (int c0 = 0; c0 < d; c0 += 256) {
+        int n0, wcols;
+        wave_cols(c0, n0, wcols);
         floatx4 acc_lo[4], acc_hi[4];
 #pragma unroll
         for (int e = 0; e < 4; ++e) acc_lo[e] = floatx4{0.f, 0.f, 0.f, 0.f}, acc_hi[e] = floatx4{0.f, 0.f, 0.f, 0.f};
+        if (c0 > 0 && wcols > 0) {  // (the first sweep's ring was primed before the staging)
+            bl.init(M, d, kpad / 16, n0, wcols, li, kk);
+            ring_prime<MODE>(bl, ring);
+        }
+        // epilogue operands that do not depend on the products: the relation row (TransR) is requested
+        // ahead of the sweep, the tail rows of this lane's eight triples (RESCAL) in one batch behind it
+        const int ecol = 4 * li < wcols ? n0 + 4 * li : 0;
+        float4 erow[MODE == 1 ? 8 : 1];
+        if constexpr (MODE == 0) erow[0] = *reinterpret_cast<const float4 *>(a.rel + rid * (int64_t)d + ecol);
 
         if (wcols > 0) {
-            if (two_blocks) gemm_sweep<MODE, true>(M, sX, pitch, d, kpad / 16, n0, wcols, li, kk, acc_lo, acc_hi);
-            else gemm_sweep<MODE, false>(M, sX, pitch, d, kpad / 16, n0, wcols, li, kk, acc_lo, acc_hi);
+            if (two_blocks) gemm_sweep<MODE, true>(bl, ring, sX, pitch, li, kk, acc_lo, acc_hi);
+            else gemm_sweep<MODE, false>(bl, ring, sX, pitch, li, kk, acc_lo, acc_hi);
+        }
+        if constexpr (MODE == 1) {  // one batch of unconditional loads (eight rows would not fit beside the ring)
+#pragma unroll
+            for (int q = 0; q < 8; ++q) {
+                const int row = 16 * (q >> 2) + 4 * kk + (q & 3);
+                erow[q] = *reinterpret_cast<const float4 *>(a.ent + s_t[row < rows ? row : 0] * (int64_t)d + ecol);
+            }
         }
 
         // epilogue for this sweep: lane holds rows 4 kk + r (and +16), columns per the mode
@@ -577,14 +634,14 @@ __global__ __launch_bounds__(256, KGE_TR_OCC) void transr_gemm_kernel(GemmArgs a
                     const int col = n0 + 4 * li;  // y[e] is column col + e
                     if (4 * li < wcols) {
                         if constexpr (MODE == 0) {
-                            const float4 rv = *reinterpret_cast<const float4 *>(a.rel + rid * (int64_t)d + col);
+                            const float4 rv = erow[0];
                             y[0] += rv.x, y[1] += rv.y, y[2] += rv.z, y[3] += rv.w;
                             float s = 0.0f;
 #pragma unroll
                             for (int e = 0; e < 4; ++e) s += a.norm_p == 1 ? fabsf(y[e]) : y[e] * y[e];
                             rowsum[4 * blk + r] += s;
                         } else {
-                            const float4 tv = *reinterpret_cast<const float4 *>(a.ent + s_t[row] * (int64_t)d + col);
+                            const float4 tv = erow[MODE == 1 ? 4 * blk + r : 0];
                             rowsum[4 * blk + r] += y[0] * tv.x + y[1] * tv.y + y[2] * tv.z + y[3] * tv.w;
                         }
                         if (a.resid)
@@ -897,7 +954,7 @@ struct RPlan {
     int64_t tiles, dtiles, dsplit, dslots;
 };
 
-static size_t plan_ints(int64_t tiles, int64_t split) { return (size_t)(64 + 3 * tiles + 3 * split + 8); }
+static size_t plan_ints(int64_t tiles, int64_t split) { return (size_t)(64 + 5 * tiles + 3 * split + 8); }
 
 static RPlan make_rplan(const kge_tables *tab, const kge_batch *bat)
 {
@@ -924,13 +981,16 @@ static RPlan make_rplan(const kge_tables *tab, const kge_batch *bat)
 static TilePlan plan_at(void *base, int64_t tiles, int64_t split)
 {
     int32_t *q = static_cast<int32_t *>(base);
-    TilePlan p{q, q + 64, q + 64 + tiles, nullptr, nullptr, nullptr, nullptr, nullptr};
+    TilePlan p{q, q + 64, q + 64 + tiles, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr};
     if (split > 0) {
         p.tile_part = q + 64 + 2 * tiles;
         p.num_split = q + 32;
-        p.split_seg = q + 64 + 3 * tiles;
+        p.split_seg = q + 64 + 5 * tiles;
         p.split_first = p.split_seg + split;
         p.split_cnt = p.split_first + split;
+    } else {
+        p.tile_end = q + 64 + 3 * tiles;
+        p.tile_rid = q + 64 + 4 * tiles;
     }
     return p;
 }
@@ -989,7 +1049,7 @@ int launch_transr_fwd(const kge_tables *tab, const kge_batch *bat, float *pos, f
     TilePlan plan = plan_at(workspace, tiles, 0);
     const RPlan rp = make_rplan(tab, bat);
     TilePlan dplan = plan_at(static_cast<char *>(workspace) + fwd_plan_bytes(tab, bat), rp.dtiles, rp.dsplit);
-    hipLaunchKernelGGL(transr_plan_kernel, dim3(2), dim3(1024), 0, st, ri->num_unique, ri->seg_offsets, plan, kTM,
+    hipLaunchKernelGGL(transr_plan_kernel, dim3(2), dim3(1024), 0, st, ri->num_unique, ri->seg_offsets, ri->unique_ids, plan, kTM,
                        dplan, kDmChunk);
     GemmArgs a{tab->ent, tab->rel, tab->aux, bat->h, bat->r, bat->t, ri->perm, ri->seg_offsets, ri->num_unique, ri->unique_ids,
                plan, nullptr, pos, resid, nullptr, nullptr, (int)tab->dim, tab->norm_p, thin_groups(tab, bat), (int)tiles};
@@ -1046,7 +1106,7 @@ int launch_transr_bwd(const kge_tables *tab, const kge_batch *bat, const kge_sav
                        f1);
     timeline_mark(bat->timeline, st, "transr_prep_kernel");
     if (!have_plans)
-        hipLaunchKernelGGL(transr_plan_kernel, dim3(2), dim3(1024), 0, st, ri->num_unique, ri->seg_offsets, plan, kTM,
+        hipLaunchKernelGGL(transr_plan_kernel, dim3(2), dim3(1024), 0, st, ri->num_unique, ri->seg_offsets, ri->unique_ids, plan, kTM,
                            dplan, kDmChunk);
     // dX = Q M^T -> occurrence rows of h (and -dX for t)
     GemmArgs ga{tab->ent, tab->rel, tab->aux, bat->h, bat->r, bat->t, ri->perm, ri->seg_offsets, ri->num_unique, ri->unique_ids,
