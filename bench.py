@@ -545,13 +545,67 @@ def run_workload(name, args, torch):
     return out
 
 
+def run_neg_transr(args, torch):
+    """TransR with shared negatives at B=4096, N=64, dim=200 (relations Zipf 1.2 over 1345, as the TransR
+    benchmark configuration): forward + backward with every negative projected once per (relation, chunk)
+    group, beside the flattened B * (1 + N) explicit triples (the reference's neg_transR,
+    apps/examples/examples.py:1447-1480).  Rows through the grouped matrix-core kernels are counted on the
+    host from the index arrays: 2 B + G N against B (1 + N), G = distinct (relation, chunk) pairs."""
+    from cuke_amd import synth
+    from cuke_amd.kge import KGEModel, inspect
+    dev = torch.device("cuda:0")
+    out = {"workload": "neg_transr_4096x64x200", "batch": 4096, "n_neg": 64, "dim": 200, "by_chunk": []}
+    for chunk in (64, 512, 4096):
+        w = synth.custom_workload("TransR", seed=args.seed, n_ent=40000, n_rel=1345, dim=200, batch=4096, chunk=chunk,
+                                  n_neg=64, norm_p=2, sigma=0.05, rel_zipf=1.2)
+        a = w.arrays
+        m = KGEModel("TransR", *[torch.from_numpy(a[k]).to(dev) for k in ("E", "R", "A")], norm_p=2)
+        ix = {k: torch.from_numpy(a[k]).to(dev) for k in ("h", "r", "t", "neg")}
+        g_pairs = len(np.unique(a["r"] * w.n_chunks + np.arange(w.batch) // chunk))
+        rows_grouped, rows_flat = 2 * w.batch + g_pairs * w.n_neg, w.batch * (1 + w.n_neg)
+        dpos = torch.ones(w.batch, device=dev)
+        dneg = torch.ones((w.batch, w.n_neg), device=dev)
+        ent_insp, rel_insp = m.inspect_batch(ix["h"], ix["r"], ix["t"], ix["neg"])
+
+        def grouped():
+            fw = m.score(ix["h"], ix["r"], ix["t"], ix["neg"], chunk, ent_insp=ent_insp, rel_insp=rel_insp)
+            return fw, m.backward(fw, dpos, dneg)
+
+        def flattened():
+            fw = m._score_projected_negatives(ix["h"], ix["r"], ix["t"], ix["neg"], chunk)
+            return fw, m.backward(fw, dpos, dneg)
+
+        fg, gg = grouped()
+        ff, gf = flattened()
+        torch.cuda.synchronize()
+        err = float((fg.neg - ff.neg).abs().max() / ff.neg.abs().max())
+        gerr = float((gg.aux_rows - gf.aux_rows).abs().max() / gf.aux_rows.abs().max())
+        if not (err < 1e-5 and gerr < 1e-4):
+            raise SpotCheckError(f"neg_transr chunk {chunk}: grouped and flattened paths differ ({err:.2e}, {gerr:.2e})")
+        del fg, gg, ff, gf
+        res = {}
+        for label, fn in (("grouped", grouped), ("flattened", flattened)):
+            for _ in range(3):
+                fn()
+            torch.cuda.synchronize()
+            res[label] = time_events(fn, max(5, min(20, args.steps)), torch)
+        out["by_chunk"].append({"chunk": chunk, "groups": g_pairs, "rows_projected_grouped": rows_grouped,
+                                "rows_projected_flattened": rows_flat, "row_ratio": rows_flat / rows_grouped,
+                                "ms_grouped": res["grouped"], "ms_flattened": res["flattened"],
+                                "max_rel_diff_scores": err, "max_rel_diff_projection_gradients": gerr})
+        del m
+        torch.cuda.empty_cache()
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=100)
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--workload", default="all",
-                    help="all (default), one of " + ", ".join(ALL_WORKLOADS) + ", or ref_transr_8192x512")
+                    help="all (default), one of " + ", ".join(ALL_WORKLOADS) + ", ref_transr_8192x512, or neg_transr "
+                         "(TransR shared negatives: grouped projection against flattened triples)")
     ap.add_argument("--batches", type=int, default=8, help="distinct seeded batches the timed loop rotates over")
     ap.add_argument("--no-graph", action="store_true", help="do not also time HIP-graph replays of the step")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline legs")
@@ -576,6 +630,13 @@ def main():
         dst.copy_(src)  # one elementwise copy kernel: reads 256 MiB, writes 256 MiB
         torch.cuda.synchronize()
         del src, dst
+    if args.workload == "neg_transr":
+        try:
+            print(json.dumps(run_neg_transr(args, torch)))
+        except SpotCheckError as e:
+            print(f"bench.py: {e}", file=sys.stderr)
+            sys.exit(1)
+        return
     names = ALL_WORKLOADS if args.workload == "all" else [args.workload]
     results = []
     for n in names:

@@ -11,6 +11,8 @@ int launch_score_neg(const kge_tables *, const kge_batch *, const float *, const
                      const FusedInsp *, hipStream_t);
 int launch_transr_fwd(const kge_tables *, const kge_batch *, float *, float *, void *, size_t, hipStream_t);
 size_t transr_fwd_workspace(const kge_tables *, const kge_batch *);
+int launch_transr_neg_fwd(const kge_tables *, const kge_batch *, float *, float *, float *, void *, size_t, hipStream_t);
+size_t transr_neg_fwd_workspace(const kge_tables *, const kge_batch *);
 
 __global__ void check_indices_kernel(const int64_t *idx, int64_t n, int64_t n_rows, int32_t *flag)
 {
@@ -168,6 +170,10 @@ int kge_timeline_elapsed(const kge_timeline *tl, float *ms)
 size_t kge_score_fwd_workspace(const kge_tables *tab, const kge_batch *bat)
 {
     if (!tab || !bat || bat->batch < 0) return 0;
+    if (tab->model == KGE_TRANSR && bat->neg && bat->rel_insp) {  // shared negatives: group list + projected rows
+        const size_t nb = transr_neg_fwd_workspace(tab, bat);
+        if (nb) return nb;
+    }
     if ((tab->model == KGE_TRANSR || tab->model == KGE_RESCAL) && bat->rel_insp) return transr_fwd_workspace(tab, bat);
     return 0;
 }
@@ -209,6 +215,8 @@ int kge_score_fwd(const kge_tables *tab, const kge_batch *bat, float *pos, float
         if ((rc = plan_fused_inspection(bat->insp_jobs, 2, 0, &fi0))) return rc;
         if ((rc = plan_fused_inspection(bat->insp_jobs, 2, 1, &fi1))) return rc;
     }
+    if (want_neg && tab->model == KGE_TRANSR && bat->rel_insp)  // positives and shared negatives in one grouped pass
+        return launch_transr_neg_fwd(tab, bat, pos, neg, residual, workspace, workspace_bytes, st);
     if (pos || side_pos || residual) {
         if ((tab->model == KGE_TRANSR || tab->model == KGE_RESCAL) && bat->rel_insp)
             rc = launch_transr_fwd(tab, bat, pos, residual, workspace, workspace_bytes, st);

@@ -855,6 +855,9 @@ static BwdPlan make_bwd_plan(const kge_tables *tab, const kge_batch *bat)
 int launch_transr_bwd(const kge_tables *, const kge_batch *, const kge_saved *, const float *,
                       const kge_grads *, void *, size_t, hipStream_t);
 size_t transr_bwd_workspace(const kge_tables *, const kge_batch *);
+int launch_transr_neg_bwd(const kge_tables *, const kge_batch *, const kge_saved *, const float *, const float *,
+                          const kge_grads *, void *, size_t, hipStream_t);
+size_t transr_neg_bwd_workspace(const kge_tables *, const kge_batch *);
 
 }  // namespace kge
 
@@ -866,6 +869,7 @@ size_t kge_score_bwd_workspace(const kge_tables *tab, const kge_batch *bat)
 {
     if (!tab || !bat || bat->batch < 0 || tab->dim <= 0) return 0;
     if (bat->neg && bat->chunk <= 0) return 0;
+    if (tab->model == KGE_TRANSR && bat->neg) return transr_neg_bwd_workspace(tab, bat);
     if (tab->model == KGE_TRANSR || tab->model == KGE_RESCAL) return transr_bwd_workspace(tab, bat);
     return make_bwd_plan(tab, bat).total;
 }
@@ -881,6 +885,8 @@ int kge_score_bwd(const kge_tables *tab, const kge_batch *bat, const kge_saved *
     if (bat->neg && (bat->chunk <= 0 || bat->n_neg <= 0 || bat->batch % bat->chunk)) return KGE_ESHAPE;
     hipStream_t st = as_stream(stream);
     KGE_CLEAR_LAUNCH_ERRORS();
+    if (tab->model == KGE_TRANSR && bat->neg)
+        return launch_transr_neg_bwd(tab, bat, saved, dpos, dneg, grads, workspace, workspace_bytes, st);
     if (tab->model == KGE_TRANSR || tab->model == KGE_RESCAL)
         return launch_transr_bwd(tab, bat, saved, dpos, grads, workspace, workspace_bytes, st);
 

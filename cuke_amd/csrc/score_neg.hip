@@ -72,7 +72,6 @@ __global__ __launch_bounds__(256, KGE_TILE_OCC) void score_neg_kernel(NegArgs a,
     constexpr int NPA = (MODEL == KGE_ROTATE || MODEL == KGE_TRANSH) ? 2 : 1;
     constexpr int NPT = MODEL == KGE_ROTATE ? 2 : 1;
     constexpr int SB = TB / 32, SN = TN / 32;  // float4 per thread per plane per step
-    constexpr int NPASS = MODEL == KGE_TRANSH ? 2 : 1;
     // TransH, L1, with the sign sums saved for backward: the second sweep's rows are staged times
     // 2^100 so that the sign of a residual element is a single clamp (tile_common.hpp)
     constexpr bool kScaled = MODEL == KGE_TRANSH && P == 1 && SAVE;

@@ -140,6 +140,7 @@ struct GemmArgs {
     const int64_t *unique_ids;
     TilePlan plan;
     const float *xs;  // TRANSPOSED pass: left operand rows in sorted order [B, d]
+    const float *rs;  // list pass (MODE 3): factor of the relation row per list row (+1, -1 or 0)
     float *pos;       // forward: [B] scores (nullable)
     float *resid;     // forward: [B, d] rows y (nullable)
     float *occ_h, *occ_t;  // backward-dX: [B, d] each (occ_t nullable)
@@ -172,7 +173,8 @@ __device__ __forceinline__ ThinTile thin_tile_of_group(const int32_t *num_unique
     return t;
 }
 
-// Y[r][:] = X[r][:] * M for the r < rows <= 4 triples of the tile (MODE 0 TransR, MODE 1 RESCAL).
+// Y[r][:] = X[r][:] * M for the r < rows <= 4 triples of the tile (MODE 0 TransR, MODE 1 RESCAL,
+// MODE 3 list rows: x = E[h] - E[t] with t = -1 standing for no row, y = x M + rs R[r], no score).
 // Thread (phase, cq) owns the four columns 4 cq .. 4 cq + 3 and the projection rows
 // k = phase, phase + P, ... (P = 256 / (d / 4) phases): consecutive threads read consecutive
 // 16-byte pieces of the projection.  The phases are summed through LDS in a fixed order.
@@ -190,13 +192,15 @@ __device__ __forceinline__ void transr_thin_fwd_body(const GemmArgs &a, float *l
     float *sPart = reinterpret_cast<float *>(sRed + P * 4 * nq4);  // [4][nq4]
     __shared__ int s_b[kThin];
     __shared__ int64_t s_h[kThin], s_t[kThin];
+    __shared__ float s_rs[kThin];
     const int64_t rid = a.unique_ids[g];
     const float4 *M4 = reinterpret_cast<const float4 *>(a.proj + rid * (int64_t)d * d);
     if (tid < kThin) {
-        const int b = tid < rows ? a.perm[tt.p0 + tid] : 0;
+        const int b = tid < rows ? (MODE == 3 ? tt.p0 + tid : a.perm[tt.p0 + tid]) : (MODE == 3 ? tt.p0 : 0);
         s_b[tid] = b;
         s_h[tid] = a.h[b];
         s_t[tid] = a.t[b];
+        if constexpr (MODE == 3) s_rs[tid] = a.rs[b];
     }
     for (int k = tid; k < kcap; k += 256) sXT[k] = make_float4(0.f, 0.f, 0.f, 0.f);
     __syncthreads();
@@ -206,6 +210,12 @@ __device__ __forceinline__ void transr_thin_fwd_body(const GemmArgs &a, float *l
         if constexpr (MODE == 0) {
             const float4 u = *reinterpret_cast<const float4 *>(a.ent + s_t[r] * (int64_t)d + k4);
             v = make_float4(v.x - u.x, v.y - u.y, v.z - u.z, v.w - u.w);
+        }
+        if constexpr (MODE == 3) {
+            if (s_t[r] >= 0) {
+                const float4 u = *reinterpret_cast<const float4 *>(a.ent + s_t[r] * (int64_t)d + k4);
+                v = make_float4(v.x - u.x, v.y - u.y, v.z - u.z, v.w - u.w);
+            }
         }
         float *col = reinterpret_cast<float *>(sXT + k4) + r;
         col[0] = v.x, col[4] = v.y, col[8] = v.z, col[12] = v.w;
@@ -252,12 +262,16 @@ __device__ __forceinline__ void transr_thin_fwd_body(const GemmArgs &a, float *l
             const float4 v = sRed[(pp * 4 + r) * nq4 + q];
             y.x += v.x, y.y += v.y, y.z += v.z, y.w += v.w;
         }
-        float sum;
+        float sum = 0.0f;
         if constexpr (MODE == 0) {
             const float4 rv = *reinterpret_cast<const float4 *>(a.rel + rid * (int64_t)d + 4 * q);
             y.x += rv.x, y.y += rv.y, y.z += rv.z, y.w += rv.w;
             sum = a.norm_p == 1 ? fabsf(y.x) + fabsf(y.y) + fabsf(y.z) + fabsf(y.w)
                                 : y.x * y.x + y.y * y.y + y.z * y.z + y.w * y.w;
+        } else if constexpr (MODE == 3) {
+            const float4 rv = *reinterpret_cast<const float4 *>(a.rel + rid * (int64_t)d + 4 * q);
+            const float f = s_rs[r];  // +-1 or 0: the products are exact, the sum rounds as in MODE 0
+            y.x += f * rv.x, y.y += f * rv.y, y.z += f * rv.z, y.w += f * rv.w;
         } else {
             const float4 tv = *reinterpret_cast<const float4 *>(a.ent + s_t[r] * (int64_t)d + 4 * q);
             sum = y.x * tv.x + y.y * tv.y + y.z * tv.z + y.w * tv.w;
@@ -309,7 +323,7 @@ __device__ __forceinline__ void transr_thin_dx_body(const GemmArgs &a, float *sY
     const int d = a.d, nq4 = d >> 2, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int li = lane & 15, sub = lane >> 4;
     __shared__ int s_b[kThin];
-    if (tid < kThin) s_b[tid] = tid < rows ? a.perm[tt.p0 + tid] : 0;
+    if (tid < kThin) s_b[tid] = tid < rows ? (a.perm ? a.perm[tt.p0 + tid] : tt.p0 + tid) : 0;  // no perm: rows stay in sorted order
     const int64_t rid = a.unique_ids[g];
     const float4 *M4 = reinterpret_cast<const float4 *>(a.proj + rid * (int64_t)d * d);
     const int jfirst = 4 * wave + sub;  // row of (step i, wave, sub): j = 16 i + 4 wave + sub
@@ -482,6 +496,8 @@ __device__ __forceinline__ void gemm_sweep(const BLoader<MODE> &bl, float4 (&rin
 // MODE 0: forward TransR   x = E[h]-E[t], y = x M + R[r], score = ||y||_p
 // MODE 1: forward RESCAL   x = E[h],      y = x M,        score = y . E[t]
 // MODE 2: backward dX      x = xs rows,   y = x M^T -> occ_h = y, occ_t = -y (when occ_t is set)
+// MODE 3: list rows        x = E[h]-E[t] (t = -1: no row), y = x M + rs R[r] -> resid rows in list order;
+//         h, t, rs are indexed by the sorted position itself (no perm), no score
 template <int MODE>
 __global__ __launch_bounds__(256, KGE_TR_OCC) void transr_gemm_kernel(GemmArgs a, FusedInsp fi)
 {
@@ -542,13 +558,17 @@ __global__ __launch_bounds__(256, KGE_TR_OCC) void transr_gemm_kernel(GemmArgs a
     // triple ids of the tile first (one dependent-load chain per row instead of one per element)
     __shared__ int s_b[kTM];
     __shared__ int64_t s_h[kTM], s_t[kTM];
+    __shared__ float s_rs[MODE == 3 ? kTM : 1];
     if (tid < kTM) {
-        const int b = tid < rows ? a.perm[p0 + tid] : 0;
+        int b;
+        if constexpr (MODE == 3) b = p0 + (tid < rows ? tid : 0);
+        else b = tid < rows ? (a.perm ? a.perm[p0 + tid] : p0 + tid) : 0;
         s_b[tid] = b;
         if constexpr (MODE != 2) {
             s_h[tid] = a.h[b];
             s_t[tid] = a.t[b];
         }
+        if constexpr (MODE == 3) s_rs[tid] = a.rs[b];
     }
     __syncthreads();
     // stage the left operand with all loads of a thread in flight together
@@ -569,6 +589,9 @@ __global__ __launch_bounds__(256, KGE_TR_OCC) void transr_gemm_kernel(GemmArgs a
                         v[q] = *reinterpret_cast<const float4 *>(a.ent + s_h[row] * (int64_t)d + k4);
                         if constexpr (MODE == 0)
                             u[q] = *reinterpret_cast<const float4 *>(a.ent + s_t[row] * (int64_t)d + k4);
+                        if constexpr (MODE == 3) {
+                            if (s_t[row] >= 0) u[q] = *reinterpret_cast<const float4 *>(a.ent + s_t[row] * (int64_t)d + k4);
+                        }
                     }
                 }
             }
@@ -604,7 +627,7 @@ __global__ __launch_bounds__(256, KGE_TR_OCC) void transr_gemm_kernel(GemmArgs a
         // ahead of the sweep, the tail rows of this lane's eight triples (RESCAL) in one batch behind it
         const int ecol = 4 * li < wcols ? n0 + 4 * li : 0;
         float4 erow[MODE == 1 ? 8 : 1];
-        if constexpr (MODE == 0) erow[0] = *reinterpret_cast<const float4 *>(a.rel + rid * (int64_t)d + ecol);
+        if constexpr (MODE == 0 || MODE == 3) erow[0] = *reinterpret_cast<const float4 *>(a.rel + rid * (int64_t)d + ecol);
 
         if (wcols > 0) {
             if (two_blocks) gemm_sweep<MODE, true>(bl, ring, sX, pitch, li, kk, acc_lo, acc_hi);
@@ -633,7 +656,11 @@ __global__ __launch_bounds__(256, KGE_TR_OCC) void transr_gemm_kernel(GemmArgs a
                 if constexpr (MODE != 2) {
                     const int col = n0 + 4 * li;  // y[e] is column col + e
                     if (4 * li < wcols) {
-                        if constexpr (MODE == 0) {
+                        if constexpr (MODE == 3) {
+                            const float4 rv = erow[0];
+                            const float f = s_rs[row];  // +-1 or 0: exact products
+                            y[0] += f * rv.x, y[1] += f * rv.y, y[2] += f * rv.z, y[3] += f * rv.w;
+                        } else if constexpr (MODE == 0) {
                             const float4 rv = erow[0];
                             y[0] += rv.x, y[1] += rv.y, y[2] += rv.z, y[3] += rv.w;
                             float s = 0.0f;
@@ -1052,7 +1079,7 @@ int launch_transr_fwd(const kge_tables *tab, const kge_batch *bat, float *pos, f
     hipLaunchKernelGGL(transr_plan_kernel, dim3(2), dim3(1024), 0, st, ri->num_unique, ri->seg_offsets, ri->unique_ids, plan, kTM,
                        dplan, kDmChunk);
     GemmArgs a{tab->ent, tab->rel, tab->aux, bat->h, bat->r, bat->t, ri->perm, ri->seg_offsets, ri->num_unique, ri->unique_ids,
-               plan, nullptr, pos, resid, nullptr, nullptr, (int)tab->dim, tab->norm_p, thin_groups(tab, bat), (int)tiles};
+               plan, nullptr, nullptr, pos, resid, nullptr, nullptr, (int)tab->dim, tab->norm_p, thin_groups(tab, bat), (int)tiles};
     const size_t lds = lds_with(fi, gemm_lds_bytes((int)tab->dim));
     const dim3 grid((unsigned)(tiles + a.thin_groups + fi.blocks));
     if (const int rc = rescal ? allow_lds<1>(lds) : allow_lds<0>(lds)) return rc;
@@ -1110,7 +1137,7 @@ int launch_transr_bwd(const kge_tables *tab, const kge_batch *bat, const kge_sav
                            dplan, kDmChunk);
     // dX = Q M^T -> occurrence rows of h (and -dX for t)
     GemmArgs ga{tab->ent, tab->rel, tab->aux, bat->h, bat->r, bat->t, ri->perm, ri->seg_offsets, ri->num_unique, ri->unique_ids,
-                plan, qs, nullptr, nullptr, occ, rescal ? nullptr : occ + B * d, d, tab->norm_p, thin_groups(tab, bat), (int)p.tiles};
+                plan, qs, nullptr, nullptr, nullptr, occ, rescal ? nullptr : occ + B * d, d, tab->norm_p, thin_groups(tab, bat), (int)p.tiles};
     if (const int rc = allow_lds<2>(lds_with(f2, gemm_lds_bytes(d)))) return rc;
     hipLaunchKernelGGL(transr_gemm_kernel<2>, dim3((unsigned)(p.tiles + ga.thin_groups + f2.blocks)), dim3(256),
                        lds_with(f2, gemm_lds_bytes(d)), st, ga, f2);
@@ -1135,5 +1162,7 @@ int launch_transr_bwd(const kge_tables *tab, const kge_batch *bat, const kge_sav
         {qs, ri, d, grads->rel_rows, reinterpret_cast<float *>(ws + p.off_part_r), true}};
     return launch_seg_reduce_jobs(jobs, rescal ? 1 : 2, st, bat->timeline);
 }
+
+#include "transr_neg.hpp"
 
 }  // namespace kge

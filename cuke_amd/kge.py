@@ -125,7 +125,8 @@ class Forward:
     side_pos: torch.Tensor | None = None
     side_neg: torch.Tensor | None = None
     residual: torch.Tensor | None = None
-    flat_pos: torch.Tensor | None = None   # TransR / RESCAL with negatives: scores of the flattened batch
+    flat_pos: torch.Tensor | None = None   # projection models scored through flattened triples: all scores
+    fwd_ws: torch.Tensor | None = None     # forward workspace that backward reads again (TransR with negatives)
     batch: tuple = ()
     neg_mode: str = "tail"
     ent_insp: Inspection | None = None
@@ -243,8 +244,16 @@ class KGEModel:
         ``neg_mode='tail'``: neg[b, k] scores (h_b, r_b, neg_k), the reference's shared-negative layout
         (apps/examples/examples.py:1404-1444); ``'head'``: (neg_k, r_b, t_b), the head-corrupted batches of
         the reference's sampler (apps/kge/data/sampler.py:287-353)."""
-        if neg is not None and self.model in ("TransR", "RESCAL"):
+        if neg is not None and self.model == "RESCAL":
             return self._score_projected_negatives(h, r, t, neg, chunk, neg_mode)
+        if neg is not None and self.model == "TransR":
+            # every negative is projected once per (relation, chunk) group of the batch; needs the
+            # relation groups.  Shapes outside the grouped kernels (dim % 4, dim > 1024) take the
+            # flattened triples instead.
+            if rel_insp is None:
+                rel_insp = inspect([_index(r, "r", self.dev)], self.n_rel)
+            if self.dim % 4 != 0 or self.dim > 1024:
+                return self._score_projected_negatives(h, r, t, neg, chunk, neg_mode)
         bat, keep = self._batch(h, r, t, neg, chunk, ent_insp, rel_insp, neg_mode)
         B, N = bat.batch, bat.n_neg
         f32 = dict(dtype=torch.float32, device=self.dev)
@@ -260,6 +269,8 @@ class KGEModel:
         _lib.check(_lib.lib().kge_score_fwd(C.byref(self._tab), C.byref(bat), _ptr(fw.pos),
                                             _ptr(fw.neg), _ptr(fw.side_pos), _ptr(fw.side_neg),
                                             _ptr(fw.residual), _ptr(ws), nb, _stream()), "kge_score_fwd")
+        if neg is not None and self.model == "TransR":
+            fw.fwd_ws = ws  # group list and projected rows, read again by backward
         return fw
 
     def _score_projected_negatives(self, h, r, t, neg, chunk, neg_mode="tail") -> Forward:
@@ -300,7 +311,9 @@ class KGEModel:
             return self.backward(flat, g)
         h, r, t, neg, C_, N = fw.batch
         if fw.ent_insp is None or fw.rel_insp is None:
-            fw.ent_insp, fw.rel_insp = self.inspect_batch(h, r, t, neg)
+            e_insp, r_insp = self.inspect_batch(h, r, t, neg)
+            fw.ent_insp = fw.ent_insp if fw.ent_insp is not None else e_insp
+            fw.rel_insp = fw.rel_insp if fw.rel_insp is not None else r_insp  # (the forward pass may have planned from it)
         bat, _ = self._batch(h, r, t, neg, C_ or None, fw.ent_insp, fw.rel_insp, fw.neg_mode)
         B = bat.batch
         f32 = dict(dtype=torch.float32, device=self.dev)
@@ -310,6 +323,8 @@ class KGEModel:
             dneg = dneg.to(**f32).contiguous()
         saved = _lib.Saved(*[(x.data_ptr() if x is not None else None) for x in
                              (fw.pos, fw.neg, fw.side_pos, fw.side_neg, fw.residual)])
+        if fw.fwd_ws is not None:
+            saved.fwd_workspace, saved.fwd_workspace_bytes = fw.fwd_ws.data_ptr(), int(fw.fwd_ws.numel())
         ent_rows = torch.empty((fw.ent_insp.n, self.dim), **f32)
         rel_rows = torch.empty((B, self.rel_dim), **f32) if self.rel_dim else None
         aux_rows = None

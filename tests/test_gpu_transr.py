@@ -118,7 +118,7 @@ def test_shared_negatives_through_flattened_triples(oracle, model):
                               rel_zipf=1.1, ent_zipf=1.1, seed=5)
     a = w.arrays
     m, ix = gpu_model(w)
-    fw = m.score(ix["h"], ix["r"], ix["t"], ix["neg"], w.chunk)
+    fw = m._score_projected_negatives(ix["h"], ix["r"], ix["t"], ix["neg"], w.chunk)
     pos, negs = oracle.score(model, a["E"], a["R"], a["A"], a["h"], a["r"], a["t"], a["neg"], w.chunk, p=2)
     assert_close(fw.pos.cpu().numpy(), pos, what="pos")
     assert_close(fw.neg.cpu().numpy(), negs, what="neg")
@@ -137,3 +137,59 @@ def test_shared_negatives_through_flattened_triples(oracle, model):
     if model == "TransR":
         assert_close(g.rel_rows.cpu().numpy(), ref.rel_rows, what="relation rows", rows=True)
     assert_close(g.aux_rows.cpu().numpy(), ref.aux_rows, what="projection gradients", rows=True)
+
+
+def _neg_case(oracle, w, mode, what):
+    a = w.arrays
+    if w.lattice:  # keep the projected rows exact too: projections on a coarse grid (L1 gradients are sums of signs)
+        a["A"] = (np.rint(a["A"] / 0.2 * 2) / 8).astype(np.float32)
+    m, ix = gpu_model(w)
+    fw = m.score(ix["h"], ix["r"], ix["t"], ix["neg"], w.chunk, neg_mode=mode)
+    assert fw.fwd_ws is not None and fw.flat_pos is None, "the grouped shared-negative path did not run"
+    pos, negs = oracle.score("TransR", a["E"], a["R"], a["A"], a["h"], a["r"], a["t"], a["neg"], w.chunk, p=w.norm_p,
+                             neg_mode=mode)
+    floor = 2.0 if (w.norm_p == 1 and w.dim >= 400) else 0.0
+    assert_close(fw.pos.cpu().numpy(), pos, what=f"{what} pos", global_floor=floor)
+    assert_close(fw.neg.cpu().numpy(), negs, what=f"{what} neg", global_floor=floor)
+    want = oracle.residual("TransR", a["E"], a["R"], a["A"], a["h"], a["r"], a["t"])
+    assert_close(fw.residual.cpu().numpy(), want, what=f"{what} residual rows of the positives", rows=True)
+    rng = np.random.default_rng(w.seed + 11)
+    dpos = rng.standard_normal(w.batch).astype(np.float32)
+    dneg = rng.standard_normal((w.batch, w.n_neg)).astype(np.float32)
+    g = m.backward(fw, torch.from_numpy(dpos).cuda(), torch.from_numpy(dneg).cuda())
+    ref = oracle.backward("TransR", a["E"], a["R"], a["A"], a["h"], a["r"], a["t"], a["neg"], w.chunk, dpos, dneg,
+                          p=w.norm_p, neg_mode=mode)
+    assert np.array_equal(g.ent_ids.cpu().numpy(), ref.ent_ids)
+    assert np.array_equal(g.rel_ids.cpu().numpy(), ref.rel_ids)
+    assert_close(g.ent_rows.cpu().numpy(), ref.ent_rows, what=f"{what} entity rows", rows=True)
+    assert_close(g.rel_rows.cpu().numpy(), ref.rel_rows, what=f"{what} relation rows", rows=True)
+    assert_close(g.aux_rows.cpu().numpy(), ref.aux_rows, what=f"{what} projection gradients", rows=True)
+    return m, ix, fw
+
+
+# Shared negatives with every negative projected once per (relation, chunk) group: the scores and
+# gradients of the reference's neg_transR (examples.py:1447-1480) without its batch * blocksize
+# vector x matrix products.
+@pytest.mark.parametrize("shape", [
+    dict(dim=40, batch=48, chunk=16, n_neg=12, n_rel=6),       # a few groups per chunk
+    dict(dim=200, batch=512, chunk=64, n_neg=64, n_rel=50),    # benchmark-like: Zipf relations, many singleton groups
+    dict(dim=300, batch=96, chunk=96, n_neg=5, n_rel=4),       # one chunk, rows wider than 256 floats, odd N
+    dict(dim=16, batch=64, chunk=8, n_neg=2, n_rel=40),        # more relations than positives per chunk; thin dM groups
+    dict(dim=64, batch=300, chunk=300, n_neg=33, n_rel=1),     # one relation: a single group
+    dict(dim=528, batch=64, chunk=32, n_neg=16, n_rel=3),      # three quads of a row per lane
+])
+@pytest.mark.parametrize("p", [1, 2])
+@pytest.mark.parametrize("mode", ["tail", "head"])
+def test_shared_negatives_projected_once_per_group(oracle, shape, p, mode):
+    w = synth.custom_workload("TransR", n_ent=500, norm_p=p, sigma=0.2, rel_zipf=1.1, ent_zipf=1.1, seed=7,
+                              lattice=(p == 1), **shape)
+    _neg_case(oracle, w, mode, f"{shape} p={p} {mode}")
+
+
+def test_shared_negatives_grouped_path_equals_the_flattened_one(oracle):
+    w = synth.custom_workload("TransR", n_ent=400, n_rel=20, dim=128, batch=256, chunk=64, n_neg=32, sigma=0.2,
+                              rel_zipf=1.2, seed=3)
+    m, ix, fw = _neg_case(oracle, w, "tail", "grouped")
+    flat = m._score_projected_negatives(ix["h"], ix["r"], ix["t"], ix["neg"], w.chunk)
+    assert_close(fw.neg.cpu().numpy(), flat.neg.cpu().numpy(), what="grouped vs flattened negative scores")
+    assert_close(fw.pos.cpu().numpy(), flat.pos.cpu().numpy(), what="grouped vs flattened positive scores")
