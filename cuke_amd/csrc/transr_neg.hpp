@@ -18,6 +18,8 @@
 //
 // This file is included by transr.hip (inside namespace kge) below the grouped kernels.
 
+constexpr int kNegSeg = 8;  // sorted positions per wave of the P-row gradient sum
+
 struct NegShape {
     int64_t B, N, C, n_chunks, NN, d, U_cap, G_cap, L_cap;
     int64_t tiles, dtiles, dsplit, dslots;
@@ -81,7 +83,7 @@ static NegFwdLayout neg_fwd_layout(const kge_tables *tab, const NegShape &s)
 }
 
 struct NegBwdLayout {
-    size_t xl, ql, dxl, occ, qr, glist, gcount, part_e, part_r, dpart, total;
+    size_t xl, ql, dxl, occ, qr, glist, gcount, ppart, part_e, part_r, dpart, total;
 };
 
 static NegBwdLayout neg_bwd_layout(const NegShape &s)
@@ -99,6 +101,7 @@ static NegBwdLayout neg_bwd_layout(const NegShape &s)
     l.qr = take(sizeof(float) * (size_t)(s.B * s.d));
     l.glist = take(sizeof(int32_t) * s.B);
     l.gcount = take(sizeof(int32_t) * s.n_chunks);
+    l.ppart = take(sizeof(float) * (size_t)(ceil_div(s.B, kNegSeg) * s.N * 2 * s.d));
     l.part_e = take(sizeof(float) * (size_t)seg_partial_floats(2 * s.B + s.NN, s.d));
     l.part_r = take(sizeof(float) * (size_t)seg_partial_floats(s.B, s.d));
     l.dpart = take(sizeof(float) * (size_t)(s.dslots * s.d * s.d));
@@ -371,60 +374,139 @@ __global__ __launch_bounds__(256) void tneg_pair_bwd_a_kernel(NegIdx x, NegPairA
     neg_store_row(a.qr + b * (int64_t)d, d, lane, qr);
 }
 
-// Backward, one wave per (group, negative): the upstream row of P_(g,k) is minus the sum over the
-// group's positives of their pair gradients, in the order of the positives.
+// Backward, upstream rows of the P rows: Q_(g,k) = - sum over the positives b of group g of their pair
+// gradients.  The positives sit next to each other in the key order, so this is a segmented sum
+// over the sorted positions whose terms are formed on the fly.  Level 1: a wave owns kNegSeg
+// consecutive sorted positions and one negative k and walks them in order; a group that lies
+// wholly inside the block is final, one that began in an earlier block goes to partial slot 0 of
+// the block, one that continues past it to slot 1 (the scheme of seg_reduce.hip).  Level 2: the
+// block in which a long group starts adds its slot-1 partial and the slot-0 partials of the
+// following blocks.  Work is spread over B N / kNegSeg waves whatever the group sizes are (a hot
+// relation's group has hundreds of positives); the order of the sum is fixed by the sorted order.
 template <int P, int NQ>
-__global__ __launch_bounds__(256) void tneg_pair_bwd_p_kernel(NegIdx x, NegPairArgs a)
+__global__ __launch_bounds__(256) void tneg_pair_bwd_p1_kernel(NegIdx x, NegPairArgs a, const int32_t *k_sseg, float *partial)
 {
     const int lane = threadIdx.x & 63;
     const int64_t w = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
-    const int N = (int)x.N;
-    const int64_t g = w / N;
+    const int N = (int)x.N, d = x.d;
+    const int64_t j = w / N;
     const int k = (int)(w % N);
-    if (g >= x.k_num[0]) return;
-    const int d = x.d;
-    const int row = x.rowp[g] + k;
-    const NegRow<NQ> p = neg_load_row<NQ>(a.y + (int64_t)row * d, d, lane);
+    const int64_t p0 = j * kNegSeg;
+    if (p0 >= x.B) return;
+    const int cnt = (int)(x.B - p0 < kNegSeg ? x.B - p0 : kNegSeg);
+    int bb[kNegSeg], gg[kNegSeg];
+#pragma unroll
+    for (int q = 0; q < kNegSeg; ++q) {
+        const int64_t pc = p0 + (q < cnt ? q : cnt - 1);  // clamped: unconditional loads, masked at their use
+        bb[q] = x.k_perm[pc], gg[q] = k_sseg[pc];
+    }
+    const int g_before = p0 > 0 ? k_sseg[p0 - 1] : -1, g_after = p0 + cnt < x.B ? k_sseg[p0 + cnt] : -1;
     NegRow<NQ> acc;
 #pragma unroll
-    for (int q = 0; q < NQ; ++q) acc.v[q] = make_float4(0.f, 0.f, 0.f, 0.f);
-    const int m0 = x.k_seg[g], m1 = x.k_seg[g + 1];
-    if (a.dneg) {
-        for (int m = m0; m < m1; m += 2) {  // two positives in flight
-            int bb[2];
-            float coef[2];
-            NegRow<NQ> ya[2];
+    for (int e = 0; e < NQ; ++e) acc.v[e] = make_float4(0.f, 0.f, 0.f, 0.f);
+    auto flush = [&](int g) {
+        float *dst;
+        if (g == g_before) dst = partial + ((j * N + k) * 2 + 0) * (int64_t)d;
+        else if (g == g_after) dst = partial + ((j * N + k) * 2 + 1) * (int64_t)d;
+        else dst = a.ql + (int64_t)(x.rowp[g] + k) * d;
+        neg_store_row(dst, d, lane, acc);
+    };
+    constexpr int kFly = NQ == 1 ? 8 : (NQ == 2 ? 4 : 2);  // positions whose rows are in flight together
 #pragma unroll
-            for (int u = 0; u < 2; ++u) bb[u] = x.k_perm[m + u < m1 ? m + u : m1 - 1];
+    for (int q0 = 0; q0 < kNegSeg; q0 += kFly) {
+        NegRow<NQ> ya[kFly], pr[kFly];
+        float coef[kFly];
 #pragma unroll
-            for (int u = 0; u < 2; ++u) {
-                ya[u] = neg_load_row<NQ>(a.y + (int64_t)x.rowa[bb[u]] * d, d, lane);
-                const float gg = a.dneg[bb[u] * (int64_t)N + k];
-                float c = gg;
+        for (int u = 0; u < kFly; ++u) {
+            const int q = q0 + u;
+            ya[u] = neg_load_row<NQ>(a.y + (int64_t)x.rowa[bb[q]] * d, d, lane);
+            pr[u] = neg_load_row<NQ>(a.y + (int64_t)(x.rowp[gg[q]] + k) * d, d, lane);
+            float c = 0.0f;
+            if (a.dneg) {  // uniform
+                c = a.dneg[bb[q] * (int64_t)N + k];
                 if constexpr (P == 2) {
-                    const float s = a.sneg[bb[u] * (int64_t)N + k];
-                    c = s > 0.0f ? gg / s : 0.0f;
+                    const float sc = a.sneg[bb[q] * (int64_t)N + k];
+                    c = sc > 0.0f ? c / sc : 0.0f;
                 }
-                coef[u] = m + u < m1 ? -c : 0.0f;
             }
+            coef[u] = -c;
+        }
 #pragma unroll
-            for (int u = 0; u < 2; ++u) neg_accumulate<P, NQ>(acc, ya[u], p, coef[u]);
+        for (int u = 0; u < kFly; ++u) {
+            const int q = q0 + u;
+            if (q < cnt) {
+                if (q > 0 && gg[q] != gg[q - 1]) {
+                    flush(gg[q - 1]);
+#pragma unroll
+                    for (int e = 0; e < NQ; ++e) acc.v[e] = make_float4(0.f, 0.f, 0.f, 0.f);
+                }
+                neg_accumulate<P, NQ>(acc, ya[u], pr[u], coef[u]);
+            }
         }
     }
-    neg_store_row(a.ql + (int64_t)row * d, d, lane, acc);
-    neg_store_row(a.xl + (int64_t)row * d, d, lane, neg_load_row<NQ>(a.ent + x.hl[row] * (int64_t)d, d, lane));
+    flush(gg[cnt - 1]);
+}
+
+template <int NQ>
+__global__ __launch_bounds__(256) void tneg_pair_bwd_p2_kernel(NegIdx x, const int32_t *k_sseg, const float *partial, float *ql)
+{
+    const int lane = threadIdx.x & 63;
+    const int64_t w = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    const int N = (int)x.N, d = x.d;
+    const int64_t j = w / N;
+    const int k = (int)(w % N);
+    const int64_t p0 = j * kNegSeg;
+    if (p0 >= x.B) return;
+    const int64_t p1 = p0 + kNegSeg < x.B ? p0 + kNegSeg : x.B;
+    const int g = k_sseg[p1 - 1];
+    const int s0 = x.k_seg[g], s1 = x.k_seg[g + 1];
+    if (s1 <= p0 + kNegSeg || s0 < p0) return;  // no group starts here and continues
+    const int64_t je = (s1 - 1) / kNegSeg;
+    NegRow<NQ> acc = neg_load_row<NQ>(partial + ((j * N + k) * 2 + 1) * (int64_t)d, d, lane);
+    constexpr int kFly = NQ == 1 ? 8 : (NQ == 2 ? 4 : 2);
+    for (int64_t jj = j + 1; jj <= je; jj += kFly) {
+        NegRow<NQ> t[kFly];
+#pragma unroll
+        for (int u = 0; u < kFly; ++u) t[u] = neg_load_row<NQ>(partial + (((jj + u <= je ? jj + u : je) * N + k) * 2) * (int64_t)d, d, lane);
+#pragma unroll
+        for (int u = 0; u < kFly; ++u)
+            if (jj + u <= je) {
+#pragma unroll
+                for (int e = 0; e < NQ; ++e)
+                    acc.v[e] = make_float4(acc.v[e].x + t[u].v[e].x, acc.v[e].y + t[u].v[e].y, acc.v[e].z + t[u].v[e].z,
+                                           acc.v[e].w + t[u].v[e].w);
+            }
+    }
+    neg_store_row(ql + (int64_t)(x.rowp[g] + k) * d, d, lane, acc);
+}
+
+// Left operands of the P rows for dM: the negatives' entity rows in list order (one wave per row).
+template <int NQ>
+__global__ __launch_bounds__(256) void tneg_prow_operands_kernel(NegIdx x, const float *ent, float *xl)
+{
+    const int lane = threadIdx.x & 63;
+    const int64_t w = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    const int64_t g = w / x.N;
+    if (g >= x.k_num[0]) return;
+    const int row = x.rowp[g] + (int)(w % x.N);
+    neg_store_row(xl + (int64_t)row * x.d, x.d, lane, neg_load_row<NQ>(ent + x.hl[row] * (int64_t)x.d, x.d, lane));
 }
 
 // Occurrence rows in the order of the entity inspection, concat(h, t, neg): the list's dX rows are
-// added up per positive (own row and a row) and per (chunk, negative) over the chunk's groups.
+// added up per positive (own row and a row: one wave each, workgroups [0, ceil(B / 4))) and per
+// (chunk, negative) over the chunk's groups (one workgroup each: its four waves take the groups
+// i = wave, wave + 4, ... and their sums are added in wave order through LDS).
 template <int NQ>
 __global__ __launch_bounds__(256) void tneg_occ_kernel(NegIdx x, const float *dxl, const int32_t *glist,
                                                        const int32_t *gcount, float *occ)
 {
-    const int lane = threadIdx.x & 63;
-    const int64_t w = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    __shared__ float4 s_part[3][NQ * kWave];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int d = x.d;
-    if (w < x.B) {
+    const int64_t pos_blocks = ceil_div(x.B, 4);
+    if ((int64_t)blockIdx.x < pos_blocks) {
+        const int64_t w = (int64_t)blockIdx.x * 4 + wave;
+        if (w >= x.B) return;
         const NegRow<NQ> dp = neg_load_row<NQ>(dxl + (int64_t)x.rowpos[w] * d, d, lane), da = neg_load_row<NQ>(dxl + (int64_t)x.rowa[w] * d, d, lane);
         NegRow<NQ> oh, ot;
 #pragma unroll
@@ -442,7 +524,7 @@ __global__ __launch_bounds__(256) void tneg_occ_kernel(NegIdx x, const float *dx
         neg_store_row(occ + (x.B + w) * (int64_t)d, d, lane, ot);
         return;
     }
-    const int64_t q = w - x.B;
+    const int64_t q = (int64_t)blockIdx.x - pos_blocks;  // (chunk, negative); uniform for the workgroup
     if (q >= x.n_chunks * x.N) return;
     const int64_t c = q / x.N;
     const int k = (int)(q % x.N);
@@ -450,20 +532,37 @@ __global__ __launch_bounds__(256) void tneg_occ_kernel(NegIdx x, const float *dx
     NegRow<NQ> acc;
 #pragma unroll
     for (int e = 0; e < NQ; ++e) acc.v[e] = make_float4(0.f, 0.f, 0.f, 0.f);
-    for (int i = 0; i < cnt; i += 4) {  // four groups in flight
-        NegRow<NQ> r[4];
+    constexpr int kFly = NQ == 1 ? 8 : (NQ == 2 ? 4 : 2);  // groups in flight per wave
+    for (int i = wave; i < cnt; i += 4 * kFly) {
+        NegRow<NQ> r[kFly];
 #pragma unroll
-        for (int u = 0; u < 4; ++u) r[u] = neg_load_row<NQ>(dxl + (int64_t)(glist[c * x.C + (i + u < cnt ? i + u : cnt - 1)] + k) * d, d, lane);
+        for (int u = 0; u < kFly; ++u) {
+            const int iu = i + 4 * u;
+            r[u] = neg_load_row<NQ>(dxl + (int64_t)(glist[c * x.C + (iu < cnt ? iu : i)] + k) * d, d, lane);
+        }
 #pragma unroll
-        for (int u = 0; u < 4; ++u)
-            if (i + u < cnt) {
+        for (int u = 0; u < kFly; ++u)
+            if (i + 4 * u < cnt) {
 #pragma unroll
                 for (int e = 0; e < NQ; ++e)
                     acc.v[e] = make_float4(acc.v[e].x + r[u].v[e].x, acc.v[e].y + r[u].v[e].y, acc.v[e].z + r[u].v[e].z,
                                            acc.v[e].w + r[u].v[e].w);
             }
     }
-    neg_store_row(occ + (2 * x.B + q) * (int64_t)d, d, lane, acc);
+    if (wave > 0) {
+#pragma unroll
+        for (int e = 0; e < NQ; ++e) s_part[wave - 1][e * kWave + lane] = acc.v[e];
+    }
+    __syncthreads();
+    if (wave == 0) {
+#pragma unroll
+        for (int e = 0; e < NQ; ++e) {
+            const float4 p1 = s_part[0][e * kWave + lane], p2 = s_part[1][e * kWave + lane], p3 = s_part[2][e * kWave + lane];
+            acc.v[e] = make_float4((acc.v[e].x + p1.x) + (p2.x + p3.x), (acc.v[e].y + p1.y) + (p2.y + p3.y),
+                                   (acc.v[e].z + p1.z) + (p2.z + p3.z), (acc.v[e].w + p1.w) + (p2.w + p3.w));
+        }
+        neg_store_row(occ + (2 * x.B + q) * (int64_t)d, d, lane, acc);
+    }
 }
 
 // ---- host side --------------------------------------------------------------------------------
@@ -619,7 +718,12 @@ int launch_transr_neg_bwd(const kge_tables *tab, const kge_batch *bat, const kge
     pa.xl = xl, pa.ql = ql, pa.qr = qr;
     const dim3 agrid((unsigned)ceil_div(s.B, 4)), pgrid((unsigned)ceil_div(s.G_cap * s.N, 4));
     TNEG_BY_WIDTH(d, TNEG_BY_NORM(tab->norm_p, tneg_pair_bwd_a_kernel, agrid, x, pa));
-    TNEG_BY_WIDTH(d, TNEG_BY_NORM(tab->norm_p, tneg_pair_bwd_p_kernel, pgrid, x, pa));
+    float *ppart = reinterpret_cast<float *>(ws + l.ppart);
+    const int32_t *k_sseg = reinterpret_cast<const int32_t *>(fws + fl.ksseg);
+    const dim3 sgrid((unsigned)ceil_div(ceil_div(s.B, kNegSeg) * s.N, 4));
+    TNEG_BY_WIDTH(d, TNEG_BY_NORM(tab->norm_p, tneg_pair_bwd_p1_kernel, sgrid, x, pa, k_sseg, ppart));
+    TNEG_BY_WIDTH(d, hipLaunchKernelGGL(tneg_pair_bwd_p2_kernel<NQ_>, sgrid, dim3(256), 0, st, x, k_sseg, ppart, ql));
+    TNEG_BY_WIDTH(d, hipLaunchKernelGGL(tneg_prow_operands_kernel<NQ_>, pgrid, dim3(256), 0, st, x, tab->ent, xl));
     hipLaunchKernelGGL(tneg_chunk_groups_kernel, dim3((unsigned)s.n_chunks), dim3(64), 0, st, x, glist, gcount);
     timeline_mark(bat->timeline, st, "tneg_pair_bwd kernels");
 
@@ -638,7 +742,7 @@ int launch_transr_neg_bwd(const kge_tables *tab, const kge_batch *bat, const kge
     hipLaunchKernelGGL(transr_dm_finish_kernel, dim3((unsigned)ceil_div((int64_t)d * d / 4, 256), (unsigned)s.dsplit), dim3(256),
                        0, st, da);
     timeline_mark(bat->timeline, st, "transr_dm_finish_kernel");
-    TNEG_BY_WIDTH(d, hipLaunchKernelGGL(tneg_occ_kernel<NQ_>, dim3((unsigned)ceil_div(s.B + s.NN, 4)), dim3(256), 0, st, x, dxl,
+    TNEG_BY_WIDTH(d, hipLaunchKernelGGL(tneg_occ_kernel<NQ_>, dim3((unsigned)(ceil_div(s.B, 4) + s.NN)), dim3(256), 0, st, x, dxl,
                                         glist, gcount, occ));
     timeline_mark(bat->timeline, st, "tneg_occ_kernel");
     KGE_CHECK_LAUNCH();

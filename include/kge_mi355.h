@@ -182,7 +182,8 @@ typedef struct kge_saved {
                                (with KGE_NEG_HEAD: counter-rotated tails t e^{-i theta}) */
     /* TransR / RESCAL, optional: the workspace the forward call of this batch was given (it
        holds the tile plans of the relation groups); kge_score_bwd then reuses them instead of
-       building its own.  NULL / 0: backward plans for itself. */
+       building its own.  NULL / 0: backward plans for itself.  Required for TransR with shared
+       negatives (the group list and the projected rows live there). */
     const void *fwd_workspace;
     size_t fwd_workspace_bytes;
 } kge_saved;
@@ -219,6 +220,15 @@ int kge_residual_fwd(const kge_tables *tab, const kge_batch *bat, float *out, vo
  * per-relation MFMA contractions and needs kge_score_fwd_workspace() bytes of workspace;
  * without it every triple streams its own projection.  `residual` [B, dim] receives the
  * projected rows (TransR: the residual, RESCAL: E[h] Proj[r]) that kge_score_bwd consumes.
+ * TransR with shared negatives (bat->neg, bat->rel_insp and neg all set; dim % 4 == 0, dim <= 1024):
+ * the pair scores of the reference's neg_transR (apps/examples/examples.py:1447-1480, one
+ * vector x matrix product per (positive, negative) pair) are formed from two projections,
+ * (x - n) M + R = (x M + R) - n M, and every negative is projected once per (relation, chunk) group
+ * of the batch instead of once per pair.  pos, neg and residual ([B, dim], the positives' residual
+ * rows) come out of the one call; the workspace (kge_score_fwd_workspace with bat->neg set) keeps
+ * the group list and the projected rows and must be handed to kge_score_bwd as
+ * kge_saved.fwd_workspace.  RESCAL with shared negatives, and TransR shapes outside the grouped
+ * kernels, are scored through kge_flatten_negatives.
  * RotatE: `residual` [B, dim] receives the rotated heads h e^{i theta}; the shared-negative
  * kernels (forward and backward) load them instead of recomputing a sincos per element, so it
  * is required whenever negatives are scored (filled by this call when pos is requested, or
@@ -313,9 +323,10 @@ int kge_build_index(const int64_t *r, int64_t *uniq, int64_t *buf, int64_t *cnt,
  * Shared negatives written out as explicit triples, the way the reference's neg_transR defines
  * them (apps/examples/examples.py:1447-1480: every view is flattened to batch * blocksize rows).
  * Outputs have B * (1 + n_neg) entries: the B positives first, then row B + b * n_neg + k =
- * (h[b], r[b], neg[(b / chunk) * n_neg + k]).  TransR / RESCAL score shared negatives through
- * this list and the grouped per-relation kernels (their projection depends on the positive's
- * relation, so a negative row cannot be staged once per chunk as for the other models).
+ * (h[b], r[b], neg[(b / chunk) * n_neg + k]).  RESCAL scores shared negatives through this list
+ * and the grouped per-relation kernels (the projection depends on the positive's relation, so a
+ * negative row cannot be staged once per chunk as for the other models); TransR has the grouped
+ * form of kge_score_fwd and uses the list only for shapes that form does not take.
  */
 int kge_flatten_negatives(const kge_batch *bat, int64_t *h_flat, int64_t *r_flat, int64_t *t_flat,
                           void *stream);
