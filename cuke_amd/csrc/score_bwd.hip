@@ -386,10 +386,11 @@ __device__ __forceinline__ void bwd_tile_body(const TileArgs &a, int lid, float 
                     for (int e = 0; e < 4; ++e) {
                         const float ur = OWNER_POS ? o0p[e] - lvp[e] : lvp[e] - o0p[e];
                         const float ui = OWNER_POS ? o1p[e] - lv1p[e] : lv1p[e] - o1p[e];
-                        const float m2 = fmaf(ur, ur, ui * ui);
-                        // u == 0 contributes k * 0 = 0 whatever k is: clamping m2 away from zero (one max)
-                        // replaces the compare-and-select that would force rs = 0 there
-                        const float rs = __builtin_amdgcn_rsqf(fmaxf(m2, 1e-37f));
+                        // u == 0 contributes k * 0 = 0 whatever k is, so |u|^2 only has to stay away from zero:
+                        // the 1e-37 rides in the multiply-add that forms it (far below one ulp of any |u|^2
+                        // that is not itself denormal) instead of a compare-and-select or a max
+                        const float m2 = fmaf(ur, ur, fmaf(ui, ui, 1e-37f));
+                        const float rs = __builtin_amdgcn_rsqf(m2);
                         const float k = OWNER_POS ? -g * rs : g * rs;  // d/da = -g u/|u| ; d/dt' = +g u/|u|
                         a0p[e] = fmaf(k, ur, a0p[e]);
                         a1p[e] = fmaf(k, ui, a1p[e]);
@@ -541,10 +542,17 @@ static int launch_tiles(TileArgs a, float *g0, float *g1, float *occ_neg, int64_
         const size_t lds = tile_lds_bytes<MODEL, 4>(fi);
         hipLaunchKernelGGL((bwd_tile_kernel<MODEL, P, 4, false>), dim3(gh + gn + nh + nn + fi.blocks), dim3(256), lds, st,
                            a, g0, g1, occ_neg, TileGrid{(int)gh, (int)gn, (int)nh, (int)nn}, fi);
-    } else {
+    } else if (big >= 512) {
         const unsigned gh = xcd_grid(gx, ceil_div(a.C, 32), n_chunks), gn = xcd_grid(gx, ceil_div(a.N, 32), n_chunks);
         const size_t lds = tile_lds_bytes<MODEL, 2>(fi);
         hipLaunchKernelGGL((bwd_tile_kernel<MODEL, P, 2, false>), dim3(gh + gn + fi.blocks), dim3(256), lds, st, a, g0, g1,
+                           occ_neg, TileGrid{(int)gh, (int)gn, 0, 0}, fi);
+    } else {
+        // a batch this small leaves one or two 32-owner workgroups per CU: 16-owner tiles double the
+        // waves that hide each other's latency
+        const unsigned gh = xcd_grid(gx, ceil_div(a.C, 16), n_chunks), gn = xcd_grid(gx, ceil_div(a.N, 16), n_chunks);
+        const size_t lds = tile_lds_bytes<MODEL, 1>(fi);
+        hipLaunchKernelGGL((bwd_tile_kernel<MODEL, P, 1, false>), dim3(gh + gn + fi.blocks), dim3(256), lds, st, a, g0, g1,
                            occ_neg, TileGrid{(int)gh, (int)gn, 0, 0}, fi);
     }
     KGE_CHECK_LAUNCH();
