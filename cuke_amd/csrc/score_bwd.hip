@@ -41,7 +41,12 @@ struct TileArgs {
 };
 
 constexpr int kTI = 64;       // columns of the row per workgroup
-constexpr int kKL = 32;       // looper rows staged per step
+// Looper rows staged per step.  The 64-owner TransH tile holds two owner planes, two accumulator
+// planes and three coefficient planes; with 32-row steps its prefetch registers spill (about 50
+// registers per lane go through scratch memory every step: same speed, three times the memory
+// traffic), with 16-row steps everything stays in registers.
+template <int MODEL, int RO>
+constexpr int looper_rows() { return MODEL == KGE_TRANSH && RO == 4 ? 16 : 32; }
 constexpr int kLP = kTI + 4;  // LDS pitch of a staged row
 
 template <int MODEL, bool OWNER_POS, int RO>
@@ -51,6 +56,7 @@ struct TileShape {
     static constexpr int NPL = (kRot || (kTH && !OWNER_POS)) ? 2 : 1;
     static constexpr int NC = kTH ? 3 : 1;
     static constexpr int PG = TO + 4;
+    static constexpr int kKL = looper_rows<MODEL, RO>();
     static constexpr int kLdsFloats = NPL * kKL * kLP + NC * kKL * PG;
 };
 
@@ -85,6 +91,7 @@ __device__ __forceinline__ void bwd_tile_body(const TileArgs &a, int lid, float 
     constexpr int NC = kTH ? 3 : 1;                             // coefficient planes: g~, c, e
     constexpr int NOUT = (kRot || (kTH && OWNER_POS)) ? 2 : 1;
     constexpr int PG = TO + 4;
+    constexpr int kKL = looper_rows<MODEL, RO>();  // (narrow tiles share the 64-owner launch and its step)
     constexpr int SL = kKL / 16;                        // looper float4 per thread per plane
     constexpr int CPT = (TO * kKL / 4 + 255) / 256;     // coefficient float4 per thread per plane
     static_assert(!NARROW || RO == 4, "narrow tiles share the 64-owner LDS layout");
@@ -224,9 +231,9 @@ __device__ __forceinline__ void bwd_tile_body(const TileArgs &a, int lid, float 
             const int f = tid + 256 * s;  // float4 index inside the block
             int bl, kl;                   // positive / negative of the first element
             bool inside;
-            if constexpr (OWNER_POS) {    // rows = owners (positives), 8 float4 of loopers each
-                const int orow = f >> 3;
-                bl = ot0 + orow, kl = l0 + (f & 7) * 4;
+            if constexpr (OWNER_POS) {    // rows = owners (positives), kKL / 4 float4 of loopers each
+                const int orow = f / (kKL / 4);
+                bl = ot0 + orow, kl = l0 + (f % (kKL / 4)) * 4;
                 inside = orow < TO && bl < a.C;
             } else {                      // rows = loopers (positives), TO/4 float4 of owners each
                 const int lrow = f / (TO / 4);
@@ -298,7 +305,7 @@ __device__ __forceinline__ void bwd_tile_body(const TileArgs &a, int lid, float 
             for (int pl = 0; pl < NC; ++pl) {
                 const float4 v = cv[pl];
                 if constexpr (OWNER_POS) {
-                    const int orow = f >> 3, l = (f & 7) * 4;
+                    const int orow = f / (kKL / 4), l = (f % (kKL / 4)) * 4;
                     if (orow < TO) {
                         sG[pl][l + 0][orow] = v.x;
                         sG[pl][l + 1][orow] = v.y;

@@ -169,7 +169,10 @@ __global__ __launch_bounds__(256, KGE_TILE_OCC) void score_neg_kernel(NegArgs a,
                         kScaled ? scale4(rt[pl][q], kSgnScale) : rt[pl][q];
             __syncthreads();
             if (s + 1 < nslice) load_slice((s + 1) * kKD, pass);
-#pragma unroll
+            // (TransH keeps three sums per pair, RotatE two row planes: unrolled all the way, the hoisted LDS reads push the
+            // 4 x 4 micro-tile over the register budget and twenty to fifty registers per lane go through
+            // scratch memory every step)
+#pragma unroll((MODEL == KGE_TRANSH || (MODEL == KGE_ROTATE && RB == 4)) ? 2 : kKD / 4)
             for (int i4 = 0; i4 < kKD / 4; ++i4) {
                 float4 av[NPA][RB], tv[NPT][RK];
 #pragma unroll
