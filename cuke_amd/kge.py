@@ -591,9 +591,10 @@ class TrainStep:
         """[(kernel name, mean milliseconds)] of one step, in launch order: ``steps`` steps are run with an
         event recorded behind every kernel (kge_batch.timeline) and read back after each step.  Event
         records between the kernels cost a little themselves, so the sum is an upper bound of the
-        step time that ``run()`` alone takes.  ``batches``: batch numbers to rotate over.  ``lead``: a
-        large tensor that is zero-filled on the stream in front of every step, so that the host has
-        enqueued the whole step before the device starts on it and the intervals hold no launch gaps."""
+        step time that ``run()`` alone takes.  ``batches``: batch numbers to rotate over.  ``lead``: work
+        enqueued on the stream in front of every step, so that the host has enqueued the whole step
+        before the device starts on it and the intervals hold no launch gaps: a callable, or a large
+        tensor that is zero-filled (which also empties the caches in front of every step)."""
         L = self.L
         tl = L.kge_timeline_create(64)
         if not tl:
@@ -608,7 +609,9 @@ class TrainStep:
                 if batches:
                     self.select(batches[i % len(batches)])
                 self.bat.timeline = tl
-                if lead is not None:
+                if callable(lead):
+                    lead()
+                elif lead is not None:
                     lead.zero_()
                 _lib.check(L.kge_timeline_begin(tl, st), "kge_timeline_begin")
                 try:

@@ -37,6 +37,7 @@ def assert_close(got, ref, rtol=RTOL, what="", rows=False, outliers=None, global
     if global_floor:
         bound = bound + global_floor * rtol * float(np.sqrt(np.mean(ref * ref)))
     bad = err > bound
+    _log_tolerance(what, err, bound, rtol, rows, outliers, global_floor)
     if outliers is not None and bad.any():
         frac, factor = outliers
         if bad.mean() <= frac and not (err > factor * bound).any():
@@ -45,6 +46,21 @@ def assert_close(got, ref, rtol=RTOL, what="", rows=False, outliers=None, global
         i = np.unravel_index(np.argmax(err - bound), err.shape)
         raise AssertionError(f"{what}: {int(bad.sum())}/{ref.size} outside tolerance; worst at {i}: "
                              f"got {got[i]!r} ref {ref[i]!r} err {err[i]:.3e} bound {bound[i]:.3e}")
+
+
+def _log_tolerance(what, err, bound, rtol, rows, outliers, global_floor):
+    """With KGE_TOL_LOG=<file> every comparison appends its worst error relative to its bound (one JSON line):
+    the measured margins behind the tolerance table of the design notes."""
+    import json
+    import os
+    path = os.environ.get("KGE_TOL_LOG")
+    if not path:
+        return
+    ratio = float(np.max(err / np.maximum(bound, 1e-300)))
+    test = os.environ.get("PYTEST_CURRENT_TEST", "").split(" ")[0]
+    with open(path, "a") as f:
+        f.write(json.dumps({"test": test, "what": what, "n": int(err.size), "worst_over_bound": ratio,
+                            "rtol": rtol, "rows": bool(rows), "outliers": outliers, "global_floor": global_floor}) + "\n")
 
 
 def gpu_model(w, device="cuda:0"):

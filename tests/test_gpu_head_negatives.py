@@ -54,7 +54,7 @@ def test_head_negatives(oracle, model, shape, p):
         pytest.skip("norm order only matters for the translation models")
     w = synth.custom_workload(model, n_ent=300, n_rel=9, norm_p=p, sigma=0.3, gamma=4.0, ent_zipf=1.1, seed=p,
                               lattice=(p == 1), **shape)
-    out = (1e-4, 4.0) if model == "RotatE" else None
+    out = (1e-5, 4.0) if model == "RotatE" else None
     compare(*both(oracle, w), what=f"{model} {shape} p={p}", outliers=out)
 
 
@@ -70,7 +70,7 @@ def test_head_negatives_random_shapes(oracle, seed):
     spec = draw(seed)
     model = spec.pop("model")
     w = synth.custom_workload(model, seed=seed, **spec)
-    out = (1e-4, 4.0) if model == "RotatE" else None
+    out = (1e-5, 4.0) if model == "RotatE" else None
     compare(*both(oracle, w, seed=seed), what=f"seed {seed} {model} {spec}", outliers=out,
             floor=0.1 if w.dim < 8 else 0.0)
 

@@ -52,7 +52,7 @@ def test_random_shape(oracle, seed):
                           p=w.norm_p)
     assert np.array_equal(g.ent_ids.cpu().numpy(), ref.ent_ids), what
     assert np.array_equal(g.rel_ids.cpu().numpy(), ref.rel_ids), what
-    out = (1e-4, 4.0) if model == "RotatE" else None
+    out = (1e-5, 4.0) if model == "RotatE" else None
     floor = 0.1 if w.dim < 8 else 0.0
     assert_close(g.ent_rows.cpu().numpy(), ref.ent_rows, what=what + " entity rows", rows=True, outliers=out, global_floor=floor)
     assert_close(g.rel_rows.cpu().numpy(), ref.rel_rows, what=what + " relation rows", rows=True, outliers=out, global_floor=floor)
