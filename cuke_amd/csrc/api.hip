@@ -8,7 +8,8 @@ int launch_score_pos(const kge_tables *, const kge_batch *, float *, float *, fl
 int launch_score_pos_fused(const kge_tables *, const kge_batch *, float *, float *, float *, const FusedInsp *,
                            hipStream_t);
 int launch_score_neg(const kge_tables *, const kge_batch *, const float *, const float *, float *, float *,
-                     const FusedInsp *, hipStream_t);
+                     const FusedInsp *, void *, size_t, hipStream_t);
+size_t neg_split_workspace(const kge_tables *, const kge_batch *);
 int launch_transr_fwd(const kge_tables *, const kge_batch *, float *, float *, void *, size_t, hipStream_t);
 size_t transr_fwd_workspace(const kge_tables *, const kge_batch *);
 int launch_transr_neg_fwd(const kge_tables *, const kge_batch *, float *, float *, float *, void *, size_t, hipStream_t);
@@ -175,6 +176,7 @@ size_t kge_score_fwd_workspace(const kge_tables *tab, const kge_batch *bat)
         if (nb) return nb;
     }
     if ((tab->model == KGE_TRANSR || tab->model == KGE_RESCAL) && bat->rel_insp) return transr_fwd_workspace(tab, bat);
+    if (tab->model == KGE_TRANSE || tab->model == KGE_ROTATE) return neg_split_workspace(tab, bat);  // small batches only
     return 0;
 }
 
@@ -228,7 +230,7 @@ int kge_score_fwd(const kge_tables *tab, const kge_batch *bat, float *pos, float
     }
     if (want_neg) {
         rc = launch_score_neg(tab, bat, side_pos, tab->model == KGE_ROTATE ? residual : nullptr, neg, side_neg,
-                              fuse ? &fi1 : nullptr, st);
+                              fuse ? &fi1 : nullptr, workspace, workspace_bytes, st);
         timeline_mark(bat->timeline, st, "score_neg_kernel");
         return rc;
     }

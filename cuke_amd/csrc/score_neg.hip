@@ -31,6 +31,11 @@ struct NegArgs {
     float gamma;
     int vec, n_chunks;
     float rsign;            // +1: negatives replace the tail; -1: the head (see load_query)
+    // Small batches: the reduction axis is split over `ksplit` workgroups per tile, each writes the raw
+    // sums of its slices to plane `split` of `partial` ([ksplit][B * N]) and score_neg_finish_kernel
+    // adds the planes and finishes the scores.  ksplit <= 1: one workgroup per tile, scores written directly.
+    int ksplit;
+    float *partial;
 };
 
 typedef float v4f __attribute__((ext_vector_type(4)));
@@ -83,7 +88,12 @@ __global__ __launch_bounds__(256, KGE_TILE_OCC) void score_neg_kernel(NegArgs a,
     const int tid = threadIdx.x, tx = tid & 15, ty = tid >> 4;
     const int srow = tid >> 3, scol = (tid & 7) * 4;
     int c, tile_y, tile_x;
-    if (!xcd_tile(blockIdx.x - fi.blocks, (a.N + TN - 1) / TN, (a.C + TB - 1) / TB, a.n_chunks, c, tile_y, tile_x)) return;
+    int lid = blockIdx.x - fi.blocks, split = 0;
+    if (a.ksplit > 1) {  // (never TransH: its w . t' sweep needs the whole row)
+        const int tiles = (int)(gridDim.x - fi.blocks) / a.ksplit;  // a multiple of 8: the tile keeps its XCD
+        split = lid / tiles, lid -= split * tiles;
+    }
+    if (!xcd_tile(lid, (a.N + TN - 1) / TN, (a.C + TB - 1) / TB, a.n_chunks, c, tile_y, tile_x)) return;
     const int bt0 = tile_y * TB, kt0 = tile_x * TN;
     const int d = a.d, half = d >> 1;
     const int klen = MODEL == KGE_ROTATE ? half : d;
@@ -147,14 +157,21 @@ __global__ __launch_bounds__(256, KGE_TILE_OCC) void score_neg_kernel(NegArgs a,
         for (int k = 0; k < RK; ++k) acc[i][k] = 0.0f, cdot[i][k] = 0.0f, acc2[i][k] = 0.0f;
 
     const int nslice = (klen + kKD - 1) / kKD;
+    int slice0 = 0, slice1 = nslice;  // this workgroup's share of the reduction axis
+    if (a.ksplit > 1) {
+        const int per = (nslice + a.ksplit - 1) / a.ksplit;
+        slice0 = split * per;
+        slice1 = slice0 + per < nslice ? slice0 + per : nslice;
+    }
     // One sweep over the reduction axis.  `pass` is a compile-time tag: TransH's first sweep (the
     // w . t' dot products) and second sweep (the norm) get their own straight-line inner loops; as a
     // run-time value it put a branch around every pair of the micro-tile.
     auto sweep = [&](auto pass_tag) {
         constexpr int pass = decltype(pass_tag)::value;
-        load_slice(0, pass);
+        constexpr int kInnerUnroll = (MODEL == KGE_TRANSH || (MODEL == KGE_ROTATE && RB == 4)) ? 2 : kKD / 4;
+        if (slice0 < slice1) load_slice(slice0 * kKD, pass);
 #pragma unroll 1
-        for (int s = 0; s < nslice; ++s) {
+        for (int s = slice0; s < slice1; ++s) {
 #pragma unroll
             for (int q = 0; q < SB; ++q)
 #pragma unroll
@@ -168,11 +185,11 @@ __global__ __launch_bounds__(256, KGE_TILE_OCC) void score_neg_kernel(NegArgs a,
                     *reinterpret_cast<float4 *>(&sT[pl][srow + 32 * q][scol]) =
                         kScaled ? scale4(rt[pl][q], kSgnScale) : rt[pl][q];
             __syncthreads();
-            if (s + 1 < nslice) load_slice((s + 1) * kKD, pass);
+            if (s + 1 < slice1) load_slice((s + 1) * kKD, pass);
             // (TransH keeps three sums per pair, RotatE two row planes: unrolled all the way, the hoisted LDS reads push the
             // 4 x 4 micro-tile over the register budget and twenty to fifty registers per lane go through
             // scratch memory every step)
-#pragma unroll((MODEL == KGE_TRANSH || (MODEL == KGE_ROTATE && RB == 4)) ? 2 : kKD / 4)
+#pragma unroll kInnerUnroll
             for (int i4 = 0; i4 < kKD / 4; ++i4) {
                 float4 av[NPA][RB], tv[NPT][RK];
 #pragma unroll
@@ -300,6 +317,10 @@ __global__ __launch_bounds__(256, KGE_TILE_OCC) void score_neg_kernel(NegArgs a,
             const int kl = kt0 + tx + 16 * k;
             if (kl >= a.N) continue;
             float s = acc[i][k];
+            if (a.ksplit > 1) {  // raw sum of this workgroup's slices; finished by score_neg_finish_kernel
+                a.partial[(int64_t)split * a.plane + rowoff + kl] = s;
+                continue;
+            }
             if constexpr (kScaled) s *= kSgnUnscale, acc2[i][k] *= kSgnUnscale;
             if constexpr (MODEL == KGE_TRANSE || MODEL == KGE_TRANSH) s = P == 2 ? sqrtf(s) : s;
             if constexpr (MODEL == KGE_ROTATE) s = a.gamma - s;
@@ -449,6 +470,44 @@ static size_t neg_lds(int planes, int TB, int TN, int planes_t, const FusedInsp 
     return fi.blocks > 0 && (size_t)fi.lds_bytes > own ? (size_t)fi.lds_bytes : own;
 }
 
+// Adds the partial planes of a split reduction axis and finishes the scores.
+template <int MODEL, int P>
+__global__ __launch_bounds__(256) void score_neg_finish_kernel(const float *partial, int ksplit, int64_t plane, float gamma,
+                                                               float *out)
+{
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= plane) return;
+    float s = partial[i];
+    for (int q = 1; q < ksplit; ++q) s += partial[(int64_t)q * plane + i];
+    if constexpr (MODEL == KGE_TRANSE) s = P == 2 ? sqrtf(s) : s;
+    if constexpr (MODEL == KGE_ROTATE) s = gamma - s;
+    out[i] = s;
+}
+
+// Workgroups per tile along the reduction axis.  A batch whose 32 x 32 tiles leave one or two
+// workgroups per CU runs every instruction at its full latency (a single wave per SIMD has nobody
+// to interleave with): splitting the row over up to four workgroups multiplies the waves.  Only
+// for the models whose pair score is one plain sum over the row (TransE, RotatE).
+int neg_ksplit(const kge_tables *tab, const kge_batch *bat)
+{
+    if (!bat->neg || bat->chunk <= 0 || (tab->model != KGE_TRANSE && tab->model != KGE_ROTATE)) return 1;
+    const int64_t n_chunks = bat->batch / bat->chunk;
+    if (n_chunks <= 0 || ceil_div(bat->chunk, 64) * ceil_div(bat->n_neg, 64) * n_chunks >= 1024) return 1;  // (64 x 64 tiles)
+    const int64_t tiles = xcd_grid(ceil_div(bat->n_neg, 32), ceil_div(bat->chunk, 32), n_chunks);
+    const int64_t klen = tab->model == KGE_ROTATE ? tab->dim / 2 : tab->dim;
+    const int64_t nslice = ceil_div(klen, kKD);
+    int64_t s = 1024 / tiles;
+    s = s > 4 ? 4 : s;
+    while (s > 1 && nslice / s < 4) --s;
+    return s < 1 ? 1 : (int)s;
+}
+
+size_t neg_split_workspace(const kge_tables *tab, const kge_batch *bat)
+{
+    const int s = neg_ksplit(tab, bat);
+    return s > 1 ? sizeof(float) * (size_t)s * (size_t)(bat->batch * bat->n_neg) : 0;
+}
+
 template <int MODEL, int P>
 static int launch_neg_mp(const NegArgs &a, int64_t n_chunks, bool dot_valu, const FusedInsp &fi, hipStream_t st)
 {
@@ -474,6 +533,18 @@ static int launch_neg_mp(const NegArgs &a, int64_t n_chunks, bool dot_valu, cons
     }
     const size_t lds = neg_lds(NPA, TB, TN, NPT, fi);
     const bool save = MODEL == KGE_TRANSH && a.side_neg;
+    if (a.ksplit > 1) {  // (neg_ksplit: 32 x 32 tiles of TransE / RotatE)
+        if constexpr (MODEL == KGE_TRANSE || MODEL == KGE_ROTATE) {
+            const unsigned tiles = xcd_grid(ceil_div(a.N, TN), ceil_div(a.C, TB), n_chunks);
+            hipLaunchKernelGGL((score_neg_kernel<MODEL, P, 2, 2, false>), dim3(tiles * a.ksplit + (unsigned)fi.blocks), dim3(256),
+                               lds, st, a, fi);
+            hipLaunchKernelGGL((score_neg_finish_kernel<MODEL, P>), dim3((unsigned)ceil_div(a.plane, 256)), dim3(256), 0, st,
+                               a.partial, a.ksplit, a.plane, a.gamma, a.out);
+            KGE_CHECK_LAUNCH();
+            return KGE_OK;
+        }
+        return KGE_EINVAL;
+    }
     if (tile == 3) {  // 32 positives x 64 negatives
         if (save) hipLaunchKernelGGL((score_neg_kernel<MODEL, P, 2, 4, true>), grid, dim3(256), lds, st, a, fi);
         else hipLaunchKernelGGL((score_neg_kernel<MODEL, P, 2, 4, false>), grid, dim3(256), lds, st, a, fi);
@@ -489,7 +560,8 @@ static int launch_neg_mp(const NegArgs &a, int64_t n_chunks, bool dot_valu, cons
 }
 
 int launch_score_neg(const kge_tables *tab, const kge_batch *bat, const float *side_pos, const float *query,
-                     float *out, float *side_neg, const FusedInsp *fused, hipStream_t st)
+                     float *out, float *side_neg, const FusedInsp *fused, void *workspace, size_t workspace_bytes,
+                     hipStream_t st)
 {
     const FusedInsp fi = fused ? *fused : FusedInsp{};
     if (bat->batch == 0) return KGE_OK;
@@ -499,7 +571,11 @@ int launch_score_neg(const kge_tables *tab, const kge_batch *bat, const float *s
     const bool head = bat->neg_mode == KGE_NEG_HEAD;
     NegArgs a{tab->ent, tab->rel, tab->aux, head ? bat->t : bat->h, bat->r, bat->neg, side_pos, query, out, side_neg,
               bat->batch * bat->n_neg, (int)bat->chunk, (int)bat->n_neg, (int)tab->dim, (int)tab->rel_dim, tab->gamma,
-              vec ? 1 : 0, (int)n_chunks, head ? -1.0f : 1.0f};
+              vec ? 1 : 0, (int)n_chunks, head ? -1.0f : 1.0f, 1, nullptr};
+    // the reduction axis is split when the caller's workspace has room for the partial planes
+    const int ksplit = neg_ksplit(tab, bat);
+    if (ksplit > 1 && workspace && workspace_bytes >= neg_split_workspace(tab, bat) && aligned16(workspace))
+        a.ksplit = ksplit, a.partial = static_cast<float *>(workspace);
     const int p = tab->norm_p;
     const bool dv = pair_sums_valu(tab);
     switch (tab->model) {

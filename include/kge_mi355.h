@@ -229,6 +229,10 @@ int kge_residual_fwd(const kge_tables *tab, const kge_batch *bat, float *out, vo
  * the group list and the projected rows and must be handed to kge_score_bwd as
  * kge_saved.fwd_workspace.  RESCAL with shared negatives, and TransR shapes outside the grouped
  * kernels, are scored through kge_flatten_negatives.
+ * TransE / RotatE with shared negatives on small batches (the 32 x 32 pair tiles would leave one or
+ * two workgroups per CU): given kge_score_fwd_workspace() bytes of workspace the reduction axis of
+ * every tile is split over up to four workgroups (partial score planes in the workspace, a finishing
+ * kernel); without the workspace the same call runs one workgroup per tile.
  * RotatE: `residual` [B, dim] receives the rotated heads h e^{i theta}; the shared-negative
  * kernels (forward and backward) load them instead of recomputing a sincos per element, so it
  * is required whenever negatives are scored (filled by this call when pos is requested, or

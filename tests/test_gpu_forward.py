@@ -111,6 +111,34 @@ def test_shared_negative_scores(oracle, model, shape, p):
     assert_close(fw.neg.cpu().numpy(), negs, what=f"{model} neg {shape}")
 
 
+@pytest.mark.parametrize("model,dim,p", [("TransE", 640, 1), ("TransE", 520, 2), ("RotatE", 1000, 2), ("RotatE", 512, 2)])
+@pytest.mark.parametrize("mode", ["tail", "head"])
+def test_small_batch_splits_the_row_over_workgroups(oracle, model, dim, p, mode):
+    """A batch that leaves one or two tiles per CU has its reduction axis split over up to four workgroups per
+    tile (partial score planes in the forward workspace, a finishing kernel); without the workspace the same
+    call runs unsplit.  Both must reproduce the oracle."""
+    import ctypes as C
+    from cuke_amd import _lib
+    w = synth.custom_workload(model, n_ent=400, n_rel=11, dim=dim, batch=96, chunk=32, n_neg=40, norm_p=p, sigma=0.3,
+                              gamma=6.0, ent_zipf=1.1, seed=dim + p)
+    a = w.arrays
+    m, ix = gpu_model(w)
+    bat, _ = m._batch(ix["h"], ix["r"], ix["t"], ix["neg"], w.chunk, neg_mode=mode)
+    assert _lib.lib().kge_score_fwd_workspace(C.byref(m._tab), C.byref(bat)) >= 2 * 4 * w.batch * w.n_neg, \
+        "this shape is meant to take the split"
+    fw = m.score(ix["h"], ix["r"], ix["t"], ix["neg"], w.chunk, neg_mode=mode)
+    pos, negs = oracle.score(model, a["E"], a["R"], a["A"], a["h"], a["r"], a["t"], a["neg"], w.chunk, p=p, gamma=w.gamma,
+                             neg_mode=mode)
+    assert_close(fw.neg.cpu().numpy(), negs, what=f"{model} split negatives")
+    # the same call without a workspace: one workgroup per tile
+    unsplit = torch.empty_like(fw.neg)
+    res = torch.empty((w.batch, w.dim), dtype=torch.float32, device=fw.neg.device) if model == "RotatE" else None
+    _lib.check(_lib.lib().kge_score_fwd(C.byref(m._tab), C.byref(bat), fw.pos.data_ptr(), unsplit.data_ptr(), None, None,
+                                        res.data_ptr() if res is not None else None, None, 0,
+                                        C.c_void_p(torch.cuda.current_stream().cuda_stream)), "kge_score_fwd")
+    assert_close(unsplit.cpu().numpy(), negs, what=f"{model} unsplit negatives")
+
+
 @pytest.mark.parametrize("name,over", [
     ("cfg2_distmult", dict(n_ent=100_000, batch=1024)),
     ("cfg2_complex", dict(n_ent=100_000, batch=1024)),
