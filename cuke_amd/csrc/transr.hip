@@ -195,6 +195,18 @@ __device__ __forceinline__ void transr_thin_fwd_body(const GemmArgs &a, float *l
     __shared__ float s_rs[kThin];
     const int64_t rid = a.unique_ids[g];
     const float4 *M4 = reinterpret_cast<const float4 *>(a.proj + rid * (int64_t)d * d);
+    // The first kThinRing loads of the projection stream only depend on the relation: they are
+    // requested before the rows are staged and fly during the index chain and the row gathers.
+    const int cq = tid % nq4, ph = tid / nq4;
+    const bool active = ph < P;
+    // x is zero for k >= d, so a clamped (always valid) address needs no branch; threads beyond the
+    // last phase read what phase P - 1 reads and compute nothing
+    const int phc = active ? ph : P - 1;
+    auto loadm = [&](int k) { return M4[(int64_t)(k < d ? k : d - 1) * nq4 + cq]; };
+    float4 ring[kThinRing];
+#pragma unroll
+    for (int u = 0; u < kThinRing; ++u) ring[u] = loadm(phc + P * u);
+    __builtin_amdgcn_sched_barrier(0);
     if (tid < kThin) {
         const int b = tid < rows ? (MODE == 3 ? tt.p0 + tid : a.perm[tt.p0 + tid]) : (MODE == 3 ? tt.p0 : 0);
         s_b[tid] = b;
@@ -222,17 +234,10 @@ __device__ __forceinline__ void transr_thin_fwd_body(const GemmArgs &a, float *l
     }
     __syncthreads();
 
-    const int cq = tid % nq4, ph = tid / nq4;
-    const bool active = ph < P;
     float4 acc[4];
 #pragma unroll
     for (int r = 0; r < 4; ++r) acc[r] = make_float4(0.f, 0.f, 0.f, 0.f);
     if (active) {
-        // x is zero for k >= d, so a clamped (always valid) address needs no branch
-        auto loadm = [&](int k) { return M4[(int64_t)(k < d ? k : d - 1) * nq4 + cq]; };
-        float4 ring[kThinRing];
-#pragma unroll
-        for (int u = 0; u < kThinRing; ++u) ring[u] = loadm(ph + P * u);
         for (int k0 = ph; k0 < d; k0 += P * kThinRing) {
 #pragma unroll
             for (int u = 0; u < kThinRing; ++u) {
