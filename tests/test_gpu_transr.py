@@ -192,3 +192,39 @@ def test_shared_negatives_grouped_path_equals_the_flattened_one(oracle):
     flat = m._score_projected_negatives(ix["h"], ix["r"], ix["t"], ix["neg"], w.chunk)
     assert_close(fw.neg.cpu().numpy(), flat.neg.cpu().numpy(), what="grouped vs flattened negative scores")
     assert_close(fw.pos.cpu().numpy(), flat.pos.cpu().numpy(), what="grouped vs flattened positive scores")
+
+
+@pytest.mark.parametrize("mode", ["tail", "head"])
+def test_train_step_with_shared_negatives_and_margin_loss(oracle, mode):
+    """The preallocated training step drives the grouped shared-negative path: relation inspection on the
+    step's stream, entity inspection beside it, forward workspace handed to backward, HIP-graph replay."""
+    from cuke_amd.kge import TrainStep
+    w = synth.custom_workload("TransR", n_ent=600, n_rel=30, dim=64, batch=384, chunk=64, n_neg=48, norm_p=2, sigma=0.2,
+                              rel_zipf=1.1, ent_zipf=1.1, seed=9)
+    a = w.arrays
+    m, ix = gpu_model(w)
+    step = TrainStep(m, ix["h"], ix["r"], ix["t"], ix["neg"], w.chunk, loss="margin", margin=2.0, sign=-1.0, neg_mode=mode)
+    assert not step.fusable
+    pos, negs = oracle.score("TransR", a["E"], a["R"], a["A"], a["h"], a["r"], a["t"], a["neg"], w.chunk, p=2, neg_mode=mode)
+
+    def check(tag):
+        torch.cuda.synchronize()
+        assert_close(step.pos.cpu().numpy(), pos, what=f"{tag} pos")
+        assert_close(step.neg.cpu().numpy(), negs, what=f"{tag} neg")
+        ref = oracle.backward("TransR", a["E"], a["R"], a["A"], a["h"], a["r"], a["t"], a["neg"], w.chunk,
+                              step.dpos.cpu().numpy(), step.dneg.cpu().numpy(), p=2, neg_mode=mode)
+        g = step.sparse_grads()
+        assert np.array_equal(g.ent_ids.cpu().numpy(), ref.ent_ids) and np.array_equal(g.rel_ids.cpu().numpy(), ref.rel_ids)
+        assert_close(g.ent_rows.cpu().numpy(), ref.ent_rows, what=f"{tag} entity rows", rows=True)
+        assert_close(g.rel_rows.cpu().numpy(), ref.rel_rows, what=f"{tag} relation rows", rows=True)
+        assert_close(g.aux_rows.cpu().numpy(), ref.aux_rows, what=f"{tag} projection gradients", rows=True)
+
+    step.run()
+    check("side-stream inspection")
+    step.run(overlap=False)
+    check("one stream")
+    graph = step.capture()
+    for i in range(3):  # replays with eager work and synchronisation between them
+        step.neg.zero_()
+        graph.replay()
+        check(f"graph replay {i}")
