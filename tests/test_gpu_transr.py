@@ -176,6 +176,8 @@ def _neg_case(oracle, w, mode, what):
     dict(dim=16, batch=64, chunk=8, n_neg=2, n_rel=40),        # more relations than positives per chunk; thin dM groups
     dict(dim=64, batch=300, chunk=300, n_neg=33, n_rel=1),     # one relation: a single group
     dict(dim=528, batch=64, chunk=32, n_neg=16, n_rel=3),      # three quads of a row per lane
+    dict(dim=8, batch=7, chunk=7, n_neg=1, n_rel=3),           # fewer positives than one reduction block, one negative
+    dict(dim=12, batch=45, chunk=5, n_neg=3, n_rel=2),         # nine chunks of five: groups straddle the reduction blocks
 ])
 @pytest.mark.parametrize("p", [1, 2])
 @pytest.mark.parametrize("mode", ["tail", "head"])
