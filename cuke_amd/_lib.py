@@ -51,7 +51,8 @@ class Batch(C.Structure):
                 ("neg", C.c_void_p), ("chunk", C.c_int64), ("n_neg", C.c_int64),
                 ("ent_insp", C.POINTER(Inspection)), ("rel_insp", C.POINTER(Inspection)),
                 ("insp_ready", C.c_void_p), ("neg_mode", C.c_int32), ("fuse_inspection", C.c_int32),
-                ("insp_jobs", C.c_void_p), ("timeline", C.POINTER(Timeline))]
+                ("insp_jobs", C.c_void_p), ("timeline", C.POINTER(Timeline)),
+                ("plans_ready", C.c_int32), ("reserved", C.c_int32)]
 
 
 class Saved(C.Structure):
@@ -76,6 +77,7 @@ EXPORTS = {
     "kge_residual_fwd": (C.c_int, [C.POINTER(Tables), C.POINTER(Batch), C.c_void_p, C.c_void_p, C.c_size_t,
                                    C.c_void_p]),
     "kge_score_fwd_workspace": (C.c_size_t, [C.POINTER(Tables), C.POINTER(Batch)]),
+    "kge_transr_plan": (C.c_int, [C.POINTER(Tables), C.POINTER(Batch), C.c_void_p, C.c_size_t, C.c_void_p]),
     "kge_score_fwd": (C.c_int, [C.POINTER(Tables), C.POINTER(Batch), C.c_void_p, C.c_void_p,
                                 C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_size_t, C.c_void_p]),
     "kge_inspect_workspace": (C.c_size_t, [C.c_int64, C.c_int64]),
@@ -106,7 +108,7 @@ EXPORTS = {
 _lib = None
 
 
-ABI_VERSION = 4  # layout of the ctypes structures above; must match kge_abi_version()
+ABI_VERSION = 5  # layout of the ctypes structures above; must match kge_abi_version()
 
 
 def lib() -> C.CDLL:

@@ -12,6 +12,7 @@ int launch_score_neg(const kge_tables *, const kge_batch *, const float *, const
 size_t neg_split_workspace(const kge_tables *, const kge_batch *);
 int launch_transr_fwd(const kge_tables *, const kge_batch *, float *, float *, void *, size_t, hipStream_t);
 size_t transr_fwd_workspace(const kge_tables *, const kge_batch *);
+int launch_transr_plan(const kge_tables *, const kge_batch *, void *, size_t, hipStream_t);
 int launch_transr_neg_fwd(const kge_tables *, const kge_batch *, float *, float *, float *, void *, size_t, hipStream_t);
 size_t transr_neg_fwd_workspace(const kge_tables *, const kge_batch *);
 
@@ -104,7 +105,7 @@ const char *kge_strerror(int status)
     }
 }
 
-int kge_abi_version(void) { return 4; }
+int kge_abi_version(void) { return 5; }
 
 kge_timeline *kge_timeline_create(int32_t capacity)
 {
@@ -178,6 +179,16 @@ size_t kge_score_fwd_workspace(const kge_tables *tab, const kge_batch *bat)
     if ((tab->model == KGE_TRANSR || tab->model == KGE_RESCAL) && bat->rel_insp) return transr_fwd_workspace(tab, bat);
     if (tab->model == KGE_TRANSE || tab->model == KGE_ROTATE) return neg_split_workspace(tab, bat);  // small batches only
     return 0;
+}
+
+int kge_transr_plan(const kge_tables *tab, const kge_batch *bat, void *workspace, size_t workspace_bytes, void *stream)
+{
+    int rc = validate_tables(tab);
+    if (rc) return rc;
+    if ((rc = validate_batch(bat))) return rc;
+    if ((tab->model != KGE_TRANSR && tab->model != KGE_RESCAL) || !bat->rel_insp) return KGE_EINVAL;
+    KGE_CLEAR_LAUNCH_ERRORS();
+    return launch_transr_plan(tab, bat, workspace, workspace_bytes, as_stream(stream));
 }
 
 int kge_residual_fwd(const kge_tables *tab, const kge_batch *bat, float *out, void *workspace,

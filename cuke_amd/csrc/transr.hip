@@ -1081,8 +1081,9 @@ int launch_transr_fwd(const kge_tables *tab, const kge_batch *bat, float *pos, f
     TilePlan plan = plan_at(workspace, tiles, 0);
     const RPlan rp = make_rplan(tab, bat);
     TilePlan dplan = plan_at(static_cast<char *>(workspace) + fwd_plan_bytes(tab, bat), rp.dtiles, rp.dsplit);
-    hipLaunchKernelGGL(transr_plan_kernel, dim3(2), dim3(1024), 0, st, ri->num_unique, ri->seg_offsets, ri->unique_ids, plan, kTM,
-                       dplan, kDmChunk);
+    if (!bat->plans_ready)
+        hipLaunchKernelGGL(transr_plan_kernel, dim3(2), dim3(1024), 0, st, ri->num_unique, ri->seg_offsets, ri->unique_ids, plan,
+                           kTM, dplan, kDmChunk);
     GemmArgs a{tab->ent, tab->rel, tab->aux, bat->h, bat->r, bat->t, ri->perm, ri->seg_offsets, ri->num_unique, ri->unique_ids,
                plan, nullptr, nullptr, pos, resid, nullptr, nullptr, (int)tab->dim, tab->norm_p, thin_groups(tab, bat), (int)tiles};
     const size_t lds = lds_with(fi, gemm_lds_bytes((int)tab->dim));
@@ -1093,6 +1094,23 @@ int launch_transr_fwd(const kge_tables *tab, const kge_batch *bat, float *pos, f
     else
         hipLaunchKernelGGL(transr_gemm_kernel<0>, grid, dim3(256), lds, st, a, fi);
     timeline_mark(bat->timeline, st, "transr_plan_kernel + transr_gemm_kernel<fwd>");
+    KGE_CHECK_LAUNCH();
+    return KGE_OK;
+}
+
+// The tile plans alone (what launch_transr_fwd builds first), for callers that plan a batch ahead.
+int launch_transr_plan(const kge_tables *tab, const kge_batch *bat, void *workspace, size_t workspace_bytes, hipStream_t st)
+{
+    if (bat->batch == 0) return KGE_OK;
+    if (bat->neg) return KGE_EUNSUPPORTED;  // the shared-negative path plans its own row list
+    if (!mfma_path_ok(tab, bat) || gemm_lds_bytes((int)tab->dim) > kMaxGemmLds) return KGE_EUNSUPPORTED;
+    if (!workspace || workspace_bytes < transr_fwd_workspace(tab, bat)) return KGE_EWORKSPACE;
+    const kge_inspection *ri = bat->rel_insp;
+    const RPlan rp = make_rplan(tab, bat);
+    TilePlan plan = plan_at(workspace, max_tiles(tab, bat), 0);
+    TilePlan dplan = plan_at(static_cast<char *>(workspace) + fwd_plan_bytes(tab, bat), rp.dtiles, rp.dsplit);
+    hipLaunchKernelGGL(transr_plan_kernel, dim3(2), dim3(1024), 0, st, ri->num_unique, ri->seg_offsets, ri->unique_ids, plan, kTM,
+                       dplan, kDmChunk);
     KGE_CHECK_LAUNCH();
     return KGE_OK;
 }

@@ -498,6 +498,10 @@ class TrainStep:
             else None
         self._ws_f_bytes = int(L.kge_score_fwd_workspace(C.byref(model._tab), C.byref(self.bat)))
         self._ws_f = torch.empty(max(self._ws_f_bytes, 1), dtype=torch.uint8, device=dev)
+        # TransR / RESCAL without negatives: the forward workspace holds the batch's tile plans, which a
+        # staged batch gets a step ahead (stage()); every set of the ring then keeps plans of its own
+        self._plans_per_set = self.needs_rel_groups and neg is None and self._ws_f_bytes > 0
+        self._sets[0].ws_f = self._ws_f
         self.loss = torch.zeros(1, **f32)
         if loss == "margin":
             self.dpos, self.dneg = torch.empty(B, **f32), torch.empty((B, N), **f32)
@@ -653,7 +657,20 @@ class TrainStep:
     def forward(self, st):
         _lib.check(self.L.kge_score_fwd(C.byref(self.m._tab), C.byref(self.bat), _ptr(self.pos), _ptr(self.neg),
                                         _ptr(self.side_pos), _ptr(self.side_neg), _ptr(self.residual),
-                                        _ptr(self._ws_f), self._ws_f_bytes, st), "kge_score_fwd")
+                                        _ptr(self._fwd_ws()), self._ws_f_bytes, st), "kge_score_fwd")
+
+    def _fwd_ws(self):
+        """The forward workspace of the current set (its own where the sets keep their tile plans apart);
+        backward is pointed at the same one."""
+        cur = self._sets[self._cur]
+        ws = self._ws_f
+        if self._plans_per_set:
+            if getattr(cur, "ws_f", None) is None:
+                cur.ws_f = torch.empty(max(self._ws_f_bytes, 1), dtype=torch.uint8, device=self.m.dev)
+            ws = cur.ws_f
+        if self.needs_rel_groups and self._ws_f_bytes:
+            self.saved.fwd_workspace = ws.data_ptr()
+        return ws
 
     def loss_grad(self, st):
         if self.loss_kind == "margin":
@@ -688,16 +705,25 @@ class TrainStep:
             (stream or torch.cuda.current_stream()).wait_event(nxt.done_event)
         return nxt.idx
 
-    def stage(self, inputs_ready=None):
+    def stage(self, inputs_ready=None, batch=None):
         """Declare the tensors of ``next_inputs()`` final -- complete once ``inputs_ready`` (a
         torch.cuda.Event; None = already complete) has fired -- and start their inspection on the
         side stream.  ``run(pipeline=True)`` consumes staged batches oldest first.  Staging one
         batch ahead of the step that is about to run lets the inspector finish before backward asks
-        for it, which also keeps the host off the slow path of waiting on a pending event."""
-        sets = self._ring()
-        at = self._stage_at
-        if len(self._staged) >= len(sets) - 1:
-            raise KgeError(f"at most {len(sets) - 1} batches can be staged ahead of run()")
+        for it, which also keeps the host off the slow path of waiting on a pending event.
+        ``batch``: stage batch number ``batch`` of ``add_batch()`` instead of the ring's next set (its
+        index tensors are used as they are; nothing is copied)."""
+        if batch is None:
+            sets = self._ring()
+            at = self._stage_at
+        else:
+            if self._pipelined:
+                raise KgeError("stage(batch=...) cannot be mixed with the ring of next_inputs()")
+            sets, at = self._sets, int(batch)
+            if not 0 <= at < len(sets) or at in self._staged:
+                raise KgeError(f"batch {batch} does not exist or is already staged")
+        if len(self._staged) >= max(len(sets) - 1, 1):
+            raise KgeError(f"at most {max(len(sets) - 1, 1)} batches can be staged ahead of run()")
         s, side = sets[at], self.side
         if s.done_event is not None:
             side.wait_event(s.done_event)  # its inspection may still be read by an earlier step
@@ -705,13 +731,26 @@ class TrainStep:
             side.wait_event(inputs_ready)
         s.inputs_ready = inputs_ready
         sst = C.c_void_p(side.cuda_stream)
-        if self.needs_rel_groups:  # the relation groups drive the forward pass: inspected in run()
+        if self._plans_per_set:
+            # the relation groups drive the forward pass: inspected and planned here, a step ahead, so
+            # that run() starts with the projection kernel
+            if getattr(s, "ws_f", None) is None:
+                s.ws_f = torch.empty(max(self._ws_f_bytes, 1), dtype=torch.uint8, device=self.m.dev)
+            _lib.check(self.L.kge_inspect_batch(C.byref(s.jobs[1]), 1, sst), "kge_inspect_batch(relations)")
+            _lib.check(self.L.kge_transr_plan(C.byref(self.m._tab), C.byref(s.bat), _ptr(s.ws_f), self._ws_f_bytes, sst),
+                       "kge_transr_plan")
+            s.planned_event = torch.cuda.Event()
+            s.planned_event.record(side)
+            s.bat.plans_ready = 1
+            _lib.check(self.L.kge_inspect_batch(C.byref(s.jobs[0]), 1, sst), "kge_inspect_batch(entities)")
+        elif self.needs_rel_groups:  # (with shared negatives the forward call plans its own row list)
             _lib.check(self.L.kge_inspect_batch(C.byref(s.jobs[0]), 1, sst), "kge_inspect_batch(entities)")
         else:
             _lib.check(self.L.kge_inspect_batch(s.jobs, 2, sst), "kge_inspect_batch")
         s.insp_event.record(side)
         self._staged.append(at)
-        self._stage_at = (at + 1) % len(sets)
+        if batch is None:
+            self._stage_at = (at + 1) % len(sets)
 
     @property
     def fusable(self):
@@ -742,6 +781,8 @@ class TrainStep:
         st = C.c_void_p(main.cuda_stream)
         for s_ in self._sets:  # cached unique counts belong to the batches of earlier steps
             s_.ent_insp._u = s_.rel_insp._u = None
+        if not pipeline:
+            self.bat.plans_ready = 0  # the forward call plans for itself
         if fused is None:
             fused = backward and not pipeline and self.fusable
         if fused:
@@ -778,7 +819,9 @@ class TrainStep:
             cur = self._sets[self._cur]
             if cur.inputs_ready is not None:
                 main.wait_event(cur.inputs_ready)  # the score kernels read the index tensors too
-            if self.needs_rel_groups:
+            if self._plans_per_set:
+                main.wait_event(cur.planned_event)  # relation groups and tile plans of this batch (made in stage())
+            elif self.needs_rel_groups:
                 _lib.check(self.L.kge_inspect_batch(C.byref(cur.jobs[1]), 1, st), "kge_inspect_batch(relations)")
         else:
             if self._staged:

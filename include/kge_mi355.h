@@ -167,6 +167,12 @@ typedef struct kge_batch {
     int32_t fuse_inspection;
     const struct kge_inspect_job *insp_jobs;
     kge_timeline *timeline;  /* optional, see kge_timeline; NULL: nothing is recorded */
+    /* TransR / RESCAL on their grouped path: non-zero = the workspace handed to kge_score_fwd already
+       holds this batch's tile plans (kge_transr_plan ran on it after rel_insp was complete), so the
+       forward call launches no plan kernel.  Lets a training loop inspect the relations and plan a
+       batch ahead on another stream. */
+    int32_t plans_ready;
+    int32_t reserved;
 } kge_batch;
 
 /* Forward outputs that backward consumes. */
@@ -239,6 +245,12 @@ int kge_residual_fwd(const kge_tables *tab, const kge_batch *bat, float *out, vo
  * left from an earlier call on the same batch).
  */
 size_t kge_score_fwd_workspace(const kge_tables *tab, const kge_batch *bat);
+/* TransR / RESCAL without negatives: builds the tile plans of the relation groups (bat->rel_insp, complete
+   on `stream`) into `workspace` (kge_score_fwd_workspace bytes), the part of kge_score_fwd that only
+   depends on the relation ids.  Pass the same workspace to kge_score_fwd with bat->plans_ready set.
+   No counterpart in the reference. */
+int kge_transr_plan(const kge_tables *tab, const kge_batch *bat, void *workspace, size_t workspace_bytes,
+                    void *stream);
 int kge_score_fwd(const kge_tables *tab, const kge_batch *bat, float *pos, float *neg,
                   float *side_pos, float *side_neg, float *residual, void *workspace,
                   size_t workspace_bytes, void *stream);

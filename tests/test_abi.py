@@ -34,7 +34,7 @@ def test_binding_table_matches_header():
 def test_strerror_and_version_without_gpu():
     from cuke_amd import _lib
     L = _lib.lib()
-    assert L.kge_abi_version() == _lib.ABI_VERSION == 4
+    assert L.kge_abi_version() == _lib.ABI_VERSION == 5
     assert L.kge_strerror(0) == b"ok"
     assert b"workspace" in L.kge_strerror(-4)
 

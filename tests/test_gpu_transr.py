@@ -230,3 +230,37 @@ def test_train_step_with_shared_negatives_and_margin_loss(oracle, mode):
         step.neg.zero_()
         graph.replay()
         check(f"graph replay {i}")
+
+
+def test_staged_batches_are_planned_a_step_ahead(oracle):
+    """stage(batch=i) inspects the relations of an added batch and builds its tile plans on the side stream
+    (kge_transr_plan); run(pipeline=True) then starts with the projection kernel (kge_batch.plans_ready).
+    Every step must match the oracle on its own batch, and a plain run() afterwards still plans for itself."""
+    from cuke_amd.kge import TrainStep
+    ws = [synth.make_workload("cfg3_transr", batch=1024, seed=s) for s in range(4)]
+    m, ix0 = gpu_model(ws[0])
+    step = TrainStep(m, ix0["h"], ix0["r"], ix0["t"])
+    for w in ws[1:]:
+        ix = {k: torch.from_numpy(w.arrays[k]).cuda() for k in ("h", "r", "t")}
+        step.add_batch(ix["h"], ix["r"], ix["t"])
+    a0 = ws[0].arrays
+
+    def check(w, tag):
+        torch.cuda.synchronize()
+        a = w.arrays
+        ref = oracle.backward("TransR", a0["E"], a0["R"], a0["A"], a["h"], a["r"], a["t"], dpos=step.dpos.cpu().numpy(), p=2)
+        g = step.sparse_grads()
+        assert np.array_equal(g.rel_ids.cpu().numpy(), ref.rel_ids), tag
+        assert_close(g.ent_rows.cpu().numpy(), ref.ent_rows, what=f"{tag} entity rows", rows=True)
+        assert_close(g.aux_rows.cpu().numpy(), ref.aux_rows, what=f"{tag} projection gradients", rows=True)
+
+    step.stage(batch=0)
+    for i in range(6):
+        step.stage(batch=(i + 1) % 4)     # one batch ahead
+        step.run(pipeline=True)           # consumes batch i % 4
+        check(ws[i % 4], f"staged step {i}")
+    step.run(pipeline=True)               # the batch still staged
+    check(ws[6 % 4], "drained")
+    step.select(1)
+    step.run()
+    check(ws[1], "plain run afterwards")
