@@ -46,18 +46,18 @@ BOUND = {"cfg1_transe": "hbm", "cfg2_distmult": "fp32", "cfg2_complex": "fp32", 
 # for the 256 MiB copy kernel of --calibrate-copy.  The summaries the numbers come from are
 # profiles/score_path_kernels_<workload>.txt; a pair that has not been measured reports null.
 MEASURED_TRAFFIC_BYTES = {
-    ('cfg5_transh', 'bwd_tile_kernel'): 1253062686,
-    ('cfg5_transh', 'score_neg_kernel'): 322443196,
+    ('cfg5_transh', 'bwd_tile_kernel'): 1249672344,
+    ('cfg5_transh', 'score_neg_kernel'): 321899447,
     ('cfg1_transe', 'score_pos_kernel'): 1684915,
     ('cfg2_distmult', 'bwd_tile_kernel'): 22893024,
     ('cfg2_distmult', 'score_neg_kernel'): 14036989,
     ('cfg2_complex', 'bwd_tile_kernel'): 22895280,
     ('cfg2_complex', 'score_neg_kernel'): 14062239,
-    ('cfg3_transr', 'transr_plan_kernel + transr_gemm_kernel<fwd>'): 165424842,
-    ('cfg3_transr', 'transr_gemm_kernel<dX>'): 169627892,
-    ('cfg3_transr', 'transr_dm_kernel'): 183154198,
-    ('cfg4_rotate', 'bwd_tile_kernel'): 20676212,
-    ('cfg4_rotate', 'score_neg_kernel'): 20660815,
+    ('cfg3_transr', 'transr_plan_kernel + transr_gemm_kernel<fwd>'): 165401787,
+    ('cfg3_transr', 'transr_gemm_kernel<dX>'): 169478021,
+    ('cfg3_transr', 'transr_dm_kernel'): 182971548,
+    ('cfg4_rotate', 'bwd_tile_kernel'): 20621914,
+    ('cfg4_rotate', 'score_neg_kernel'): 20619347,
 }
 
 
