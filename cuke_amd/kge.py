@@ -862,6 +862,67 @@ class TrainStep:
     def replay(self):
         self.graph.replay()
 
+    def capture_staged(self, cur: int, nxt: int, backward=True):
+        """One HIP graph with two branches: the step of batch ``cur`` on the capturing stream and, beside it on
+        the side stream, the inspection of batch ``nxt`` (TransR / RESCAL: its relation groups and tile plans
+        too).  Replaying the graphs (cur, nxt) = (0, 1), (1, 2), ... one after the other is the staged issue
+        of ``stage(batch=...)`` / ``run(pipeline=True)`` with one launch per step: the inspection of batch
+        ``cur`` was made by the replay before (graph launches on one stream run one after the other), so
+        nothing inside the graph waits for it.  Before the first replay batch ``cur`` of the first graph has
+        to be inspected once: ``prime_staged(cur)``."""
+        if self._staged or self._pipelined:
+            raise KgeError("capture_staged() cannot be mixed with the staged pipeline")
+        self.prime_staged(cur)
+        self.prime_staged(nxt)
+        self._run_staged_pair(cur, nxt, backward)  # warm-up outside capture (module loading, lazy init)
+        torch.cuda.synchronize()
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g):
+            self._run_staged_pair(cur, nxt, backward)
+        return g
+
+    def use_batch(self, i: int) -> None:
+        """Point ``sparse_grads()`` and the inspection properties at batch ``i`` (after replaying a graph of
+        ``capture_staged(i, ...)``, which Python does not see)."""
+        self._cur = i
+        for s_ in self._sets:
+            s_.ent_insp._u = s_.rel_insp._u = None
+
+    def prime_staged(self, i: int) -> None:
+        """Inspect (and, for TransR / RESCAL, plan) batch ``i`` on the current stream: what the side branch of
+        the graph before would have done."""
+        self._inspect_ahead(self._sets[i], C.c_void_p(torch.cuda.current_stream().cuda_stream))
+
+    def _inspect_ahead(self, s, sst) -> None:
+        if self._plans_per_set:
+            if getattr(s, "ws_f", None) is None:
+                s.ws_f = torch.empty(max(self._ws_f_bytes, 1), dtype=torch.uint8, device=self.m.dev)
+            _lib.check(self.L.kge_inspect_batch(C.byref(s.jobs[1]), 1, sst), "kge_inspect_batch(relations)")
+            _lib.check(self.L.kge_transr_plan(C.byref(self.m._tab), C.byref(s.bat), _ptr(s.ws_f), self._ws_f_bytes, sst),
+                       "kge_transr_plan")
+            s.bat.plans_ready = 1
+            _lib.check(self.L.kge_inspect_batch(C.byref(s.jobs[0]), 1, sst), "kge_inspect_batch(entities)")
+        elif self.needs_rel_groups:
+            _lib.check(self.L.kge_inspect_batch(C.byref(s.jobs[0]), 1, sst), "kge_inspect_batch(entities)")
+        else:
+            _lib.check(self.L.kge_inspect_batch(s.jobs, 2, sst), "kge_inspect_batch")
+
+    def _run_staged_pair(self, cur: int, nxt: int, backward: bool) -> None:
+        main, side = torch.cuda.current_stream(), self.side
+        st = C.c_void_p(main.cuda_stream)
+        side.wait_stream(main)                                   # fork
+        self._inspect_ahead(self._sets[nxt], C.c_void_p(side.cuda_stream))
+        self.use_batch(cur)
+        bat = self.bat
+        bat.insp_ready, bat.fuse_inspection = None, 0
+        if self.needs_rel_groups and not self._plans_per_set:    # (shared negatives: groups needed by the forward call)
+            _lib.check(self.L.kge_inspect_batch(C.byref(self._jobs[1]), 1, st), "kge_inspect_batch(relations)")
+        self.forward(st)
+        if backward:
+            self.loss_grad(st)
+            self.backward(st)
+        main.wait_stream(side)                                   # join
+
     def sparse_grads(self) -> SparseGrads:
         ue, ur = self.ent_insp.num_unique, self.rel_insp.num_unique
         return SparseGrads(self.ent_insp.unique_ids[:ue], self.ent_rows[:ue], self.rel_insp.unique_ids[:ur],

@@ -341,3 +341,33 @@ def test_pair_sums_on_matrix_cores_and_on_vector_alus_agree(oracle, model):
     for unit in ("matrix_cores", "vector_alus"):
         g, ref = run_both(oracle, w, seed=3, pair_sums=unit)
         compare(g, ref, f"{model} pair sums on the {unit}")
+
+
+@pytest.mark.parametrize("name,over", [("cfg2_distmult", dict(n_ent=50_000, batch=512)), ("cfg3_transr", dict(batch=1024)),
+                                       ("cfg4_rotate", dict(batch=256))])
+def test_staged_issue_as_two_branch_graphs(oracle, name, over):
+    """capture_staged(i, i + 1): the step of batch i and, on a second branch of the same HIP graph, the inspection
+    of batch i + 1.  The graphs are replayed in a ring several times with eager work and synchronisation between
+    the replays; every replay must reproduce the oracle's gradients of its own batch."""
+    from cuke_amd.kge import TrainStep
+    ws = [synth.make_workload(name, seed=s, **over) for s in range(3)]
+    m, ix0 = gpu_model(ws[0])
+    w = ws[0]
+    sign = -1.0 if w.model in ("TransR", "TransH") else 1.0
+    step = TrainStep(m, ix0["h"], ix0["r"], ix0["t"], ix0.get("neg"), w.chunk or None, loss=w.loss, margin=w.margin, sign=sign)
+    for o in ws[1:]:
+        ix = {k: torch.from_numpy(o.arrays[k]).cuda() for k in ("h", "r", "t", "neg") if o.arrays.get(k) is not None}
+        step.add_batch(ix["h"], ix["r"], ix["t"], ix.get("neg"))
+    graphs = [step.capture_staged(i, (i + 1) % 3) for i in range(3)]
+    a0 = ws[0].arrays
+    for rep in range(7):
+        i = rep % 3
+        step.ent_rows.zero_()                      # eager work between the replays
+        graphs[i].replay()
+        step.use_batch(i)
+        torch.cuda.synchronize()
+        a = ws[i].arrays
+        ref = oracle.backward(w.model, a0["E"], a0["R"], a0["A"], a["h"], a["r"], a["t"], a.get("neg"), w.chunk,
+                              step.dpos.cpu().numpy(), step.dneg.cpu().numpy() if step.dneg is not None else None, p=w.norm_p)
+        compare(step.sparse_grads(), ref, f"{name} staged graph replay {rep}",
+                outliers=(1e-5, 4.0) if w.model == "RotatE" else None)
