@@ -49,6 +49,27 @@ def test_build_index_exhaustive_three_values(oracle):
     assert np.array_equal(cnt.cpu().numpy(), rc)
 
 
+def test_build_index_chunks_of_every_number_of_distinct_values(oracle):
+    """1 to 15 distinct values per chunk, sorted and unsorted, ties between run lengths: the HIP kernel against
+    the oracle, which the CPU suite pins on the same chunk family against the reference kernel run in lockstep."""
+    from cuke_amd.kge import inspector
+    rng = np.random.default_rng(21)
+    rel_num = 40
+    chunks = []
+    for distinct in range(1, 16):
+        for rep in range(40):
+            vals = rng.choice(rel_num, distinct, replace=False)
+            row = np.concatenate([vals, rng.choice(vals, 16 - distinct)])
+            chunks.append(np.sort(row) if rep % 2 == 0 else rng.permutation(row))
+    r = np.concatenate(chunks).astype(np.int64)
+    uniq, buf, cnt = inspector(torch.from_numpy(r).to(DEV), rel_num)
+    ru, rb, rc, undefined = oracle.build_index(r, rel_num)
+    assert not undefined
+    assert np.array_equal(uniq.cpu().numpy(), ru)
+    assert np.array_equal(buf.cpu().numpy(), rb)
+    assert np.array_equal(cnt.cpu().numpy(), rc)
+
+
 def test_check_indices():
     import ctypes as C
     from cuke_amd import _lib

@@ -367,6 +367,113 @@ def test_build_index_exhaustive_three_values(oracle):
             assert counts[list(vals).index(cached[0])] == multi[0]
 
 
+def lockstep_build_index(chunk, rel_num):
+    """The reference's build_index kernel (apps/kge/inspection/inspector.cu:39-136) executed as written:
+    sixteen threads in lockstep, one numpy array per __shared__ array, every statement applied to all
+    threads at once (reads before writes, as the lanes of a wavefront execute it).  A restatement at the
+    thread level, independent of the oracle's sequential one.  Returns (uniq[16], buf[16], cnt) or None
+    where the kernel writes out of bounds (16 distinct values)."""
+    C_, T_ = 16, 2
+    tid = np.arange(C_)
+    idx = np.array(chunk, dtype=np.int64)
+    ord_uniq, pcount = tid.copy(), np.zeros(C_, np.int64)
+    count, idx_count = np.full(C_, -1, np.int64), np.full(C_, -1, np.int64)
+    # bitonic_sort(idx, ord): inspector.cu:39-66
+    arr, sord = idx.copy(), tid.copy()
+    k = 2
+    while k <= C_:
+        j = k >> 1
+        while j > 0:
+            ixj = tid ^ j
+            a_old, o_old = arr.copy(), sord.copy()
+            for t in range(C_):
+                x = ixj[t]
+                if x > t:
+                    up = (t & k) == 0
+                    if (up and a_old[t] > a_old[x]) or (not up and a_old[t] < a_old[x]):
+                        arr[t], arr[x], sord[t], sord[x] = a_old[x], a_old[t], o_old[x], o_old[t]
+            j >>= 1
+        k <<= 1
+    idx = arr
+    ord_ = np.empty(C_, np.int64)
+    ord_[sord] = tid
+    # head flags and their inclusive scan: inspector.cu:80-88
+    ibuf = np.where((tid > 0) & (idx > np.roll(idx, 1)), 1, 0).astype(np.int64)
+    ibuf[0] = 0
+    offset = 1
+    while offset < C_:
+        old = ibuf.copy()
+        ibuf[offset:] = old[offset:] + old[:-offset]
+        offset *= 2
+    # run starts: inspector.cu:90-94
+    if ibuf[C_ - 1] + 1 >= C_:
+        return None  # pcount[16] = C: out of bounds
+    pcount[ibuf[C_ - 1] + 1] = C_
+    for t in range(1, C_):
+        if idx[t] > idx[t - 1]:
+            pcount[ibuf[t]] = t
+    iuniq = np.full(C_, rel_num, np.int64)
+    # run lengths and the tournament for the two longest: inspector.cu:97-113
+    old_p = pcount.copy()
+    for t in range(1, C_):
+        if old_p[t] - old_p[t - 1] > 0:
+            count[t - 1] = old_p[t] - old_p[t - 1]
+            idx_count[t - 1] = old_p[t] - 1
+    sdist = C_ // 2
+    while sdist > 0:
+        c_old, i_old, o_old = count.copy(), idx_count.copy(), ord_uniq.copy()
+        for t in range(sdist):
+            if c_old[t] < c_old[t + sdist]:
+                count[t], count[t + sdist] = c_old[t + sdist], c_old[t]
+                idx_count[t], idx_count[t + sdist] = i_old[t + sdist], i_old[t]
+                ord_uniq[t], ord_uniq[t + sdist] = o_old[t + sdist], o_old[t]
+        sdist >>= 1
+    if count[1] < count[2]:
+        count[1], count[2] = count[2], count[1]
+        idx_count[1], idx_count[2] = idx_count[2], idx_count[1]
+        ord_uniq[1], ord_uniq[2] = ord_uniq[2], ord_uniq[1]
+    # cache slots for runs of at least T: inspector.cu:117-119
+    for t in range(T_):
+        if count[t] > T_ - 1:
+            iuniq[t] = idx[idx_count[t]]
+    # slot or id + C per element: inspector.cu:121-133
+    new_ibuf = ibuf.copy()
+    for t in range(C_):
+        if ibuf[t] == ord_uniq[0] and iuniq[0] < rel_num:
+            new_ibuf[t] = 0
+        elif ibuf[t] == ord_uniq[1] and iuniq[1] < rel_num:
+            new_ibuf[t] = 1
+        else:
+            new_ibuf[t] = idx[t] + C_
+    cnt = 0
+    for t in range(C_ - 1):
+        if iuniq[t] < rel_num and iuniq[t + 1] == rel_num:
+            cnt = t + 1
+    return iuniq, new_ibuf[ord_], cnt
+
+
+def test_build_index_equals_the_kernel_run_in_lockstep(oracle):
+    """Chunks with 1 to 15 distinct values, sorted (the reference's use) and unsorted, random run lengths and
+    ties between run lengths: the oracle's sequential restatement against the thread-level one."""
+    rng = np.random.default_rng(21)
+    rel_num = 40
+    chunks = []
+    for distinct in range(1, 16):
+        for rep in range(40):
+            vals = rng.choice(rel_num, distinct, replace=False)
+            row = np.concatenate([vals, rng.choice(vals, 16 - distinct)])
+            chunks.append(np.sort(row) if rep % 2 == 0 else rng.permutation(row))
+    r = np.concatenate(chunks).astype(np.int64)
+    uniq, buf, cnt, undefined = oracle.build_index(r, rel_num)
+    assert not undefined
+    for b, chunk in enumerate(chunks):
+        want = lockstep_build_index(chunk, rel_num)
+        assert want is not None
+        assert uniq[b].tolist() == want[0].tolist(), (b, chunk.tolist())
+        assert buf[b].tolist() == want[1].tolist(), (b, chunk.tolist())
+        assert cnt[b] == want[2], (b, chunk.tolist())
+
+
 def test_build_index_flags_sixteen_distinct(oracle):
     r = np.arange(16, dtype=np.int64)
     *_, undefined = oracle.build_index(r, 100)
