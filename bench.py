@@ -642,6 +642,27 @@ def run_neg_transr(args, torch):
     return out
 
 
+def stream_calibration(torch, dev):
+    """What a plain streaming kernel reaches on this GPU: read + written bytes over time of torch's
+    256 MiB elementwise copy kernel, sources rotating over 1 GiB so that no cache holds a pass."""
+    n = 64 * 1024 * 1024
+    srcs = [torch.empty(n, dtype=torch.float32, device=dev).normal_() for _ in range(4)]
+    dst = torch.empty_like(srcs[0])
+    it = [0]
+
+    def copy():
+        dst.copy_(srcs[it[0] % 4])
+        it[0] += 1
+
+    for _ in range(4):
+        copy()
+    ms = time_events(copy, 12, torch)
+    del srcs, dst
+    torch.cuda.empty_cache()
+    return {"stream_copy_gbs": 2 * 4 * n / (ms * 1e-3) / 1e9, "peak_gbs": HBM_PEAK_GBS,
+            "sample": "256 MiB device-to-device copy kernel, (bytes read + bytes written) / time, 4 rotating sources"}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -684,6 +705,7 @@ def main():
             sys.exit(1)
         return
     names = ALL_WORKLOADS if args.workload == "all" else [args.workload]
+    machine = stream_calibration(torch, dev)
     results = []
     for n in names:
         t0 = time.perf_counter()
@@ -698,6 +720,7 @@ def main():
               f"{res['roofline']['kernel']} {res['roofline']['frac']:.3f} of {res['roofline']['bound']}",
               file=sys.stderr, flush=True)
     out = results[0]
+    out["machine"] = machine
     if len(results) > 1:
         out["per_workload"] = results[1:]
     print(json.dumps(out))

@@ -504,11 +504,8 @@ __device__ __forceinline__ void gemm_sweep(const BLoader<MODE> &bl, float4 (&rin
 // MODE 3: list rows        x = E[h]-E[t] (t = -1: no row), y = x M + rs R[r] -> resid rows in list order;
 //         h, t, rs are indexed by the sorted position itself (no perm), no score
 template <int MODE>
-__global__ __launch_bounds__(256, KGE_TR_OCC) void transr_gemm_kernel(GemmArgs a, FusedInsp fi)
+__device__ __forceinline__ void transr_gemm_body(const GemmArgs &a, float *lds, int bid)
 {
-    extern __shared__ __align__(16) float lds[];
-    if (fused_insp_block(fi, reinterpret_cast<uint32_t *>(lds))) return;  // an inspector workgroup riding along
-    const int bid = (int)blockIdx.x - fi.blocks;
     // Workgroups [0, max_tiles) take the planned 32-triple tiles, the following `thin_groups`
     // stream the thin group tails.  The tiles come first because each is one long chain of
     // dependent loads and matrix-core steps (about 20 us whatever else runs); the thin
@@ -715,6 +712,14 @@ __global__ __launch_bounds__(256, KGE_TR_OCC) void transr_gemm_kernel(GemmArgs a
     }
 }
 
+template <int MODE>
+__global__ __launch_bounds__(256, KGE_TR_OCC) void transr_gemm_kernel(GemmArgs a, FusedInsp fi)
+{
+    extern __shared__ __align__(16) float lds[];
+    if (fused_insp_block(fi, reinterpret_cast<uint32_t *>(lds))) return;  // an inspector workgroup riding along
+    transr_gemm_body<MODE>(a, lds, (int)blockIdx.x - fi.blocks);
+}
+
 static size_t gemm_lds_bytes(int d)  // the larger of the tile layout and the thin layouts
 {
     const int kpad = (d + 15) & ~15;
@@ -905,11 +910,8 @@ __device__ __forceinline__ void dm_sweep(const float *xs, const float *qs, int d
 // of one group, 32 rows i); the four waves split the columns j; K runs over the chunk's triples,
 // operands prefetched four supersteps ahead.  Groups longer than one chunk write per-chunk
 // partial matrices that transr_dm_finish_kernel adds up (keeps the longest K loop at 16 supersteps).
-__global__ __launch_bounds__(256, KGE_TR_OCC) void transr_dm_kernel(DmArgs a, FusedInsp fi)
+__device__ __forceinline__ void transr_dm_body(const DmArgs &a, float *lds, int bid)
 {
-    extern __shared__ __align__(16) float lds[];  // thin groups: d float4; inspector workgroups: their own need
-    if (fused_insp_block(fi, reinterpret_cast<uint32_t *>(lds))) return;
-    const int bid = (int)blockIdx.x - fi.blocks;
     if (bid >= a.max_items) {
         transr_thin_dm_body(a, lds, bid - a.max_items);
         return;
@@ -957,6 +959,32 @@ __global__ __launch_bounds__(256, KGE_TR_OCC) void transr_dm_kernel(DmArgs a, Fu
                     *reinterpret_cast<float4 *>(dst + (int64_t)row * d + n0 + 4 * li) = v;
                 }
         }
+    }
+}
+
+__global__ __launch_bounds__(256, KGE_TR_OCC) void transr_dm_kernel(DmArgs a, FusedInsp fi)
+{
+    extern __shared__ __align__(16) float lds[];  // thin groups: d float4; inspector workgroups: their own need
+    if (fused_insp_block(fi, reinterpret_cast<uint32_t *>(lds))) return;
+    transr_dm_body(a, lds, (int)blockIdx.x - fi.blocks);
+}
+
+// dX and dM of one backward pass in ONE launch (no inspector riders): the two are independent, one
+// streams the projections in while the other streams the projection gradients out, and either alone
+// leaves the memory system waiting on its dependent chains.  Order of the workgroups: the dX tiles,
+// the dM work items, then the thin groups of both in alternation.
+__global__ __launch_bounds__(256, KGE_TR_OCC) void transr_dx_dm_kernel(GemmArgs ga, DmArgs da)
+{
+    extern __shared__ __align__(16) float lds[];
+    const int bid = (int)blockIdx.x;
+    if (bid < ga.max_tiles) {
+        transr_gemm_body<2>(ga, lds, bid);
+    } else if (bid < ga.max_tiles + da.max_items) {
+        transr_dm_body(da, lds, bid - ga.max_tiles);
+    } else {
+        const int q = bid - ga.max_tiles - da.max_items;
+        if (q & 1) transr_dm_body(da, lds, da.max_items + (q >> 1));
+        else transr_gemm_body<2>(ga, lds, ga.max_tiles + (q >> 1));
     }
 }
 
@@ -1161,17 +1189,28 @@ int launch_transr_bwd(const kge_tables *tab, const kge_batch *bat, const kge_sav
     // dX = Q M^T -> occurrence rows of h (and -dX for t)
     GemmArgs ga{tab->ent, tab->rel, tab->aux, bat->h, bat->r, bat->t, ri->perm, ri->seg_offsets, ri->num_unique, ri->unique_ids,
                 plan, qs, nullptr, nullptr, nullptr, occ, rescal ? nullptr : occ + B * d, d, tab->norm_p, thin_groups(tab, bat), (int)p.tiles};
-    if (const int rc = allow_lds<2>(lds_with(f2, gemm_lds_bytes(d)))) return rc;
-    hipLaunchKernelGGL(transr_gemm_kernel<2>, dim3((unsigned)(p.tiles + ga.thin_groups + f2.blocks)), dim3(256),
-                       lds_with(f2, gemm_lds_bytes(d)), st, ga, f2);
-    timeline_mark(bat->timeline, st, "transr_gemm_kernel<dX>");
     // dM = X^T Q per relation group
     const int dm_items = (int)(ceil_div(d, 32) * p.dtiles);
     DmArgs da{xs, qs, ri->seg_offsets, dplan, grads->aux_rows, reinterpret_cast<float *>(ws + p.off_dpart), d,
               ri->num_unique, dm_items};
-    hipLaunchKernelGGL(transr_dm_kernel, dim3((unsigned)(dm_items + thin_groups(tab, bat) + f3.blocks)), dim3(256),
-                       lds_with(f3, sizeof(float) * 4 * (size_t)d), st, da, f3);
-    timeline_mark(bat->timeline, st, "transr_dm_kernel");
+    if (!bat->fuse_inspection) {  // nothing rides along: both in one launch
+        const size_t lds = gemm_lds_bytes(d) > sizeof(float) * 4 * (size_t)d ? gemm_lds_bytes(d) : sizeof(float) * 4 * (size_t)d;
+        if (lds > 64 * 1024 &&
+            hipFuncSetAttribute(reinterpret_cast<const void *>(&transr_dx_dm_kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                (int)kMaxGemmLds) != hipSuccess)
+            return KGE_ELAUNCH;
+        hipLaunchKernelGGL(transr_dx_dm_kernel, dim3((unsigned)(p.tiles + dm_items + 2 * ga.thin_groups)), dim3(256), lds, st, ga,
+                           da);
+        timeline_mark(bat->timeline, st, "transr_dx_dm_kernel");
+    } else {
+        if (const int rc = allow_lds<2>(lds_with(f2, gemm_lds_bytes(d)))) return rc;
+        hipLaunchKernelGGL(transr_gemm_kernel<2>, dim3((unsigned)(p.tiles + ga.thin_groups + f2.blocks)), dim3(256),
+                           lds_with(f2, gemm_lds_bytes(d)), st, ga, f2);
+        timeline_mark(bat->timeline, st, "transr_gemm_kernel<dX>");
+        hipLaunchKernelGGL(transr_dm_kernel, dim3((unsigned)(dm_items + thin_groups(tab, bat) + f3.blocks)), dim3(256),
+                           lds_with(f3, sizeof(float) * 4 * (size_t)d), st, da, f3);
+        timeline_mark(bat->timeline, st, "transr_dm_kernel");
+    }
     hipLaunchKernelGGL(transr_dm_finish_kernel, dim3((unsigned)ceil_div((int64_t)d * d / 4, 256), (unsigned)p.dsplit),
                        dim3(256), 0, st, da);
     timeline_mark(bat->timeline, st, "transr_dm_finish_kernel");
