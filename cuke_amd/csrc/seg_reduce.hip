@@ -24,9 +24,34 @@ struct SegArgs3 {
     SegArgs j[3];
 };
 
-template <int V>
-__global__ __launch_bounds__(256) void seg_reduce_l1(SegArgs3 jobs)
+// The rider's sums: a work item is (sum i, 256 float4 of the row); the slice's workgroups stride over the items.
+__device__ __forceinline__ void sum_rider_body(const SumRider &r)
 {
+    const int nsum = r.num[0] < r.max_sums ? r.num[0] : r.max_sums;
+    const int64_t q4 = r.row_floats / 4;
+    const int64_t nb = (q4 + 255) / 256;
+    for (int64_t it = blockIdx.x; it < nsum * nb; it += gridDim.x) {
+        const int i = (int)(it / nb);
+        const int64_t f = (it % nb) * 256 + threadIdx.x;
+        if (f >= q4) continue;
+        const int cnt = r.cnt[i];
+        const float4 *src = reinterpret_cast<const float4 *>(r.part) + (int64_t)r.first[i] * q4 + f;
+        float4 acc = src[0];
+        for (int c = 1; c < cnt; ++c) {
+            const float4 v = src[(int64_t)c * q4];
+            acc.x += v.x, acc.y += v.y, acc.z += v.z, acc.w += v.w;
+        }
+        reinterpret_cast<float4 *>(r.out)[(int64_t)r.seg[i] * q4 + f] = acc;
+    }
+}
+
+template <int V>
+__global__ __launch_bounds__(256) void seg_reduce_l1(SegArgs3 jobs, SumRider rider)
+{
+    if (rider.max_sums > 0 && blockIdx.y == gridDim.y - 1) {  // the last slice of the grid is the rider's
+        sum_rider_body(rider);
+        return;
+    }
     const SegArgs &a = jobs.j[blockIdx.y];
     const int lane = threadIdx.x & (kWave - 1);
     const int d = a.d;
@@ -147,8 +172,10 @@ __global__ __launch_bounds__(256) void seg_reduce_l2(SegArgs3 jobs)
     }
 }
 
-int launch_seg_reduce_jobs(const SegJob *jobs, int n_jobs, hipStream_t st, kge_timeline *timeline)
+int launch_seg_reduce_jobs(const SegJob *jobs, int n_jobs, hipStream_t st, kge_timeline *timeline, const SumRider *rider)
 {
+    const SumRider rd = rider && rider->max_sums > 0 ? *rider : SumRider{};
+    if (rd.max_sums > 0 && (rd.row_floats % 4 != 0 || !aligned16(rd.part) || !aligned16(rd.out))) return KGE_EINVAL;
     SegArgs3 args{};
     int m = 0;
     int64_t max_waves = 0, max_blocks = 0;
@@ -161,7 +188,7 @@ int launch_seg_reduce_jobs(const SegJob *jobs, int n_jobs, hipStream_t st, kge_t
         v4 = v4 && jb.d % 4 == 0 && aligned16(jb.occ) && aligned16(jb.out) && aligned16(jb.partial);
         ++m;
     }
-    if (m == 0) return KGE_OK;
+    if (m == 0 && rd.max_sums == 0) return KGE_OK;
     for (int q = 0; q < m; ++q) {
         const int V = v4 ? 4 : 1;
         const int64_t nblk = ceil_div(args.j[q].n, kSegL);
@@ -170,15 +197,17 @@ int launch_seg_reduce_jobs(const SegJob *jobs, int n_jobs, hipStream_t st, kge_t
         max_blocks = nblk > max_blocks ? nblk : max_blocks;
     }
     for (int q = m; q < 3; ++q) args.j[q] = args.j[0], args.j[q].n = 0;  // unused slots do nothing
-    const dim3 g1((unsigned)ceil_div(max_waves, 4), (unsigned)m), g2((unsigned)max_blocks, (unsigned)m), block(256);
+    int64_t g1x = ceil_div(max_waves, 4);
+    if (rd.max_sums > 0 && g1x < 256) g1x = 256;  // (a small reduction still gives the rider a grid's worth of workgroups)
+    const dim3 g1((unsigned)g1x, (unsigned)(m + (rd.max_sums > 0 ? 1 : 0))), g2((unsigned)max_blocks, (unsigned)m), block(256);
     if (v4) {
-        hipLaunchKernelGGL(seg_reduce_l1<4>, g1, block, 0, st, args);
+        hipLaunchKernelGGL(seg_reduce_l1<4>, g1, block, 0, st, args, rd);
         timeline_mark(timeline, st, "seg_reduce_l1");
-        hipLaunchKernelGGL(seg_reduce_l2<4>, g2, block, 0, st, args);
+        if (m > 0) hipLaunchKernelGGL(seg_reduce_l2<4>, g2, block, 0, st, args);
     } else {
-        hipLaunchKernelGGL(seg_reduce_l1<1>, g1, block, 0, st, args);
+        hipLaunchKernelGGL(seg_reduce_l1<1>, g1, block, 0, st, args, rd);
         timeline_mark(timeline, st, "seg_reduce_l1");
-        hipLaunchKernelGGL(seg_reduce_l2<1>, g2, block, 0, st, args);
+        if (m > 0) hipLaunchKernelGGL(seg_reduce_l2<1>, g2, block, 0, st, args);
     }
     timeline_mark(timeline, st, "seg_reduce_l2");
     KGE_CHECK_LAUNCH();

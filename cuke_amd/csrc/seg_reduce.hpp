@@ -18,7 +18,20 @@ struct SegJob {
 
 inline int64_t seg_partial_floats(int64_t n, int64_t d) { return ceil_div(n > 0 ? n : 1, kSegL) * 2 * d; }
 
+// Work that depends on nothing the reduction produces and rides in its level-1 launch (one more
+// slice of the grid): out row seg[i] = part row first[i] + ... + part row first[i] + cnt[i] - 1, for
+// i < num[0] (all four arrays live on the device).  TransR's split relation groups finish their
+// projection gradients this way instead of in a launch of their own.
+struct SumRider {
+    const float *part = nullptr;
+    float *out = nullptr;
+    const int32_t *num = nullptr, *seg = nullptr, *first = nullptr, *cnt = nullptr;
+    int64_t row_floats = 0;  // a multiple of 4
+    int max_sums = 0;        // 0: no rider
+};
+
 // Up to three jobs share the same two launches.
-int launch_seg_reduce_jobs(const SegJob *jobs, int n_jobs, hipStream_t st, kge_timeline *timeline = nullptr);
+int launch_seg_reduce_jobs(const SegJob *jobs, int n_jobs, hipStream_t st, kge_timeline *timeline = nullptr,
+                           const SumRider *rider = nullptr);
 
 }  // namespace kge

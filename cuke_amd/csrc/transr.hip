@@ -909,7 +909,7 @@ __device__ __forceinline__ void dm_sweep(const float *xs, const float *qs, int d
 // dM[g][i][j] = sum_{p in group g} xs[p][i] * qs[p][j].  A work item is (chunk of <= 256 triples
 // of one group, 32 rows i); the four waves split the columns j; K runs over the chunk's triples,
 // operands prefetched four supersteps ahead.  Groups longer than one chunk write per-chunk
-// partial matrices that transr_dm_finish_kernel adds up (keeps the longest K loop at 16 supersteps).
+// partial matrices that are added up beside the segmented reduction (keeps the longest K loop at 16 supersteps).
 __device__ __forceinline__ void transr_dm_body(const DmArgs &a, float *lds, int bid)
 {
     if (bid >= a.max_items) {
@@ -988,22 +988,16 @@ __global__ __launch_bounds__(256, KGE_TR_OCC) void transr_dx_dm_kernel(GemmArgs 
     }
 }
 
-// dM of a split group = sum of its partial matrices (slot order = ascending chunk order)
-__global__ __launch_bounds__(256) void transr_dm_finish_kernel(DmArgs a)
+// dM of a split group = sum of its partial matrices (slot order = ascending chunk order); the sums
+// ride in the segmented reduction's first launch
+static SumRider dm_finish_rider(const DmArgs &a, int64_t max_split)
 {
-    const int sidx = blockIdx.y;
-    if (sidx >= a.plan.num_split[0]) return;
-    const int64_t dd4 = (int64_t)a.d * a.d / 4;
-    const int64_t f = (int64_t)blockIdx.x * 256 + threadIdx.x;
-    if (f >= dd4) return;
-    const int g = a.plan.split_seg[sidx], first = a.plan.split_first[sidx], cnt = a.plan.split_cnt[sidx];
-    const float4 *src = reinterpret_cast<const float4 *>(a.part) + (int64_t)first * dd4 + f;
-    float4 acc = src[0];
-    for (int c = 1; c < cnt; ++c) {
-        const float4 v = src[(int64_t)c * dd4];
-        acc.x += v.x, acc.y += v.y, acc.z += v.z, acc.w += v.w;
-    }
-    reinterpret_cast<float4 *>(a.dm)[(int64_t)g * dd4 + f] = acc;
+    SumRider r;
+    r.part = a.part, r.out = a.dm;
+    r.num = a.plan.num_split, r.seg = a.plan.split_seg, r.first = a.plan.split_first, r.cnt = a.plan.split_cnt;
+    r.row_floats = (int64_t)a.d * a.d;
+    r.max_sums = (int)max_split;
+    return r;
 }
 
 // ---- host side -----------------------------------------------------------------------------
@@ -1211,9 +1205,6 @@ int launch_transr_bwd(const kge_tables *tab, const kge_batch *bat, const kge_sav
                            lds_with(f3, sizeof(float) * 4 * (size_t)d), st, da, f3);
         timeline_mark(bat->timeline, st, "transr_dm_kernel");
     }
-    hipLaunchKernelGGL(transr_dm_finish_kernel, dim3((unsigned)ceil_div((int64_t)d * d / 4, 256), (unsigned)p.dsplit),
-                       dim3(256), 0, st, da);
-    timeline_mark(bat->timeline, st, "transr_dm_finish_kernel");
     KGE_CHECK_LAUNCH();
     if (bat->insp_ready && hipStreamWaitEvent(st, reinterpret_cast<hipEvent_t>(bat->insp_ready), 0) != hipSuccess)
         return KGE_ELAUNCH;
@@ -1222,7 +1213,8 @@ int launch_transr_bwd(const kge_tables *tab, const kge_batch *bat, const kge_sav
     const SegJob jobs[2] = {
         {occ, bat->ent_insp, d, grads->ent_rows, reinterpret_cast<float *>(ws + p.off_part_e), false},
         {qs, ri, d, grads->rel_rows, reinterpret_cast<float *>(ws + p.off_part_r), true}};
-    return launch_seg_reduce_jobs(jobs, rescal ? 1 : 2, st, bat->timeline);
+    const SumRider finish = dm_finish_rider(da, p.dsplit);
+    return launch_seg_reduce_jobs(jobs, rescal ? 1 : 2, st, bat->timeline, &finish);
 }
 
 #include "transr_neg.hpp"

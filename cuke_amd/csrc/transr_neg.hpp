@@ -739,9 +739,6 @@ int launch_transr_neg_bwd(const kge_tables *tab, const kge_batch *bat, const kge
     hipLaunchKernelGGL(transr_dm_kernel, dim3((unsigned)(dm_items + s.U_cap)), dim3(256), sizeof(float) * 4 * (size_t)d, st, da,
                        FusedInsp{});
     timeline_mark(bat->timeline, st, "transr_dm_kernel");
-    hipLaunchKernelGGL(transr_dm_finish_kernel, dim3((unsigned)ceil_div((int64_t)d * d / 4, 256), (unsigned)s.dsplit), dim3(256),
-                       0, st, da);
-    timeline_mark(bat->timeline, st, "transr_dm_finish_kernel");
     TNEG_BY_WIDTH(d, hipLaunchKernelGGL(tneg_occ_kernel<NQ_>, dim3((unsigned)(ceil_div(s.B, 4) + s.NN)), dim3(256), 0, st, x, dxl,
                                         glist, gcount, occ));
     timeline_mark(bat->timeline, st, "tneg_occ_kernel");
@@ -750,5 +747,6 @@ int launch_transr_neg_bwd(const kge_tables *tab, const kge_batch *bat, const kge
         return KGE_ELAUNCH;
     const SegJob jobs[2] = {{occ, bat->ent_insp, d, grads->ent_rows, reinterpret_cast<float *>(ws + l.part_e), false},
                             {qr, ri, d, grads->rel_rows, reinterpret_cast<float *>(ws + l.part_r), false}};
-    return launch_seg_reduce_jobs(jobs, 2, st, bat->timeline);
+    const SumRider finish = dm_finish_rider(da, s.dsplit);  // the split groups' partial matrices
+    return launch_seg_reduce_jobs(jobs, 2, st, bat->timeline, &finish);
 }
