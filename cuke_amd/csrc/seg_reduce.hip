@@ -117,22 +117,25 @@ __global__ __launch_bounds__(256) void seg_reduce_l1(SegArgs3 jobs, SumRider rid
     flush(seg[cnt - 1]);
 }
 
+// One workgroup per (block, chunk of 64 V columns): the column chunks of a wide row are independent
+// chains of round trips and run side by side (nch = chunks of the widest job of the launch).
 template <int V>
-__global__ __launch_bounds__(256) void seg_reduce_l2(SegArgs3 jobs)
+__global__ __launch_bounds__(256) void seg_reduce_l2(SegArgs3 jobs, int nch)
 {
     __shared__ float s_part[4][kWave * 4];
     const SegArgs &a = jobs.j[blockIdx.y];
     const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x >> 6;
-    const int64_t j = blockIdx.x;
+    const int64_t j = blockIdx.x / nch;
+    const int c0 = (int)(blockIdx.x % nch) * kWave * V;
     const int64_t p0 = j * kSegL;
-    if (p0 >= a.n) return;  // uniform for the workgroup
+    if (p0 >= a.n || c0 >= a.d) return;  // uniform for the workgroup
     const int64_t p1 = p0 + kSegL < a.n ? p0 + kSegL : a.n;
     const int sg = a.sorted_seg[p1 - 1];
     const int s0 = a.seg_offsets[sg], s1 = a.seg_offsets[sg + 1];
     if (s1 <= p0 + kSegL || s0 < p0) return;  // no run starts here and continues
     const int64_t je = (s1 - 1) / kSegL;
     const int d = a.d;
-    for (int c0 = 0; c0 < d; c0 += kWave * V) {
+    {
         const int colv = c0 + lane * V;
         const bool active = colv < d;
         Vec<V> acc;
@@ -168,7 +171,6 @@ __global__ __launch_bounds__(256) void seg_reduce_l2(SegArgs3 jobs)
                           (s_part[2][lane * V + e] + s_part[3][lane * V + e]);
             r.store(a.out + (int64_t)sg * d + colv);
         }
-        __syncthreads();
     }
 }
 
@@ -178,7 +180,7 @@ int launch_seg_reduce_jobs(const SegJob *jobs, int n_jobs, hipStream_t st, kge_t
     if (rd.max_sums > 0 && (rd.row_floats % 4 != 0 || !aligned16(rd.part) || !aligned16(rd.out))) return KGE_EINVAL;
     SegArgs3 args{};
     int m = 0;
-    int64_t max_waves = 0, max_blocks = 0;
+    int64_t max_waves = 0, max_blocks = 0, max_nch = 1;
     bool v4 = true;
     for (int q = 0; q < n_jobs && m < 3; ++q) {
         const SegJob &jb = jobs[q];
@@ -195,19 +197,20 @@ int launch_seg_reduce_jobs(const SegJob *jobs, int n_jobs, hipStream_t st, kge_t
         const int64_t nch = ceil_div(args.j[q].d, kWave * V);
         max_waves = nblk * nch > max_waves ? nblk * nch : max_waves;
         max_blocks = nblk > max_blocks ? nblk : max_blocks;
+        max_nch = nch > max_nch ? nch : max_nch;
     }
     for (int q = m; q < 3; ++q) args.j[q] = args.j[0], args.j[q].n = 0;  // unused slots do nothing
     int64_t g1x = ceil_div(max_waves, 4);
     if (rd.max_sums > 0 && g1x < 256) g1x = 256;  // (a small reduction still gives the rider a grid's worth of workgroups)
-    const dim3 g1((unsigned)g1x, (unsigned)(m + (rd.max_sums > 0 ? 1 : 0))), g2((unsigned)max_blocks, (unsigned)m), block(256);
+    const dim3 g1((unsigned)g1x, (unsigned)(m + (rd.max_sums > 0 ? 1 : 0))), g2((unsigned)(max_blocks * max_nch), (unsigned)m), block(256);
     if (v4) {
         hipLaunchKernelGGL(seg_reduce_l1<4>, g1, block, 0, st, args, rd);
         timeline_mark(timeline, st, "seg_reduce_l1");
-        if (m > 0) hipLaunchKernelGGL(seg_reduce_l2<4>, g2, block, 0, st, args);
+        if (m > 0) hipLaunchKernelGGL(seg_reduce_l2<4>, g2, block, 0, st, args, (int)max_nch);
     } else {
         hipLaunchKernelGGL(seg_reduce_l1<1>, g1, block, 0, st, args, rd);
         timeline_mark(timeline, st, "seg_reduce_l1");
-        if (m > 0) hipLaunchKernelGGL(seg_reduce_l2<1>, g2, block, 0, st, args);
+        if (m > 0) hipLaunchKernelGGL(seg_reduce_l2<1>, g2, block, 0, st, args, (int)max_nch);
     }
     timeline_mark(timeline, st, "seg_reduce_l2");
     KGE_CHECK_LAUNCH();
