@@ -8,7 +8,8 @@ int launch_score_pos(const kge_tables *, const kge_batch *, float *, float *, fl
 int launch_score_pos_fused(const kge_tables *, const kge_batch *, float *, float *, float *, const FusedInsp *,
                            hipStream_t);
 int launch_score_neg(const kge_tables *, const kge_batch *, const float *, const float *, float *, float *,
-                     const FusedInsp *, void *, size_t, hipStream_t);
+                     const FusedInsp *, void *, size_t, hipStream_t, float *carry_pos);
+bool score_neg_carries_positives(const kge_tables *, const kge_batch *);
 size_t neg_split_workspace(const kge_tables *, const kge_batch *);
 int launch_transr_fwd(const kge_tables *, const kge_batch *, float *, float *, void *, size_t, hipStream_t);
 size_t transr_fwd_workspace(const kge_tables *, const kge_batch *);
@@ -230,7 +231,9 @@ int kge_score_fwd(const kge_tables *tab, const kge_batch *bat, float *pos, float
     }
     if (want_neg && tab->model == KGE_TRANSR && bat->rel_insp)  // positives and shared negatives in one grouped pass
         return launch_transr_neg_fwd(tab, bat, pos, neg, residual, workspace, workspace_bytes, st);
-    if (pos || side_pos || residual) {
+    // DistMult / ComplEx: the positives ride in the tile launch where nothing else does
+    const bool carry = want_neg && pos && !side_pos && !residual && !fuse && score_neg_carries_positives(tab, bat);
+    if (!carry && (pos || side_pos || residual)) {
         if ((tab->model == KGE_TRANSR || tab->model == KGE_RESCAL) && bat->rel_insp)
             rc = launch_transr_fwd(tab, bat, pos, residual, workspace, workspace_bytes, st);
         else {
@@ -241,7 +244,7 @@ int kge_score_fwd(const kge_tables *tab, const kge_batch *bat, float *pos, float
     }
     if (want_neg) {
         rc = launch_score_neg(tab, bat, side_pos, tab->model == KGE_ROTATE ? residual : nullptr, neg, side_neg,
-                              fuse ? &fi1 : nullptr, workspace, workspace_bytes, st);
+                              fuse ? &fi1 : nullptr, workspace, workspace_bytes, st, carry ? pos : nullptr);
         timeline_mark(bat->timeline, st, "score_neg_kernel");
         return rc;
     }

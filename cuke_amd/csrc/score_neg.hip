@@ -13,6 +13,7 @@
 #include <type_traits>
 
 #include "inspector_mid.hpp"
+#include "score_pos_body.hpp"
 #include "tile_common.hpp"
 
 namespace kge {
@@ -36,6 +37,11 @@ struct NegArgs {
     // adds the planes and finishes the scores.  ksplit <= 1: one workgroup per tile, scores written directly.
     int ksplit;
     float *partial;
+    // DistMult / ComplEx on the matrix-core tiles, nothing riding along: the workgroups behind the
+    // `tile_blocks` tile workgroups score the positives (their score does not enter the tiles, so the
+    // two need not be two launches).  pos_blocks == 0: none.
+    PosArgs pos;
+    int tile_blocks, pos_blocks;
 };
 
 typedef float v4f __attribute__((ext_vector_type(4)));
@@ -349,6 +355,11 @@ __global__ __launch_bounds__(256, KGE_TILE_OCC) void score_neg_mfma_kernel(NegAr
     extern __shared__ __align__(16) char dyn_smem[];
     if (fused_insp_block(fi, reinterpret_cast<uint32_t *>(dyn_smem))) return;
     static_assert(MODEL == KGE_DISTMULT || MODEL == KGE_COMPLEX || MODEL == KGE_TRANSF, "dot-product scores only");
+    if (a.pos_blocks > 0 && (int)blockIdx.x - fi.blocks >= a.tile_blocks) {  // the positives carried along
+        if constexpr (MODEL != KGE_TRANSF)
+            score_pos_body<MODEL, 2, 4>(a.pos, nullptr, (int64_t)((int)blockIdx.x - fi.blocks - a.tile_blocks));
+        return;
+    }
     constexpr int TB = 16 * RB, TN = 16 * RK;
     constexpr int SB = TB / 32, SN = TN / 32;
     constexpr int MB = RB / 2, NB = RK / 2;  // 16 x 16 blocks per wave
@@ -524,6 +535,16 @@ static int launch_neg_mp(const NegArgs &a, int64_t n_chunks, bool dot_valu, cons
     if constexpr (kDotModel) {
         if (!dot_valu) {
             const size_t lds = neg_lds(1, TB, TN, 1, fi);
+            if (a.pos_blocks > 0) {
+                NegArgs ac = a;
+                ac.tile_blocks = (int)(grid.x - (unsigned)fi.blocks);
+                const dim3 gridc(grid.x + (unsigned)a.pos_blocks);
+                if (tile == 4) hipLaunchKernelGGL((score_neg_mfma_kernel<MODEL, 4, 4>), gridc, dim3(256), lds, st, ac, fi);
+                else if (tile == 3) hipLaunchKernelGGL((score_neg_mfma_kernel<MODEL, 2, 4>), gridc, dim3(256), lds, st, ac, fi);
+                else hipLaunchKernelGGL((score_neg_mfma_kernel<MODEL, 2, 2>), gridc, dim3(256), lds, st, ac, fi);
+                KGE_CHECK_LAUNCH();
+                return KGE_OK;
+            }
             if (tile == 4) hipLaunchKernelGGL((score_neg_mfma_kernel<MODEL, 4, 4>), grid, dim3(256), lds, st, a, fi);
             else if (tile == 3) hipLaunchKernelGGL((score_neg_mfma_kernel<MODEL, 2, 4>), grid, dim3(256), lds, st, a, fi);
             else hipLaunchKernelGGL((score_neg_mfma_kernel<MODEL, 2, 2>), grid, dim3(256), lds, st, a, fi);
@@ -559,19 +580,34 @@ static int launch_neg_mp(const NegArgs &a, int64_t n_chunks, bool dot_valu, cons
     return KGE_OK;
 }
 
+// True if the shared-negative launch of this batch can score the positives as well (carry_pos of
+// launch_score_neg): DistMult / ComplEx on the matrix-core tiles with 128-bit row loads and no
+// inspector workgroups in the launch.
+bool score_neg_carries_positives(const kge_tables *tab, const kge_batch *bat)
+{
+    return (tab->model == KGE_DISTMULT || tab->model == KGE_COMPLEX) && bat->neg && bat->batch > 0 && !bat->fuse_inspection &&
+           !pair_sums_valu(tab) && rows_vectorizable(tab) && ceil_div(bat->batch, kPosWaves) < (1 << 30);
+}
+
 int launch_score_neg(const kge_tables *tab, const kge_batch *bat, const float *side_pos, const float *query,
                      float *out, float *side_neg, const FusedInsp *fused, void *workspace, size_t workspace_bytes,
-                     hipStream_t st)
+                     hipStream_t st, float *carry_pos)
 {
     const FusedInsp fi = fused ? *fused : FusedInsp{};
     if (bat->batch == 0) return KGE_OK;
+    if (carry_pos && (fused || !score_neg_carries_positives(tab, bat))) return KGE_EINVAL;
     const int64_t n_chunks = bat->batch / bat->chunk;
     if (n_chunks >= (1 << 24) || bat->chunk >= (1 << 30) || bat->n_neg >= (1 << 30)) return KGE_ESHAPE;
     const bool vec = rows_vectorizable(tab);
     const bool head = bat->neg_mode == KGE_NEG_HEAD;
     NegArgs a{tab->ent, tab->rel, tab->aux, head ? bat->t : bat->h, bat->r, bat->neg, side_pos, query, out, side_neg,
               bat->batch * bat->n_neg, (int)bat->chunk, (int)bat->n_neg, (int)tab->dim, (int)tab->rel_dim, tab->gamma,
-              vec ? 1 : 0, (int)n_chunks, head ? -1.0f : 1.0f, 1, nullptr};
+              vec ? 1 : 0, (int)n_chunks, head ? -1.0f : 1.0f, 1, nullptr, PosArgs{}, 0, 0};
+    if (carry_pos) {
+        a.pos = PosArgs{tab->ent, tab->rel, tab->aux, bat->h, bat->r, bat->t, bat->batch, (int)tab->dim, (int)tab->rel_dim,
+                        tab->gamma, carry_pos, nullptr, nullptr, 0};
+        a.pos_blocks = (int)ceil_div(bat->batch, kPosWaves);
+    }
     // the reduction axis is split when the caller's workspace has room for the partial planes
     const int ksplit = neg_ksplit(tab, bat);
     if (ksplit > 1 && workspace && workspace_bytes >= neg_split_workspace(tab, bat) && aligned16(workspace))
