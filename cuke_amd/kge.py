@@ -29,8 +29,27 @@ __all__ = ["KGEModel", "TrainStep", "Inspection", "Forward", "SparseGrads", "ins
 NEG_MODES = {"tail": 0, "head": 1}  # KGE_NEG_TAIL / KGE_NEG_HEAD
 
 
+_raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+_stream_objects: dict = {}
+
+
 def _stream() -> C.c_void_p:
+    if _raw_stream is not None:
+        return C.c_void_p(_raw_stream(torch.cuda.current_device()))
     return C.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def _current_stream(dev_index: int):
+    """``torch.cuda.current_stream()`` of a loop that asks every step: the raw handle is one C call,
+    and the Stream object that belongs to a handle is looked up once (torch's streams live in a pool
+    for the life of the process; ``current_stream()`` itself costs about 8 us of host time)."""
+    if _raw_stream is None:
+        return torch.cuda.current_stream(dev_index)
+    key = (dev_index, _raw_stream(dev_index))
+    st = _stream_objects.get(key)
+    if st is None:
+        st = _stream_objects[key] = torch.cuda.current_stream(dev_index)
+    return st
 
 
 def _ptr(t: torch.Tensor | None) -> C.c_void_p | None:
@@ -489,6 +508,7 @@ class TrainStep:
         self._pipelined = False   # the ring of run(pipeline=True) has been set up
         self._timeline = None     # set by kernel_times()
         self.side = torch.cuda.Stream(device=dev)  # default priority
+        self._dev_index = dev.index if dev.index is not None else torch.cuda.current_device()
         self.pos = torch.empty(B, **f32)
         self.neg = torch.empty((B, N), **f32) if neg is not None else None
         self.side_pos = torch.empty(B, **f32) if (model.model == "TransH" or
@@ -777,7 +797,7 @@ class TrainStep:
         inspections live in a ring of sets, so the side stream never waits for the step before.
         Results (``sparse_grads()``, ``pos`` ...) are those of the step enqueued last.  Not
         capturable into one graph: the dependencies cross steps."""
-        main = torch.cuda.current_stream()
+        main = _current_stream(self._dev_index)
         st = C.c_void_p(main.cuda_stream)
         for s_ in self._sets:  # cached unique counts belong to the batches of earlier steps
             s_.ent_insp._u = s_.rel_insp._u = None
