@@ -172,6 +172,12 @@ def test_train_step_eager_overlapped_and_graph_replays(oracle, name, over):
     assert step.fusable
     step.run()  # inspection fused into the score kernels' launches where the batch qualifies
     check("fused" if step.fusable else "default")
+    other = torch.cuda.Stream()  # a caller's own stream: the step follows torch's current stream
+    other.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(other):
+        step.run(overlap=True, fused=False)
+        step.run()
+    check("on a second stream")
     step.capture()
     for i in range(3):
         step.replay()

@@ -105,3 +105,20 @@ def test_sparse_optimizer_steps(oracle, dim):
     want_t, want_s = oracle.sparse_adagrad(table, state, ids, rows_full[:U], 0.05)
     assert_close(t_dev.cpu().numpy(), want_t, what="adagrad table", rows=True)
     assert_close(s_dev.cpu().numpy(), want_s, what="adagrad state")
+
+
+def test_current_stream_lookup_follows_the_stream_context():
+    """The step loop's cached lookup of torch's current stream: the Stream object that belongs to the
+    raw handle of the moment, inside and outside a stream context, and the same object on a second call."""
+    from cuke_amd import kge
+    idx = torch.cuda.current_device()
+    default = kge._current_stream(idx)
+    assert default.cuda_stream == torch.cuda.current_stream().cuda_stream
+    other = torch.cuda.Stream()
+    with torch.cuda.stream(other):
+        inside = kge._current_stream(idx)
+        assert inside.cuda_stream == other.cuda_stream
+        assert kge._current_stream(idx) is inside
+        assert kge._stream().value == other.cuda_stream
+    assert kge._current_stream(idx) is default
+    assert (kge._stream().value or 0) == torch.cuda.current_stream().cuda_stream
