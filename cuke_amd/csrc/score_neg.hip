@@ -37,9 +37,9 @@ struct NegArgs {
     // adds the planes and finishes the scores.  ksplit <= 1: one workgroup per tile, scores written directly.
     int ksplit;
     float *partial;
-    // DistMult / ComplEx on the matrix-core tiles, nothing riding along: the workgroups behind the
-    // `tile_blocks` tile workgroups score the positives (their score does not enter the tiles, so the
-    // two need not be two launches).  pos_blocks == 0: none.
+    // TransE, DistMult / ComplEx on the matrix-core tiles, nothing riding along: the workgroups behind
+    // the `tile_blocks` tile workgroups score the positives (their score does not enter the tiles, so
+    // the two need not be two launches).  pos_blocks == 0: none.
     PosArgs pos;
     int tile_blocks, pos_blocks;
 };
@@ -79,6 +79,12 @@ __global__ __launch_bounds__(256, KGE_TILE_OCC) void score_neg_kernel(NegArgs a,
 {
     extern __shared__ __align__(16) char dyn_smem[];
     if (fused_insp_block(fi, reinterpret_cast<uint32_t *>(dyn_smem))) return;
+    if constexpr (MODEL == KGE_TRANSE) {  // the positives carried along (NegArgs::pos)
+        if (a.pos_blocks > 0 && (int)blockIdx.x - fi.blocks >= a.tile_blocks) {
+            score_pos_body<MODEL, P, 4>(a.pos, nullptr, (int64_t)((int)blockIdx.x - fi.blocks - a.tile_blocks));
+            return;
+        }
+    }
     constexpr int TB = 16 * RB, TN = 16 * RK;
     constexpr int NPA = (MODEL == KGE_ROTATE || MODEL == KGE_TRANSH) ? 2 : 1;
     constexpr int NPT = MODEL == KGE_ROTATE ? 2 : 1;
@@ -96,7 +102,7 @@ __global__ __launch_bounds__(256, KGE_TILE_OCC) void score_neg_kernel(NegArgs a,
     int c, tile_y, tile_x;
     int lid = blockIdx.x - fi.blocks, split = 0;
     if (a.ksplit > 1) {  // (never TransH: its w . t' sweep needs the whole row)
-        const int tiles = (int)(gridDim.x - fi.blocks) / a.ksplit;  // a multiple of 8: the tile keeps its XCD
+        const int tiles = a.tile_blocks / a.ksplit;  // a multiple of 8: the tile keeps its XCD
         split = lid / tiles, lid -= split * tiles;
     }
     if (!xcd_tile(lid, (a.N + TN - 1) / TN, (a.C + TB - 1) / TB, a.n_chunks, c, tile_y, tile_x)) return;
@@ -520,8 +526,9 @@ size_t neg_split_workspace(const kge_tables *tab, const kge_batch *bat)
 }
 
 template <int MODEL, int P>
-static int launch_neg_mp(const NegArgs &a, int64_t n_chunks, bool dot_valu, const FusedInsp &fi, hipStream_t st)
+static int launch_neg_mp(const NegArgs &a_in, int64_t n_chunks, bool dot_valu, const FusedInsp &fi, hipStream_t st)
 {
+    NegArgs a = a_in;
     constexpr int NPA = (MODEL == KGE_ROTATE || MODEL == KGE_TRANSH) ? 2 : 1, NPT = MODEL == KGE_ROTATE ? 2 : 1;
     const int64_t big_tiles = ceil_div(a.C, 64) * ceil_div(a.N, 64) * n_chunks;
     // Small tiles up to about 1024 big tiles: more waves to hide latency (32x32 is ~20 % faster than
@@ -531,20 +538,13 @@ static int launch_neg_mp(const NegArgs &a, int64_t n_chunks, bool dot_valu, cons
     constexpr bool kDotModel = MODEL == KGE_DISTMULT || MODEL == KGE_COMPLEX || MODEL == KGE_TRANSF;
     const int tile = big_tiles >= 1024 ? 4 : (kDotModel && !dot_valu ? 3 : 2);  // 2: 32x32, 3: 32x64, 4: 64x64
     const int TB = tile == 4 ? 64 : 32, TN = tile == 2 ? 32 : 64;
-    const dim3 grid(xcd_grid(ceil_div(a.N, TN), ceil_div(a.C, TB), n_chunks) + (unsigned)fi.blocks);
+    // (workgroups that score the positives, if the launch carries them, follow the tiles')
+    const unsigned tile_blocks = xcd_grid(ceil_div(a.N, TN), ceil_div(a.C, TB), n_chunks) * (unsigned)(a.ksplit > 1 ? a.ksplit : 1);
+    a.tile_blocks = (int)tile_blocks;
+    const dim3 grid(tile_blocks + (unsigned)fi.blocks + (unsigned)a.pos_blocks);
     if constexpr (kDotModel) {
         if (!dot_valu) {
             const size_t lds = neg_lds(1, TB, TN, 1, fi);
-            if (a.pos_blocks > 0) {
-                NegArgs ac = a;
-                ac.tile_blocks = (int)(grid.x - (unsigned)fi.blocks);
-                const dim3 gridc(grid.x + (unsigned)a.pos_blocks);
-                if (tile == 4) hipLaunchKernelGGL((score_neg_mfma_kernel<MODEL, 4, 4>), gridc, dim3(256), lds, st, ac, fi);
-                else if (tile == 3) hipLaunchKernelGGL((score_neg_mfma_kernel<MODEL, 2, 4>), gridc, dim3(256), lds, st, ac, fi);
-                else hipLaunchKernelGGL((score_neg_mfma_kernel<MODEL, 2, 2>), gridc, dim3(256), lds, st, ac, fi);
-                KGE_CHECK_LAUNCH();
-                return KGE_OK;
-            }
             if (tile == 4) hipLaunchKernelGGL((score_neg_mfma_kernel<MODEL, 4, 4>), grid, dim3(256), lds, st, a, fi);
             else if (tile == 3) hipLaunchKernelGGL((score_neg_mfma_kernel<MODEL, 2, 4>), grid, dim3(256), lds, st, a, fi);
             else hipLaunchKernelGGL((score_neg_mfma_kernel<MODEL, 2, 2>), grid, dim3(256), lds, st, a, fi);
@@ -556,9 +556,7 @@ static int launch_neg_mp(const NegArgs &a, int64_t n_chunks, bool dot_valu, cons
     const bool save = MODEL == KGE_TRANSH && a.side_neg;
     if (a.ksplit > 1) {  // (neg_ksplit: 32 x 32 tiles of TransE / RotatE)
         if constexpr (MODEL == KGE_TRANSE || MODEL == KGE_ROTATE) {
-            const unsigned tiles = xcd_grid(ceil_div(a.N, TN), ceil_div(a.C, TB), n_chunks);
-            hipLaunchKernelGGL((score_neg_kernel<MODEL, P, 2, 2, false>), dim3(tiles * a.ksplit + (unsigned)fi.blocks), dim3(256),
-                               lds, st, a, fi);
+            hipLaunchKernelGGL((score_neg_kernel<MODEL, P, 2, 2, false>), grid, dim3(256), lds, st, a, fi);
             hipLaunchKernelGGL((score_neg_finish_kernel<MODEL, P>), dim3((unsigned)ceil_div(a.plane, 256)), dim3(256), 0, st,
                                a.partial, a.ksplit, a.plane, a.gamma, a.out);
             KGE_CHECK_LAUNCH();
@@ -581,12 +579,14 @@ static int launch_neg_mp(const NegArgs &a, int64_t n_chunks, bool dot_valu, cons
 }
 
 // True if the shared-negative launch of this batch can score the positives as well (carry_pos of
-// launch_score_neg): DistMult / ComplEx on the matrix-core tiles with 128-bit row loads and no
-// inspector workgroups in the launch.
+// launch_score_neg): TransE, or DistMult / ComplEx on the matrix-core tiles, with 128-bit row loads
+// and no inspector workgroups in the launch (these models' tiles do not read what the positives'
+// kernel writes).
 bool score_neg_carries_positives(const kge_tables *tab, const kge_batch *bat)
 {
-    return (tab->model == KGE_DISTMULT || tab->model == KGE_COMPLEX) && bat->neg && bat->batch > 0 && !bat->fuse_inspection &&
-           !pair_sums_valu(tab) && rows_vectorizable(tab) && ceil_div(bat->batch, kPosWaves) < (1 << 30);
+    const bool dot = (tab->model == KGE_DISTMULT || tab->model == KGE_COMPLEX) && !pair_sums_valu(tab);
+    return (dot || tab->model == KGE_TRANSE) && bat->neg && bat->batch > 0 && !bat->fuse_inspection && rows_vectorizable(tab) &&
+           ceil_div(bat->batch, kPosWaves) < (1 << 30);
 }
 
 int launch_score_neg(const kge_tables *tab, const kge_batch *bat, const float *side_pos, const float *query,
