@@ -139,6 +139,30 @@ def test_small_batch_splits_the_row_over_workgroups(oracle, model, dim, p, mode)
     assert_close(unsplit.cpu().numpy(), negs, what=f"{model} unsplit negatives")
 
 
+@pytest.mark.parametrize("model,p", [("TransE", 1), ("TransE", 2), ("DistMult", 2), ("ComplEx", 2)])
+@pytest.mark.parametrize("mode", ["tail", "head"])
+@pytest.mark.parametrize("batch,chunk,n_neg,dim", [(130, 26, 7, 64), (96, 32, 40, 640), (1024, 256, 256, 256)])
+def test_positives_carried_by_the_tile_launch(oracle, model, p, mode, batch, chunk, n_neg, dim):
+    """TransE / DistMult / ComplEx with shared negatives: the positives are scored by workgroups of the tile
+    launch (no launch of their own).  Their scores must equal, bit for bit, those of the positives' own kernel
+    (a call without negatives), also where the batch is not a multiple of the four positives of a workgroup,
+    where the tile launch splits the reduction axis, and where the pair sums stay on the vector ALUs (then the
+    dot-product models launch the positives' kernel themselves)."""
+    w = synth.custom_workload(model, n_ent=500, n_rel=13, dim=dim, batch=batch, chunk=chunk, n_neg=n_neg, norm_p=p,
+                              sigma=0.3, ent_zipf=1.1, seed=batch + dim + p)
+    a = w.arrays
+    m, ix = gpu_model(w)
+    alone = m.score(ix["h"], ix["r"], ix["t"]).pos
+    fw = m.score(ix["h"], ix["r"], ix["t"], ix["neg"], w.chunk, neg_mode=mode)
+    assert torch.equal(fw.pos, alone)
+    pos, negs = oracle.score(model, a["E"], a["R"], a["A"], a["h"], a["r"], a["t"], a["neg"], w.chunk, p=p, neg_mode=mode)
+    assert_close(fw.pos.cpu().numpy(), pos, what=f"{model} carried positives")
+    assert_close(fw.neg.cpu().numpy(), negs, what=f"{model} negatives beside carried positives")
+    m.pair_sums = "vector_alus"
+    fv = m.score(ix["h"], ix["r"], ix["t"], ix["neg"], w.chunk, neg_mode=mode)
+    assert torch.equal(fv.pos, alone)
+
+
 @pytest.mark.parametrize("name,over", [
     ("cfg2_distmult", dict(n_ent=100_000, batch=1024)),
     ("cfg2_complex", dict(n_ent=100_000, batch=1024)),
