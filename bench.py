@@ -34,6 +34,7 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0       # MI355X HBM3E, published
+WARMUP_MIN_S = 0.02         # least untimed warm-up in front of every timed region
 FP32_PEAK_TFLOPS = 157.3    # MI355X fp32 vector / fp32 MFMA, published
 
 ALL_WORKLOADS = ["cfg5_transh", "cfg1_transe", "cfg2_distmult", "cfg2_complex", "cfg3_transr", "cfg4_rotate"]
@@ -450,8 +451,14 @@ def run_workload(name, args, torch):
         check["seconds"] = round(time.perf_counter() - t0, 2)
 
     def timed(one):
-        for _ in range(args.warmup):
+        # untimed warm-up: the W steps asked for, and at least WARMUP_MIN_S of device work (a timed region
+        # of 20 steps of 60 us is over before the clocks have settled otherwise)
+        t0, n = time.perf_counter(), 0
+        while n < args.warmup or time.perf_counter() - t0 < WARMUP_MIN_S:
             one()
+            n += 1
+            if n % 16 == 0:
+                torch.cuda.synchronize()
         torch.cuda.synchronize()
         return time_events(one, args.steps, torch)
 
@@ -571,7 +578,7 @@ def run_workload(name, args, torch):
         "data": "synthetic (seeded N(0,sigma) tables, Zipf/uniform indices, shared negatives per chunk)",
         "config": {"workload": w.name, "score_function": w.model, "n_ent": w.n_ent, "n_rel": w.n_rel, "dim": w.dim,
                    "batch": w.batch, "chunk": w.chunk, "n_neg": w.n_neg, "norm_p": w.norm_p,
-                   "backward": do_bwd, "loss": w.loss, "issue": issue, "rotating_batches": nb,
+                   "backward": do_bwd, "loss": w.loss, "issue": issue, "rotating_batches": nb, "warmup_min_ms": WARMUP_MIN_S * 1e3,
                    "pair_sums": "matrix cores, fp32" if w.model in ("DistMult", "ComplEx") and w.chunk else "vector ALUs",
                    "ms_per_step_rotating_direct": ms_rot, "ms_per_step_rotating_graph": ms_graph,
                    "ms_per_step_rotating_staged": ms_staged,
