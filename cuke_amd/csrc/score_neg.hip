@@ -74,7 +74,7 @@ __device__ __forceinline__ void pair_elem(float &acc, float &acc2, float a0, flo
     }
 }
 
-template <int MODEL, int P, int RB, int RK, bool SAVE>
+template <int MODEL, int P, int RB, int RK, bool SAVE, bool VEC4>
 __global__ __launch_bounds__(256, KGE_TILE_OCC) void score_neg_kernel(NegArgs a, FusedInsp fi)
 {
     extern __shared__ __align__(16) char dyn_smem[];
@@ -109,7 +109,8 @@ __global__ __launch_bounds__(256, KGE_TILE_OCC) void score_neg_kernel(NegArgs a,
     const int bt0 = tile_y * TB, kt0 = tile_x * TN;
     const int d = a.d, half = d >> 1;
     const int klen = MODEL == KGE_ROTATE ? half : d;
-    const bool vec = a.vec != 0;
+    constexpr bool vec = VEC4;  // 128-bit row loads: a compile-time choice (as a run-time one the two forms
+                                // of the raw loads are merged into the scalar one)
 
     // rows this thread stages
     const float *ph[SB], *pr[SB], *pw[SB], *pq[SB];
@@ -136,30 +137,54 @@ __global__ __launch_bounds__(256, KGE_TILE_OCC) void score_neg_kernel(NegArgs a,
         pt[s] = a.ent + a.neg[(int64_t)c * a.N + (okk[s] ? kl : a.N - 1)] * (int64_t)d;
     }
 
-    float4 ra[NPA][SB], rt[NPT][SN];
+    // The rows of the next slice are requested as raw operands -- clamped addresses, no select, no
+    // arithmetic on what was loaded -- and only become query rows (h o r, h + r - (w.h) w ..., zeros
+    // outside the tile) when the slice is written to LDS: anything that touches a loaded register makes
+    // the compiler wait for the loads where they are issued, i.e. in front of the compute they are meant
+    // to overlap.
+    constexpr int NRAW = query_raw_count<MODEL>();
+    float4 qraw[SB][NRAW], rt[NPT][SN];
 
     auto load_slice_v = [&](auto vtag, int j0) {
         constexpr bool VEC = decltype(vtag)::value;
         const int j = j0 + scol;
 #pragma unroll
-        for (int s = 0; s < SB; ++s) {
-            const int lim = okb[s] ? klen : 0;
-            float4 q0, q1;
-            load_query<MODEL, VEC>(ph[s], pr[s], pw[s], pa[s], j, lim, half, q0, q1, pq[s], a.rsign);
-            ra[0][s] = q0;
-            if constexpr (NPA == 2) ra[1][s] = q1;
-        }
+        for (int s = 0; s < SB; ++s)
+            load_query_raw<MODEL, VEC>(ph[s], pr[s], pw[s], pq[s], j, okb[s] ? klen : 0, half, qraw[s]);
 #pragma unroll
         for (int s = 0; s < SN; ++s) {
             const int lim = okk[s] ? klen : 0;
-            rt[0][s] = ld4<VEC>(pt[s], j, lim);
-            if constexpr (MODEL == KGE_ROTATE) rt[1][s] = ld4<VEC>(pt[s] + half, j, lim);
+            rt[0][s] = ld4_raw<VEC>(pt[s], j, lim);
+            if constexpr (MODEL == KGE_ROTATE) rt[1][s] = ld4_raw<VEC>(pt[s] + half, j, lim);
         }
     };
 
     auto load_slice = [&](int j0, int) {  // one uniform branch per slice, none per load
-        if (vec) load_slice_v(std::true_type{}, j0);
-        else load_slice_v(std::false_type{}, j0);
+        load_slice_v(std::integral_constant<bool, VEC4>{}, j0);
+    };
+
+    // the slice that load_slice(j0) requested: query rows formed, tails masked, written to LDS
+    auto stage_slice_v = [&](auto vtag, int j0) {
+        constexpr bool VEC = decltype(vtag)::value;
+        const int j = j0 + scol;
+#pragma unroll
+        for (int q = 0; q < SB; ++q) {
+            float4 q0, q1;
+            combine_query<MODEL, VEC>(qraw[q], pa[q], j, okb[q] ? klen : 0, half, a.rsign, q0, q1);
+            *reinterpret_cast<float4 *>(&sA[0][srow + 32 * q][scol]) = kScaled ? scale4(q0, kSgnScale) : q0;
+            if constexpr (NPA == 2)
+                *reinterpret_cast<float4 *>(&sA[1][srow + 32 * q][scol]) = kScaled ? scale4(q1, kSgnScale) : q1;
+        }
+#pragma unroll
+        for (int q = 0; q < SN; ++q)
+#pragma unroll
+            for (int pl = 0; pl < NPT; ++pl) {
+                const float4 v = mask4<VEC>(rt[pl][q], j, okk[q] ? klen : 0);
+                *reinterpret_cast<float4 *>(&sT[pl][srow + 32 * q][scol]) = kScaled ? scale4(v, kSgnScale) : v;
+            }
+    };
+    auto stage_slice = [&](int j0) {
+        stage_slice_v(std::integral_constant<bool, VEC4>{}, j0);
     };
 
     float acc[RB][RK], cdot[RB][RK], acc2[RB][RK];
@@ -184,20 +209,10 @@ __global__ __launch_bounds__(256, KGE_TILE_OCC) void score_neg_kernel(NegArgs a,
         if (slice0 < slice1) load_slice(slice0 * kKD, pass);
 #pragma unroll 1
         for (int s = slice0; s < slice1; ++s) {
-#pragma unroll
-            for (int q = 0; q < SB; ++q)
-#pragma unroll
-                for (int pl = 0; pl < NPA; ++pl)
-                    *reinterpret_cast<float4 *>(&sA[pl][srow + 32 * q][scol]) =
-                        kScaled ? scale4(ra[pl][q], kSgnScale) : ra[pl][q];
-#pragma unroll
-            for (int q = 0; q < SN; ++q)
-#pragma unroll
-                for (int pl = 0; pl < NPT; ++pl)
-                    *reinterpret_cast<float4 *>(&sT[pl][srow + 32 * q][scol]) =
-                        kScaled ? scale4(rt[pl][q], kSgnScale) : rt[pl][q];
+            stage_slice(s * kKD);
             __syncthreads();
             if (s + 1 < slice1) load_slice((s + 1) * kKD, pass);
+            __builtin_amdgcn_sched_barrier(0);  // (the requests go out before the compute, not after it)
             // (TransH keeps three sums per pair, RotatE two row planes: unrolled all the way, the hoisted LDS reads push the
             // 4 x 4 micro-tile over the register budget and twenty to fifty registers per lane go through
             // scratch memory every step)
@@ -255,27 +270,31 @@ __global__ __launch_bounds__(256, KGE_TILE_OCC) void score_neg_kernel(NegArgs a,
         float4 rw[SB];
         auto load_w = [&](int j0) {  // one uniform branch per slice, none per load
             const int j = j0 + scol;
-            if (vec) {
 #pragma unroll
-                for (int q = 0; q < SB; ++q) rw[q] = ld4<true>(pw[q], j, okb[q] ? d : 0);
+            for (int q = 0; q < SB; ++q) rw[q] = ld4_raw<VEC4>(pw[q], j, okb[q] ? d : 0);
 #pragma unroll
-                for (int q = 0; q < SN; ++q) rt[0][q] = ld4<true>(pt[q], j, okk[q] ? d : 0);
-            } else {
+            for (int q = 0; q < SN; ++q) rt[0][q] = ld4_raw<VEC4>(pt[q], j, okk[q] ? d : 0);
+        };
+        auto stage_w = [&](int j0) {  // (raw loads, masked when written: see load_slice_v)
+            const int j = j0 + scol;
 #pragma unroll
-                for (int q = 0; q < SB; ++q) rw[q] = ld4<false>(pw[q], j, okb[q] ? d : 0);
+            for (int q = 0; q < SB; ++q) {
+                const int lim = okb[q] ? d : 0;
+                *reinterpret_cast<float4 *>(&sA[1][srow + 32 * q][scol]) = mask4<VEC4>(rw[q], j, lim);
+            }
 #pragma unroll
-                for (int q = 0; q < SN; ++q) rt[0][q] = ld4<false>(pt[q], j, okk[q] ? d : 0);
+            for (int q = 0; q < SN; ++q) {
+                const int lim = okk[q] ? d : 0;
+                *reinterpret_cast<float4 *>(&sT[0][srow + 32 * q][scol]) = mask4<VEC4>(rt[0][q], j, lim);
             }
         };
         load_w(0);
 #pragma unroll 1
         for (int s = 0; s < nslice; ++s) {
-#pragma unroll
-            for (int q = 0; q < SB; ++q) *reinterpret_cast<float4 *>(&sA[1][srow + 32 * q][scol]) = rw[q];
-#pragma unroll
-            for (int q = 0; q < SN; ++q) *reinterpret_cast<float4 *>(&sT[0][srow + 32 * q][scol]) = rt[0][q];
+            stage_w(s * kKD);
             __syncthreads();
             if (s + 1 < nslice) load_w((s + 1) * kKD);
+            __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
             for (int g = 0; g < kKD / 16; ++g) {
                 float4 av[MB], tv[NB];
@@ -355,7 +374,7 @@ __global__ __launch_bounds__(256, KGE_TILE_OCC) void score_neg_kernel(NegArgs a,
 // s pairs lane group g = l / 16 with k = 4 g + s (any pairing works as long as both operands use
 // it), so a lane's values for four steps are one 128-bit LDS read of its row.
 
-template <int MODEL, int RB, int RK>
+template <int MODEL, int RB, int RK, bool VEC4>
 __global__ __launch_bounds__(256, KGE_TILE_OCC) void score_neg_mfma_kernel(NegArgs a, FusedInsp fi)
 {
     extern __shared__ __align__(16) char dyn_smem[];
@@ -383,7 +402,8 @@ __global__ __launch_bounds__(256, KGE_TILE_OCC) void score_neg_mfma_kernel(NegAr
     if (!xcd_tile(blockIdx.x - fi.blocks, (a.N + TN - 1) / TN, (a.C + TB - 1) / TB, a.n_chunks, c, tile_y, tile_x)) return;
     const int bt0 = tile_y * TB, kt0 = tile_x * TN;
     const int d = a.d, half = d >> 1;
-    const bool vec = a.vec != 0;
+    constexpr bool vec = VEC4;  // 128-bit row loads: a compile-time choice (as a run-time one the two forms
+                                // of the raw loads are merged into the scalar one)
 
     const float *ph[SB], *pr[SB];
     bool okb[SB];
@@ -404,21 +424,30 @@ __global__ __launch_bounds__(256, KGE_TILE_OCC) void score_neg_mfma_kernel(NegAr
         pt[s] = a.ent + a.neg[(int64_t)c * a.N + (okk[s] ? kl : a.N - 1)] * (int64_t)d;
     }
 
-    float4 ra[SB], rt[SN];
-    auto load_slice_v = [&](auto vtag, int j0) {
-        constexpr bool VEC = decltype(vtag)::value;
+    // Raw operands of the next slice are in flight during the matrix-core work of this one; they are
+    // combined into the query rows and masked when they are written to LDS (see score_neg_kernel).
+    // (Two or four slices ahead measure the same: the launch is bound by its index chains and its
+    // eight barrier pairs, not by the rows' latency.)
+    constexpr int NRAW = query_raw_count<MODEL>();
+    float4 qraw[SB][NRAW], rt[SN];
+    auto load_slice = [&](int j0, float4 (&qr)[SB][NRAW], float4 (&tr)[SN]) {
         const int j = j0 + scol;
 #pragma unroll
-        for (int s = 0; s < SB; ++s) {
-            float4 q1;
-            load_query<MODEL, VEC>(ph[s], pr[s], nullptr, 0.0f, j, okb[s] ? d : 0, half, ra[s], q1, nullptr, a.rsign);
+        for (int s = 0; s < SB; ++s) load_query_raw<MODEL, VEC4>(ph[s], pr[s], nullptr, nullptr, j, okb[s] ? d : 0, half, qr[s]);
+#pragma unroll
+        for (int s = 0; s < SN; ++s) tr[s] = ld4_raw<VEC4>(pt[s], j, okk[s] ? d : 0);
+    };
+    auto stage_slice = [&](int j0, const float4 (&qr)[SB][NRAW], const float4 (&tr)[SN]) {
+        const int j = j0 + scol;
+#pragma unroll
+        for (int q = 0; q < SB; ++q) {
+            float4 q0, q1;
+            combine_query<MODEL, VEC4>(qr[q], 0.0f, j, okb[q] ? d : 0, half, a.rsign, q0, q1);
+            *reinterpret_cast<float4 *>(&sA[srow + 32 * q][scol]) = q0;
         }
 #pragma unroll
-        for (int s = 0; s < SN; ++s) rt[s] = ld4<VEC>(pt[s], j, okk[s] ? d : 0);
-    };
-    auto load_slice = [&](int j0) {
-        if (vec) load_slice_v(std::true_type{}, j0);
-        else load_slice_v(std::false_type{}, j0);
+        for (int q = 0; q < SN; ++q)
+            *reinterpret_cast<float4 *>(&sT[srow + 32 * q][scol]) = mask4<VEC4>(tr[q], j, okk[q] ? d : 0);
     };
 
     // two accumulators per block (one per half of the slice) keep consecutive MFMAs independent
@@ -431,15 +460,13 @@ __global__ __launch_bounds__(256, KGE_TILE_OCC) void score_neg_mfma_kernel(NegAr
             for (int n = 0; n < NB; ++n) acc[g][m][n] = v4f{0.0f, 0.0f, 0.0f, 0.0f};
 
     const int nslice = (d + kKD - 1) / kKD;
-    load_slice(0);
+    load_slice(0, qraw, rt);
 #pragma unroll 1
     for (int s = 0; s < nslice; ++s) {
-#pragma unroll
-        for (int q = 0; q < SB; ++q) *reinterpret_cast<float4 *>(&sA[srow + 32 * q][scol]) = ra[q];
-#pragma unroll
-        for (int q = 0; q < SN; ++q) *reinterpret_cast<float4 *>(&sT[srow + 32 * q][scol]) = rt[q];
+        stage_slice(s * kKD, qraw, rt);
         __syncthreads();
-        if (s + 1 < nslice) load_slice((s + 1) * kKD);
+        if (s + 1 < nslice) load_slice((s + 1) * kKD, qraw, rt);
+        __builtin_amdgcn_sched_barrier(0);  // (the requests go out before the matrix-core work, not after it)
 #pragma unroll
         for (int g = 0; g < kKD / 16; ++g) {
             float4 av[MB], tv[NB];
@@ -525,6 +552,17 @@ size_t neg_split_workspace(const kge_tables *tab, const kge_batch *bat)
     return s > 1 ? sizeof(float) * (size_t)s * (size_t)(bat->batch * bat->n_neg) : 0;
 }
 
+// one launch, the 128-bit-load form of the kernel where the rows allow it
+template <typename K>
+static void launch_neg_k(K kernel, dim3 grid, size_t lds, hipStream_t st, const NegArgs &a, const FusedInsp &fi)
+{
+    hipLaunchKernelGGL(kernel, grid, dim3(256), lds, st, a, fi);
+}
+#define NEG_LAUNCH(KERNEL, ...)                                                    \
+    (a.vec ? launch_neg_k(KERNEL<__VA_ARGS__, true>, grid, lds, st, a, fi)         \
+           : launch_neg_k(KERNEL<__VA_ARGS__, false>, grid, lds, st, a, fi))
+#define NEG_LAUNCH_VEC(KERNEL, ...) launch_neg_k(KERNEL<__VA_ARGS__, true>, grid, lds, st, a, fi)
+
 template <int MODEL, int P>
 static int launch_neg_mp(const NegArgs &a_in, int64_t n_chunks, bool dot_valu, const FusedInsp &fi, hipStream_t st)
 {
@@ -536,7 +574,9 @@ static int launch_neg_mp(const NegArgs &a_in, int64_t n_chunks, bool dot_valu, c
     // launches are bound by the rows its workgroups pull from L2, does best with 32x64).  The
     // inspector workgroups that share the machine with these launches raise their wave priority.
     constexpr bool kDotModel = MODEL == KGE_DISTMULT || MODEL == KGE_COMPLEX || MODEL == KGE_TRANSF;
-    const int tile = big_tiles >= 1024 ? 4 : (kDotModel && !dot_valu ? 3 : 2);  // 2: 32x32, 3: 32x64, 4: 64x64
+    // Rows without 128-bit loads (dim % 4 != 0, unaligned tables) take the 32x32 tile whatever the size:
+    // only that tile is compiled in the scalar-load form.
+    const int tile = !a.vec ? 2 : big_tiles >= 1024 ? 4 : (kDotModel && !dot_valu ? 3 : 2);  // 2: 32x32, 3: 32x64, 4: 64x64
     const int TB = tile == 4 ? 64 : 32, TN = tile == 2 ? 32 : 64;
     // (workgroups that score the positives, if the launch carries them, follow the tiles')
     const unsigned tile_blocks = xcd_grid(ceil_div(a.N, TN), ceil_div(a.C, TB), n_chunks) * (unsigned)(a.ksplit > 1 ? a.ksplit : 1);
@@ -545,9 +585,9 @@ static int launch_neg_mp(const NegArgs &a_in, int64_t n_chunks, bool dot_valu, c
     if constexpr (kDotModel) {
         if (!dot_valu) {
             const size_t lds = neg_lds(1, TB, TN, 1, fi);
-            if (tile == 4) hipLaunchKernelGGL((score_neg_mfma_kernel<MODEL, 4, 4>), grid, dim3(256), lds, st, a, fi);
-            else if (tile == 3) hipLaunchKernelGGL((score_neg_mfma_kernel<MODEL, 2, 4>), grid, dim3(256), lds, st, a, fi);
-            else hipLaunchKernelGGL((score_neg_mfma_kernel<MODEL, 2, 2>), grid, dim3(256), lds, st, a, fi);
+            if (tile == 4) NEG_LAUNCH_VEC(score_neg_mfma_kernel, MODEL, 4, 4);
+            else if (tile == 3) NEG_LAUNCH_VEC(score_neg_mfma_kernel, MODEL, 2, 4);
+            else NEG_LAUNCH(score_neg_mfma_kernel, MODEL, 2, 2);
             KGE_CHECK_LAUNCH();
             return KGE_OK;
         }
@@ -556,7 +596,7 @@ static int launch_neg_mp(const NegArgs &a_in, int64_t n_chunks, bool dot_valu, c
     const bool save = MODEL == KGE_TRANSH && a.side_neg;
     if (a.ksplit > 1) {  // (neg_ksplit: 32 x 32 tiles of TransE / RotatE)
         if constexpr (MODEL == KGE_TRANSE || MODEL == KGE_ROTATE) {
-            hipLaunchKernelGGL((score_neg_kernel<MODEL, P, 2, 2, false>), grid, dim3(256), lds, st, a, fi);
+            NEG_LAUNCH(score_neg_kernel, MODEL, P, 2, 2, false);
             hipLaunchKernelGGL((score_neg_finish_kernel<MODEL, P>), dim3((unsigned)ceil_div(a.plane, 256)), dim3(256), 0, st,
                                a.partial, a.ksplit, a.plane, a.gamma, a.out);
             KGE_CHECK_LAUNCH();
@@ -565,14 +605,14 @@ static int launch_neg_mp(const NegArgs &a_in, int64_t n_chunks, bool dot_valu, c
         return KGE_EINVAL;
     }
     if (tile == 3) {  // 32 positives x 64 negatives
-        if (save) hipLaunchKernelGGL((score_neg_kernel<MODEL, P, 2, 4, true>), grid, dim3(256), lds, st, a, fi);
-        else hipLaunchKernelGGL((score_neg_kernel<MODEL, P, 2, 4, false>), grid, dim3(256), lds, st, a, fi);
+        if (save) NEG_LAUNCH_VEC(score_neg_kernel, MODEL, P, 2, 4, true);
+        else NEG_LAUNCH_VEC(score_neg_kernel, MODEL, P, 2, 4, false);
     } else if (tile == 4) {
-        if (save) hipLaunchKernelGGL((score_neg_kernel<MODEL, P, 4, 4, true>), grid, dim3(256), lds, st, a, fi);
-        else hipLaunchKernelGGL((score_neg_kernel<MODEL, P, 4, 4, false>), grid, dim3(256), lds, st, a, fi);
+        if (save) NEG_LAUNCH_VEC(score_neg_kernel, MODEL, P, 4, 4, true);
+        else NEG_LAUNCH_VEC(score_neg_kernel, MODEL, P, 4, 4, false);
     } else {
-        if (save) hipLaunchKernelGGL((score_neg_kernel<MODEL, P, 2, 2, true>), grid, dim3(256), lds, st, a, fi);
-        else hipLaunchKernelGGL((score_neg_kernel<MODEL, P, 2, 2, false>), grid, dim3(256), lds, st, a, fi);
+        if (save) NEG_LAUNCH(score_neg_kernel, MODEL, P, 2, 2, true);
+        else NEG_LAUNCH(score_neg_kernel, MODEL, P, 2, 2, false);
     }
     KGE_CHECK_LAUNCH();
     return KGE_OK;
