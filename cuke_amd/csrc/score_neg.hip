@@ -109,8 +109,8 @@ __global__ __launch_bounds__(256, KGE_TILE_OCC) void score_neg_kernel(NegArgs a,
     const int bt0 = tile_y * TB, kt0 = tile_x * TN;
     const int d = a.d, half = d >> 1;
     const int klen = MODEL == KGE_ROTATE ? half : d;
-    constexpr bool vec = VEC4;  // 128-bit row loads: a compile-time choice (as a run-time one the two forms
-                                // of the raw loads are merged into the scalar one)
+    // (VEC4, 128-bit row loads, is a compile-time choice: as a run-time one the compiler merges the two
+    // forms of the raw loads into the scalar one)
 
     // rows this thread stages
     const float *ph[SB], *pr[SB], *pw[SB], *pq[SB];
@@ -402,8 +402,8 @@ __global__ __launch_bounds__(256, KGE_TILE_OCC) void score_neg_mfma_kernel(NegAr
     if (!xcd_tile(blockIdx.x - fi.blocks, (a.N + TN - 1) / TN, (a.C + TB - 1) / TB, a.n_chunks, c, tile_y, tile_x)) return;
     const int bt0 = tile_y * TB, kt0 = tile_x * TN;
     const int d = a.d, half = d >> 1;
-    constexpr bool vec = VEC4;  // 128-bit row loads: a compile-time choice (as a run-time one the two forms
-                                // of the raw loads are merged into the scalar one)
+    // (VEC4, 128-bit row loads, is a compile-time choice: as a run-time one the compiler merges the two
+    // forms of the raw loads into the scalar one)
 
     const float *ph[SB], *pr[SB];
     bool okb[SB];
