@@ -55,8 +55,14 @@ __device__ __forceinline__ float4 add4(float4 p, float4 q)
     return make_float4(p.x + q.x, p.y + q.y, p.z + q.z, p.w + q.w);
 }
 
-// sign(u) in two VALU ops: u * 2^100 clamped to [-1, 1] (exact 0 stays 0; |u| < 2^-100
-// would give a fraction, far below any fp32 residual that is not exactly zero).
+// sign(u) as a clamp: u * 2^100 clamped to [-1, 1] (exact 0 stays 0; |u| < 2^-100 would give a
+// fraction, far below any fp32 residual that is not exactly zero).  The multiply is paid once per
+// staged row element instead of once per pair element: scaling by a power of two commutes with
+// every fp32 rounding (no overflow: table values times 2^100 stay far below 2^127), so a residual
+// formed from rows that carry the factor 2^100 is exactly 2^100 times the residual of the plain
+// rows, and its sign is one clamp away.  The L1 tile kernels of TransE / TransH stage their rows
+// scaled; sums of |U| and of sign(U) * W are scaled back once per pair, and coefficients that
+// multiply a scaled row carry 2^-100.
 // Measured alternatives that did not pay (TransH, L1, 16384 x 1024 pairs x 400): clamping
 // u * copysign(2^100, g) to [-|g|, |g|] to get g * sign(u) directly (forward 0.92 -> 1.10 ms, gradient
 // tiles 1.74 -> 1.86 ms: v_med3_f32 and v_bfi_b32 issue at two thirds of the rate of add / mul / fmac);
@@ -64,17 +70,6 @@ __device__ __forceinline__ float4 add4(float4 p, float4 q)
 // per step (one instruction fewer per element, same forward time, gradient tiles 1.74 -> 1.80 ms: a
 // v_fma_f32 with a scalar-register operand issues at 60 % of the vector-operand rate, and with the
 // factor in a vector register the per-pair bookkeeping ate the gain).
-__device__ __forceinline__ float fast_sgn(float u)
-{
-    return __builtin_amdgcn_fmed3f(u * 0x1p100f, -1.0f, 1.0f);
-}
-
-// The multiply of fast_sgn() can be paid once per staged row element instead of once per pair
-// element: scaling by a power of two commutes with every fp32 rounding (no overflow: table values
-// times 2^100 stay far below 2^127), so a residual formed from rows that carry the factor 2^100 is
-// exactly 2^100 times the residual of the plain rows, and its sign is one clamp away.  The L1 tile
-// kernels of TransE / TransH stage their rows scaled; sums of |U| and of sign(U) * W are scaled
-// back once per pair, and coefficients that multiply a scaled row carry 2^-100.
 constexpr float kSgnScale = 0x1p100f, kSgnUnscale = 0x1p-100f;
 __device__ __forceinline__ float sgn_of_scaled(float U) { return __builtin_amdgcn_fmed3f(U, -1.0f, 1.0f); }
 __device__ __forceinline__ float4 scale4(float4 v, float s) { return make_float4(v.x * s, v.y * s, v.z * s, v.w * s); }
