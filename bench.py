@@ -42,24 +42,54 @@ ALL_WORKLOADS = ["cfg5_transh", "cfg1_transe", "cfg2_distmult", "cfg2_complex", 
 BOUND = {"cfg1_transe": "hbm", "cfg2_distmult": "fp32", "cfg2_complex": "fp32", "cfg3_transr": "hbm",
          "cfg4_rotate": "fp32", "cfg5_transh": "fp32", "ref_transr_8192x512": "hbm"}
 
-# HBM bytes per launch of a workload's dominant kernel, from rocprofv3 --pmc FETCH_SIZE and --pmc
-# WRITE_SIZE runs of this script (KiB per dispatch), each scaled by what the same counter reads
-# for the 256 MiB copy kernel of --calibrate-copy.  The summaries the numbers come from are
-# profiles/score_path_kernels_<workload>.txt; a pair that has not been measured reports null.
-MEASURED_TRAFFIC_BYTES = {
-    ('cfg5_transh', 'bwd_tile_kernel'): 1249672344,
-    ('cfg5_transh', 'score_neg_kernel'): 321899447,
-    ('cfg1_transe', 'score_pos_kernel'): 1684915,
-    ('cfg2_distmult', 'bwd_tile_kernel'): 22893024,
-    ('cfg2_distmult', 'score_neg_kernel'): 14036989,
-    ('cfg2_complex', 'bwd_tile_kernel'): 22895280,
-    ('cfg2_complex', 'score_neg_kernel'): 14062239,
-    ('cfg3_transr', 'transr_plan_kernel + transr_gemm_kernel<fwd>'): 165401787,
-    ('cfg3_transr', 'transr_gemm_kernel<dX>'): 169478021,
-    ('cfg3_transr', 'transr_dm_kernel'): 182971548,
-    ('cfg4_rotate', 'bwd_tile_kernel'): 20621914,
-    ('cfg4_rotate', 'score_neg_kernel'): 20619347,
+# Kernels of the profile summaries (profiles/score_path_kernels_<workload>.txt) behind a timeline label.
+PROFILE_KERNELS = {
+    "score_pos_kernel": ["score_pos_kernel"],
+    "score_neg_kernel": ["score_neg_kernel", "score_neg_mfma_kernel", "score_neg_finish_kernel"],
+    "bwd_tile_kernel": ["bwd_tile_kernel"],
+    "bwd_pos_kernel": ["bwd_pos_kernel"],
+    "seg_reduce_l1": ["seg_reduce_l1"],
+    "seg_reduce_l2": ["seg_reduce_l2"],
+    "transr_plan_kernel + transr_gemm_kernel<fwd>": ["transr_plan_kernel", "transr_gemm_kernel<0>"],
+    "transr_gemm_kernel<dX>": ["transr_gemm_kernel<2>"],
+    "transr_dm_kernel": ["transr_dm_kernel"],
+    "transr_dx_dm_kernel": ["transr_dx_dm_kernel"],
 }
+
+
+def measured_traffic(workload, label, matrix_core_tiles=False):
+    """HBM bytes per launch of the kernel(s) behind a timeline label, read from the committed profile
+    summary of the workload: rocprofv3 --pmc FETCH_SIZE and --pmc WRITE_SIZE runs of this script (KiB
+    per dispatch), each scaled by what the same counter reads for the 256 MiB copy kernel of
+    --calibrate-copy (the file states the factors).  Returns (bytes or None, the profile's kernel
+    names) so that the line shows which compiled kernels the figure belongs to.  matrix_core_tiles: the
+    workload's tile kernels are the matrix-core forms (the profile of such a workload also holds the
+    vector-ALU forms that the run times beside them)."""
+    import re
+    path = os.path.join(ROOT, "profiles", f"score_path_kernels_{workload}.txt")
+    want = PROFILE_KERNELS.get(label)
+    if not want or not os.path.exists(path):
+        return None, []
+    rows, in_table = {}, False
+    for line in open(path):
+        if line.startswith("## HBM traffic per dispatch"):
+            in_table = True
+            continue
+        if in_table and line.startswith("## "):
+            break
+        m = re.match(r"^(kge::.*?)\s+([\d.]+)\s+([\d.]+)\s+([\d.]+)\s+([\d.]+)\s*$", line) if in_table else None
+        if m:
+            rows[m.group(1)] = (float(m.group(4)) + float(m.group(5))) * 1e6
+    total, names = 0.0, []
+    for key in want:
+        for name, by in rows.items():
+            base = name.replace("kge::", "")
+            if base == key or base.startswith(key + "<") or (key.endswith(">") and base.replace(" ", "") == key.replace(" ", "")):
+                if matrix_core_tiles and ((key == "score_neg_kernel") or (key == "bwd_tile_kernel" and not base.endswith("true>"))):
+                    continue  # the vector-ALU form of a tile kernel
+                total += by
+                names.append(name)
+    return (int(total) if names else None), names
 
 
 # ---- algorithmic bytes and flops ---------------------------------------------------------------
@@ -80,7 +110,8 @@ def algorithmic_bytes(w, u_ent, u_rel):
     fwd = rows + idx + scores
     bwd = scores + rows + idx + 4 * (u_ent * d + u_rel * (rd + aux_row)) + 8 * (u_ent + u_rel)
     if w.model in ("TransR", "RESCAL"):
-        bwd += 4 * u_rel * d * d
+        # one gradient per distinct relation: dense d x d, or the 2 d floats per triple of a group left factored
+        bwd += 4 * (w.dense_rel * d * d + 2 * w.factored_rows * d) if hasattr(w, "dense_rel") else 4 * u_rel * d * d
     return fwd, bwd
 
 
@@ -140,10 +171,14 @@ def kernel_model(w, label, u_ent, u_rel):
     if label.startswith("transr_plan_kernel") or label == "transr_gemm_kernel<dX>":
         by = 4 * (u_rel * d * d + 3 * B * d + u_rel * d) + 8 * 3 * B
         return by, 2 * B * d * d, "mfma"
+    # dM: the x rows (two entity rows for TransR) and the residual rows in, one gradient per distinct relation out
+    # (dense d x d, or 2 d floats per triple for the groups left factored: `dense_rel` / `factored_rows` say how many)
+    dm_out = 4 * (w.dense_rel * d * d + 2 * w.factored_rows * d) if hasattr(w, "dense_rel") else 4 * u_rel * d * d
     if label == "transr_dm_kernel":
-        return 4 * (u_rel * d * d + 2 * B * d), 2 * B * d * d, "mfma"
-    if label == "transr_prep_kernel":
-        return 4 * 5 * B * d, 3 * B * d, "valu"
+        return dm_out + 4 * 3 * B * d, 2 * B * d * d, "mfma"
+    if label == "transr_dx_dm_kernel":
+        by = 4 * (u_rel * d * d + 3 * B * d) + 8 * 3 * B + dm_out + 4 * 3 * B * d
+        return by, 4 * B * d * d, "mfma"
     return 0, 0, "valu"
 
 
@@ -289,6 +324,15 @@ def spot_check(w, model, step, ix, n_pairs=4096, n_pos=512, n_rows=64, n_rel_row
         return checked, flips
 
     ent_rows_dev, rel_rows_dev, aux_rows_dev = g.ent_rows, g.rel_rows, g.aux_rows
+    seg = g.rel_seg_offsets.cpu().numpy() if g.factor_max else None
+
+    def aux_row_dev(u):
+        """Row u of the auxiliary-table gradients; a factored relation group multiplied out on the host."""
+        if seg is not None and seg[u + 1] - seg[u] <= g.factor_max:
+            x = g.aux_x[seg[u]:seg[u + 1]].cpu().numpy().astype(np.float64)
+            q = g.aux_q[seg[u]:seg[u + 1]].cpu().numpy().astype(np.float64)
+            return (x.T @ q).reshape(-1)
+        return aux_rows_dev[u].cpu().numpy()
 
     def oracle_rows(fh, fr, ft, fg):
         E, R, A, me, mr = gathered(np.concatenate([fh, ft]), fr)
@@ -343,7 +387,7 @@ def spot_check(w, model, step, ix, n_pairs=4096, n_pos=512, n_rows=64, n_rel_row
     if aux_rows_dev is not None:
         done_r.clear()
         n_a, f_a = check_rows("relation (aux table)", rpick[: n_rel_rows],
-                              lambda e: aux_rows_dev[rpos_of[int(e)]].cpu().numpy(), lambda e: rel_ref(e, True))
+                              lambda e: aux_row_dev(rpos_of[int(e)]), lambda e: rel_ref(e, True))
     report.update({"entity_rows_checked": len(done), "gradient_elements_checked": int(n_e + n_r + n_a),
                    "l1_sign_flips": int(f_e + f_r + f_a)})
     return report
@@ -426,7 +470,23 @@ def make_named_workload(name, seed):
     return synth.make_workload(name, seed=seed, tables=False)
 
 
-def run_workload(name, args, torch):
+def same_bits(torch, step, ref):
+    """The outputs of the step enqueued last against clones taken from another issue of the same batch."""
+    g = step.sparse_grads()
+    cur = [step.pos, step.neg, g.ent_ids, g.ent_rows, g.rel_ids, g.rel_rows]
+    if g.factor_max:
+        seg = g.rel_seg_offsets
+        dense = (seg[1:] - seg[:-1]) > g.factor_max
+        rows = torch.repeat_interleave(~dense, (seg[1:] - seg[:-1]).long())
+        cur += [g.aux_rows[dense], g.aux_x[: rows.numel()][rows], g.aux_q[: rows.numel()][rows]]
+    else:
+        cur.append(g.aux_rows)
+    if ref is None:
+        return [x.clone() if x is not None else None for x in cur]
+    return all((a is None and b is None) or torch.equal(a, b) for a, b in zip(cur, ref))
+
+
+def run_workload(name, args, torch, factor_max=0):
     from cuke_amd.kge import KGEModel, TrainStep
     dev = torch.device("cuda:0")
     w = make_named_workload(name, args.seed)
@@ -439,7 +499,10 @@ def run_workload(name, args, torch):
     sign = 1.0 if w.model in ("DistMult", "ComplEx", "RotatE", "TransF", "RESCAL") else -1.0
     ix = ixs[0]
     step = TrainStep(model, ix["h"], ix["r"], ix["t"], ix.get("neg"), w.chunk or None, loss=w.loss,
-                     margin=w.margin, sign=sign)
+                     margin=w.margin, sign=sign, factor_max=factor_max)
+    if w.model in ("TransR", "RESCAL"):  # what the projection gradients of batch 0 cost to write (algorithmic bytes)
+        cnt = np.unique(w.arrays["r"], return_counts=True)[1]
+        w.dense_rel, w.factored_rows = int((cnt > factor_max).sum()), int(cnt[cnt <= factor_max].sum())
     for o in ixs[1:]:
         step.add_batch(o["h"], o["r"], o["t"], o.get("neg"))
     do_bwd = w.backward
@@ -504,7 +567,19 @@ def run_workload(name, args, torch):
             step.stage(batch=nxt)
             step.run(pipeline=True)
 
+        # the staged issue takes other launch forms than the direct one (no riding inspection, merged
+        # launches): before it is timed, its outputs for batch 0 must be the direct issue's, bit for bit
+        step.select(0)
+        step.run(do_bwd)
         torch.cuda.synchronize()
+        ref_bits = same_bits(torch, step, None)
+        step.stage(batch=0)
+        step.run(pipeline=True)
+        torch.cuda.synchronize()
+        if not same_bits(torch, step, ref_bits):
+            raise SpotCheckError(f"{w.name}: the staged issue's outputs differ from the direct issue's for batch 0")
+        check["staged_equals_direct_bits"] = True
+        del ref_bits
         step.stage(batch=state["next"])          # one batch ahead from here on
         state["next"] = (state["next"] + 1) % nb
         if nb >= 3:
@@ -558,9 +633,10 @@ def run_workload(name, args, torch):
     main_roof, other = (hbm_roof, fp32_roof) if bound == "hbm" else (fp32_roof, hbm_roof)
     step_gbs = total_b / (ms * 1e-3) / 1e9
     step_tfs = total_f / (ms * 1e-3) / 1e12
+    traffic, profile_kernels = measured_traffic(name, kname, w.model in ("DistMult", "ComplEx") and bool(w.chunk))
     roofline = {"kernel": kname, "bound": "hbm" if bound == "hbm" else "mfma" if k_unit == "mfma" else "fp32_valu",
                 "achieved": main_roof["achieved"], "peak": main_roof["peak"], "unit": main_roof["unit"],
-                "frac": main_roof["frac"], "traffic": MEASURED_TRAFFIC_BYTES.get((name, kname)),
+                "frac": main_roof["frac"], "traffic": traffic, "traffic_profile_kernels": profile_kernels,
                 "kernel_ms": k_ms, "kernel_share_of_step": k_ms / kt_sum if kt_sum else None,
                 "algorithmic_bytes_per_launch": k_bytes, "algorithmic_flops_per_launch": k_flops,
                 "other_roof": {"bound": "fp32" if bound == "hbm" else "hbm", **other},
@@ -584,7 +660,10 @@ def run_workload(name, args, torch):
                    "ms_per_step_rotating_staged": ms_staged,
                    "ms_per_step_same_batch": ms_same, "ms_per_step_by_pair_sum_unit": ms_forms,
                    "scores_per_step": scores, "positives_per_s": w.batch / (ms * 1e-3),
-                   "unique_entity_rows": u_ent, "unique_relation_rows": u_rel},
+                   "unique_entity_rows": u_ent, "unique_relation_rows": u_rel,
+                   "projection_gradients": (None if w.model not in ("TransR", "RESCAL") else
+                                            {"factor_max": factor_max, "dense_groups": w.dense_rel,
+                                             "factored_rows": w.factored_rows})},
         "kernels_ms": [[n_, round(m_, 6)] for n_, m_ in kt],
         "roofline": roofline,
         **check,
@@ -684,6 +763,8 @@ def main():
                     help="do not also time the staged issue (next batch inspected on a side stream)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline legs")
     ap.add_argument("--no-check", action="store_true", help="skip the parity spot check (profiling runs)")
+    ap.add_argument("--dense-only", action="store_true",
+                    help="TransR: time only the step that writes every projection gradient dense (profiling runs)")
     ap.add_argument("--cpu-seconds", type=float, default=4.0, help="one-thread CPU work per workload")
     ap.add_argument("--seed", type=int, default=0)
     ap.add_argument("--calibrate-copy", action="store_true",
@@ -717,19 +798,52 @@ def main():
     for n in names:
         t0 = time.perf_counter()
         try:
-            res = run_workload(n, args, torch)
+            if n in ("cfg3_transr", "ref_transr_8192x512") and not args.dense_only:
+                # The projection gradients of relation groups of at most four triples (most relations of a
+                # long-tailed batch) are left factored, the form the optimizer entry points consume; the same
+                # step with every gradient written dense is timed in the same run and reported beside it.
+                res = run_workload(n, args, torch, factor_max=4)
+                saved_no_cpu, args.no_cpu = args.no_cpu, True
+                dense = run_workload(n, args, torch, factor_max=0)
+                args.no_cpu = saved_no_cpu
+                res["config"]["dense_projection_gradients"] = {
+                    k: dense[k] for k in ("ms_per_step", "value", "kernels_ms", "roofline")}
+                res["config"]["dense_projection_gradients"]["issue"] = dense["config"]["issue"]
+            else:
+                res = run_workload(n, args, torch)
         except SpotCheckError as e:
             print(f"bench.py: parity spot check failed, nothing is reported: {e}", file=sys.stderr)
             sys.exit(1)
         res["bench_seconds"] = round(time.perf_counter() - t0, 1)
         results.append(res)
+        dn = res["config"].get("dense_projection_gradients")
         print(f"[bench] {n}: {res['ms_per_step']:.4f} ms/step, {res['value']:.3e} scores/s, dominant "
-              f"{res['roofline']['kernel']} {res['roofline']['frac']:.3f} of {res['roofline']['bound']}",
+              f"{res['roofline']['kernel']} {res['roofline']['frac']:.3f} of {res['roofline']['bound']}, step "
+              f"{res['roofline']['step']['frac']:.3f} of {res['roofline']['step']['bound']}"
+              + (f"; every projection gradient dense: {dn['ms_per_step']:.4f} ms/step, step "
+                 f"{dn['roofline']['step']['frac']:.3f}" if dn else ""),
               file=sys.stderr, flush=True)
     out = results[0]
     out["machine"] = machine
     if len(results) > 1:
         out["per_workload"] = results[1:]
+    # one compact row per workload inside `roofline` (the full records are in per_workload)
+    table = []
+    for r in results:
+        rf, cb = r["roofline"], r.get("cpu_baseline") or {}
+        row = {"workload": r["config"]["workload"], "ms_per_step": round(r["ms_per_step"], 5), "issue": r["config"]["issue"],
+               "scores_per_s": float(f"{r['value']:.4g}"), "kernel": rf["kernel"], "kernel_ms": round(rf["kernel_ms"], 5),
+               "bound": rf["bound"], "frac": round(rf["frac"], 4), "step_bound": rf["step"]["bound"],
+               "step_frac": round(rf["step"]["frac"], 4), "traffic": rf["traffic"],
+               "cpu_1_thread": float(f"{cb['value']:.4g}") if cb else None,
+               "cpu_all_cores": float(f"{cb['all_cores']['value']:.4g}") if cb else None,
+               "cpu_cores": cb["all_cores"]["cores"] if cb else None}
+        dn = r["config"].get("dense_projection_gradients")
+        if dn:
+            row["dense_ms_per_step"] = round(dn["ms_per_step"], 5)
+            row["dense_step_frac"] = round(dn["roofline"]["step"]["frac"], 4)
+        table.append(row)
+    out["roofline"]["per_workload"] = table
     print(json.dumps(out))
 
 

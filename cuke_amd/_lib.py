@@ -40,7 +40,7 @@ class InspectJob(C.Structure):
 
 class Timeline(C.Structure):
     _fields_ = [("begin", C.c_void_p), ("events", C.POINTER(C.c_void_p)), ("labels", C.POINTER(C.c_char_p)),
-                ("capacity", C.c_int32), ("count", C.c_int32)]
+                ("capacity", C.c_int32), ("count", C.c_int32), ("dropped", C.c_int32), ("reserved", C.c_int32)]
 
 
 PAIR_SUMS_VALU = 1  # kge_tables.flags
@@ -62,7 +62,8 @@ class Saved(C.Structure):
 
 
 class Grads(C.Structure):
-    _fields_ = [("ent_rows", C.c_void_p), ("rel_rows", C.c_void_p), ("aux_rows", C.c_void_p)]
+    _fields_ = [("ent_rows", C.c_void_p), ("rel_rows", C.c_void_p), ("aux_rows", C.c_void_p),
+                ("aux_x", C.c_void_p), ("aux_q", C.c_void_p), ("aux_factor_max", C.c_int32), ("reserved", C.c_int32)]
 
 
 EXPORTS = {
@@ -101,6 +102,10 @@ EXPORTS = {
                                  C.c_void_p]),
     "kge_sparse_adagrad": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int64, C.c_void_p, C.c_void_p, C.c_int64,
                                      C.c_void_p, C.c_float, C.c_float, C.c_void_p]),
+    "kge_sparse_sgd_factored": (C.c_int, [C.c_void_p, C.c_int64, C.POINTER(Inspection), C.POINTER(Grads), C.c_float,
+                                          C.c_void_p]),
+    "kge_sparse_adagrad_factored": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int64, C.POINTER(Inspection), C.POINTER(Grads),
+                                              C.c_float, C.c_float, C.c_void_p]),
     "kge_sample_negatives": (C.c_int, [C.c_void_p, C.c_int64, C.c_int64, C.c_uint64, C.c_uint64, C.c_void_p]),
     "kge_check_indices": (C.c_int, [C.c_void_p, C.c_int64, C.c_int64, C.c_void_p, C.c_void_p]),
 }
@@ -108,7 +113,7 @@ EXPORTS = {
 _lib = None
 
 
-ABI_VERSION = 5  # layout of the ctypes structures above; must match kge_abi_version()
+ABI_VERSION = 6  # layout of the ctypes structures above; must match kge_abi_version()
 
 
 def lib() -> C.CDLL:

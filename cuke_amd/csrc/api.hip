@@ -106,7 +106,7 @@ const char *kge_strerror(int status)
     }
 }
 
-int kge_abi_version(void) { return 5; }
+int kge_abi_version(void) { return 6; }
 
 kge_timeline *kge_timeline_create(int32_t capacity)
 {
@@ -145,7 +145,7 @@ void kge_timeline_destroy(kge_timeline *tl)
 int kge_timeline_begin(kge_timeline *tl, void *stream)
 {
     if (!tl || !tl->begin) return KGE_EINVAL;
-    tl->count = 0;
+    tl->count = 0, tl->dropped = 0;
     return hipEventRecord(reinterpret_cast<hipEvent_t>(tl->begin), as_stream(stream)) == hipSuccess ? KGE_OK : KGE_ELAUNCH;
 }
 
@@ -161,6 +161,7 @@ int kge_timeline_mark(kge_timeline *tl, const char *label, void *stream)
 int kge_timeline_elapsed(const kge_timeline *tl, float *ms)
 {
     if (!tl || !ms || !tl->begin) return KGE_EINVAL;
+    if (tl->dropped > 0) return KGE_EWORKSPACE;  // more kernels than capacity (or a failed record): no truncated table
     hipEvent_t prev = reinterpret_cast<hipEvent_t>(tl->begin);
     for (int i = 0; i < tl->count; ++i) {
         hipEvent_t cur = reinterpret_cast<hipEvent_t>(tl->events[i]);
@@ -231,7 +232,10 @@ int kge_score_fwd(const kge_tables *tab, const kge_batch *bat, float *pos, float
     }
     if (want_neg && tab->model == KGE_TRANSR && bat->rel_insp)  // positives and shared negatives in one grouped pass
         return launch_transr_neg_fwd(tab, bat, pos, neg, residual, workspace, workspace_bytes, st);
-    // DistMult / ComplEx: the positives ride in the tile launch where nothing else does
+    // TransE, DistMult / ComplEx on the matrix-core tiles: the positives ride in the tile launch where
+    // nothing else does (score_neg_carries_positives; also with the reduction axis of small TransE
+    // batches split, where their workgroups follow tile_blocks * ksplit tile workgroups).  `pos` is then
+    // written by the negatives' launch, and its timeline entry "score_neg_kernel" includes the positives.
     const bool carry = want_neg && pos && !side_pos && !residual && !fuse && score_neg_carries_positives(tab, bat);
     if (!carry && (pos || side_pos || residual)) {
         if ((tab->model == KGE_TRANSR || tab->model == KGE_RESCAL) && bat->rel_insp)

@@ -71,8 +71,12 @@ inline bool pair_sums_valu(const kge_tables *tab) { return (tab->flags & KGE_PAI
 // One entry of the caller's timeline (kge_batch.timeline): the kernel launched last ends here.
 inline void timeline_mark(kge_timeline *tl, hipStream_t st, const char *label)
 {
-    if (!tl || !tl->events || !tl->labels || tl->count < 0 || tl->count >= tl->capacity) return;
-    if (hipEventRecord(reinterpret_cast<hipEvent_t>(tl->events[tl->count]), st) != hipSuccess) return;
+    if (!tl || !tl->events || !tl->labels) return;
+    if (tl->count < 0 || tl->count >= tl->capacity ||
+        hipEventRecord(reinterpret_cast<hipEvent_t>(tl->events[tl->count]), st) != hipSuccess) {
+        ++tl->dropped;  // kge_timeline_elapsed refuses a table with holes
+        return;
+    }
     tl->labels[tl->count++] = label;
 }
 

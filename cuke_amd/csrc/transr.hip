@@ -132,6 +132,48 @@ __global__ __launch_bounds__(1024) void transr_plan_kernel(const int32_t *num_un
     }
 }
 
+// Where the backward kernels take their operands from when no kernel has written them out.  Sorted
+// position p of the relation order names the triple b = perm[p]; its upstream row is
+//   TransR  q = c * phi(resid[b]),  c = dpos[b] and phi = sign (L1), or c = dpos[b] / pos[b] and phi = identity (L2)
+//   RESCAL  q = c * E[t[b]],        c = dpos[b]
+// and its left operand x = E[h[b]] - E[t[b]] (TransR) or E[h[b]] (RESCAL).  The dX and dM kernels form
+// both while they stage their tiles: the few scalars per row ride in the index chain the tiles walk
+// anyway, and nothing of size B x d is written to memory and read back in between.
+struct BwdSrc {
+    const float *ent, *resid, *dpos, *spos;
+    const int64_t *h, *t;
+    const int32_t *perm;
+    int norm_p, rescal;
+    float *occ_v;  // RESCAL: [B, d] occurrence rows of the tails, g * (E[h] Proj[r]); written by the dX kernel
+};
+
+struct RowMeta {
+    int b;         // triple
+    float coef;    // c above
+    int64_t qoff;  // offset of the row phi() is applied to, in qbase() floats
+    int64_t xh, xt;
+};
+
+__device__ __forceinline__ const float *bwd_qbase(const BwdSrc &s) { return s.rescal ? s.ent : s.resid; }
+
+__device__ __forceinline__ RowMeta bwd_row_meta(const BwdSrc &s, int p, int d)
+{
+    RowMeta m;
+    m.b = s.perm[p];
+    const float g = s.dpos ? s.dpos[m.b] : 0.0f;
+    m.coef = g;
+    if (!s.rescal && s.norm_p == 2) {
+        const float sc = s.spos[m.b];
+        m.coef = sc > 0.0f ? g / sc : 0.0f;
+    }
+    m.xh = s.h[m.b], m.xt = s.t[m.b];
+    m.qoff = s.rescal ? m.xt * d : (int64_t)m.b * d;
+    return m;
+}
+
+__device__ __forceinline__ float4 sgn4(float4 v) { return make_float4(sgn(v.x), sgn(v.y), sgn(v.z), sgn(v.w)); }
+__device__ __forceinline__ float4 scaled4(float c, float4 v) { return make_float4(c * v.x, c * v.y, c * v.z, c * v.w); }
+
 // ---- grouped GEMM tile: Y[32 x d] = X[32 x d] * M (or * M^T) -----------------------------
 struct GemmArgs {
     const float *ent, *rel, *proj;
@@ -139,7 +181,7 @@ struct GemmArgs {
     const int32_t *perm, *seg_offsets, *num_unique;
     const int64_t *unique_ids;
     TilePlan plan;
-    const float *xs;  // TRANSPOSED pass: left operand rows in sorted order [B, d]
+    const float *xs;  // TRANSPOSED pass: left operand rows in sorted order [B, d]; null: formed from `src`
     const float *rs;  // list pass (MODE 3): factor of the relation row per list row (+1, -1 or 0)
     float *pos;       // forward: [B] scores (nullable)
     float *resid;     // forward: [B, d] rows y (nullable)
@@ -147,6 +189,7 @@ struct GemmArgs {
     int d, norm_p;
     int thin_groups;       // upper bound of the number of relation groups = trailing thin workgroups
     int max_tiles;         // leading workgroups: planned tiles
+    BwdSrc src;            // TRANSPOSED pass without xs
 };
 
 // ---- thin path: the last <= kThin triples of a relation group ---------------------------------
@@ -328,7 +371,23 @@ __device__ __forceinline__ void transr_thin_dx_body(const GemmArgs &a, float *sY
     const int d = a.d, nq4 = d >> 2, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int li = lane & 15, sub = lane >> 4;
     __shared__ int s_b[kThin];
-    if (tid < kThin) s_b[tid] = tid < rows ? (a.perm ? a.perm[tt.p0 + tid] : tt.p0 + tid) : 0;  // no perm: rows stay in sorted order
+    const bool derived = a.xs == nullptr;  // the upstream rows are formed here (BwdSrc)
+    // (the same addresses in every lane: the compiler turns these into scalar loads)
+    const float *qrow[4];
+    float qcoef[4], qg[4];
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+        const int p = tt.p0 + (r < rows ? r : 0);
+        if (derived) {
+            const RowMeta m = bwd_row_meta(a.src, p, d);
+            qrow[r] = bwd_qbase(a.src) + m.qoff, qcoef[r] = m.coef, qg[r] = a.src.dpos ? a.src.dpos[m.b] : 0.0f;
+            if (tid == r) s_b[r] = m.b;
+        } else {
+            qrow[r] = a.xs + (int64_t)p * d, qcoef[r] = 1.0f, qg[r] = 0.0f;
+            if (tid == r) s_b[r] = r < rows ? (a.perm ? a.perm[p] : p) : 0;  // no perm: rows stay in sorted order
+        }
+    }
+    const bool sign_rows = derived && !a.src.rescal && a.src.norm_p == 1;
     const int64_t rid = a.unique_ids[g];
     const float4 *M4 = reinterpret_cast<const float4 *>(a.proj + rid * (int64_t)d * d);
     const int jfirst = 4 * wave + sub;  // row of (step i, wave, sub): j = 16 i + 4 wave + sub
@@ -340,10 +399,11 @@ __device__ __forceinline__ void transr_thin_dx_body(const GemmArgs &a, float *sY
             const int c = c0 + li + 16 * s;
             qc[s] = c < nq4 ? c : 0;
 #pragma unroll
-            for (int r = 0; r < 4; ++r)  // zero beyond the row and beyond `rows`: clamped loads then add nothing
-                q[s][r] = (c < nq4 && r < rows)
-                              ? *reinterpret_cast<const float4 *>(a.xs + (int64_t)(tt.p0 + r) * d + 4 * c)
-                              : make_float4(0.f, 0.f, 0.f, 0.f);
+            for (int r = 0; r < 4; ++r) {  // zero beyond the row and beyond `rows`: clamped loads then add nothing
+                q[s][r] = (c < nq4 && r < rows) ? *reinterpret_cast<const float4 *>(qrow[r] + 4 * c)
+                                                : make_float4(0.f, 0.f, 0.f, 0.f);
+                if (derived) q[s][r] = scaled4(qcoef[r], sign_rows ? sgn4(q[s][r]) : q[s][r]);
+            }
         }
         auto loadrow = [&](int j, float4 *dst) {
             const int64_t base = (int64_t)(j < d ? j : d - 1) * nq4;
@@ -386,6 +446,10 @@ __device__ __forceinline__ void transr_thin_dx_body(const GemmArgs &a, float *sY
         const int64_t o = (int64_t)s_b[r] * d + 4 * c;
         *reinterpret_cast<float4 *>(a.occ_h + o) = y;
         if (a.occ_t) *reinterpret_cast<float4 *>(a.occ_t + o) = make_float4(-y.x, -y.y, -y.z, -y.w);
+        if (derived && a.src.occ_v) {  // RESCAL: the tail's occurrence row g * (E[h] Proj[r])
+            const float gr = r == 0 ? qg[0] : (r == 1 ? qg[1] : (r == 2 ? qg[2] : qg[3]));
+            *reinterpret_cast<float4 *>(a.src.occ_v + o) = scaled4(gr, *reinterpret_cast<const float4 *>(a.src.resid + o));
+        }
     }
 }
 
@@ -561,10 +625,17 @@ __device__ __forceinline__ void transr_gemm_body(const GemmArgs &a, float *lds, 
     __shared__ int s_b[kTM];
     __shared__ int64_t s_h[kTM], s_t[kTM];
     __shared__ float s_rs[MODE == 3 ? kTM : 1];
+    __shared__ float s_coef[MODE == 2 ? kTM : 1], s_g[MODE == 2 ? kTM : 1];
+    __shared__ int64_t s_qoff[MODE == 2 ? kTM : 1];
+    const bool derived = MODE == 2 && a.xs == nullptr;  // the upstream rows are formed while staging (BwdSrc)
     if (tid < kTM) {
         int b;
         if constexpr (MODE == 3) b = p0 + (tid < rows ? tid : 0);
-        else b = tid < rows ? (a.perm ? a.perm[p0 + tid] : p0 + tid) : 0;
+        else if (derived) {
+            const RowMeta m = bwd_row_meta(a.src, p0 + (tid < rows ? tid : 0), d);
+            b = m.b;
+            if constexpr (MODE == 2) s_coef[tid] = m.coef, s_qoff[tid] = m.qoff, s_g[tid] = a.src.dpos ? a.src.dpos[m.b] : 0.0f;
+        } else b = tid < rows ? (a.perm ? a.perm[p0 + tid] : p0 + tid) : 0;
         s_b[tid] = b;
         if constexpr (MODE != 2) {
             s_h[tid] = a.h[b];
@@ -586,7 +657,12 @@ __device__ __forceinline__ void transr_gemm_body(const GemmArgs &a, float *lds, 
                 v[q] = make_float4(0.f, 0.f, 0.f, 0.f), u[q] = v[q];
                 if (f < kTM * per_row && row < rows && k4 < d) {
                     if constexpr (MODE == 2) {
-                        v[q] = *reinterpret_cast<const float4 *>(a.xs + (int64_t)(p0 + row) * d + k4);
+                        if (derived) {  // uniform
+                            v[q] = *reinterpret_cast<const float4 *>(bwd_qbase(a.src) + s_qoff[row] + k4);
+                            if (a.src.occ_v) u[q] = *reinterpret_cast<const float4 *>(a.src.resid + (int64_t)s_b[row] * d + k4);
+                        } else {
+                            v[q] = *reinterpret_cast<const float4 *>(a.xs + (int64_t)(p0 + row) * d + k4);
+                        }
                     } else {
                         v[q] = *reinterpret_cast<const float4 *>(a.ent + s_h[row] * (int64_t)d + k4);
                         if constexpr (MODE == 0)
@@ -602,8 +678,16 @@ __device__ __forceinline__ void transr_gemm_body(const GemmArgs &a, float *lds, 
                 const int f = f0 + 256 * q;
                 if (f < kTM * per_row) {
                     const int row = f / per_row, k4 = (f % per_row) * 4;
-                    *reinterpret_cast<float4 *>(&sX[row * pitch + k4]) =
-                        make_float4(v[q].x - u[q].x, v[q].y - u[q].y, v[q].z - u[q].z, v[q].w - u[q].w);
+                    float4 x = make_float4(v[q].x - u[q].x, v[q].y - u[q].y, v[q].z - u[q].z, v[q].w - u[q].w);
+                    if constexpr (MODE == 2) {
+                        if (derived) {
+                            const bool l1 = !a.src.rescal && a.src.norm_p == 1;
+                            x = row < rows ? scaled4(s_coef[row], l1 ? sgn4(v[q]) : v[q]) : make_float4(0.f, 0.f, 0.f, 0.f);
+                            if (a.src.occ_v && row < rows && k4 < d)  // RESCAL: the tail's occurrence row g * (E[h] Proj[r])
+                                *reinterpret_cast<float4 *>(a.src.occ_v + (int64_t)s_b[row] * d + k4) = scaled4(s_g[row], u[q]);
+                        }
+                    }
+                    *reinterpret_cast<float4 *>(&sX[row * pitch + k4]) = x;
                 }
             }
         }
@@ -751,58 +835,11 @@ bool transr_grouped_path_ok(const kge_tables *tab, const kge_batch *bat)
 }
 
 // ---- backward kernels ----------------------------------------------------------------------
-struct PrepArgs {
-    const float *ent;
-    const int64_t *h, *t;
-    const int32_t *perm;
-    const float *dpos, *spos, *resid;
-    float *xs, *qs;  // [B, d] in sorted order
-    float *occ_t;    // RESCAL: g * v
-    int64_t B;
-    int d, norm_p, rescal;
-};
-
-// One wave per sorted position p (triple b = perm[p]):
-//   TransR: xs[p] = E[h]-E[t], qs[p] = g * d||e||/de     RESCAL: xs[p] = E[h], qs[p] = g * E[t], occ_t[b] = g * v
-__global__ __launch_bounds__(256) void transr_prep_kernel(PrepArgs a, FusedInsp fi)
-{
-    extern __shared__ __align__(16) float lds[];  // inspector workgroups only
-    if (fused_insp_block(fi, reinterpret_cast<uint32_t *>(lds))) return;
-    const int lane = threadIdx.x & 63;
-    const int64_t p = (int64_t)((int)blockIdx.x - fi.blocks) * 4 + (threadIdx.x >> 6);
-    if (p >= a.B) return;
-    const int b = a.perm[p];
-    const int d = a.d;
-    const float g = a.dpos ? a.dpos[b] : 0.0f;
-    const float *eh = a.ent + a.h[b] * (int64_t)d, *et = a.ent + a.t[b] * (int64_t)d;
-    const float *e = a.resid + (int64_t)b * d;
-    float gs = g;
-    if (!a.rescal && a.norm_p == 2) {
-        const float s = a.spos[b];
-        gs = s > 0.0f ? g / s : 0.0f;
-    }
-    for (int j = lane * 4; j < d; j += 256) {
-        const float4 vh = *reinterpret_cast<const float4 *>(eh + j), vt = *reinterpret_cast<const float4 *>(et + j);
-        const float4 ve = *reinterpret_cast<const float4 *>(e + j);
-        float4 x, q;
-        if (a.rescal) {
-            x = vh;
-            q = make_float4(g * vt.x, g * vt.y, g * vt.z, g * vt.w);
-            *reinterpret_cast<float4 *>(a.occ_t + (int64_t)b * d + j) = make_float4(g * ve.x, g * ve.y, g * ve.z, g * ve.w);
-        } else {
-            x = make_float4(vh.x - vt.x, vh.y - vt.y, vh.z - vt.z, vh.w - vt.w);
-            if (a.norm_p == 1) q = make_float4(gs * sgn(ve.x), gs * sgn(ve.y), gs * sgn(ve.z), gs * sgn(ve.w));
-            else q = make_float4(gs * ve.x, gs * ve.y, gs * ve.z, gs * ve.w);
-        }
-        *reinterpret_cast<float4 *>(a.xs + p * d + j) = x;
-        *reinterpret_cast<float4 *>(a.qs + p * d + j) = q;
-    }
-}
-
 constexpr int kDmChunk = 256;  // triples of one relation group per dM work item
+constexpr int kDmXP = 36;      // LDS pitch of a staged left-operand row (32 columns + 4: the four lane groups of an MFMA step read distinct banks)
 
 struct DmArgs {
-    const float *xs, *qs;  // sorted order [B, d]
+    const float *xs, *qs;  // operand rows in sorted order [B, d]; null: formed from `src` (BwdSrc)
     const int32_t *seg_offsets;
     TilePlan plan;   // tiles of kDmChunk positions, with split bookkeeping
     float *dm;       // [U, d, d]
@@ -810,11 +847,19 @@ struct DmArgs {
     int d;
     const int32_t *num_unique;
     int max_items;   // leading workgroups: (tile, 32-row block) items; the rest: one thin group each
+    BwdSrc src;
+    // Factored output (kge_grads.aux_x / aux_q): a group of at most factor_max (<= kThin) triples writes its
+    // operand rows x_p, q_p to fx[p], fq[p] (p = its sorted positions) instead of the dense d x d sum of
+    // their outer products.  fx null: every group dense.
+    float *fx, *fq;
+    int factor_max;
+    ZeroRider zero;  // the reduction's tickets (this is the last kernel in front of it)
 };
 
 // dM of a group of at most kThin triples: four outer products written as one contiguous stream.
 // Thread (phase, cq) keeps its column quad of the Q rows in registers and walks the rows
 // k = phase, phase + P, ... of the output, so consecutive threads write consecutive 16 bytes.
+// With factored output the rows themselves are the result (2 * rows * d floats instead of d * d).
 __device__ __forceinline__ void transr_thin_dm_body(const DmArgs &a, float *lds, int g)
 {
     if (g >= a.num_unique[0]) return;
@@ -822,20 +867,55 @@ __device__ __forceinline__ void transr_thin_dm_body(const DmArgs &a, float *lds,
     if (rows > kThin) return;
     const int d = a.d, nq4 = d >> 2, tid = threadIdx.x;
     const int P = 256 / nq4;
+    const bool derived = a.xs == nullptr;
+    // (the same addresses in every lane: scalar loads)
+    const float *xh[4], *xt[4], *qrow[4];
+    float qcoef[4];
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+        const int p = s0 + (r < rows ? r : 0);
+        if (derived) {
+            const RowMeta m = bwd_row_meta(a.src, p, d);
+            xh[r] = a.src.ent + m.xh * d, xt[r] = a.src.ent + m.xt * d;
+            qrow[r] = bwd_qbase(a.src) + m.qoff, qcoef[r] = m.coef;
+        } else {
+            xh[r] = a.xs + (int64_t)p * d, xt[r] = xh[r], qrow[r] = a.qs + (int64_t)p * d, qcoef[r] = 1.0f;
+        }
+    }
+    const bool sub_t = derived && !a.src.rescal, sign_rows = derived && !a.src.rescal && a.src.norm_p == 1;
+    const bool factored = a.fx && rows <= a.factor_max;
     float4 *sXT = reinterpret_cast<float4 *>(lds);  // [d] x[0..3][k]
     for (int f = tid; f < 4 * nq4; f += 256) {
         const int r = f / nq4, k4 = (f % nq4) * 4;
-        const float4 v = r < rows ? *reinterpret_cast<const float4 *>(a.xs + (int64_t)(s0 + r) * d + k4)
-                                  : make_float4(0.f, 0.f, 0.f, 0.f);
-        float *col = reinterpret_cast<float *>(sXT + k4) + r;
-        col[0] = v.x, col[4] = v.y, col[8] = v.z, col[12] = v.w;
+        const float *ph = r == 0 ? xh[0] : (r == 1 ? xh[1] : (r == 2 ? xh[2] : xh[3]));
+        const float *pt = r == 0 ? xt[0] : (r == 1 ? xt[1] : (r == 2 ? xt[2] : xt[3]));
+        float4 v = *reinterpret_cast<const float4 *>(ph + k4);
+        const float4 u = *reinterpret_cast<const float4 *>(pt + k4);
+        if (sub_t) v = make_float4(v.x - u.x, v.y - u.y, v.z - u.z, v.w - u.w);
+        if (r >= rows) v = make_float4(0.f, 0.f, 0.f, 0.f);
+        if (factored) {
+            if (r < rows) *reinterpret_cast<float4 *>(a.fx + (int64_t)(s0 + r) * d + k4) = v;
+        } else {
+            float *col = reinterpret_cast<float *>(sXT + k4) + r;
+            col[0] = v.x, col[4] = v.y, col[8] = v.z, col[12] = v.w;
+        }
     }
     const int cq = tid % nq4, ph = tid / nq4;
     float4 q[4];
 #pragma unroll
-    for (int r = 0; r < 4; ++r)
-        q[r] = r < rows ? *reinterpret_cast<const float4 *>(a.qs + (int64_t)(s0 + r) * d + 4 * cq)
-                        : make_float4(0.f, 0.f, 0.f, 0.f);
+    for (int r = 0; r < 4; ++r) {
+        q[r] = *reinterpret_cast<const float4 *>(qrow[r] + 4 * cq);
+        if (derived) q[r] = scaled4(qcoef[r], sign_rows ? sgn4(q[r]) : q[r]);
+        if (r >= rows) q[r] = make_float4(0.f, 0.f, 0.f, 0.f);
+    }
+    if (factored) {
+        if (ph == 0) {
+#pragma unroll
+            for (int r = 0; r < 4; ++r)
+                if (r < rows) *reinterpret_cast<float4 *>(a.fq + (int64_t)(s0 + r) * d + 4 * cq) = q[r];
+        }
+        return;
+    }
     __syncthreads();
     if (ph >= P) return;
     float4 *out = reinterpret_cast<float4 *>(a.dm + (int64_t)g * d * d);
@@ -850,35 +930,28 @@ __device__ __forceinline__ void transr_thin_dm_body(const DmArgs &a, float *lds,
     }
 }
 
-// K loop of a dM work item: acc (+)= X[p, i0 .. i0+31]^T Q[p, n0 .. n0+wcols) over the positions
-// p in [s0, s1).  As in gemm_sweep the loads of a superstep are free of branches: addresses are
-// clamped (a position past s1 re-reads s1 - 1 and its X value is selected to zero, a lane outside
-// the row / column range reads column i0 / n0 and produces values nobody stores), the issue
-// order of the prefetch is pinned, and the 16- or 32-row variant is a template parameter.
-template <bool TWO>
-__device__ __forceinline__ void dm_sweep(const float *xs, const float *qs, int d, int s0, int s1, int nq, int i0,
-                                         int n0, int wcols, int li, int kk, floatx4 (&acc_lo)[4], floatx4 (&acc_hi)[4])
+// K loop of a dM work item: acc (+)= X[p, i0 .. i0+31]^T Q[p, n0 .. n0+wcols) over the item's n
+// positions.  The left operand comes from LDS (sX: [16 * nq][kDmXP], staged by transr_dm_body with
+// zeros beyond n and beyond the row width), the right operand straight from memory through the row
+// offsets sOff (one 128-bit load per position and lane).  As in gemm_sweep the loads of a superstep
+// are free of branches: a position past the end re-reads the last one (its X is zero), a lane
+// outside the column range reads column n0 and produces values nobody stores, and the issue order of
+// the prefetch is pinned.  SIGN: the right operand is sign(row) (TransR, L1: the coefficient sits in X).
+template <bool TWO, bool SIGN>
+__device__ __forceinline__ void dm_sweep(const float *qbase, const float *sX, const int64_t *sOff, int n, int nq, int n0,
+                                         int wcols, int li, int kk, floatx4 (&acc_lo)[4], floatx4 (&acc_hi)[4])
 {
-    struct Stage {
-        float al[4], ah[4];
-        float4 bv[4];
-    };
-    const bool ilo = i0 + li < d, ihi = i0 + 16 + li < d;
-    const float *xlo = xs + i0 + (ilo ? li : 0), *xhi = xs + i0 + (ihi ? 16 + li : 0);
-    const float *qb = qs + n0 + (4 * li < wcols ? 4 * li : 0);
-    auto load_stage = [&](int q, Stage &st) {
+    const float *qb = qbase + n0 + (4 * li < wcols ? 4 * li : 0);
+    auto load_stage = [&](int q, float4 (&bv)[4]) {
 #pragma unroll
         for (int s = 0; s < 4; ++s) {
-            const int p = s0 + 16 * q + 4 * kk + s;
-            const int64_t row = (int64_t)(p < s1 ? p : s1 - 1) * d;
-            st.al[s] = xlo[row];
-            if constexpr (TWO) st.ah[s] = xhi[row];
-            st.bv[s] = *reinterpret_cast<const float4 *>(qb + row);
+            const int i = 16 * q + 4 * kk + s;
+            bv[s] = *reinterpret_cast<const float4 *>(qb + sOff[i < n ? i : n - 1]);
         }
     };
     // Most work items are short (a group of 5..16 triples is a single superstep), so unlike in
     // gemm_sweep the prefetch is skipped past the end: a uniform branch per superstep, none per load.
-    Stage ring[kDmRing];
+    float4 ring[kDmRing][4];
 #pragma unroll
     for (int u = 0; u + 1 < kDmRing; ++u)
         if (u < nq) load_stage(u, ring[u]);
@@ -889,13 +962,13 @@ __device__ __forceinline__ void dm_sweep(const float *xs, const float *qs, int d
             if (qq >= nq) break;
             if (qq + kDmRing - 1 < nq) load_stage(qq + kDmRing - 1, ring[(u + kDmRing - 1) % kDmRing]);
             __builtin_amdgcn_sched_barrier(0);
-            const Stage &cur = ring[u];
 #pragma unroll
             for (int s = 0; s < 4; ++s) {
-                const bool live = s0 + 16 * qq + 4 * kk + s < s1;
-                const float al = (live && ilo) ? cur.al[s] : 0.0f;
-                const float ah = (TWO && live && ihi) ? cur.ah[s] : 0.0f;
-                const float b4[4] = {cur.bv[s].x, cur.bv[s].y, cur.bv[s].z, cur.bv[s].w};
+                const int i = 16 * qq + 4 * kk + s;
+                const float al = sX[i * kDmXP + li];
+                const float ah = TWO ? sX[i * kDmXP + 16 + li] : 0.0f;
+                const float4 bq = SIGN ? sgn4(ring[u][s]) : ring[u][s];
+                const float b4[4] = {bq.x, bq.y, bq.z, bq.w};
 #pragma unroll
                 for (int e = 0; e < 4; ++e) {
                     acc_lo[e] = __builtin_amdgcn_mfma_f32_16x16x4f32(al, b4[e], acc_lo[e], 0, 0, 0);
@@ -906,10 +979,11 @@ __device__ __forceinline__ void dm_sweep(const float *xs, const float *qs, int d
     }
 }
 
-// dM[g][i][j] = sum_{p in group g} xs[p][i] * qs[p][j].  A work item is (chunk of <= 256 triples
-// of one group, 32 rows i); the four waves split the columns j; K runs over the chunk's triples,
-// operands prefetched four supersteps ahead.  Groups longer than one chunk write per-chunk
-// partial matrices that are added up beside the segmented reduction (keeps the longest K loop at 16 supersteps).
+// dM[g][i][j] = sum_{p in group g} x[p][i] * q[p][j].  A work item is (chunk of <= 256 triples
+// of one group, 32 rows i); it stages its 32 columns of the chunk's x rows in LDS (coefficients
+// folded in), the four waves split the columns j and K runs over the chunk's triples.  Groups longer
+// than one chunk write per-chunk partial matrices that are added up beside the segmented reduction
+// (keeps the longest K loop at 16 supersteps).
 __device__ __forceinline__ void transr_dm_body(const DmArgs &a, float *lds, int bid)
 {
     if (bid >= a.max_items) {
@@ -931,7 +1005,50 @@ __device__ __forceinline__ void transr_dm_body(const DmArgs &a, float *lds, int 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int li = lane & 15, kk = lane >> 4;
     const bool two_blocks = i0 + 16 < d;
-    const int nq = (s1 - s0 + 15) / 16;
+    const int n = s1 - s0, nq = (n + 15) / 16;
+    const bool derived = a.xs == nullptr;
+
+    // stage: thread i owns position s0 + i: the row's offset for the right operand, and the 32 columns
+    // i0 .. i0 + 31 of its left operand (eight 128-bit loads, sixteen for TransR's two entity rows, all in
+    // flight together), times the row's coefficient
+    float *sX = lds;                                                      // [kDmChunk][kDmXP]
+    int64_t *sOff = reinterpret_cast<int64_t *>(lds + kDmChunk * kDmXP);  // [kDmChunk]
+    if (tid < 16 * nq) {
+        const int p = s0 + (tid < n ? tid : n - 1);
+        const float *ph, *pt;
+        float coef = 1.0f;
+        bool sub_t = false;
+        if (derived) {
+            const RowMeta m = bwd_row_meta(a.src, p, d);
+            ph = a.src.ent + m.xh * d, pt = a.src.ent + m.xt * d;
+            sOff[tid] = m.qoff, coef = m.coef, sub_t = !a.src.rescal;
+        } else {
+            ph = a.xs + (int64_t)p * d, pt = ph;
+            sOff[tid] = (int64_t)p * d;
+        }
+        float4 v[8], u[8];
+#pragma unroll
+        for (int c = 0; c < 8; ++c) {
+            const int col = i0 + 4 * c < d ? i0 + 4 * c : 0;  // clamped: unconditional loads, masked below
+            v[c] = *reinterpret_cast<const float4 *>(ph + col);
+        }
+        if (sub_t) {  // uniform
+#pragma unroll
+            for (int c = 0; c < 8; ++c) u[c] = *reinterpret_cast<const float4 *>(pt + (i0 + 4 * c < d ? i0 + 4 * c : 0));
+        } else {
+#pragma unroll
+            for (int c = 0; c < 8; ++c) u[c] = make_float4(0.f, 0.f, 0.f, 0.f);
+        }
+#pragma unroll
+        for (int c = 0; c < 8; ++c) {
+            float4 x = make_float4(v[c].x - u[c].x, v[c].y - u[c].y, v[c].z - u[c].z, v[c].w - u[c].w);
+            x = (tid < n && i0 + 4 * c < d) ? scaled4(coef, x) : make_float4(0.f, 0.f, 0.f, 0.f);
+            *reinterpret_cast<float4 *>(&sX[tid * kDmXP + 4 * c]) = x;
+        }
+    }
+    __syncthreads();
+    const float *qbase = derived ? bwd_qbase(a.src) : a.qs;
+    const bool sign_rows = derived && !a.src.rescal && a.src.norm_p == 1;
 
     for (int c0 = 0; c0 < d; c0 += 256) {
         const int span = d - c0 < 256 ? d - c0 : 256;
@@ -944,8 +1061,13 @@ __device__ __forceinline__ void transr_dm_body(const DmArgs &a, float *lds, int 
 #pragma unroll
         for (int e = 0; e < 4; ++e) acc_lo[e] = floatx4{0.f, 0.f, 0.f, 0.f}, acc_hi[e] = floatx4{0.f, 0.f, 0.f, 0.f};
 
-        if (two_blocks) dm_sweep<true>(a.xs, a.qs, d, s0, s1, nq, i0, n0, wcols, li, kk, acc_lo, acc_hi);
-        else dm_sweep<false>(a.xs, a.qs, d, s0, s1, nq, i0, n0, wcols, li, kk, acc_lo, acc_hi);
+        if (sign_rows) {
+            if (two_blocks) dm_sweep<true, true>(qbase, sX, sOff, n, nq, n0, wcols, li, kk, acc_lo, acc_hi);
+            else dm_sweep<false, true>(qbase, sX, sOff, n, nq, n0, wcols, li, kk, acc_lo, acc_hi);
+        } else {
+            if (two_blocks) dm_sweep<true, false>(qbase, sX, sOff, n, nq, n0, wcols, li, kk, acc_lo, acc_hi);
+            else dm_sweep<false, false>(qbase, sX, sOff, n, nq, n0, wcols, li, kk, acc_lo, acc_hi);
+        }
         if (colok) {
 #pragma unroll
             for (int blk = 0; blk < 2; ++blk)
@@ -962,11 +1084,26 @@ __device__ __forceinline__ void transr_dm_body(const DmArgs &a, float *lds, int 
     }
 }
 
+static size_t dm_lds_bytes(int d)  // the staged left operand and its row offsets, or the thin groups' transposed rows
+{
+    const size_t item = sizeof(float) * kDmChunk * kDmXP + sizeof(int64_t) * kDmChunk, thin = sizeof(float) * 4 * (size_t)d;
+    return item > thin ? item : thin;
+}
+
 __global__ __launch_bounds__(256, KGE_TR_OCC) void transr_dm_kernel(DmArgs a, FusedInsp fi)
 {
-    extern __shared__ __align__(16) float lds[];  // thin groups: d float4; inspector workgroups: their own need
+    extern __shared__ __align__(16) float lds[];  // dm_lds_bytes(); inspector workgroups: their own need
+    zero_rider(a.zero);
     if (fused_insp_block(fi, reinterpret_cast<uint32_t *>(lds))) return;
     transr_dm_body(a, lds, (int)blockIdx.x - fi.blocks);
+}
+
+// An inspector step that rides with nothing: the fused entity inspection of a TransR / RESCAL step has
+// four dependent steps and the step three kernels of its own (forward, dX, dM).
+__global__ __launch_bounds__(256) void transr_insp_step_kernel(FusedInsp fi)
+{
+    extern __shared__ __align__(16) float lds[];
+    (void)fused_insp_block(fi, reinterpret_cast<uint32_t *>(lds));
 }
 
 // dX and dM of one backward pass in ONE launch (no inspector riders): the two are independent, one
@@ -976,6 +1113,7 @@ __global__ __launch_bounds__(256, KGE_TR_OCC) void transr_dm_kernel(DmArgs a, Fu
 __global__ __launch_bounds__(256, KGE_TR_OCC) void transr_dx_dm_kernel(GemmArgs ga, DmArgs da)
 {
     extern __shared__ __align__(16) float lds[];
+    zero_rider(da.zero);
     const int bid = (int)blockIdx.x;
     if (bid < ga.max_tiles) {
         transr_gemm_body<2>(ga, lds, bid);
@@ -1004,8 +1142,8 @@ static SumRider dm_finish_rider(const DmArgs &a, int64_t max_split)
 static size_t up256(size_t x) { return (x + 255) & ~size_t(255); }
 
 struct RPlan {
-    size_t off_plan, off_dplan, off_xs, off_qs, off_occ, off_part_e, off_part_r, off_dpart, total;
-    int64_t tiles, dtiles, dsplit, dslots;
+    size_t off_plan, off_dplan, off_occ, off_part_e, off_part_r, off_dpart, off_tickets, total;
+    int64_t tiles, dtiles, dsplit, dslots, tick_e, tick_r;
 };
 
 static size_t plan_ints(int64_t tiles, int64_t split) { return (size_t)(64 + 5 * tiles + 3 * split + 8); }
@@ -1022,12 +1160,12 @@ static RPlan make_rplan(const kge_tables *tab, const kge_batch *bat)
     size_t o = 0;
     p.off_plan = o, o += up256(sizeof(int32_t) * plan_ints(p.tiles, 0));
     p.off_dplan = o, o += up256(sizeof(int32_t) * plan_ints(p.dtiles, p.dsplit));
-    p.off_xs = o, o += up256(sizeof(float) * (size_t)(B * d));
-    p.off_qs = o, o += up256(sizeof(float) * (size_t)(B * d));
     p.off_occ = o, o += up256(sizeof(float) * (size_t)(2 * B * d));
     p.off_part_e = o, o += up256(sizeof(float) * (size_t)seg_partial_floats(2 * B, d));
     p.off_part_r = o, o += up256(sizeof(float) * (size_t)seg_partial_floats(B, d));
     p.off_dpart = o, o += up256(sizeof(float) * (size_t)(p.dslots * d * d));
+    p.tick_e = seg_ticket_ints(2 * B, d), p.tick_r = seg_ticket_ints(B, d);
+    p.off_tickets = o, o += up256(sizeof(int32_t) * (size_t)(p.tick_e + p.tick_r));
     p.total = o;
     return p;
 }
@@ -1107,7 +1245,8 @@ int launch_transr_fwd(const kge_tables *tab, const kge_batch *bat, float *pos, f
         hipLaunchKernelGGL(transr_plan_kernel, dim3(2), dim3(1024), 0, st, ri->num_unique, ri->seg_offsets, ri->unique_ids, plan,
                            kTM, dplan, kDmChunk);
     GemmArgs a{tab->ent, tab->rel, tab->aux, bat->h, bat->r, bat->t, ri->perm, ri->seg_offsets, ri->num_unique, ri->unique_ids,
-               plan, nullptr, nullptr, pos, resid, nullptr, nullptr, (int)tab->dim, tab->norm_p, thin_groups(tab, bat), (int)tiles};
+               plan, nullptr, nullptr, pos, resid, nullptr, nullptr, (int)tab->dim, tab->norm_p, thin_groups(tab, bat), (int)tiles,
+               BwdSrc{}};
     const size_t lds = lds_with(fi, gemm_lds_bytes((int)tab->dim));
     const dim3 grid((unsigned)(tiles + a.thin_groups + fi.blocks));
     if (const int rc = rescal ? allow_lds<1>(lds) : allow_lds<0>(lds)) return rc;
@@ -1147,14 +1286,19 @@ int launch_transr_bwd(const kge_tables *tab, const kge_batch *bat, const kge_sav
     if (!mfma_path_ok(tab, bat) || gemm_lds_bytes((int)tab->dim) > kMaxGemmLds) return KGE_EUNSUPPORTED;
     if (!saved->residual || !grads->aux_rows || !grads->ent_rows) return KGE_EINVAL;
     if (!rescal && (!grads->rel_rows || (tab->norm_p == 2 && !saved->pos))) return KGE_EINVAL;
+    // factored projection gradients of the small groups: both arrays, 16-byte aligned, at most kThin rows
+    const bool factored = grads->aux_factor_max > 0;
+    if (grads->aux_factor_max < 0 || grads->aux_factor_max > kThin) return KGE_EINVAL;
+    if (factored && (!grads->aux_x || !grads->aux_q || !aligned16(grads->aux_x) || !aligned16(grads->aux_q))) return KGE_EINVAL;
+    if (!aligned16(saved->residual)) return KGE_EINVAL;
     const RPlan p = make_rplan(tab, bat);
     if (!workspace || workspace_bytes < p.total) return KGE_EWORKSPACE;
     if (bat->ent_insp->n != 2 * bat->batch) return KGE_ESHAPE;
     const int64_t B = bat->batch;
     const int d = (int)tab->dim;
     char *ws = static_cast<char *>(workspace);
-    float *xs = reinterpret_cast<float *>(ws + p.off_xs), *qs = reinterpret_cast<float *>(ws + p.off_qs);
     float *occ = reinterpret_cast<float *>(ws + p.off_occ);
+    int32_t *tickets = reinterpret_cast<int32_t *>(ws + p.off_tickets);
     const kge_inspection *ri = bat->rel_insp;
     // the plans: left behind by the forward pass, or built here
     const bool have_plans = saved->fwd_workspace && saved->fwd_workspace_bytes >= transr_fwd_workspace(tab, bat);
@@ -1163,9 +1307,8 @@ int launch_transr_bwd(const kge_tables *tab, const kge_batch *bat, const kge_sav
     TilePlan dplan = have_plans ? plan_at(pbase + fwd_plan_bytes(tab, bat), p.dtiles, p.dsplit)
                                 : plan_at(ws + p.off_dplan, p.dtiles, p.dsplit);
 
-    PrepArgs pa{tab->ent, bat->h, bat->t, ri->perm, dpos, saved->pos, saved->residual, xs, qs, occ + B * d, B, d,
-                tab->norm_p, rescal ? 1 : 0};
-    // fused entity inspection: first digit pass with prep, second with the dX GEMM, dedup with dM
+    // fused entity inspection (its histogram rode with the forward GEMM): first digit pass in a launch
+    // of its own, second with the dX GEMM, dedup with dM
     FusedInsp f1{}, f2{}, f3{};
     if (bat->fuse_inspection) {
         if (!bat->insp_jobs) return KGE_EINVAL;
@@ -1173,22 +1316,27 @@ int launch_transr_bwd(const kge_tables *tab, const kge_batch *bat, const kge_sav
         if ((rc = plan_fused_inspection(bat->insp_jobs, 1, 1, &f1))) return rc;
         if ((rc = plan_fused_inspection(bat->insp_jobs, 1, 2, &f2))) return rc;
         if ((rc = plan_fused_inspection(bat->insp_jobs, 1, 3, &f3))) return rc;
+        hipLaunchKernelGGL(transr_insp_step_kernel, dim3((unsigned)f1.blocks), dim3(256), lds_with(f1, 0), st, f1);
+        timeline_mark(bat->timeline, st, "inspector step");
     }
-    hipLaunchKernelGGL(transr_prep_kernel, dim3((unsigned)(ceil_div(B, 4) + f1.blocks)), dim3(256), lds_with(f1, 0), st, pa,
-                       f1);
-    timeline_mark(bat->timeline, st, "transr_prep_kernel");
     if (!have_plans)
         hipLaunchKernelGGL(transr_plan_kernel, dim3(2), dim3(1024), 0, st, ri->num_unique, ri->seg_offsets, ri->unique_ids, plan, kTM,
                            dplan, kDmChunk);
+    // Upstream rows q and left operands x are formed inside the two kernels from the forward pass's rows
+    // (BwdSrc); RESCAL's tail occurrence rows g * v come out of the dX kernel's staging.
+    const BwdSrc src{tab->ent, saved->residual, dpos, saved->pos, bat->h, bat->t, ri->perm, tab->norm_p, rescal ? 1 : 0,
+                     rescal ? occ + B * d : nullptr};
     // dX = Q M^T -> occurrence rows of h (and -dX for t)
     GemmArgs ga{tab->ent, tab->rel, tab->aux, bat->h, bat->r, bat->t, ri->perm, ri->seg_offsets, ri->num_unique, ri->unique_ids,
-                plan, qs, nullptr, nullptr, nullptr, occ, rescal ? nullptr : occ + B * d, d, tab->norm_p, thin_groups(tab, bat), (int)p.tiles};
+                plan, nullptr, nullptr, nullptr, nullptr, occ, rescal ? nullptr : occ + B * d, d, tab->norm_p, thin_groups(tab, bat),
+                (int)p.tiles, src};
     // dM = X^T Q per relation group
     const int dm_items = (int)(ceil_div(d, 32) * p.dtiles);
-    DmArgs da{xs, qs, ri->seg_offsets, dplan, grads->aux_rows, reinterpret_cast<float *>(ws + p.off_dpart), d,
-              ri->num_unique, dm_items};
+    DmArgs da{nullptr, nullptr, ri->seg_offsets, dplan, grads->aux_rows, reinterpret_cast<float *>(ws + p.off_dpart), d,
+              ri->num_unique, dm_items, src, factored ? grads->aux_x : nullptr, factored ? grads->aux_q : nullptr,
+              grads->aux_factor_max, ZeroRider{tickets, p.tick_e + p.tick_r}};
     if (!bat->fuse_inspection) {  // nothing rides along: both in one launch
-        const size_t lds = gemm_lds_bytes(d) > sizeof(float) * 4 * (size_t)d ? gemm_lds_bytes(d) : sizeof(float) * 4 * (size_t)d;
+        const size_t lds = gemm_lds_bytes(d) > dm_lds_bytes(d) ? gemm_lds_bytes(d) : dm_lds_bytes(d);
         if (lds > 64 * 1024 &&
             hipFuncSetAttribute(reinterpret_cast<const void *>(&transr_dx_dm_kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
                                 (int)kMaxGemmLds) != hipSuccess)
@@ -1202,17 +1350,20 @@ int launch_transr_bwd(const kge_tables *tab, const kge_batch *bat, const kge_sav
                            lds_with(f2, gemm_lds_bytes(d)), st, ga, f2);
         timeline_mark(bat->timeline, st, "transr_gemm_kernel<dX>");
         hipLaunchKernelGGL(transr_dm_kernel, dim3((unsigned)(dm_items + thin_groups(tab, bat) + f3.blocks)), dim3(256),
-                           lds_with(f3, sizeof(float) * 4 * (size_t)d), st, da, f3);
+                           lds_with(f3, dm_lds_bytes(d)), st, da, f3);
         timeline_mark(bat->timeline, st, "transr_dm_kernel");
     }
     KGE_CHECK_LAUNCH();
     if (bat->insp_ready && hipStreamWaitEvent(st, reinterpret_cast<hipEvent_t>(bat->insp_ready), 0) != hipSuccess)
         return KGE_ELAUNCH;
-    // entity rows from the h / t occurrence rows; dR[g] = sum of the group's q rows, which are
-    // already stored in sorted order
-    const SegJob jobs[2] = {
-        {occ, bat->ent_insp, d, grads->ent_rows, reinterpret_cast<float *>(ws + p.off_part_e), false},
-        {qs, ri, d, grads->rel_rows, reinterpret_cast<float *>(ws + p.off_part_r), true}};
+    // entity rows from the h / t occurrence rows; dR[g] = sum of the group's upstream rows, formed from the
+    // residual rows as the reduction loads them (scale dpos or dpos / pos, sign for L1).  One launch: the
+    // kernel above cleared the tickets.
+    SegJob jobs[2] = {{occ, bat->ent_insp, d, grads->ent_rows, reinterpret_cast<float *>(ws + p.off_part_e), false, tickets},
+                      {saved->residual, ri, d, grads->rel_rows, reinterpret_cast<float *>(ws + p.off_part_r), false,
+                       tickets + p.tick_e}};
+    jobs[1].scaled = true, jobs[1].sign_rows = tab->norm_p == 1;
+    jobs[1].scale_num = dpos, jobs[1].scale_den = tab->norm_p == 2 ? saved->pos : nullptr;
     const SumRider finish = dm_finish_rider(da, p.dsplit);
     return launch_seg_reduce_jobs(jobs, rescal ? 1 : 2, st, bat->timeline, &finish);
 }

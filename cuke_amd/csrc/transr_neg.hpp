@@ -673,7 +673,7 @@ int launch_transr_neg_fwd(const kge_tables *tab, const kge_batch *bat, float *po
     // one grouped pass projects every list row
     float *y = reinterpret_cast<float *>(ws + l.y);
     GemmArgs ga{tab->ent, tab->rel, tab->aux, x.hl, nullptr, x.tl, nullptr, x.segl, ri->num_unique, ri->unique_ids,
-                plan, nullptr, x.rsl, nullptr, y, nullptr, nullptr, d, tab->norm_p, (int)s.U_cap, (int)s.tiles};
+                plan, nullptr, x.rsl, nullptr, y, nullptr, nullptr, d, tab->norm_p, (int)s.U_cap, (int)s.tiles, BwdSrc{}};
     const size_t lds = gemm_lds_bytes(d);
     if (const int rc = allow_lds<3>(lds)) return rc;
     hipLaunchKernelGGL(transr_gemm_kernel<3>, dim3((unsigned)(s.tiles + s.U_cap)), dim3(256), lds, st, ga, FusedInsp{});
@@ -700,7 +700,9 @@ int launch_transr_neg_bwd(const kge_tables *tab, const kge_batch *bat, const kge
     if (!saved->fwd_workspace || saved->fwd_workspace_bytes < fl.total) return KGE_EINVAL;
     if (!workspace || workspace_bytes < l.total || !aligned16(workspace)) return KGE_EWORKSPACE;
     if (!grads->ent_rows || !grads->rel_rows || !grads->aux_rows) return KGE_EINVAL;
-    if (tab->norm_p == 2 && ((dpos && !saved->pos) || (dneg && !saved->neg))) return KGE_EINVAL;
+    // the per-positive kernel reads the positive scores whenever the norm is L2 (dpos == NULL stands for
+    // zeros, not for "skip"), so they are required as in launch_transr_bwd
+    if (tab->norm_p == 2 && (!saved->pos || (dneg && !saved->neg))) return KGE_EINVAL;
     if (!bat->ent_insp || bat->ent_insp->n != 2 * s.B + s.NN) return KGE_ESHAPE;
     char *fws = static_cast<char *>(const_cast<void *>(saved->fwd_workspace)), *ws = static_cast<char *>(workspace);
     const NegIdx x = neg_idx(tab, bat, s, fl, fws);
@@ -729,15 +731,15 @@ int launch_transr_neg_bwd(const kge_tables *tab, const kge_batch *bat, const kge
 
     // dX = Q M^T over the list (rows stay in list order), dM = X^T Q per relation
     GemmArgs ga{tab->ent, tab->rel, tab->aux, x.hl, nullptr, x.tl, nullptr, x.segl, ri->num_unique, ri->unique_ids,
-                plan, ql, nullptr, nullptr, nullptr, dxl, nullptr, d, tab->norm_p, (int)s.U_cap, (int)s.tiles};
+                plan, ql, nullptr, nullptr, nullptr, dxl, nullptr, d, tab->norm_p, (int)s.U_cap, (int)s.tiles, BwdSrc{}};
     const size_t lds = gemm_lds_bytes(d);
     if (const int rc = allow_lds<2>(lds)) return rc;
     hipLaunchKernelGGL(transr_gemm_kernel<2>, dim3((unsigned)(s.tiles + s.U_cap)), dim3(256), lds, st, ga, FusedInsp{});
     timeline_mark(bat->timeline, st, "transr_gemm_kernel<dX>");
     const int dm_items = (int)(ceil_div(d, 32) * s.dtiles);
-    DmArgs da{xl, ql, x.segl, dplan, grads->aux_rows, reinterpret_cast<float *>(ws + l.dpart), d, ri->num_unique, dm_items};
-    hipLaunchKernelGGL(transr_dm_kernel, dim3((unsigned)(dm_items + s.U_cap)), dim3(256), sizeof(float) * 4 * (size_t)d, st, da,
-                       FusedInsp{});
+    DmArgs da{xl, ql, x.segl, dplan, grads->aux_rows, reinterpret_cast<float *>(ws + l.dpart), d, ri->num_unique, dm_items,
+              BwdSrc{}, nullptr, nullptr, 0, ZeroRider{}};
+    hipLaunchKernelGGL(transr_dm_kernel, dim3((unsigned)(dm_items + s.U_cap)), dim3(256), dm_lds_bytes(d), st, da, FusedInsp{});
     timeline_mark(bat->timeline, st, "transr_dm_kernel");
     TNEG_BY_WIDTH(d, hipLaunchKernelGGL(tneg_occ_kernel<NQ_>, dim3((unsigned)(ceil_div(s.B, 4) + s.NN)), dim3(256), 0, st, x, dxl,
                                         glist, gcount, occ));

@@ -23,7 +23,8 @@ from . import _lib
 from ._lib import KgeError, MODELS
 
 __all__ = ["KGEModel", "TrainStep", "Inspection", "Forward", "SparseGrads", "inspect", "inspector", "transE",
-           "transH", "transR", "transF", "RESCAL", "margin_loss", "sparse_sgd", "sparse_adagrad", "KgeError"]
+           "transH", "transR", "transF", "RESCAL", "margin_loss", "sparse_sgd", "sparse_adagrad",
+           "sparse_sgd_factored", "sparse_adagrad_factored", "KgeError"]
 
 
 NEG_MODES = {"tail": 0, "head": 1}  # KGE_NEG_TAIL / KGE_NEG_HEAD
@@ -160,6 +161,15 @@ class SparseGrads:
     rel_ids: torch.Tensor
     rel_rows: torch.Tensor | None
     aux_rows: torch.Tensor | None
+    # TransR / RESCAL with factor_max > 0 (kge_grads.aux_x / aux_q): the projection gradient of a relation
+    # group of at most factor_max triples is sum_p aux_x[p]^T aux_q[p] over its sorted positions
+    # p in [rel_seg_offsets[u], rel_seg_offsets[u + 1]) and its aux_rows[u] is not written
+    aux_x: torch.Tensor | None = None
+    aux_q: torch.Tensor | None = None
+    factor_max: int = 0
+    rel_seg_offsets: torch.Tensor | None = None
+    _c: object = None          # the kge_grads struct these arrays were written through
+    _rel_insp: object = None
 
 
 class KGEModel:
@@ -315,8 +325,12 @@ class KGEModel:
         return inspect(parts, int(self.E.shape[0])), inspect([r], max(self.n_rel, 1))
 
     # -- gradients ---------------------------------------------------------------------------
-    def backward(self, fw: Forward, dpos=None, dneg=None) -> SparseGrads:
-        """Sparse row gradients of sum(dpos * pos) + sum(dneg * neg)."""
+    def backward(self, fw: Forward, dpos=None, dneg=None, factor_max: int = 0) -> SparseGrads:
+        """Sparse row gradients of sum(dpos * pos) + sum(dneg * neg).
+
+        ``factor_max`` (TransR / RESCAL without negatives, 0..4): relation groups of at most that many
+        triples leave their projection gradient factored (``SparseGrads.aux_x`` / ``aux_q``) instead of
+        writing a dense dim x dim matrix; ``sparse_sgd_factored`` / ``sparse_adagrad_factored`` apply it."""
         if getattr(fw, "flat_pos", None) is not None:  # TransR / RESCAL negatives: one flat batch
             B, N = fw.neg.shape
             f32 = dict(dtype=torch.float32, device=self.dev)
@@ -326,7 +340,7 @@ class KGEModel:
             if dneg is not None:
                 g[B:] = dneg.to(**f32).reshape(-1)
             flat = Forward(fw.flat_pos, None, residual=fw.residual, batch=fw.batch, ent_insp=fw.ent_insp,
-                           rel_insp=fw.rel_insp)
+                           rel_insp=fw.rel_insp, fwd_ws=fw.fwd_ws)
             return self.backward(flat, g)
         h, r, t, neg, C_, N = fw.batch
         if fw.ent_insp is None or fw.rel_insp is None:
@@ -351,7 +365,12 @@ class KGEModel:
             aux_rows = torch.empty((B, self.dim), **f32)
         elif self.model in ("TransR", "RESCAL"):
             aux_rows = torch.empty((min(B, self.n_rel), self.dim * self.dim), **f32)
-        grads = _lib.Grads(_ptr(ent_rows), _ptr(rel_rows), _ptr(aux_rows))
+        aux_x = aux_q = None
+        if factor_max:
+            if self.model not in ("TransR", "RESCAL") or neg is not None:
+                raise ValueError("factor_max applies to TransR / RESCAL without shared negatives")
+            aux_x, aux_q = torch.empty((B, self.dim), **f32), torch.empty((B, self.dim), **f32)
+        grads = _lib.Grads(_ptr(ent_rows), _ptr(rel_rows), _ptr(aux_rows), _ptr(aux_x), _ptr(aux_q), int(factor_max), 0)
         L = _lib.lib()
         ws_bytes = int(L.kge_score_bwd_workspace(C.byref(self._tab), C.byref(bat)))
         ws = torch.empty(max(ws_bytes, 1), dtype=torch.uint8, device=self.dev)
@@ -361,7 +380,9 @@ class KGEModel:
         ue, ur = fw.ent_insp.num_unique, fw.rel_insp.num_unique
         return SparseGrads(fw.ent_insp.ids(), ent_rows[:ue], fw.rel_insp.ids(),
                            rel_rows[:ur] if rel_rows is not None else None,
-                           aux_rows[:ur] if aux_rows is not None else None)
+                           aux_rows[:ur] if aux_rows is not None else None,
+                           aux_x, aux_q, int(factor_max), fw.rel_insp.offsets() if factor_max else None,
+                           grads, fw.rel_insp)
 
 
 def margin_loss(pos: torch.Tensor, neg: torch.Tensor, margin: float, sign: float = 1.0):
@@ -402,6 +423,24 @@ def sparse_adagrad(table: torch.Tensor, state: torch.Tensor, insp: Inspection, r
     _lib.check(_lib.lib().kge_sparse_adagrad(_ptr(t), _ptr(state), int(rows.shape[1]), _ptr(insp.unique_ids),
                                              _ptr(insp.num_unique_dev), int(rows.shape[0]), _ptr(rows), float(lr),
                                              float(eps), _stream()), "kge_sparse_adagrad")
+
+
+def sparse_sgd_factored(proj: torch.Tensor, g: SparseGrads, lr: float) -> None:
+    """Proj[id] -= lr * dM for the projection gradients of ``KGEModel.backward(..., factor_max=m)`` /
+    ``TrainStep(..., factor_max=m)``: dense groups from ``aux_rows``, factored groups straight from their rows."""
+    t = _inplace_table(proj)
+    _lib.check(_lib.lib().kge_sparse_sgd_factored(_ptr(t), int(proj.shape[1]), C.byref(g._rel_insp._c), C.byref(g._c),
+                                                  float(lr), _stream()), "kge_sparse_sgd_factored")
+
+
+def sparse_adagrad_factored(proj: torch.Tensor, state: torch.Tensor, g: SparseGrads, lr: float, eps: float = 1e-10) -> None:
+    """Row-wise Adagrad on the projection table from partly factored gradients (state: [n_rel])."""
+    t = _inplace_table(proj)
+    if not state.is_contiguous():
+        raise ValueError("state must be contiguous: it is updated in place")
+    _lib.check(_lib.lib().kge_sparse_adagrad_factored(_ptr(t), _ptr(state), int(proj.shape[1]), C.byref(g._rel_insp._c),
+                                                      C.byref(g._c), float(lr), float(eps), _stream()),
+               "kge_sparse_adagrad_factored")
 
 
 # ---- the reference's positional call shapes --------------------------------------------------
@@ -485,7 +524,7 @@ class TrainStep:
     kPipelineSets = 3  # one running, one being inspected, one being refilled
 
     def __init__(self, model: KGEModel, h, r, t, neg=None, chunk=None, loss="sum", margin=1.0,
-                 sign=1.0, dpos=None, dneg=None, neg_mode="tail"):
+                 sign=1.0, dpos=None, dneg=None, neg_mode="tail", factor_max=0):
         self.m = model
         dev = model.dev
         L = self.L = _lib.lib()
@@ -542,7 +581,14 @@ class TrainStep:
             self.aux_rows = torch.empty((B, model.dim), **f32)
         elif model.model in ("TransR", "RESCAL"):
             self.aux_rows = torch.empty((min(B, model.n_rel), model.dim * model.dim), **f32)
-        self.grads = _lib.Grads(_ptr(self.ent_rows), _ptr(self.rel_rows), _ptr(self.aux_rows))
+        self.factor_max = int(factor_max)
+        self.aux_x = self.aux_q = None
+        if self.factor_max:
+            if model.model not in ("TransR", "RESCAL") or neg is not None:
+                raise ValueError("factor_max applies to TransR / RESCAL without shared negatives")
+            self.aux_x, self.aux_q = torch.empty((B, model.dim), **f32), torch.empty((B, model.dim), **f32)
+        self.grads = _lib.Grads(_ptr(self.ent_rows), _ptr(self.rel_rows), _ptr(self.aux_rows), _ptr(self.aux_x),
+                                _ptr(self.aux_q), self.factor_max, 0)
         self._ws_b_bytes = int(L.kge_score_bwd_workspace(C.byref(model._tab), C.byref(self.bat)))
         self._ws_b = torch.empty(max(self._ws_b_bytes, 1), dtype=torch.uint8, device=dev)
         self.graph = None
@@ -947,4 +993,6 @@ class TrainStep:
         ue, ur = self.ent_insp.num_unique, self.rel_insp.num_unique
         return SparseGrads(self.ent_insp.unique_ids[:ue], self.ent_rows[:ue], self.rel_insp.unique_ids[:ur],
                            self.rel_rows[:ur] if self.rel_rows is not None else None,
-                           self.aux_rows[:ur] if self.aux_rows is not None else None)
+                           self.aux_rows[:ur] if self.aux_rows is not None else None,
+                           self.aux_x, self.aux_q, self.factor_max,
+                           self.rel_insp.seg_offsets[:ur + 1] if self.factor_max else None, self.grads, self.rel_insp)

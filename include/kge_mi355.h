@@ -84,7 +84,9 @@ enum { KGE_PAIR_SUMS_VALU = 1 };
  *   kge_timeline_begin    count = 0 and records `begin` on the stream
  *   kge_timeline_mark     the caller's own entry (work enqueued between two library calls)
  *   kge_timeline_elapsed  ms[k] for k < count; call after the stream has been synchronised;
- *                         returns count or a negative status
+ *                         returns count or a negative status (KGE_EWORKSPACE when the call launched
+ *                         more kernels than `capacity`, or an event could not be recorded: `dropped`
+ *                         counts the entries that are missing, so a truncated table is never returned)
  */
 typedef struct kge_timeline {
     void *begin;          /* hipEvent_t */
@@ -92,6 +94,8 @@ typedef struct kge_timeline {
     const char **labels;  /* host array of `capacity` slots, filled with static strings */
     int32_t capacity;
     int32_t count;        /* in / out */
+    int32_t dropped;      /* entries lost since kge_timeline_begin (timeline full, failed event record) */
+    int32_t reserved;
 } kge_timeline;
 kge_timeline *kge_timeline_create(int32_t capacity);
 void kge_timeline_destroy(kge_timeline *tl);
@@ -157,8 +161,8 @@ typedef struct kge_batch {
          and first digit pass with the two forward kernels of kge_score_fwd (pos and neg scores
          must be requested), last pass and dedup with the two gradient kernels of kge_score_bwd.
        - TransR / RESCAL on their grouped path (no negatives, rel_insp complete before
-         kge_score_fwd): job [0] rides with the forward GEMM, then with the prep, dX and dM kernels
-         of kge_score_bwd; job [1] is not used.
+         kge_score_fwd): job [0] rides with the forward GEMM, then (after one step in a launch of its
+         own) with the dX and dM kernels of kge_score_bwd; job [1] is not used.
        Requirements: each riding index set at most 65536 ids, tables of at most 2^22 rows
        (kge_fused_inspection_ok says whether a batch qualifies); kge_score_fwd and kge_score_bwd
        must both be called, in this order, on one stream, and the riding inspections hold their
@@ -200,6 +204,22 @@ typedef struct kge_grads {
     float *ent_rows;  /* [ent_insp->n, dim]        first U_ent rows written */
     float *rel_rows;  /* [B, rel_dim]              first U_rel rows written */
     float *aux_rows;  /* TransH: [B, dim]; TransR / RESCAL: [min(B, n_rel), dim*dim] */
+    /* TransR / RESCAL without shared negatives, optional: FACTORED projection gradients of the small
+       relation groups.  The gradient of relation group u (the u-th unique relation, sorted positions
+       p in [seg_offsets[u], seg_offsets[u+1]) of rel_insp) is the sum over its triples of the outer
+       products x_p^T q_p (x_p = E[h] - E[t], or E[h] for RESCAL; q_p the upstream row of the projected
+       vector).  A group of one triple, as most relations of a long-tailed batch are, costs dim*dim
+       floats of memory traffic to write out and again to read in the optimizer, for 2*dim floats of
+       information.  With aux_factor_max = m in 1..4, a group of at most m triples leaves its rows
+       x_p in aux_x[p] and q_p in aux_q[p] and its aux_rows[u] is NOT written; larger groups are written
+       dense as always (their aux_x / aux_q rows are not written).  kge_sparse_sgd_factored /
+       kge_sparse_adagrad_factored apply either form.  aux_factor_max = 0: every group dense (the
+       form the parity tests check; the factored rows are tested against it).  No counterpart in the
+       reference, whose printed gradient kernels are per-triple dense (apps/kge/kge.py:413-418). */
+    float *aux_x;            /* [B, dim], 16-byte aligned */
+    float *aux_q;            /* [B, dim], 16-byte aligned */
+    int32_t aux_factor_max;  /* 0..4 */
+    int32_t reserved;
 } kge_grads;
 
 const char *kge_strerror(int status);
@@ -239,6 +259,10 @@ int kge_residual_fwd(const kge_tables *tab, const kge_batch *bat, float *out, vo
  * two workgroups per CU): given kge_score_fwd_workspace() bytes of workspace the reduction axis of
  * every tile is split over up to four workgroups (partial score planes in the workspace, a finishing
  * kernel); without the workspace the same call runs one workgroup per tile.
+ * TransE, and DistMult / ComplEx on the matrix-core tiles: when pos and neg are both requested, no
+ * side output is and no inspection rides along, the positives are scored by extra workgroups of the
+ * shared-negative launch (one launch instead of two; a timeline then has no "score_pos_kernel"
+ * entry and its "score_neg_kernel" entry includes the positives).  Results are the same bits.
  * RotatE: `residual` [B, dim] receives the rotated heads h e^{i theta}; the shared-negative
  * kernels (forward and backward) load them instead of recomputing a sincos per element, so it
  * is required whenever negatives are scored (filled by this call when pos is requested, or
@@ -359,6 +383,20 @@ int kge_sparse_sgd(float *table, int64_t dim, const int64_t *ids, const int32_t 
                    const float *rows, float lr, void *stream);
 int kge_sparse_adagrad(float *table, float *state, int64_t dim, const int64_t *ids, const int32_t *num_unique,
                        int64_t capacity, const float *rows, float lr, float eps, void *stream);
+
+/*
+ * The same two rules on the projection table of TransR / RESCAL (proj: [n_rel, dim, dim]) from gradients
+ * that kge_score_bwd left partly factored (kge_grads.aux_x / aux_q / aux_factor_max, groups delimited by
+ * rel_insp): a factored group's update is applied as  Proj[id] -= scale * sum_p x_p^T q_p  straight from
+ * its rows, a dense group's from grads->aux_rows[u].  Adagrad's row statistic mean(g^2) of a factored
+ * group is sum_{p,p'} (x_p . x_p')(q_p . q_p') / dim^2, the squared Frobenius norm of the sum of outer
+ * products.  state: [n_rel].  With aux_factor_max = 0 both reduce to kge_sparse_sgd / kge_sparse_adagrad
+ * on aux_rows.  dim % 4 == 0, 16-byte aligned arrays.
+ */
+int kge_sparse_sgd_factored(float *proj, int64_t dim, const kge_inspection *rel_insp, const kge_grads *grads,
+                            float lr, void *stream);
+int kge_sparse_adagrad_factored(float *proj, float *state, int64_t dim, const kge_inspection *rel_insp,
+                                const kge_grads *grads, float lr, float eps, void *stream);
 
 /*
  * Uniform negative entity ids for one batch, drawn on the device: out[i] for i < count is

@@ -34,7 +34,7 @@ def test_binding_table_matches_header():
 def test_strerror_and_version_without_gpu():
     from cuke_amd import _lib
     L = _lib.lib()
-    assert L.kge_abi_version() == _lib.ABI_VERSION == 5
+    assert L.kge_abi_version() == _lib.ABI_VERSION == 6
     assert L.kge_strerror(0) == b"ok"
     assert b"workspace" in L.kge_strerror(-4)
 
@@ -107,6 +107,29 @@ def test_argument_validation_returns_status_codes_without_touching_the_gpu():
     assert L.kge_score_fwd(C.byref(tables()), C.byref(batch(B=0, h=None, r=None, t=None)), None, None, None, None,
                            None, None, 0, None) == 0
     assert L.kge_sample_negatives(None, 0, 5, 1, 0, None) == 0
+
+
+def test_transr_negatives_backward_requires_the_positive_scores_for_l2():
+    """TransR with shared negatives, L2: the per-positive gradient kernel divides by the saved positive scores
+    whether or not dpos is given (dpos == NULL means zeros), so a missing kge_saved.pos is an argument error on
+    the host, before anything is launched (the pointers below are never dereferenced)."""
+    import ctypes as C
+    from cuke_amd import _lib
+    L = _lib.lib()
+    fake = 0x10000
+    B, N, d, n_rel = 64, 8, 16, 5
+    tab = _lib.Tables(_lib.MODELS["TransR"], 2, 0.0, 0, d, d, 100, n_rel, fake, fake, fake)
+    rel = _lib.Inspection(B, n_rel, fake, fake, fake, fake, fake, fake)
+    ent = _lib.Inspection(2 * B + (B // 16) * N, 100, fake, fake, fake, fake, fake, fake)
+    bat = _lib.Batch(B, fake, fake, fake, fake, 16, N, C.pointer(ent), C.pointer(rel), None, 0, 0)
+    fwd_bytes = int(L.kge_score_fwd_workspace(C.byref(tab), C.byref(bat)))
+    bwd_bytes = int(L.kge_score_bwd_workspace(C.byref(tab), C.byref(bat)))
+    assert fwd_bytes > 0 and bwd_bytes > 0
+    grads = _lib.Grads(fake, fake, fake)
+    for dpos in (None, fake):
+        saved = _lib.Saved(None, fake, None, None, fake, fake, fwd_bytes)   # pos missing, everything else there
+        assert L.kge_score_bwd(C.byref(tab), C.byref(bat), C.byref(saved), dpos, fake, C.byref(grads), fake, bwd_bytes,
+                               None) == -1
 
 
 def test_fused_inspection_eligibility_is_decided_on_the_host():

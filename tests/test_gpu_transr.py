@@ -85,6 +85,126 @@ def test_grouped_backward(oracle, model, shape, p):
     assert_close(g.aux_rows.cpu().numpy(), ref.aux_rows, what="projection gradients", rows=True)
 
 
+def dense_projection_gradients(g):
+    """Dense [U, dim * dim] projection gradients from partly factored ones: a factored group's matrix is the sum
+    of the outer products of its rows (float64 on the host; what the device left in aux_rows for such a group
+    is ignored)."""
+    off = g.rel_seg_offsets.cpu().numpy()
+    x, q = g.aux_x.cpu().numpy().astype(np.float64), g.aux_q.cpu().numpy().astype(np.float64)
+    out = g.aux_rows.cpu().numpy().astype(np.float64).copy()
+    d = x.shape[1]
+    factored = 0
+    for u in range(len(off) - 1):
+        if off[u + 1] - off[u] <= g.factor_max:
+            out[u] = (x[off[u]:off[u + 1]].T @ q[off[u]:off[u + 1]]).reshape(d * d)
+            factored += 1
+    return out, factored
+
+
+@pytest.mark.parametrize("model", ["TransR", "RESCAL"])
+@pytest.mark.parametrize("p", [1, 2])
+@pytest.mark.parametrize("fmax", [1, 3, 4])
+@pytest.mark.parametrize("shape", [dict(dim=200, batch=300, n_rel=150), dict(dim=36, batch=130, n_rel=60),
+                                   dict(dim=512, batch=64, n_rel=40)])
+def test_factored_projection_gradients_equal_the_dense_ones(oracle, model, p, fmax, shape):
+    """kge_grads.aux_x / aux_q: groups of at most fmax triples leave x_p, q_p instead of the dense matrix;
+    sum_p x_p^T q_p must be the oracle's dense gradient, larger groups stay dense, and the poisoned dense rows
+    of the factored groups must not have been written."""
+    if model == "RESCAL" and p == 1:
+        pytest.skip("no norm in RESCAL")
+    w = synth.custom_workload(model, n_ent=120, norm_p=p, sigma=0.2, rel_zipf=1.2, ent_zipf=1.1,
+                              seed=shape["dim"] + p, lattice=(p == 1 and model == "TransR"), **shape)
+    a = w.arrays
+    if w.lattice:
+        a["A"] = (np.rint(a["A"] / 0.2 * 2) / 8).astype(np.float32)
+    m, ix = gpu_model(w)
+    fw, rel = grouped_forward(m, ix)
+    dpos = np.random.default_rng(1).standard_normal(w.batch).astype(np.float32)
+    dense = m.backward(fw, torch.from_numpy(dpos).cuda())
+    g = m.backward(fw, torch.from_numpy(dpos).cuda(), factor_max=fmax)
+    ref = oracle.backward(model, a["E"], a["R"], a["A"], a["h"], a["r"], a["t"], dpos=dpos, p=p)
+    got, n_fact = dense_projection_gradients(g)
+    counts = np.diff(g.rel_seg_offsets.cpu().numpy())
+    assert n_fact == int((counts <= fmax).sum()) and 0 < n_fact < len(counts), "the shape must mix both kinds of group"
+    assert_close(got, ref.aux_rows, what=f"{model} fmax={fmax} projection gradients (factored groups multiplied out)", rows=True)
+    # the other outputs do not depend on the form, bit for bit
+    assert torch.equal(g.ent_rows, dense.ent_rows)
+    if model == "TransR":
+        assert torch.equal(g.rel_rows, dense.rel_rows)
+    big = torch.from_numpy(counts > fmax).cuda()
+    assert torch.equal(g.aux_rows[big], dense.aux_rows[big]), "dense groups are the same bits in both forms"
+
+
+@pytest.mark.parametrize("model", ["TransR", "RESCAL"])
+@pytest.mark.parametrize("rule", ["sgd", "adagrad"])
+def test_factored_optimizer_step_equals_the_dense_one(oracle, model, rule):
+    """kge_sparse_sgd_factored / kge_sparse_adagrad_factored on partly factored gradients against
+    kge_sparse_sgd / kge_sparse_adagrad on the dense gradients of the same batch (the oracle-pinned rules)."""
+    from cuke_amd import kge
+    w = synth.custom_workload(model, n_ent=200, n_rel=80, dim=64, batch=256, norm_p=2, sigma=0.2, rel_zipf=1.2, seed=11)
+    m, ix = gpu_model(w)
+    fw, rel = grouped_forward(m, ix)
+    dpos = torch.from_numpy(np.random.default_rng(2).standard_normal(w.batch).astype(np.float32)).cuda()
+    dense = m.backward(fw, dpos)
+    fact = m.backward(fw, dpos, factor_max=4)
+    n_rel, d = m.A.shape[0], m.dim
+    ref_tab, got_tab = m.A.clone().view(n_rel, d * d), m.A.clone()
+    if rule == "sgd":
+        kge.sparse_sgd(ref_tab, rel, dense.aux_rows, 0.1)
+        kge.sparse_sgd_factored(got_tab, fact, 0.1)
+    else:
+        st0 = torch.rand(n_rel, device="cuda") * 1e-3
+        ref_state, got_state = st0.clone(), st0.clone()
+        kge.sparse_adagrad(ref_tab, ref_state, rel, dense.aux_rows, 0.1)
+        kge.sparse_adagrad_factored(got_tab, got_state, fact, 0.1)
+        assert_close(got_state.cpu().numpy(), ref_state.cpu().numpy(), what="Adagrad state")
+    assert_close(got_tab.view(n_rel, d * d).cpu().numpy(), ref_tab.cpu().numpy(), what=f"{model} {rule} projection table", rows=True)
+    touched = torch.zeros(n_rel, dtype=torch.bool, device="cuda")
+    touched[fact.rel_ids] = True
+    assert torch.equal(got_tab[~touched], m.A[~touched]), "rows of relations outside the batch must not move"
+
+
+def test_train_step_factored_all_issue_forms(oracle):
+    """TrainStep(factor_max=4) through the one-stream, fused, side-stream and staged issues: every form leaves
+    the same factored rows, and multiplied out they are the oracle's dense gradients."""
+    from cuke_amd.kge import TrainStep
+    ws = [synth.make_workload("cfg3_transr", batch=1024, seed=s) for s in range(3)]
+    m, ix0 = gpu_model(ws[0])
+    step = TrainStep(m, ix0["h"], ix0["r"], ix0["t"], factor_max=4)
+    for w in ws[1:]:
+        ix = {k: torch.from_numpy(w.arrays[k]).cuda() for k in ("h", "r", "t")}
+        step.add_batch(ix["h"], ix["r"], ix["t"])
+    a0 = ws[0].arrays
+
+    def check(w, tag):
+        torch.cuda.synchronize()
+        a = w.arrays
+        ref = oracle.backward("TransR", a0["E"], a0["R"], a0["A"], a["h"], a["r"], a["t"], dpos=step.dpos.cpu().numpy(), p=2)
+        g = step.sparse_grads()
+        assert np.array_equal(g.rel_ids.cpu().numpy(), ref.rel_ids), tag
+        got, n_fact = dense_projection_gradients(g)
+        assert n_fact > 0
+        assert_close(got, ref.aux_rows, what=f"{tag} projection gradients", rows=True)
+        assert_close(g.ent_rows.cpu().numpy(), ref.ent_rows, what=f"{tag} entity rows", rows=True)
+        assert_close(g.rel_rows.cpu().numpy(), ref.rel_rows, what=f"{tag} relation rows", rows=True)
+
+    step.run(overlap=False, fused=False)
+    check(ws[0], "one stream")
+    if step.fusable:
+        step.aux_x.zero_(), step.aux_q.zero_()
+        step.run(fused=True)
+        check(ws[0], "fused inspection")
+    step.run(fused=False)
+    check(ws[0], "side-stream inspection")
+    step.stage(batch=1)
+    for i in (1, 2, 0):
+        step.stage(batch=(i + 1) % 3)
+        step.run(pipeline=True)
+        check(ws[i], f"staged batch {i}")
+    step.run(pipeline=True)
+    check(ws[1], "drained")
+
+
 def test_cfg3_scaled(oracle):
     w = synth.make_workload("cfg3_transr", batch=2048)
     a = w.arrays
