@@ -614,15 +614,21 @@ def run_workload(name, args, torch, factor_max=0):
     # per-kernel durations, live: an event behind every kernel, rotating batches; a spin kernel of
     # about 0.2 ms in front of each step lets the host enqueue the whole step before the device starts
     # it (no memory traffic: the caches hold what the timed loop's previous step left, as there)
+    # The timeline follows the issue that is reported: the staged issue launches other kernel forms than the
+    # direct one (no riding inspection, merged launches); its inspection runs on the side stream a batch
+    # ahead, so those entries (taken here in front of the step on one stream) are not part of the step.
+    kt_fused = False if issue == "staged" else None
     if hasattr(torch.cuda, "_sleep"):
         kt = step.kernel_times(steps=max(8, min(32, args.steps)), backward=do_bwd, batches=list(range(nb)),
-                               lead=lambda: torch.cuda._sleep(400_000))
+                               lead=lambda: torch.cuda._sleep(400_000), fused=kt_fused)
     else:
         lead = torch.empty(1024 * 1024, dtype=torch.float32, device=dev)
-        kt = step.kernel_times(steps=max(8, min(32, args.steps)), backward=do_bwd, batches=list(range(nb)), lead=lead)
+        kt = step.kernel_times(steps=max(8, min(32, args.steps)), backward=do_bwd, batches=list(range(nb)), lead=lead,
+                               fused=kt_fused)
         del lead
-    kt_sum = sum(ms_k for _, ms_k in kt)
-    kname, k_ms = max(kt, key=lambda x: x[1])
+    on_step = [(n_, m_) for n_, m_ in kt if not (issue == "staged" and n_.startswith("inspect"))]
+    kt_sum = sum(ms_k for _, ms_k in on_step)
+    kname, k_ms = max(on_step, key=lambda x: x[1])
     k_bytes, k_flops, k_unit = kernel_model(w, kname, u_ent, u_rel)
     bound = BOUND.get(name, "hbm")
     gbs = k_bytes / (k_ms * 1e-3) / 1e9
@@ -664,7 +670,8 @@ def run_workload(name, args, torch, factor_max=0):
                    "projection_gradients": (None if w.model not in ("TransR", "RESCAL") else
                                             {"factor_max": factor_max, "dense_groups": w.dense_rel,
                                              "factored_rows": w.factored_rows})},
-        "kernels_ms": [[n_, round(m_, 6)] for n_, m_ in kt],
+        "kernels_ms": [[n_ + (" (side stream, a batch ahead)" if (n_, m_) not in on_step else ""), round(m_, 6)]
+                       for n_, m_ in kt],
         "roofline": roofline,
         **check,
     }

@@ -581,7 +581,6 @@ struct PosBwdArgs {
     float *occ_w;          // [B, d] TransH
     int64_t B;
     int d, rel_dim;
-    ZeroRider zero;        // the segmented reduction's tickets, cleared here for the launch that follows
 };
 
 template <int V>
@@ -602,7 +601,6 @@ template <int MODEL, int P, int V, bool HEAD>
 __global__ __launch_bounds__(256) void bwd_pos_kernel(PosBwdArgs a, FusedInsp fi)
 {
     extern __shared__ __align__(16) char dyn_smem[];  // inspector workgroups only
-    zero_rider(a.zero);
     if (fused_insp_block(fi, reinterpret_cast<uint32_t *>(dyn_smem))) return;
     const int lane = threadIdx.x & (kWave - 1);
     const int64_t b = (int64_t)((int)blockIdx.x - fi.blocks) * 4 + (threadIdx.x >> 6);
@@ -840,8 +838,7 @@ __global__ void fill_zero_kernel(float *p, int64_t n)
 // ---------------------------------------------------------------------------------------
 struct BwdPlan {
     int64_t n_occ, nn;
-    size_t off_occ_e, off_occ_r, off_occ_w, off_g0, off_g1, off_part_e, off_part_r, off_part_w, off_tickets, total;
-    int64_t tick_e, tick_r, tick_w;  // ticket counters of the three reduction jobs
+    size_t off_occ_e, off_occ_r, off_occ_w, off_g0, off_g1, off_part_e, off_part_r, off_part_w, total;
 };
 
 static size_t up256(size_t x) { return (x + 255) & ~size_t(255); }
@@ -866,9 +863,6 @@ static BwdPlan make_bwd_plan(const kge_tables *tab, const kge_batch *bat)
     p.off_part_e = take(seg_partial_floats(p.n_occ, d));
     p.off_part_r = take(seg_partial_floats(B, rd));
     p.off_part_w = take(tab->model == KGE_TRANSH ? seg_partial_floats(B, d) : 0);
-    p.tick_e = seg_ticket_ints(p.n_occ, d), p.tick_r = rd > 0 ? seg_ticket_ints(B, rd) : 0;
-    p.tick_w = tab->model == KGE_TRANSH ? seg_ticket_ints(B, d) : 0;
-    p.off_tickets = take(p.tick_e + p.tick_r + p.tick_w);  // (int32 counters: same size as floats)
     p.total = o;
     return p;
 }
@@ -982,9 +976,7 @@ int kge_score_bwd(const kge_tables *tab, const kge_batch *bat, const kge_saved *
 
     PosBwdArgs pa{tab->ent, tab->rel, tab->aux, bat->h, bat->r, bat->t, dpos, saved->pos, saved->side_pos,
                   g0, g1, have_neg ? dneg : nullptr, bat->n_neg, occ_e, occ_e + B * d, occ_r, occ_w, B, (int)d,
-                  (int)tab->rel_dim, ZeroRider{}};
-    int32_t *tickets = reinterpret_cast<int32_t *>(ws + p.off_tickets);
-    pa.zero = ZeroRider{tickets, p.tick_e + p.tick_r + p.tick_w};
+                  (int)tab->rel_dim};
     switch (model) {
     case KGE_TRANSE:
         rc = P == 1 ? launch_pos_bwd<KGE_TRANSE, 1>(pa, vec, head, fi_dedup, st) : launch_pos_bwd<KGE_TRANSE, 2>(pa, vec, head, fi_dedup, st);
@@ -1003,13 +995,10 @@ int kge_score_bwd(const kge_tables *tab, const kge_batch *bat, const kge_saved *
 
     if (bat->insp_ready && hipStreamWaitEvent(st, reinterpret_cast<hipEvent_t>(bat->insp_ready), 0) != hipSuccess)
         return KGE_ELAUNCH;
-    // (the per-positive kernel above cleared the tickets: the reduction is one launch)
     const SegJob jobs[3] = {
-        {occ_e, bat->ent_insp, (int)d, grads->ent_rows, reinterpret_cast<float *>(ws + p.off_part_e), false, tickets},
-        {occ_r, bat->rel_insp, (int)tab->rel_dim, grads->rel_rows, reinterpret_cast<float *>(ws + p.off_part_r), false,
-         tickets + p.tick_e},
-        {occ_w, bat->rel_insp, (int)d, grads->aux_rows, reinterpret_cast<float *>(ws + p.off_part_w), false,
-         tickets + p.tick_e + p.tick_r}};
+        {occ_e, bat->ent_insp, (int)d, grads->ent_rows, reinterpret_cast<float *>(ws + p.off_part_e), false},
+        {occ_r, bat->rel_insp, (int)tab->rel_dim, grads->rel_rows, reinterpret_cast<float *>(ws + p.off_part_r), false},
+        {occ_w, bat->rel_insp, (int)d, grads->aux_rows, reinterpret_cast<float *>(ws + p.off_part_w), false}};
     return launch_seg_reduce_jobs(jobs, model == KGE_TRANSH ? 3 : 2, st, bat->timeline);
 }
 

@@ -6,13 +6,9 @@
 // the rows).  All its row loads are issued at once; then the positions are walked in order.
 // A run that lies wholly inside the block is final.  A run that began in an earlier block is
 // stored to partial slot 0 of the block, one that continues past the block to slot 1.
-// Level 2: a long run's slot-1 partial of the block it starts in and the slot-0 partials of the
-// following blocks are added up in block order.  With tickets (SegJob::tickets) this happens inside
-// the level-1 launch: every wave that stored a partial of the run counts itself in on the run's
-// ticket (release fence, integer atomic), and the wave that arrives last (it then sees every
-// partial: acquire fence) adds them up.  Nobody waits for anybody.  Without tickets a second launch does it (the block in which the
-// run starts; four waves share the following blocks, combined through LDS).
-// Either way the summation order is fixed by the sorted order, so results are deterministic.
+// Level 2: the block in which a long run STARTS adds that run's slot-1 partial and the slot-0
+// partials of the following blocks (four waves share the blocks, combined through LDS).
+// The summation order is fixed by the sorted order, so results are deterministic.
 #include "seg_reduce.hpp"
 
 namespace kge {
@@ -23,7 +19,6 @@ struct SegArgs {
     int64_t n;
     int d;
     float *out, *partial;
-    int32_t *tickets;                     // null: level 2 is a launch of its own
     const float *scale_num, *scale_den;   // row transform (SegJob), transform bit 0 = scaled, bit 1 = sign
     int transform;
 };
@@ -138,43 +133,6 @@ __global__ __launch_bounds__(256) void seg_reduce_l1(SegArgs3 jobs, SumRider rid
         }
     }
     flush(seg[cnt - 1]);
-
-    if (!a.tickets) return;
-    // Runs that cross a block boundary and that this block holds a part of: the one that comes in
-    // (it shares the first position's id) and the one that goes out (the last position's), the same
-    // run when the block lies inside it.  The ticket of a run sits with the block it starts in.
-    const int run_in = seg[0] == prev_id ? seg[0] : -1;
-    const int run_out = (seg[cnt - 1] == next_id && seg[cnt - 1] != run_in) ? seg[cnt - 1] : -1;
-    if (run_in < 0 && run_out < 0) return;
-    __threadfence();  // this wave's partial rows are visible to every other workgroup before it counts itself in
-#pragma unroll 1
-    for (int which = 0; which < 2; ++which) {
-        const int sg = which == 0 ? run_in : run_out;
-        if (sg < 0) continue;
-        const int s0 = a.seg_offsets[sg], s1 = a.seg_offsets[sg + 1];
-        const int64_t js = s0 / kSegL, je = (s1 - 1) / kSegL;
-        int32_t *ticket = a.tickets + js * nch + (w % nch);
-        int old = 0;
-        if (lane == 0) old = atomicAdd(ticket, 1);
-        old = __shfl(old, 0, kWave);
-        if (old != (int)(je - js)) continue;  // somebody else arrives after this wave
-        __threadfence();  // every other part of the run has been counted in: their rows are visible now
-        Vec<V> r = Vec<V>::load(a.partial + (js * 2 + 1) * (int64_t)d + cc);
-        constexpr int kFly = 16;  // partial rows in flight (the hottest row's chain is the long pole)
-        for (int64_t jj = js + 1; jj <= je; jj += kFly) {
-            Vec<V> t[kFly];
-#pragma unroll
-            for (int u = 0; u < kFly; ++u) t[u] = Vec<V>::load(a.partial + ((jj + u <= je ? jj + u : je) * 2) * (int64_t)d + cc);
-#pragma unroll
-            for (int u = 0; u < kFly; ++u)
-                if (jj + u <= je) {
-#pragma unroll
-                    for (int e = 0; e < V; ++e) r.v[e] += t[u].v[e];
-                }
-        }
-        if (active) r.store(a.out + (int64_t)sg * d + colv);
-        if (lane == 0) *ticket = 0;  // left as it was found
-    }
 }
 
 // One workgroup per (block, chunk of 64 V columns): the column chunks of a wide row are independent
@@ -241,19 +199,16 @@ int launch_seg_reduce_jobs(const SegJob *jobs, int n_jobs, hipStream_t st, kge_t
     SegArgs3 args{};
     int m = 0;
     int64_t max_waves = 0, max_blocks = 0, max_nch = 1;
-    bool v4 = true, one_launch = true;
+    bool v4 = true;
     for (int q = 0; q < n_jobs && m < 3; ++q) {
         const SegJob &jb = jobs[q];
         if (!jb.ins || jb.ins->n == 0 || jb.d == 0) continue;
         args.j[m] = SegArgs{jb.occ, jb.identity_perm ? nullptr : jb.ins->perm, jb.ins->sorted_seg,
-                            jb.ins->seg_offsets, jb.ins->n, jb.d, jb.out, jb.partial, jb.tickets,
+                            jb.ins->seg_offsets, jb.ins->n, jb.d, jb.out, jb.partial,
                             jb.scale_num, jb.scale_den, (jb.scaled ? 1 : 0) | (jb.sign_rows ? 2 : 0)};
         v4 = v4 && jb.d % 4 == 0 && aligned16(jb.occ) && aligned16(jb.out) && aligned16(jb.partial);
-        one_launch = one_launch && jb.tickets != nullptr;
         ++m;
     }
-    if (!one_launch)  // all jobs or none: the level-2 launch would redo what the tickets finished
-        for (int q = 0; q < m; ++q) args.j[q].tickets = nullptr;
     if (m == 0 && rd.max_sums == 0) return KGE_OK;
     for (int q = 0; q < m; ++q) {
         const int V = v4 ? 4 : 1;
@@ -267,7 +222,7 @@ int launch_seg_reduce_jobs(const SegJob *jobs, int n_jobs, hipStream_t st, kge_t
     int64_t g1x = ceil_div(max_waves, 4);
     if (rd.max_sums > 0 && g1x < 256) g1x = 256;  // (a small reduction still gives the rider a grid's worth of workgroups)
     const dim3 g1((unsigned)g1x, (unsigned)(m + (rd.max_sums > 0 ? 1 : 0))), g2((unsigned)(max_blocks * max_nch), (unsigned)m), block(256);
-    const bool level2 = m > 0 && !one_launch;
+    const bool level2 = m > 0;
     if (v4) {
         hipLaunchKernelGGL(seg_reduce_l1<4>, g1, block, 0, st, args, rd);
         timeline_mark(timeline, st, "seg_reduce_l1");

@@ -657,14 +657,16 @@ class TrainStep:
         if self._timeline is not None:
             _lib.check(self.L.kge_timeline_mark(self._timeline, self._LABELS[label], st), "kge_timeline_mark")
 
-    def kernel_times(self, steps: int = 10, backward: bool = True, batches=None, lead=None):
+    def kernel_times(self, steps: int = 10, backward: bool = True, batches=None, lead=None, fused=None):
         """[(kernel name, mean milliseconds)] of one step, in launch order: ``steps`` steps are run with an
         event recorded behind every kernel (kge_batch.timeline) and read back after each step.  Event
         records between the kernels cost a little themselves, so the sum is an upper bound of the
         step time that ``run()`` alone takes.  ``batches``: batch numbers to rotate over.  ``lead``: work
         enqueued on the stream in front of every step, so that the host has enqueued the whole step
         before the device starts on it and the intervals hold no launch gaps: a callable, or a large
-        tensor that is zero-filled (which also empties the caches in front of every step)."""
+        tensor that is zero-filled (which also empties the caches in front of every step).  ``fused``: as in
+        ``run()``; False times the launch forms of the staged issue (no riding inspection, merged launches) with
+        the inspection in front of the step on the same stream."""
         L = self.L
         tl = L.kge_timeline_create(64)
         if not tl:
@@ -685,7 +687,7 @@ class TrainStep:
                     lead.zero_()
                 _lib.check(L.kge_timeline_begin(tl, st), "kge_timeline_begin")
                 try:
-                    self.run(backward, overlap=False)
+                    self.run(backward, overlap=False, fused=fused)
                 finally:
                     self.bat.timeline = None
                 main.synchronize()
