@@ -22,7 +22,6 @@ namespace kge {
 typedef float floatx4 __attribute__((ext_vector_type(4)));
 
 constexpr int kTM = 32;          // triples per tile
-constexpr int kDmChunk = 256;    // triples of one relation group per dM work item
 #ifndef KGE_TR_RING
 #define KGE_TR_RING 3
 #endif
@@ -35,9 +34,12 @@ constexpr int kRing = KGE_TR_RING;  // supersteps of B operands kept in flight p
 #endif
 constexpr int kDmRing = KGE_TR_DM_RING;  // the same for the dM kernel's operand stages
 #ifndef KGE_TR_SPLIT_BWD
-#define KGE_TR_SPLIT_BWD 0
+#define KGE_TR_SPLIT_BWD 1
 #endif
-constexpr bool kSplitBwd = KGE_TR_SPLIT_BWD != 0;  // measurement builds: dX and dM always as two launches
+// dX and dM as two launches (default) or as one.  Measured on the TransR benchmark configuration, one box: two
+// launches 0.160 ms per step against 0.171 with every projection gradient dense; 0.151 against 0.150 with the
+// thin groups factored.
+constexpr bool kSplitBwd = KGE_TR_SPLIT_BWD != 0;
 constexpr int kThin = 4;            // a group's last tile with at most this many triples takes the thin path
 constexpr int kThinRing = 8;        // 128-bit projection loads in flight per thread on the thin path
 constexpr int kMaxDimMfma = 1024;
@@ -48,23 +50,13 @@ constexpr size_t kMaxGemmLds = 158 * 1024;
 
 int launch_score_pos(const kge_tables *, const kge_batch *, float *, float *, float *, hipStream_t);
 
-// ---- plans: the work items of a batch's relation groups, as compact lists ---------------------
-// The grouped kernels run as a fixed number of workgroups that stride over these lists
-// (kPersistWgs): how many items a batch has is only known on the device, and a grid sized for the
-// worst case (one tile per possible relation, seven row blocks per tile) launched ten thousand
-// workgroups that found out, after one to three dependent loads each, that they had nothing to do;
-// a workgroup lives for a few microseconds however little it does, and those held the slots.
+// ---- tile plan: one entry per (relation group, block of `tile` sorted positions) -----------
 struct TilePlan {
     int32_t *num_tiles;  // [1]
-    int32_t *num_thin;   // [1] entries of thin_g
-    int32_t *num_items;  // [2] chunked plan: long items (from the front of item_*), small-group items (from the back)
     int32_t *tile_seg;   // [max_tiles] group (unique-relation index)
     int32_t *tile_p0;    // [max_tiles] first sorted position
     int32_t *tile_end;   // [max_tiles] end of the tile's group in sorted positions (GEMM plan only, else null)
     int32_t *tile_rid;   // [max_tiles] relation id of the group (GEMM plan only, else null)
-    // GEMM plan: groups whose last tile has at most kThin rows (that tile is not in the tile list: a
-    // thin workgroup streams it); chunked plan: groups of at most kThin triples (they have no tiles)
-    int32_t *thin_g;     // [groups]
     // groups longer than one tile ("split" groups, used by the dM kernel): every tile of such
     // a group writes a partial result to slot tile_part[tile]; -1 for unsplit groups
     int32_t *tile_part;   // [max_tiles] or null
@@ -72,13 +64,7 @@ struct TilePlan {
     int32_t *split_seg;   // [max_split] group of the split
     int32_t *split_first; // [max_split] first partial slot
     int32_t *split_cnt;   // [max_split] number of partial slots
-    // chunked plan: work items of the dM kernel, (tile, 32-row block) or (tile, -1) = every row block of a
-    // small group by one workgroup
-    int32_t *item_tile, *item_blk;  // [max_items]
-    int max_items;
 };
-
-constexpr int kPersistWgs = 3 * 256;  // workgroups of a grouped launch: three per CU, what their registers allow
 
 // Inclusive scan over the 1024 threads of the block: shuffle scan inside each wave, then the 16
 // wave totals are scanned by every wave for itself (two barriers in all).
@@ -99,50 +85,38 @@ __device__ int block_inclusive_scan_1024(int v, int *s_scan)
     return v + before;
 }
 
-// One workgroup per plan: block 0 builds `plan0` (GEMM plan, tiles of `tile0` positions), block 1
-// (when launched) `plan1` (chunked plan of the dM kernel, chunks of `tile1` positions; `nib` row
-// blocks per chunk; groups of at most `small_max` triples become one item).
+// One workgroup per plan: block 0 builds `plan0` with tiles of `tile0` positions, block 1 (when
+// launched) `plan1` with `tile1`.
 __global__ __launch_bounds__(1024) void transr_plan_kernel(const int32_t *num_unique, const int32_t *seg_offsets,
                                                           const int64_t *unique_ids, TilePlan plan0, int tile0,
-                                                          TilePlan plan1, int tile1, int nib, int small_max)
+                                                          TilePlan plan1, int tile1)
 {
-    const bool chunked = blockIdx.x != 0;
-    const TilePlan &plan = chunked ? plan1 : plan0;
-    const int tile = chunked ? tile1 : tile0;
+    const TilePlan &plan = blockIdx.x == 0 ? plan0 : plan1;
+    const int tile = blockIdx.x == 0 ? tile0 : tile1;
     __shared__ int s_scan[1024];
-    __shared__ int s_carry[6];  // tiles, split slots, splits, thin groups, long items, small items
+    __shared__ int s_carry[3];
     const int U = num_unique[0];
-    if (threadIdx.x < 6) s_carry[threadIdx.x] = 0;
+    if (threadIdx.x < 3) s_carry[threadIdx.x] = 0;
     __syncthreads();
     for (int base = 0; base < U; base += 1024) {
         const int g = base + threadIdx.x;
-        int s0 = 0, s1 = 0, cnt = 0, rid = 0, thin = 0, n_long = 0, n_small = 0;
+        int s0 = 0, s1 = 0, cnt = 0, rid = 0;
         if (g < U) {
             s0 = seg_offsets[g], s1 = seg_offsets[g + 1];
             rid = (int)unique_ids[g];
-            const int n = s1 - s0;
-            cnt = (n + tile - 1) / tile;
-            if (chunked) {
-                thin = n <= kThin ? 1 : 0;
-                if (thin) cnt = 0;
-                else if (n <= small_max) n_small = 1;
-                else n_long = cnt * nib;
-            } else {
-                thin = (n - 1) % tile + 1 <= kThin ? 1 : 0;  // the last tile goes to a thin workgroup
-                cnt -= thin;
-            }
+            cnt = (s1 - s0 + tile - 1) / tile;
+            // the chunked plan of the dM kernel (the one with split bookkeeping) has no tiles for groups of
+            // at most kThin triples: thin workgroups write those, and a tile that only finds out that it has
+            // nothing to do holds a workgroup slot for three dependent loads
+            if (plan.tile_part && s1 - s0 <= kThin) cnt = 0;
         }
         const int inc_t = block_inclusive_scan_1024(cnt, s_scan);
         const int start = s_carry[0] + inc_t - cnt;
-        const int inc_th = block_inclusive_scan_1024(thin, s_scan);
-        if (thin) plan.thin_g[s_carry[3] + inc_th - 1] = g;
-        int pstart = -1, inc_p = 0, inc_s = 0, inc_l = 0, inc_m = 0;
-        if (chunked) {
+        int pstart = -1;
+        if (plan.tile_part) {
             const int pc = cnt > 1 ? cnt : 0, sg = cnt > 1 ? 1 : 0;
-            inc_p = block_inclusive_scan_1024(pc, s_scan);
-            inc_s = block_inclusive_scan_1024(sg, s_scan);
-            inc_l = block_inclusive_scan_1024(n_long, s_scan);
-            inc_m = block_inclusive_scan_1024(n_small, s_scan);
+            const int inc_p = block_inclusive_scan_1024(pc, s_scan);
+            const int inc_s = block_inclusive_scan_1024(sg, s_scan);
             if (sg) {
                 pstart = s_carry[1] + inc_p - pc;
                 const int si = s_carry[2] + inc_s - 1;
@@ -150,13 +124,8 @@ __global__ __launch_bounds__(1024) void transr_plan_kernel(const int32_t *num_un
                 plan.split_first[si] = pstart;
                 plan.split_cnt[si] = cnt;
             }
-            if (n_small) {  // from the back of the list
-                const int at = plan.max_items - 1 - (s_carry[5] + inc_m - 1);
-                plan.item_tile[at] = start, plan.item_blk[at] = -1;
-            }
-            int at = s_carry[4] + inc_l - n_long;
-            for (int q = 0; q < (n_long ? cnt : 0); ++q)
-                for (int ib = 0; ib < nib; ++ib, ++at) plan.item_tile[at] = start + q, plan.item_blk[at] = ib;
+            __syncthreads();
+            if (threadIdx.x == 1023) s_carry[1] += inc_p, s_carry[2] += inc_s;
         }
         for (int q = 0; q < cnt; ++q) {
             plan.tile_seg[start + q] = g;
@@ -165,17 +134,12 @@ __global__ __launch_bounds__(1024) void transr_plan_kernel(const int32_t *num_un
             if (plan.tile_part) plan.tile_part[start + q] = pstart >= 0 ? pstart + q : -1;
         }
         __syncthreads();
-        if (threadIdx.x == 1023) {
-            s_carry[0] += inc_t, s_carry[3] += inc_th;
-            s_carry[1] += inc_p, s_carry[2] += inc_s, s_carry[4] += inc_l, s_carry[5] += inc_m;
-        }
+        if (threadIdx.x == 1023) s_carry[0] += inc_t;
         __syncthreads();
     }
     if (threadIdx.x == 0) {
         plan.num_tiles[0] = s_carry[0];
-        plan.num_thin[0] = s_carry[3];
         if (plan.num_split) plan.num_split[0] = s_carry[2];
-        if (chunked) plan.num_items[0] = s_carry[4], plan.num_items[1] = s_carry[5];
     }
 }
 
@@ -234,6 +198,8 @@ struct GemmArgs {
     float *resid;     // forward: [B, d] rows y (nullable)
     float *occ_h, *occ_t;  // backward-dX: [B, d] each (occ_t nullable)
     int d, norm_p;
+    int thin_groups;       // upper bound of the number of relation groups = trailing thin workgroups
+    int max_tiles;         // leading workgroups: planned tiles
     BwdSrc src;            // TRANSPOSED pass without xs
 };
 
@@ -613,21 +579,25 @@ __device__ __forceinline__ void gemm_sweep(const BLoader<MODE> &bl, float4 (&rin
 // MODE 3: list rows        x = E[h]-E[t] (t = -1: no row), y = x M + rs R[r] -> resid rows in list order;
 //         h, t, rs are indexed by the sorted position itself (no perm), no score
 template <int MODE>
-__device__ __forceinline__ void transr_gemm_thin(const GemmArgs &a, float *lds, int g)
+__device__ __forceinline__ void transr_gemm_body(const GemmArgs &a, float *lds, int bid)
 {
-    if constexpr (MODE == 2) {
-        const int ns = (a.d / 4 + 15) / 16;  // k-quads per lane of a 16-lane row group
-        if (ns <= 1) transr_thin_dx_body<1>(a, lds, g);
-        else if (ns <= 2) transr_thin_dx_body<2>(a, lds, g);
-        else transr_thin_dx_body<4>(a, lds, g);
-    } else {
-        transr_thin_fwd_body<MODE>(a, lds, g);
+    // Workgroups [0, max_tiles) take the planned 32-triple tiles, the following `thin_groups`
+    // stream the thin group tails.  The tiles come first because each is one long chain of
+    // dependent loads and matrix-core steps (about 20 us whatever else runs); the thin
+    // workgroups then fill the remaining slots and the memory bandwidth.
+    if (bid >= a.max_tiles) {
+        if constexpr (MODE == 2) {
+            const int ns = (a.d / 4 + 15) / 16;  // k-quads per lane of a 16-lane row group
+            if (ns <= 1) transr_thin_dx_body<1>(a, lds, bid - a.max_tiles);
+            else if (ns <= 2) transr_thin_dx_body<2>(a, lds, bid - a.max_tiles);
+            else transr_thin_dx_body<4>(a, lds, bid - a.max_tiles);
+        } else {
+            transr_thin_fwd_body<MODE>(a, lds, bid - a.max_tiles);
+        }
+        return;
     }
-}
-
-template <int MODE>
-__device__ __forceinline__ void transr_gemm_tile(const GemmArgs &a, float *lds, int tile)
-{
+    const int tile = bid;
+    if (tile >= a.plan.num_tiles[0]) return;
     const int d = a.d;
     const int kpad = (d + 15) & ~15;
     const int pitch = kpad + 4;
@@ -638,6 +608,7 @@ __device__ __forceinline__ void transr_gemm_tile(const GemmArgs &a, float *lds, 
     const int p0 = a.plan.tile_p0[tile], seg_end = a.plan.tile_end[tile];
     const int64_t rid = a.plan.tile_rid[tile];
     const int rows = seg_end - p0 < kTM ? seg_end - p0 : kTM;
+    if (rows <= kThin) return;  // streamed by a thin workgroup
     const float *M = a.proj + rid * (int64_t)d * d;
     const int li = lane & 15, kk = lane >> 4;
 
@@ -836,27 +807,12 @@ __device__ __forceinline__ void transr_gemm_tile(const GemmArgs &a, float *lds, 
     }
 }
 
-// Item `it` of a grouped GEMM pass: the planned 32-triple tiles first (each is one long chain of dependent
-// loads and matrix-core steps, about 20 us whatever else runs), then the thin group tails, which fill
-// the remaining slots and the memory bandwidth.  False: past the end of the list.
-template <int MODE>
-__device__ __forceinline__ bool transr_gemm_item(const GemmArgs &a, float *lds, int it, int n_tiles, int n_thin)
-{
-    if (it < n_tiles) transr_gemm_tile<MODE>(a, lds, it);
-    else if (it < n_tiles + n_thin) transr_gemm_thin<MODE>(a, lds, a.plan.thin_g[it - n_tiles]);
-    else return false;
-    return true;
-}
-
 template <int MODE>
 __global__ __launch_bounds__(256, KGE_TR_OCC) void transr_gemm_kernel(GemmArgs a, FusedInsp fi)
 {
     extern __shared__ __align__(16) float lds[];
     if (fused_insp_block(fi, reinterpret_cast<uint32_t *>(lds))) return;  // an inspector workgroup riding along
-    const int n_tiles = a.plan.num_tiles[0], n_thin = a.plan.num_thin[0];
-    const int stride = (int)gridDim.x - fi.blocks;
-    for (int it = (int)blockIdx.x - fi.blocks; transr_gemm_item<MODE>(a, lds, it, n_tiles, n_thin); it += stride)
-        __syncthreads();  // the next item reuses the staging buffers
+    transr_gemm_body<MODE>(a, lds, (int)blockIdx.x - fi.blocks);
 }
 
 static size_t gemm_lds_bytes(int d)  // the larger of the tile layout and the thin layouts
@@ -867,22 +823,16 @@ static size_t gemm_lds_bytes(int d)  // the larger of the tile layout and the th
     return tile > thin ? tile : thin;
 }
 
-// Capacities of a plan's lists for `rows` sorted positions in at most `groups` relation groups (how many
-// entries a batch fills is only known on the device).
-struct PlanShape {
-    int64_t tiles, split, groups, items;
-};
-static PlanShape gemm_plan_shape(int64_t groups, int64_t rows) { return PlanShape{groups + rows / kTM + 1, 0, groups, 0}; }
-static PlanShape dm_plan_shape(int64_t groups, int64_t rows, int64_t d)
+static int thin_groups(const kge_tables *tab, const kge_batch *bat)
 {
-    const int64_t tiles = groups + rows / kDmChunk + 1;
-    return PlanShape{tiles, rows / kDmChunk + 1 /* a split group has more than kDmChunk rows */, groups, tiles * ceil_div(d, 32)};
+    return (int)(bat->batch < tab->n_rel ? bat->batch : tab->n_rel);
 }
-static int64_t dm_partial_slots(int64_t rows) { return 2 * (rows / kDmChunk) + 2; }  // sum over split groups of ceil(n_g / chunk)
-static int64_t group_cap(const kge_tables *tab, const kge_batch *bat) { return bat->batch < tab->n_rel ? bat->batch : tab->n_rel; }
 
-// workgroups of a grouped launch over a plan with these capacities
-static unsigned persist_grid(int64_t max_items) { return (unsigned)(max_items < kPersistWgs ? (max_items > 0 ? max_items : 1) : kPersistWgs); }
+static int64_t max_tiles(const kge_tables *tab, const kge_batch *bat)
+{
+    const int64_t groups = bat->batch < tab->n_rel ? bat->batch : tab->n_rel;
+    return groups + bat->batch / kTM + 1;
+}
 
 static bool mfma_path_ok(const kge_tables *tab, const kge_batch *bat)
 {
@@ -896,6 +846,7 @@ bool transr_grouped_path_ok(const kge_tables *tab, const kge_batch *bat)
 }
 
 // ---- backward kernels ----------------------------------------------------------------------
+constexpr int kDmChunk = 256;  // triples of one relation group per dM work item
 constexpr int kDmXP = 36;      // LDS pitch of a staged left-operand row (32 columns + 4: the four lane groups of an MFMA step read distinct banks)
 
 struct DmArgs {
@@ -906,6 +857,7 @@ struct DmArgs {
     float *part;     // [max_slots, d, d] partial results of split groups
     int d;
     const int32_t *num_unique;
+    int max_items;   // leading workgroups: (tile, 32-row block) items; the rest: one thin group each
     BwdSrc src;
     // Factored output (kge_grads.aux_x / aux_q): a group of at most factor_max (<= kThin) triples writes its
     // operand rows x_p, q_p to fx[p], fq[p] (p = its sorted positions) instead of the dense d x d sum of
@@ -1161,17 +1113,27 @@ __device__ __forceinline__ void transr_dm_small_body(const DmArgs &a, float *lds
 // folded in), the four waves split the columns j and K runs over the chunk's triples.  Groups longer
 // than one chunk write per-chunk partial matrices that are added up beside the segmented reduction
 // (keeps the longest K loop at 16 supersteps).
-__device__ __forceinline__ void transr_dm_item(const DmArgs &a, float *lds, int tile, int blk)
+__device__ __forceinline__ void transr_dm_body(const DmArgs &a, float *lds, int bid)
 {
+    if (bid >= a.max_items) {
+        transr_thin_dm_body(a, lds, bid - a.max_items);
+        return;
+    }
     const int d = a.d;
-    const int i0 = blk * 32;
+    const int nib = (d + 31) / 32;
+    const int tile = bid / nib;
+    if (tile >= a.plan.num_tiles[0]) return;
+    const int i0 = (bid % nib) * 32;
     const int g = a.plan.tile_seg[tile];
     const int s0 = a.plan.tile_p0[tile];
     const int seg_end = a.seg_offsets[g + 1];
-    if (blk < 0) {  // a small group, whole, by this workgroup
+    const int gn = seg_end - a.seg_offsets[g];
+    if (gn <= kThin) return;  // written by a thin workgroup
+    if (gn <= kDmSmall && dm_small_fits(d)) {  // the whole group by the workgroup of its first row block
+        if (i0 != 0) return;
         float *whole = a.dm + (int64_t)g * d * d;
-        if (a.xs == nullptr && !a.src.rescal && a.src.norm_p == 1) transr_dm_small_body<true>(a, lds, s0, seg_end - s0, whole);
-        else transr_dm_small_body<false>(a, lds, s0, seg_end - s0, whole);
+        if (a.xs == nullptr && !a.src.rescal && a.src.norm_p == 1) transr_dm_small_body<true>(a, lds, s0, gn, whole);
+        else transr_dm_small_body<false>(a, lds, s0, gn, whole);
         return;
     }
     const int s1 = s0 + kDmChunk < seg_end ? s0 + kDmChunk : seg_end;
@@ -1265,24 +1227,11 @@ static size_t dm_lds_bytes(int d)  // the staged left operand and its row offset
     return item > thin ? item : thin;
 }
 
-// Item `it` of a dM pass: the (chunk, row block) items of the larger groups first (the long chains), the
-// small groups, then the thin ones.  False: past the end of the list.
-__device__ __forceinline__ bool transr_dm_work(const DmArgs &a, float *lds, int it, int n_long, int n_small, int n_thin)
-{
-    if (it < n_long) transr_dm_item(a, lds, a.plan.item_tile[it], a.plan.item_blk[it]);
-    else if (it < n_long + n_small) transr_dm_item(a, lds, a.plan.item_tile[a.plan.max_items - 1 - (it - n_long)], -1);
-    else if (it < n_long + n_small + n_thin) transr_thin_dm_body(a, lds, a.plan.thin_g[it - n_long - n_small]);
-    else return false;
-    return true;
-}
-
 __global__ __launch_bounds__(256, KGE_TR_OCC) void transr_dm_kernel(DmArgs a, FusedInsp fi)
 {
     extern __shared__ __align__(16) float lds[];  // dm_lds_bytes(); inspector workgroups: their own need
     if (fused_insp_block(fi, reinterpret_cast<uint32_t *>(lds))) return;
-    const int n_long = a.plan.num_items[0], n_small = a.plan.num_items[1], n_thin = a.plan.num_thin[0];
-    const int stride = (int)gridDim.x - fi.blocks;
-    for (int it = (int)blockIdx.x - fi.blocks; transr_dm_work(a, lds, it, n_long, n_small, n_thin); it += stride) __syncthreads();
+    transr_dm_body(a, lds, (int)blockIdx.x - fi.blocks);
 }
 
 // An inspector step that rides with nothing: the fused entity inspection of a TransR / RESCAL step has
@@ -1294,20 +1243,21 @@ __global__ __launch_bounds__(256) void transr_insp_step_kernel(FusedInsp fi)
 }
 
 // dX and dM of one backward pass in ONE launch (no inspector riders): the two are independent, one
-// streams the projections in while the other streams the projection gradients out.  One list: the dX
-// tiles, the dM items of the larger groups, the small groups' dM, then the thin groups of dX and of dM.
+// streams the projections in while the other streams the projection gradients out, and either alone
+// leaves the memory system waiting on its dependent chains.  Order of the workgroups: the dX tiles,
+// the dM work items, then the thin groups of both in alternation.
 __global__ __launch_bounds__(256, KGE_TR_OCC) void transr_dx_dm_kernel(GemmArgs ga, DmArgs da)
 {
     extern __shared__ __align__(16) float lds[];
-    const int nt = ga.plan.num_tiles[0], nth = ga.plan.num_thin[0];
-    const int nl = da.plan.num_items[0], ns = da.plan.num_items[1], ndt = da.plan.num_thin[0];
-    const int total = nt + nl + ns + nth + ndt;
-    for (int it = (int)blockIdx.x; it < total; it += (int)gridDim.x) {
-        if (it < nt) transr_gemm_tile<2>(ga, lds, it);
-        else if (it < nt + nl + ns) (void)transr_dm_work(da, lds, it - nt, nl, ns, 0);
-        else if (it < nt + nl + ns + nth) transr_gemm_thin<2>(ga, lds, ga.plan.thin_g[it - nt - nl - ns]);
-        else transr_thin_dm_body(da, lds, da.plan.thin_g[it - nt - nl - ns - nth]);
-        __syncthreads();
+    const int bid = (int)blockIdx.x;
+    if (bid < ga.max_tiles) {
+        transr_gemm_body<2>(ga, lds, bid);
+    } else if (bid < ga.max_tiles + da.max_items) {
+        transr_dm_body(da, lds, bid - ga.max_tiles);
+    } else {
+        const int q = bid - ga.max_tiles - da.max_items;
+        if (q & 1) transr_dm_body(da, lds, da.max_items + (q >> 1));
+        else transr_gemm_body<2>(ga, lds, ga.max_tiles + (q >> 1));
     }
 }
 
@@ -1328,22 +1278,23 @@ static size_t up256(size_t x) { return (x + 255) & ~size_t(255); }
 
 struct RPlan {
     size_t off_plan, off_dplan, off_occ, off_part_e, off_part_r, off_dpart, total;
-    PlanShape gs, ds;
-    int64_t dslots;
+    int64_t tiles, dtiles, dsplit, dslots;
 };
 
-static size_t plan_ints(const PlanShape &s) { return (size_t)(64 + 5 * s.tiles + 3 * s.split + s.groups + 2 * s.items + 8); }
+static size_t plan_ints(int64_t tiles, int64_t split) { return (size_t)(64 + 5 * tiles + 3 * split + 8); }
 
 static RPlan make_rplan(const kge_tables *tab, const kge_batch *bat)
 {
     RPlan p{};
     const int64_t B = bat->batch, d = tab->dim;
-    p.gs = gemm_plan_shape(group_cap(tab, bat), B);
-    p.ds = dm_plan_shape(group_cap(tab, bat), B, d);
-    p.dslots = dm_partial_slots(B);
+    const int64_t groups = B < tab->n_rel ? B : tab->n_rel;
+    p.tiles = max_tiles(tab, bat);
+    p.dtiles = groups + B / kDmChunk + 1;
+    p.dsplit = B / kDmChunk + 1;            // a split group has more than kDmChunk triples
+    p.dslots = 2 * (B / kDmChunk) + 2;      // sum over split groups of ceil(n_g / chunk)
     size_t o = 0;
-    p.off_plan = o, o += up256(sizeof(int32_t) * plan_ints(p.gs));
-    p.off_dplan = o, o += up256(sizeof(int32_t) * plan_ints(p.ds));
+    p.off_plan = o, o += up256(sizeof(int32_t) * plan_ints(p.tiles, 0));
+    p.off_dplan = o, o += up256(sizeof(int32_t) * plan_ints(p.dtiles, p.dsplit));
     p.off_occ = o, o += up256(sizeof(float) * (size_t)(2 * B * d));
     p.off_part_e = o, o += up256(sizeof(float) * (size_t)seg_partial_floats(2 * B, d));
     p.off_part_r = o, o += up256(sizeof(float) * (size_t)seg_partial_floats(B, d));
@@ -1352,49 +1303,35 @@ static RPlan make_rplan(const kge_tables *tab, const kge_batch *bat)
     return p;
 }
 
-static TilePlan plan_at(void *base, const PlanShape &sh)
+static TilePlan plan_at(void *base, int64_t tiles, int64_t split)
 {
     int32_t *q = static_cast<int32_t *>(base);
-    TilePlan p{};
-    p.num_tiles = q, p.num_thin = q + 1, p.num_items = q + 2;
-    p.tile_seg = q + 64, p.tile_p0 = q + 64 + sh.tiles;
-    if (sh.split > 0) {
-        p.tile_part = q + 64 + 2 * sh.tiles;
+    TilePlan p{q, q + 64, q + 64 + tiles, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr};
+    if (split > 0) {
+        p.tile_part = q + 64 + 2 * tiles;
         p.num_split = q + 32;
-        p.split_seg = q + 64 + 5 * sh.tiles;
-        p.split_first = p.split_seg + sh.split;
-        p.split_cnt = p.split_first + sh.split;
+        p.split_seg = q + 64 + 5 * tiles;
+        p.split_first = p.split_seg + split;
+        p.split_cnt = p.split_first + split;
     } else {
-        p.tile_end = q + 64 + 3 * sh.tiles;
-        p.tile_rid = q + 64 + 4 * sh.tiles;
+        p.tile_end = q + 64 + 3 * tiles;
+        p.tile_rid = q + 64 + 4 * tiles;
     }
-    p.thin_g = q + 64 + 5 * sh.tiles + 3 * sh.split;
-    p.item_tile = p.thin_g + sh.groups;
-    p.item_blk = p.item_tile + sh.items;
-    p.max_items = (int)sh.items;
     return p;
 }
 
-// Builds both plans of a set of relation groups (sorted positions delimited by seg_offsets).
-static void launch_plans(const int32_t *num_unique, const int32_t *seg_offsets, const int64_t *unique_ids, const TilePlan &plan,
-                         const TilePlan &dplan, int d, hipStream_t st)
-{
-    hipLaunchKernelGGL(transr_plan_kernel, dim3(2), dim3(1024), 0, st, num_unique, seg_offsets, unique_ids, plan, kTM, dplan, kDmChunk,
-                       (int)ceil_div(d, 32), dm_small_fits(d) ? kDmSmall : 0);
-}
-
-// The forward workspace holds both plans of the batch: the 32-triple tiles of the GEMM kernels
+// The forward workspace holds both tile plans of the batch: the 32-triple tiles of the GEMM kernels
 // and the chunked plan of the dM kernel.  A backward pass that is handed this workspace
 // (kge_saved.fwd_workspace) finds its plans there and launches no plan kernel of its own.
 static size_t fwd_plan_bytes(const kge_tables *tab, const kge_batch *bat)
 {
-    return up256(sizeof(int32_t) * plan_ints(gemm_plan_shape(group_cap(tab, bat), bat->batch)));
+    return up256(sizeof(int32_t) * plan_ints(max_tiles(tab, bat), 0));
 }
 
 size_t transr_fwd_workspace(const kge_tables *tab, const kge_batch *bat)
 {
     const RPlan p = make_rplan(tab, bat);
-    return fwd_plan_bytes(tab, bat) + up256(sizeof(int32_t) * plan_ints(p.ds));
+    return fwd_plan_bytes(tab, bat) + up256(sizeof(int32_t) * plan_ints(p.dtiles, p.dsplit));
 }
 
 // A launch with more than 64 KB of dynamic LDS has to be allowed per kernel first.
@@ -1433,14 +1370,18 @@ int launch_transr_fwd(const kge_tables *tab, const kge_batch *bat, float *pos, f
         return rc;
     }
     const kge_inspection *ri = bat->rel_insp;
+    const int64_t tiles = max_tiles(tab, bat);
+    TilePlan plan = plan_at(workspace, tiles, 0);
     const RPlan rp = make_rplan(tab, bat);
-    TilePlan plan = plan_at(workspace, rp.gs);
-    TilePlan dplan = plan_at(static_cast<char *>(workspace) + fwd_plan_bytes(tab, bat), rp.ds);
-    if (!bat->plans_ready) launch_plans(ri->num_unique, ri->seg_offsets, ri->unique_ids, plan, dplan, (int)tab->dim, st);
+    TilePlan dplan = plan_at(static_cast<char *>(workspace) + fwd_plan_bytes(tab, bat), rp.dtiles, rp.dsplit);
+    if (!bat->plans_ready)
+        hipLaunchKernelGGL(transr_plan_kernel, dim3(2), dim3(1024), 0, st, ri->num_unique, ri->seg_offsets, ri->unique_ids, plan,
+                           kTM, dplan, kDmChunk);
     GemmArgs a{tab->ent, tab->rel, tab->aux, bat->h, bat->r, bat->t, ri->perm, ri->seg_offsets, ri->num_unique, ri->unique_ids,
-               plan, nullptr, nullptr, pos, resid, nullptr, nullptr, (int)tab->dim, tab->norm_p, BwdSrc{}};
+               plan, nullptr, nullptr, pos, resid, nullptr, nullptr, (int)tab->dim, tab->norm_p, thin_groups(tab, bat), (int)tiles,
+               BwdSrc{}};
     const size_t lds = lds_with(fi, gemm_lds_bytes((int)tab->dim));
-    const dim3 grid(persist_grid(rp.gs.tiles + rp.gs.groups) + fi.blocks);
+    const dim3 grid((unsigned)(tiles + a.thin_groups + fi.blocks));
     if (const int rc = rescal ? allow_lds<1>(lds) : allow_lds<0>(lds)) return rc;
     if (rescal)
         hipLaunchKernelGGL(transr_gemm_kernel<1>, grid, dim3(256), lds, st, a, fi);
@@ -1460,9 +1401,10 @@ int launch_transr_plan(const kge_tables *tab, const kge_batch *bat, void *worksp
     if (!workspace || workspace_bytes < transr_fwd_workspace(tab, bat)) return KGE_EWORKSPACE;
     const kge_inspection *ri = bat->rel_insp;
     const RPlan rp = make_rplan(tab, bat);
-    TilePlan plan = plan_at(workspace, rp.gs);
-    TilePlan dplan = plan_at(static_cast<char *>(workspace) + fwd_plan_bytes(tab, bat), rp.ds);
-    launch_plans(ri->num_unique, ri->seg_offsets, ri->unique_ids, plan, dplan, (int)tab->dim, st);
+    TilePlan plan = plan_at(workspace, max_tiles(tab, bat), 0);
+    TilePlan dplan = plan_at(static_cast<char *>(workspace) + fwd_plan_bytes(tab, bat), rp.dtiles, rp.dsplit);
+    hipLaunchKernelGGL(transr_plan_kernel, dim3(2), dim3(1024), 0, st, ri->num_unique, ri->seg_offsets, ri->unique_ids, plan, kTM,
+                       dplan, kDmChunk);
     KGE_CHECK_LAUNCH();
     return KGE_OK;
 }
@@ -1493,8 +1435,9 @@ int launch_transr_bwd(const kge_tables *tab, const kge_batch *bat, const kge_sav
     // the plans: left behind by the forward pass, or built here
     const bool have_plans = saved->fwd_workspace && saved->fwd_workspace_bytes >= transr_fwd_workspace(tab, bat);
     char *pbase = have_plans ? static_cast<char *>(const_cast<void *>(saved->fwd_workspace)) : nullptr;
-    TilePlan plan = have_plans ? plan_at(pbase, p.gs) : plan_at(ws + p.off_plan, p.gs);
-    TilePlan dplan = have_plans ? plan_at(pbase + fwd_plan_bytes(tab, bat), p.ds) : plan_at(ws + p.off_dplan, p.ds);
+    TilePlan plan = have_plans ? plan_at(pbase, p.tiles, 0) : plan_at(ws + p.off_plan, p.tiles, 0);
+    TilePlan dplan = have_plans ? plan_at(pbase + fwd_plan_bytes(tab, bat), p.dtiles, p.dsplit)
+                                : plan_at(ws + p.off_dplan, p.dtiles, p.dsplit);
 
     // fused entity inspection (its histogram rode with the forward GEMM): first digit pass in a launch
     // of its own, second with the dX GEMM, dedup with dM
@@ -1505,37 +1448,41 @@ int launch_transr_bwd(const kge_tables *tab, const kge_batch *bat, const kge_sav
         if ((rc = plan_fused_inspection(bat->insp_jobs, 1, 1, &f1))) return rc;
         if ((rc = plan_fused_inspection(bat->insp_jobs, 1, 2, &f2))) return rc;
         if ((rc = plan_fused_inspection(bat->insp_jobs, 1, 3, &f3))) return rc;
-        if (f1.blocks > 0) hipLaunchKernelGGL(transr_insp_step_kernel, dim3((unsigned)f1.blocks), dim3(256), lds_with(f1, 0), st, f1);
+        hipLaunchKernelGGL(transr_insp_step_kernel, dim3((unsigned)f1.blocks), dim3(256), lds_with(f1, 0), st, f1);
         timeline_mark(bat->timeline, st, "inspector step");
     }
-    if (!have_plans) launch_plans(ri->num_unique, ri->seg_offsets, ri->unique_ids, plan, dplan, d, st);
+    if (!have_plans)
+        hipLaunchKernelGGL(transr_plan_kernel, dim3(2), dim3(1024), 0, st, ri->num_unique, ri->seg_offsets, ri->unique_ids, plan, kTM,
+                           dplan, kDmChunk);
     // Upstream rows q and left operands x are formed inside the two kernels from the forward pass's rows
     // (BwdSrc); RESCAL's tail occurrence rows g * v come out of the dX kernel's staging.
     const BwdSrc src{tab->ent, saved->residual, dpos, saved->pos, bat->h, bat->t, ri->perm, tab->norm_p, rescal ? 1 : 0,
                      rescal ? occ + B * d : nullptr};
     // dX = Q M^T -> occurrence rows of h (and -dX for t)
     GemmArgs ga{tab->ent, tab->rel, tab->aux, bat->h, bat->r, bat->t, ri->perm, ri->seg_offsets, ri->num_unique, ri->unique_ids,
-                plan, nullptr, nullptr, nullptr, nullptr, occ, rescal ? nullptr : occ + B * d, d, tab->norm_p, src};
+                plan, nullptr, nullptr, nullptr, nullptr, occ, rescal ? nullptr : occ + B * d, d, tab->norm_p, thin_groups(tab, bat),
+                (int)p.tiles, src};
     // dM = X^T Q per relation group
+    const int dm_items = (int)(ceil_div(d, 32) * p.dtiles);
     DmArgs da{nullptr, nullptr, ri->seg_offsets, dplan, grads->aux_rows, reinterpret_cast<float *>(ws + p.off_dpart), d,
-              ri->num_unique, src, factored ? grads->aux_x : nullptr, factored ? grads->aux_q : nullptr,
+              ri->num_unique, dm_items, src, factored ? grads->aux_x : nullptr, factored ? grads->aux_q : nullptr,
               grads->aux_factor_max};
-    const int64_t dx_cap = p.gs.tiles + p.gs.groups, dm_cap = p.ds.items + p.ds.groups;
-    if (!bat->fuse_inspection && !kSplitBwd) {  // nothing rides along: both in one launch
+    if (!bat->fuse_inspection && !kSplitBwd) {  // both in one launch
         const size_t lds = gemm_lds_bytes(d) > dm_lds_bytes(d) ? gemm_lds_bytes(d) : dm_lds_bytes(d);
         if (lds > 64 * 1024 &&
             hipFuncSetAttribute(reinterpret_cast<const void *>(&transr_dx_dm_kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
                                 (int)kMaxGemmLds) != hipSuccess)
             return KGE_ELAUNCH;
-        hipLaunchKernelGGL(transr_dx_dm_kernel, dim3(persist_grid(dx_cap + dm_cap)), dim3(256), lds, st, ga, da);
+        hipLaunchKernelGGL(transr_dx_dm_kernel, dim3((unsigned)(p.tiles + dm_items + 2 * ga.thin_groups)), dim3(256), lds, st, ga,
+                           da);
         timeline_mark(bat->timeline, st, "transr_dx_dm_kernel");
     } else {
         if (const int rc = allow_lds<2>(lds_with(f2, gemm_lds_bytes(d)))) return rc;
-        hipLaunchKernelGGL(transr_gemm_kernel<2>, dim3(persist_grid(dx_cap) + f2.blocks), dim3(256),
+        hipLaunchKernelGGL(transr_gemm_kernel<2>, dim3((unsigned)(p.tiles + ga.thin_groups + f2.blocks)), dim3(256),
                            lds_with(f2, gemm_lds_bytes(d)), st, ga, f2);
         timeline_mark(bat->timeline, st, "transr_gemm_kernel<dX>");
-        hipLaunchKernelGGL(transr_dm_kernel, dim3(persist_grid(dm_cap) + f3.blocks), dim3(256), lds_with(f3, dm_lds_bytes(d)), st,
-                           da, f3);
+        hipLaunchKernelGGL(transr_dm_kernel, dim3((unsigned)(dm_items + thin_groups(tab, bat) + f3.blocks)), dim3(256),
+                           lds_with(f3, dm_lds_bytes(d)), st, da, f3);
         timeline_mark(bat->timeline, st, "transr_dm_kernel");
     }
     KGE_CHECK_LAUNCH();
@@ -1547,7 +1494,7 @@ int launch_transr_bwd(const kge_tables *tab, const kge_batch *bat, const kge_sav
                       {saved->residual, ri, d, grads->rel_rows, reinterpret_cast<float *>(ws + p.off_part_r), false}};
     jobs[1].scaled = true, jobs[1].sign_rows = tab->norm_p == 1;
     jobs[1].scale_num = dpos, jobs[1].scale_den = tab->norm_p == 2 ? saved->pos : nullptr;
-    const SumRider finish = dm_finish_rider(da, p.ds.split);
+    const SumRider finish = dm_finish_rider(da, p.dsplit);
     return launch_seg_reduce_jobs(jobs, rescal ? 1 : 2, st, bat->timeline, &finish);
 }
 

@@ -22,8 +22,7 @@ constexpr int kNegSeg = 8;  // sorted positions per wave of the P-row gradient s
 
 struct NegShape {
     int64_t B, N, C, n_chunks, NN, d, U_cap, G_cap, L_cap;
-    PlanShape gs, ds;
-    int64_t dslots;
+    int64_t tiles, dtiles, dsplit, dslots;
 };
 
 static NegShape neg_shape(const kge_tables *tab, const kge_batch *bat)
@@ -36,9 +35,10 @@ static NegShape neg_shape(const kge_tables *tab, const kge_batch *bat)
     const int64_t pairs = tab->n_rel * s.n_chunks;
     s.G_cap = s.B < pairs ? s.B : pairs;
     s.L_cap = 2 * s.B + s.G_cap * s.N;
-    s.gs = gemm_plan_shape(s.U_cap, s.L_cap);
-    s.ds = dm_plan_shape(s.U_cap, s.L_cap, s.d);
-    s.dslots = dm_partial_slots(s.L_cap);
+    s.tiles = s.U_cap + s.L_cap / kTM + 1;
+    s.dtiles = s.U_cap + s.L_cap / kDmChunk + 1;
+    s.dsplit = s.L_cap / kDmChunk + 1;
+    s.dslots = 2 * (s.L_cap / kDmChunk) + 2;
     return s;
 }
 
@@ -75,8 +75,8 @@ static NegFwdLayout neg_fwd_layout(const kge_tables *tab, const NegShape &s)
     l.hl = take(sizeof(int64_t) * s.L_cap);
     l.tl = take(sizeof(int64_t) * s.L_cap);
     l.rsl = take(sizeof(float) * s.L_cap);
-    l.plan = take(sizeof(int32_t) * plan_ints(s.gs));
-    l.dplan = take(sizeof(int32_t) * plan_ints(s.ds));
+    l.plan = take(sizeof(int32_t) * plan_ints(s.tiles, 0));
+    l.dplan = take(sizeof(int32_t) * plan_ints(s.dtiles, s.dsplit));
     l.y = take(sizeof(float) * (size_t)(s.L_cap * s.d));
     l.total = o;
     return l;
@@ -665,17 +665,18 @@ int launch_transr_neg_fwd(const kge_tables *tab, const kge_batch *bat, float *po
     const int64_t list_threads = s.B + s.G_cap * s.N;
     const int64_t list_blocks = ceil_div(list_threads, 256);
     hipLaunchKernelGGL(tneg_list_kernel, dim3((unsigned)(list_blocks < 8192 ? list_blocks : 8192)), dim3(256), 0, st, x);
-    TilePlan plan = plan_at(ws + l.plan, s.gs), dplan = plan_at(ws + l.dplan, s.ds);
-    launch_plans(ri->num_unique, x.segl, ri->unique_ids, plan, dplan, d, st);
+    TilePlan plan = plan_at(ws + l.plan, s.tiles, 0), dplan = plan_at(ws + l.dplan, s.dtiles, s.dsplit);
+    hipLaunchKernelGGL(transr_plan_kernel, dim3(2), dim3(1024), 0, st, ri->num_unique, x.segl, ri->unique_ids, plan, kTM, dplan,
+                       kDmChunk);
     timeline_mark(bat->timeline, st, "row list + transr_plan_kernel");
 
     // one grouped pass projects every list row
     float *y = reinterpret_cast<float *>(ws + l.y);
     GemmArgs ga{tab->ent, tab->rel, tab->aux, x.hl, nullptr, x.tl, nullptr, x.segl, ri->num_unique, ri->unique_ids,
-                plan, nullptr, x.rsl, nullptr, y, nullptr, nullptr, d, tab->norm_p, BwdSrc{}};
+                plan, nullptr, x.rsl, nullptr, y, nullptr, nullptr, d, tab->norm_p, (int)s.U_cap, (int)s.tiles, BwdSrc{}};
     const size_t lds = gemm_lds_bytes(d);
     if (const int rc = allow_lds<3>(lds)) return rc;
-    hipLaunchKernelGGL(transr_gemm_kernel<3>, dim3(persist_grid(s.gs.tiles + s.gs.groups)), dim3(256), lds, st, ga, FusedInsp{});
+    hipLaunchKernelGGL(transr_gemm_kernel<3>, dim3((unsigned)(s.tiles + s.U_cap)), dim3(256), lds, st, ga, FusedInsp{});
     timeline_mark(bat->timeline, st, "transr_gemm_kernel<list>");
 
     NegPairArgs pa{};
@@ -712,7 +713,7 @@ int launch_transr_neg_bwd(const kge_tables *tab, const kge_batch *bat, const kge
     float *dxl = reinterpret_cast<float *>(ws + l.dxl), *occ = reinterpret_cast<float *>(ws + l.occ);
     float *qr = reinterpret_cast<float *>(ws + l.qr);
     int32_t *glist = reinterpret_cast<int32_t *>(ws + l.glist), *gcount = reinterpret_cast<int32_t *>(ws + l.gcount);
-    TilePlan plan = plan_at(fws + fl.plan, s.gs), dplan = plan_at(fws + fl.dplan, s.ds);
+    TilePlan plan = plan_at(fws + fl.plan, s.tiles, 0), dplan = plan_at(fws + fl.dplan, s.dtiles, s.dsplit);
 
     NegPairArgs pa{};
     pa.ent = tab->ent, pa.y = y, pa.dpos = dpos, pa.dneg = dneg, pa.spos = saved->pos, pa.sneg = saved->neg;
@@ -730,14 +731,15 @@ int launch_transr_neg_bwd(const kge_tables *tab, const kge_batch *bat, const kge
 
     // dX = Q M^T over the list (rows stay in list order), dM = X^T Q per relation
     GemmArgs ga{tab->ent, tab->rel, tab->aux, x.hl, nullptr, x.tl, nullptr, x.segl, ri->num_unique, ri->unique_ids,
-                plan, ql, nullptr, nullptr, nullptr, dxl, nullptr, d, tab->norm_p, BwdSrc{}};
+                plan, ql, nullptr, nullptr, nullptr, dxl, nullptr, d, tab->norm_p, (int)s.U_cap, (int)s.tiles, BwdSrc{}};
     const size_t lds = gemm_lds_bytes(d);
     if (const int rc = allow_lds<2>(lds)) return rc;
-    hipLaunchKernelGGL(transr_gemm_kernel<2>, dim3(persist_grid(s.gs.tiles + s.gs.groups)), dim3(256), lds, st, ga, FusedInsp{});
+    hipLaunchKernelGGL(transr_gemm_kernel<2>, dim3((unsigned)(s.tiles + s.U_cap)), dim3(256), lds, st, ga, FusedInsp{});
     timeline_mark(bat->timeline, st, "transr_gemm_kernel<dX>");
-    DmArgs da{xl, ql, x.segl, dplan, grads->aux_rows, reinterpret_cast<float *>(ws + l.dpart), d, ri->num_unique, BwdSrc{},
-              nullptr, nullptr, 0};
-    hipLaunchKernelGGL(transr_dm_kernel, dim3(persist_grid(s.ds.items + s.ds.groups)), dim3(256), dm_lds_bytes(d), st, da, FusedInsp{});
+    const int dm_items = (int)(ceil_div(d, 32) * s.dtiles);
+    DmArgs da{xl, ql, x.segl, dplan, grads->aux_rows, reinterpret_cast<float *>(ws + l.dpart), d, ri->num_unique, dm_items,
+              BwdSrc{}, nullptr, nullptr, 0};
+    hipLaunchKernelGGL(transr_dm_kernel, dim3((unsigned)(dm_items + s.U_cap)), dim3(256), dm_lds_bytes(d), st, da, FusedInsp{});
     timeline_mark(bat->timeline, st, "transr_dm_kernel");
     TNEG_BY_WIDTH(d, hipLaunchKernelGGL(tneg_occ_kernel<NQ_>, dim3((unsigned)(ceil_div(s.B, 4) + s.NN)), dim3(256), 0, st, x, dxl,
                                         glist, gcount, occ));
@@ -747,6 +749,6 @@ int launch_transr_neg_bwd(const kge_tables *tab, const kge_batch *bat, const kge
         return KGE_ELAUNCH;
     const SegJob jobs[2] = {{occ, bat->ent_insp, d, grads->ent_rows, reinterpret_cast<float *>(ws + l.part_e), false},
                             {qr, ri, d, grads->rel_rows, reinterpret_cast<float *>(ws + l.part_r), false}};
-    const SumRider finish = dm_finish_rider(da, s.ds.split);  // the split groups' partial matrices
+    const SumRider finish = dm_finish_rider(da, s.dsplit);  // the split groups' partial matrices
     return launch_seg_reduce_jobs(jobs, 2, st, bat->timeline, &finish);
 }
