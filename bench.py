@@ -617,7 +617,7 @@ def run_workload(name, args, torch, factor_max=0):
     # The timeline follows the issue that is reported: the staged issue launches other kernel forms than the
     # direct one (no riding inspection, merged launches); its inspection runs on the side stream a batch
     # ahead, so those entries (taken here in front of the step on one stream) are not part of the step.
-    kt_fused = False if issue == "staged" else None
+    kt_fused = False if issue.startswith("staged") else None
     if hasattr(torch.cuda, "_sleep"):
         kt = step.kernel_times(steps=max(8, min(32, args.steps)), backward=do_bwd, batches=list(range(nb)),
                                lead=lambda: torch.cuda._sleep(400_000), fused=kt_fused)
@@ -626,7 +626,7 @@ def run_workload(name, args, torch, factor_max=0):
         kt = step.kernel_times(steps=max(8, min(32, args.steps)), backward=do_bwd, batches=list(range(nb)), lead=lead,
                                fused=kt_fused)
         del lead
-    on_step = [(n_, m_) for n_, m_ in kt if not (issue == "staged" and n_.startswith("inspect"))]
+    on_step = [(n_, m_) for n_, m_ in kt if not (issue.startswith("staged") and n_.startswith("inspect"))]
     kt_sum = sum(ms_k for _, ms_k in on_step)
     kname, k_ms = max(on_step, key=lambda x: x[1])
     k_bytes, k_flops, k_unit = kernel_model(w, kname, u_ent, u_rel)

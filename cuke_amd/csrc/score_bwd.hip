@@ -26,6 +26,42 @@ typedef float v4f __attribute__((ext_vector_type(4)));
 // over all "loopers" of the chunk, which stream through LDS together with the
 // per-(owner, looper) coefficients.
 // ---------------------------------------------------------------------------------------
+// The positive chain of the dot-product models, one element: G is the gradient with respect to the query
+// row a = f(kept entity, relation) summed over the chunk's negatives, g the positive's own upstream
+// gradient.  "kept" is the side of the positive the negatives do not replace (the head; the tail with
+// head negatives), "other" the side they do.  Shared by the per-positive kernel and the tile kernel's
+// epilogue, so both produce the same bits.
+__device__ __forceinline__ void distmult_chain(float g, float k, float o, float r, float G, float &dk, float &dr, float &dother)
+{
+    const float Q = fmaf(g, o, G);  // a = k * r, score = a . other
+    dk = r * Q;
+    dr = k * Q;
+    dother = g * (k * r);
+}
+
+// ComplEx: Re<h, r, conj t>.  Tail negatives: a = h o r;  head negatives: a = conj(r) o t.
+template <bool HEAD>
+__device__ __forceinline__ void complex_chain(float g, float kr, float ki, float or_, float oi, float qr, float qi, float Gr, float Gi,
+                                              float &dkr, float &dki, float &drr, float &dri, float &dor, float &doi)
+{
+    const float Qr = fmaf(g, or_, Gr), Qi = fmaf(g, oi, Gi);
+    if constexpr (HEAD) {
+        dkr = fmaf(Qr, qr, -(Qi * qi));
+        dki = fmaf(Qi, qr, Qr * qi);
+        drr = fmaf(Qr, kr, Qi * ki);
+        dri = fmaf(Qr, ki, -(Qi * kr));
+        dor = g * fmaf(qr, kr, qi * ki);
+        doi = g * fmaf(qr, ki, -(qi * kr));
+    } else {
+        dkr = fmaf(Qr, qr, Qi * qi);
+        dki = fmaf(Qi, qr, -(Qr * qi));
+        drr = fmaf(Qr, kr, Qi * ki);
+        dri = fmaf(Qi, kr, -(Qr * ki));
+        dor = g * fmaf(kr, qr, -(ki * qi));
+        doi = g * fmaf(kr, qi, ki * qr);
+    }
+}
+
 struct TileArgs {
     const float *ent, *rel, *aux;
     const int64_t *h, *r, *neg;
@@ -38,6 +74,15 @@ struct TileArgs {
     int64_t plane;  // B * N
     int C, N, d, rel_dim, vec, vecn, n_chunks;
     float rsign;    // +1: negatives replace the tail; -1: the head (h then holds the tails; see load_query)
+    // Positive chain in the epilogue (DistMult / ComplEx on the matrix-core tiles, 128-bit rows, nothing
+    // riding along): the workgroup that owns 64 positives x 64 columns holds the COMPLETE sum G over the
+    // chunk's negatives for them, so it chains G through the query, adds the positive triple's own term and
+    // writes the occurrence rows of both entities and of the relation itself.  No G rows go to memory and
+    // come back, and no per-positive kernel runs.  chain == 0: G rows are written (out0) as for the other models.
+    int chain;
+    const int64_t *other;        // the positives' replaced side (tails; heads with head negatives)
+    const float *dpos;           // [B] or null
+    float *occ_k, *occ_o, *occ_r;  // occurrence rows [B, d] of the kept side, the replaced side, and [B, rel_dim]
 };
 
 constexpr int kTI = 64;       // columns of the row per workgroup
@@ -106,11 +151,21 @@ __device__ __forceinline__ void bwd_tile_body(const TileArgs &a, int lid, float 
     int c, tile_y, tile_x;
     // wide tiles cover the columns [0, tiles_x * 64); a narrow tile the 16 columns from col_base on
     constexpr bool kHasNarrow = RO == 4 && !MF;  // launches of this shape hand a short remainder to narrow tiles
-    const int wide_tiles_x = (kHasNarrow && narrow_cols(klen)) ? klen / kTI : (klen + kTI - 1) / kTI;
+    // ComplEx on the matrix cores (128-bit rows): a column tile is 32 real columns and the matching 32
+    // imaginary ones, [32 x, 32 x + 32) and half + [32 x, 32 x + 32), so that one workgroup holds both parts of
+    // every complex element it owns (the positive chain in the epilogue needs them together, and a staging
+    // step asks for half as many distinct row pieces of h and r)
+    const bool pair = MODEL == KGE_COMPLEX && MF && !NARROW && a.vec != 0;
+    const int wide_tiles_x = pair ? (half + 31) / 32
+                                  : ((kHasNarrow && narrow_cols(klen)) ? klen / kTI : (klen + kTI - 1) / kTI);
     if (!xcd_tile(lid, NARROW ? 1 : wide_tiles_x, (n_own + TO - 1) / TO, a.n_chunks, c, tile_y, tile_x)) return;
-    const int scol = (NARROW ? col_base : tile_x * kTI) + tx * 4;            // columns this thread stages
+    // local column lc (a multiple of 4 in 0..63) of the tile -> column of the row; and `lim` where the tile has
+    // that column, else 0 (a paired tile's last columns may lie beyond the half row)
+    auto gcol = [&](int lc) { return pair ? (lc < 32 ? tile_x * 32 + lc : half + tile_x * 32 + (lc - 32)) : (NARROW ? col_base : tile_x * kTI) + lc; };
+    auto climit = [&](int lc, int lim) { return (pair && tile_x * 32 + (lc & 31) >= half) ? 0 : lim; };
+    const int scol = gcol(tx * 4);                                           // columns this thread stages
     const int ctx = NARROW ? (tx & 3) : tx;                                  // column lane it computes
-    const int col = (NARROW ? col_base : tile_x * kTI) + ctx * 4;            // columns it owns
+    const int col = gcol(ctx * 4);                                           // columns it owns
     const int ot0 = tile_y * TO;
     auto orow = [&](int o) { return NARROW ? (tx >> 2) * 16 + ty : ty * RO_ + o; };  // owner row inside the tile
     const bool vec = a.vec != 0;
@@ -123,7 +178,7 @@ __device__ __forceinline__ void bwd_tile_body(const TileArgs &a, int lid, float 
 #pragma unroll
     for (int o = 0; o < RO_; ++o) {
         const int ol = ot0 + orow(o);
-        const int lim = ol < n_own ? klen : 0;
+        const int lim = climit(ctx * 4, ol < n_own ? klen : 0);
         const int oc = ol < n_own ? ol : n_own - 1;
         alo[o] = 0.0f;
         if constexpr (OWNER_POS) {
@@ -208,7 +263,7 @@ __device__ __forceinline__ void bwd_tile_body(const TileArgs &a, int lid, float 
 #pragma unroll
         for (int s = 0; s < SL; ++s) {
             const int ll = l0 + ty + 16 * s;
-            const int lim = ll < n_loop ? klen : 0;
+            const int lim = climit(tx * 4, ll < n_loop ? klen : 0);
             if constexpr (OWNER_POS) {
                 const float *pt = a.ent + li0[s] * (int64_t)d;
                 rraw[s][0] = ld4_raw<VEC>(pt, scol, lim);
@@ -282,7 +337,7 @@ __device__ __forceinline__ void bwd_tile_body(const TileArgs &a, int lid, float 
                 if constexpr (NPL == 2) q1 = rraw[s][NRAW - 1];
             } else {
                 const int ll = l0 + ty + 16 * s;
-                combine_query<MODEL, VEC>(rraw[s], 0.0f, scol, ll < n_loop ? klen : 0, half, a.rsign, q0, q1);
+                combine_query<MODEL, VEC>(rraw[s], 0.0f, scol, climit(tx * 4, ll < n_loop ? klen : 0), half, a.rsign, q0, q1);
             }
             if constexpr (kSc) q0 = scale4(q0, kSgnScale), q1 = scale4(q1, kSgnScale);
             *reinterpret_cast<float4 *>(&sL[0][ty + 16 * s][tx * 4]) = q0;
@@ -434,13 +489,92 @@ __device__ __forceinline__ void bwd_tile_body(const TileArgs &a, int lid, float 
     }
 
     if constexpr (kMf) {
+        if constexpr (OWNER_POS && EW == 4 && (MODEL == KGE_DISTMULT || MODEL == KGE_COMPLEX)) {
+            if (a.chain) {  // uniform: the positive chain right here, from the sums in the accumulators
+                const int lc = 4 * fj;
+                const int c0 = gcol(lc);
+                const bool colok = climit(lc, klen) != 0 && c0 + 4 <= d;
+                const int cc = colok ? c0 : 0;  // clamped: unconditional loads
+                int64_t idk[4], ido[4], idr[4];
+                float gp[4];
+                bool rowok[4];
+#pragma unroll
+                for (int v = 0; v < 4; ++v) {
+                    const int ol = ot0 + ob * 16 + 4 * fg + v;
+                    rowok[v] = ol < n_own;
+                    const int64_t b = (int64_t)c * a.C + (rowok[v] ? ol : n_own - 1);
+                    idk[v] = a.h[b], ido[v] = a.other[b], idr[v] = a.r[b];
+                    gp[v] = a.dpos ? a.dpos[b] : 0.0f;
+                }
+                if constexpr (MODEL == KGE_DISTMULT) {
+                    float4 xk[4], xo[4], xr[4];
+#pragma unroll
+                    for (int v = 0; v < 4; ++v) {
+                        xk[v] = *reinterpret_cast<const float4 *>(a.ent + idk[v] * (int64_t)d + cc);
+                        xo[v] = *reinterpret_cast<const float4 *>(a.ent + ido[v] * (int64_t)d + cc);
+                        xr[v] = *reinterpret_cast<const float4 *>(a.rel + idr[v] * (int64_t)a.rel_dim + cc);
+                    }
+#pragma unroll
+                    for (int v = 0; v < 4; ++v) {
+                        const float k4[4] = {xk[v].x, xk[v].y, xk[v].z, xk[v].w}, o4[4] = {xo[v].x, xo[v].y, xo[v].z, xo[v].w};
+                        const float r4[4] = {xr[v].x, xr[v].y, xr[v].z, xr[v].w};
+                        float dk[4], dr[4], dother[4];
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) distmult_chain(gp[v], k4[e], o4[e], r4[e], macc[e][v], dk[e], dr[e], dother[e]);
+                        if (rowok[v] && colok) {
+                            const int64_t b = (int64_t)c * a.C + ot0 + ob * 16 + 4 * fg + v;
+                            *reinterpret_cast<float4 *>(a.occ_k + b * (int64_t)d + c0) = make_float4(dk[0], dk[1], dk[2], dk[3]);
+                            *reinterpret_cast<float4 *>(a.occ_r + b * (int64_t)a.rel_dim + c0) = make_float4(dr[0], dr[1], dr[2], dr[3]);
+                            *reinterpret_cast<float4 *>(a.occ_o + b * (int64_t)d + c0) = make_float4(dother[0], dother[1], dother[2], dother[3]);
+                        }
+                    }
+                } else {
+                    // lanes fj < 8 hold the real parts of complex elements idx .. idx + 3, lanes fj + 8 the imaginary
+                    // parts of the same elements: each takes the other part from its partner and writes its own side
+                    const bool is_re = fj < 8;
+                    const int idx = tile_x * 32 + 4 * (fj & 7);
+                    const int ci = colok ? idx : 0;
+#pragma unroll
+                    for (int v = 0; v < 4; ++v) {
+                        float Gm[4], Gp[4];
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) Gm[e] = macc[e][v], Gp[e] = __shfl_xor(macc[e][v], 8, kWave);
+                        const float *pk = a.ent + idk[v] * (int64_t)d + ci, *po = a.ent + ido[v] * (int64_t)d + ci;
+                        const float *pr = a.rel + idr[v] * (int64_t)a.rel_dim + ci;
+                        const float4 kr4 = *reinterpret_cast<const float4 *>(pk), ki4 = *reinterpret_cast<const float4 *>(pk + half);
+                        const float4 or4 = *reinterpret_cast<const float4 *>(po), oi4 = *reinterpret_cast<const float4 *>(po + half);
+                        const float4 qr4 = *reinterpret_cast<const float4 *>(pr), qi4 = *reinterpret_cast<const float4 *>(pr + half);
+                        const float kr[4] = {kr4.x, kr4.y, kr4.z, kr4.w}, ki[4] = {ki4.x, ki4.y, ki4.z, ki4.w};
+                        const float orr[4] = {or4.x, or4.y, or4.z, or4.w}, oi[4] = {oi4.x, oi4.y, oi4.z, oi4.w};
+                        const float qr[4] = {qr4.x, qr4.y, qr4.z, qr4.w}, qi[4] = {qi4.x, qi4.y, qi4.z, qi4.w};
+                        float dk[4], dr[4], dother[4];
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) {
+                            const float Gr = is_re ? Gm[e] : Gp[e], Gi = is_re ? Gp[e] : Gm[e];
+                            float dkr, dki, drr, dri, dor, doi;
+                            if (a.rsign < 0.0f) complex_chain<true>(gp[v], kr[e], ki[e], orr[e], oi[e], qr[e], qi[e], Gr, Gi, dkr, dki, drr, dri, dor, doi);
+                            else complex_chain<false>(gp[v], kr[e], ki[e], orr[e], oi[e], qr[e], qi[e], Gr, Gi, dkr, dki, drr, dri, dor, doi);
+                            dk[e] = is_re ? dkr : dki, dr[e] = is_re ? drr : dri, dother[e] = is_re ? dor : doi;
+                        }
+                        if (rowok[v] && colok) {
+                            const int64_t b = (int64_t)c * a.C + ot0 + ob * 16 + 4 * fg + v;
+                            *reinterpret_cast<float4 *>(a.occ_k + b * (int64_t)d + c0) = make_float4(dk[0], dk[1], dk[2], dk[3]);
+                            *reinterpret_cast<float4 *>(a.occ_r + b * (int64_t)a.rel_dim + c0) = make_float4(dr[0], dr[1], dr[2], dr[3]);
+                            *reinterpret_cast<float4 *>(a.occ_o + b * (int64_t)d + c0) = make_float4(dother[0], dother[1], dother[2], dother[3]);
+                        }
+                    }
+                }
+                return;
+            }
+        }
 #pragma unroll
         for (int v = 0; v < 4; ++v) {
             const int ol = ot0 + ob * 16 + 4 * fg + v;
             if (ol >= n_own) continue;
             const int64_t row = OWNER_POS ? (int64_t)c * a.C + ol : (int64_t)c * a.N + ol;
             float *dst = a.out0 + row * (int64_t)d;
-            const int c0 = tile_x * kTI + 4 * fj + e0;
+            const int c0 = gcol(4 * fj + e0);
+            if (pair && climit(4 * fj + e0, klen) == 0) continue;
             if (vec && c0 + EW <= klen) {  // rows 16-byte aligned and d % 4 == 0: whole group inside
                 if constexpr (EW == 4)
                     *reinterpret_cast<float4 *>(dst + c0) = make_float4(macc[0][v], macc[1][v], macc[2][v], macc[3][v]);
@@ -534,7 +668,9 @@ static int launch_tiles(TileArgs a, float *g0, float *g1, float *occ_neg, int64_
         // matrix-core inner loop (KGE_PAIR_SUMS_VALU keeps the vector-ALU loop): a wave gets all 64
         // columns of its 16 owners with 64-owner tiles, which win at every size
         if (!dot_valu) {
-            const unsigned gh = xcd_grid(gx, ceil_div(a.C, 64), n_chunks), gn = xcd_grid(gx, ceil_div(a.N, 64), n_chunks);
+            // (ComplEx with 128-bit rows: column tiles pair 32 real with the matching 32 imaginary columns)
+            const int64_t gxm = (MODEL == KGE_COMPLEX && a.vec) ? ceil_div(a.d / 2, 32) : gx;
+            const unsigned gh = xcd_grid(gxm, ceil_div(a.C, 64), n_chunks), gn = xcd_grid(gxm, ceil_div(a.N, 64), n_chunks);
             const size_t lds = tile_lds_bytes<MODEL, 4>(fi);
             hipLaunchKernelGGL((bwd_tile_kernel<MODEL, P, 4, true>), dim3(gh + gn + fi.blocks), dim3(256), lds, st, a,
                                g0, g1, occ_neg, TileGrid{(int)gh, (int)gn, 0, 0}, fi);
@@ -649,17 +785,8 @@ __global__ __launch_bounds__(256) void bwd_pos_kernel(PosBwdArgs a, FusedInsp fi
             Vec<V> dh, dr, dt;
 #pragma unroll
             for (int e = 0; e < V; ++e) {
-                if constexpr (HEAD) {  // a = t * r
-                    const float Q = fmaf(g, vh.v[e], G.v[e]);
-                    dt.v[e] = vr.v[e] * Q;
-                    dr.v[e] = vt.v[e] * Q;
-                    dh.v[e] = g * (vt.v[e] * vr.v[e]);
-                } else {
-                    const float Q = fmaf(g, vt.v[e], G.v[e]);
-                    dh.v[e] = vr.v[e] * Q;
-                    dr.v[e] = vh.v[e] * Q;
-                    dt.v[e] = g * (vh.v[e] * vr.v[e]);
-                }
+                if constexpr (HEAD) distmult_chain(g, vt.v[e], vh.v[e], vr.v[e], G.v[e], dt.v[e], dr.v[e], dh.v[e]);  // a = t * r
+                else distmult_chain(g, vh.v[e], vt.v[e], vr.v[e], G.v[e], dh.v[e], dr.v[e], dt.v[e]);
             }
             dh.store(oh + j), dr.store(orr + j), dt.store(ot + j);
         }
@@ -700,24 +827,12 @@ __global__ __launch_bounds__(256) void bwd_pos_kernel(PosBwdArgs a, FusedInsp fi
             Vec<V> dhr, dhi, drr, dri, dtr, dti;
 #pragma unroll
             for (int e = 0; e < V; ++e) {
-                if constexpr (HEAD) {
-                    // s = Re<n, r, conj t> = n . (conj(r) o t): a = conj(r) o t, Q = g h + G
-                    const float Qr = fmaf(g, hr.v[e], Gr.v[e]), Qi = fmaf(g, hi.v[e], Gi.v[e]);
-                    dtr.v[e] = Qr * qr.v[e] - Qi * qi.v[e];
-                    dti.v[e] = Qi * qr.v[e] + Qr * qi.v[e];
-                    drr.v[e] = Qr * tr.v[e] + Qi * ti.v[e];
-                    dri.v[e] = Qr * ti.v[e] - Qi * tr.v[e];
-                    dhr.v[e] = g * (qr.v[e] * tr.v[e] + qi.v[e] * ti.v[e]);
-                    dhi.v[e] = g * (qr.v[e] * ti.v[e] - qi.v[e] * tr.v[e]);
-                } else {
-                    const float Qr = fmaf(g, tr.v[e], Gr.v[e]), Qi = fmaf(g, ti.v[e], Gi.v[e]);
-                    dhr.v[e] = Qr * qr.v[e] + Qi * qi.v[e];
-                    dhi.v[e] = Qi * qr.v[e] - Qr * qi.v[e];
-                    drr.v[e] = Qr * hr.v[e] + Qi * hi.v[e];
-                    dri.v[e] = Qi * hr.v[e] - Qr * hi.v[e];
-                    dtr.v[e] = g * (hr.v[e] * qr.v[e] - hi.v[e] * qi.v[e]);
-                    dti.v[e] = g * (hr.v[e] * qi.v[e] + hi.v[e] * qr.v[e]);
-                }
+                if constexpr (HEAD)  // s = Re<n, r, conj t> = n . (conj(r) o t): a = conj(r) o t, Q = g h + G
+                    complex_chain<true>(g, tr.v[e], ti.v[e], hr.v[e], hi.v[e], qr.v[e], qi.v[e], Gr.v[e], Gi.v[e], dtr.v[e], dti.v[e],
+                                        drr.v[e], dri.v[e], dhr.v[e], dhi.v[e]);
+                else
+                    complex_chain<false>(g, hr.v[e], hi.v[e], tr.v[e], ti.v[e], qr.v[e], qi.v[e], Gr.v[e], Gi.v[e], dhr.v[e], dhi.v[e],
+                                         drr.v[e], dri.v[e], dtr.v[e], dti.v[e]);
             }
             dhr.store(oh + j), dhi.store(oh + half + j);
             drr.store(orr + j), dri.store(orr + half + j);
@@ -931,6 +1046,7 @@ int kge_score_bwd(const kge_tables *tab, const kge_batch *bat, const kge_saved *
     float *g0 = have_neg ? reinterpret_cast<float *>(ws + p.off_g0) : nullptr;
     float *g1 = have_neg && model == KGE_TRANSH ? reinterpret_cast<float *>(ws + p.off_g1) : nullptr;
     const bool vec = rows_vectorizable(tab);
+    bool chained = false;  // the gradient tile kernel wrote the positives' occurrence rows itself
     int rc = KGE_OK;
     // inspection fused into the score kernels' launches: the histogram and the first digit pass
     // rode with the two forward kernels; the last pass rides with the gradient tile kernel, the
@@ -947,12 +1063,15 @@ int kge_score_bwd(const kge_tables *tab, const kge_batch *bat, const kge_saved *
         if (n_chunks >= (1 << 24)) return KGE_ESHAPE;
         const bool vecn = bat->n_neg % 4 == 0 && aligned16(dneg) && (!saved->neg || aligned16(saved->neg)) &&
                           (!saved->side_neg || aligned16(saved->side_neg));
+        const bool dv = pair_sums_valu(tab);
+        // the positive chain in the tile kernel's epilogue: see TileArgs::chain
+        chained = (model == KGE_DISTMULT || model == KGE_COMPLEX) && !dv && vec && !bat->fuse_inspection;
         TileArgs a{tab->ent, tab->rel, tab->aux, head ? bat->t : bat->h, bat->r, bat->neg, dneg, saved->neg,
                    saved->side_pos, saved->side_neg, model == KGE_ROTATE ? saved->residual : nullptr, nullptr, nullptr,
                    B * bat->n_neg, (int)bat->chunk, (int)bat->n_neg, (int)d, (int)tab->rel_dim, vec ? 1 : 0,
-                   vecn ? 1 : 0, (int)n_chunks, head ? -1.0f : 1.0f};
+                   vecn ? 1 : 0, (int)n_chunks, head ? -1.0f : 1.0f,
+                   chained ? 1 : 0, head ? bat->h : bat->t, dpos, head ? occ_e + B * d : occ_e, head ? occ_e : occ_e + B * d, occ_r};
         float *occ_neg = occ_e + 2 * B * d;
-        const bool dv = pair_sums_valu(tab);
         switch (model) {
         case KGE_TRANSE:
             rc = P == 1 ? launch_tiles<KGE_TRANSE, 1>(a, g0, g1, occ_neg, n_chunks, dv, fi_pass, st)
@@ -974,6 +1093,7 @@ int kge_score_bwd(const kge_tables *tab, const kge_batch *bat, const kge_saved *
         hipLaunchKernelGGL(fill_zero_kernel, dim3(1024), dim3(256), 0, st, occ_e + 2 * B * d, p.nn * d);
     }
 
+    if (!chained) {
     PosBwdArgs pa{tab->ent, tab->rel, tab->aux, bat->h, bat->r, bat->t, dpos, saved->pos, saved->side_pos,
                   g0, g1, have_neg ? dneg : nullptr, bat->n_neg, occ_e, occ_e + B * d, occ_r, occ_w, B, (int)d,
                   (int)tab->rel_dim};
@@ -992,6 +1112,7 @@ int kge_score_bwd(const kge_tables *tab, const kge_batch *bat, const kge_saved *
     }
     timeline_mark(bat->timeline, st, "bwd_pos_kernel");
     if (rc) return rc;
+    }
 
     if (bat->insp_ready && hipStreamWaitEvent(st, reinterpret_cast<hipEvent_t>(bat->insp_ready), 0) != hipSuccess)
         return KGE_ELAUNCH;

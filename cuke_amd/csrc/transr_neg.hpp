@@ -589,13 +589,21 @@ __global__ __launch_bounds__(256) void tneg_occ_kernel(NegIdx x, const float *dx
         if ((p_) == 1) hipLaunchKernelGGL((kern<1, NQ_>), grid_, dim3(256), 0, st, __VA_ARGS__);    \
         else hipLaunchKernelGGL((kern<2, NQ_>), grid_, dim3(256), 0, st, __VA_ARGS__);              \
     } while (0)
+// The workspaces are sized for the worst case G = min(B, n_rel * n_chunks) groups (the count is only known on
+// the device): about four arrays of (2 B + G N) * dim floats, with many relations about four times the
+// B * N * dim floats of the flattened triples.  Above this many bytes (forward + backward) the path declines and
+// the caller scores the flattened triples (or sees the shape in the error), instead of running out of memory.
+constexpr size_t kNegWorkspaceCap = size_t(24) << 30;
+
 static bool transr_neg_path_ok(const kge_tables *tab, const kge_batch *bat)
 {
     if (tab->model != KGE_TRANSR || !bat->neg || !bat->rel_insp) return false;
     if (!mfma_path_ok(tab, bat) || gemm_lds_bytes((int)tab->dim) > kMaxGemmLds) return false;
     const NegShape s = neg_shape(tab, bat);
-    return s.n_chunks > 0 && tab->n_rel * s.n_chunks < (int64_t(1) << 31) && s.L_cap < (int64_t(1) << 31) &&
-           s.L_cap * s.d < (int64_t(1) << 40);
+    if (!(s.n_chunks > 0 && tab->n_rel * s.n_chunks < (int64_t(1) << 31) && s.L_cap < (int64_t(1) << 31) &&
+          s.L_cap * s.d < (int64_t(1) << 36)))
+        return false;
+    return neg_fwd_layout(tab, s).total + neg_bwd_layout(s).total <= kNegWorkspaceCap;
 }
 
 size_t transr_neg_fwd_workspace(const kge_tables *tab, const kge_batch *bat)

@@ -262,6 +262,11 @@ class KGEModel:
                                                _stream()), "kge_residual_fwd")
         return out
 
+    def _grouped_negatives_fit(self, bat) -> bool:
+        """TransR with shared negatives: True if the grouped path takes this shape (its worst-case workspaces stay
+        under the library's byte cap); the size query of the backward workspace answers 0 otherwise."""
+        return int(_lib.lib().kge_score_bwd_workspace(C.byref(self._tab), C.byref(bat))) > 0
+
     def _fwd_workspace(self, bat):
         nb = int(_lib.lib().kge_score_fwd_workspace(C.byref(self._tab), C.byref(bat)))
         return torch.empty(max(nb, 1), dtype=torch.uint8, device=self.dev), nb
@@ -284,6 +289,10 @@ class KGEModel:
             if self.dim % 4 != 0 or self.dim > 1024:
                 return self._score_projected_negatives(h, r, t, neg, chunk, neg_mode)
         bat, keep = self._batch(h, r, t, neg, chunk, ent_insp, rel_insp, neg_mode)
+        if neg is not None and self.model == "TransR" and not self._grouped_negatives_fit(bat):
+            # the grouped path sizes its workspaces for the worst case min(B, n_rel * n_chunks) groups; above
+            # its byte cap the pairs are scored as explicit triples
+            return self._score_projected_negatives(h, r, t, neg, chunk, neg_mode)
         B, N = bat.batch, bat.n_neg
         f32 = dict(dtype=torch.float32, device=self.dev)
         fw = Forward(torch.empty(B, **f32), torch.empty((B, N), **f32) if neg is not None else None,
@@ -555,6 +564,10 @@ class TrainStep:
         self.side_neg = torch.empty((2, B, N), **f32) if (model.model == "TransH" and neg is not None) else None
         self.residual = torch.empty((B, model.dim), **f32) if model.model in ("TransR", "RESCAL", "RotatE") \
             else None
+        if model.model == "TransR" and neg is not None and not model._grouped_negatives_fit(self.bat):
+            raise KgeError(f"TransR with shared negatives at batch {B} x {N} negatives, dim {model.dim}, {model.n_rel} relations: "
+                           "the grouped path's worst-case workspaces exceed the library's cap; score the pairs as "
+                           "explicit triples (KGEModel.score) or use smaller chunks of the batch")
         self._ws_f_bytes = int(L.kge_score_fwd_workspace(C.byref(model._tab), C.byref(self.bat)))
         self._ws_f = torch.empty(max(self._ws_f_bytes, 1), dtype=torch.uint8, device=dev)
         # TransR / RESCAL without negatives: the forward workspace holds the batch's tile plans, which a

@@ -180,9 +180,9 @@ def backward(model, E, R, A, h, r, t, neg=None, chunk=0, dpos=None, dneg=None, p
 
 
 def l1_ambiguous_rows(model, E, R, A, h, r, t, neg=None, chunk=0, eps=6e-8, fast=False, neg_mode="tail"):
-    """Rows of the sparse L1 gradient (TransE / TransH) that a sign ambiguity can reach: masks over the
-    unique entity ids and the unique relation ids (same order as ``backward``), plus the number of residual
-    elements with |u| <= eps that caused them."""
+    """Rows of the sparse L1 gradient (TransE / TransH) that a sign ambiguity can reach: for every unique
+    entity id and every unique relation id (same order as ``backward``) the number of residual elements with
+    |u| <= eps in the triples and pairs that touch the row (0 = the row is clear), plus their total."""
     E, R, A = _f32(E), _f32(R), _f32(A)
     h, r, t, neg = _i64(h), _i64(r), _i64(t), _i64(neg)
     B, d = h.shape[0], E.shape[1]
@@ -196,8 +196,8 @@ def l1_ambiguous_rows(model, E, R, A, h, r, t, neg=None, chunk=0, eps=6e-8, fast
     slot_h = np.ascontiguousarray(ins_e.inverse[:B])
     slot_t = np.ascontiguousarray(ins_e.inverse[B:2 * B])
     slot_n = np.ascontiguousarray(ins_e.inverse[2 * B:]) if neg is not None else None
-    flag_e = np.zeros(ins_e.unique_ids.shape[0], np.uint8)
-    flag_r = np.zeros(ins_r.unique_ids.shape[0], np.uint8)
+    flag_e = np.zeros(ins_e.unique_ids.shape[0], np.int32)
+    flag_r = np.zeros(ins_r.unique_ids.shape[0], np.int32)
     fn = _lib(fast).orc_l1_ambiguous
     fn.restype = ctypes.c_int64
     n = fn(ctypes.c_int(MODELS[model]), ctypes.c_int64(B), ctypes.c_int64(d), _fp(E), _fp(R), _fp(A),
@@ -206,7 +206,7 @@ def l1_ambiguous_rows(model, E, R, A, h, r, t, neg=None, chunk=0, eps=6e-8, fast
            _fp(np.ascontiguousarray(ins_r.inverse)), _fp(flag_e), _fp(flag_r))
     if n < 0:
         raise ValueError(f"{model} has no L1 form")
-    return flag_e.astype(bool), flag_r.astype(bool), int(n)
+    return flag_e, flag_r, int(n)
 
 
 def margin_loss(pos, neg, margin, sign=1.0):

@@ -384,9 +384,9 @@ static void add_row(double *acc, const float *src, int64_t n)
     for (int64_t i = 0; i < n; ++i) acc[i] += (double)src[i];
 }
 
-/* The triples b0 <= b < b1, accumulated into aE / aR / aA (double).  tmp: 3d + 1 floats,
- * one: 3d + aux_width + 1 floats. */
-static void bwd_range(int model, int p, int64_t b0, int64_t b1, int64_t d, const float *E, const float *R,
+/* The triples order[i] (or i itself without an order) for b0 <= i < b1, accumulated into aE / aR / aA
+ * (double).  tmp: 3d + 1 floats, one: 3d + aux_width + 1 floats. */
+static void bwd_range(int model, int p, const int64_t *order, int64_t b0, int64_t b1, int64_t d, const float *E, const float *R,
                       const float *A, const int64_t *h, const int64_t *r, const int64_t *t,
                       const int64_t *neg, int64_t C, int64_t N, int neg_head, const float *dpos, const float *dneg,
                       const int64_t *slot_h, const int64_t *slot_t, const int64_t *slot_neg,
@@ -394,7 +394,8 @@ static void bwd_range(int model, int p, int64_t b0, int64_t b1, int64_t d, const
 {
     const int64_t rw = rel_width(model, d), aw = aux_width(model, d);
     float *dh = one, *dr = one + d, *dt = one + 2 * d, *da = one + 3 * d;
-    for (int64_t b = b0; b < b1; ++b) {
+    for (int64_t i = b0; i < b1; ++i) {
+        const int64_t b = order ? order[i] : i;
         const float *eh = E + h[b] * d, *rr = R ? R + r[b] * rw : NULL;
         const float *ax = A ? A + r[b] * aw : NULL;
         const int64_t n_t = 1 + ((neg && dneg) ? N : 0);
@@ -424,7 +425,12 @@ static void bwd_range(int model, int p, int64_t b0, int64_t b1, int64_t d, const
 
 /* With OpenMP (the timed multi-thread leg of the benchmark only; the checker is built without
  * it) the batch is cut into one contiguous range per thread, every thread accumulates into
- * double arrays of its own, and the per-thread arrays are added up in thread order. */
+ * double arrays of its own, and the per-thread arrays are added up in thread order.
+ * The projection models (a d x d gradient per relation) are cut by RELATION instead: the triples are
+ * ordered by relation slot, every thread takes a contiguous range of whole relations (balanced by
+ * triple count) and accumulates their relation and projection rows straight into the one shared
+ * array (no other thread touches those rows); only the entity rows are kept per thread.  A dense
+ * n_slots_r x d x d double array per thread made that leg slower than one thread. */
 int orc_backward(int model, int p, int64_t B, int64_t d, const float *E, const float *R,
                  const float *A, const int64_t *h, const int64_t *r, const int64_t *t,
                  const int64_t *neg, int64_t C, int64_t N, int neg_head, const float *dpos, const float *dneg,
@@ -441,11 +447,38 @@ int orc_backward(int model, int p, int64_t B, int64_t d, const float *E, const f
     T = omp_get_max_threads();
     if (T > B) T = B > 0 ? (int)B : 1;
 #endif
+    const int by_relation = T > 1 && aw == d * d && n_slots_r > 0;
+    const int TR = by_relation ? 1 : T;  /* copies of the relation-side accumulators */
     double *aE = (double *)calloc(nE * (size_t)T, sizeof(double));
-    double *aR = (double *)calloc(nR * (size_t)T, sizeof(double));
-    double *aA = (double *)calloc(nA * (size_t)T, sizeof(double));
-    if (!aE || !aR || !aA) {
-        free(aE); free(aR); free(aA);
+    double *aR = (double *)calloc(nR * (size_t)TR, sizeof(double));
+    double *aA = (double *)calloc(nA * (size_t)TR, sizeof(double));
+    int64_t *order = NULL, *cut = NULL;
+    if (by_relation) {  /* counting sort of the triples by relation slot; cut[q] = first position of thread q */
+        order = (int64_t *)malloc(sizeof(int64_t) * (size_t)(B + 1));
+        cut = (int64_t *)malloc(sizeof(int64_t) * (size_t)(T + 1));
+        int64_t *start = (int64_t *)calloc((size_t)(n_slots_r + 1), sizeof(int64_t));
+        if (order && cut && start) {
+            for (int64_t b = 0; b < B; ++b) start[slot_r[b] + 1]++;
+            for (int64_t u = 0; u < n_slots_r; ++u) start[u + 1] += start[u];
+            int q = 0;
+            cut[0] = 0;
+            for (int64_t u = 0; u < n_slots_r && q + 1 < T; ++u)  /* thread q ends at the relation boundary nearest to its share */
+                while (q + 1 < T && start[u + 1] >= B * (q + 1) / T) cut[++q] = start[u + 1];
+            while (q < T) cut[++q] = B;
+            int64_t *fill = (int64_t *)malloc(sizeof(int64_t) * (size_t)(n_slots_r + 1));
+            if (fill) {
+                memcpy(fill, start, sizeof(int64_t) * (size_t)(n_slots_r + 1));
+                for (int64_t b = 0; b < B; ++b) order[fill[slot_r[b]]++] = b;
+                free(fill);
+            } else {
+                free(order);
+                order = NULL;
+            }
+        }
+        free(start);
+    }
+    if (!aE || !aR || !aA || (by_relation && (!order || !cut))) {
+        free(aE); free(aR); free(aA); free(order); free(cut);
         return -2;
     }
     int failed = 0;
@@ -462,13 +495,16 @@ int orc_backward(int model, int p, int64_t B, int64_t d, const float *E, const f
         if (!tmp || !one) {
             failed = 1;
         } else {
-            const int64_t b0 = B * tid / T, b1 = B * (tid + 1) / T;
-            bwd_range(model, p, b0, b1, d, E, R, A, h, r, t, neg, C, N, neg_head, dpos, dneg, slot_h, slot_t,
-                      slot_neg, slot_r, aE + nE * (size_t)tid, aR + nR * (size_t)tid, aA + nA * (size_t)tid, tmp, one);
+            const int64_t b0 = by_relation ? cut[tid] : B * tid / T, b1 = by_relation ? cut[tid + 1] : B * (tid + 1) / T;
+            const size_t rel_copy = by_relation ? 0 : (size_t)tid;
+            bwd_range(model, p, order, b0, b1, d, E, R, A, h, r, t, neg, C, N, neg_head, dpos, dneg, slot_h, slot_t,
+                      slot_neg, slot_r, aE + nE * (size_t)tid, aR + nR * rel_copy, aA + nA * rel_copy, tmp, one);
         }
         free(tmp);
         free(one);
     }
+    free(order);
+    free(cut);
     if (failed) {
         free(aE); free(aR); free(aA);
         return -2;
@@ -484,7 +520,7 @@ int orc_backward(int model, int p, int64_t B, int64_t d, const float *E, const f
     if (gR) {
         for (int64_t i = 0; i < n_slots_r * rw; ++i) {
             double s = aR[i];
-            for (int q = 1; q < T; ++q) s += aR[nR * (size_t)q + (size_t)i];
+            for (int q = 1; q < TR; ++q) s += aR[nR * (size_t)q + (size_t)i];
             gR[i] = (float)s;
         }
     }
@@ -494,7 +530,7 @@ int orc_backward(int model, int p, int64_t B, int64_t d, const float *E, const f
 #endif
         for (int64_t i = 0; i < n_slots_r * aw; ++i) {
             double s = aA[i];
-            for (int q = 1; q < T; ++q) s += aA[nA * (size_t)q + (size_t)i];
+            for (int q = 1; q < TR; ++q) s += aA[nA * (size_t)q + (size_t)i];
             gA[i] = (float)s;
         }
     }
@@ -508,15 +544,14 @@ int orc_backward(int model, int p, int64_t B, int64_t d, const float *E, const f
  * from two correct fp32 implementations, and (TransH) one flipped sign moves every column of
  * the rows of that triple through q.w.  For every triple and pair of the batch whose residual
  * holds an element with |u_j| <= eps this marks the slots of its head, tail / negative and
- * relation rows in flagE[n_slots_e] / flagR[n_slots_r] (bytes, caller-zeroed; writes of 1
- * only, so threads may race on them).  Returns the number of such elements, -1 for a model
- * without an L1 form.
+ * relation rows by adding the number of such elements to cntE[n_slots_e] / cntR[n_slots_r]
+ * (int32, caller-zeroed): a row's count bounds how many sign flips can reach that row.  Returns
+ * the total number of such elements, -1 for a model without an L1 form.
  */
 int64_t orc_l1_ambiguous(int model, int64_t B, int64_t d, const float *E, const float *R, const float *A,
                          const int64_t *h, const int64_t *r, const int64_t *t, const int64_t *neg, int64_t C,
                          int64_t N, int neg_head, float eps, const int64_t *slot_h, const int64_t *slot_t,
-                         const int64_t *slot_neg, const int64_t *slot_r, unsigned char *flagE,
-                         unsigned char *flagR)
+                         const int64_t *slot_neg, const int64_t *slot_r, int32_t *cntE, int32_t *cntR)
 {
     if (model != ORC_TRANSE && model != ORC_TRANSH) return -1;
     int64_t total = 0;
@@ -544,7 +579,18 @@ int64_t orc_l1_ambiguous(int model, int64_t B, int64_t d, const float *E, const 
                 int64_t n = 0;
                 for (int64_t j = 0; j < d; ++j) n += fabsf(u[j]) <= eps;
                 if (n) {
-                    flagE[sh] = 1, flagE[st] = 1, flagR[slot_r[b]] = 1;
+#ifdef _OPENMP
+#pragma omp atomic
+#endif
+                    cntE[sh] += (int32_t)n;
+#ifdef _OPENMP
+#pragma omp atomic
+#endif
+                    cntE[st] += (int32_t)n;
+#ifdef _OPENMP
+#pragma omp atomic
+#endif
+                    cntR[slot_r[b]] += (int32_t)n;
                     total += n;
                 }
             }

@@ -132,6 +132,28 @@ def test_transr_negatives_backward_requires_the_positive_scores_for_l2():
                                None) == -1
 
 
+def test_transr_negatives_grouped_path_declines_shapes_whose_worst_case_workspace_is_huge():
+    """The grouped shared-negative TransR path sizes its workspaces for min(B, n_rel * n_chunks) groups; above
+    its byte cap both size queries answer 0 (and the host scores the pairs as explicit triples) instead of
+    asking the caller for tens of gigabytes."""
+    import ctypes as C
+    from cuke_amd import _lib
+    L = _lib.lib()
+    fake = 0x10000
+
+    def sizes(B, N, chunk, d, n_rel):
+        tab = _lib.Tables(_lib.MODELS["TransR"], 2, 0.0, 0, d, d, 1000, n_rel, fake, fake, fake)
+        rel = _lib.Inspection(B, n_rel, fake, fake, fake, fake, fake, fake)
+        bat = _lib.Batch(B, fake, fake, fake, fake, chunk, N, None, C.pointer(rel), None, 0, 0)
+        return (int(L.kge_score_fwd_workspace(C.byref(tab), C.byref(bat))),
+                int(L.kge_score_bwd_workspace(C.byref(tab), C.byref(bat))))
+
+    f, b = sizes(4096, 64, 512, 200, 1345)
+    assert 0 < f + b <= 24 << 30
+    f_big, b_big = sizes(16384, 1024, 1024, 400, 10000)   # (2 B + B N) * dim floats, four times over: ~100 GB
+    assert b_big == 0
+
+
 def test_fused_inspection_eligibility_is_decided_on_the_host():
     """kge_fused_inspection_ok only reads the descriptors: shared negatives, index sets of at most 65536 ids and
     tables of at most 2^22 rows qualify; larger sets and larger tables do not,

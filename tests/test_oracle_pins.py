@@ -520,8 +520,8 @@ def test_openmp_build_of_the_oracle_gives_the_checkers_results(oracle):
 
 
 def test_l1_ambiguity_mask_vs_numpy(oracle):
-    """l1_ambiguous_rows marks exactly the rows of the triples and pairs whose residual has an element with
-    |u| <= eps (brute force in numpy; eps chosen large enough that a fraction of the rows is marked)."""
+    """l1_ambiguous_rows counts, per row, exactly the residual elements with |u| <= eps of the triples and pairs
+    that touch the row (brute force in numpy; eps chosen large enough that a fraction of the rows is marked)."""
     w = synth.custom_workload("TransH", n_ent=60, n_rel=5, dim=8, batch=24, chunk=12, n_neg=6, norm_p=1, sigma=0.2,
                               seed=4)
     a = w.arrays
@@ -529,7 +529,7 @@ def test_l1_ambiguity_mask_vs_numpy(oracle):
     fe, fr, n = oracle.l1_ambiguous_rows("TransH", a["E"], a["R"], a["A"], a["h"], a["r"], a["t"], a["neg"], w.chunk,
                                          eps=eps)
     ue, ur = np.unique(np.concatenate([a["h"], a["t"], a["neg"]])), np.unique(a["r"])
-    we, wr, total = np.zeros(ue.size, bool), np.zeros(ur.size, bool), 0
+    we, wr, total = np.zeros(ue.size, np.int64), np.zeros(ur.size, np.int64), 0
     for b in range(w.batch):
         tails = [a["t"][b]] + list(a["neg"][(b // w.chunk) * w.n_neg:(b // w.chunk + 1) * w.n_neg])
         for tl in tails:
@@ -537,7 +537,11 @@ def test_l1_ambiguity_mask_vs_numpy(oracle):
             k = int((np.abs(u) <= np.float32(eps)).sum())
             if k:
                 total += k
-                we[np.searchsorted(ue, [a["h"][b], tl])] = True
-                wr[np.searchsorted(ur, a["r"][b])] = True
-    assert n == total and 0 < we.sum() < we.size
+                for e in (a["h"][b], tl):
+                    we[np.searchsorted(ue, e)] += k
+                wr[np.searchsorted(ur, a["r"][b])] += k
+    assert n == total and 0 < (we > 0).sum() < we.size
     assert np.array_equal(fe, we) and np.array_equal(fr, wr)
+    fe2, fr2, n2 = oracle.l1_ambiguous_rows("TransH", a["E"], a["R"], a["A"], a["h"], a["r"], a["t"], a["neg"], w.chunk,
+                                            eps=eps, fast="omp")
+    assert n2 == n and np.array_equal(fe2, fe) and np.array_equal(fr2, fr), "the OpenMP build counts the same"
