@@ -682,24 +682,27 @@ def run_workload(name, args, torch, factor_max=0):
     return out
 
 
-def run_neg_transr(args, torch):
-    """TransR with shared negatives at B=4096, N=64, dim=200 (relations Zipf 1.2 over 1345, as the TransR
-    benchmark configuration): forward + backward with every negative projected once per (relation, chunk)
-    group, beside the flattened B * (1 + N) explicit triples (the reference's neg_transR,
-    apps/examples/examples.py:1447-1480).  Rows through the grouped matrix-core kernels are counted on the
-    host from the index arrays: 2 B + G N against B (1 + N), G = distinct (relation, chunk) pairs."""
+def run_neg_transr(args, torch, model_name="TransR"):
+    """TransR (or RESCAL) with shared negatives at B=4096, N=64, dim=200 (relations Zipf 1.2 over 1345, as the
+    TransR benchmark configuration), forward + backward, beside the flattened B * (1 + N) explicit triples (the
+    reference's neg_transR, apps/examples/examples.py:1447-1480).  TransR: every negative projected once per
+    (relation, chunk) group; rows through the grouped matrix-core kernels are counted on the host from the
+    index arrays, 2 B + G N against B (1 + N), G = distinct (relation, chunk) pairs.  RESCAL: the pair score
+    (E[h] Proj[r]) . E[t'] needs the B projected rows only (a dot-product tile over them)."""
     from cuke_amd import synth
     from cuke_amd.kge import KGEModel, inspect
     dev = torch.device("cuda:0")
-    out = {"workload": "neg_transr_4096x64x200", "batch": 4096, "n_neg": 64, "dim": 200, "by_chunk": []}
+    out = {"workload": f"neg_{model_name.lower()}_4096x64x200", "batch": 4096, "n_neg": 64, "dim": 200, "by_chunk": []}
     for chunk in (64, 512, 4096):
-        w = synth.custom_workload("TransR", seed=args.seed, n_ent=40000, n_rel=1345, dim=200, batch=4096, chunk=chunk,
+        w = synth.custom_workload(model_name, seed=args.seed, n_ent=40000, n_rel=1345, dim=200, batch=4096, chunk=chunk,
                                   n_neg=64, norm_p=2, sigma=0.05, rel_zipf=1.2)
         a = w.arrays
-        m = KGEModel("TransR", *[torch.from_numpy(a[k]).to(dev) for k in ("E", "R", "A")], norm_p=2)
+        m = KGEModel(model_name, torch.from_numpy(a["E"]).to(dev), torch.from_numpy(a["R"]).to(dev) if model_name == "TransR" else None,
+                     torch.from_numpy(a["A"]).to(dev), norm_p=2)
         ix = {k: torch.from_numpy(a[k]).to(dev) for k in ("h", "r", "t", "neg")}
         g_pairs = len(np.unique(a["r"] * w.n_chunks + np.arange(w.batch) // chunk))
-        rows_grouped, rows_flat = 2 * w.batch + g_pairs * w.n_neg, w.batch * (1 + w.n_neg)
+        rows_grouped = 2 * w.batch + g_pairs * w.n_neg if model_name == "TransR" else w.batch
+        rows_flat = w.batch * (1 + w.n_neg)
         dpos = torch.ones(w.batch, device=dev)
         dneg = torch.ones((w.batch, w.n_neg), device=dev)
         ent_insp, rel_insp = m.inspect_batch(ix["h"], ix["r"], ix["t"], ix["neg"])
@@ -762,8 +765,8 @@ def main():
     ap.add_argument("--steps", type=int, default=100)
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--workload", default="all",
-                    help="all (default), one of " + ", ".join(ALL_WORKLOADS) + ", ref_transr_8192x512, or neg_transr "
-                         "(TransR shared negatives: grouped projection against flattened triples)")
+                    help="all (default), one of " + ", ".join(ALL_WORKLOADS) + ", ref_transr_8192x512, or neg_transr / "
+                         "neg_rescal (shared negatives of the projection models: grouped form against flattened triples)")
     ap.add_argument("--batches", type=int, default=8, help="distinct seeded batches the timed loop rotates over")
     ap.add_argument("--no-graph", action="store_true", help="do not also time HIP-graph replays of the step")
     ap.add_argument("--no-staged", action="store_true",
@@ -792,9 +795,9 @@ def main():
         dst.copy_(src)  # one elementwise copy kernel: reads 256 MiB, writes 256 MiB
         torch.cuda.synchronize()
         del src, dst
-    if args.workload == "neg_transr":
+    if args.workload in ("neg_transr", "neg_rescal"):
         try:
-            print(json.dumps(run_neg_transr(args, torch)))
+            print(json.dumps(run_neg_transr(args, torch, "TransR" if args.workload == "neg_transr" else "RESCAL")))
         except SpotCheckError as e:
             print(f"bench.py: {e}", file=sys.stderr)
             sys.exit(1)

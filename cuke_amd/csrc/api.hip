@@ -220,6 +220,8 @@ int kge_score_fwd(const kge_tables *tab, const kge_batch *bat, float *pos, float
     const bool want_neg = neg && bat->neg;
     if (want_neg && (tab->model == KGE_TRANSH || tab->model == KGE_TRANSF) && !side_pos) return KGE_EINVAL;
     if (want_neg && tab->model == KGE_ROTATE && !residual) return KGE_EINVAL;  // rotated heads buffer
+    if (want_neg && tab->model == KGE_RESCAL && (!residual || bat->neg_mode != KGE_NEG_TAIL))
+        return residual ? KGE_EUNSUPPORTED : KGE_EINVAL;  // the projected rows are the pair kernel's queries
     // fused inspection: first digit pass with the per-positive kernel, second with the tile kernel
     const bool grouped_model = tab->model == KGE_TRANSR || tab->model == KGE_RESCAL;
     const bool fuse = bat->fuse_inspection != 0 && !grouped_model;  // (the grouped kernels plan their own riders)
@@ -247,7 +249,7 @@ int kge_score_fwd(const kge_tables *tab, const kge_batch *bat, float *pos, float
         if (rc) return rc;
     }
     if (want_neg) {
-        rc = launch_score_neg(tab, bat, side_pos, tab->model == KGE_ROTATE ? residual : nullptr, neg, side_neg,
+        rc = launch_score_neg(tab, bat, side_pos, (tab->model == KGE_ROTATE || tab->model == KGE_RESCAL) ? residual : nullptr, neg, side_neg,
                               fuse ? &fi1 : nullptr, workspace, workspace_bytes, st, carry ? pos : nullptr);
         timeline_mark(bat->timeline, st, "score_neg_kernel");
         return rc;

@@ -69,7 +69,7 @@ struct TileArgs {
     const float *sneg;      // [B, N] forward scores (L2 normalisation)
     const float *side_pos;  // TransH: w.h per positive
     const float *side_neg;  // TransH: [2, B, N]
-    const float *query;     // RotatE: rotated heads [B, d] saved by the forward pass, or null
+    const float *query;     // RotatE: rotated heads [B, d] saved by the forward pass; RESCAL: projected rows E[h] Proj[r]; else null
     float *out0, *out1;
     int64_t plane;  // B * N
     int C, N, d, rel_dim, vec, vecn, n_chunks;
@@ -124,7 +124,8 @@ __device__ __forceinline__ void bwd_tile_body(const TileArgs &a, int lid, float 
     constexpr int RO_ = NARROW ? 1 : RO;           // owners per thread
     constexpr int TO = NARROW ? 64 : 16 * RO;      // owners per tile
     constexpr bool kRot = MODEL == KGE_ROTATE, kTH = MODEL == KGE_TRANSH;
-    constexpr bool kDot = MODEL == KGE_DISTMULT || MODEL == KGE_COMPLEX || MODEL == KGE_TRANSF;  // score = query . t' (+ const)
+    constexpr bool kDot = MODEL == KGE_DISTMULT || MODEL == KGE_COMPLEX || MODEL == KGE_TRANSF ||
+                          MODEL == KGE_RESCAL;  // score = query . t' (+ const)
     constexpr bool kMf = kDot && MF;  // the sum over loopers on the matrix cores (else on the vector ALUs)
     constexpr bool kL2 = (MODEL == KGE_TRANSE || kTH) && P == 2;
     // L1 translation models: owner and looper rows carry the factor 2^100, so the sign of a residual
@@ -272,7 +273,7 @@ __device__ __forceinline__ void bwd_tile_body(const TileArgs &a, int lid, float 
                 const int64_t b = (int64_t)c * a.C + (ll < n_loop ? ll : n_loop - 1);
                 const float *ph = a.ent + li0[s] * (int64_t)d, *pr = a.rel + li1[s] * (int64_t)a.rel_dim;
                 const float *pw = kTH ? a.aux + li1[s] * (int64_t)d : nullptr;
-                const float *pq = kRot ? a.query + b * (int64_t)d : nullptr;
+                const float *pq = (kRot || MODEL == KGE_RESCAL) ? a.query + b * (int64_t)d : nullptr;
                 if constexpr (kDefer) {
                     load_query_raw<MODEL, VEC>(ph, pr, pw, pq, scol, lim, half, rraw[s]);
                 } else {
@@ -663,7 +664,7 @@ static int launch_tiles(TileArgs a, float *g0, float *g1, float *occ_neg, int64_
     const int64_t gxw = narrow ? klen / kTI : gx;    // wide column tiles of such a launch
     const int64_t big = gx * (ceil_div(a.C, 64) + ceil_div(a.N, 64)) * n_chunks;
     // the size rule follows launch_neg_mp (see there)
-    constexpr bool kDotModel = MODEL == KGE_DISTMULT || MODEL == KGE_COMPLEX || MODEL == KGE_TRANSF;
+    constexpr bool kDotModel = MODEL == KGE_DISTMULT || MODEL == KGE_COMPLEX || MODEL == KGE_TRANSF || MODEL == KGE_RESCAL;
     if constexpr (kDotModel) {
         // matrix-core inner loop (KGE_PAIR_SUMS_VALU keeps the vector-ALU loop): a wave gets all 64
         // columns of its 16 owners with 64-owner tiles, which win at every size
@@ -982,12 +983,29 @@ static BwdPlan make_bwd_plan(const kge_tables *tab, const kge_batch *bat)
     return p;
 }
 
+// RESCAL with shared negatives (tail mode): the gradient tiles of the dot-product score over the projected
+// query rows; g0[B, d] receives dL/dq summed over the chunk's negatives, occ_neg[nn, d] the negatives' rows.
+// Called by the grouped backward pass in transr.hip.
+int launch_rescal_neg_tiles(const kge_tables *tab, const kge_batch *bat, const float *query, const float *dneg, float *g0,
+                            float *occ_neg, hipStream_t st)
+{
+    const int64_t B = bat->batch, d = tab->dim, n_chunks = B / bat->chunk;
+    if (n_chunks >= (1 << 24)) return KGE_ESHAPE;
+    const bool vec = rows_vectorizable(tab), vecn = bat->n_neg % 4 == 0 && aligned16(dneg);
+    TileArgs a{tab->ent, nullptr, nullptr, bat->h, bat->r, bat->neg, dneg, nullptr, nullptr, nullptr, query, nullptr, nullptr,
+               B * bat->n_neg, (int)bat->chunk, (int)bat->n_neg, (int)d, 0, vec ? 1 : 0, vecn ? 1 : 0, (int)n_chunks, 1.0f,
+               0, nullptr, nullptr, nullptr, nullptr, nullptr};
+    return launch_tiles<KGE_RESCAL, 2>(a, g0, nullptr, occ_neg, n_chunks, pair_sums_valu(tab), FusedInsp{}, st);
+}
+
 int launch_transr_bwd(const kge_tables *, const kge_batch *, const kge_saved *, const float *,
                       const kge_grads *, void *, size_t, hipStream_t);
 size_t transr_bwd_workspace(const kge_tables *, const kge_batch *);
 int launch_transr_neg_bwd(const kge_tables *, const kge_batch *, const kge_saved *, const float *, const float *,
                           const kge_grads *, void *, size_t, hipStream_t);
 size_t transr_neg_bwd_workspace(const kge_tables *, const kge_batch *);
+int launch_rescal_neg_bwd(const kge_tables *, const kge_batch *, const kge_saved *, const float *, const float *,
+                          const kge_grads *, void *, size_t, hipStream_t);
 
 }  // namespace kge
 
@@ -1017,6 +1035,8 @@ int kge_score_bwd(const kge_tables *tab, const kge_batch *bat, const kge_saved *
     KGE_CLEAR_LAUNCH_ERRORS();
     if (tab->model == KGE_TRANSR && bat->neg)
         return launch_transr_neg_bwd(tab, bat, saved, dpos, dneg, grads, workspace, workspace_bytes, st);
+    if (tab->model == KGE_RESCAL && bat->neg)
+        return launch_rescal_neg_bwd(tab, bat, saved, dpos, dneg, grads, workspace, workspace_bytes, st);
     if (tab->model == KGE_TRANSR || tab->model == KGE_RESCAL)
         return launch_transr_bwd(tab, bat, saved, dpos, grads, workspace, workspace_bytes, st);
 

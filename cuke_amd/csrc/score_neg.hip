@@ -22,7 +22,7 @@ struct NegArgs {
     const float *ent, *rel, *aux;
     const int64_t *h, *r, *neg;  // h: the side of the positive that is kept (tails with head negatives)
     const float *side_pos;  // TransH: w_b . h_b; TransF: r_b . h_b (the kept side: t_b with head negatives)
-    const float *query;     // RotatE: rotated heads [B, d] from the positive kernel (required)
+    const float *query;     // RotatE: rotated heads [B, d] from the positive kernel; RESCAL: projected rows E[h] Proj[r] (required)
     float *out;             // [B, N]
     float *side_neg;        // TransH save-for-backward [2, B, N] (optional):
                             //   plane 0: c = w_b . t'_k ; plane 1: sum_i phi(u_i) w_i with
@@ -55,7 +55,7 @@ template <int MODEL, int P, bool SAVE>
 __device__ __forceinline__ void pair_elem(float &acc, float &acc2, float a0, float a1, float t0, float t1,
                                           float c)
 {
-    if constexpr (MODEL == KGE_DISTMULT || MODEL == KGE_COMPLEX || MODEL == KGE_TRANSF) {
+    if constexpr (MODEL == KGE_DISTMULT || MODEL == KGE_COMPLEX || MODEL == KGE_TRANSF || MODEL == KGE_RESCAL) {
         acc = fmaf(a0, t0, acc);
     } else if constexpr (MODEL == KGE_TRANSE) {
         const float u = a0 - t0;
@@ -126,7 +126,7 @@ __global__ __launch_bounds__(256, KGE_TILE_OCC) void score_neg_kernel(NegArgs a,
         pr[s] = a.rel + rid * (int64_t)a.rel_dim;
         pw[s] = MODEL == KGE_TRANSH ? a.aux + rid * (int64_t)d : nullptr;
         pa[s] = MODEL == KGE_TRANSH ? a.side_pos[b] : 0.0f;
-        pq[s] = MODEL == KGE_ROTATE ? a.query + b * (int64_t)d : nullptr;
+        pq[s] = (MODEL == KGE_ROTATE || MODEL == KGE_RESCAL) ? a.query + b * (int64_t)d : nullptr;
     }
     const float *pt[SN];
     bool okk[SN];
@@ -379,9 +379,10 @@ __global__ __launch_bounds__(256, KGE_TILE_OCC) void score_neg_mfma_kernel(NegAr
 {
     extern __shared__ __align__(16) char dyn_smem[];
     if (fused_insp_block(fi, reinterpret_cast<uint32_t *>(dyn_smem))) return;
-    static_assert(MODEL == KGE_DISTMULT || MODEL == KGE_COMPLEX || MODEL == KGE_TRANSF, "dot-product scores only");
+    static_assert(MODEL == KGE_DISTMULT || MODEL == KGE_COMPLEX || MODEL == KGE_TRANSF || MODEL == KGE_RESCAL,
+                  "dot-product scores only");
     if (a.pos_blocks > 0 && (int)blockIdx.x - fi.blocks >= a.tile_blocks) {  // the positives carried along
-        if constexpr (MODEL != KGE_TRANSF)
+        if constexpr (MODEL == KGE_DISTMULT || MODEL == KGE_COMPLEX)
             score_pos_body<MODEL, 2, 4>(a.pos, nullptr, (int64_t)((int)blockIdx.x - fi.blocks - a.tile_blocks));
         return;
     }
@@ -405,7 +406,7 @@ __global__ __launch_bounds__(256, KGE_TILE_OCC) void score_neg_mfma_kernel(NegAr
     // (VEC4, 128-bit row loads, is a compile-time choice: as a run-time one the compiler merges the two
     // forms of the raw loads into the scalar one)
 
-    const float *ph[SB], *pr[SB];
+    const float *ph[SB], *pr[SB], *pq[SB];
     bool okb[SB];
 #pragma unroll
     for (int s = 0; s < SB; ++s) {
@@ -414,6 +415,7 @@ __global__ __launch_bounds__(256, KGE_TILE_OCC) void score_neg_mfma_kernel(NegAr
         const int64_t b = (int64_t)c * a.C + (okb[s] ? bl : a.C - 1);
         ph[s] = a.ent + a.h[b] * (int64_t)d;
         pr[s] = a.rel + a.r[b] * (int64_t)a.rel_dim;
+        pq[s] = MODEL == KGE_RESCAL ? a.query + b * (int64_t)d : nullptr;
     }
     const float *pt[SN];
     bool okk[SN];
@@ -433,7 +435,7 @@ __global__ __launch_bounds__(256, KGE_TILE_OCC) void score_neg_mfma_kernel(NegAr
     auto load_slice = [&](int j0, float4 (&qr)[SB][NRAW], float4 (&tr)[SN]) {
         const int j = j0 + scol;
 #pragma unroll
-        for (int s = 0; s < SB; ++s) load_query_raw<MODEL, VEC4>(ph[s], pr[s], nullptr, nullptr, j, okb[s] ? d : 0, half, qr[s]);
+        for (int s = 0; s < SB; ++s) load_query_raw<MODEL, VEC4>(ph[s], pr[s], nullptr, pq[s], j, okb[s] ? d : 0, half, qr[s]);
 #pragma unroll
         for (int s = 0; s < SN; ++s) tr[s] = ld4_raw<VEC4>(pt[s], j, okk[s] ? d : 0);
     };
@@ -573,7 +575,7 @@ static int launch_neg_mp(const NegArgs &a_in, int64_t n_chunks, bool dot_valu, c
     // 64x64 on a 256-big-tile workload with the vector-ALU loop; the matrix-core loop, whose
     // launches are bound by the rows its workgroups pull from L2, does best with 32x64).  The
     // inspector workgroups that share the machine with these launches raise their wave priority.
-    constexpr bool kDotModel = MODEL == KGE_DISTMULT || MODEL == KGE_COMPLEX || MODEL == KGE_TRANSF;
+    constexpr bool kDotModel = MODEL == KGE_DISTMULT || MODEL == KGE_COMPLEX || MODEL == KGE_TRANSF || MODEL == KGE_RESCAL;
     // Rows without 128-bit loads (dim % 4 != 0, unaligned tables) take the 32x32 tile whatever the size:
     // only that tile is compiled in the scalar-load form.
     const int tile = !a.vec ? 2 : big_tiles >= 1024 ? 4 : (kDotModel && !dot_valu ? 3 : 2);  // 2: 32x32, 3: 32x64, 4: 64x64
@@ -665,7 +667,10 @@ int launch_score_neg(const kge_tables *tab, const kge_batch *bat, const float *s
     case KGE_COMPLEX: return launch_neg_mp<KGE_COMPLEX, 2>(a, n_chunks, dv, fi, st);
     case KGE_ROTATE: return launch_neg_mp<KGE_ROTATE, 2>(a, n_chunks, dv, fi, st);
     case KGE_TRANSF: return launch_neg_mp<KGE_TRANSF, 2>(a, n_chunks, dv, fi, st);
-    default: return KGE_EUNSUPPORTED;  // TransR / RESCAL: their projection depends on the positive's relation
+    case KGE_RESCAL:  // negatives that replace the tail: a dot-product tile over the projected rows E[h] Proj[r]
+        if (!query || head) return KGE_EUNSUPPORTED;
+        return launch_neg_mp<KGE_RESCAL, 2>(a, n_chunks, dv, fi, st);
+    default: return KGE_EUNSUPPORTED;  // TransR: its own grouped path
     }
 }
 

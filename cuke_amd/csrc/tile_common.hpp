@@ -87,6 +87,8 @@ __device__ __forceinline__ int pair_len(int d)
 //   TransH    q0 = h + r - al*w (al = w.h), q1 = w
 //   TransF    q0 = 2h + r: score = (h + r).t' + (t' - r).h = (2h + r).t' - r.h, a dot product with
 //             the query plus a constant per positive
+//   RESCAL    q0 = E[h] Proj[r], the projected row that the grouped forward pass left in pq:
+//             score = (h M_r) . t' needs no projection of the negatives at all
 // lim == 0 yields zeros (row outside the tile).
 // RotatE takes its query rows from pq, the [B, d] buffer of rotated heads.
 //
@@ -135,6 +137,8 @@ __device__ __forceinline__ void load_query(const float *ph, const float *pr, con
             }
         }
         q0 = make_float4(q[0], q[1], q[2], q[3]);
+    } else if constexpr (MODEL == KGE_RESCAL) {
+        q0 = ld4<VEC>(pq, j, lim);
     } else if constexpr (MODEL == KGE_ROTATE) {
         // the rotated head h e^{i theta} was written by the positive kernel ([re | im] row pq):
         // a plain load here instead of a sincos per element in every tile that needs the row
@@ -208,6 +212,9 @@ __device__ __forceinline__ void load_query_raw(const float *ph, const float *pr,
 #pragma unroll
             for (int n = 0; n < 4; ++n) raw[n] = make_float4(v[n][0], v[n][1], v[n][2], v[n][3]);
         }
+    } else if constexpr (MODEL == KGE_RESCAL) {
+        raw[0] = ld4_raw<VEC>(pq, j, lim);
+        raw[1] = raw[0];
     } else if constexpr (MODEL == KGE_ROTATE) {
         raw[0] = ld4_raw<VEC>(pq, j, lim);
         raw[1] = ld4_raw<VEC>(pq + half, j, lim);
@@ -247,6 +254,8 @@ __device__ __forceinline__ void combine_query(const float4 (&raw)[N], float al, 
             q[e] = jj < lim ? v : 0.0f;
         }
         q0 = make_float4(q[0], q[1], q[2], q[3]);
+    } else if constexpr (MODEL == KGE_RESCAL) {
+        q0 = mask4<VEC>(raw[0], j, lim);
     } else if constexpr (MODEL == KGE_ROTATE) {
         q0 = mask4<VEC>(raw[0], j, lim);
         q1 = mask4<VEC>(raw[1], j, lim);

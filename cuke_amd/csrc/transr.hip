@@ -1409,13 +1409,129 @@ int launch_transr_plan(const kge_tables *tab, const kge_batch *bat, void *worksp
     return KGE_OK;
 }
 
-size_t transr_bwd_workspace(const kge_tables *tab, const kge_batch *bat) { return make_rplan(tab, bat).total; }
+// ---- RESCAL with shared negatives that replace the tail ---------------------------------------------
+// score(b, k) = (E[h_b] Proj[r_b]) . E[n_k] = q_b . E[n_k]: the negatives need no projection at all.  Forward:
+// the grouped pass leaves q_b (and the positive score q_b . E[t_b]); the pair scores are the dot-product
+// tile of DistMult with q_b as the query rows.  Backward: the gradient tiles give the negatives' rows and
+// G_b = sum_k dneg[b][k] E[n_k] = dL/dq_b from the pairs; with the positive's own term the upstream row of
+// the projected vector is Q_b = dpos[b] E[t_b] + G_b, and dX = Q M^T, dM = X^T Q (X = E[h]) run as the
+// grouped passes over B rows instead of B (1 + N) flattened triples.
+int launch_rescal_neg_tiles(const kge_tables *, const kge_batch *, const float *, const float *, float *, float *, hipStream_t);
+
+struct RescalNegPlan {
+    size_t off_plan, off_dplan, off_xs, off_qs, off_g0, off_occ, off_part_e, off_dpart, total;
+    int64_t tiles, dtiles, dsplit, dslots, nn;
+};
+
+static RescalNegPlan make_rescal_neg_plan(const kge_tables *tab, const kge_batch *bat)
+{
+    RescalNegPlan p{};
+    const RPlan r = make_rplan(tab, bat);
+    const int64_t B = bat->batch, d = tab->dim;
+    p.tiles = r.tiles, p.dtiles = r.dtiles, p.dsplit = r.dsplit, p.dslots = r.dslots;
+    p.nn = bat->chunk > 0 ? (B / bat->chunk) * bat->n_neg : 0;
+    size_t o = 0;
+    auto take = [&](size_t bytes) {
+        const size_t at = o;
+        o += up256(bytes > 0 ? bytes : 1);
+        return at;
+    };
+    p.off_plan = take(sizeof(int32_t) * plan_ints(p.tiles, 0));
+    p.off_dplan = take(sizeof(int32_t) * plan_ints(p.dtiles, p.dsplit));
+    p.off_xs = take(sizeof(float) * (size_t)(B * d));
+    p.off_qs = take(sizeof(float) * (size_t)(B * d));
+    p.off_g0 = take(sizeof(float) * (size_t)(B * d));
+    p.off_occ = take(sizeof(float) * (size_t)((2 * B + p.nn) * d));
+    p.off_part_e = take(sizeof(float) * (size_t)seg_partial_floats(2 * B + p.nn, d));
+    p.off_dpart = take(sizeof(float) * (size_t)(p.dslots * d * d));
+    p.total = o;
+    return p;
+}
+
+size_t transr_bwd_workspace(const kge_tables *tab, const kge_batch *bat)
+{
+    if (tab->model == KGE_RESCAL && bat->neg) return make_rescal_neg_plan(tab, bat).total;
+    return make_rplan(tab, bat).total;
+}
+
+// One wave per sorted position p (triple b = perm[p]): xs[p] = E[h], qs[p] = g E[t] + G[b], occ_t[b] = g v[b].
+__global__ __launch_bounds__(256) void rescal_neg_prep_kernel(const float *ent, const int64_t *h, const int64_t *t, const int32_t *perm,
+                                                              const float *dpos, const float *G, const float *resid, float *xs,
+                                                              float *qs, float *occ_t, int64_t B, int d)
+{
+    const int lane = threadIdx.x & 63;
+    const int64_t p = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (p >= B) return;
+    const int b = perm[p];
+    const float g = dpos ? dpos[b] : 0.0f;
+    const float *eh = ent + h[b] * (int64_t)d, *et = ent + t[b] * (int64_t)d;
+    for (int j = lane * 4; j < d; j += 256) {
+        const float4 vh = *reinterpret_cast<const float4 *>(eh + j), vt = *reinterpret_cast<const float4 *>(et + j);
+        const float4 ve = *reinterpret_cast<const float4 *>(resid + (int64_t)b * d + j);
+        const float4 vg = G ? *reinterpret_cast<const float4 *>(G + (int64_t)b * d + j) : make_float4(0.f, 0.f, 0.f, 0.f);
+        *reinterpret_cast<float4 *>(xs + p * d + j) = vh;
+        *reinterpret_cast<float4 *>(qs + p * d + j) = make_float4(fmaf(g, vt.x, vg.x), fmaf(g, vt.y, vg.y), fmaf(g, vt.z, vg.z), fmaf(g, vt.w, vg.w));
+        *reinterpret_cast<float4 *>(occ_t + (int64_t)b * d + j) = scaled4(g, ve);
+    }
+}
+
+__global__ void rescal_fill_zero_kernel(float *p, int64_t n)
+{
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (int64_t)gridDim.x * blockDim.x) p[i] = 0.0f;
+}
+
+int launch_rescal_neg_bwd(const kge_tables *tab, const kge_batch *bat, const kge_saved *saved, const float *dpos,
+                                 const float *dneg, const kge_grads *grads, void *workspace, size_t workspace_bytes, hipStream_t st)
+{
+    if (bat->neg_mode != KGE_NEG_TAIL) return KGE_EUNSUPPORTED;  // (head negatives: the flattened triples)
+    if (!mfma_path_ok(tab, bat) || gemm_lds_bytes((int)tab->dim) > kMaxGemmLds) return KGE_EUNSUPPORTED;
+    if (bat->fuse_inspection) return KGE_EINVAL;
+    if (!saved->residual || !aligned16(saved->residual) || !grads->aux_rows || !grads->ent_rows) return KGE_EINVAL;
+    if (grads->aux_factor_max != 0) return KGE_EUNSUPPORTED;
+    const RescalNegPlan p = make_rescal_neg_plan(tab, bat);
+    if (!workspace || workspace_bytes < p.total || !aligned16(workspace)) return KGE_EWORKSPACE;
+    if (bat->ent_insp->n != 2 * bat->batch + p.nn) return KGE_ESHAPE;
+    const int64_t B = bat->batch;
+    const int d = (int)tab->dim;
+    char *ws = static_cast<char *>(workspace);
+    float *xs = reinterpret_cast<float *>(ws + p.off_xs), *qs = reinterpret_cast<float *>(ws + p.off_qs);
+    float *g0 = reinterpret_cast<float *>(ws + p.off_g0), *occ = reinterpret_cast<float *>(ws + p.off_occ);
+    const kge_inspection *ri = bat->rel_insp;
+    if (dneg) {
+        const int rc = launch_rescal_neg_tiles(tab, bat, saved->residual, dneg, g0, occ + 2 * B * d, st);
+        timeline_mark(bat->timeline, st, "bwd_tile_kernel");
+        if (rc) return rc;
+    } else if (p.nn > 0) {  // no upstream gradient on the pairs: the negatives' occurrence rows are zero
+        hipLaunchKernelGGL(rescal_fill_zero_kernel, dim3(1024), dim3(256), 0, st, occ + 2 * B * d, p.nn * d);
+    }
+    hipLaunchKernelGGL(rescal_neg_prep_kernel, dim3((unsigned)ceil_div(B, 4)), dim3(256), 0, st, tab->ent, bat->h, bat->t, ri->perm, dpos,
+                       dneg ? g0 : nullptr, saved->residual, xs, qs, occ + B * d, B, d);
+    TilePlan plan = plan_at(ws + p.off_plan, p.tiles, 0), dplan = plan_at(ws + p.off_dplan, p.dtiles, p.dsplit);
+    hipLaunchKernelGGL(transr_plan_kernel, dim3(2), dim3(1024), 0, st, ri->num_unique, ri->seg_offsets, ri->unique_ids, plan, kTM, dplan,
+                       kDmChunk);
+    GemmArgs ga{tab->ent, tab->rel, tab->aux, bat->h, bat->r, bat->t, ri->perm, ri->seg_offsets, ri->num_unique, ri->unique_ids,
+                plan, qs, nullptr, nullptr, nullptr, occ, nullptr, d, tab->norm_p, thin_groups(tab, bat), (int)p.tiles, BwdSrc{}};
+    if (const int rc = allow_lds<2>(gemm_lds_bytes(d))) return rc;
+    hipLaunchKernelGGL(transr_gemm_kernel<2>, dim3((unsigned)(p.tiles + ga.thin_groups)), dim3(256), gemm_lds_bytes(d), st, ga, FusedInsp{});
+    timeline_mark(bat->timeline, st, "transr_gemm_kernel<dX>");
+    const int dm_items = (int)(ceil_div(d, 32) * p.dtiles);
+    DmArgs da{xs, qs, ri->seg_offsets, dplan, grads->aux_rows, reinterpret_cast<float *>(ws + p.off_dpart), d, ri->num_unique, dm_items,
+              BwdSrc{}, nullptr, nullptr, 0};
+    hipLaunchKernelGGL(transr_dm_kernel, dim3((unsigned)(dm_items + thin_groups(tab, bat))), dim3(256), dm_lds_bytes(d), st, da, FusedInsp{});
+    timeline_mark(bat->timeline, st, "transr_dm_kernel");
+    KGE_CHECK_LAUNCH();
+    if (bat->insp_ready && hipStreamWaitEvent(st, reinterpret_cast<hipEvent_t>(bat->insp_ready), 0) != hipSuccess)
+        return KGE_ELAUNCH;
+    const SegJob jobs[1] = {{occ, bat->ent_insp, d, grads->ent_rows, reinterpret_cast<float *>(ws + p.off_part_e), false}};
+    const SumRider finish = dm_finish_rider(da, p.dsplit);
+    return launch_seg_reduce_jobs(jobs, 1, st, bat->timeline, &finish);
+}
 
 int launch_transr_bwd(const kge_tables *tab, const kge_batch *bat, const kge_saved *saved, const float *dpos,
                       const kge_grads *grads, void *workspace, size_t workspace_bytes, hipStream_t st)
 {
     const bool rescal = tab->model == KGE_RESCAL;
-    if (bat->neg) return KGE_EUNSUPPORTED;  // positives only for the projection models
+    if (bat->neg) return KGE_EUNSUPPORTED;  // (shared negatives: launch_transr_neg_bwd / launch_rescal_neg_bwd)
     if (!mfma_path_ok(tab, bat) || gemm_lds_bytes((int)tab->dim) > kMaxGemmLds) return KGE_EUNSUPPORTED;
     if (!saved->residual || !grads->aux_rows || !grads->ent_rows) return KGE_EINVAL;
     if (!rescal && (!grads->rel_rows || (tab->norm_p == 2 && !saved->pos))) return KGE_EINVAL;

@@ -279,7 +279,12 @@ class KGEModel:
         (apps/examples/examples.py:1404-1444); ``'head'``: (neg_k, r_b, t_b), the head-corrupted batches of
         the reference's sampler (apps/kge/data/sampler.py:287-353)."""
         if neg is not None and self.model == "RESCAL":
-            return self._score_projected_negatives(h, r, t, neg, chunk, neg_mode)
+            # tail negatives: (E[h] Proj[r]) . E[t'] is a dot-product tile over the B projected rows; head
+            # negatives and shapes outside the grouped kernels: the pairs as explicit triples
+            if neg_mode != "tail" or self.dim % 4 != 0 or self.dim > 1024:
+                return self._score_projected_negatives(h, r, t, neg, chunk, neg_mode)
+            if rel_insp is None:
+                rel_insp = inspect([_index(r, "r", self.dev)], self.n_rel)
         if neg is not None and self.model == "TransR":
             # every negative is projected once per (relation, chunk) group of the batch; needs the
             # relation groups.  Shapes outside the grouped kernels (dim % 4, dim > 1024) take the

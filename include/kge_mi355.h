@@ -253,8 +253,14 @@ int kge_residual_fwd(const kge_tables *tab, const kge_batch *bat, float *out, vo
  * of the batch instead of once per pair.  pos, neg and residual ([B, dim], the positives' residual
  * rows) come out of the one call; the workspace (kge_score_fwd_workspace with bat->neg set) keeps
  * the group list and the projected rows and must be handed to kge_score_bwd as
- * kge_saved.fwd_workspace.  RESCAL with shared negatives, and TransR shapes outside the grouped
- * kernels, are scored through kge_flatten_negatives.
+ * kge_saved.fwd_workspace.  TransR shapes outside the grouped kernels are scored through
+ * kge_flatten_negatives.
+ * RESCAL with shared negatives that replace the tail (KGE_NEG_TAIL): the pair score
+ * (E[h] Proj[r]) . E[t'] needs no projection of the negatives, so pos, neg and `residual` ([B, dim],
+ * the projected rows E[h] Proj[r], required) come out of one call: the grouped pass over the B
+ * positives, then the dot-product tile kernel of DistMult with the projected rows as its query rows.
+ * kge_score_bwd chains the pairs' gradient through the same B rows.  KGE_NEG_HEAD returns
+ * KGE_EUNSUPPORTED here (kge_flatten_negatives covers it).
  * TransE / RotatE with shared negatives on small batches (the 32 x 32 pair tiles would leave one or
  * two workgroups per CU): given kge_score_fwd_workspace() bytes of workspace the reduction axis of
  * every tile is split over up to four workgroups (partial score planes in the workspace, a finishing
@@ -363,10 +369,9 @@ int kge_build_index(const int64_t *r, int64_t *uniq, int64_t *buf, int64_t *cnt,
  * Shared negatives written out as explicit triples, the way the reference's neg_transR defines
  * them (apps/examples/examples.py:1447-1480: every view is flattened to batch * blocksize rows).
  * Outputs have B * (1 + n_neg) entries: the B positives first, then row B + b * n_neg + k =
- * (h[b], r[b], neg[(b / chunk) * n_neg + k]).  RESCAL scores shared negatives through this list
- * and the grouped per-relation kernels (the projection depends on the positive's relation, so a
- * negative row cannot be staged once per chunk as for the other models); TransR has the grouped
- * form of kge_score_fwd and uses the list only for shapes that form does not take.
+ * (h[b], r[b], neg[(b / chunk) * n_neg + k]).  TransR and RESCAL have grouped forms of kge_score_fwd
+ * (see there) and use the list only for what those do not take: shapes outside the grouped kernels,
+ * and RESCAL with negatives that replace the head.
  */
 int kge_flatten_negatives(const kge_batch *bat, int64_t *h_flat, int64_t *r_flat, int64_t *t_flat,
                           void *stream);

@@ -259,6 +259,51 @@ def test_shared_negatives_through_flattened_triples(oracle, model):
     assert_close(g.aux_rows.cpu().numpy(), ref.aux_rows, what="projection gradients", rows=True)
 
 
+@pytest.mark.parametrize("shape", [
+    dict(dim=40, batch=48, chunk=16, n_neg=12, n_rel=6),
+    dict(dim=200, batch=512, chunk=64, n_neg=64, n_rel=50),    # Zipf relations, many thin groups
+    dict(dim=64, batch=300, chunk=300, n_neg=33, n_rel=1),     # one relation, odd N, ragged tiles
+    dict(dim=256, batch=1024, chunk=256, n_neg=256, n_rel=300),
+    dict(dim=16, batch=7, chunk=7, n_neg=1, n_rel=3),
+])
+def test_rescal_shared_negatives_as_a_dot_product_tile(oracle, shape):
+    """RESCAL with negatives that replace the tail: (E[h] Proj[r]) . E[t'] from the B projected rows and the
+    dot-product tile kernel (no projection of the negatives, no flattened triples), forward and backward
+    against the oracle's explicit pairs; with missing upstream gradients; and through TrainStep."""
+    from cuke_amd.kge import TrainStep
+    w = synth.custom_workload("RESCAL", n_ent=400, norm_p=2, sigma=0.2, rel_zipf=1.1, ent_zipf=1.1, seed=13, **shape)
+    a = w.arrays
+    m, ix = gpu_model(w)
+    fw = m.score(ix["h"], ix["r"], ix["t"], ix["neg"], w.chunk)
+    assert fw.flat_pos is None, "the flattened triples ran instead of the tile path"
+    pos, negs = oracle.score("RESCAL", a["E"], a["R"], a["A"], a["h"], a["r"], a["t"], a["neg"], w.chunk)
+    assert_close(fw.pos.cpu().numpy(), pos, what="pos")
+    assert_close(fw.neg.cpu().numpy(), negs, what="neg")
+    rng = np.random.default_rng(5)
+    dpos = rng.standard_normal(w.batch).astype(np.float32)
+    dneg = rng.standard_normal((w.batch, w.n_neg)).astype(np.float32)
+    for gp, gn, tag in ((dpos, dneg, "both"), (None, dneg, "pairs only"), (dpos, None, "positives only")):
+        g = m.backward(fw, None if gp is None else torch.from_numpy(gp).cuda(), None if gn is None else torch.from_numpy(gn).cuda())
+        ref = oracle.backward("RESCAL", a["E"], a["R"], a["A"], a["h"], a["r"], a["t"], a["neg"], w.chunk,
+                              gp if gp is not None else np.zeros_like(dpos), gn if gn is not None else np.zeros_like(dneg))
+        assert np.array_equal(g.ent_ids.cpu().numpy(), ref.ent_ids) and np.array_equal(g.rel_ids.cpu().numpy(), ref.rel_ids)
+        assert_close(g.ent_rows.cpu().numpy(), ref.ent_rows, what=f"{tag}: entity rows", rows=True)
+        assert_close(g.aux_rows.cpu().numpy(), ref.aux_rows, what=f"{tag}: projection gradients", rows=True)
+    # the flattened formulation of the reference must agree
+    flat = m._score_projected_negatives(ix["h"], ix["r"], ix["t"], ix["neg"], w.chunk)
+    assert_close(fw.neg.cpu().numpy(), flat.neg.cpu().numpy(), what="tile path vs flattened triples")
+    step = TrainStep(m, ix["h"], ix["r"], ix["t"], ix["neg"], w.chunk, dpos=torch.from_numpy(dpos).cuda(),
+                     dneg=torch.from_numpy(dneg).cuda())
+    ref = oracle.backward("RESCAL", a["E"], a["R"], a["A"], a["h"], a["r"], a["t"], a["neg"], w.chunk, dpos, dneg)
+    for tag, kw in (("side stream", {}), ("one stream", dict(overlap=False))):
+        step.run(**kw)
+        torch.cuda.synchronize()
+        g = step.sparse_grads()
+        assert_close(step.neg.cpu().numpy(), negs, what=f"TrainStep {tag} neg")
+        assert_close(g.ent_rows.cpu().numpy(), ref.ent_rows, what=f"TrainStep {tag} entity rows", rows=True)
+        assert_close(g.aux_rows.cpu().numpy(), ref.aux_rows, what=f"TrainStep {tag} projection gradients", rows=True)
+
+
 def _neg_case(oracle, w, mode, what):
     a = w.arrays
     if w.lattice:  # keep the projected rows exact too: projections on a coarse grid (L1 gradients are sums of signs)
