@@ -1328,8 +1328,17 @@ static size_t fwd_plan_bytes(const kge_tables *tab, const kge_batch *bat)
     return up256(sizeof(int32_t) * plan_ints(max_tiles(tab, bat), 0));
 }
 
+static bool pad_path_ok(const kge_tables *, const kge_batch *);
+static size_t transr_fwd_workspace_padded(const kge_tables *, const kge_batch *);
+static size_t transr_bwd_workspace_padded(const kge_tables *, const kge_batch *);
+static int launch_transr_fwd_padded(const kge_tables *, const kge_batch *, float *, float *, void *, size_t, hipStream_t);
+static int launch_transr_plan_padded(const kge_tables *, const kge_batch *, void *, size_t, hipStream_t);
+static int launch_transr_bwd_padded(const kge_tables *, const kge_batch *, const kge_saved *, const float *, const kge_grads *, void *,
+                                    size_t, hipStream_t);
+
 size_t transr_fwd_workspace(const kge_tables *tab, const kge_batch *bat)
 {
+    if (pad_path_ok(tab, bat)) return transr_fwd_workspace_padded(tab, bat);  // row width not a multiple of four
     const RPlan p = make_rplan(tab, bat);
     return fwd_plan_bytes(tab, bat) + up256(sizeof(int32_t) * plan_ints(p.dtiles, p.dsplit));
 }
@@ -1354,6 +1363,8 @@ int launch_transr_fwd(const kge_tables *tab, const kge_batch *bat, float *pos, f
                       size_t workspace_bytes, hipStream_t st)
 {
     if (bat->batch == 0) return KGE_OK;
+    if (pad_path_ok(tab, bat) && workspace && workspace_bytes >= transr_fwd_workspace_padded(tab, bat))
+        return launch_transr_fwd_padded(tab, bat, pos, resid, workspace, workspace_bytes, st);
     const bool rescal = tab->model == KGE_RESCAL;
     const bool grouped = mfma_path_ok(tab, bat) && workspace && workspace_bytes >= transr_fwd_workspace(tab, bat) &&
                          gemm_lds_bytes((int)tab->dim) <= kMaxGemmLds;
@@ -1397,6 +1408,7 @@ int launch_transr_plan(const kge_tables *tab, const kge_batch *bat, void *worksp
 {
     if (bat->batch == 0) return KGE_OK;
     if (bat->neg) return KGE_EUNSUPPORTED;  // the shared-negative path plans its own row list
+    if (pad_path_ok(tab, bat)) return launch_transr_plan_padded(tab, bat, workspace, workspace_bytes, st);
     if (!mfma_path_ok(tab, bat) || gemm_lds_bytes((int)tab->dim) > kMaxGemmLds) return KGE_EUNSUPPORTED;
     if (!workspace || workspace_bytes < transr_fwd_workspace(tab, bat)) return KGE_EWORKSPACE;
     const kge_inspection *ri = bat->rel_insp;
@@ -1451,6 +1463,7 @@ static RescalNegPlan make_rescal_neg_plan(const kge_tables *tab, const kge_batch
 size_t transr_bwd_workspace(const kge_tables *tab, const kge_batch *bat)
 {
     if (tab->model == KGE_RESCAL && bat->neg) return make_rescal_neg_plan(tab, bat).total;
+    if (pad_path_ok(tab, bat)) return transr_bwd_workspace_padded(tab, bat);
     return make_rplan(tab, bat).total;
 }
 
@@ -1532,6 +1545,7 @@ int launch_transr_bwd(const kge_tables *tab, const kge_batch *bat, const kge_sav
 {
     const bool rescal = tab->model == KGE_RESCAL;
     if (bat->neg) return KGE_EUNSUPPORTED;  // (shared negatives: launch_transr_neg_bwd / launch_rescal_neg_bwd)
+    if (pad_path_ok(tab, bat)) return launch_transr_bwd_padded(tab, bat, saved, dpos, grads, workspace, workspace_bytes, st);
     if (!mfma_path_ok(tab, bat) || gemm_lds_bytes((int)tab->dim) > kMaxGemmLds) return KGE_EUNSUPPORTED;
     if (!saved->residual || !grads->aux_rows || !grads->ent_rows) return KGE_EINVAL;
     if (!rescal && (!grads->rel_rows || (tab->norm_p == 2 && !saved->pos))) return KGE_EINVAL;
@@ -1615,5 +1629,6 @@ int launch_transr_bwd(const kge_tables *tab, const kge_batch *bat, const kge_sav
 }
 
 #include "transr_neg.hpp"
+#include "transr_pad.hpp"
 
 }  // namespace kge

@@ -26,6 +26,10 @@ def grouped_forward(m, ix):
     dict(dim=496, batch=24, n_rel=20),
     dict(dim=512, batch=4096, n_rel=30),     # the reference's own sweep shapes (apps/kge/scripts/test_fig9c_cuke.sh):
     dict(dim=1024, batch=1024, n_rel=12),    # left-operand tiles of 66.5 KB and 129 KB in LDS
+    dict(dim=50, batch=300, n_rel=40),       # row widths that are not multiples of four: the batch is copied into a
+    dict(dim=101, batch=64, n_rel=5),        # padded compact problem (dim is a free variable of the reference's
+    dict(dim=202, batch=700, n_rel=90),      # transR, apps/kge/kge.py:321-343)
+    dict(dim=7, batch=9, n_rel=2),
 ])
 @pytest.mark.parametrize("p", [1, 2])
 def test_grouped_forward(oracle, model, shape, p):
@@ -56,6 +60,10 @@ def test_grouped_forward(oracle, model, shape, p):
     dict(dim=496, batch=24, n_rel=20),
     dict(dim=512, batch=4096, n_rel=30),
     dict(dim=1024, batch=1024, n_rel=12),
+    dict(dim=50, batch=300, n_rel=40),
+    dict(dim=101, batch=64, n_rel=5),
+    dict(dim=202, batch=700, n_rel=90),
+    dict(dim=7, batch=9, n_rel=2),
 ])
 @pytest.mark.parametrize("p", [1, 2])
 def test_grouped_backward(oracle, model, shape, p):
@@ -195,6 +203,45 @@ def test_train_step_factored_all_issue_forms(oracle):
         step.run(fused=True)
         check(ws[0], "fused inspection")
     step.run(fused=False)
+    check(ws[0], "side-stream inspection")
+    step.stage(batch=1)
+    for i in (1, 2, 0):
+        step.stage(batch=(i + 1) % 3)
+        step.run(pipeline=True)
+        check(ws[i], f"staged batch {i}")
+    step.run(pipeline=True)
+    check(ws[1], "drained")
+
+
+def test_train_step_with_an_odd_row_width(oracle):
+    """TransR at dim 50 through TrainStep: one stream, side-stream inspection and the staged issue (tile plans a
+    batch ahead, kge_transr_plan on the padded problem), against the oracle."""
+    from cuke_amd.kge import TrainStep
+    ws = [synth.custom_workload("TransR", n_ent=300, n_rel=25, dim=50, batch=256, norm_p=2, sigma=0.2, rel_zipf=1.2, seed=s)
+          for s in range(3)]
+    m, ix0 = gpu_model(ws[0])
+    step = TrainStep(m, ix0["h"], ix0["r"], ix0["t"])
+    assert not step.fusable
+    for w in ws[1:]:
+        ix = {k: torch.from_numpy(w.arrays[k]).cuda() for k in ("h", "r", "t")}
+        step.add_batch(ix["h"], ix["r"], ix["t"])
+    a0 = ws[0].arrays
+
+    def check(w, tag):
+        torch.cuda.synchronize()
+        a = w.arrays
+        pos, _ = oracle.score("TransR", a0["E"], a0["R"], a0["A"], a["h"], a["r"], a["t"], p=2)
+        assert_close(step.pos.cpu().numpy(), pos, what=f"{tag} scores")
+        ref = oracle.backward("TransR", a0["E"], a0["R"], a0["A"], a["h"], a["r"], a["t"], dpos=step.dpos.cpu().numpy(), p=2)
+        g = step.sparse_grads()
+        assert np.array_equal(g.rel_ids.cpu().numpy(), ref.rel_ids), tag
+        assert_close(g.ent_rows.cpu().numpy(), ref.ent_rows, what=f"{tag} entity rows", rows=True)
+        assert_close(g.rel_rows.cpu().numpy(), ref.rel_rows, what=f"{tag} relation rows", rows=True)
+        assert_close(g.aux_rows.cpu().numpy(), ref.aux_rows, what=f"{tag} projection gradients", rows=True)
+
+    step.run(overlap=False)
+    check(ws[0], "one stream")
+    step.run()
     check(ws[0], "side-stream inspection")
     step.stage(batch=1)
     for i in (1, 2, 0):
