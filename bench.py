@@ -558,6 +558,7 @@ def run_workload(name, args, torch, factor_max=0):
     # while batch i's step runs; every timed step still inspects one batch and runs one forward / loss /
     # backward.  The riding (fused) inspection of `direct` is not used in this form.
     ms_staged = None
+    ref_bits0 = None
     if do_bwd and not args.no_staged:
         state = {"next": 0}
 
@@ -579,7 +580,7 @@ def run_workload(name, args, torch, factor_max=0):
         if not same_bits(torch, step, ref_bits):
             raise SpotCheckError(f"{w.name}: the staged issue's outputs differ from the direct issue's for batch 0")
         check["staged_equals_direct_bits"] = True
-        del ref_bits
+        ref_bits0 = ref_bits
         step.stage(batch=state["next"])          # one batch ahead from here on
         state["next"] = (state["next"] + 1) % nb
         if nb >= 3:
@@ -591,6 +592,27 @@ def run_workload(name, args, torch, factor_max=0):
         else:
             step.run(pipeline=True)
             torch.cuda.synchronize()
+
+    # The staged issue from native code: the same launches, one library call per step (kge_train_step_staged).
+    ms_native = None
+    if do_bwd and not args.no_staged and nb >= 3:
+        step.run_native(None, 0)
+        step.run_native(0, 1)
+        torch.cuda.synchronize()
+        if ref_bits0 is not None and not same_bits(torch, step, ref_bits0):
+            raise SpotCheckError(f"{w.name}: the native staged issue differs from the direct issue for batch 0")
+        check["native_equals_direct_bits"] = True
+        state = {"cur": 1}
+
+        def native_step():
+            cur = state["cur"]
+            state["cur"] = (cur + 1) % nb
+            step.run_native(cur, (cur + 1) % nb)
+
+        ms_native = timed(native_step)
+        torch.cuda.synchronize()
+        if ms_native < ms:
+            issue, ms = "staged_native", ms_native
 
     # DistMult / ComplEx: the same rotating loop with the pair sums of the tile kernels on the vector ALUs
     ms_forms = None
@@ -663,7 +685,7 @@ def run_workload(name, args, torch, factor_max=0):
                    "backward": do_bwd, "loss": w.loss, "issue": issue, "rotating_batches": nb, "warmup_min_ms": WARMUP_MIN_S * 1e3,
                    "pair_sums": "matrix cores, fp32" if w.model in ("DistMult", "ComplEx") and w.chunk else "vector ALUs",
                    "ms_per_step_rotating_direct": ms_rot, "ms_per_step_rotating_graph": ms_graph,
-                   "ms_per_step_rotating_staged": ms_staged,
+                   "ms_per_step_rotating_staged": ms_staged, "ms_per_step_rotating_staged_native": ms_native,
                    "ms_per_step_same_batch": ms_same, "ms_per_step_by_pair_sum_unit": ms_forms,
                    "scores_per_step": scores, "positives_per_s": w.batch / (ms * 1e-3),
                    "unique_entity_rows": u_ent, "unique_relation_rows": u_rel,

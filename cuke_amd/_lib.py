@@ -66,6 +66,20 @@ class Grads(C.Structure):
                 ("aux_x", C.c_void_p), ("aux_q", C.c_void_p), ("aux_factor_max", C.c_int32), ("reserved", C.c_int32)]
 
 
+class StepBatch(C.Structure):
+    _fields_ = [("bat", Batch), ("fwd_workspace", C.c_void_p), ("fwd_workspace_bytes", C.c_size_t),
+                ("inspected", C.c_void_p), ("planned", C.c_void_p), ("released", C.c_void_p),
+                ("released_valid", C.c_int32), ("reserved", C.c_int32)]
+
+
+class StepBuffers(C.Structure):
+    _fields_ = [("pos", C.c_void_p), ("neg", C.c_void_p), ("side_pos", C.c_void_p), ("side_neg", C.c_void_p),
+                ("residual", C.c_void_p), ("fwd_workspace", C.c_void_p), ("fwd_workspace_bytes", C.c_size_t),
+                ("loss", C.c_void_p), ("margin", C.c_float), ("sign", C.c_float), ("loss_workspace", C.c_void_p),
+                ("loss_workspace_bytes", C.c_size_t), ("dpos", C.c_void_p), ("dneg", C.c_void_p), ("grads", Grads),
+                ("bwd_workspace", C.c_void_p), ("bwd_workspace_bytes", C.c_size_t)]
+
+
 EXPORTS = {
     # name: (restype, argtypes)
     "kge_strerror": (C.c_char_p, [C.c_int]),
@@ -106,6 +120,8 @@ EXPORTS = {
                                           C.c_void_p]),
     "kge_sparse_adagrad_factored": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int64, C.POINTER(Inspection), C.POINTER(Grads),
                                               C.c_float, C.c_float, C.c_void_p]),
+    "kge_train_step_staged": (C.c_int, [C.POINTER(Tables), C.POINTER(StepBatch), C.POINTER(StepBatch), C.POINTER(StepBuffers),
+                                        C.c_void_p, C.c_void_p]),
     "kge_sample_negatives": (C.c_int, [C.c_void_p, C.c_int64, C.c_int64, C.c_uint64, C.c_uint64, C.c_void_p]),
     "kge_check_indices": (C.c_int, [C.c_void_p, C.c_int64, C.c_int64, C.c_void_p, C.c_void_p]),
 }

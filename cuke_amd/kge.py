@@ -1009,6 +1009,61 @@ class TrainStep:
             self.backward(st)
         main.wait_stream(side)                                   # join
 
+    # ---- the staged issue from native code: one library call per step ----
+    def _native_state(self):
+        """kge_step_batch per batch (events created once) and the kge_step_buffers of this TrainStep."""
+        if getattr(self, "_native", None) is not None:
+            return self._native
+        main = torch.cuda.current_stream()
+
+        def event():
+            ev = torch.cuda.Event()
+            ev.record(main)       # (torch creates the underlying event at its first record)
+            return ev
+
+        batches = []
+        for s_ in self._sets:
+            sb = _lib.StepBatch()
+            sb.bat = s_.bat
+            sb.bat.insp_ready, sb.bat.fuse_inspection, sb.bat.plans_ready, sb.bat.timeline = None, 0, 0, None
+            if self._plans_per_set:
+                if getattr(s_, "ws_f", None) is None:
+                    s_.ws_f = torch.empty(max(self._ws_f_bytes, 1), dtype=torch.uint8, device=self.m.dev)
+                sb.fwd_workspace, sb.fwd_workspace_bytes = s_.ws_f.data_ptr(), self._ws_f_bytes
+            s_.native_events = [event() for _ in range(3)]
+            sb.inspected, sb.planned, sb.released = (e.cuda_event for e in s_.native_events)
+            sb.released_valid = 0
+            batches.append(sb)
+        buf = _lib.StepBuffers()
+        for name in ("pos", "neg", "side_pos", "side_neg", "residual", "dpos", "dneg"):
+            t = getattr(self, name)
+            setattr(buf, name, t.data_ptr() if t is not None else None)
+        buf.fwd_workspace, buf.fwd_workspace_bytes = self._ws_f.data_ptr(), self._ws_f_bytes
+        if self.loss_kind == "margin":
+            buf.loss, buf.margin, buf.sign = self.loss.data_ptr(), self.margin, self.sign
+            buf.loss_workspace, buf.loss_workspace_bytes = self._ws_l.data_ptr(), self._ws_l.numel()
+        buf.grads = self.grads
+        buf.bwd_workspace, buf.bwd_workspace_bytes = self._ws_b.data_ptr(), self._ws_b_bytes
+        torch.cuda.synchronize()
+        self._native = (batches, buf)
+        return self._native
+
+    def run_native(self, cur, nxt) -> None:
+        """The staged issue in ONE library call (kge_train_step_staged): the step of batch ``cur`` on the current
+        stream and, on the side stream, the inspection of batch ``nxt`` (TransR / RESCAL: its tile plans too) for
+        the call that follows.  ``cur=None`` only stages ``nxt`` (in front of the first step); ``nxt=None`` only
+        runs ``cur``.  Same launches in the same order as ``stage(batch=nxt)`` + ``run(pipeline=True)``, hence
+        the same results bit for bit; what it saves is the host's time per step."""
+        if self._staged or self._pipelined:
+            raise KgeError("run_native() cannot be mixed with the staged pipeline")
+        batches, buf = self._native_state()
+        st = C.c_void_p(_current_stream(self._dev_index).cuda_stream)
+        _lib.check(self.L.kge_train_step_staged(C.byref(self.m._tab), C.byref(batches[cur]) if cur is not None else None,
+                                                C.byref(batches[nxt]) if nxt is not None else None, C.byref(buf), st,
+                                                C.c_void_p(self.side.cuda_stream)), "kge_train_step_staged")
+        if cur is not None:
+            self.use_batch(cur)
+
     def sparse_grads(self) -> SparseGrads:
         ue, ur = self.ent_insp.num_unique, self.rel_insp.num_unique
         return SparseGrads(self.ent_insp.unique_ids[:ue], self.ent_rows[:ue], self.rel_insp.unique_ids[:ur],

@@ -413,6 +413,55 @@ int kge_sparse_adagrad_factored(float *proj, float *state, int64_t dim, const kg
  */
 int kge_sample_negatives(int64_t *out, int64_t count, int64_t n_ent, uint64_t seed, uint64_t step, void *stream);
 
+/*
+ * One step of a staged training loop in ONE call (host-side sequencing only; no counterpart in the
+ * reference, which has no training loop).  It enqueues what a host loop would enqueue with seven to ten
+ * calls: on `side_stream` the inspection of the NEXT batch (TransR / RESCAL without negatives: the relation
+ * inspection, the tile plans into next->fwd_workspace, then the entity inspection), on `stream` the step
+ * of the CURRENT batch -- kge_score_fwd, kge_margin_loss when buf->loss is set, kge_score_bwd -- and the
+ * events between the two streams.  For steps so short (tens of microseconds) that the host's per-call
+ * overhead, not the device, would set the pace.
+ *   cur == NULL   only stage `next` (in front of the first step);  next == NULL   only run `cur`.
+ * A kge_step_batch keeps what belongs to one batch across steps: its index arrays and inspections
+ * (bat.insp_jobs[0] = the entity index set, [1] = the relations; bat.ent_insp / rel_insp point to their
+ * `out`), and three events the caller creates once (hipEventCreate; default flags are fine):
+ *   inspected  recorded on side_stream behind the batch's inspection; kge_score_bwd waits for it right
+ *              before its segmented reduction (kge_batch.insp_ready)
+ *   planned    TransR / RESCAL without negatives: recorded behind the relation inspection and the tile
+ *              plans; `stream` waits for it before the forward pass.  Else unused (may be NULL).
+ *   released   recorded on `stream` behind the step; a later staging of the same kge_step_batch makes
+ *              side_stream wait for it before it overwrites the inspection (released_valid says whether
+ *              it has been recorded yet; zero-initialise it).
+ * Scores, gradients and workspaces (kge_step_buffers) are shared by all batches; sizes as for the
+ * individual calls.  buf->loss == NULL: dpos / dneg are the caller's upstream gradients (inputs).
+ * Results are those of the individual calls, bit for bit (the same launches in the same order).
+ */
+typedef struct kge_step_batch {
+    kge_batch bat;
+    void *fwd_workspace;        /* TransR / RESCAL without negatives: this batch's own forward workspace (plans), else NULL */
+    size_t fwd_workspace_bytes;
+    void *inspected, *planned, *released;  /* hipEvent_t */
+    int32_t released_valid;
+    int32_t reserved;
+} kge_step_batch;
+
+typedef struct kge_step_buffers {
+    float *pos, *neg, *side_pos, *side_neg, *residual;  /* as kge_score_fwd */
+    void *fwd_workspace;        /* for batches without one of their own */
+    size_t fwd_workspace_bytes;
+    float *loss;                /* [1] or NULL */
+    float margin, sign;
+    void *loss_workspace;
+    size_t loss_workspace_bytes;
+    float *dpos, *dneg;         /* [B], [B, n_neg] (either may be NULL = 0 where kge_score_bwd allows it) */
+    kge_grads grads;
+    void *bwd_workspace;
+    size_t bwd_workspace_bytes;
+} kge_step_buffers;
+
+int kge_train_step_staged(const kge_tables *tab, kge_step_batch *cur, kge_step_batch *next, const kge_step_buffers *buf,
+                          void *stream, void *side_stream);
+
 /* Sets flag[0] (int32, caller-zeroed) to 1 if any idx[i] is outside [0, n_rows). */
 int kge_check_indices(const int64_t *idx, int64_t n, int64_t n_rows, int32_t *flag, void *stream);
 

@@ -56,3 +56,63 @@ def test_training_steps_track_the_oracle(oracle, model, p, opt):
     assert_close(E.cpu().numpy(), Eo, what=f"{model} {opt} entity table after 6 steps")
     assert_close(R.cpu().numpy(), Ro, what=f"{model} {opt} relation table after 6 steps")
     assert all(after < before for before, after in losses), losses
+
+
+@pytest.mark.parametrize("model,kw", [
+    ("DistMult", dict(chunk=64, n_neg=32)),
+    ("RotatE", dict(chunk=64, n_neg=32, loss="margin")),
+    ("TransH", dict(chunk=32, n_neg=16, norm_p=1)),
+    ("TransR", dict()),                          # relation groups and tile plans a batch ahead
+    ("TransR", dict(chunk=32, n_neg=8)),         # grouped shared negatives: relations inspected by the step itself
+    ("RESCAL", dict(chunk=64, n_neg=16)),
+])
+def test_native_staged_step_equals_the_call_by_call_issue(oracle, model, kw):
+    """kge_train_step_staged (one library call per step) against stage() + run(pipeline=True) of the same
+    batches: the same launches in the same order, so the outputs must be the same bits; and against the oracle."""
+    from cuke_amd.kge import TrainStep
+    from helpers import gpu_model
+    kw = dict(kw)
+    loss = kw.pop("loss", "sum")
+    lattice = kw.get("norm_p") == 1
+    ws = [synth.custom_workload(model, n_ent=400, n_rel=12, dim=48, batch=256, sigma=0.2, gamma=4.0, rel_zipf=1.1, ent_zipf=1.1,
+                                seed=20 + s, lattice=lattice, **kw) for s in range(3)]
+    m, ix0 = gpu_model(ws[0])
+    sign = 1.0 if model in ("DistMult", "RotatE", "RESCAL") else -1.0
+
+    def make():
+        st = TrainStep(m, ix0["h"], ix0["r"], ix0["t"], ix0.get("neg"), ws[0].chunk or None, loss=loss, margin=1.0, sign=sign)
+        for w in ws[1:]:
+            ix = {k: torch.from_numpy(w.arrays[k]).cuda() for k in ("h", "r", "t", "neg") if k in w.arrays}
+            st.add_batch(ix["h"], ix["r"], ix["t"], ix.get("neg"))
+        return st
+
+    def outputs(st):
+        torch.cuda.synchronize()
+        g = st.sparse_grads()
+        return [x.clone() for x in (st.pos, g.ent_ids, g.ent_rows, g.rel_ids) if x is not None] + \
+               [x.clone() for x in (st.neg, g.rel_rows, g.aux_rows) if x is not None]
+
+    ref_step, nat = make(), make()
+    order = [0, 1, 2, 0, 1]
+    want = []
+    ref_step.stage(batch=order[0])
+    for i, b in enumerate(order):
+        if i + 1 < len(order):
+            ref_step.stage(batch=order[i + 1])
+        ref_step.run(pipeline=True)
+        want.append(outputs(ref_step))
+    nat.run_native(None, order[0])
+    for i, b in enumerate(order):
+        nat.run_native(b, order[i + 1] if i + 1 < len(order) else None)
+        got = outputs(nat)
+        assert len(got) == len(want[i]) and all(torch.equal(x, y) for x, y in zip(got, want[i])), f"step {i} (batch {b})"
+    # the last step against the oracle
+    a0, a = ws[0].arrays, ws[order[-1]].arrays
+    dpos = nat.dpos.cpu().numpy()
+    dneg = nat.dneg.cpu().numpy() if nat.dneg is not None else None
+    ref = oracle.backward(model, a0["E"], a0["R"], a0["A"], a["h"], a["r"], a["t"], a.get("neg"), ws[0].chunk, dpos, dneg,
+                          p=ws[0].norm_p)
+    g = nat.sparse_grads()
+    assert np.array_equal(g.ent_ids.cpu().numpy(), ref.ent_ids)
+    out = (1e-5, 4.0) if model == "RotatE" else None
+    assert_close(g.ent_rows.cpu().numpy(), ref.ent_rows, what=f"{model} entity rows", rows=True, outliers=out)
