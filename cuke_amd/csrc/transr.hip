@@ -33,13 +33,7 @@ constexpr int kRing = KGE_TR_RING;  // supersteps of B operands kept in flight p
 #define KGE_TR_DM_RING 4
 #endif
 constexpr int kDmRing = KGE_TR_DM_RING;  // the same for the dM kernel's operand stages
-#ifndef KGE_TR_SPLIT_BWD
-#define KGE_TR_SPLIT_BWD 1
-#endif
-// dX and dM as two launches (default) or as one.  Measured on the TransR benchmark configuration, one box: two
-// launches 0.160 ms per step against 0.171 with every projection gradient dense; 0.151 against 0.150 with the
-// thin groups factored.
-constexpr bool kSplitBwd = KGE_TR_SPLIT_BWD != 0;
+
 constexpr int kThin = 4;            // a group's last tile with at most this many triples takes the thin path
 constexpr int kThinRing = 8;        // 128-bit projection loads in flight per thread on the thin path
 constexpr int kMaxDimMfma = 1024;
@@ -64,7 +58,22 @@ struct TilePlan {
     int32_t *split_seg;   // [max_split] group of the split
     int32_t *split_first; // [max_split] first partial slot
     int32_t *split_cnt;   // [max_split] number of partial slots
+    // Chunked plan only: the dM kernel's work as compact lists.  How many entries a batch has is only
+    // known on the device, and a grid sized for the worst case (one chunk per possible relation, seven row
+    // blocks per chunk, one thin workgroup per possible relation: eleven thousand workgroups for a few
+    // hundred items) spends 25 us merely being dispatched: the kernel runs kDmWgs workgroups that stride
+    // over the lists instead.
+    int32_t *num_items;   // [2] long items (from the front of item_*), small-group items (from the back)
+    int32_t *item_tile, *item_blk;  // [max_items] (tile, 32-row block), or (tile, -1) = every row block of a small group
+    int32_t *num_thin;    // [1]
+    int32_t *thin_g;      // [max_tiles] groups of at most kThin triples (no tiles)
+    int max_items;
 };
+
+#ifndef KGE_TR_DM_WGS
+#define KGE_TR_DM_WGS (3 * 256)
+#endif
+constexpr int kDmWgs = KGE_TR_DM_WGS;  // workgroups of a dM launch: three per CU, what its registers allow
 
 // Inclusive scan over the 1024 threads of the block: shuffle scan inside each wave, then the 16
 // wave totals are scanned by every wave for itself (two barriers in all).
@@ -85,38 +94,46 @@ __device__ int block_inclusive_scan_1024(int v, int *s_scan)
     return v + before;
 }
 
-// One workgroup per plan: block 0 builds `plan0` with tiles of `tile0` positions, block 1 (when
-// launched) `plan1` with `tile1`.
+// One workgroup per plan: block 0 builds `plan0` with tiles of `tile0` positions (the GEMM plan), block 1
+// (when launched) `plan1`, the chunked plan of the dM kernel: chunks of `tile1` positions, `nib` row blocks per
+// chunk, groups of at most `small_max` triples as one item.
 __global__ __launch_bounds__(1024) void transr_plan_kernel(const int32_t *num_unique, const int32_t *seg_offsets,
                                                           const int64_t *unique_ids, TilePlan plan0, int tile0,
-                                                          TilePlan plan1, int tile1)
+                                                          TilePlan plan1, int tile1, int nib, int small_max)
 {
-    const TilePlan &plan = blockIdx.x == 0 ? plan0 : plan1;
-    const int tile = blockIdx.x == 0 ? tile0 : tile1;
+    const bool chunked = blockIdx.x != 0;
+    const TilePlan &plan = chunked ? plan1 : plan0;
+    const int tile = chunked ? tile1 : tile0;
     __shared__ int s_scan[1024];
-    __shared__ int s_carry[3];
+    __shared__ int s_carry[6];  // tiles, split slots, splits, thin groups, long items, small items
     const int U = num_unique[0];
-    if (threadIdx.x < 3) s_carry[threadIdx.x] = 0;
+    if (threadIdx.x < 6) s_carry[threadIdx.x] = 0;
     __syncthreads();
     for (int base = 0; base < U; base += 1024) {
         const int g = base + threadIdx.x;
-        int s0 = 0, s1 = 0, cnt = 0, rid = 0;
+        int s0 = 0, s1 = 0, cnt = 0, rid = 0, thin = 0, n_long = 0, n_small = 0;
         if (g < U) {
             s0 = seg_offsets[g], s1 = seg_offsets[g + 1];
             rid = (int)unique_ids[g];
-            cnt = (s1 - s0 + tile - 1) / tile;
-            // the chunked plan of the dM kernel (the one with split bookkeeping) has no tiles for groups of
-            // at most kThin triples: thin workgroups write those, and a tile that only finds out that it has
-            // nothing to do holds a workgroup slot for three dependent loads
-            if (plan.tile_part && s1 - s0 <= kThin) cnt = 0;
+            const int n = s1 - s0;
+            cnt = (n + tile - 1) / tile;
+            if (chunked) {  // groups of at most kThin triples have no tiles: thin work writes those
+                thin = n <= kThin ? 1 : 0;
+                if (thin) cnt = 0;
+                else if (n <= small_max) n_small = 1;
+                else n_long = cnt * nib;
+            }
         }
         const int inc_t = block_inclusive_scan_1024(cnt, s_scan);
         const int start = s_carry[0] + inc_t - cnt;
-        int pstart = -1;
-        if (plan.tile_part) {
+        int pstart = -1, inc_p = 0, inc_s = 0, inc_th = 0, inc_l = 0, inc_m = 0;
+        if (chunked) {
             const int pc = cnt > 1 ? cnt : 0, sg = cnt > 1 ? 1 : 0;
-            const int inc_p = block_inclusive_scan_1024(pc, s_scan);
-            const int inc_s = block_inclusive_scan_1024(sg, s_scan);
+            inc_p = block_inclusive_scan_1024(pc, s_scan);
+            inc_s = block_inclusive_scan_1024(sg, s_scan);
+            inc_th = block_inclusive_scan_1024(thin, s_scan);
+            inc_l = block_inclusive_scan_1024(n_long, s_scan);
+            inc_m = block_inclusive_scan_1024(n_small, s_scan);
             if (sg) {
                 pstart = s_carry[1] + inc_p - pc;
                 const int si = s_carry[2] + inc_s - 1;
@@ -124,8 +141,14 @@ __global__ __launch_bounds__(1024) void transr_plan_kernel(const int32_t *num_un
                 plan.split_first[si] = pstart;
                 plan.split_cnt[si] = cnt;
             }
-            __syncthreads();
-            if (threadIdx.x == 1023) s_carry[1] += inc_p, s_carry[2] += inc_s;
+            if (thin) plan.thin_g[s_carry[3] + inc_th - 1] = g;
+            if (n_small) {  // from the back of the list
+                const int at = plan.max_items - 1 - (s_carry[5] + inc_m - 1);
+                plan.item_tile[at] = start, plan.item_blk[at] = -1;
+            }
+            int at = s_carry[4] + inc_l - n_long;
+            for (int q = 0; q < (n_long ? cnt : 0); ++q)
+                for (int ib = 0; ib < nib; ++ib, ++at) plan.item_tile[at] = start + q, plan.item_blk[at] = ib;
         }
         for (int q = 0; q < cnt; ++q) {
             plan.tile_seg[start + q] = g;
@@ -134,12 +157,19 @@ __global__ __launch_bounds__(1024) void transr_plan_kernel(const int32_t *num_un
             if (plan.tile_part) plan.tile_part[start + q] = pstart >= 0 ? pstart + q : -1;
         }
         __syncthreads();
-        if (threadIdx.x == 1023) s_carry[0] += inc_t;
+        if (threadIdx.x == 1023) {
+            s_carry[0] += inc_t;
+            s_carry[1] += inc_p, s_carry[2] += inc_s, s_carry[3] += inc_th, s_carry[4] += inc_l, s_carry[5] += inc_m;
+        }
         __syncthreads();
     }
     if (threadIdx.x == 0) {
         plan.num_tiles[0] = s_carry[0];
-        if (plan.num_split) plan.num_split[0] = s_carry[2];
+        if (chunked) {
+            plan.num_split[0] = s_carry[2];
+            plan.num_thin[0] = s_carry[3];
+            plan.num_items[0] = s_carry[4], plan.num_items[1] = s_carry[5];
+        }
     }
 }
 
@@ -846,7 +876,10 @@ bool transr_grouped_path_ok(const kge_tables *tab, const kge_batch *bat)
 }
 
 // ---- backward kernels ----------------------------------------------------------------------
-constexpr int kDmChunk = 256;  // triples of one relation group per dM work item
+#ifndef KGE_TR_DM_CHUNK
+#define KGE_TR_DM_CHUNK 256
+#endif
+constexpr int kDmChunk = KGE_TR_DM_CHUNK;  // triples of one relation group per dM work item (at most 256: one per thread when staging)
 constexpr int kDmXP = 36;      // LDS pitch of a staged left-operand row (32 columns + 4: the four lane groups of an MFMA step read distinct banks)
 
 struct DmArgs {
@@ -857,7 +890,6 @@ struct DmArgs {
     float *part;     // [max_slots, d, d] partial results of split groups
     int d;
     const int32_t *num_unique;
-    int max_items;   // leading workgroups: (tile, 32-row block) items; the rest: one thin group each
     BwdSrc src;
     // Factored output (kge_grads.aux_x / aux_q): a group of at most factor_max (<= kThin) triples writes its
     // operand rows x_p, q_p to fx[p], fq[p] (p = its sorted positions) instead of the dense d x d sum of
@@ -995,7 +1027,8 @@ __device__ __forceinline__ void dm_sweep(const float *qbase, const float *sX, co
 // loads.  As (chunk, row block) work items such a group costs ceil(d / 32) workgroups that each walk the
 // same index chain and re-read the same q rows for a single superstep of matrix-core work.
 constexpr int kDmSmall = 32;
-__host__ __device__ inline bool dm_small_fits(int d) { return kDmSmall * (d + 4) <= kDmChunk * kDmXP; }
+constexpr int kDmSmallLdsFloats = 256 * kDmXP;  // what the small-group layout may take (36 KB: three workgroups per CU with room to spare)
+__host__ __device__ inline bool dm_small_fits(int d) { return kDmSmall * (d + 4) <= kDmSmallLdsFloats; }
 
 template <bool SIGN>
 __device__ __forceinline__ void transr_dm_small_body(const DmArgs &a, float *lds, int s0, int n, float *dst)
@@ -1005,7 +1038,7 @@ __device__ __forceinline__ void transr_dm_small_body(const DmArgs &a, float *lds
     const int nq = (n + 15) / 16;  // 1 or 2
     const bool derived = a.xs == nullptr;
     float *sX = lds;                                                      // [kDmSmall][pitch]
-    int64_t *sOff = reinterpret_cast<int64_t *>(lds + kDmChunk * kDmXP);  // [kDmSmall] (behind the rows, as in the item layout)
+    int64_t *sOff = reinterpret_cast<int64_t *>(lds + kDmSmallLdsFloats);  // [kDmSmall]
     __shared__ int64_t s_xh[kDmSmall], s_xt[kDmSmall];
     __shared__ float s_c[kDmSmall];
     if (tid < kDmSmall) {
@@ -1113,27 +1146,17 @@ __device__ __forceinline__ void transr_dm_small_body(const DmArgs &a, float *lds
 // folded in), the four waves split the columns j and K runs over the chunk's triples.  Groups longer
 // than one chunk write per-chunk partial matrices that are added up beside the segmented reduction
 // (keeps the longest K loop at 16 supersteps).
-__device__ __forceinline__ void transr_dm_body(const DmArgs &a, float *lds, int bid)
+__device__ __forceinline__ void transr_dm_item(const DmArgs &a, float *lds, int tile, int blk)
 {
-    if (bid >= a.max_items) {
-        transr_thin_dm_body(a, lds, bid - a.max_items);
-        return;
-    }
     const int d = a.d;
-    const int nib = (d + 31) / 32;
-    const int tile = bid / nib;
-    if (tile >= a.plan.num_tiles[0]) return;
-    const int i0 = (bid % nib) * 32;
+    const int i0 = blk * 32;
     const int g = a.plan.tile_seg[tile];
     const int s0 = a.plan.tile_p0[tile];
     const int seg_end = a.seg_offsets[g + 1];
-    const int gn = seg_end - a.seg_offsets[g];
-    if (gn <= kThin) return;  // written by a thin workgroup
-    if (gn <= kDmSmall && dm_small_fits(d)) {  // the whole group by the workgroup of its first row block
-        if (i0 != 0) return;
+    if (blk < 0) {  // a small group, whole, by this workgroup
         float *whole = a.dm + (int64_t)g * d * d;
-        if (a.xs == nullptr && !a.src.rescal && a.src.norm_p == 1) transr_dm_small_body<true>(a, lds, s0, gn, whole);
-        else transr_dm_small_body<false>(a, lds, s0, gn, whole);
+        if (a.xs == nullptr && !a.src.rescal && a.src.norm_p == 1) transr_dm_small_body<true>(a, lds, s0, seg_end - s0, whole);
+        else transr_dm_small_body<false>(a, lds, s0, seg_end - s0, whole);
         return;
     }
     const int s1 = s0 + kDmChunk < seg_end ? s0 + kDmChunk : seg_end;
@@ -1224,14 +1247,29 @@ __device__ __forceinline__ void transr_dm_body(const DmArgs &a, float *lds, int 
 static size_t dm_lds_bytes(int d)  // the staged left operand and its row offsets, or the thin groups' transposed rows
 {
     const size_t item = sizeof(float) * kDmChunk * kDmXP + sizeof(int64_t) * kDmChunk, thin = sizeof(float) * 4 * (size_t)d;
-    return item > thin ? item : thin;
+    const size_t small = dm_small_fits(d) ? sizeof(float) * kDmSmallLdsFloats + sizeof(int64_t) * kDmSmall : 0;
+    return item > thin ? (item > small ? item : small) : (thin > small ? thin : small);
+}
+
+// Item `it` of a dM pass: the (chunk, row block) items of the larger groups first (the long chains), then the
+// small groups, then the thin ones.  False: past the end of the lists.
+__device__ __forceinline__ bool transr_dm_work(const DmArgs &a, float *lds, int it, int n_long, int n_small, int n_thin)
+{
+    if (it < n_long) transr_dm_item(a, lds, a.plan.item_tile[it], a.plan.item_blk[it]);
+    else if (it < n_long + n_small) transr_dm_item(a, lds, a.plan.item_tile[a.plan.max_items - 1 - (it - n_long)], -1);
+    else if (it < n_long + n_small + n_thin) transr_thin_dm_body(a, lds, a.plan.thin_g[it - n_long - n_small]);
+    else return false;
+    return true;
 }
 
 __global__ __launch_bounds__(256, KGE_TR_OCC) void transr_dm_kernel(DmArgs a, FusedInsp fi)
 {
     extern __shared__ __align__(16) float lds[];  // dm_lds_bytes(); inspector workgroups: their own need
     if (fused_insp_block(fi, reinterpret_cast<uint32_t *>(lds))) return;
-    transr_dm_body(a, lds, (int)blockIdx.x - fi.blocks);
+    const int n_long = a.plan.num_items[0], n_small = a.plan.num_items[1], n_thin = a.plan.num_thin[0];
+    const int stride = (int)gridDim.x - fi.blocks;
+    for (int it = (int)blockIdx.x - fi.blocks; transr_dm_work(a, lds, it, n_long, n_small, n_thin); it += stride)
+        __syncthreads();  // the next item reuses the staging buffers
 }
 
 // An inspector step that rides with nothing: the fused entity inspection of a TransR / RESCAL step has
@@ -1240,25 +1278,6 @@ __global__ __launch_bounds__(256) void transr_insp_step_kernel(FusedInsp fi)
 {
     extern __shared__ __align__(16) float lds[];
     (void)fused_insp_block(fi, reinterpret_cast<uint32_t *>(lds));
-}
-
-// dX and dM of one backward pass in ONE launch (no inspector riders): the two are independent, one
-// streams the projections in while the other streams the projection gradients out, and either alone
-// leaves the memory system waiting on its dependent chains.  Order of the workgroups: the dX tiles,
-// the dM work items, then the thin groups of both in alternation.
-__global__ __launch_bounds__(256, KGE_TR_OCC) void transr_dx_dm_kernel(GemmArgs ga, DmArgs da)
-{
-    extern __shared__ __align__(16) float lds[];
-    const int bid = (int)blockIdx.x;
-    if (bid < ga.max_tiles) {
-        transr_gemm_body<2>(ga, lds, bid);
-    } else if (bid < ga.max_tiles + da.max_items) {
-        transr_dm_body(da, lds, bid - ga.max_tiles);
-    } else {
-        const int q = bid - ga.max_tiles - da.max_items;
-        if (q & 1) transr_dm_body(da, lds, da.max_items + (q >> 1));
-        else transr_gemm_body<2>(ga, lds, ga.max_tiles + (q >> 1));
-    }
 }
 
 // dM of a split group = sum of its partial matrices (slot order = ascending chunk order); the sums
@@ -1281,7 +1300,15 @@ struct RPlan {
     int64_t tiles, dtiles, dsplit, dslots;
 };
 
-static size_t plan_ints(int64_t tiles, int64_t split) { return (size_t)(64 + 5 * tiles + 3 * split + 8); }
+// (items > 0: a chunked plan with its work lists)
+static size_t plan_ints(int64_t tiles, int64_t split, int64_t items = 0)
+{
+    return (size_t)(64 + 5 * tiles + 3 * split + (items > 0 ? tiles + 2 * items : 0) + 8);
+}
+static int dm_nib(int64_t d) { return (int)ceil_div(d, 32); }
+static int dm_small_max(int64_t d) { return dm_small_fits((int)d) ? kDmSmall : kThin; }
+static int64_t dm_item_cap(int64_t dtiles, int64_t d) { return dtiles * ceil_div(d, 32); }
+static size_t dplan_ints(int64_t dtiles, int64_t dsplit, int64_t d) { return plan_ints(dtiles, dsplit, dm_item_cap(dtiles, d)); }
 
 static RPlan make_rplan(const kge_tables *tab, const kge_batch *bat)
 {
@@ -1294,7 +1321,7 @@ static RPlan make_rplan(const kge_tables *tab, const kge_batch *bat)
     p.dslots = 2 * (B / kDmChunk) + 2;      // sum over split groups of ceil(n_g / chunk)
     size_t o = 0;
     p.off_plan = o, o += up256(sizeof(int32_t) * plan_ints(p.tiles, 0));
-    p.off_dplan = o, o += up256(sizeof(int32_t) * plan_ints(p.dtiles, p.dsplit));
+    p.off_dplan = o, o += up256(sizeof(int32_t) * dplan_ints(p.dtiles, p.dsplit, d));
     p.off_occ = o, o += up256(sizeof(float) * (size_t)(2 * B * d));
     p.off_part_e = o, o += up256(sizeof(float) * (size_t)seg_partial_floats(2 * B, d));
     p.off_part_r = o, o += up256(sizeof(float) * (size_t)seg_partial_floats(B, d));
@@ -1303,21 +1330,31 @@ static RPlan make_rplan(const kge_tables *tab, const kge_batch *bat)
     return p;
 }
 
-static TilePlan plan_at(void *base, int64_t tiles, int64_t split)
+static TilePlan plan_at(void *base, int64_t tiles, int64_t split, int64_t items = 0)
 {
     int32_t *q = static_cast<int32_t *>(base);
-    TilePlan p{q, q + 64, q + 64 + tiles, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr};
+    TilePlan p{};
+    p.num_tiles = q, p.tile_seg = q + 64, p.tile_p0 = q + 64 + tiles;
     if (split > 0) {
         p.tile_part = q + 64 + 2 * tiles;
         p.num_split = q + 32;
         p.split_seg = q + 64 + 5 * tiles;
         p.split_first = p.split_seg + split;
         p.split_cnt = p.split_first + split;
+        p.num_thin = q + 1, p.num_items = q + 2;
+        p.thin_g = q + 64 + 5 * tiles + 3 * split;
+        p.item_tile = p.thin_g + tiles;
+        p.item_blk = p.item_tile + items;
+        p.max_items = (int)items;
     } else {
         p.tile_end = q + 64 + 3 * tiles;
         p.tile_rid = q + 64 + 4 * tiles;
     }
     return p;
+}
+static TilePlan dplan_at(void *base, int64_t dtiles, int64_t dsplit, int64_t d)
+{
+    return plan_at(base, dtiles, dsplit, dm_item_cap(dtiles, d));
 }
 
 // The forward workspace holds both tile plans of the batch: the 32-triple tiles of the GEMM kernels
@@ -1340,7 +1377,7 @@ size_t transr_fwd_workspace(const kge_tables *tab, const kge_batch *bat)
 {
     if (pad_path_ok(tab, bat)) return transr_fwd_workspace_padded(tab, bat);  // row width not a multiple of four
     const RPlan p = make_rplan(tab, bat);
-    return fwd_plan_bytes(tab, bat) + up256(sizeof(int32_t) * plan_ints(p.dtiles, p.dsplit));
+    return fwd_plan_bytes(tab, bat) + up256(sizeof(int32_t) * dplan_ints(p.dtiles, p.dsplit, tab->dim));
 }
 
 // A launch with more than 64 KB of dynamic LDS has to be allowed per kernel first.
@@ -1384,10 +1421,10 @@ int launch_transr_fwd(const kge_tables *tab, const kge_batch *bat, float *pos, f
     const int64_t tiles = max_tiles(tab, bat);
     TilePlan plan = plan_at(workspace, tiles, 0);
     const RPlan rp = make_rplan(tab, bat);
-    TilePlan dplan = plan_at(static_cast<char *>(workspace) + fwd_plan_bytes(tab, bat), rp.dtiles, rp.dsplit);
+    TilePlan dplan = dplan_at(static_cast<char *>(workspace) + fwd_plan_bytes(tab, bat), rp.dtiles, rp.dsplit, tab->dim);
     if (!bat->plans_ready)
         hipLaunchKernelGGL(transr_plan_kernel, dim3(2), dim3(1024), 0, st, ri->num_unique, ri->seg_offsets, ri->unique_ids, plan,
-                           kTM, dplan, kDmChunk);
+                           kTM, dplan, kDmChunk, dm_nib(tab->dim), dm_small_max(tab->dim));
     GemmArgs a{tab->ent, tab->rel, tab->aux, bat->h, bat->r, bat->t, ri->perm, ri->seg_offsets, ri->num_unique, ri->unique_ids,
                plan, nullptr, nullptr, pos, resid, nullptr, nullptr, (int)tab->dim, tab->norm_p, thin_groups(tab, bat), (int)tiles,
                BwdSrc{}};
@@ -1414,9 +1451,9 @@ int launch_transr_plan(const kge_tables *tab, const kge_batch *bat, void *worksp
     const kge_inspection *ri = bat->rel_insp;
     const RPlan rp = make_rplan(tab, bat);
     TilePlan plan = plan_at(workspace, max_tiles(tab, bat), 0);
-    TilePlan dplan = plan_at(static_cast<char *>(workspace) + fwd_plan_bytes(tab, bat), rp.dtiles, rp.dsplit);
+    TilePlan dplan = dplan_at(static_cast<char *>(workspace) + fwd_plan_bytes(tab, bat), rp.dtiles, rp.dsplit, tab->dim);
     hipLaunchKernelGGL(transr_plan_kernel, dim3(2), dim3(1024), 0, st, ri->num_unique, ri->seg_offsets, ri->unique_ids, plan, kTM,
-                       dplan, kDmChunk);
+                       dplan, kDmChunk, dm_nib(tab->dim), dm_small_max(tab->dim));
     KGE_CHECK_LAUNCH();
     return KGE_OK;
 }
@@ -1449,7 +1486,7 @@ static RescalNegPlan make_rescal_neg_plan(const kge_tables *tab, const kge_batch
         return at;
     };
     p.off_plan = take(sizeof(int32_t) * plan_ints(p.tiles, 0));
-    p.off_dplan = take(sizeof(int32_t) * plan_ints(p.dtiles, p.dsplit));
+    p.off_dplan = take(sizeof(int32_t) * dplan_ints(p.dtiles, p.dsplit, d));
     p.off_xs = take(sizeof(float) * (size_t)(B * d));
     p.off_qs = take(sizeof(float) * (size_t)(B * d));
     p.off_g0 = take(sizeof(float) * (size_t)(B * d));
@@ -1519,18 +1556,17 @@ int launch_rescal_neg_bwd(const kge_tables *tab, const kge_batch *bat, const kge
     }
     hipLaunchKernelGGL(rescal_neg_prep_kernel, dim3((unsigned)ceil_div(B, 4)), dim3(256), 0, st, tab->ent, bat->h, bat->t, ri->perm, dpos,
                        dneg ? g0 : nullptr, saved->residual, xs, qs, occ + B * d, B, d);
-    TilePlan plan = plan_at(ws + p.off_plan, p.tiles, 0), dplan = plan_at(ws + p.off_dplan, p.dtiles, p.dsplit);
+    TilePlan plan = plan_at(ws + p.off_plan, p.tiles, 0), dplan = dplan_at(ws + p.off_dplan, p.dtiles, p.dsplit, d);
     hipLaunchKernelGGL(transr_plan_kernel, dim3(2), dim3(1024), 0, st, ri->num_unique, ri->seg_offsets, ri->unique_ids, plan, kTM, dplan,
-                       kDmChunk);
+                       kDmChunk, dm_nib(d), dm_small_max(d));
     GemmArgs ga{tab->ent, tab->rel, tab->aux, bat->h, bat->r, bat->t, ri->perm, ri->seg_offsets, ri->num_unique, ri->unique_ids,
                 plan, qs, nullptr, nullptr, nullptr, occ, nullptr, d, tab->norm_p, thin_groups(tab, bat), (int)p.tiles, BwdSrc{}};
     if (const int rc = allow_lds<2>(gemm_lds_bytes(d))) return rc;
     hipLaunchKernelGGL(transr_gemm_kernel<2>, dim3((unsigned)(p.tiles + ga.thin_groups)), dim3(256), gemm_lds_bytes(d), st, ga, FusedInsp{});
     timeline_mark(bat->timeline, st, "transr_gemm_kernel<dX>");
-    const int dm_items = (int)(ceil_div(d, 32) * p.dtiles);
-    DmArgs da{xs, qs, ri->seg_offsets, dplan, grads->aux_rows, reinterpret_cast<float *>(ws + p.off_dpart), d, ri->num_unique, dm_items,
+    DmArgs da{xs, qs, ri->seg_offsets, dplan, grads->aux_rows, reinterpret_cast<float *>(ws + p.off_dpart), d, ri->num_unique,
               BwdSrc{}, nullptr, nullptr, 0};
-    hipLaunchKernelGGL(transr_dm_kernel, dim3((unsigned)(dm_items + thin_groups(tab, bat))), dim3(256), dm_lds_bytes(d), st, da, FusedInsp{});
+    hipLaunchKernelGGL(transr_dm_kernel, dim3((unsigned)kDmWgs), dim3(256), dm_lds_bytes(d), st, da, FusedInsp{});
     timeline_mark(bat->timeline, st, "transr_dm_kernel");
     KGE_CHECK_LAUNCH();
     if (bat->insp_ready && hipStreamWaitEvent(st, reinterpret_cast<hipEvent_t>(bat->insp_ready), 0) != hipSuccess)
@@ -1566,8 +1602,8 @@ int launch_transr_bwd(const kge_tables *tab, const kge_batch *bat, const kge_sav
     const bool have_plans = saved->fwd_workspace && saved->fwd_workspace_bytes >= transr_fwd_workspace(tab, bat);
     char *pbase = have_plans ? static_cast<char *>(const_cast<void *>(saved->fwd_workspace)) : nullptr;
     TilePlan plan = have_plans ? plan_at(pbase, p.tiles, 0) : plan_at(ws + p.off_plan, p.tiles, 0);
-    TilePlan dplan = have_plans ? plan_at(pbase + fwd_plan_bytes(tab, bat), p.dtiles, p.dsplit)
-                                : plan_at(ws + p.off_dplan, p.dtiles, p.dsplit);
+    TilePlan dplan = have_plans ? dplan_at(pbase + fwd_plan_bytes(tab, bat), p.dtiles, p.dsplit, d)
+                                : dplan_at(ws + p.off_dplan, p.dtiles, p.dsplit, d);
 
     // fused entity inspection (its histogram rode with the forward GEMM): first digit pass in a launch
     // of its own, second with the dX GEMM, dedup with dM
@@ -1583,7 +1619,7 @@ int launch_transr_bwd(const kge_tables *tab, const kge_batch *bat, const kge_sav
     }
     if (!have_plans)
         hipLaunchKernelGGL(transr_plan_kernel, dim3(2), dim3(1024), 0, st, ri->num_unique, ri->seg_offsets, ri->unique_ids, plan, kTM,
-                           dplan, kDmChunk);
+                           dplan, kDmChunk, dm_nib(d), dm_small_max(d));
     // Upstream rows q and left operands x are formed inside the two kernels from the forward pass's rows
     // (BwdSrc); RESCAL's tail occurrence rows g * v come out of the dX kernel's staging.
     const BwdSrc src{tab->ent, saved->residual, dpos, saved->pos, bat->h, bat->t, ri->perm, tab->norm_p, rescal ? 1 : 0,
@@ -1593,28 +1629,14 @@ int launch_transr_bwd(const kge_tables *tab, const kge_batch *bat, const kge_sav
                 plan, nullptr, nullptr, nullptr, nullptr, occ, rescal ? nullptr : occ + B * d, d, tab->norm_p, thin_groups(tab, bat),
                 (int)p.tiles, src};
     // dM = X^T Q per relation group
-    const int dm_items = (int)(ceil_div(d, 32) * p.dtiles);
     DmArgs da{nullptr, nullptr, ri->seg_offsets, dplan, grads->aux_rows, reinterpret_cast<float *>(ws + p.off_dpart), d,
-              ri->num_unique, dm_items, src, factored ? grads->aux_x : nullptr, factored ? grads->aux_q : nullptr,
-              grads->aux_factor_max};
-    if (!bat->fuse_inspection && !kSplitBwd) {  // both in one launch
-        const size_t lds = gemm_lds_bytes(d) > dm_lds_bytes(d) ? gemm_lds_bytes(d) : dm_lds_bytes(d);
-        if (lds > 64 * 1024 &&
-            hipFuncSetAttribute(reinterpret_cast<const void *>(&transr_dx_dm_kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                (int)kMaxGemmLds) != hipSuccess)
-            return KGE_ELAUNCH;
-        hipLaunchKernelGGL(transr_dx_dm_kernel, dim3((unsigned)(p.tiles + dm_items + 2 * ga.thin_groups)), dim3(256), lds, st, ga,
-                           da);
-        timeline_mark(bat->timeline, st, "transr_dx_dm_kernel");
-    } else {
-        if (const int rc = allow_lds<2>(lds_with(f2, gemm_lds_bytes(d)))) return rc;
-        hipLaunchKernelGGL(transr_gemm_kernel<2>, dim3((unsigned)(p.tiles + ga.thin_groups + f2.blocks)), dim3(256),
-                           lds_with(f2, gemm_lds_bytes(d)), st, ga, f2);
-        timeline_mark(bat->timeline, st, "transr_gemm_kernel<dX>");
-        hipLaunchKernelGGL(transr_dm_kernel, dim3((unsigned)(dm_items + thin_groups(tab, bat) + f3.blocks)), dim3(256),
-                           lds_with(f3, dm_lds_bytes(d)), st, da, f3);
-        timeline_mark(bat->timeline, st, "transr_dm_kernel");
-    }
+              ri->num_unique, src, factored ? grads->aux_x : nullptr, factored ? grads->aux_q : nullptr, grads->aux_factor_max};
+    if (const int rc = allow_lds<2>(lds_with(f2, gemm_lds_bytes(d)))) return rc;
+    hipLaunchKernelGGL(transr_gemm_kernel<2>, dim3((unsigned)(p.tiles + ga.thin_groups + f2.blocks)), dim3(256),
+                       lds_with(f2, gemm_lds_bytes(d)), st, ga, f2);
+    timeline_mark(bat->timeline, st, "transr_gemm_kernel<dX>");
+    hipLaunchKernelGGL(transr_dm_kernel, dim3((unsigned)(kDmWgs + f3.blocks)), dim3(256), lds_with(f3, dm_lds_bytes(d)), st, da, f3);
+    timeline_mark(bat->timeline, st, "transr_dm_kernel");
     KGE_CHECK_LAUNCH();
     if (bat->insp_ready && hipStreamWaitEvent(st, reinterpret_cast<hipEvent_t>(bat->insp_ready), 0) != hipSuccess)
         return KGE_ELAUNCH;

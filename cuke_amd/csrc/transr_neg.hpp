@@ -76,7 +76,7 @@ static NegFwdLayout neg_fwd_layout(const kge_tables *tab, const NegShape &s)
     l.tl = take(sizeof(int64_t) * s.L_cap);
     l.rsl = take(sizeof(float) * s.L_cap);
     l.plan = take(sizeof(int32_t) * plan_ints(s.tiles, 0));
-    l.dplan = take(sizeof(int32_t) * plan_ints(s.dtiles, s.dsplit));
+    l.dplan = take(sizeof(int32_t) * dplan_ints(s.dtiles, s.dsplit, s.d));
     l.y = take(sizeof(float) * (size_t)(s.L_cap * s.d));
     l.total = o;
     return l;
@@ -673,9 +673,9 @@ int launch_transr_neg_fwd(const kge_tables *tab, const kge_batch *bat, float *po
     const int64_t list_threads = s.B + s.G_cap * s.N;
     const int64_t list_blocks = ceil_div(list_threads, 256);
     hipLaunchKernelGGL(tneg_list_kernel, dim3((unsigned)(list_blocks < 8192 ? list_blocks : 8192)), dim3(256), 0, st, x);
-    TilePlan plan = plan_at(ws + l.plan, s.tiles, 0), dplan = plan_at(ws + l.dplan, s.dtiles, s.dsplit);
+    TilePlan plan = plan_at(ws + l.plan, s.tiles, 0), dplan = dplan_at(ws + l.dplan, s.dtiles, s.dsplit, d);
     hipLaunchKernelGGL(transr_plan_kernel, dim3(2), dim3(1024), 0, st, ri->num_unique, x.segl, ri->unique_ids, plan, kTM, dplan,
-                       kDmChunk);
+                       kDmChunk, dm_nib(d), dm_small_max(d));
     timeline_mark(bat->timeline, st, "row list + transr_plan_kernel");
 
     // one grouped pass projects every list row
@@ -721,7 +721,7 @@ int launch_transr_neg_bwd(const kge_tables *tab, const kge_batch *bat, const kge
     float *dxl = reinterpret_cast<float *>(ws + l.dxl), *occ = reinterpret_cast<float *>(ws + l.occ);
     float *qr = reinterpret_cast<float *>(ws + l.qr);
     int32_t *glist = reinterpret_cast<int32_t *>(ws + l.glist), *gcount = reinterpret_cast<int32_t *>(ws + l.gcount);
-    TilePlan plan = plan_at(fws + fl.plan, s.tiles, 0), dplan = plan_at(fws + fl.dplan, s.dtiles, s.dsplit);
+    TilePlan plan = plan_at(fws + fl.plan, s.tiles, 0), dplan = dplan_at(fws + fl.dplan, s.dtiles, s.dsplit, d);
 
     NegPairArgs pa{};
     pa.ent = tab->ent, pa.y = y, pa.dpos = dpos, pa.dneg = dneg, pa.spos = saved->pos, pa.sneg = saved->neg;
@@ -744,10 +744,9 @@ int launch_transr_neg_bwd(const kge_tables *tab, const kge_batch *bat, const kge
     if (const int rc = allow_lds<2>(lds)) return rc;
     hipLaunchKernelGGL(transr_gemm_kernel<2>, dim3((unsigned)(s.tiles + s.U_cap)), dim3(256), lds, st, ga, FusedInsp{});
     timeline_mark(bat->timeline, st, "transr_gemm_kernel<dX>");
-    const int dm_items = (int)(ceil_div(d, 32) * s.dtiles);
-    DmArgs da{xl, ql, x.segl, dplan, grads->aux_rows, reinterpret_cast<float *>(ws + l.dpart), d, ri->num_unique, dm_items,
+    DmArgs da{xl, ql, x.segl, dplan, grads->aux_rows, reinterpret_cast<float *>(ws + l.dpart), d, ri->num_unique,
               BwdSrc{}, nullptr, nullptr, 0};
-    hipLaunchKernelGGL(transr_dm_kernel, dim3((unsigned)(dm_items + s.U_cap)), dim3(256), dm_lds_bytes(d), st, da, FusedInsp{});
+    hipLaunchKernelGGL(transr_dm_kernel, dim3((unsigned)kDmWgs), dim3(256), dm_lds_bytes(d), st, da, FusedInsp{});
     timeline_mark(bat->timeline, st, "transr_dm_kernel");
     TNEG_BY_WIDTH(d, hipLaunchKernelGGL(tneg_occ_kernel<NQ_>, dim3((unsigned)(ceil_div(s.B, 4) + s.NN)), dim3(256), 0, st, x, dxl,
                                         glist, gcount, occ));
