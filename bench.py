@@ -53,18 +53,18 @@ PROFILE_KERNELS = {
     "transr_plan_kernel + transr_gemm_kernel<fwd>": ["transr_plan_kernel", "transr_gemm_kernel<0>"],
     "transr_gemm_kernel<dX>": ["transr_gemm_kernel<2>"],
     "transr_dm_kernel": ["transr_dm_kernel"],
-    "transr_dx_dm_kernel": ["transr_dx_dm_kernel"],
 }
 
 
-def measured_traffic(workload, label, matrix_core_tiles=False):
+def measured_traffic(workload, label, matrix_core_tiles=False, dense=False):
     """HBM bytes per launch of the kernel(s) behind a timeline label, read from the committed profile
     summary of the workload: rocprofv3 --pmc FETCH_SIZE and --pmc WRITE_SIZE runs of this script (KiB
     per dispatch), each scaled by what the same counter reads for the 256 MiB copy kernel of
     --calibrate-copy (the file states the factors).  Returns (bytes or None, the profile's kernel
     names) so that the line shows which compiled kernels the figure belongs to.  matrix_core_tiles: the
     workload's tile kernels are the matrix-core forms (the profile of such a workload also holds the
-    vector-ALU forms that the run times beside them)."""
+    vector-ALU forms that the run times beside them).  dense: rows of the profile's second table (the
+    TransR step that writes every projection gradient dense) replace those of the first."""
     import re
     path = os.path.join(ROOT, "profiles", f"score_path_kernels_{workload}.txt")
     want = PROFILE_KERNELS.get(label)
@@ -73,10 +73,11 @@ def measured_traffic(workload, label, matrix_core_tiles=False):
     rows, in_table = {}, False
     for line in open(path):
         if line.startswith("## HBM traffic per dispatch"):
-            in_table = True
+            in_table = dense or "dense" not in line
             continue
         if in_table and line.startswith("## "):
-            break
+            in_table = False
+            continue
         m = re.match(r"^(kge::.*?)\s+([\d.]+)\s+([\d.]+)\s+([\d.]+)\s+([\d.]+)\s*$", line) if in_table else None
         if m:
             rows[m.group(1)] = (float(m.group(4)) + float(m.group(5))) * 1e6
@@ -176,9 +177,6 @@ def kernel_model(w, label, u_ent, u_rel):
     dm_out = 4 * (w.dense_rel * d * d + 2 * w.factored_rows * d) if hasattr(w, "dense_rel") else 4 * u_rel * d * d
     if label == "transr_dm_kernel":
         return dm_out + 4 * 3 * B * d, 2 * B * d * d, "mfma"
-    if label == "transr_dx_dm_kernel":
-        by = 4 * (u_rel * d * d + 3 * B * d) + 8 * 3 * B + dm_out + 4 * 3 * B * d
-        return by, 4 * B * d * d, "mfma"
     return 0, 0, "valu"
 
 
@@ -637,7 +635,7 @@ def run_workload(name, args, torch, factor_max=0):
     # about 0.2 ms in front of each step lets the host enqueue the whole step before the device starts
     # it (no memory traffic: the caches hold what the timed loop's previous step left, as there)
     # The timeline follows the issue that is reported: the staged issue launches other kernel forms than the
-    # direct one (no riding inspection, merged launches); its inspection runs on the side stream a batch
+    # direct one (no inspection riding along); its inspection runs on the side stream a batch
     # ahead, so those entries (taken here in front of the step on one stream) are not part of the step.
     kt_fused = False if issue.startswith("staged") else None
     if hasattr(torch.cuda, "_sleep"):
@@ -661,7 +659,8 @@ def run_workload(name, args, torch, factor_max=0):
     main_roof, other = (hbm_roof, fp32_roof) if bound == "hbm" else (fp32_roof, hbm_roof)
     step_gbs = total_b / (ms * 1e-3) / 1e9
     step_tfs = total_f / (ms * 1e-3) / 1e12
-    traffic, profile_kernels = measured_traffic(name, kname, w.model in ("DistMult", "ComplEx") and bool(w.chunk))
+    traffic, profile_kernels = measured_traffic(name, kname, w.model in ("DistMult", "ComplEx") and bool(w.chunk),
+                                                dense=w.model in ("TransR", "RESCAL") and factor_max == 0)
     roofline = {"kernel": kname, "bound": "hbm" if bound == "hbm" else "mfma" if k_unit == "mfma" else "fp32_valu",
                 "achieved": main_roof["achieved"], "peak": main_roof["peak"], "unit": main_roof["unit"],
                 "frac": main_roof["frac"], "traffic": traffic, "traffic_profile_kernels": profile_kernels,
@@ -797,6 +796,9 @@ def main():
     ap.add_argument("--no-check", action="store_true", help="skip the parity spot check (profiling runs)")
     ap.add_argument("--dense-only", action="store_true",
                     help="TransR: time only the step that writes every projection gradient dense (profiling runs)")
+    ap.add_argument("--factored-only", action="store_true",
+                    help="TransR: time only the headline step (small groups' projection gradients factored), not "
+                         "the dense one beside it (profiling runs)")
     ap.add_argument("--cpu-seconds", type=float, default=4.0, help="one-thread CPU work per workload")
     ap.add_argument("--seed", type=int, default=0)
     ap.add_argument("--calibrate-copy", action="store_true",
@@ -835,12 +837,13 @@ def main():
                 # long-tailed batch) are left factored, the form the optimizer entry points consume; the same
                 # step with every gradient written dense is timed in the same run and reported beside it.
                 res = run_workload(n, args, torch, factor_max=4)
-                saved_no_cpu, args.no_cpu = args.no_cpu, True
-                dense = run_workload(n, args, torch, factor_max=0)
-                args.no_cpu = saved_no_cpu
-                res["config"]["dense_projection_gradients"] = {
-                    k: dense[k] for k in ("ms_per_step", "value", "kernels_ms", "roofline")}
-                res["config"]["dense_projection_gradients"]["issue"] = dense["config"]["issue"]
+                if not args.factored_only:
+                    saved_no_cpu, args.no_cpu = args.no_cpu, True
+                    dense = run_workload(n, args, torch, factor_max=0)
+                    args.no_cpu = saved_no_cpu
+                    res["config"]["dense_projection_gradients"] = {
+                        k: dense[k] for k in ("ms_per_step", "value", "kernels_ms", "roofline")}
+                    res["config"]["dense_projection_gradients"]["issue"] = dense["config"]["issue"]
             else:
                 res = run_workload(n, args, torch)
         except SpotCheckError as e:
