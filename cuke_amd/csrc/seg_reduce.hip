@@ -13,19 +13,6 @@
 
 namespace kge {
 
-struct SegArgs {
-    const float *occ;
-    const int32_t *perm, *sorted_seg, *seg_offsets;
-    int64_t n;
-    int d;
-    float *out, *partial;
-    const float *scale_num, *scale_den;   // row transform (SegJob), transform bit 0 = scaled, bit 1 = sign
-    int transform;
-};
-struct SegArgs3 {
-    SegArgs j[3];
-};
-
 // The rider's sums: a work item is (sum i, 256 float4 of the row); the slice's workgroups stride over the items.
 __device__ __forceinline__ void sum_rider_body(const SumRider &r)
 {
@@ -38,10 +25,15 @@ __device__ __forceinline__ void sum_rider_body(const SumRider &r)
         if (f >= q4) continue;
         const int cnt = r.cnt[i];
         const float4 *src = reinterpret_cast<const float4 *>(r.part) + (int64_t)r.first[i] * q4 + f;
-        float4 acc = src[0];
-        for (int c = 1; c < cnt; ++c) {
-            const float4 v = src[(int64_t)c * q4];
-            acc.x += v.x, acc.y += v.y, acc.z += v.z, acc.w += v.w;
+        float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
+        constexpr int kFly = 8;  // rows in flight: unconditional loads (a row past the end re-reads the last one), masked afterwards
+        for (int c0 = 0; c0 < cnt; c0 += kFly) {
+            float4 v[kFly];
+#pragma unroll
+            for (int u = 0; u < kFly; ++u) v[u] = src[(int64_t)(c0 + u < cnt ? c0 + u : cnt - 1) * q4];
+#pragma unroll
+            for (int u = 0; u < kFly; ++u)
+                if (c0 + u < cnt) acc.x += v[u].x, acc.y += v[u].y, acc.z += v[u].z, acc.w += v[u].w;
         }
         reinterpret_cast<float4 *>(r.out)[(int64_t)r.seg[i] * q4 + f] = acc;
     }
@@ -54,93 +46,19 @@ __global__ __launch_bounds__(256) void seg_reduce_l1(SegArgs3 jobs, SumRider rid
         sum_rider_body(rider);
         return;
     }
-    const SegArgs &a = jobs.j[blockIdx.y];
-    const int lane = threadIdx.x & (kWave - 1);
-    const int d = a.d;
-    const int nch = (d + kWave * V - 1) / (kWave * V);
-    const int64_t w = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
-    const int64_t j = w / nch;
-    const int colv = (int)(w % nch) * kWave * V + lane * V;
-    const int64_t p0 = j * kSegL;
-    if (p0 >= a.n) return;
-    const int cnt = (int)((a.n - p0) < kSegL ? (a.n - p0) : kSegL);
-    const bool active = colv < d;
-
-    // Everything the walk needs is loaded up front in batches of unconditional loads (positions
-    // past the end re-read the last valid one, an inactive lane reads column 0, both are masked
-    // afterwards): a branch or a select around a load would make the compiler wait for each load
-    // on the spot and turn the eight rows into eight serial round trips.
-    int64_t pc[kSegL];
-#pragma unroll
-    for (int q = 0; q < kSegL; ++q) pc[q] = p0 + (q < cnt ? q : cnt - 1);
-    int src[kSegL], seg[kSegL];
-    if (a.perm) {  // uniform
-#pragma unroll
-        for (int q = 0; q < kSegL; ++q) src[q] = a.perm[pc[q]];
-    } else {
-#pragma unroll
-        for (int q = 0; q < kSegL; ++q) src[q] = (int)pc[q];
-    }
-#pragma unroll
-    for (int q = 0; q < kSegL; ++q) seg[q] = a.sorted_seg[pc[q]];
-    const int cc = active ? colv : 0;
-    Vec<V> v[kSegL];
-#pragma unroll
-    for (int q = 0; q < kSegL; ++q) v[q] = Vec<V>::load(a.occ + (int64_t)src[q] * d + cc);
-    if (a.transform) {  // uniform: the rows count as scale * phi(row)
-        float sc[kSegL];
-#pragma unroll
-        for (int q = 0; q < kSegL; ++q) sc[q] = (a.transform & 1) ? (a.scale_num ? a.scale_num[src[q]] : 0.0f) : 1.0f;
-        if ((a.transform & 1) && a.scale_den) {
-            float den[kSegL];
-#pragma unroll
-            for (int q = 0; q < kSegL; ++q) den[q] = a.scale_den[src[q]];
-#pragma unroll
-            for (int q = 0; q < kSegL; ++q) sc[q] = den[q] > 0.0f ? sc[q] / den[q] : 0.0f;
-        }
-#pragma unroll
-        for (int q = 0; q < kSegL; ++q)
-#pragma unroll
-            for (int e = 0; e < V; ++e) v[q].v[e] = sc[q] * ((a.transform & 2) ? sgn(v[q].v[e]) : v[q].v[e]);
-    }
-    // A run starts before this block iff it shares its id with the position in front of the block,
-    // and runs on past it iff it shares it with the position behind: two loads instead of the run
-    // bounds of every position.
-    const int seg_before = a.sorted_seg[p0 > 0 ? p0 - 1 : 0], seg_after = a.sorted_seg[p0 + cnt < a.n ? p0 + cnt : p0];
-    const int prev_id = p0 > 0 ? seg_before : -1;
-    const int next_id = p0 + cnt < a.n ? seg_after : -1;
-
-    Vec<V> acc;
-#pragma unroll
-    for (int e = 0; e < V; ++e) acc.v[e] = 0.0f;
-    auto flush = [&](int sg) {
-        float *dst;
-        if (sg == prev_id) dst = a.partial + (j * 2 + 0) * (int64_t)d;       // began in an earlier block
-        else if (sg == next_id) dst = a.partial + (j * 2 + 1) * (int64_t)d;  // continues in a later block
-        else dst = a.out + (int64_t)sg * d;                                   // wholly inside: final
-        if (active) acc.store(dst + colv);
-    };
-#pragma unroll
-    for (int q = 0; q < kSegL; ++q) {
-        if (q < cnt) {
-            if (q > 0 && seg[q] != seg[q - 1]) {
-                flush(seg[q - 1]);
-#pragma unroll
-                for (int e = 0; e < V; ++e) acc.v[e] = 0.0f;
-            }
-#pragma unroll
-            for (int e = 0; e < V; ++e) acc.v[e] += v[q].v[e];
-        }
-    }
-    flush(seg[cnt - 1]);
+    seg_l1_wave<V>(jobs.j[blockIdx.y], (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6));
 }
 
 // One workgroup per (block, chunk of 64 V columns): the column chunks of a wide row are independent
 // chains of round trips and run side by side (nch = chunks of the widest job of the launch).
 template <int V>
-__global__ __launch_bounds__(256) void seg_reduce_l2(SegArgs3 jobs, int nch)
+__global__ __launch_bounds__(256) void seg_reduce_l2(SegArgs3 jobs, int nch, SumRider rider)
 {
     __shared__ float s_part[4][kWave * 4];
+    if (rider.max_sums > 0 && blockIdx.y == gridDim.y - 1) {  // (when level 1 rode in the launch the sums depend on)
+        sum_rider_body(rider);
+        return;
+    }
     const SegArgs &a = jobs.j[blockIdx.y];
     const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x >> 6;
     const int64_t j = blockIdx.x / nch;
@@ -192,45 +110,77 @@ __global__ __launch_bounds__(256) void seg_reduce_l2(SegArgs3 jobs, int nch)
     }
 }
 
-int launch_seg_reduce_jobs(const SegJob *jobs, int n_jobs, hipStream_t st, kge_timeline *timeline, const SumRider *rider)
+// Kernel arguments and grid of the level-1 pass over `jobs`.
+static int plan_jobs(const SegJob *jobs, int n_jobs, SegL1Rider *out, int64_t *max_blocks, int64_t *max_nch)
 {
-    const SumRider rd = rider && rider->max_sums > 0 ? *rider : SumRider{};
-    if (rd.max_sums > 0 && (rd.row_floats % 4 != 0 || !aligned16(rd.part) || !aligned16(rd.out))) return KGE_EINVAL;
-    SegArgs3 args{};
+    SegL1Rider r{};
     int m = 0;
-    int64_t max_waves = 0, max_blocks = 0, max_nch = 1;
+    int64_t max_waves = 0;
+    *max_blocks = 0, *max_nch = 1;
     bool v4 = true;
     for (int q = 0; q < n_jobs && m < 3; ++q) {
         const SegJob &jb = jobs[q];
         if (!jb.ins || jb.ins->n == 0 || jb.d == 0) continue;
-        args.j[m] = SegArgs{jb.occ, jb.identity_perm ? nullptr : jb.ins->perm, jb.ins->sorted_seg,
-                            jb.ins->seg_offsets, jb.ins->n, jb.d, jb.out, jb.partial,
-                            jb.scale_num, jb.scale_den, (jb.scaled ? 1 : 0) | (jb.sign_rows ? 2 : 0)};
+        r.jobs.j[m] = SegArgs{jb.occ, jb.identity_perm ? nullptr : jb.ins->perm, jb.ins->sorted_seg,
+                              jb.ins->seg_offsets, jb.ins->n, jb.d, jb.out, jb.partial,
+                              jb.scale_num, jb.scale_den, (jb.scaled ? 1 : 0) | (jb.sign_rows ? 2 : 0)};
         v4 = v4 && jb.d % 4 == 0 && aligned16(jb.occ) && aligned16(jb.out) && aligned16(jb.partial);
         ++m;
     }
-    if (m == 0 && rd.max_sums == 0) return KGE_OK;
     for (int q = 0; q < m; ++q) {
         const int V = v4 ? 4 : 1;
-        const int64_t nblk = ceil_div(args.j[q].n, kSegL);
-        const int64_t nch = ceil_div(args.j[q].d, kWave * V);
+        const int64_t nblk = ceil_div(r.jobs.j[q].n, kSegL);
+        const int64_t nch = ceil_div(r.jobs.j[q].d, kWave * V);
         max_waves = nblk * nch > max_waves ? nblk * nch : max_waves;
-        max_blocks = nblk > max_blocks ? nblk : max_blocks;
-        max_nch = nch > max_nch ? nch : max_nch;
+        *max_blocks = nblk > *max_blocks ? nblk : *max_blocks;
+        *max_nch = nch > *max_nch ? nch : *max_nch;
     }
-    for (int q = m; q < 3; ++q) args.j[q] = args.j[0], args.j[q].n = 0;  // unused slots do nothing
-    int64_t g1x = ceil_div(max_waves, 4);
+    for (int q = m; q < 3; ++q) r.jobs.j[q] = r.jobs.j[0], r.jobs.j[q].n = 0;  // unused slots do nothing
+    r.n_jobs = m, r.v4 = v4 ? 1 : 0;
+    r.blocks_x = (int)ceil_div(max_waves, 4);
+    *out = r;
+    return m;
+}
+
+SegL1Rider plan_seg_l1_rider(const SegJob *jobs, int n_jobs)
+{
+    SegL1Rider r{};
+    int64_t mb, mn;
+    plan_jobs(jobs, n_jobs, &r, &mb, &mn);
+    return r;
+}
+
+int launch_seg_reduce_jobs(const SegJob *jobs, int n_jobs, hipStream_t st, kge_timeline *timeline, const SumRider *rider,
+                           bool level1_rode)
+{
+    const SumRider rd = rider && rider->max_sums > 0 ? *rider : SumRider{};
+    if (rd.max_sums > 0 && (rd.row_floats % 4 != 0 || !aligned16(rd.part) || !aligned16(rd.out))) return KGE_EINVAL;
+    SegL1Rider pl{};
+    int64_t max_blocks = 0, max_nch = 1;
+    const int m = plan_jobs(jobs, n_jobs, &pl, &max_blocks, &max_nch);
+    if (m == 0 && rd.max_sums == 0) return KGE_OK;
+    const SegArgs3 &args = pl.jobs;
+    const bool v4 = pl.v4 != 0;
+    const SumRider none{};
+    int64_t g1x = pl.blocks_x;
     if (rd.max_sums > 0 && g1x < 256) g1x = 256;  // (a small reduction still gives the rider a grid's worth of workgroups)
-    const dim3 g1((unsigned)g1x, (unsigned)(m + (rd.max_sums > 0 ? 1 : 0))), g2((unsigned)(max_blocks * max_nch), (unsigned)m), block(256);
-    const bool level2 = m > 0;
+    int64_t g2x = max_blocks * max_nch;
+    if (level1_rode && rd.max_sums > 0 && g2x < 256) g2x = 256;
+    const bool r1 = !level1_rode && rd.max_sums > 0, r2 = level1_rode && rd.max_sums > 0;
+    const dim3 g1((unsigned)g1x, (unsigned)(m + (r1 ? 1 : 0))), g2((unsigned)g2x, (unsigned)(m + (r2 ? 1 : 0))), block(256);
+    const bool level2 = m > 0 || r2;
     if (v4) {
-        hipLaunchKernelGGL(seg_reduce_l1<4>, g1, block, 0, st, args, rd);
-        timeline_mark(timeline, st, "seg_reduce_l1");
-        if (level2) hipLaunchKernelGGL(seg_reduce_l2<4>, g2, block, 0, st, args, (int)max_nch);
+        if (!level1_rode) {
+            hipLaunchKernelGGL(seg_reduce_l1<4>, g1, block, 0, st, args, r1 ? rd : none);
+            timeline_mark(timeline, st, "seg_reduce_l1");
+        }
+        if (level2) hipLaunchKernelGGL(seg_reduce_l2<4>, g2, block, 0, st, args, (int)max_nch, r2 ? rd : none);
     } else {
-        hipLaunchKernelGGL(seg_reduce_l1<1>, g1, block, 0, st, args, rd);
-        timeline_mark(timeline, st, "seg_reduce_l1");
-        if (level2) hipLaunchKernelGGL(seg_reduce_l2<1>, g2, block, 0, st, args, (int)max_nch);
+        if (!level1_rode) {
+            hipLaunchKernelGGL(seg_reduce_l1<1>, g1, block, 0, st, args, r1 ? rd : none);
+            timeline_mark(timeline, st, "seg_reduce_l1");
+        }
+        if (level2) hipLaunchKernelGGL(seg_reduce_l2<1>, g2, block, 0, st, args, (int)max_nch, r2 ? rd : none);
     }
     if (level2) timeline_mark(timeline, st, "seg_reduce_l2");
     KGE_CHECK_LAUNCH();

@@ -1262,13 +1262,20 @@ __device__ __forceinline__ bool transr_dm_work(const DmArgs &a, float *lds, int 
     return true;
 }
 
-__global__ __launch_bounds__(256, KGE_TR_OCC) void transr_dm_kernel(DmArgs a, FusedInsp fi)
+// Grid: inspector workgroups (if any), kDmWgs workgroups of dM work, then the level-1 workgroups of the step's
+// segmented reductions (entity rows from the dX launch's occurrence rows, relation rows from the forward's
+// residual rows): they depend on nothing this kernel writes and run in the shadow of its long items.
+__global__ __launch_bounds__(256, KGE_TR_OCC) void transr_dm_kernel(DmArgs a, FusedInsp fi, SegL1Rider sr)
 {
     extern __shared__ __align__(16) float lds[];  // dm_lds_bytes(); inspector workgroups: their own need
     if (fused_insp_block(fi, reinterpret_cast<uint32_t *>(lds))) return;
+    const int bid = (int)blockIdx.x - fi.blocks;
+    if (bid >= kDmWgs) {
+        seg_l1_rider_block(sr, bid - kDmWgs);
+        return;
+    }
     const int n_long = a.plan.num_items[0], n_small = a.plan.num_items[1], n_thin = a.plan.num_thin[0];
-    const int stride = (int)gridDim.x - fi.blocks;
-    for (int it = (int)blockIdx.x - fi.blocks; transr_dm_work(a, lds, it, n_long, n_small, n_thin); it += stride)
+    for (int it = bid; transr_dm_work(a, lds, it, n_long, n_small, n_thin); it += kDmWgs)
         __syncthreads();  // the next item reuses the staging buffers
 }
 
@@ -1566,7 +1573,7 @@ int launch_rescal_neg_bwd(const kge_tables *tab, const kge_batch *bat, const kge
     timeline_mark(bat->timeline, st, "transr_gemm_kernel<dX>");
     DmArgs da{xs, qs, ri->seg_offsets, dplan, grads->aux_rows, reinterpret_cast<float *>(ws + p.off_dpart), d, ri->num_unique,
               BwdSrc{}, nullptr, nullptr, 0};
-    hipLaunchKernelGGL(transr_dm_kernel, dim3((unsigned)kDmWgs), dim3(256), dm_lds_bytes(d), st, da, FusedInsp{});
+    hipLaunchKernelGGL(transr_dm_kernel, dim3((unsigned)kDmWgs), dim3(256), dm_lds_bytes(d), st, da, FusedInsp{}, SegL1Rider{});
     timeline_mark(bat->timeline, st, "transr_dm_kernel");
     KGE_CHECK_LAUNCH();
     if (bat->insp_ready && hipStreamWaitEvent(st, reinterpret_cast<hipEvent_t>(bat->insp_ready), 0) != hipSuccess)
@@ -1635,19 +1642,25 @@ int launch_transr_bwd(const kge_tables *tab, const kge_batch *bat, const kge_sav
     hipLaunchKernelGGL(transr_gemm_kernel<2>, dim3((unsigned)(p.tiles + ga.thin_groups + f2.blocks)), dim3(256),
                        lds_with(f2, gemm_lds_bytes(d)), st, ga, f2);
     timeline_mark(bat->timeline, st, "transr_gemm_kernel<dX>");
-    hipLaunchKernelGGL(transr_dm_kernel, dim3((unsigned)(kDmWgs + f3.blocks)), dim3(256), lds_with(f3, dm_lds_bytes(d)), st, da, f3);
-    timeline_mark(bat->timeline, st, "transr_dm_kernel");
-    KGE_CHECK_LAUNCH();
-    if (bat->insp_ready && hipStreamWaitEvent(st, reinterpret_cast<hipEvent_t>(bat->insp_ready), 0) != hipSuccess)
-        return KGE_ELAUNCH;
     // entity rows from the h / t occurrence rows; dR[g] = sum of the group's upstream rows, formed from the
-    // residual rows as the reduction loads them (scale dpos or dpos / pos, sign for L1)
+    // residual rows as the reduction loads them (scale dpos or dpos / pos, sign for L1).  Level 1 of both rides
+    // in the dM launch, level 2 (with the sums that finish the split groups' dM) follows it.
     SegJob jobs[2] = {{occ, bat->ent_insp, d, grads->ent_rows, reinterpret_cast<float *>(ws + p.off_part_e), false},
                       {saved->residual, ri, d, grads->rel_rows, reinterpret_cast<float *>(ws + p.off_part_r), false}};
     jobs[1].scaled = true, jobs[1].sign_rows = tab->norm_p == 1;
     jobs[1].scale_num = dpos, jobs[1].scale_den = tab->norm_p == 2 ? saved->pos : nullptr;
+    const int n_jobs = rescal ? 1 : 2;
+    if (bat->insp_ready && hipStreamWaitEvent(st, reinterpret_cast<hipEvent_t>(bat->insp_ready), 0) != hipSuccess)
+        return KGE_ELAUNCH;
+    // (not when the last step of a fused entity inspection rides in this launch: level 1 reads its result)
+    const bool ride = f3.blocks == 0;
+    const SegL1Rider sr = ride ? plan_seg_l1_rider(jobs, n_jobs) : SegL1Rider{};
+    hipLaunchKernelGGL(transr_dm_kernel, dim3((unsigned)(kDmWgs + f3.blocks + sr.blocks())), dim3(256), lds_with(f3, dm_lds_bytes(d)), st,
+                       da, f3, sr);
+    timeline_mark(bat->timeline, st, "transr_dm_kernel");
+    KGE_CHECK_LAUNCH();
     const SumRider finish = dm_finish_rider(da, p.dsplit);
-    return launch_seg_reduce_jobs(jobs, rescal ? 1 : 2, st, bat->timeline, &finish);
+    return launch_seg_reduce_jobs(jobs, n_jobs, st, bat->timeline, &finish, ride);
 }
 
 #include "transr_neg.hpp"

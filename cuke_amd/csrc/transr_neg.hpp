@@ -746,7 +746,7 @@ int launch_transr_neg_bwd(const kge_tables *tab, const kge_batch *bat, const kge
     timeline_mark(bat->timeline, st, "transr_gemm_kernel<dX>");
     DmArgs da{xl, ql, x.segl, dplan, grads->aux_rows, reinterpret_cast<float *>(ws + l.dpart), d, ri->num_unique,
               BwdSrc{}, nullptr, nullptr, 0};
-    hipLaunchKernelGGL(transr_dm_kernel, dim3((unsigned)kDmWgs), dim3(256), dm_lds_bytes(d), st, da, FusedInsp{});
+    hipLaunchKernelGGL(transr_dm_kernel, dim3((unsigned)kDmWgs), dim3(256), dm_lds_bytes(d), st, da, FusedInsp{}, SegL1Rider{});
     timeline_mark(bat->timeline, st, "transr_dm_kernel");
     TNEG_BY_WIDTH(d, hipLaunchKernelGGL(tneg_occ_kernel<NQ_>, dim3((unsigned)(ceil_div(s.B, 4) + s.NN)), dim3(256), 0, st, x, dxl,
                                         glist, gcount, occ));
