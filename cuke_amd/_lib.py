@@ -52,13 +52,13 @@ class Batch(C.Structure):
                 ("ent_insp", C.POINTER(Inspection)), ("rel_insp", C.POINTER(Inspection)),
                 ("insp_ready", C.c_void_p), ("neg_mode", C.c_int32), ("fuse_inspection", C.c_int32),
                 ("insp_jobs", C.c_void_p), ("timeline", C.POINTER(Timeline)),
-                ("plans_ready", C.c_int32), ("reserved", C.c_int32)]
+                ("plans_ready", C.c_int32), ("reserved", C.c_int32), ("back_rows", C.c_void_p)]
 
 
 class Saved(C.Structure):
     _fields_ = [("pos", C.c_void_p), ("neg", C.c_void_p), ("side_pos", C.c_void_p),
                 ("side_neg", C.c_void_p), ("residual", C.c_void_p),
-                ("fwd_workspace", C.c_void_p), ("fwd_workspace_bytes", C.c_size_t)]
+                ("fwd_workspace", C.c_void_p), ("fwd_workspace_bytes", C.c_size_t), ("back_rows", C.c_void_p)]
 
 
 class Grads(C.Structure):
@@ -100,6 +100,7 @@ EXPORTS = {
                               C.POINTER(Inspection), C.c_void_p, C.c_size_t, C.c_void_p]),
     "kge_inspect_batch": (C.c_int, [C.POINTER(InspectJob), C.c_int, C.c_void_p]),
     "kge_fused_inspection_ok": (C.c_int, [C.POINTER(Tables), C.POINTER(Batch), C.POINTER(InspectJob)]),
+    "kge_back_rows_ok": (C.c_int, [C.POINTER(Tables), C.POINTER(Batch)]),
     "kge_margin_loss_workspace": (C.c_size_t, [C.c_int64, C.c_int64]),
     "kge_margin_loss": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int64, C.c_int64, C.c_float,
                                   C.c_float, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p,
@@ -129,7 +130,7 @@ EXPORTS = {
 _lib = None
 
 
-ABI_VERSION = 6  # layout of the ctypes structures above; must match kge_abi_version()
+ABI_VERSION = 7  # layout of the ctypes structures above; must match kge_abi_version()
 
 
 def lib() -> C.CDLL:

@@ -12,6 +12,7 @@ int launch_score_neg(const kge_tables *, const kge_batch *, const float *, const
 bool score_neg_carries_positives(const kge_tables *, const kge_batch *);
 size_t neg_split_workspace(const kge_tables *, const kge_batch *);
 int launch_transr_fwd(const kge_tables *, const kge_batch *, float *, float *, void *, size_t, hipStream_t);
+bool back_rows_ok(const kge_tables *, const kge_batch *);
 size_t transr_fwd_workspace(const kge_tables *, const kge_batch *);
 int launch_transr_plan(const kge_tables *, const kge_batch *, void *, size_t, hipStream_t);
 int launch_transr_neg_fwd(const kge_tables *, const kge_batch *, float *, float *, float *, void *, size_t, hipStream_t);
@@ -106,7 +107,13 @@ const char *kge_strerror(int status)
     }
 }
 
-int kge_abi_version(void) { return 6; }
+int kge_abi_version(void) { return 7; }
+
+int kge_back_rows_ok(const kge_tables *tab, const kge_batch *bat)
+{
+    if (!tab || !bat || bat->batch <= 0 || validate_tables(tab) != KGE_OK) return 0;
+    return kge::back_rows_ok(tab, bat) ? 1 : 0;
+}
 
 kge_timeline *kge_timeline_create(int32_t capacity)
 {
@@ -218,6 +225,7 @@ int kge_score_fwd(const kge_tables *tab, const kge_batch *bat, float *pos, float
     hipStream_t st = as_stream(stream);
     KGE_CLEAR_LAUNCH_ERRORS();
     const bool want_neg = neg && bat->neg;
+    if (bat->back_rows && !back_rows_ok(tab, bat)) return KGE_EUNSUPPORTED;  // (only TransR's grouped forward writes them)
     if (want_neg && (tab->model == KGE_TRANSH || tab->model == KGE_TRANSF) && !side_pos) return KGE_EINVAL;
     if (want_neg && tab->model == KGE_ROTATE && !residual) return KGE_EINVAL;  // rotated heads buffer
     if (want_neg && tab->model == KGE_RESCAL && (!residual || bat->neg_mode != KGE_NEG_TAIL))

@@ -123,7 +123,7 @@ static int plan_jobs(const SegJob *jobs, int n_jobs, SegL1Rider *out, int64_t *m
         if (!jb.ins || jb.ins->n == 0 || jb.d == 0) continue;
         r.jobs.j[m] = SegArgs{jb.occ, jb.identity_perm ? nullptr : jb.ins->perm, jb.ins->sorted_seg,
                               jb.ins->seg_offsets, jb.ins->n, jb.d, jb.out, jb.partial,
-                              jb.scale_num, jb.scale_den, (jb.scaled ? 1 : 0) | (jb.sign_rows ? 2 : 0)};
+                              jb.scale_num, jb.scale_den, (jb.scaled ? 1 : 0) | (jb.sign_rows ? 2 : 0), (int)jb.wrap};
         v4 = v4 && jb.d % 4 == 0 && aligned16(jb.occ) && aligned16(jb.out) && aligned16(jb.partial);
         ++m;
     }

@@ -20,6 +20,9 @@ struct SegJob {
     // kernel that writes them out first.  scaled with num null: the rows count as zero.
     bool scaled = false, sign_rows = false;
     const float *scale_num = nullptr, *scale_den = nullptr;
+    // wrap > 0: occurrence i >= wrap takes row i - wrap (and its scale) with the opposite sign: the head and tail
+    // occurrences of a translation model's triple share one row, +row for the head and -row for the tail.
+    int64_t wrap = 0;
 };
 
 inline int64_t seg_partial_floats(int64_t n, int64_t d) { return ceil_div(n > 0 ? n : 1, kSegL) * 2 * d; }
@@ -44,6 +47,7 @@ struct SegArgs {
     float *out, *partial;
     const float *scale_num, *scale_den;   // row transform (SegJob), transform bit 0 = scaled, bit 1 = sign
     int transform;
+    int wrap;                             // SegJob::wrap (0: none)
 };
 struct SegArgs3 {
     SegArgs j[3];
@@ -99,6 +103,13 @@ __device__ __forceinline__ void seg_l1_wave(const SegArgs &a, int64_t w)
     }
 #pragma unroll
     for (int q = 0; q < kSegL; ++q) seg[q] = a.sorted_seg[pc[q]];
+    float wsign[kSegL];
+#pragma unroll
+    for (int q = 0; q < kSegL; ++q) {
+        const bool second = a.wrap > 0 && src[q] >= a.wrap;
+        wsign[q] = second ? -1.0f : 1.0f;
+        src[q] = second ? src[q] - a.wrap : src[q];
+    }
     const int cc = active ? colv : 0;
     Vec<V> v[kSegL];
 #pragma unroll
@@ -117,7 +128,12 @@ __device__ __forceinline__ void seg_l1_wave(const SegArgs &a, int64_t w)
 #pragma unroll
         for (int q = 0; q < kSegL; ++q)
 #pragma unroll
-            for (int e = 0; e < V; ++e) v[q].v[e] = sc[q] * ((a.transform & 2) ? sgn(v[q].v[e]) : v[q].v[e]);
+            for (int e = 0; e < V; ++e) v[q].v[e] = wsign[q] * (sc[q] * ((a.transform & 2) ? sgn(v[q].v[e]) : v[q].v[e]));
+    } else if (a.wrap > 0) {
+#pragma unroll
+        for (int q = 0; q < kSegL; ++q)
+#pragma unroll
+            for (int e = 0; e < V; ++e) v[q].v[e] *= wsign[q];
     }
     // A run starts before this block iff it shares its id with the position in front of the block,
     // and runs on past it iff it shares it with the position behind: two loads instead of the run

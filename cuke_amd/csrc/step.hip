@@ -63,7 +63,7 @@ extern "C" int kge_train_step_staged(const kge_tables *tab, kge_step_batch *cur,
                                   buf->loss_workspace, buf->loss_workspace_bytes, stream)))
             return rc;
     }
-    kge_saved saved{buf->pos, buf->neg, buf->side_pos, buf->side_neg, buf->residual, nullptr, 0};
+    kge_saved saved{buf->pos, buf->neg, buf->side_pos, buf->side_neg, buf->residual, nullptr, 0, bat->back_rows};
     if (projection) saved.fwd_workspace = fws, saved.fwd_workspace_bytes = fws_bytes;
     if ((rc = kge_score_bwd(tab, bat, &saved, buf->dpos, buf->dneg, &buf->grads, buf->bwd_workspace, buf->bwd_workspace_bytes, stream)))
         return rc;

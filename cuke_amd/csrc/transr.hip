@@ -186,6 +186,7 @@ struct BwdSrc {
     const int32_t *perm;
     int norm_p, rescal;
     float *occ_v;  // RESCAL: [B, d] occurrence rows of the tails, g * (E[h] Proj[r]); written by the dX kernel
+    int unit;      // non-zero: every coefficient is 1 (the rows phi(residual) Proj^T themselves: GemmArgs::back)
 };
 
 struct RowMeta {
@@ -201,9 +202,9 @@ __device__ __forceinline__ RowMeta bwd_row_meta(const BwdSrc &s, int p, int d)
 {
     RowMeta m;
     m.b = s.perm[p];
-    const float g = s.dpos ? s.dpos[m.b] : 0.0f;
+    const float g = s.unit ? 1.0f : (s.dpos ? s.dpos[m.b] : 0.0f);
     m.coef = g;
-    if (!s.rescal && s.norm_p == 2) {
+    if (!s.unit && !s.rescal && s.norm_p == 2) {
         const float sc = s.spos[m.b];
         m.coef = sc > 0.0f ? g / sc : 0.0f;
     }
@@ -231,6 +232,7 @@ struct GemmArgs {
     int thin_groups;       // upper bound of the number of relation groups = trailing thin workgroups
     int max_tiles;         // leading workgroups: planned tiles
     BwdSrc src;            // TRANSPOSED pass without xs
+    float *back;           // forward TransR, optional: [B, d] rows phi(y_b) Proj^T, a second sweep of the tile / thin group
 };
 
 // ---- thin path: the last <= kThin triples of a relation group ---------------------------------
@@ -843,6 +845,19 @@ __global__ __launch_bounds__(256, KGE_TR_OCC) void transr_gemm_kernel(GemmArgs a
     extern __shared__ __align__(16) float lds[];
     if (fused_insp_block(fi, reinterpret_cast<uint32_t *>(lds))) return;  // an inspector workgroup riding along
     transr_gemm_body<MODE>(a, lds, (int)blockIdx.x - fi.blocks);
+    if constexpr (MODE == 0) {
+        // The entity gradients of the backward pass are coef_b * (phi(y_b) Proj^T): everything but the coefficient
+        // is known here, while this workgroup's projection is still in the caches and no launch, index chain or
+        // ramp stands between the two sweeps.  The rows y_b were written by this workgroup's own waves: the
+        // barrier makes them visible to all of them.
+        if (a.back) {  // uniform
+            __syncthreads();
+            GemmArgs z = a;
+            z.xs = nullptr, z.pos = nullptr, z.resid = nullptr, z.occ_h = a.back, z.occ_t = nullptr;
+            z.src = BwdSrc{a.ent, a.resid, nullptr, nullptr, a.h, a.t, a.perm, a.norm_p, 0, nullptr, 1};
+            transr_gemm_body<2>(z, lds, (int)blockIdx.x - fi.blocks);
+        }
+    }
 }
 
 static size_t gemm_lds_bytes(int d)  // the larger of the tile layout and the thin layouts
@@ -1403,15 +1418,24 @@ static size_t lds_with(const FusedInsp &fi, size_t own)
     return fi.blocks > 0 && (size_t)fi.lds_bytes > own ? (size_t)fi.lds_bytes : own;
 }
 
+// Whether the forward pass of this batch can also write the rows phi(y_b) Proj^T (kge_batch.back_rows).
+bool back_rows_ok(const kge_tables *tab, const kge_batch *bat)
+{
+    return tab->model == KGE_TRANSR && bat->rel_insp && !bat->neg && !pad_path_ok(tab, bat) && mfma_path_ok(tab, bat) &&
+           gemm_lds_bytes((int)tab->dim) <= kMaxGemmLds;
+}
+
 int launch_transr_fwd(const kge_tables *tab, const kge_batch *bat, float *pos, float *resid, void *workspace,
                       size_t workspace_bytes, hipStream_t st)
 {
     if (bat->batch == 0) return KGE_OK;
+    if (bat->back_rows && (!back_rows_ok(tab, bat) || !resid || !aligned16(bat->back_rows))) return KGE_EUNSUPPORTED;
     if (pad_path_ok(tab, bat) && workspace && workspace_bytes >= transr_fwd_workspace_padded(tab, bat))
         return launch_transr_fwd_padded(tab, bat, pos, resid, workspace, workspace_bytes, st);
     const bool rescal = tab->model == KGE_RESCAL;
     const bool grouped = mfma_path_ok(tab, bat) && workspace && workspace_bytes >= transr_fwd_workspace(tab, bat) &&
                          gemm_lds_bytes((int)tab->dim) <= kMaxGemmLds;
+    if (bat->back_rows && !grouped) return KGE_EWORKSPACE;
     // fused entity inspection: its histogram step rides with the forward GEMM
     FusedInsp fi{};
     if (bat->fuse_inspection) {
@@ -1434,7 +1458,7 @@ int launch_transr_fwd(const kge_tables *tab, const kge_batch *bat, float *pos, f
                            kTM, dplan, kDmChunk, dm_nib(tab->dim), dm_small_max(tab->dim));
     GemmArgs a{tab->ent, tab->rel, tab->aux, bat->h, bat->r, bat->t, ri->perm, ri->seg_offsets, ri->num_unique, ri->unique_ids,
                plan, nullptr, nullptr, pos, resid, nullptr, nullptr, (int)tab->dim, tab->norm_p, thin_groups(tab, bat), (int)tiles,
-               BwdSrc{}};
+               BwdSrc{}, bat->back_rows};
     const size_t lds = lds_with(fi, gemm_lds_bytes((int)tab->dim));
     const dim3 grid((unsigned)(tiles + a.thin_groups + fi.blocks));
     if (const int rc = rescal ? allow_lds<1>(lds) : allow_lds<0>(lds)) return rc;
@@ -1588,6 +1612,7 @@ int launch_transr_bwd(const kge_tables *tab, const kge_batch *bat, const kge_sav
 {
     const bool rescal = tab->model == KGE_RESCAL;
     if (bat->neg) return KGE_EUNSUPPORTED;  // (shared negatives: launch_transr_neg_bwd / launch_rescal_neg_bwd)
+    if (saved->back_rows && !back_rows_ok(tab, bat)) return KGE_EINVAL;  // (no forward pass writes them for this batch)
     if (pad_path_ok(tab, bat)) return launch_transr_bwd_padded(tab, bat, saved, dpos, grads, workspace, workspace_bytes, st);
     if (!mfma_path_ok(tab, bat) || gemm_lds_bytes((int)tab->dim) > kMaxGemmLds) return KGE_EUNSUPPORTED;
     if (!saved->residual || !grads->aux_rows || !grads->ent_rows) return KGE_EINVAL;
@@ -1638,10 +1663,19 @@ int launch_transr_bwd(const kge_tables *tab, const kge_batch *bat, const kge_sav
     // dM = X^T Q per relation group
     DmArgs da{nullptr, nullptr, ri->seg_offsets, dplan, grads->aux_rows, reinterpret_cast<float *>(ws + p.off_dpart), d,
               ri->num_unique, src, factored ? grads->aux_x : nullptr, factored ? grads->aux_q : nullptr, grads->aux_factor_max};
-    if (const int rc = allow_lds<2>(lds_with(f2, gemm_lds_bytes(d)))) return rc;
-    hipLaunchKernelGGL(transr_gemm_kernel<2>, dim3((unsigned)(p.tiles + ga.thin_groups + f2.blocks)), dim3(256),
-                       lds_with(f2, gemm_lds_bytes(d)), st, ga, f2);
-    timeline_mark(bat->timeline, st, "transr_gemm_kernel<dX>");
+    // With the forward pass's rows z_b = phi(y_b) Proj^T at hand (kge_saved.back_rows) the entity gradients are
+    // +-coef_b z_b and no kernel reads the projections again: the reduction scales the rows as it loads them.
+    const bool have_back = saved->back_rows != nullptr;
+    if (have_back && (rescal || !aligned16(saved->back_rows))) return KGE_EINVAL;
+    if (!have_back) {
+        if (const int rc = allow_lds<2>(lds_with(f2, gemm_lds_bytes(d)))) return rc;
+        hipLaunchKernelGGL(transr_gemm_kernel<2>, dim3((unsigned)(p.tiles + ga.thin_groups + f2.blocks)), dim3(256),
+                           lds_with(f2, gemm_lds_bytes(d)), st, ga, f2);
+        timeline_mark(bat->timeline, st, "transr_gemm_kernel<dX>");
+    } else if (f2.blocks > 0) {  // the inspector step that would have ridden with dX
+        hipLaunchKernelGGL(transr_insp_step_kernel, dim3((unsigned)f2.blocks), dim3(256), lds_with(f2, 0), st, f2);
+        timeline_mark(bat->timeline, st, "inspector step");
+    }
     // entity rows from the h / t occurrence rows; dR[g] = sum of the group's upstream rows, formed from the
     // residual rows as the reduction loads them (scale dpos or dpos / pos, sign for L1).  Level 1 of both rides
     // in the dM launch, level 2 (with the sums that finish the split groups' dM) follows it.
@@ -1649,6 +1683,10 @@ int launch_transr_bwd(const kge_tables *tab, const kge_batch *bat, const kge_sav
                       {saved->residual, ri, d, grads->rel_rows, reinterpret_cast<float *>(ws + p.off_part_r), false}};
     jobs[1].scaled = true, jobs[1].sign_rows = tab->norm_p == 1;
     jobs[1].scale_num = dpos, jobs[1].scale_den = tab->norm_p == 2 ? saved->pos : nullptr;
+    if (have_back) {  // occurrence i < B is +coef z_i (the head's), occurrence B + i is -coef z_i (the tail's)
+        jobs[0].occ = saved->back_rows, jobs[0].scaled = true, jobs[0].wrap = B;
+        jobs[0].scale_num = dpos, jobs[0].scale_den = tab->norm_p == 2 ? saved->pos : nullptr;
+    }
     const int n_jobs = rescal ? 1 : 2;
     if (bat->insp_ready && hipStreamWaitEvent(st, reinterpret_cast<hipEvent_t>(bat->insp_ready), 0) != hipSuccess)
         return KGE_ELAUNCH;

@@ -147,6 +147,7 @@ class Forward:
     residual: torch.Tensor | None = None
     flat_pos: torch.Tensor | None = None   # projection models scored through flattened triples: all scores
     fwd_ws: torch.Tensor | None = None     # forward workspace that backward reads again (TransR with negatives)
+    back_rows: torch.Tensor | None = None  # TransR: phi(residual) Proj^T rows written by the forward pass (for_backward)
     batch: tuple = ()
     neg_mode: str = "tail"
     ent_insp: Inspection | None = None
@@ -272,8 +273,13 @@ class KGEModel:
         return torch.empty(max(nb, 1), dtype=torch.uint8, device=self.dev), nb
 
     # -- scalar scores ---------------------------------------------------------------------
-    def score(self, h, r, t, neg=None, chunk=None, ent_insp=None, rel_insp=None, neg_mode="tail") -> Forward:
+    def score(self, h, r, t, neg=None, chunk=None, ent_insp=None, rel_insp=None, neg_mode="tail",
+              for_backward: bool = False) -> Forward:
         """pos[B] and, with shared negatives, neg[B, N] scores.
+
+        ``for_backward`` (TransR without negatives, relation inspection given, dim % 4 == 0): the forward kernel
+        also forms the rows phi(residual) Proj^T while it holds the projections (``Forward.back_rows``), and
+        ``backward()`` then reads no projection again.
 
         ``neg_mode='tail'``: neg[b, k] scores (h_b, r_b, neg_k), the reference's shared-negative layout
         (apps/examples/examples.py:1404-1444); ``'head'``: (neg_k, r_b, t_b), the head-corrupted batches of
@@ -308,6 +314,9 @@ class KGEModel:
                 fw.side_neg = torch.empty((2, B, N), **f32)
         if self.model in ("TransR", "RESCAL", "RotatE"):
             fw.residual = torch.empty((B, self.dim), **f32)
+        if for_backward and B > 0 and _lib.lib().kge_back_rows_ok(C.byref(self._tab), C.byref(bat)):
+            fw.back_rows = torch.empty((B, self.dim), **f32)
+            bat.back_rows = fw.back_rows.data_ptr()
         ws, nb = self._fwd_workspace(bat)
         _lib.check(_lib.lib().kge_score_fwd(C.byref(self._tab), C.byref(bat), _ptr(fw.pos),
                                             _ptr(fw.neg), _ptr(fw.side_pos), _ptr(fw.side_neg),
@@ -372,6 +381,8 @@ class KGEModel:
                              (fw.pos, fw.neg, fw.side_pos, fw.side_neg, fw.residual)])
         if fw.fwd_ws is not None:
             saved.fwd_workspace, saved.fwd_workspace_bytes = fw.fwd_ws.data_ptr(), int(fw.fwd_ws.numel())
+        if fw.back_rows is not None:
+            saved.back_rows = fw.back_rows.data_ptr()
         ent_rows = torch.empty((fw.ent_insp.n, self.dim), **f32)
         rel_rows = torch.empty((B, self.rel_dim), **f32) if self.rel_dim else None
         aux_rows = None
@@ -538,7 +549,7 @@ class TrainStep:
     kPipelineSets = 3  # one running, one being inspected, one being refilled
 
     def __init__(self, model: KGEModel, h, r, t, neg=None, chunk=None, loss="sum", margin=1.0,
-                 sign=1.0, dpos=None, dneg=None, neg_mode="tail", factor_max=0):
+                 sign=1.0, dpos=None, dneg=None, neg_mode="tail", factor_max=0, back_rows=True):
         self.m = model
         dev = model.dev
         L = self.L = _lib.lib()
@@ -573,6 +584,12 @@ class TrainStep:
             raise KgeError(f"TransR with shared negatives at batch {B} x {N} negatives, dim {model.dim}, {model.n_rel} relations: "
                            "the grouped path's worst-case workspaces exceed the library's cap; score the pairs as "
                            "explicit triples (KGEModel.score) or use smaller chunks of the batch")
+        # TransR without negatives: the forward kernel also writes phi(residual) Proj^T, and the backward pass
+        # reads no projection again (back_rows=False: backward forms the entity gradients with its own pass)
+        self.back_rows = None
+        if back_rows and B > 0 and L.kge_back_rows_ok(C.byref(model._tab), C.byref(self.bat)):
+            self.back_rows = torch.empty((B, model.dim), **f32)
+            self._sets[0].bat.back_rows = self.back_rows.data_ptr()
         self._ws_f_bytes = int(L.kge_score_fwd_workspace(C.byref(model._tab), C.byref(self.bat)))
         self._ws_f = torch.empty(max(self._ws_f_bytes, 1), dtype=torch.uint8, device=dev)
         # TransR / RESCAL without negatives: the forward workspace holds the batch's tile plans, which a
@@ -592,6 +609,8 @@ class TrainStep:
                                   (self.pos, self.neg, self.side_pos, self.side_neg, self.residual)])
         if self.needs_rel_groups and self._ws_f_bytes:  # backward reuses the forward pass's tile plans
             self.saved.fwd_workspace, self.saved.fwd_workspace_bytes = self._ws_f.data_ptr(), self._ws_f_bytes
+        if self.back_rows is not None:
+            self.saved.back_rows = self.back_rows.data_ptr()
         self.ent_rows = torch.empty((n_occ, model.dim), **f32)
         self.rel_rows = torch.empty((B, model.rel_dim), **f32) if model.rel_dim else None
         self.aux_rows = None
@@ -642,6 +661,8 @@ class TrainStep:
                            neg.data_ptr() if neg is not None else None, self.C, self.N,
                            C.pointer(s.ent_insp._c), C.pointer(s.rel_insp._c), None, NEG_MODES[self._neg_mode], 0)
         s.bat.insp_jobs = C.addressof(s.jobs)
+        if getattr(self, "back_rows", None) is not None:
+            s.bat.back_rows = self.back_rows.data_ptr()
         s.fusable = bool(L.kge_fused_inspection_ok(C.byref(m._tab), C.byref(s.bat), s.jobs))
         s.insp_event = torch.cuda.Event()
         s.done_event = None  # recorded on the main stream after the last pipelined step that used this set
@@ -740,8 +761,11 @@ class TrainStep:
         elif self.needs_rel_groups:
             _lib.check(self.L.kge_inspect_batch(C.byref(self._jobs[1]), 1, st), "kge_inspect_batch")
 
-    def forward(self, st):
-        _lib.check(self.L.kge_score_fwd(C.byref(self.m._tab), C.byref(self.bat), _ptr(self.pos), _ptr(self.neg),
+    def forward(self, st, for_backward=True):
+        bat = self.bat
+        if self.back_rows is not None:  # a forward-only step does not pay for the rows of the backward pass
+            bat.back_rows = self.back_rows.data_ptr() if for_backward else None
+        _lib.check(self.L.kge_score_fwd(C.byref(self.m._tab), C.byref(bat), _ptr(self.pos), _ptr(self.neg),
                                         _ptr(self.side_pos), _ptr(self.side_neg), _ptr(self.residual),
                                         _ptr(self._fwd_ws()), self._ws_f_bytes, st), "kge_score_fwd")
 
@@ -893,7 +917,7 @@ class TrainStep:
             self.inspect(st, backward)
             if backward or self.needs_rel_groups:
                 self._mark("inspect", st)
-            self.forward(st)
+            self.forward(st, backward)
             if backward:
                 self.loss_grad(st)
                 self.backward(st)
@@ -1003,7 +1027,7 @@ class TrainStep:
         bat.insp_ready, bat.fuse_inspection = None, 0
         if self.needs_rel_groups and not self._plans_per_set:    # (shared negatives: groups needed by the forward call)
             _lib.check(self.L.kge_inspect_batch(C.byref(self._jobs[1]), 1, st), "kge_inspect_batch(relations)")
-        self.forward(st)
+        self.forward(st, backward)
         if backward:
             self.loss_grad(st)
             self.backward(st)
@@ -1026,6 +1050,7 @@ class TrainStep:
             sb = _lib.StepBatch()
             sb.bat = s_.bat
             sb.bat.insp_ready, sb.bat.fuse_inspection, sb.bat.plans_ready, sb.bat.timeline = None, 0, 0, None
+            sb.bat.back_rows = self.back_rows.data_ptr() if self.back_rows is not None else None
             if self._plans_per_set:
                 if getattr(s_, "ws_f", None) is None:
                     s_.ws_f = torch.empty(max(self._ws_f_bytes, 1), dtype=torch.uint8, device=self.m.dev)

@@ -177,6 +177,16 @@ typedef struct kge_batch {
        batch ahead on another stream. */
     int32_t plans_ready;
     int32_t reserved;
+    /* TransR on its grouped path without shared negatives, optional (kge_back_rows_ok says whether a batch
+       qualifies; kge_score_fwd returns KGE_EUNSUPPORTED for a batch that sets it and does not): [B, dim]
+       floats that kge_score_fwd fills with z_b = phi(y_b) Proj[r_b]^T, y_b the residual row of triple b and
+       phi = sign for L1, identity for L2, formed by the forward kernel while it holds the projection.  The
+       entity gradient of triple b is +-coef_b z_b (coef_b = dpos_b for L1, dpos_b / pos_b for L2), so a
+       backward call that is handed the rows (kge_saved.back_rows) needs no second pass over the
+       projections: it launches no dX kernel and its reduction scales the rows as it loads them.  The
+       residual rows must be requested in the same call.  No counterpart in the reference, which has no
+       executed backward pass (apps/kge/kge.py:393-515). */
+    float *back_rows;
 } kge_batch;
 
 /* Forward outputs that backward consumes. */
@@ -196,6 +206,9 @@ typedef struct kge_saved {
        negatives (the group list and the projected rows live there). */
     const void *fwd_workspace;
     size_t fwd_workspace_bytes;
+    /* TransR, optional: the rows kge_score_fwd wrote to kge_batch.back_rows for this batch (see there).
+       NULL: kge_score_bwd forms the entity gradients with its own pass over the projections. */
+    const float *back_rows;
 } kge_saved;
 
 /* Sparse row gradients: row u of each array belongs to the u-th unique id of the
@@ -318,6 +331,10 @@ int kge_inspect_batch(const kge_inspect_job *jobs, int n_jobs, void *stream);
 /* 1 if a batch with these two jobs (see kge_batch.fuse_inspection) can have its inspection fused
    into the score kernels, else 0. */
 int kge_fused_inspection_ok(const kge_tables *tab, const kge_batch *bat, const kge_inspect_job *jobs);
+/* 1 if kge_score_fwd fills kge_batch.back_rows for this batch (TransR, relation inspection given, no shared
+   negatives, row width a multiple of four and within the grouped kernels' range), else 0.  No counterpart in
+   the reference. */
+int kge_back_rows_ok(const kge_tables *tab, const kge_batch *bat);
 
 /*
  * Margin-ranking loss over score pairs and its gradient:

@@ -34,7 +34,7 @@ def test_binding_table_matches_header():
 def test_strerror_and_version_without_gpu():
     from cuke_amd import _lib
     L = _lib.lib()
-    assert L.kge_abi_version() == _lib.ABI_VERSION == 6
+    assert L.kge_abi_version() == _lib.ABI_VERSION == 7
     assert L.kge_strerror(0) == b"ok"
     assert b"workspace" in L.kge_strerror(-4)
 
@@ -192,3 +192,49 @@ def test_fused_inspection_eligibility_is_decided_on_the_host():
     bat = batch()
     bat.fuse_inspection = 1
     assert L.kge_score_fwd(C.byref(tables("DistMult")), C.byref(bat), fake, fake, None, None, None, None, 0, None) == -1
+
+
+def test_back_rows_are_offered_only_where_the_forward_pass_writes_them():
+    """kge_batch.back_rows (the rows phi(residual) Proj^T that spare the backward pass its second read of the
+    projections): kge_back_rows_ok says which batches qualify, and the forward call refuses the others before
+    it launches anything."""
+    import ctypes as C
+    from cuke_amd import _lib
+    L = _lib.lib()
+    EUNSUPPORTED = -5
+    fake = C.c_void_p(0x1000)
+
+    def tables(model, dim=200, p=2):
+        rel_dim = 0 if model == "RESCAL" else dim
+        aux = fake if model in ("TransH", "TransR", "RESCAL") else None
+        return _lib.Tables(_lib.MODELS[model], p, 0.0, 0, dim, rel_dim, 1000, 100, fake, fake if rel_dim else None, aux)
+
+    rel = _lib.Inspection(64, 100, fake, fake, fake, fake, fake, fake)
+
+    def batch(neg=False, with_rel=True):
+        return _lib.Batch(64, fake, fake, fake, fake if neg else None, 64 if neg else 0, 8 if neg else 0, None,
+                          C.pointer(rel) if with_rel else None, None, 0, 0, None)
+
+    ok = lambda model, bat, **kw: L.kge_back_rows_ok(C.byref(tables(model, **kw)), C.byref(bat))
+    assert ok("TransR", batch()) == 1
+    assert ok("TransR", batch(), p=1) == 1
+    assert ok("TransR", batch(), dim=1024) == 1
+    assert ok("TransR", batch(), dim=202) == 0          # padded problem: no rows
+    assert ok("TransR", batch(), dim=2048) == 0         # outside the grouped kernels
+    assert ok("TransR", batch(neg=True)) == 0
+    assert ok("TransR", batch(with_rel=False)) == 0
+    assert ok("RESCAL", batch()) == 0
+    assert ok("TransE", batch()) == 0
+    # the forward call refuses a batch that asks for the rows and does not qualify
+    bat = batch()
+    bat.back_rows = fake
+    assert L.kge_score_fwd(C.byref(tables("TransE")), C.byref(bat), fake, None, None, None, None, None, 0, None) == EUNSUPPORTED
+    assert L.kge_score_fwd(C.byref(tables("RESCAL")), C.byref(bat), fake, None, None, None, fake, fake, 1 << 20, None) == EUNSUPPORTED
+    # and a backward call that is handed rows for such a batch is an error of the caller
+    saved = _lib.Saved(fake, None, None, None, fake, None, 0, fake)
+    grads = _lib.Grads(fake, fake, fake, None, None, 0, 0)
+    ent = _lib.Inspection(128, 1000, fake, fake, fake, fake, fake, fake)
+    b2 = batch()
+    b2.ent_insp = C.pointer(ent)
+    assert L.kge_score_bwd(C.byref(tables("TransR", dim=202)), C.byref(b2), C.byref(saved), fake, None, C.byref(grads),
+                           fake, 1 << 30, None) == -1

@@ -9,10 +9,10 @@ from helpers import assert_close, gpu_model
 pytestmark = pytest.mark.gpu
 
 
-def grouped_forward(m, ix):
+def grouped_forward(m, ix, for_backward=False):
     from cuke_amd.kge import inspect
     rel = inspect([ix["r"]], m.n_rel)
-    return m.score(ix["h"], ix["r"], ix["t"], rel_insp=rel), rel
+    return m.score(ix["h"], ix["r"], ix["t"], rel_insp=rel, for_backward=for_backward), rel
 
 
 @pytest.mark.parametrize("model", ["TransR", "RESCAL"])
@@ -66,16 +66,22 @@ def test_grouped_forward(oracle, model, shape, p):
     dict(dim=7, batch=9, n_rel=2),
 ])
 @pytest.mark.parametrize("p", [1, 2])
-def test_grouped_backward(oracle, model, shape, p):
+@pytest.mark.parametrize("back", [False, True])
+def test_grouped_backward(oracle, model, shape, p, back):
+    """back: the forward pass also writes the rows phi(residual) Proj^T (Forward.back_rows) and the backward
+    pass reads no projection again; without them it forms the entity gradients with its own pass."""
     if model == "RESCAL" and p == 1:
         pytest.skip("no norm in RESCAL")
+    if back and (model == "RESCAL" or shape["dim"] % 4 != 0):
+        pytest.skip("back rows: TransR with row widths that are multiples of four")
     w = synth.custom_workload(model, n_ent=120, norm_p=p, sigma=0.2, rel_zipf=1.2, ent_zipf=1.1,
                               seed=shape["dim"] + p, lattice=(p == 1 and model == "TransR"), **shape)
     a = w.arrays
     if w.lattice:  # keep the projected residual exact too: projections on a coarse grid
         a["A"] = (np.rint(a["A"] / 0.2 * 2) / 8).astype(np.float32)
     m, ix = gpu_model(w)
-    fw, rel = grouped_forward(m, ix)
+    fw, rel = grouped_forward(m, ix, for_backward=back)
+    assert (fw.back_rows is not None) == back
     dpos = np.random.default_rng(1).standard_normal(w.batch).astype(np.float32)
     g = m.backward(fw, torch.from_numpy(dpos).to(fw.pos.device))
     ref = oracle.backward(model, a["E"], a["R"], a["A"], a["h"], a["r"], a["t"], dpos=dpos, p=p)
@@ -476,3 +482,36 @@ def test_staged_batches_are_planned_a_step_ahead(oracle):
     step.select(1)
     step.run()
     check(ws[1], "plain run afterwards")
+
+
+@pytest.mark.parametrize("p", [1, 2])
+def test_train_step_with_and_without_back_rows(oracle, p):
+    """TrainStep(back_rows=True), the default where the batch qualifies, against back_rows=False: scores, relation
+    rows and projection gradients come from the same kernels (bit-identical), the entity rows from different
+    ones (coefficient applied after instead of before the product with the transposed projection): both meet
+    the oracle."""
+    from cuke_amd.kge import TrainStep
+    w = synth.make_workload("cfg3_transr", batch=2048, seed=5, norm_p=p)
+    m, ix = gpu_model(w)
+    a = w.arrays
+    dpos = torch.from_numpy(np.random.default_rng(3).standard_normal(w.batch).astype(np.float32)).cuda()
+    steps = [TrainStep(m, ix["h"], ix["r"], ix["t"], dpos=dpos, back_rows=b) for b in (True, False)]
+    assert steps[0].back_rows is not None and steps[1].back_rows is None
+    ref = oracle.backward("TransR", a["E"], a["R"], a["A"], a["h"], a["r"], a["t"], dpos=dpos.cpu().numpy(), p=p)
+    outs = []
+    for st in steps:
+        st.run(overlap=False, fused=False)
+        torch.cuda.synchronize()
+        g = st.sparse_grads()
+        if p == 2:
+            assert_close(g.ent_rows.cpu().numpy(), ref.ent_rows, what="entity rows", rows=True)
+        outs.append((st.pos.clone(), g.ent_ids.clone(), g.ent_rows.clone(), g.rel_rows.clone(), g.aux_rows.clone()))
+    assert torch.equal(outs[0][0], outs[1][0]) and torch.equal(outs[0][1], outs[1][1])
+    assert torch.equal(outs[0][3], outs[1][3]) and torch.equal(outs[0][4], outs[1][4])
+    assert_close(outs[0][2].cpu().numpy(), outs[1][2].cpu().numpy(), what="entity rows, back rows against the dX pass",
+                 rows=True, global_floor=0.5 if p == 1 else 0.0)
+    # a forward-only step leaves the rows alone
+    steps[0].back_rows.fill_(7.0)
+    steps[0].run(backward=False)
+    torch.cuda.synchronize()
+    assert bool((steps[0].back_rows == 7.0).all())
