@@ -51,6 +51,7 @@ PROFILE_KERNELS = {
     "seg_reduce_l1": ["seg_reduce_l1"],
     "seg_reduce_l2": ["seg_reduce_l2"],
     "transr_plan_kernel + transr_gemm_kernel<fwd>": ["transr_plan_kernel", "transr_gemm_kernel<0>"],
+    "transr_plan_kernel + transr_gemm_kernel<fwd + back rows>": ["transr_plan_kernel", "transr_gemm_kernel<0>"],
     "transr_gemm_kernel<dX>": ["transr_gemm_kernel<2>"],
     "transr_dm_kernel": ["transr_dm_kernel"],
 }
@@ -171,6 +172,8 @@ def kernel_model(w, label, u_ent, u_rel):
         return 4 * (u_ent * d) // 8, 0, "valu"
     if label.startswith("transr_plan_kernel") or label == "transr_gemm_kernel<dX>":
         by = 4 * (u_rel * d * d + 3 * B * d + u_rel * d) + 8 * 3 * B
+        if "back rows" in label:  # the forward kernel also does the backward pass's product with the transposed projections
+            return 2 * by, 4 * B * d * d, "mfma"
         return by, 2 * B * d * d, "mfma"
     # dM: the x rows (two entity rows for TransR) and the residual rows in, one gradient per distinct relation out
     # (dense d x d, or 2 d floats per triple for the groups left factored: `dense_rel` / `factored_rows` say how many)
@@ -497,7 +500,7 @@ def run_workload(name, args, torch, factor_max=0):
     sign = 1.0 if w.model in ("DistMult", "ComplEx", "RotatE", "TransF", "RESCAL") else -1.0
     ix = ixs[0]
     step = TrainStep(model, ix["h"], ix["r"], ix["t"], ix.get("neg"), w.chunk or None, loss=w.loss,
-                     margin=w.margin, sign=sign, factor_max=factor_max)
+                     margin=w.margin, sign=sign, factor_max=factor_max, back_rows=not args.no_back_rows)
     if w.model in ("TransR", "RESCAL"):  # what the projection gradients of batch 0 cost to write (algorithmic bytes)
         cnt = np.unique(w.arrays["r"], return_counts=True)[1]
         w.dense_rel, w.factored_rows = int((cnt > factor_max).sum()), int(cnt[cnt <= factor_max].sum())
@@ -690,7 +693,8 @@ def run_workload(name, args, torch, factor_max=0):
                    "unique_entity_rows": u_ent, "unique_relation_rows": u_rel,
                    "projection_gradients": (None if w.model not in ("TransR", "RESCAL") else
                                             {"factor_max": factor_max, "dense_groups": w.dense_rel,
-                                             "factored_rows": w.factored_rows})},
+                                             "factored_rows": w.factored_rows,
+                                             "back_rows_from_forward": step.back_rows is not None})},
         "kernels_ms": [[n_ + (" (side stream, a batch ahead)" if (n_, m_) not in on_step else ""), round(m_, 6)]
                        for n_, m_ in kt],
         "roofline": roofline,
@@ -796,6 +800,9 @@ def main():
     ap.add_argument("--no-check", action="store_true", help="skip the parity spot check (profiling runs)")
     ap.add_argument("--dense-only", action="store_true",
                     help="TransR: time only the step that writes every projection gradient dense (profiling runs)")
+    ap.add_argument("--no-back-rows", action="store_true",
+                    help="TransR: the forward pass does not also form phi(residual) Proj^T; the backward pass reads the "
+                         "projections a second time in a dX kernel of its own (the form before back rows)")
     ap.add_argument("--factored-only", action="store_true",
                     help="TransR: time only the headline step (small groups' projection gradients factored), not "
                          "the dense one beside it (profiling runs)")

@@ -1466,7 +1466,8 @@ int launch_transr_fwd(const kge_tables *tab, const kge_batch *bat, float *pos, f
         hipLaunchKernelGGL(transr_gemm_kernel<1>, grid, dim3(256), lds, st, a, fi);
     else
         hipLaunchKernelGGL(transr_gemm_kernel<0>, grid, dim3(256), lds, st, a, fi);
-    timeline_mark(bat->timeline, st, "transr_plan_kernel + transr_gemm_kernel<fwd>");
+    timeline_mark(bat->timeline, st, a.back ? "transr_plan_kernel + transr_gemm_kernel<fwd + back rows>"
+                                            : "transr_plan_kernel + transr_gemm_kernel<fwd>");
     KGE_CHECK_LAUNCH();
     return KGE_OK;
 }
