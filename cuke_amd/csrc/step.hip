@@ -50,7 +50,9 @@ extern "C" int kge_train_step_staged(const kge_tables *tab, kge_step_batch *cur,
     size_t fws_bytes = buf->fwd_workspace_bytes;
     if (projection && !bat->neg && cur->fwd_workspace) {
         if (!bat->plans_ready || !cur->planned) return KGE_EINVAL;  // staged by an earlier call
-        if (hipStreamWaitEvent(st, as_event(cur->planned), 0) != hipSuccess) return KGE_ELAUNCH;
+        // plans and entity inspection were enqueued together, a step ahead: one wait on the later event covers both
+        if (hipStreamWaitEvent(st, as_event(cur->inspected), 0) != hipSuccess) return KGE_ELAUNCH;
+        bat->insp_ready = nullptr;
         fws = cur->fwd_workspace, fws_bytes = cur->fwd_workspace_bytes;
     } else if (projection) {
         const int rc = kge_inspect_batch(&bat->insp_jobs[1], 1, stream);

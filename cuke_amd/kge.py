@@ -930,7 +930,17 @@ class TrainStep:
             if cur.inputs_ready is not None:
                 main.wait_event(cur.inputs_ready)  # the score kernels read the index tensors too
             if self._plans_per_set:
-                main.wait_event(cur.planned_event)  # relation groups and tile plans of this batch (made in stage())
+                # Relation groups, tile plans and the entity inspection of this batch were all enqueued by stage(), a
+                # step ahead, on the side stream: ONE wait on the event recorded behind the last of them covers the
+                # forward pass (plans) and the backward pass (entity inspection); a second wait in front of the
+                # reduction would cost its 2-3 us for an event that has long fired.
+                main.wait_event(cur.insp_event)
+                cur.bat.insp_ready = None
+                self.forward(st)
+                self.loss_grad(st)
+                self.backward(st)
+                self._record_done(main, pipeline)
+                return
             elif self.needs_rel_groups:
                 _lib.check(self.L.kge_inspect_batch(C.byref(cur.jobs[1]), 1, st), "kge_inspect_batch(relations)")
         else:

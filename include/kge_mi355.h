@@ -443,9 +443,11 @@ int kge_sample_negatives(int64_t *out, int64_t count, int64_t n_ent, uint64_t se
  * (bat.insp_jobs[0] = the entity index set, [1] = the relations; bat.ent_insp / rel_insp point to their
  * `out`), and three events the caller creates once (hipEventCreate; default flags are fine):
  *   inspected  recorded on side_stream behind the batch's inspection; kge_score_bwd waits for it right
- *              before its segmented reduction (kge_batch.insp_ready)
+ *              before its segmented reduction (kge_batch.insp_ready).  TransR / RESCAL without negatives:
+ *              `stream` waits for it once, before the forward pass (it is recorded behind the plans too, and
+ *              the batch was staged a step ahead), and kge_score_bwd has no wait of its own.
  *   planned    TransR / RESCAL without negatives: recorded behind the relation inspection and the tile
- *              plans; `stream` waits for it before the forward pass.  Else unused (may be NULL).
+ *              plans (for callers that pipeline deeper).  Else unused (may be NULL).
  *   released   recorded on `stream` behind the step; a later staging of the same kge_step_batch makes
  *              side_stream wait for it before it overwrites the inspection (released_valid says whether
  *              it has been recorded yet; zero-initialise it).

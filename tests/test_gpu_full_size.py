@@ -223,7 +223,8 @@ def test_preallocated_step_with_riding_inspection_equals_the_eager_path_bit_for_
         pytest.skip("forward-only configuration")
     dpos, dneg = upstream(w, 5)
     g = m.backward(fw, dev(dpos), dev(dneg))
-    step = TrainStep(m, ix["h"], ix["r"], ix["t"], ix.get("neg"), w.chunk or None, dpos=dev(dpos), dneg=dev(dneg))
+    step = TrainStep(m, ix["h"], ix["r"], ix["t"], ix.get("neg"), w.chunk or None, dpos=dev(dpos), dneg=dev(dneg),
+                     back_rows=fw.back_rows is not None)  # (TransR: the same form of the entity gradients as the eager call)
     assert step.fusable
     step.run()
     torch.cuda.synchronize()
