@@ -550,24 +550,24 @@ struct BLoader {
 // ring_prime() issues the first kRing - 1 supersteps; a tile calls it before it stages its left
 // operand (the projection only depends on the tile's relation), so those loads fly during the
 // index chain and the row gathers of the staging.
-template <int MODE>
-__device__ __forceinline__ void ring_prime(const BLoader<MODE> &bl, float4 (&ring)[kRing][4])
+template <int MODE, int RING>
+__device__ __forceinline__ void ring_prime(const BLoader<MODE> &bl, float4 (&ring)[RING][4])
 {
 #pragma unroll
-    for (int u = 0; u + 1 < kRing; ++u) bl.load(u, ring[u]);
+    for (int u = 0; u + 1 < RING; ++u) bl.load(u, ring[u]);
 }
 
-template <int MODE, bool TWO>
-__device__ __forceinline__ void gemm_sweep(const BLoader<MODE> &bl, float4 (&ring)[kRing][4], const float *sX, int pitch,
+template <int MODE, bool TWO, int RING>
+__device__ __forceinline__ void gemm_sweep(const BLoader<MODE> &bl, float4 (&ring)[RING][4], const float *sX, int pitch,
                                            int li, int kk, floatx4 (&acc_lo)[4], floatx4 (&acc_hi)[4])
 {
     const int nq = bl.nq;
     const float *xlo = sX + li * pitch + 4 * kk, *xhi = sX + (16 + li) * pitch + 4 * kk;
-    for (int q = 0; q < nq; q += kRing) {
+    for (int q = 0; q < nq; q += RING) {
 #pragma unroll
-        for (int u = 0; u < kRing; ++u) {
+        for (int u = 0; u < RING; ++u) {
             const int qq = q + u;
-            bl.load(qq + kRing - 1, ring[(u + kRing - 1) % kRing]);
+            bl.load(qq + RING - 1, ring[(u + RING - 1) % RING]);
             __builtin_amdgcn_sched_barrier(0);
             float4 bc[4];
 #pragma unroll
@@ -610,7 +610,7 @@ __device__ __forceinline__ void gemm_sweep(const BLoader<MODE> &bl, float4 (&rin
 // MODE 2: backward dX      x = xs rows,   y = x M^T -> occ_h = y, occ_t = -y (when occ_t is set)
 // MODE 3: list rows        x = E[h]-E[t] (t = -1: no row), y = x M + rs R[r] -> resid rows in list order;
 //         h, t, rs are indexed by the sorted position itself (no perm), no score
-template <int MODE>
+template <int MODE, int RING = kRing>
 __device__ __forceinline__ void transr_gemm_body(const GemmArgs &a, float *lds, int bid)
 {
     // Workgroups [0, max_tiles) take the planned 32-triple tiles, the following `thin_groups`
@@ -653,13 +653,13 @@ __device__ __forceinline__ void transr_gemm_body(const GemmArgs &a, float *lds, 
         wcols = n0 >= c0 + span ? 0 : (c0 + span - n0 < cw ? c0 + span - n0 : cw);
     };
     BLoader<MODE> bl;
-    float4 ring[kRing][4];
+    float4 ring[RING][4];
     {
         int n0, wcols;
         wave_cols(0, n0, wcols);
         if (wcols > 0) {  // per wave; a wave without columns (narrow rows) sits the sweep out
             bl.init(M, d, kpad / 16, n0, wcols, li, kk);
-            ring_prime<MODE>(bl, ring);
+            ring_prime<MODE, RING>(bl, ring);
         }
         __builtin_amdgcn_sched_barrier(0);
     }
@@ -750,7 +750,7 @@ __device__ __forceinline__ void transr_gemm_body(const GemmArgs &a, float *lds, 
         for (int e = 0; e < 4; ++e) acc_lo[e] = floatx4{0.f, 0.f, 0.f, 0.f}, acc_hi[e] = floatx4{0.f, 0.f, 0.f, 0.f};
         if (c0 > 0 && wcols > 0) {  // (the first sweep's ring was primed before the staging)
             bl.init(M, d, kpad / 16, n0, wcols, li, kk);
-            ring_prime<MODE>(bl, ring);
+            ring_prime<MODE, RING>(bl, ring);
         }
         // epilogue operands that do not depend on the products: the relation row (TransR) is requested
         // ahead of the sweep, the tail rows of this lane's eight triples (RESCAL) in one batch behind it
@@ -759,8 +759,8 @@ __device__ __forceinline__ void transr_gemm_body(const GemmArgs &a, float *lds, 
         if constexpr (MODE == 0 || MODE == 3) erow[0] = *reinterpret_cast<const float4 *>(a.rel + rid * (int64_t)d + ecol);
 
         if (wcols > 0) {
-            if (two_blocks) gemm_sweep<MODE, true>(bl, ring, sX, pitch, li, kk, acc_lo, acc_hi);
-            else gemm_sweep<MODE, false>(bl, ring, sX, pitch, li, kk, acc_lo, acc_hi);
+            if (two_blocks) gemm_sweep<MODE, true, RING>(bl, ring, sX, pitch, li, kk, acc_lo, acc_hi);
+            else gemm_sweep<MODE, false, RING>(bl, ring, sX, pitch, li, kk, acc_lo, acc_hi);
         }
         if constexpr (MODE == 1) {  // one batch of unconditional loads (eight rows would not fit beside the ring)
 #pragma unroll
@@ -845,19 +845,172 @@ __global__ __launch_bounds__(256, KGE_TR_OCC) void transr_gemm_kernel(GemmArgs a
     extern __shared__ __align__(16) float lds[];
     if (fused_insp_block(fi, reinterpret_cast<uint32_t *>(lds))) return;  // an inspector workgroup riding along
     transr_gemm_body<MODE>(a, lds, (int)blockIdx.x - fi.blocks);
-    if constexpr (MODE == 0) {
-        // The entity gradients of the backward pass are coef_b * (phi(y_b) Proj^T): everything but the coefficient
-        // is known here, while this workgroup's projection is still in the caches and no launch, index chain or
-        // ramp stands between the two sweeps.  The rows y_b were written by this workgroup's own waves: the
-        // barrier makes them visible to all of them.
-        if (a.back) {  // uniform
-            __syncthreads();
-            GemmArgs z = a;
-            z.xs = nullptr, z.pos = nullptr, z.resid = nullptr, z.occ_h = a.back, z.occ_t = nullptr;
-            z.src = BwdSrc{a.ent, a.resid, nullptr, nullptr, a.h, a.t, a.perm, a.norm_p, 0, nullptr, 1};
-            transr_gemm_body<2>(z, lds, (int)blockIdx.x - fi.blocks);
+}
+
+// ---- forward TransR with the back rows (GemmArgs::back) ---------------------------------------------------
+// The entity gradients of the backward pass are coef_b * (phi(y_b) Proj^T): everything but the coefficient is known
+// at the end of the forward tile.
+//
+// A thin group (at most kThin triples, most distinct relations of a long-tailed batch and four fifths of the
+// projection bytes) reads its projection ONCE for both products: the workgroup requests all of it at the start
+// (RMAX * NQ 128-bit loads per thread, the whole 4 d^2 bytes in flight) and keeps it in registers.  Thread
+// (row group rg = lane / 16 + 4 wave, li = lane % 16) holds rows j = rg + 16 i and the quads c = li + 16 s of each.
+//   y[b][c] = sum_j x[b][j] M[j][c]: per-thread sums over its rows, the four row groups of a wave added with two
+//             cross-lane steps, the four waves through LDS in a fixed order;
+//   z[b][j] = sum_c phi(y)[b][c] M[j][c]: per-thread dot products, the sixteen lanes of a row added with four
+//             DPP steps (as the thin dX pass does).
+// Needs RMAX * NQ * 4 registers for the projection: row widths up to 208 (NQ = ceil(d / 64), RMAX rows per thread).
+template <int NQ>
+__device__ __forceinline__ void transr_thin_both_body(const GemmArgs &a, float *lds, int g)
+{
+    constexpr int RMAX = NQ == 1 ? 4 : (NQ == 2 ? 8 : (NQ == 3 ? 12 : 13));
+    constexpr int RX = 16 * RMAX;  // >= d
+    const ThinTile tt = thin_tile_of_group(a.num_unique, a.seg_offsets, g);
+    const int rows = tt.rows;
+    if (rows == 0) return;
+    const int d = a.d, nq4 = d >> 2, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int li = lane & 15, sub = lane >> 4, rg = 4 * wave + sub;
+    float *sx = lds;                                        // [4][RX] x rows, zero beyond d and beyond `rows`
+    float4 *sW = reinterpret_cast<float4 *>(lds + 4 * RX);  // [4 waves][4 rows][64 quads]
+    float4 *sq = sW + 4 * 4 * 64;                           // [4 rows][64 quads] phi(y), zero beyond the row
+    float *sz = reinterpret_cast<float *>(sq + 4 * 64);     // [4][RX]
+    __shared__ int s_b[kThin];
+    __shared__ int64_t s_h[kThin], s_t[kThin];
+    const int64_t rid = a.unique_ids[g];
+    const float4 *M4 = reinterpret_cast<const float4 *>(a.proj + rid * (int64_t)d * d);
+    float4 m[RMAX][NQ];
+#pragma unroll
+    for (int i = 0; i < RMAX; ++i) {
+        const int j = rg + 16 * i;
+        const int64_t base = (int64_t)(j < d ? j : d - 1) * nq4;  // clamped: unconditional loads, x is zero there
+#pragma unroll
+        for (int q = 0; q < NQ; ++q) {
+            const int c = li + 16 * q;
+            m[i][q] = M4[base + (c < nq4 ? c : 0)];
         }
     }
+    __builtin_amdgcn_sched_barrier(0);
+    if (tid < kThin) {
+        const int b = tid < rows ? a.perm[tt.p0 + tid] : 0;
+        s_b[tid] = b;
+        s_h[tid] = a.h[b];
+        s_t[tid] = a.t[b];
+    }
+    for (int k = tid; k < 4 * RX; k += 256) sx[k] = 0.0f;
+    __syncthreads();
+    for (int f = tid; f < rows * nq4; f += 256) {
+        const int r = f / nq4, k4 = (f % nq4) * 4;
+        const float4 v = *reinterpret_cast<const float4 *>(a.ent + s_h[r] * (int64_t)d + k4);
+        const float4 u = *reinterpret_cast<const float4 *>(a.ent + s_t[r] * (int64_t)d + k4);
+        *reinterpret_cast<float4 *>(&sx[r * RX + k4]) = make_float4(v.x - u.x, v.y - u.y, v.z - u.z, v.w - u.w);
+    }
+    __syncthreads();
+    // y = x M: this thread's rows, then the wave's four row groups
+#pragma unroll
+    for (int b = 0; b < 4; ++b) {
+        float4 acc[NQ];
+#pragma unroll
+        for (int q = 0; q < NQ; ++q) acc[q] = make_float4(0.f, 0.f, 0.f, 0.f);
+#pragma unroll
+        for (int i = 0; i < RMAX; ++i) {
+            const float xv = sx[b * RX + rg + 16 * i];
+#pragma unroll
+            for (int q = 0; q < NQ; ++q) {
+                acc[q].x = fmaf(xv, m[i][q].x, acc[q].x);
+                acc[q].y = fmaf(xv, m[i][q].y, acc[q].y);
+                acc[q].z = fmaf(xv, m[i][q].z, acc[q].z);
+                acc[q].w = fmaf(xv, m[i][q].w, acc[q].w);
+            }
+        }
+#pragma unroll
+        for (int q = 0; q < NQ; ++q) {
+            float v[4] = {acc[q].x, acc[q].y, acc[q].z, acc[q].w};
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                v[e] += __shfl_xor(v[e], 16, kWave);
+                v[e] += __shfl_xor(v[e], 32, kWave);
+            }
+            if (sub == 0) sW[(wave * 4 + b) * 64 + li + 16 * q] = make_float4(v[0], v[1], v[2], v[3]);
+        }
+    }
+    __syncthreads();
+    {   // thread (row b = wave, quad c = lane): the four waves' sums in order, the relation row, the score
+        const int b = wave, c = lane;
+        float4 y = sW[b * 64 + c];
+#pragma unroll
+        for (int w = 1; w < 4; ++w) {
+            const float4 v = sW[(w * 4 + b) * 64 + c];
+            y.x += v.x, y.y += v.y, y.z += v.z, y.w += v.w;
+        }
+        float sum = 0.0f;
+        float4 q = make_float4(0.f, 0.f, 0.f, 0.f);
+        if (c < nq4 && b < rows) {
+            const float4 rv = *reinterpret_cast<const float4 *>(a.rel + rid * (int64_t)d + 4 * c);
+            y.x += rv.x, y.y += rv.y, y.z += rv.z, y.w += rv.w;
+            sum = a.norm_p == 1 ? fabsf(y.x) + fabsf(y.y) + fabsf(y.z) + fabsf(y.w)
+                                : y.x * y.x + y.y * y.y + y.z * y.z + y.w * y.w;
+            if (a.resid) *reinterpret_cast<float4 *>(a.resid + (int64_t)s_b[b] * d + 4 * c) = y;
+            q = a.norm_p == 1 ? sgn4(y) : y;
+        }
+        sq[b * 64 + c] = q;
+        sum = wave_sum(sum);
+        if (lane == 0 && b < rows && a.pos) a.pos[s_b[b]] = a.norm_p == 2 ? sqrtf(sum) : sum;
+    }
+    __syncthreads();
+    // z = phi(y) M^T
+#pragma unroll
+    for (int b = 0; b < 4; ++b) {
+        float4 qv[NQ];
+#pragma unroll
+        for (int q = 0; q < NQ; ++q) qv[q] = sq[b * 64 + li + 16 * q];  // zero beyond the row: clamped quads add nothing
+#pragma unroll
+        for (int i = 0; i < RMAX; ++i) {
+            float p = 0.0f;
+#pragma unroll
+            for (int q = 0; q < NQ; ++q)
+                p = fmaf(qv[q].x, m[i][q].x, fmaf(qv[q].y, m[i][q].y, fmaf(qv[q].z, m[i][q].z, fmaf(qv[q].w, m[i][q].w, p))));
+            p = row16_sum(p);
+            if (li == 0) sz[b * RX + rg + 16 * i] = p;
+        }
+    }
+    __syncthreads();
+    for (int f = tid; f < rows * nq4; f += 256) {
+        const int r = f / nq4, k4 = (f % nq4) * 4;
+        *reinterpret_cast<float4 *>(a.back + (int64_t)s_b[r] * d + k4) = *reinterpret_cast<const float4 *>(&sz[r * RX + k4]);
+    }
+}
+
+constexpr int kThinBothMaxDim = 208;
+constexpr int kBackRing = kRing;  // prefetch stages of the tiles in this kernel (4 to 8 stages, which its register budget would allow, measured slower)
+static size_t thin_both_lds_bytes(int d)
+{
+    if (d > kThinBothMaxDim) return 0;
+    const int nq = (d / 4 + 15) / 16, rmax = nq == 1 ? 4 : (nq == 2 ? 8 : (nq == 3 ? 12 : 13));
+    return sizeof(float) * (size_t)(8 * 16 * rmax) + sizeof(float4) * (size_t)(4 * 4 * 64 + 4 * 64);
+}
+
+// Tiles: the second sweep (the dX body on the rows this workgroup has just written, coefficient 1) follows the
+// first at once: no launch, no index chains, no ramp or tail between them; the barrier makes the rows visible to
+// all waves of the workgroup.  Two workgroups per CU: the thin groups' projections live in registers.
+__global__ __launch_bounds__(256, 2) void transr_fwd_back_kernel(GemmArgs a, FusedInsp fi)
+{
+    extern __shared__ __align__(16) float lds[];
+    if (fused_insp_block(fi, reinterpret_cast<uint32_t *>(lds))) return;
+    const int bid = (int)blockIdx.x - fi.blocks;
+    if (bid >= a.max_tiles && a.d <= kThinBothMaxDim) {
+        const int nq = (a.d / 4 + 15) / 16;
+        if (nq <= 1) transr_thin_both_body<1>(a, lds, bid - a.max_tiles);
+        else if (nq == 2) transr_thin_both_body<2>(a, lds, bid - a.max_tiles);
+        else if (nq == 3) transr_thin_both_body<3>(a, lds, bid - a.max_tiles);
+        else transr_thin_both_body<4>(a, lds, bid - a.max_tiles);
+        return;
+    }
+    transr_gemm_body<0, kBackRing>(a, lds, bid);
+    __syncthreads();
+    GemmArgs z = a;
+    z.xs = nullptr, z.pos = nullptr, z.resid = nullptr, z.occ_h = a.back, z.occ_t = nullptr;
+    z.src = BwdSrc{a.ent, a.resid, nullptr, nullptr, a.h, a.t, a.perm, a.norm_p, 0, nullptr, 1};
+    transr_gemm_body<2, kBackRing>(z, lds, bid);
 }
 
 static size_t gemm_lds_bytes(int d)  // the larger of the tile layout and the thin layouts
@@ -1459,13 +1612,22 @@ int launch_transr_fwd(const kge_tables *tab, const kge_batch *bat, float *pos, f
     GemmArgs a{tab->ent, tab->rel, tab->aux, bat->h, bat->r, bat->t, ri->perm, ri->seg_offsets, ri->num_unique, ri->unique_ids,
                plan, nullptr, nullptr, pos, resid, nullptr, nullptr, (int)tab->dim, tab->norm_p, thin_groups(tab, bat), (int)tiles,
                BwdSrc{}, bat->back_rows};
-    const size_t lds = lds_with(fi, gemm_lds_bytes((int)tab->dim));
+    size_t own = gemm_lds_bytes((int)tab->dim);
+    if (a.back && thin_both_lds_bytes((int)tab->dim) > own) own = thin_both_lds_bytes((int)tab->dim);
+    const size_t lds = lds_with(fi, own);
     const dim3 grid((unsigned)(tiles + a.thin_groups + fi.blocks));
-    if (const int rc = rescal ? allow_lds<1>(lds) : allow_lds<0>(lds)) return rc;
-    if (rescal)
-        hipLaunchKernelGGL(transr_gemm_kernel<1>, grid, dim3(256), lds, st, a, fi);
-    else
-        hipLaunchKernelGGL(transr_gemm_kernel<0>, grid, dim3(256), lds, st, a, fi);
+    if (a.back) {
+        if (lds > 64 * 1024 && hipFuncSetAttribute(reinterpret_cast<const void *>(&transr_fwd_back_kernel),
+                                                   hipFuncAttributeMaxDynamicSharedMemorySize, (int)kMaxGemmLds) != hipSuccess)
+            return KGE_ELAUNCH;
+        hipLaunchKernelGGL(transr_fwd_back_kernel, grid, dim3(256), lds, st, a, fi);
+    } else {
+        if (const int rc = rescal ? allow_lds<1>(lds) : allow_lds<0>(lds)) return rc;
+        if (rescal)
+            hipLaunchKernelGGL(transr_gemm_kernel<1>, grid, dim3(256), lds, st, a, fi);
+        else
+            hipLaunchKernelGGL(transr_gemm_kernel<0>, grid, dim3(256), lds, st, a, fi);
+    }
     timeline_mark(bat->timeline, st, a.back ? "transr_plan_kernel + transr_gemm_kernel<fwd + back rows>"
                                             : "transr_plan_kernel + transr_gemm_kernel<fwd>");
     KGE_CHECK_LAUNCH();

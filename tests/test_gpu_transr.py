@@ -64,6 +64,10 @@ def test_grouped_forward(oracle, model, shape, p):
     dict(dim=101, batch=64, n_rel=5),
     dict(dim=202, batch=700, n_rel=90),
     dict(dim=7, batch=9, n_rel=2),
+    dict(dim=100, batch=200, n_rel=120),   # thin groups of the back-row kernel: two quads per lane
+    dict(dim=160, batch=200, n_rel=120),   # three
+    dict(dim=208, batch=300, n_rel=200),   # four, the widest row it keeps in registers
+    dict(dim=212, batch=300, n_rel=200),   # the first that takes two sweeps again
 ])
 @pytest.mark.parametrize("p", [1, 2])
 @pytest.mark.parametrize("back", [False, True])
@@ -486,10 +490,9 @@ def test_staged_batches_are_planned_a_step_ahead(oracle):
 
 @pytest.mark.parametrize("p", [1, 2])
 def test_train_step_with_and_without_back_rows(oracle, p):
-    """TrainStep(back_rows=True), the default where the batch qualifies, against back_rows=False: scores, relation
-    rows and projection gradients come from the same kernels (bit-identical), the entity rows from different
-    ones (coefficient applied after instead of before the product with the transposed projection): both meet
-    the oracle."""
+    """TrainStep(back_rows=True), the default where the batch qualifies, against back_rows=False: the two forms
+    round differently (another summation order in the thin groups' forward products; the coefficient applied
+    after instead of before the product with the transposed projection) and both meet the oracle."""
     from cuke_amd.kge import TrainStep
     w = synth.make_workload("cfg3_transr", batch=2048, seed=5, norm_p=p)
     m, ix = gpu_model(w)
@@ -506,8 +509,12 @@ def test_train_step_with_and_without_back_rows(oracle, p):
         if p == 2:
             assert_close(g.ent_rows.cpu().numpy(), ref.ent_rows, what="entity rows", rows=True)
         outs.append((st.pos.clone(), g.ent_ids.clone(), g.ent_rows.clone(), g.rel_rows.clone(), g.aux_rows.clone()))
-    assert torch.equal(outs[0][0], outs[1][0]) and torch.equal(outs[0][1], outs[1][1])
-    assert torch.equal(outs[0][3], outs[1][3]) and torch.equal(outs[0][4], outs[1][4])
+    # (the forward kernel that also writes the back rows sums a thin group's products in another order)
+    assert torch.equal(outs[0][1], outs[1][1])
+    assert_close(outs[0][0].cpu().numpy(), outs[1][0].cpu().numpy(), what="scores")
+    if p == 2:
+        assert_close(outs[0][3].cpu().numpy(), outs[1][3].cpu().numpy(), what="relation rows", rows=True)
+        assert_close(outs[0][4].cpu().numpy(), outs[1][4].cpu().numpy(), what="projection gradients", rows=True)
     assert_close(outs[0][2].cpu().numpy(), outs[1][2].cpu().numpy(), what="entity rows, back rows against the dX pass",
                  rows=True, global_floor=0.5 if p == 1 else 0.0)
     # a forward-only step leaves the rows alone
