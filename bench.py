@@ -51,7 +51,7 @@ PROFILE_KERNELS = {
     "seg_reduce_l1": ["seg_reduce_l1"],
     "seg_reduce_l2": ["seg_reduce_l2"],
     "transr_plan_kernel + transr_gemm_kernel<fwd>": ["transr_plan_kernel", "transr_gemm_kernel<0>"],
-    "transr_plan_kernel + transr_gemm_kernel<fwd + back rows>": ["transr_plan_kernel", "transr_gemm_kernel<0>"],
+    "transr_plan_kernel + transr_fwd_back_kernel": ["transr_plan_kernel", "transr_fwd_back_kernel"],
     "transr_gemm_kernel<dX>": ["transr_gemm_kernel<2>"],
     "transr_dm_kernel": ["transr_dm_kernel"],
 }
@@ -172,7 +172,7 @@ def kernel_model(w, label, u_ent, u_rel):
         return 4 * (u_ent * d) // 8, 0, "valu"
     if label.startswith("transr_plan_kernel") or label == "transr_gemm_kernel<dX>":
         by = 4 * (u_rel * d * d + 3 * B * d + u_rel * d) + 8 * 3 * B
-        if "back rows" in label:  # the forward kernel also does the backward pass's product with the transposed projections
+        if "fwd_back" in label:  # the forward kernel also does the backward pass's product with the transposed projections
             return 2 * by, 4 * B * d * d, "mfma"
         return by, 2 * B * d * d, "mfma"
     # dM: the x rows (two entity rows for TransR) and the residual rows in, one gradient per distinct relation out

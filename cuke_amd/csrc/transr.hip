@@ -1628,7 +1628,7 @@ int launch_transr_fwd(const kge_tables *tab, const kge_batch *bat, float *pos, f
         else
             hipLaunchKernelGGL(transr_gemm_kernel<0>, grid, dim3(256), lds, st, a, fi);
     }
-    timeline_mark(bat->timeline, st, a.back ? "transr_plan_kernel + transr_gemm_kernel<fwd + back rows>"
+    timeline_mark(bat->timeline, st, a.back ? "transr_plan_kernel + transr_fwd_back_kernel"
                                             : "transr_plan_kernel + transr_gemm_kernel<fwd>");
     KGE_CHECK_LAUNCH();
     return KGE_OK;
