@@ -28,11 +28,11 @@ extern "C" int kge_train_step_staged(const kge_tables *tab, kge_step_batch *cur,
         if (projection && !next->bat.neg && next->fwd_workspace) {
             // the relation groups drive the forward pass: inspected and planned here, a step ahead
             if (!next->planned) return KGE_EINVAL;
-            if ((rc = kge_inspect_batch(&jobs[1], 1, side_stream))) return rc;
+            // (both index sets in one batch of launches, then the plans: the step waits for all of it at once)
+            if ((rc = kge_inspect_batch(jobs, 2, side_stream))) return rc;
             if ((rc = kge_transr_plan(tab, &next->bat, next->fwd_workspace, next->fwd_workspace_bytes, side_stream))) return rc;
             if (hipEventRecord(as_event(next->planned), side) != hipSuccess) return KGE_ELAUNCH;
             next->bat.plans_ready = 1;
-            rc = kge_inspect_batch(&jobs[0], 1, side_stream);
         } else if (projection) {
             rc = kge_inspect_batch(&jobs[0], 1, side_stream);  // (the relations are inspected on the main stream, by the step)
         } else {

@@ -846,13 +846,13 @@ class TrainStep:
             # that run() starts with the projection kernel
             if getattr(s, "ws_f", None) is None:
                 s.ws_f = torch.empty(max(self._ws_f_bytes, 1), dtype=torch.uint8, device=self.m.dev)
-            _lib.check(self.L.kge_inspect_batch(C.byref(s.jobs[1]), 1, sst), "kge_inspect_batch(relations)")
+            # (both index sets in one batch of launches, then the plans: the step waits for all of it at once)
+            _lib.check(self.L.kge_inspect_batch(s.jobs, 2, sst), "kge_inspect_batch")
             _lib.check(self.L.kge_transr_plan(C.byref(self.m._tab), C.byref(s.bat), _ptr(s.ws_f), self._ws_f_bytes, sst),
                        "kge_transr_plan")
             s.planned_event = torch.cuda.Event()
             s.planned_event.record(side)
             s.bat.plans_ready = 1
-            _lib.check(self.L.kge_inspect_batch(C.byref(s.jobs[0]), 1, sst), "kge_inspect_batch(entities)")
         elif self.needs_rel_groups:  # (with shared negatives the forward call plans its own row list)
             _lib.check(self.L.kge_inspect_batch(C.byref(s.jobs[0]), 1, sst), "kge_inspect_batch(entities)")
         else:

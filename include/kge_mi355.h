@@ -433,8 +433,8 @@ int kge_sample_negatives(int64_t *out, int64_t count, int64_t n_ent, uint64_t se
 /*
  * One step of a staged training loop in ONE call (host-side sequencing only; no counterpart in the
  * reference, which has no training loop).  It enqueues what a host loop would enqueue with seven to ten
- * calls: on `side_stream` the inspection of the NEXT batch (TransR / RESCAL without negatives: the relation
- * inspection, the tile plans into next->fwd_workspace, then the entity inspection), on `stream` the step
+ * calls: on `side_stream` the inspection of the NEXT batch (TransR / RESCAL without negatives: both
+ * inspections in one batch of launches, then the tile plans into next->fwd_workspace), on `stream` the step
  * of the CURRENT batch -- kge_score_fwd, kge_margin_loss when buf->loss is set, kge_score_bwd -- and the
  * events between the two streams.  For steps so short (tens of microseconds) that the host's per-call
  * overhead, not the device, would set the pace.
@@ -446,8 +446,8 @@ int kge_sample_negatives(int64_t *out, int64_t count, int64_t n_ent, uint64_t se
  *              before its segmented reduction (kge_batch.insp_ready).  TransR / RESCAL without negatives:
  *              `stream` waits for it once, before the forward pass (it is recorded behind the plans too, and
  *              the batch was staged a step ahead), and kge_score_bwd has no wait of its own.
- *   planned    TransR / RESCAL without negatives: recorded behind the relation inspection and the tile
- *              plans (for callers that pipeline deeper).  Else unused (may be NULL).
+ *   planned    TransR / RESCAL without negatives: recorded behind the inspections and the tile plans.  Else
+ *              unused (may be NULL).
  *   released   recorded on `stream` behind the step; a later staging of the same kge_step_batch makes
  *              side_stream wait for it before it overwrites the inspection (released_valid says whether
  *              it has been recorded yet; zero-initialise it).
