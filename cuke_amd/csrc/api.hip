@@ -13,6 +13,7 @@ bool score_neg_carries_positives(const kge_tables *, const kge_batch *);
 size_t neg_split_workspace(const kge_tables *, const kge_batch *);
 int launch_transr_fwd(const kge_tables *, const kge_batch *, float *, float *, void *, size_t, hipStream_t);
 bool back_rows_ok(const kge_tables *, const kge_batch *);
+int launch_rescal_head_rows(const kge_tables *, const kge_batch *, float *, void *, size_t, hipStream_t);
 size_t transr_fwd_workspace(const kge_tables *, const kge_batch *);
 int launch_transr_plan(const kge_tables *, const kge_batch *, void *, size_t, hipStream_t);
 int launch_transr_neg_fwd(const kge_tables *, const kge_batch *, float *, float *, float *, void *, size_t, hipStream_t);
@@ -228,8 +229,9 @@ int kge_score_fwd(const kge_tables *tab, const kge_batch *bat, float *pos, float
     if (bat->back_rows && !back_rows_ok(tab, bat)) return KGE_EUNSUPPORTED;  // (only TransR's grouped forward writes them)
     if (want_neg && (tab->model == KGE_TRANSH || tab->model == KGE_TRANSF) && !side_pos) return KGE_EINVAL;
     if (want_neg && tab->model == KGE_ROTATE && !residual) return KGE_EINVAL;  // rotated heads buffer
-    if (want_neg && tab->model == KGE_RESCAL && (!residual || bat->neg_mode != KGE_NEG_TAIL))
-        return residual ? KGE_EUNSUPPORTED : KGE_EINVAL;  // the projected rows are the pair kernel's queries
+    if (want_neg && tab->model == KGE_RESCAL && !residual) return KGE_EINVAL;  // the projected rows are the pair kernel's queries
+    const bool rescal_head = want_neg && tab->model == KGE_RESCAL && bat->neg_mode == KGE_NEG_HEAD;
+    if (rescal_head && !bat->rel_insp) return KGE_EUNSUPPORTED;  // (the rows Proj[r] E[t] come from the grouped pass)
     // fused inspection: first digit pass with the per-positive kernel, second with the tile kernel
     const bool grouped_model = tab->model == KGE_TRANSR || tab->model == KGE_RESCAL;
     const bool fuse = bat->fuse_inspection != 0 && !grouped_model;  // (the grouped kernels plan their own riders)
@@ -248,7 +250,13 @@ int kge_score_fwd(const kge_tables *tab, const kge_batch *bat, float *pos, float
     // written by the negatives' launch, and its timeline entry "score_neg_kernel" includes the positives.
     const bool carry = want_neg && pos && !side_pos && !residual && !fuse && score_neg_carries_positives(tab, bat);
     if (!carry && (pos || side_pos || residual)) {
-        if ((tab->model == KGE_TRANSR || tab->model == KGE_RESCAL) && bat->rel_insp)
+        if (rescal_head) {
+            // corrupted heads: the positives' scores from the usual pass, then `residual` takes the rows
+            // u_b = Proj[r_b] E[t_b] that the pair scores E[h'] . u_b (and the backward pass) are formed from
+            rc = pos ? launch_transr_fwd(tab, bat, pos, nullptr, workspace, workspace_bytes, st)
+                     : launch_transr_plan(tab, bat, workspace, workspace_bytes, st);
+            if (!rc) rc = launch_rescal_head_rows(tab, bat, residual, workspace, workspace_bytes, st);
+        } else if ((tab->model == KGE_TRANSR || tab->model == KGE_RESCAL) && bat->rel_insp)
             rc = launch_transr_fwd(tab, bat, pos, residual, workspace, workspace_bytes, st);
         else {
             rc = launch_score_pos_fused(tab, bat, pos, residual, side_pos, fuse ? &fi0 : nullptr, st);

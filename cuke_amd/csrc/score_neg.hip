@@ -667,8 +667,9 @@ int launch_score_neg(const kge_tables *tab, const kge_batch *bat, const float *s
     case KGE_COMPLEX: return launch_neg_mp<KGE_COMPLEX, 2>(a, n_chunks, dv, fi, st);
     case KGE_ROTATE: return launch_neg_mp<KGE_ROTATE, 2>(a, n_chunks, dv, fi, st);
     case KGE_TRANSF: return launch_neg_mp<KGE_TRANSF, 2>(a, n_chunks, dv, fi, st);
-    case KGE_RESCAL:  // negatives that replace the tail: a dot-product tile over the projected rows E[h] Proj[r]
-        if (!query || head) return KGE_EUNSUPPORTED;
+    case KGE_RESCAL:  // a dot-product tile over the projected rows: E[h] Proj[r] against replaced tails,
+                      // Proj[r] E[t] against replaced heads
+        if (!query) return KGE_EUNSUPPORTED;
         return launch_neg_mp<KGE_RESCAL, 2>(a, n_chunks, dv, fi, st);
     default: return KGE_EUNSUPPORTED;  // TransR: its own grouped path
     }

@@ -223,7 +223,8 @@ struct GemmArgs {
     const int32_t *perm, *seg_offsets, *num_unique;
     const int64_t *unique_ids;
     TilePlan plan;
-    const float *xs;  // TRANSPOSED pass: left operand rows in sorted order [B, d]; null: formed from `src`
+    const float *xs;  // TRANSPOSED pass: left operand rows in sorted order [B, d]; null: formed from `src`.
+                      // RESCAL forward (MODE 1), optional: the rows x in sorted order instead of E[h]
     const float *rs;  // list pass (MODE 3): factor of the relation row per list row (+1, -1 or 0)
     float *pos;       // forward: [B] scores (nullable)
     float *resid;     // forward: [B, d] rows y (nullable)
@@ -304,7 +305,8 @@ __device__ __forceinline__ void transr_thin_fwd_body(const GemmArgs &a, float *l
     __syncthreads();
     for (int f = tid; f < rows * nq4; f += 256) {
         const int r = f / nq4, k4 = (f % nq4) * 4;
-        float4 v = *reinterpret_cast<const float4 *>(a.ent + s_h[r] * (int64_t)d + k4);
+        float4 v = (MODE == 1 && a.xs) ? *reinterpret_cast<const float4 *>(a.xs + (int64_t)(tt.p0 + r) * d + k4)
+                                       : *reinterpret_cast<const float4 *>(a.ent + s_h[r] * (int64_t)d + k4);
         if constexpr (MODE == 0) {
             const float4 u = *reinterpret_cast<const float4 *>(a.ent + s_t[r] * (int64_t)d + k4);
             v = make_float4(v.x - u.x, v.y - u.y, v.z - u.z, v.w - u.w);
@@ -707,7 +709,10 @@ __device__ __forceinline__ void transr_gemm_body(const GemmArgs &a, float *lds, 
                             v[q] = *reinterpret_cast<const float4 *>(a.xs + (int64_t)(p0 + row) * d + k4);
                         }
                     } else {
-                        v[q] = *reinterpret_cast<const float4 *>(a.ent + s_h[row] * (int64_t)d + k4);
+                        if (MODE == 1 && a.xs)  // uniform: left operand rows given in sorted order
+                            v[q] = *reinterpret_cast<const float4 *>(a.xs + (int64_t)(p0 + row) * d + k4);
+                        else
+                            v[q] = *reinterpret_cast<const float4 *>(a.ent + s_h[row] * (int64_t)d + k4);
                         if constexpr (MODE == 0)
                             u[q] = *reinterpret_cast<const float4 *>(a.ent + s_t[row] * (int64_t)d + k4);
                         if constexpr (MODE == 3) {
@@ -1634,11 +1639,35 @@ int launch_transr_fwd(const kge_tables *tab, const kge_batch *bat, float *pos, f
     return KGE_OK;
 }
 
+// RESCAL with corrupted heads: the pair score E[h'] . (Proj[r] E[t]) needs the rows u_b = E[t_b] Proj[r_b]^T.  Same
+// grouped pass as dX with E[t] as its upstream rows and coefficient 1; the plans are the ones the forward call of
+// the positives left in `workspace`.
+int launch_rescal_head_rows(const kge_tables *tab, const kge_batch *bat, float *u, void *workspace, size_t workspace_bytes,
+                            hipStream_t st)
+{
+    if (bat->batch == 0) return KGE_OK;
+    if (tab->model != KGE_RESCAL || !bat->rel_insp || !u || !aligned16(u)) return KGE_EINVAL;
+    if (pad_path_ok(tab, bat) || !mfma_path_ok(tab, bat) || gemm_lds_bytes((int)tab->dim) > kMaxGemmLds) return KGE_EUNSUPPORTED;
+    if (!workspace || workspace_bytes < transr_fwd_workspace(tab, bat)) return KGE_EWORKSPACE;
+    const kge_inspection *ri = bat->rel_insp;
+    const int d = (int)tab->dim;
+    const int64_t tiles = max_tiles(tab, bat);
+    TilePlan plan = plan_at(workspace, tiles, 0);
+    const BwdSrc src{tab->ent, nullptr, nullptr, nullptr, bat->h, bat->t, ri->perm, tab->norm_p, 1, nullptr, 1};
+    GemmArgs ga{tab->ent, tab->rel, tab->aux, bat->h, bat->r, bat->t, ri->perm, ri->seg_offsets, ri->num_unique, ri->unique_ids,
+                plan, nullptr, nullptr, nullptr, nullptr, u, nullptr, d, tab->norm_p, thin_groups(tab, bat), (int)tiles, src};
+    if (const int rc = allow_lds<2>(gemm_lds_bytes(d))) return rc;
+    hipLaunchKernelGGL(transr_gemm_kernel<2>, dim3((unsigned)(tiles + ga.thin_groups)), dim3(256), gemm_lds_bytes(d), st, ga, FusedInsp{});
+    timeline_mark(bat->timeline, st, "transr_gemm_kernel<head rows>");
+    KGE_CHECK_LAUNCH();
+    return KGE_OK;
+}
+
 // The tile plans alone (what launch_transr_fwd builds first), for callers that plan a batch ahead.
 int launch_transr_plan(const kge_tables *tab, const kge_batch *bat, void *workspace, size_t workspace_bytes, hipStream_t st)
 {
     if (bat->batch == 0) return KGE_OK;
-    if (bat->neg) return KGE_EUNSUPPORTED;  // the shared-negative path plans its own row list
+    if (bat->neg && tab->model == KGE_TRANSR) return KGE_EUNSUPPORTED;  // TransR's shared-negative path plans its own row list
     if (pad_path_ok(tab, bat)) return launch_transr_plan_padded(tab, bat, workspace, workspace_bytes, st);
     if (!mfma_path_ok(tab, bat) || gemm_lds_bytes((int)tab->dim) > kMaxGemmLds) return KGE_EUNSUPPORTED;
     if (!workspace || workspace_bytes < transr_fwd_workspace(tab, bat)) return KGE_EWORKSPACE;
@@ -1698,10 +1727,12 @@ size_t transr_bwd_workspace(const kge_tables *tab, const kge_batch *bat)
     return make_rplan(tab, bat).total;
 }
 
-// One wave per sorted position p (triple b = perm[p]): xs[p] = E[h], qs[p] = g E[t] + G[b], occ_t[b] = g v[b].
+// One wave per sorted position p (triple b = perm[p]).  Replaced tails: xs[p] = E[h], qs[p] = g E[t] + G[b],
+// occ_o[b] = g v[b] (the tail's occurrence row, v = E[h] Proj[r]).  Replaced heads (head != 0): xs[p] = g E[h] + G[b],
+// qs[p] = E[t], occ_o[b] = g u[b] (the head's occurrence row, u = Proj[r] E[t]).
 __global__ __launch_bounds__(256) void rescal_neg_prep_kernel(const float *ent, const int64_t *h, const int64_t *t, const int32_t *perm,
                                                               const float *dpos, const float *G, const float *resid, float *xs,
-                                                              float *qs, float *occ_t, int64_t B, int d)
+                                                              float *qs, float *occ_o, int64_t B, int d, int head)
 {
     const int lane = threadIdx.x & 63;
     const int64_t p = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
@@ -1713,9 +1744,14 @@ __global__ __launch_bounds__(256) void rescal_neg_prep_kernel(const float *ent, 
         const float4 vh = *reinterpret_cast<const float4 *>(eh + j), vt = *reinterpret_cast<const float4 *>(et + j);
         const float4 ve = *reinterpret_cast<const float4 *>(resid + (int64_t)b * d + j);
         const float4 vg = G ? *reinterpret_cast<const float4 *>(G + (int64_t)b * d + j) : make_float4(0.f, 0.f, 0.f, 0.f);
-        *reinterpret_cast<float4 *>(xs + p * d + j) = vh;
-        *reinterpret_cast<float4 *>(qs + p * d + j) = make_float4(fmaf(g, vt.x, vg.x), fmaf(g, vt.y, vg.y), fmaf(g, vt.z, vg.z), fmaf(g, vt.w, vg.w));
-        *reinterpret_cast<float4 *>(occ_t + (int64_t)b * d + j) = scaled4(g, ve);
+        if (head) {  // uniform
+            *reinterpret_cast<float4 *>(xs + p * d + j) = make_float4(fmaf(g, vh.x, vg.x), fmaf(g, vh.y, vg.y), fmaf(g, vh.z, vg.z), fmaf(g, vh.w, vg.w));
+            *reinterpret_cast<float4 *>(qs + p * d + j) = vt;
+        } else {
+            *reinterpret_cast<float4 *>(xs + p * d + j) = vh;
+            *reinterpret_cast<float4 *>(qs + p * d + j) = make_float4(fmaf(g, vt.x, vg.x), fmaf(g, vt.y, vg.y), fmaf(g, vt.z, vg.z), fmaf(g, vt.w, vg.w));
+        }
+        *reinterpret_cast<float4 *>(occ_o + (int64_t)b * d + j) = scaled4(g, ve);
     }
 }
 
@@ -1727,7 +1763,7 @@ __global__ void rescal_fill_zero_kernel(float *p, int64_t n)
 int launch_rescal_neg_bwd(const kge_tables *tab, const kge_batch *bat, const kge_saved *saved, const float *dpos,
                                  const float *dneg, const kge_grads *grads, void *workspace, size_t workspace_bytes, hipStream_t st)
 {
-    if (bat->neg_mode != KGE_NEG_TAIL) return KGE_EUNSUPPORTED;  // (head negatives: the flattened triples)
+    const bool head = bat->neg_mode == KGE_NEG_HEAD;
     if (!mfma_path_ok(tab, bat) || gemm_lds_bytes((int)tab->dim) > kMaxGemmLds) return KGE_EUNSUPPORTED;
     if (bat->fuse_inspection) return KGE_EINVAL;
     if (!saved->residual || !aligned16(saved->residual) || !grads->aux_rows || !grads->ent_rows) return KGE_EINVAL;
@@ -1748,16 +1784,29 @@ int launch_rescal_neg_bwd(const kge_tables *tab, const kge_batch *bat, const kge
     } else if (p.nn > 0) {  // no upstream gradient on the pairs: the negatives' occurrence rows are zero
         hipLaunchKernelGGL(rescal_fill_zero_kernel, dim3(1024), dim3(256), 0, st, occ + 2 * B * d, p.nn * d);
     }
+    // (occurrence rows: [h of the B positives | t of the B positives | negatives])
     hipLaunchKernelGGL(rescal_neg_prep_kernel, dim3((unsigned)ceil_div(B, 4)), dim3(256), 0, st, tab->ent, bat->h, bat->t, ri->perm, dpos,
-                       dneg ? g0 : nullptr, saved->residual, xs, qs, occ + B * d, B, d);
+                       dneg ? g0 : nullptr, saved->residual, xs, qs, head ? occ : occ + B * d, B, d, head ? 1 : 0);
     TilePlan plan = plan_at(ws + p.off_plan, p.tiles, 0), dplan = dplan_at(ws + p.off_dplan, p.dtiles, p.dsplit, d);
     hipLaunchKernelGGL(transr_plan_kernel, dim3(2), dim3(1024), 0, st, ri->num_unique, ri->seg_offsets, ri->unique_ids, plan, kTM, dplan,
                        kDmChunk, dm_nib(d), dm_small_max(d));
-    GemmArgs ga{tab->ent, tab->rel, tab->aux, bat->h, bat->r, bat->t, ri->perm, ri->seg_offsets, ri->num_unique, ri->unique_ids,
-                plan, qs, nullptr, nullptr, nullptr, occ, nullptr, d, tab->norm_p, thin_groups(tab, bat), (int)p.tiles, BwdSrc{}};
-    if (const int rc = allow_lds<2>(gemm_lds_bytes(d))) return rc;
-    hipLaunchKernelGGL(transr_gemm_kernel<2>, dim3((unsigned)(p.tiles + ga.thin_groups)), dim3(256), gemm_lds_bytes(d), st, ga, FusedInsp{});
+    if (head) {
+        // the tails' rows: (g E[h] + G) Proj[r], the forward product on rows given as an array, written per triple
+        GemmArgs ga{tab->ent, tab->rel, tab->aux, bat->h, bat->r, bat->t, ri->perm, ri->seg_offsets, ri->num_unique, ri->unique_ids,
+                    plan, xs, nullptr, nullptr, occ + B * d, nullptr, nullptr, d, tab->norm_p, thin_groups(tab, bat), (int)p.tiles,
+                    BwdSrc{}};
+        if (const int rc = allow_lds<1>(gemm_lds_bytes(d))) return rc;
+        hipLaunchKernelGGL(transr_gemm_kernel<1>, dim3((unsigned)(p.tiles + ga.thin_groups)), dim3(256), gemm_lds_bytes(d), st, ga,
+                           FusedInsp{});
+    } else {
+        GemmArgs ga{tab->ent, tab->rel, tab->aux, bat->h, bat->r, bat->t, ri->perm, ri->seg_offsets, ri->num_unique, ri->unique_ids,
+                    plan, qs, nullptr, nullptr, nullptr, occ, nullptr, d, tab->norm_p, thin_groups(tab, bat), (int)p.tiles, BwdSrc{}};
+        if (const int rc = allow_lds<2>(gemm_lds_bytes(d))) return rc;
+        hipLaunchKernelGGL(transr_gemm_kernel<2>, dim3((unsigned)(p.tiles + ga.thin_groups)), dim3(256), gemm_lds_bytes(d), st, ga,
+                           FusedInsp{});
+    }
     timeline_mark(bat->timeline, st, "transr_gemm_kernel<dX>");
+    // dProj[r][i][j] = sum over the group of xs[i] qs[j] in both modes
     DmArgs da{xs, qs, ri->seg_offsets, dplan, grads->aux_rows, reinterpret_cast<float *>(ws + p.off_dpart), d, ri->num_unique,
               BwdSrc{}, nullptr, nullptr, 0};
     hipLaunchKernelGGL(transr_dm_kernel, dim3((unsigned)kDmWgs), dim3(256), dm_lds_bytes(d), st, da, FusedInsp{}, SegL1Rider{});

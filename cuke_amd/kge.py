@@ -285,9 +285,10 @@ class KGEModel:
         (apps/examples/examples.py:1404-1444); ``'head'``: (neg_k, r_b, t_b), the head-corrupted batches of
         the reference's sampler (apps/kge/data/sampler.py:287-353)."""
         if neg is not None and self.model == "RESCAL":
-            # tail negatives: (E[h] Proj[r]) . E[t'] is a dot-product tile over the B projected rows; head
-            # negatives and shapes outside the grouped kernels: the pairs as explicit triples
-            if neg_mode != "tail" or self.dim % 4 != 0 or self.dim > 1024:
+            # a dot-product tile over B projected rows: (E[h] Proj[r]) . E[t'] for replaced tails,
+            # E[h'] . (Proj[r] E[t]) for replaced heads; shapes outside the grouped kernels: the pairs as
+            # explicit triples
+            if self.dim % 4 != 0 or self.dim > 1024:
                 return self._score_projected_negatives(h, r, t, neg, chunk, neg_mode)
             if rel_insp is None:
                 rel_insp = inspect([_index(r, "r", self.dev)], self.n_rel)

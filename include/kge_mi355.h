@@ -197,7 +197,8 @@ typedef struct kge_saved {
                                negatives r.h (r.t); TransR: unused */
     const float *side_neg;  /* [2, B, n_neg]: TransH, plane 0 = w_b . e_k per pair (e_k the negative),
                                plane 1 = sum_i phi(u_i) w_i (phi = sign for L1, u/||u|| for L2) */
-    const float *residual;  /* [B, dim]: TransR residual rows / RESCAL E[h] Proj[r] rows;
+    const float *residual;  /* [B, dim]: TransR residual rows / RESCAL E[h] Proj[r] rows (with shared negatives
+                               that replace the head: Proj[r] E[t] rows);
                                RotatE: rotated heads h e^{i theta} as [re | im]
                                (with KGE_NEG_HEAD: counter-rotated tails t e^{-i theta}) */
     /* TransR / RESCAL, optional: the workspace the forward call of this batch was given (it
@@ -272,8 +273,9 @@ int kge_residual_fwd(const kge_tables *tab, const kge_batch *bat, float *out, vo
  * (E[h] Proj[r]) . E[t'] needs no projection of the negatives, so pos, neg and `residual` ([B, dim],
  * the projected rows E[h] Proj[r], required) come out of one call: the grouped pass over the B
  * positives, then the dot-product tile kernel of DistMult with the projected rows as its query rows.
- * kge_score_bwd chains the pairs' gradient through the same B rows.  KGE_NEG_HEAD returns
- * KGE_EUNSUPPORTED here (kge_flatten_negatives covers it).
+ * kge_score_bwd chains the pairs' gradient through the same B rows.  With KGE_NEG_HEAD the pair score is
+ * E[h'] . (Proj[r] E[t]): `residual` then receives the rows Proj[r_b] E[t_b] (one more grouped pass, with the
+ * transposed projections), which are the tile's query rows and what kge_score_bwd expects in kge_saved.residual.
  * TransE / RotatE with shared negatives on small batches (the 32 x 32 pair tiles would leave one or
  * two workgroups per CU): given kge_score_fwd_workspace() bytes of workspace the reduction axis of
  * every tile is split over up to four workgroups (partial score planes in the workspace, a finishing
@@ -387,8 +389,7 @@ int kge_build_index(const int64_t *r, int64_t *uniq, int64_t *buf, int64_t *cnt,
  * them (apps/examples/examples.py:1447-1480: every view is flattened to batch * blocksize rows).
  * Outputs have B * (1 + n_neg) entries: the B positives first, then row B + b * n_neg + k =
  * (h[b], r[b], neg[(b / chunk) * n_neg + k]).  TransR and RESCAL have grouped forms of kge_score_fwd
- * (see there) and use the list only for what those do not take: shapes outside the grouped kernels,
- * and RESCAL with negatives that replace the head.
+ * (see there) and use the list only for what those do not take: shapes outside the grouped kernels.
  */
 int kge_flatten_negatives(const kge_batch *bat, int64_t *h_flat, int64_t *r_flat, int64_t *t_flat,
                           void *stream);

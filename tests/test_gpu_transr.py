@@ -323,17 +323,19 @@ def test_shared_negatives_through_flattened_triples(oracle, model):
     dict(dim=256, batch=1024, chunk=256, n_neg=256, n_rel=300),
     dict(dim=16, batch=7, chunk=7, n_neg=1, n_rel=3),
 ])
-def test_rescal_shared_negatives_as_a_dot_product_tile(oracle, shape):
-    """RESCAL with negatives that replace the tail: (E[h] Proj[r]) . E[t'] from the B projected rows and the
-    dot-product tile kernel (no projection of the negatives, no flattened triples), forward and backward
-    against the oracle's explicit pairs; with missing upstream gradients; and through TrainStep."""
+@pytest.mark.parametrize("mode", ["tail", "head"])
+def test_rescal_shared_negatives_as_a_dot_product_tile(oracle, shape, mode):
+    """RESCAL with shared negatives: (E[h] Proj[r]) . E[t'] for replaced tails, E[h'] . (Proj[r] E[t]) for replaced
+    heads, from B projected rows and the dot-product tile kernel (no projection of the negatives, no flattened
+    triples), forward and backward against the oracle's explicit pairs; with missing upstream gradients; and
+    through TrainStep."""
     from cuke_amd.kge import TrainStep
     w = synth.custom_workload("RESCAL", n_ent=400, norm_p=2, sigma=0.2, rel_zipf=1.1, ent_zipf=1.1, seed=13, **shape)
     a = w.arrays
     m, ix = gpu_model(w)
-    fw = m.score(ix["h"], ix["r"], ix["t"], ix["neg"], w.chunk)
+    fw = m.score(ix["h"], ix["r"], ix["t"], ix["neg"], w.chunk, neg_mode=mode)
     assert fw.flat_pos is None, "the flattened triples ran instead of the tile path"
-    pos, negs = oracle.score("RESCAL", a["E"], a["R"], a["A"], a["h"], a["r"], a["t"], a["neg"], w.chunk)
+    pos, negs = oracle.score("RESCAL", a["E"], a["R"], a["A"], a["h"], a["r"], a["t"], a["neg"], w.chunk, neg_mode=mode)
     assert_close(fw.pos.cpu().numpy(), pos, what="pos")
     assert_close(fw.neg.cpu().numpy(), negs, what="neg")
     rng = np.random.default_rng(5)
@@ -342,16 +344,18 @@ def test_rescal_shared_negatives_as_a_dot_product_tile(oracle, shape):
     for gp, gn, tag in ((dpos, dneg, "both"), (None, dneg, "pairs only"), (dpos, None, "positives only")):
         g = m.backward(fw, None if gp is None else torch.from_numpy(gp).cuda(), None if gn is None else torch.from_numpy(gn).cuda())
         ref = oracle.backward("RESCAL", a["E"], a["R"], a["A"], a["h"], a["r"], a["t"], a["neg"], w.chunk,
-                              gp if gp is not None else np.zeros_like(dpos), gn if gn is not None else np.zeros_like(dneg))
+                              gp if gp is not None else np.zeros_like(dpos), gn if gn is not None else np.zeros_like(dneg),
+                              neg_mode=mode)
         assert np.array_equal(g.ent_ids.cpu().numpy(), ref.ent_ids) and np.array_equal(g.rel_ids.cpu().numpy(), ref.rel_ids)
         assert_close(g.ent_rows.cpu().numpy(), ref.ent_rows, what=f"{tag}: entity rows", rows=True)
         assert_close(g.aux_rows.cpu().numpy(), ref.aux_rows, what=f"{tag}: projection gradients", rows=True)
     # the flattened formulation of the reference must agree
-    flat = m._score_projected_negatives(ix["h"], ix["r"], ix["t"], ix["neg"], w.chunk)
+    flat = m._score_projected_negatives(ix["h"], ix["r"], ix["t"], ix["neg"], w.chunk, mode)
     assert_close(fw.neg.cpu().numpy(), flat.neg.cpu().numpy(), what="tile path vs flattened triples")
     step = TrainStep(m, ix["h"], ix["r"], ix["t"], ix["neg"], w.chunk, dpos=torch.from_numpy(dpos).cuda(),
-                     dneg=torch.from_numpy(dneg).cuda())
-    ref = oracle.backward("RESCAL", a["E"], a["R"], a["A"], a["h"], a["r"], a["t"], a["neg"], w.chunk, dpos, dneg)
+                     dneg=torch.from_numpy(dneg).cuda(), neg_mode=mode)
+    ref = oracle.backward("RESCAL", a["E"], a["R"], a["A"], a["h"], a["r"], a["t"], a["neg"], w.chunk, dpos, dneg,
+                          neg_mode=mode)
     for tag, kw in (("side stream", {}), ("one stream", dict(overlap=False))):
         step.run(**kw)
         torch.cuda.synchronize()
