@@ -851,9 +851,7 @@ class TrainStep:
             _lib.check(self.L.kge_inspect_batch(s.jobs, 2, sst), "kge_inspect_batch")
             _lib.check(self.L.kge_transr_plan(C.byref(self.m._tab), C.byref(s.bat), _ptr(s.ws_f), self._ws_f_bytes, sst),
                        "kge_transr_plan")
-            s.planned_event = torch.cuda.Event()
-            s.planned_event.record(side)
-            s.bat.plans_ready = 1
+            s.bat.plans_ready = 1  # (run() waits for insp_event, recorded below behind the plans)
         elif self.needs_rel_groups:  # (with shared negatives the forward call plans its own row list)
             _lib.check(self.L.kge_inspect_batch(C.byref(s.jobs[0]), 1, sst), "kge_inspect_batch(entities)")
         else:
