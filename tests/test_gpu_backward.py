@@ -11,7 +11,7 @@ pytestmark = pytest.mark.gpu
 NEG_MODELS = ["TransE", "TransH", "DistMult", "ComplEx", "RotatE", "TransF"]
 
 
-def run_both(oracle, w, seed=0, use_pos=True, use_neg=True, pair_sums="matrix_cores", fast=False):
+def run_both(oracle, w, seed=0, use_pos=True, use_neg=True, pair_sums="matrix_cores", fast=False, neg_mode="tail"):
     a = w.arrays
     rng = np.random.default_rng(seed)
     dpos = rng.standard_normal(w.batch).astype(np.float32) if use_pos else None
@@ -19,12 +19,12 @@ def run_both(oracle, w, seed=0, use_pos=True, use_neg=True, pair_sums="matrix_co
     dneg = rng.standard_normal((w.batch, w.n_neg)).astype(np.float32) if (has_neg and use_neg) else None
     m, ix = gpu_model(w)
     m.pair_sums = pair_sums
-    fw = m.score(ix["h"], ix["r"], ix["t"], ix.get("neg"), w.chunk or None)
+    fw = m.score(ix["h"], ix["r"], ix["t"], ix.get("neg"), w.chunk or None, neg_mode=neg_mode)
     dev = fw.pos.device
     g = m.backward(fw, None if dpos is None else torch.from_numpy(dpos).to(dev),
                    None if dneg is None else torch.from_numpy(dneg).to(dev))
     ref = oracle.backward(w.model, a["E"], a["R"], a["A"], a["h"], a["r"], a["t"], a.get("neg"), w.chunk,
-                          dpos, dneg, p=w.norm_p, fast=fast)
+                          dpos, dneg, p=w.norm_p, fast=fast, neg_mode=neg_mode)
     return g, ref
 
 
@@ -75,6 +75,27 @@ def test_row_widths_that_end_in_a_narrow_column_tile(oracle, model, p, dim):
                               sigma=0.2, gamma=4.0, ent_zipf=1.1, seed=dim + p, lattice=(p == 1))
     g, ref = run_both(oracle, w, seed=5, fast="omp")
     compare(g, ref, f"{model} p={p} dim={dim}", outliers=(1e-5, 4.0) if model == "RotatE" else None)
+
+
+@pytest.mark.parametrize("model,p,pair_sums", [
+    ("TransE", 1, None), ("TransE", 2, None), ("TransH", 1, None), ("TransH", 2, None), ("RotatE", 2, None),
+    ("DistMult", 2, "vector_alus"), ("ComplEx", 2, "vector_alus"), ("TransF", 2, "vector_alus")])
+@pytest.mark.parametrize("shape", [
+    dict(dim=520, batch=96 * 8, chunk=96, n_neg=72),    # three looper steps either way
+    dict(dim=132, batch=40 * 24, chunk=40, n_neg=200),  # seven steps over the negatives, two over the positives
+    dict(dim=130, batch=64 * 32, chunk=64, n_neg=33),   # rows that are not 16-byte multiples
+])
+@pytest.mark.parametrize("mode", ["tail", "head"])
+def test_batches_of_a_few_hundred_tiles_in_both_negative_modes(oracle, model, p, pair_sums, shape, mode):
+    """Batches between 128 and 511 64-owner tiles (the vector-ALU gradient tiles then own 16 rows each and a CU holds a
+    few of them), looper counts that are no multiples of the 32-row step, corrupted tails and corrupted heads."""
+    klen = shape["dim"] // 2 if model == "RotatE" else shape["dim"]
+    big = -(-klen // 64) * (-(-shape["chunk"] // 64) + -(-shape["n_neg"] // 64)) * (shape["batch"] // shape["chunk"])
+    assert 128 <= big < 512, "this shape is meant for the 16-owner tiles"
+    w = synth.custom_workload(model, n_ent=500, n_rel=11, norm_p=p, sigma=0.2, gamma=4.0, ent_zipf=1.1,
+                              seed=shape["dim"] + p, lattice=(p == 1), **shape)
+    g, ref = run_both(oracle, w, seed=9, pair_sums=pair_sums or "matrix_cores", neg_mode=mode, fast="omp")
+    compare(g, ref, f"{model} {shape} p={p} {mode}", outliers=(1e-5, 4.0) if model == "RotatE" else None)
 
 
 def test_missing_upstream_gradients_mean_zero(oracle):
