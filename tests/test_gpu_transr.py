@@ -320,7 +320,7 @@ def test_shared_negatives_through_flattened_triples(oracle, model):
     dict(dim=40, batch=48, chunk=16, n_neg=12, n_rel=6),
     dict(dim=200, batch=512, chunk=64, n_neg=64, n_rel=50),    # Zipf relations, many thin groups
     dict(dim=64, batch=300, chunk=300, n_neg=33, n_rel=1),     # one relation, odd N, ragged tiles
-    dict(dim=256, batch=1024, chunk=256, n_neg=256, n_rel=300),
+    dict(dim=128, batch=512, chunk=128, n_neg=128, n_rel=100),  # several 64-row tiles per chunk on both sides
     dict(dim=16, batch=7, chunk=7, n_neg=1, n_rel=3),
 ])
 @pytest.mark.parametrize("mode", ["tail", "head"])
